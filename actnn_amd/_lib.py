@@ -1,0 +1,92 @@
+"""Build and load ``libactnn_hip.so`` - the C-ABI library of gfx950 kernels (include/actnn_hip.h).
+
+The library is compiled in-tree with hipcc and loaded with ctypes; there is no CPU fallback:
+if the library is missing, ``load()`` raises.
+"""
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(_HERE, "csrc")
+LIB_PATH = os.path.join(_HERE, "libactnn_hip.so")
+SOURCES = ["minimax.hip", "pack_mixed.hip", "pack_single.hip", "mask_ops.hip", "maxpool.hip",
+           "linear_gw.hip", "misc.hip", "calc_precision.cpp"]
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-ffp-contract=off",                      # bit-exact quantiser: no implicit FMA
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",   # no packed-FP32 codegen
+    "-Wno-unused-command-line-argument",
+]
+
+c_i64, c_i32, c_u64, c_vp = ctypes.c_int64, ctypes.c_int, ctypes.c_uint64, ctypes.c_void_p
+
+# name -> argtypes (restype is int unless listed in _RESTYPES); mirrors include/actnn_hip.h
+SIGNATURES = {
+    "actnn_strerror": [c_i32],
+    "actnn_version": [],
+    "actnn_minimax": [c_vp, c_vp, c_vp, c_i64, c_i64, c_i32, c_vp],
+    "actnn_bits_prefix": [c_vp, c_vp, c_i64, c_vp],
+    "actnn_pack_mixed": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u64, c_u64,
+                         c_i64, c_i64, c_i64, c_i32, c_vp],
+    "actnn_unpack_mixed": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i32, c_vp],
+    "actnn_pack_single": [c_vp, c_vp, c_vp, c_i32, c_vp, c_vp, c_vp, c_u64, c_u64,
+                          c_i64, c_i64, c_i64, c_i32, c_vp],
+    "actnn_unpack_single": [c_vp, c_i32, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i32, c_vp],
+    "actnn_relu_forward": [c_vp, c_vp, c_vp, c_i64, c_i32, c_vp],
+    "actnn_relu_backward": [c_vp, c_vp, c_vp, c_i64, c_i32, c_vp],
+    "actnn_dropout_forward": [c_vp, c_vp, c_vp, c_i64, ctypes.c_float, c_u64, c_u64, c_i32, c_vp],
+    "actnn_dropout_backward": [c_vp, c_vp, c_vp, c_i64, ctypes.c_float, c_i32, c_vp],
+    "actnn_max_pool2d_forward": [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
+                                 c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
+    "actnn_max_pool2d_backward": [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
+                                  c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
+    "actnn_calc_precision": [c_vp, c_vp, c_vp, c_i64, ctypes.c_double],
+    "actnn_linear_grad_weight_q2": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64,
+                                    c_i32, c_i32, c_i32, c_vp],
+    "actnn_stream_copy": [c_vp, c_vp, c_i64, c_vp],
+}
+_RESTYPES = {"actnn_strerror": ctypes.c_char_p, "actnn_version": ctypes.c_char_p}
+
+_lib = None
+
+
+def build(verbose=False):
+    """Compile every source under csrc/ into libactnn_hip.so (always recompiles)."""
+    srcs = [os.path.join(CSRC, s) for s in SOURCES]
+    tmp = LIB_PATH + ".tmp"
+    cmd = ["hipcc", *HIPCC_FLAGS, *srcs, "-o", tmp]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    os.replace(tmp, LIB_PATH)
+    global _lib
+    _lib = None
+    return LIB_PATH
+
+
+def load():
+    """Load the library (once) and attach argument types.  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: the HIP kernels are not built. Run "
+            "`python -c 'import __graft_entry__ as g; g.build()'` (needs hipcc). "
+            "There is no CPU fallback.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)            # AttributeError if the header and library disagree
+        fn.argtypes = argtypes
+        fn.restype = _RESTYPES.get(name, ctypes.c_int)
+    _lib = lib
+    return lib
+
+
+def check(rc, what):
+    """Turn a non-zero return code into RuntimeError (the reference raises c10::Error ->
+    RuntimeError from TORCH_CHECK, ext_common.h)."""
+    if rc != 0:
+        msg = load().actnn_strerror(int(rc)).decode()
+        raise RuntimeError(f"{what} failed: {msg} (code {rc})")

@@ -1,0 +1,337 @@
+"""Operators of the reference's ``actnn.cpp_extension.quantization`` module
+(cpp_extension/quantization.cc:198-206), same names and positional arguments, running the
+gfx950 kernels through the C ABI.  Extras that the reference does not have are keyword-only:
+``noise=`` (deterministic mode) on the two pack functions.
+"""
+import torch
+from torch.autograd import Function
+
+from . import _glue as g
+from .._lib import check
+
+MASK_BLOCK = 512
+
+
+# ------------------------------------------------------------------------------------------
+# per-sample bit widths: host copy, total and device prefix sums travel with the tensor
+# ------------------------------------------------------------------------------------------
+def attach_bits_host(bits_dev, bits_host):
+    """Remember the host copy of a device ``bits`` tensor so that pack/unpack need no
+    device->host sync (the reference syncs twice per pack: .cu:92, :98)."""
+    bits_dev._actnn_host = bits_host
+    return bits_dev
+
+
+def _bits_info(bits):
+    """(sum(bits), device exclusive prefix [N+1]) of an int32 device tensor, cached on it."""
+    cached = getattr(bits, "_actnn_info", None)
+    if cached is not None:
+        return cached
+    host = getattr(bits, "_actnn_host", None)
+    if host is None:
+        host = bits.cpu()                              # sync, like the reference's .item() calls
+    if host.numel() and (int(host.min()) < 1 or int(host.max()) > 8):
+        raise RuntimeError("pack_mixed_precision supports 1..8 bits per sample")
+    total = int(host.sum())
+    N = bits.numel()
+    prefix = torch.empty(N + 1, dtype=torch.int32, device=bits.device)
+    with torch.cuda.device(bits.device):
+        check(g.lib().actnn_bits_prefix(bits.data_ptr(), prefix.data_ptr(), N,
+                                        g.stream_ptr(bits.device)), "bits_prefix")
+    bits._actnn_info = (total, prefix)
+    return bits._actnn_info
+
+
+# ------------------------------------------------------------------------------------------
+# pack / unpack, mixed precision  (quantization.cc:46-73)
+# ------------------------------------------------------------------------------------------
+def pack_mixed_precision(data, min, max, bits, stochastic, *, noise=None):
+    g.check_float(data, "data", 3)
+    g.check_float(min, "min", 3)
+    g.check_float(max, "max", 3)
+    g.check_typed(bits, "bits", torch.int32, 1)
+    if not stochastic:
+        raise RuntimeError("pack_mixed_precision: stochastic must be true")      # .cu:122
+    N, G, gs = data.shape
+    if gs % 32 != 0:
+        raise RuntimeError("group_size must be a multiple of 32")                  # .cu:94
+    if min.dtype != data.dtype or max.dtype != data.dtype:
+        raise RuntimeError("The type of min/max is not correct!")
+    if min.numel() != N * G or max.numel() != N * G or bits.numel() != N:
+        raise RuntimeError("pack_mixed_precision: shape mismatch")
+    if noise is not None:
+        g.check_float(noise, "noise", 3)
+        if noise.shape != data.shape or noise.dtype != data.dtype:
+            raise RuntimeError("noise must match data in shape and dtype")
+        noise = g.aligned(noise)
+    data = g.aligned(data)
+    total, prefix = _bits_info(bits)
+    n_words = (total * G * gs + 31) // 32                                          # .cu:98-100
+    packed = torch.empty(n_words, dtype=torch.int32, device=data.device)
+    scale = torch.empty(N, G, 1, dtype=data.dtype, device=data.device)
+    seed, offset = (0, 0) if noise is not None else g.philox_args(data.device)
+    with torch.cuda.device(data.device):
+        check(g.lib().actnn_pack_mixed(
+            data.data_ptr(), min.data_ptr(), max.data_ptr(), bits.data_ptr(), prefix.data_ptr(),
+            scale.data_ptr(), packed.data_ptr(), noise.data_ptr() if noise is not None else None,
+            seed, offset, N, G, gs, g.DTYPE_CODE[data.dtype], g.stream_ptr(data.device)),
+            "pack_mixed_precision")
+    return packed, scale
+
+
+def unpack_mixed_precision(data, bits, scale, min, N, num_groups, group_size):
+    g.check_typed(data, "data", torch.int32, 1)
+    g.check_typed(bits, "bits", torch.int32, 1)
+    g.check_float(scale, "scale", 3)
+    g.check_float(min, "min", 3)
+    if group_size % 32 != 0:
+        raise RuntimeError("group_size must be a multiple of 32")                  # .cu:186
+    if min.dtype != scale.dtype:
+        raise RuntimeError("The type of min is not correct!")
+    if scale.numel() != N * num_groups or min.numel() != N * num_groups or bits.numel() != N:
+        raise RuntimeError("unpack_mixed_precision: shape mismatch")
+    total, prefix = _bits_info(bits)
+    if data.numel() < (total * num_groups * group_size + 31) // 32:
+        raise RuntimeError("unpack_mixed_precision: packed stream is too short")
+    out = torch.empty(N, num_groups, group_size, dtype=scale.dtype, device=data.device)
+    with torch.cuda.device(data.device):
+        check(g.lib().actnn_unpack_mixed(
+            data.data_ptr(), bits.data_ptr(), prefix.data_ptr(), scale.data_ptr(), min.data_ptr(),
+            out.data_ptr(), N, num_groups, group_size, g.DTYPE_CODE[scale.dtype],
+            g.stream_ptr(data.device)), "unpack_mixed_precision")
+    return out
+
+
+# ------------------------------------------------------------------------------------------
+# pack / unpack, single precision  (quantization.cc:77-102)
+# ------------------------------------------------------------------------------------------
+def single_packed_bytes(N, G, gs, bits):
+    wpt = 8 // bits
+    n_round = N + (wpt - N % wpt) % wpt                                            # .cu:274
+    return (bits * n_round * G * gs + 8) // 8                                      # .cu:275-277
+
+
+def pack_single_precision(data, min, max, bits, stochastic, *, noise=None):
+    g.check_float(data, "data", 3)
+    g.check_float(min, "min", 3)
+    g.check_float(max, "max", 3)
+    bits = int(bits)
+    if bits < 1 or 8 % bits != 0:
+        raise RuntimeError("pack_single_precision: 8 % bits must be 0")            # .cu:272
+    if not stochastic:
+        raise RuntimeError("pack_single_precision: stochastic must be true")     # .cu:298
+    N, G, gs = data.shape
+    if gs % 8 != 0:
+        raise RuntimeError("group_size must be a multiple of 8")
+    if min.dtype != data.dtype or max.dtype != data.dtype:
+        raise RuntimeError("The type of min/max is not correct!")
+    if min.numel() != N * G or max.numel() != N * G:
+        raise RuntimeError("pack_single_precision: shape mismatch")
+    if noise is not None:
+        g.check_float(noise, "noise", 3)
+        if noise.shape != data.shape or noise.dtype != data.dtype:
+            raise RuntimeError("noise must match data in shape and dtype")
+        noise = g.aligned(noise)
+    data = g.aligned(data)
+    packed = torch.empty(single_packed_bytes(N, G, gs, bits), dtype=torch.int8, device=data.device)
+    scale = torch.empty(N, G, 1, dtype=data.dtype, device=data.device)
+    wpt = 8 // bits
+    seed, offset = (0, 0) if noise is not None else g.philox_args(data.device)
+    with torch.cuda.device(data.device):
+        check(g.lib().actnn_pack_single(
+            data.data_ptr(), min.data_ptr(), max.data_ptr(), bits, scale.data_ptr(),
+            packed.data_ptr(), noise.data_ptr() if noise is not None else None, seed, offset,
+            N, G, gs, g.DTYPE_CODE[data.dtype], g.stream_ptr(data.device)), "pack_single_precision")
+    del wpt
+    return packed, scale
+
+
+def unpack_single_precision(data, bits, scale, min, N, num_groups, group_size):
+    g.check_typed(data, "data", torch.int8, 1)
+    g.check_float(scale, "scale", 3)
+    g.check_float(min, "min", 3)
+    bits = int(bits)
+    if bits < 1 or 8 % bits != 0:
+        raise RuntimeError("unpack_single_precision: 8 % bits must be 0")          # .cu:375
+    if min.dtype != scale.dtype:
+        raise RuntimeError("The type of min is not correct!")
+    if scale.numel() != N * num_groups or min.numel() != N * num_groups:
+        raise RuntimeError("unpack_single_precision: shape mismatch")
+    if data.numel() < single_packed_bytes(N, num_groups, group_size, bits) - 1:
+        raise RuntimeError("unpack_single_precision: packed stream is too short")
+    out = torch.empty(N, num_groups, group_size, dtype=scale.dtype, device=data.device)
+    with torch.cuda.device(data.device):
+        check(g.lib().actnn_unpack_single(
+            data.data_ptr(), bits, scale.data_ptr(), min.data_ptr(), out.data_ptr(), N, num_groups,
+            group_size, g.DTYPE_CODE[scale.dtype], g.stream_ptr(data.device)),
+            "unpack_single_precision")
+    return out
+
+
+# ------------------------------------------------------------------------------------------
+# ReLU / Dropout with 1-bit masks  (quantization.cc:106-148)
+# ------------------------------------------------------------------------------------------
+def mask_words(n):
+    """int32 words of the mask of ``n`` elements: 16 per block of 512 elements.  Equals the
+    reference's ceil(n/32) when n % 512 == 0; its tail block writes 16 words regardless
+    (.cu:441-443), so the whole block is allocated here."""
+    return (n + MASK_BLOCK - 1) // MASK_BLOCK * 16
+
+
+def relu_forward(x):
+    x = g.aligned(x)
+    n = x.numel()
+    y = torch.empty_like(x)
+    mask = torch.empty(mask_words(n), dtype=torch.int32, device=x.device)
+    with torch.cuda.device(x.device):
+        check(g.lib().actnn_relu_forward(x.data_ptr(), y.data_ptr(), mask.data_ptr(), n,
+                                         g.DTYPE_CODE[x.dtype], g.stream_ptr(x.device)), "relu_forward")
+    return y, mask
+
+
+def relu_backward(grad_output, mask):
+    grad_output = g.aligned(grad_output.contiguous())
+    gin = torch.empty_like(grad_output)
+    with torch.cuda.device(gin.device):
+        check(g.lib().actnn_relu_backward(grad_output.data_ptr(), mask.data_ptr(), gin.data_ptr(),
+                                          gin.numel(), g.DTYPE_CODE[gin.dtype],
+                                          g.stream_ptr(gin.device)), "relu_backward")
+    return gin
+
+
+class ActQuantizedReLU(Function):
+    """quantization.cc:106-119: saves only the 1-bit mask."""
+
+    @staticmethod
+    def forward(ctx, input):
+        output, mask = relu_forward(input)
+        ctx.save_for_backward(mask)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (mask,) = ctx.saved_tensors
+        return relu_backward(grad_output, mask)
+
+
+def act_quantized_relu(input):
+    g.check_float(input, "input")                                                  # quantization.cc:122
+    return ActQuantizedReLU.apply(input)
+
+
+def dropout_forward(x, p):
+    x = g.aligned(x)
+    n = x.numel()
+    y = torch.empty_like(x)
+    mask = torch.empty(mask_words(n), dtype=torch.int32, device=x.device)
+    seed, offset = g.philox_args(x.device)
+    with torch.cuda.device(x.device):
+        check(g.lib().actnn_dropout_forward(x.data_ptr(), y.data_ptr(), mask.data_ptr(), n, float(p),
+                                            seed, offset, g.DTYPE_CODE[x.dtype],
+                                            g.stream_ptr(x.device)), "dropout_forward")
+    return y, mask
+
+
+def dropout_backward(grad_output, mask, p):
+    grad_output = g.aligned(grad_output.contiguous())
+    gin = torch.empty_like(grad_output)
+    with torch.cuda.device(gin.device):
+        check(g.lib().actnn_dropout_backward(grad_output.data_ptr(), mask.data_ptr(), gin.data_ptr(),
+                                             gin.numel(), float(p), g.DTYPE_CODE[gin.dtype],
+                                             g.stream_ptr(gin.device)), "dropout_backward")
+    return gin
+
+
+class ActQuantizedDropout(Function):
+    """quantization.cc:128-143."""
+
+    @staticmethod
+    def forward(ctx, input, dropout_p):
+        output, mask = dropout_forward(input, dropout_p)
+        ctx.save_for_backward(mask)
+        ctx.dropout_p = float(dropout_p)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (mask,) = ctx.saved_tensors
+        return dropout_backward(grad_output, mask, ctx.dropout_p), None
+
+
+def act_quantized_dropout(input, dropout_p):
+    g.check_float(input, "input")                                                  # quantization.cc:146
+    return ActQuantizedDropout.apply(input, dropout_p)
+
+
+# ------------------------------------------------------------------------------------------
+# MaxPool2d with int8 arg-max indices  (quantization.cc:152-196)
+# ------------------------------------------------------------------------------------------
+def _pair_check(v, name):
+    v = [int(a) for a in v]
+    if len(v) != 2:
+        raise RuntimeError(f"{name} must have 2 elements")                        # quantization.cc:156-159
+    return v
+
+
+def max_pool2d_forward(x, kernel_size, stride, padding, dilation):
+    N, C, H, W = x.shape
+    KH, KW = kernel_size
+    Ho = (H + 2 * padding[0] - dilation[0] * (KH - 1) - 1) // stride[0] + 1       # .cu:679
+    Wo = (W + 2 * padding[1] - dilation[1] * (KW - 1) - 1) // stride[1] + 1       # .cu:680
+    y = torch.empty(N, C, Ho, Wo, dtype=x.dtype, device=x.device)
+    idx = torch.empty(N, C, Ho, Wo, dtype=torch.int8, device=x.device)
+    with torch.cuda.device(x.device):
+        check(g.lib().actnn_max_pool2d_forward(
+            x.data_ptr(), y.data_ptr(), idx.data_ptr(), N, C, H, W, Ho, Wo, KH, KW, stride[0],
+            stride[1], padding[0], padding[1], g.DTYPE_CODE[x.dtype], g.stream_ptr(x.device)),
+            "max_pool2d_forward")
+    return y, idx
+
+
+def max_pool2d_backward(grad_output, idx, input_shape, kernel_size, stride, padding):
+    grad_output = grad_output.contiguous()
+    N, C, H, W = input_shape
+    Ho, Wo = grad_output.shape[2], grad_output.shape[3]
+    gin = torch.empty(N, C, H, W, dtype=grad_output.dtype, device=grad_output.device)
+    with torch.cuda.device(gin.device):
+        check(g.lib().actnn_max_pool2d_backward(
+            grad_output.data_ptr(), idx.data_ptr(), gin.data_ptr(), N, C, H, W, Ho, Wo,
+            kernel_size[0], kernel_size[1], stride[0], stride[1], padding[0], padding[1],
+            g.DTYPE_CODE[gin.dtype], g.stream_ptr(gin.device)), "max_pool2d_backward")
+    return gin
+
+
+class ActQuantizedMaxPool2d(Function):
+    """quantization.cc:152-191."""
+
+    @staticmethod
+    def forward(ctx, input, kernel_size, stride, padding, dilation, ceil_mode, return_indices):
+        kernel_size = _pair_check(kernel_size, "kernel_size")
+        stride = _pair_check(stride, "stride")
+        padding = _pair_check(padding, "padding")
+        dilation = _pair_check(dilation, "dilation")
+        if ceil_mode:
+            raise RuntimeError("Do not support ceil_mode")                         # .cu:684
+        if return_indices:
+            raise RuntimeError("Do not support return_indices")                    # .cu:685
+        if kernel_size[0] * kernel_size[1] >= 16:
+            raise RuntimeError("kernel_size[0] * kernel_size[1] must be < 16")    # quantization.cc:162
+        if input.dim() != 4:
+            raise RuntimeError("The dimension of input is not correct!")
+        output, idx = max_pool2d_forward(input, kernel_size, stride, padding, dilation)
+        ctx.save_for_backward(idx)
+        ctx.geom = (tuple(input.shape), kernel_size, stride, padding)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (idx,) = ctx.saved_tensors
+        shape, kernel_size, stride, padding = ctx.geom
+        gin = max_pool2d_backward(grad_output, idx, shape, kernel_size, stride, padding)
+        return gin, None, None, None, None, None, None
+
+
+def act_quantized_max_pool2d(input, kernel_size, stride, padding, dilation, ceil_mode, return_indices):
+    g.check_float(input, "input")                                                  # quantization.cc:194
+    return ActQuantizedMaxPool2d.apply(input, kernel_size, stride, padding, dilation, ceil_mode,
+                                       return_indices)

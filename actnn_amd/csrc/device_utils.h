@@ -1,0 +1,197 @@
+// Device-side helpers shared by the gfx950 kernels: typed 128-bit loads/stores,
+// cross-lane exchange (DPP / ds_swizzle), the 32x32 bit transpose that turns per-lane code
+// bits into the reference's ballot-style words, and Philox4x32-10.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "../../include/actnn_hip.h"
+
+namespace actnn {
+
+struct bf16_t { uint16_t bits; };   // raw bfloat16 storage
+
+#define ACTNN_DEV __device__ __forceinline__
+
+// ------------------------------------------------------------------ scalar conversions
+ACTNN_DEV float bf16_bits_to_float(uint32_t b) { return __builtin_bit_cast(float, b << 16); }
+ACTNN_DEV uint32_t float_to_bf16_bits(float f) {           // round to nearest even
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;   // quiet NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+ACTNN_DEV float half_bits_to_float(uint32_t b) {
+  return __half2float(__builtin_bit_cast(__half, (uint16_t)b));
+}
+ACTNN_DEV uint32_t float_to_half_bits(float f) {
+  return __builtin_bit_cast(uint16_t, __float2half_rn(f));
+}
+
+template <typename T> struct Conv;
+template <> struct Conv<float> {
+  static constexpr int kBytes = 4;
+  static ACTNN_DEV float load(const float* p, int64_t i) { return p[i]; }
+  static ACTNN_DEV void store(float* p, int64_t i, float v) { p[i] = v; }
+  static ACTNN_DEV float round(float v) { return v; }
+};
+template <> struct Conv<__half> {
+  static constexpr int kBytes = 2;
+  static ACTNN_DEV float load(const __half* p, int64_t i) { return __half2float(p[i]); }
+  static ACTNN_DEV void store(__half* p, int64_t i, float v) { p[i] = __float2half_rn(v); }
+  static ACTNN_DEV float round(float v) { return __half2float(__float2half_rn(v)); }
+};
+template <> struct Conv<bf16_t> {
+  static constexpr int kBytes = 2;
+  static ACTNN_DEV float load(const bf16_t* p, int64_t i) { return bf16_bits_to_float(p[i].bits); }
+  static ACTNN_DEV void store(bf16_t* p, int64_t i, float v) { p[i].bits = (uint16_t)float_to_bf16_bits(v); }
+  static ACTNN_DEV float round(float v) { return bf16_bits_to_float(float_to_bf16_bits(v)); }
+};
+
+// ------------------------------------------------------------------ 8 / 16 contiguous elements
+// load8: 8 consecutive elements starting at p (32-byte aligned for f32, 16 for 16-bit types).
+ACTNN_DEV void load8(const float* p, float (&v)[8]) {
+  const float4 a = reinterpret_cast<const float4*>(p)[0];
+  const float4 b = reinterpret_cast<const float4*>(p)[1];
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+ACTNN_DEV void load8(const __half* p, float (&v)[8]) {
+  const uint4 a = reinterpret_cast<const uint4*>(p)[0];
+  const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = half_bits_to_float(w[i] & 0xffffu);
+    v[2 * i + 1] = half_bits_to_float(w[i] >> 16);
+  }
+}
+ACTNN_DEV void load8(const bf16_t* p, float (&v)[8]) {
+  const uint4 a = reinterpret_cast<const uint4*>(p)[0];
+  const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = __builtin_bit_cast(float, w[i] << 16);
+    v[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xffff0000u);
+  }
+}
+ACTNN_DEV void store8(float* p, const float (&v)[8]) {
+  reinterpret_cast<float4*>(p)[0] = make_float4(v[0], v[1], v[2], v[3]);
+  reinterpret_cast<float4*>(p)[1] = make_float4(v[4], v[5], v[6], v[7]);
+}
+ACTNN_DEV void store8(__half* p, const float (&v)[8]) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = float_to_half_bits(v[2 * i]) | (float_to_half_bits(v[2 * i + 1]) << 16);
+  reinterpret_cast<uint4*>(p)[0] = make_uint4(w[0], w[1], w[2], w[3]);
+}
+ACTNN_DEV void store8(bf16_t* p, const float (&v)[8]) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = float_to_bf16_bits(v[2 * i]) | (float_to_bf16_bits(v[2 * i + 1]) << 16);
+  reinterpret_cast<uint4*>(p)[0] = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// ------------------------------------------------------------------ cross-lane exchange
+// Value held by lane (lane ^ D), D in {1, 2, 4, 8, 16}.  1/2/8 are DPP moves, 4/16 go
+// through ds_swizzle (LDS crossbar, no memory), so they do not take a VALU slot.
+template <int D> ACTNN_DEV uint32_t lane_xor(uint32_t x);
+template <> ACTNN_DEV uint32_t lane_xor<1>(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, false);   // quad_perm [1,0,3,2]
+}
+template <> ACTNN_DEV uint32_t lane_xor<2>(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, false);   // quad_perm [2,3,0,1]
+}
+template <> ACTNN_DEV uint32_t lane_xor<4>(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_ds_swizzle((int)x, 0x101F);                      // xor 4
+}
+template <> ACTNN_DEV uint32_t lane_xor<8>(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x128, 0xF, 0xF, false);  // row_ror:8
+}
+template <> ACTNN_DEV uint32_t lane_xor<16>(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_ds_swizzle((int)x, 0x401F);                      // xor 16
+}
+
+template <int S> ACTNN_DEV uint32_t transpose_stage(uint32_t x, uint32_t lane) {
+  constexpr uint32_t M = S == 16 ? 0xFFFF0000u : S == 8 ? 0xFF00FF00u : S == 4 ? 0xF0F0F0F0u
+                       : S == 2 ? 0xCCCCCCCCu : 0xAAAAAAAAu;
+  const uint32_t p = lane_xor<S>(x);
+  const bool hi = (lane & S) != 0;
+  const uint32_t u = __builtin_amdgcn_alignbit(p, p, hi ? S : 32 - S);   // hi: p >> S, lo: p << S (rotations)
+  const uint32_t sel = hi ? M : ~M;
+  return (x & sel) | (u & ~sel);
+}
+
+// 32x32 bit transpose inside each 32-lane half of the wave: afterwards bit j of lane p is
+// what bit p of lane j was.  `lane` is the lane index (any value congruent mod 32).
+ACTNN_DEV uint32_t transpose32(uint32_t x, uint32_t lane) {
+  x = transpose_stage<16>(x, lane);
+  x = transpose_stage<8>(x, lane);
+  x = transpose_stage<4>(x, lane);
+  x = transpose_stage<2>(x, lane);
+  x = transpose_stage<1>(x, lane);
+  return x;
+}
+
+// Reductions over a DPP row (16 consecutive lanes); every lane ends with the result.
+ACTNN_DEV float row16_max(float v) {
+  v = fmaxf(v, __builtin_bit_cast(float, lane_xor<1>(__builtin_bit_cast(uint32_t, v))));
+  v = fmaxf(v, __builtin_bit_cast(float, lane_xor<2>(__builtin_bit_cast(uint32_t, v))));
+  v = fmaxf(v, __builtin_bit_cast(float, (uint32_t)__builtin_amdgcn_update_dpp(
+                   0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false)));   // row_half_mirror
+  v = fmaxf(v, __builtin_bit_cast(float, (uint32_t)__builtin_amdgcn_update_dpp(
+                   0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false)));   // row_mirror
+  return v;
+}
+ACTNN_DEV float row16_min(float v) {
+  v = fminf(v, __builtin_bit_cast(float, lane_xor<1>(__builtin_bit_cast(uint32_t, v))));
+  v = fminf(v, __builtin_bit_cast(float, lane_xor<2>(__builtin_bit_cast(uint32_t, v))));
+  v = fminf(v, __builtin_bit_cast(float, (uint32_t)__builtin_amdgcn_update_dpp(
+                   0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false)));
+  v = fminf(v, __builtin_bit_cast(float, (uint32_t)__builtin_amdgcn_update_dpp(
+                   0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false)));
+  return v;
+}
+
+// ------------------------------------------------------------------ Philox4x32-10
+struct Philox4 { uint32_t x, y, z, w; };
+
+ACTNN_DEV Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
+                                uint32_t k0, uint32_t k1) {
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+    const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    c1 = (uint32_t)p1;
+    c3 = (uint32_t)p0;
+    c0 = n0;
+    c2 = n2;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  return Philox4{c0, c1, c2, c3};
+}
+
+// The eight 16-bit noises of the octet of elements [8*o, 8*o + 8): element k uses the
+// (k & 1)-th half (low first) of output word k >> 1.
+ACTNN_DEV void philox_octet(uint64_t octet, uint64_t seed, uint64_t offset, uint32_t (&r16)[8]) {
+  const Philox4 r = philox4x32_10((uint32_t)octet, (uint32_t)(octet >> 32), (uint32_t)offset,
+                                  (uint32_t)(offset >> 32), (uint32_t)seed, (uint32_t)(seed >> 32));
+  r16[0] = r.x & 0xffffu; r16[1] = r.x >> 16;
+  r16[2] = r.y & 0xffffu; r16[3] = r.y >> 16;
+  r16[4] = r.z & 0xffffu; r16[5] = r.z >> 16;
+  r16[6] = r.w & 0xffffu; r16[7] = r.w >> 16;
+}
+
+// ------------------------------------------------------------------ host-side helpers
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+#define ACTNN_RETURN_LAUNCH_STATUS()                       \
+  do {                                                     \
+    hipError_t e_ = hipGetLastError();                     \
+    return e_ == hipSuccess ? ACTNN_OK : (int)e_;          \
+  } while (0)
+
+}  // namespace actnn

@@ -1,0 +1,205 @@
+// ReLU and Dropout with 1-bit masks (replaces quantization_cuda_kernel.cu:411-627).
+//
+// Mask layout (kept from the reference): elements are cut into blocks of 512; element
+// t = 16*j + k of a block is bit j of the block's word k (16 int32 words per block).  Lane j
+// of a 32-lane half-wave therefore owns 16 contiguous elements; two blocks fill a 32-bit
+// register per lane and one 32x32 bit transpose leaves the 32 mask words of the two blocks in
+// lanes 0..31, stored as one contiguous 128-byte run.  A 256-thread block covers 16 mask
+// blocks (8192 elements).
+#include "device_utils.h"
+
+namespace actnn {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kMaskBlock = 512;
+constexpr int kMaskBlocksPerBlock = (kThreads / 32) * 2;   // 16
+
+enum class Op { kRelu, kDropout };
+
+// Forward.  OP selects the keep rule: x > 0 (ReLU) or Philox r16 >= threshold (Dropout).
+template <typename T, Op OP>
+__global__ __launch_bounds__(kThreads) void mask_forward_kernel(const T* __restrict__ x,
+                                                                T* __restrict__ y,
+                                                                int32_t* __restrict__ mask, int64_t n,
+                                                                int64_t n_mask_blocks, uint32_t thr,
+                                                                float keep_div, uint64_t seed,
+                                                                uint64_t offset) {
+  const uint32_t lane = threadIdx.x & 31;
+  const int64_t mb0 = (int64_t)blockIdx.x * kMaskBlocksPerBlock + (threadIdx.x >> 5) * 2;
+  uint32_t acc = 0;
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const int64_t e0 = (mb0 + r) * kMaskBlock + lane * 16;
+    if (e0 >= n) continue;
+    float v[16];
+    const bool full = e0 + 16 <= n;
+    if (full) {
+      load8(x + e0, reinterpret_cast<float(&)[8]>(v[0]));
+      load8(x + e0 + 8, reinterpret_cast<float(&)[8]>(v[8]));
+    } else {
+#pragma unroll
+      for (int k = 0; k < 16; ++k) v[k] = e0 + k < n ? Conv<T>::load(x, e0 + k) : 0.0f;
+    }
+    uint32_t bitsr = 0;
+    if (OP == Op::kRelu) {
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const bool keep = v[k] > 0.0f;
+        v[k] = keep ? v[k] : 0.0f;
+        bitsr |= (uint32_t)keep << k;
+      }
+    } else {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        uint32_t r16[8];
+        philox_octet((uint64_t)(e0 >> 3) + h, seed, offset, r16);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const bool keep = r16[k] >= thr && e0 + h * 8 + k < n;
+          v[h * 8 + k] = keep ? v[h * 8 + k] / keep_div : 0.0f;
+          bitsr |= (uint32_t)keep << (h * 8 + k);
+        }
+      }
+    }
+    acc |= bitsr << (16 * r);
+    if (full) {
+      store8(y + e0, reinterpret_cast<const float(&)[8]>(v[0]));
+      store8(y + e0 + 8, reinterpret_cast<const float(&)[8]>(v[8]));
+    } else {
+#pragma unroll
+      for (int k = 0; k < 16; ++k)
+        if (e0 + k < n) Conv<T>::store(y, e0 + k, v[k]);
+    }
+  }
+  const uint32_t w = transpose32(acc, lane);       // lane p: word p % 16 of mask block mb0 + p / 16
+  if (mb0 + (lane >> 4) < n_mask_blocks) mask[mb0 * 16 + lane] = (int32_t)w;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void mask_backward_kernel(const T* __restrict__ gout,
+                                                                 const int32_t* __restrict__ mask,
+                                                                 T* __restrict__ gin, int64_t n,
+                                                                 int64_t n_mask_blocks, float keep_div,
+                                                                 bool divide) {
+  const uint32_t lane = threadIdx.x & 31;
+  const int64_t mb0 = (int64_t)blockIdx.x * kMaskBlocksPerBlock + (threadIdx.x >> 5) * 2;
+  uint32_t w = 0;
+  if (mb0 + (lane >> 4) < n_mask_blocks) w = (uint32_t)mask[mb0 * 16 + lane];
+  const uint32_t acc = transpose32(w, lane);       // bits 16*r + k: keep flag of element 16*lane + k of block r
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const int64_t e0 = (mb0 + r) * kMaskBlock + lane * 16;
+    if (e0 >= n) continue;
+    float v[16];
+    const bool full = e0 + 16 <= n;
+    if (full) {
+      load8(gout + e0, reinterpret_cast<float(&)[8]>(v[0]));
+      load8(gout + e0 + 8, reinterpret_cast<float(&)[8]>(v[8]));
+    } else {
+#pragma unroll
+      for (int k = 0; k < 16; ++k) v[k] = e0 + k < n ? Conv<T>::load(gout, e0 + k) : 0.0f;
+    }
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const bool keep = (acc >> (16 * r + k)) & 1u;
+      v[k] = keep ? (divide ? v[k] / keep_div : v[k]) : 0.0f;
+    }
+    if (full) {
+      store8(gin + e0, reinterpret_cast<const float(&)[8]>(v[0]));
+      store8(gin + e0 + 8, reinterpret_cast<const float(&)[8]>(v[8]));
+    } else {
+#pragma unroll
+      for (int k = 0; k < 16; ++k)
+        if (e0 + k < n) Conv<T>::store(gin, e0 + k, v[k]);
+    }
+  }
+}
+
+template <typename T, Op OP>
+int launch_forward(const void* x, void* y, int32_t* mask, int64_t n, uint32_t thr, float keep_div,
+                   uint64_t seed, uint64_t offset, hipStream_t s) {
+  const int64_t nmb = (n + kMaskBlock - 1) / kMaskBlock;
+  const int64_t blocks = (nmb + kMaskBlocksPerBlock - 1) / kMaskBlocksPerBlock;
+  if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
+  mask_forward_kernel<T, OP><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+      static_cast<const T*>(x), static_cast<T*>(y), mask, n, nmb, thr, keep_div, seed, offset);
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
+
+template <typename T>
+int launch_backward(const void* gout, const int32_t* mask, void* gin, int64_t n, float keep_div,
+                    bool divide, hipStream_t s) {
+  const int64_t nmb = (n + kMaskBlock - 1) / kMaskBlock;
+  const int64_t blocks = (nmb + kMaskBlocksPerBlock - 1) / kMaskBlocksPerBlock;
+  if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
+  mask_backward_kernel<T><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+      static_cast<const T*>(gout), mask, static_cast<T*>(gin), n, nmb, keep_div, divide);
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
+
+template <Op OP>
+int dispatch_forward(const void* x, void* y, int32_t* mask, int64_t n, uint32_t thr, float keep_div,
+                     uint64_t seed, uint64_t offset, int dtype, void* stream) {
+  if (n < 0) return ACTNN_EINVAL;
+  if (n == 0) return ACTNN_OK;
+  if (!x || !y || !mask) return ACTNN_EINVAL;
+  if (!aligned16(x) || !aligned16(y)) return ACTNN_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case ACTNN_F32: return launch_forward<float, OP>(x, y, mask, n, thr, keep_div, seed, offset, s);
+    case ACTNN_F16: return launch_forward<__half, OP>(x, y, mask, n, thr, keep_div, seed, offset, s);
+    case ACTNN_BF16: return launch_forward<bf16_t, OP>(x, y, mask, n, thr, keep_div, seed, offset, s);
+    default: return ACTNN_EDTYPE;
+  }
+}
+
+int dispatch_backward(const void* gout, const int32_t* mask, void* gin, int64_t n, float keep_div,
+                      bool divide, int dtype, void* stream) {
+  if (n < 0) return ACTNN_EINVAL;
+  if (n == 0) return ACTNN_OK;
+  if (!gout || !gin || !mask) return ACTNN_EINVAL;
+  if (!aligned16(gout) || !aligned16(gin)) return ACTNN_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case ACTNN_F32: return launch_backward<float>(gout, mask, gin, n, keep_div, divide, s);
+    case ACTNN_F16: return launch_backward<__half>(gout, mask, gin, n, keep_div, divide, s);
+    case ACTNN_BF16: return launch_backward<bf16_t>(gout, mask, gin, n, keep_div, divide, s);
+    default: return ACTNN_EDTYPE;
+  }
+}
+
+// keep iff r16 >= thr, r16 uniform on [0, 2^16): P(keep) = 1 - thr / 2^16 ~ 1 - p.
+inline uint32_t dropout_threshold(float p) {
+  double t = (double)p * 65536.0;
+  t = t < 0.0 ? 0.0 : (t > 65536.0 ? 65536.0 : t);
+  return (uint32_t)(t + 0.5);
+}
+
+}  // namespace
+}  // namespace actnn
+
+extern "C" int actnn_relu_forward(const void* x, void* y, int32_t* mask, int64_t n, int dtype,
+                                  void* stream) {
+  return actnn::dispatch_forward<actnn::Op::kRelu>(x, y, mask, n, 0u, 1.0f, 0, 0, dtype, stream);
+}
+
+extern "C" int actnn_relu_backward(const void* grad_out, const int32_t* mask, void* grad_in,
+                                   int64_t n, int dtype, void* stream) {
+  return actnn::dispatch_backward(grad_out, mask, grad_in, n, 1.0f, false, dtype, stream);
+}
+
+extern "C" int actnn_dropout_forward(const void* x, void* y, int32_t* mask, int64_t n, float p,
+                                     uint64_t seed, uint64_t offset, int dtype, void* stream) {
+  if (!(p >= 0.0f && p <= 1.0f)) return ACTNN_EINVAL;
+  const float keep_div = (float)(1.0 - (double)p);     // x / (1.0 - p), .cu:540
+  return actnn::dispatch_forward<actnn::Op::kDropout>(x, y, mask, n, actnn::dropout_threshold(p),
+                                                      keep_div, seed, offset, dtype, stream);
+}
+
+extern "C" int actnn_dropout_backward(const void* grad_out, const int32_t* mask, void* grad_in,
+                                      int64_t n, float p, int dtype, void* stream) {
+  if (!(p >= 0.0f && p <= 1.0f)) return ACTNN_EINVAL;
+  const float keep_div = (float)(1.0 - (double)p);     // .cu:601
+  return actnn::dispatch_backward(grad_out, mask, grad_in, n, keep_div, true, dtype, stream);
+}

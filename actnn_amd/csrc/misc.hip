@@ -1,0 +1,49 @@
+// Library-level helpers: error strings, version, and the plain streaming copy used to
+// calibrate bandwidth counters.
+#include "device_utils.h"
+
+namespace actnn {
+namespace {
+
+__global__ __launch_bounds__(256) void stream_copy_kernel(const uint4* __restrict__ src,
+                                                          uint4* __restrict__ dst, int64_t nvec) {
+  // each block copies a contiguous run of 4 * 256 vectors (16 KiB); four loads in flight per lane
+  const int64_t base = (int64_t)blockIdx.x * 1024 + threadIdx.x;
+  uint4 v[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (base + i * 256 < nvec) v[i] = src[base + i * 256];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (base + i * 256 < nvec) dst[base + i * 256] = v[i];
+}
+
+}  // namespace
+}  // namespace actnn
+
+extern "C" int actnn_stream_copy(const void* src, void* dst, int64_t bytes, void* stream) {
+  using namespace actnn;
+  if (bytes < 0 || bytes % 16 != 0) return ACTNN_EINVAL;
+  if (bytes == 0) return ACTNN_OK;
+  if (!src || !dst) return ACTNN_EINVAL;
+  if (!aligned16(src) || !aligned16(dst)) return ACTNN_EALIGN;
+  const int64_t nvec = bytes / 16;
+  const int64_t blocks = (nvec + 1023) / 1024;
+  if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
+  stream_copy_kernel<<<dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<const uint4*>(src), static_cast<uint4*>(dst), nvec);
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" const char* actnn_strerror(int code) {
+  switch (code) {
+    case ACTNN_OK: return "success";
+    case ACTNN_EINVAL: return "invalid size, null pointer or unsupported combination";
+    case ACTNN_EDTYPE: return "unknown dtype";
+    case ACTNN_EBITS: return "unsupported bit width";
+    case ACTNN_EALIGN: return "pointer is not aligned as required (16 bytes)";
+    default: return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "unknown error";
+  }
+}
+
+extern "C" const char* actnn_version(void) { return "actnn_amd 0.1 (gfx950)"; }

@@ -1,0 +1,418 @@
+// Mixed-precision pack / unpack (replaces quantization_cuda_kernel.cu:22-205).
+//
+// Stream layout (kept from the reference): sample n with b = bits[n] owns
+// b * G * gs / 32 consecutive int32 words starting at prefix[n] * G * gs / 32; inside a group
+// of gs = 32 * E elements, bit i of the code of element d = E * j + k is bit j of word
+// k * b + i.  So a word is a 32-lane "ballot" over j, where lane j owns the E consecutive
+// elements E*j .. E*j+E-1.
+//
+// gs == 256 fast path: a 32-lane half-wave owns a group; lane j loads its 8 contiguous
+// elements (one 16-byte load for 16-bit types, two for f32), quantises them and
+// concatenates the 8 codes into 8*b bits of a register (several groups share a register
+// when 8*b <= 16).  One 32x32 bit transpose per register (5 exchange stages) then leaves
+// word p in lane p, which is stored coalesced.  A 256-thread block handles 32 groups of one
+// sample (4 per half-wave, all loads issued before any arithmetic); their 32 scales are
+// computed by the first 32 threads and shared through LDS.
+//
+// Other group sizes (multiples of 32 up to 1024) take a simple LDS-staged kernel.
+#include "quant_math.h"
+
+namespace actnn {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kHalfWaves = kThreads / 32;
+constexpr int kGroupsPerHalf = 4;
+constexpr int kGroupsPerBlock = kHalfWaves * kGroupsPerHalf;   // 32
+constexpr int kGs = 256;
+
+template <int BITS> struct Tile {
+  static constexpr int kWordsPerGroup = 8 * BITS;
+  static constexpr int kGroupsPerReg = BITS == 1 ? 4 : BITS == 2 ? 2 : 1;   // groups sharing one transpose
+  static constexpr bool kTwoRegs = BITS > 4;                                  // 8*BITS > 32
+};
+
+// ---------------------------------------------------------------------------- pack (gs = 256)
+template <typename T, int BITS, bool DET>
+ACTNN_DEV void pack_groups(const T* __restrict__ data, const T* __restrict__ noise,
+                           int32_t* __restrict__ packed, int64_t elem_base, int64_t word_base,
+                           int groups_valid, const float* s_mul, const float* s_sub,
+                           uint64_t seed, uint64_t offset) {
+  using TL = Tile<BITS>;
+  constexpr int R = TL::kGroupsPerReg;
+  constexpr int WPG = TL::kWordsPerGroup;
+  constexpr float Bf = (float)((1 << BITS) - 1);
+  const uint32_t lane = threadIdx.x & 31;
+  const int gl0 = (threadIdx.x >> 5) * kGroupsPerHalf;
+
+  float v[kGroupsPerHalf][8];
+  float nz[DET ? kGroupsPerHalf : 1][8];
+#pragma unroll
+  for (int q = 0; q < kGroupsPerHalf; ++q) {
+    if (gl0 + q < groups_valid) {
+      const int64_t e = elem_base + (int64_t)(gl0 + q) * kGs + lane * 8;
+      load8(data + e, v[q]);
+      if (DET) load8(noise + e, nz[DET ? q : 0]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) { v[q][k] = 0.0f; if (DET) nz[DET ? q : 0][k] = 0.0f; }
+    }
+  }
+
+#pragma unroll
+  for (int q0 = 0; q0 < kGroupsPerHalf; q0 += R) {
+    uint64_t acc = 0;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int q = q0 + r;
+      const float mul = s_mul[gl0 + q];
+      const float sub = s_sub[gl0 + q];
+      uint32_t r16[8];
+      if (!DET) philox_octet((uint64_t)(elem_base >> 3) + (uint64_t)(gl0 + q) * 32 + lane, seed, offset, r16);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const uint32_t c = DET ? det_code<T>(v[q][k], nz[DET ? q : 0][k], mul, sub, Bf)
+                               : rng_code(v[q][k], r16[k], mul, sub, Bf * 65536.0f);
+        acc |= (uint64_t)c << (r * WPG + k * BITS);
+      }
+    }
+    const int64_t tile_words = word_base + (int64_t)(gl0 + q0) * WPG;
+    const uint32_t lo = transpose32((uint32_t)acc, lane);
+    if (TL::kTwoRegs) {
+      const uint32_t hi = transpose32((uint32_t)(acc >> 32), lane);
+      if (gl0 + q0 < groups_valid) {
+        packed[tile_words + lane] = (int32_t)lo;
+        if ((int)lane < WPG - 32) packed[tile_words + 32 + lane] = (int32_t)hi;
+      }
+    } else {
+      if ((int)lane < R * WPG && gl0 + q0 + (int)lane / WPG < groups_valid)
+        packed[tile_words + lane] = (int32_t)lo;
+    }
+  }
+}
+
+template <typename T, bool DET>
+__global__ __launch_bounds__(kThreads) void pack_mixed_kernel(
+    const T* __restrict__ data, const T* __restrict__ mn, const T* __restrict__ mx,
+    const int32_t* __restrict__ bits, const int32_t* __restrict__ prefix, T* __restrict__ scale,
+    int32_t* __restrict__ packed, const T* __restrict__ noise, uint64_t seed, uint64_t offset,
+    int64_t G, int blocks_per_sample) {
+  __shared__ float s_mul[kGroupsPerBlock];
+  __shared__ float s_sub[kGroupsPerBlock];
+  const int64_t n = blockIdx.x / blocks_per_sample;
+  const int64_t gb = (int64_t)(blockIdx.x % blocks_per_sample) * kGroupsPerBlock;
+  const int b = bits[n];
+  const int groups_valid = (int)((G - gb) < kGroupsPerBlock ? (G - gb) : kGroupsPerBlock);
+
+  if (threadIdx.x < kGroupsPerBlock) {
+    float mul = 0.0f, sub = 0.0f;
+    if ((int)threadIdx.x < groups_valid) {
+      const int64_t gi = n * G + gb + threadIdx.x;
+      const float sc = GroupQuant<T, DET>::prepare(Conv<T>::load(mn, gi), Conv<T>::load(mx, gi), b, mul, sub);
+      Conv<T>::store(scale, gi, sc);
+    }
+    s_mul[threadIdx.x] = mul;
+    s_sub[threadIdx.x] = sub;
+  }
+  __syncthreads();
+
+  const int64_t elem_base = (n * G + gb) * kGs;
+  const int64_t word_base = (int64_t)prefix[n] * G * 8 + gb * 8 * b;
+  switch (b) {
+#define ACTNN_CASE(B_)                                                                          \
+  case B_:                                                                                      \
+    pack_groups<T, B_, DET>(data, noise, packed, elem_base, word_base, groups_valid, s_mul,     \
+                            s_sub, seed, offset);                                               \
+    break;
+    ACTNN_CASE(1) ACTNN_CASE(2) ACTNN_CASE(3) ACTNN_CASE(4)
+    ACTNN_CASE(5) ACTNN_CASE(6) ACTNN_CASE(7) ACTNN_CASE(8)
+#undef ACTNN_CASE
+    default: break;   // bits outside 1..8 are rejected on the host when known; nothing is written
+  }
+}
+
+// ---------------------------------------------------------------------------- unpack (gs = 256)
+template <typename T, int BITS>
+ACTNN_DEV void unpack_groups(const int32_t* __restrict__ packed, T* __restrict__ out,
+                             int64_t elem_base, int64_t word_base, int groups_valid,
+                             const float* s_scale, const float* s_min) {
+  using TL = Tile<BITS>;
+  constexpr int R = TL::kGroupsPerReg;
+  constexpr int WPG = TL::kWordsPerGroup;
+  constexpr uint32_t kMask = (1u << BITS) - 1u;
+  const uint32_t lane = threadIdx.x & 31;
+  const int gl0 = (threadIdx.x >> 5) * kGroupsPerHalf;
+
+  uint32_t wlo[kGroupsPerHalf / R], whi[kGroupsPerHalf / R];
+#pragma unroll
+  for (int t = 0; t < kGroupsPerHalf / R; ++t) {
+    const int q0 = t * R;
+    const int64_t tile_words = word_base + (int64_t)(gl0 + q0) * WPG;
+    wlo[t] = 0;
+    whi[t] = 0;
+    if (TL::kTwoRegs) {
+      if (gl0 + q0 < groups_valid) {
+        wlo[t] = (uint32_t)packed[tile_words + lane];
+        if ((int)lane < WPG - 32) whi[t] = (uint32_t)packed[tile_words + 32 + lane];
+      }
+    } else {
+      if ((int)lane < R * WPG && gl0 + q0 + (int)lane / WPG < groups_valid)
+        wlo[t] = (uint32_t)packed[tile_words + lane];
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < kGroupsPerHalf / R; ++t) {
+    const int q0 = t * R;
+    uint64_t acc = transpose32(wlo[t], lane);
+    if (TL::kTwoRegs) acc |= (uint64_t)transpose32(whi[t], lane) << 32;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int q = q0 + r;
+      if (gl0 + q < groups_valid) {
+        const float sc = s_scale[gl0 + q];
+        const float m = s_min[gl0 + q];
+        float v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const uint32_t c = (uint32_t)(acc >> (r * WPG + k * BITS)) & kMask;
+          // (scalar_t)val / scale + min, one rounding per operation (.cu:171)
+          v[k] = Conv<T>::round(Conv<T>::round((float)c / sc) + m);
+        }
+        store8(out + elem_base + (int64_t)(gl0 + q) * kGs + lane * 8, v);
+      }
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void unpack_mixed_kernel(
+    const int32_t* __restrict__ packed, const int32_t* __restrict__ bits,
+    const int32_t* __restrict__ prefix, const T* __restrict__ scale, const T* __restrict__ mn,
+    T* __restrict__ out, int64_t G, int blocks_per_sample) {
+  __shared__ float s_scale[kGroupsPerBlock];
+  __shared__ float s_min[kGroupsPerBlock];
+  const int64_t n = blockIdx.x / blocks_per_sample;
+  const int64_t gb = (int64_t)(blockIdx.x % blocks_per_sample) * kGroupsPerBlock;
+  const int b = bits[n];
+  const int groups_valid = (int)((G - gb) < kGroupsPerBlock ? (G - gb) : kGroupsPerBlock);
+  if ((int)threadIdx.x < groups_valid) {
+    const int64_t gi = n * G + gb + threadIdx.x;
+    s_scale[threadIdx.x] = Conv<T>::load(scale, gi);
+    s_min[threadIdx.x] = Conv<T>::load(mn, gi);
+  }
+  __syncthreads();
+  const int64_t elem_base = (n * G + gb) * kGs;
+  const int64_t word_base = (int64_t)prefix[n] * G * 8 + gb * 8 * b;
+  switch (b) {
+#define ACTNN_CASE(B_)                                                                          \
+  case B_:                                                                                      \
+    unpack_groups<T, B_>(packed, out, elem_base, word_base, groups_valid, s_scale, s_min);      \
+    break;
+    ACTNN_CASE(1) ACTNN_CASE(2) ACTNN_CASE(3) ACTNN_CASE(4)
+    ACTNN_CASE(5) ACTNN_CASE(6) ACTNN_CASE(7) ACTNN_CASE(8)
+#undef ACTNN_CASE
+    default: break;
+  }
+}
+
+// ---------------------------------------------------------------------------- generic group size
+// One block per (sample, group); codes staged as bytes in LDS, then thread w assembles word w.
+template <typename T, bool DET>
+__global__ __launch_bounds__(kThreads) void pack_mixed_generic_kernel(
+    const T* __restrict__ data, const T* __restrict__ mn, const T* __restrict__ mx,
+    const int32_t* __restrict__ bits, const int32_t* __restrict__ prefix, T* __restrict__ scale,
+    int32_t* __restrict__ packed, const T* __restrict__ noise, uint64_t seed, uint64_t offset,
+    int64_t G, int gs) {
+  __shared__ uint8_t s_code[1024];
+  __shared__ float s_par[2];
+  const int64_t n = blockIdx.x / G;
+  const int64_t g = blockIdx.x % G;
+  const int b = bits[n];
+  if (b < 1 || b > 8) return;
+  const int64_t gi = n * G + g;
+  if (threadIdx.x == 0) {
+    float mul, sub;
+    const float sc = GroupQuant<T, DET>::prepare(Conv<T>::load(mn, gi), Conv<T>::load(mx, gi), b, mul, sub);
+    Conv<T>::store(scale, gi, sc);
+    s_par[0] = mul;
+    s_par[1] = sub;
+  }
+  __syncthreads();
+  const float mul = s_par[0], sub = s_par[1];
+  const float Bf = (float)((1 << b) - 1);
+  for (int d = threadIdx.x; d < gs; d += kThreads) {
+    const int64_t e = gi * gs + d;
+    const float x = Conv<T>::load(data, e);
+    uint32_t c;
+    if (DET) {
+      c = det_code<T>(x, Conv<T>::load(noise, e), mul, sub, Bf);
+    } else {
+      uint32_t r16[8];
+      philox_octet((uint64_t)e >> 3, seed, offset, r16);
+      uint32_t r = r16[0];
+#pragma unroll
+      for (int k = 1; k < 8; ++k) r = ((int)(e & 7) == k) ? r16[k] : r;
+      c = rng_code(x, r, mul, sub, Bf * 65536.0f);
+    }
+    s_code[d] = (uint8_t)c;
+  }
+  __syncthreads();
+  const int E = gs / 32;
+  const int L = E * b;
+  const int64_t word_base = ((int64_t)prefix[n] * G + (int64_t)b * g) * E;
+  for (int w = threadIdx.x; w < L; w += kThreads) {
+    const int k = w / b, i = w % b;
+    uint32_t word = 0;
+    for (int j = 0; j < 32; ++j) word |= ((uint32_t)(s_code[E * j + k] >> i) & 1u) << j;
+    packed[word_base + w] = (int32_t)word;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void unpack_mixed_generic_kernel(
+    const int32_t* __restrict__ packed, const int32_t* __restrict__ bits,
+    const int32_t* __restrict__ prefix, const T* __restrict__ scale, const T* __restrict__ mn,
+    T* __restrict__ out, int64_t G, int gs) {
+  __shared__ uint32_t s_word[256];   // E * b <= 32 * 8
+  const int64_t n = blockIdx.x / G;
+  const int64_t g = blockIdx.x % G;
+  const int b = bits[n];
+  if (b < 1 || b > 8) return;
+  const int E = gs / 32;
+  const int L = E * b;
+  const int64_t word_base = ((int64_t)prefix[n] * G + (int64_t)b * g) * E;
+  for (int w = threadIdx.x; w < L; w += kThreads) s_word[w] = (uint32_t)packed[word_base + w];
+  __syncthreads();
+  const int64_t gi = n * G + g;
+  const float sc = Conv<T>::load(scale, gi);
+  const float m = Conv<T>::load(mn, gi);
+  for (int d = threadIdx.x; d < gs; d += kThreads) {
+    const int j = d / E, k = d % E;
+    uint32_t c = 0;
+    for (int i = 0; i < b; ++i) c |= ((s_word[k * b + i] >> j) & 1u) << i;
+    Conv<T>::store(out, gi * gs + d, Conv<T>::round((float)c / sc) + m);
+  }
+}
+
+// ---------------------------------------------------------------------------- prefix sum
+__global__ __launch_bounds__(1024) void bits_prefix_kernel(const int32_t* __restrict__ bits,
+                                                           int32_t* __restrict__ prefix, int64_t N) {
+  __shared__ int32_t s_part[1024];
+  // thread t owns the contiguous chunk [t * per, (t + 1) * per)
+  const int64_t per = (N + 1023) / 1024;
+  const int64_t lo = (int64_t)threadIdx.x * per;
+  const int64_t hi = lo + per < N ? lo + per : N;
+  int32_t sum = 0;
+  for (int64_t i = lo; i < hi; ++i) sum += bits[i];
+  s_part[threadIdx.x] = sum;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {           // inclusive Hillis-Steele scan
+    int32_t add = threadIdx.x >= (unsigned)off ? s_part[threadIdx.x - off] : 0;
+    __syncthreads();
+    s_part[threadIdx.x] += add;
+    __syncthreads();
+  }
+  int32_t run = threadIdx.x == 0 ? 0 : s_part[threadIdx.x - 1];
+  if (threadIdx.x == 0) prefix[0] = 0;
+  for (int64_t i = lo; i < hi; ++i) {
+    run += bits[i];
+    prefix[i + 1] = run;
+  }
+}
+
+template <typename T>
+int launch_pack(const void* data, const void* mn, const void* mx, const int32_t* bits,
+                const int32_t* prefix, void* scale, int32_t* packed, const void* noise,
+                uint64_t seed, uint64_t offset, int64_t N, int64_t G, int64_t gs, hipStream_t s) {
+  const T* d = static_cast<const T*>(data);
+  const T* nz = static_cast<const T*>(noise);
+  if (gs == kGs) {
+    const int64_t bps = (G + kGroupsPerBlock - 1) / kGroupsPerBlock;
+    if (N * bps > 0x7fffffffLL) return ACTNN_EINVAL;
+    const dim3 grid((unsigned)(N * bps));
+    if (noise)
+      pack_mixed_kernel<T, true><<<grid, dim3(kThreads), 0, s>>>(
+          d, static_cast<const T*>(mn), static_cast<const T*>(mx), bits, prefix,
+          static_cast<T*>(scale), packed, nz, seed, offset, G, (int)bps);
+    else
+      pack_mixed_kernel<T, false><<<grid, dim3(kThreads), 0, s>>>(
+          d, static_cast<const T*>(mn), static_cast<const T*>(mx), bits, prefix,
+          static_cast<T*>(scale), packed, nz, seed, offset, G, (int)bps);
+  } else {
+    if (N * G > 0x7fffffffLL) return ACTNN_EINVAL;
+    const dim3 grid((unsigned)(N * G));
+    if (noise)
+      pack_mixed_generic_kernel<T, true><<<grid, dim3(kThreads), 0, s>>>(
+          d, static_cast<const T*>(mn), static_cast<const T*>(mx), bits, prefix,
+          static_cast<T*>(scale), packed, nz, seed, offset, G, (int)gs);
+    else
+      pack_mixed_generic_kernel<T, false><<<grid, dim3(kThreads), 0, s>>>(
+          d, static_cast<const T*>(mn), static_cast<const T*>(mx), bits, prefix,
+          static_cast<T*>(scale), packed, nz, seed, offset, G, (int)gs);
+  }
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
+
+template <typename T>
+int launch_unpack(const int32_t* packed, const int32_t* bits, const int32_t* prefix,
+                  const void* scale, const void* mn, void* out, int64_t N, int64_t G, int64_t gs,
+                  hipStream_t s) {
+  if (gs == kGs) {
+    const int64_t bps = (G + kGroupsPerBlock - 1) / kGroupsPerBlock;
+    if (N * bps > 0x7fffffffLL) return ACTNN_EINVAL;
+    unpack_mixed_kernel<T><<<dim3((unsigned)(N * bps)), dim3(kThreads), 0, s>>>(
+        packed, bits, prefix, static_cast<const T*>(scale), static_cast<const T*>(mn),
+        static_cast<T*>(out), G, (int)bps);
+  } else {
+    if (N * G > 0x7fffffffLL) return ACTNN_EINVAL;
+    unpack_mixed_generic_kernel<T><<<dim3((unsigned)(N * G)), dim3(kThreads), 0, s>>>(
+        packed, bits, prefix, static_cast<const T*>(scale), static_cast<const T*>(mn),
+        static_cast<T*>(out), G, (int)gs);
+  }
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
+
+}  // namespace
+}  // namespace actnn
+
+extern "C" int actnn_bits_prefix(const int32_t* bits, int32_t* prefix, int64_t N, void* stream) {
+  using namespace actnn;
+  if (N < 0 || !prefix || (N > 0 && !bits)) return ACTNN_EINVAL;
+  bits_prefix_kernel<<<dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream)>>>(bits, prefix, N);
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int actnn_pack_mixed(const void* data, const void* mn, const void* mx,
+                                const int32_t* bits, const int32_t* prefix, void* scale,
+                                int32_t* packed, const void* noise, uint64_t seed, uint64_t offset,
+                                int64_t N, int64_t G, int64_t gs, int dtype, void* stream) {
+  using namespace actnn;
+  if (N < 0 || G < 0 || gs < 32 || gs > 1024 || gs % 32 != 0) return ACTNN_EINVAL;
+  if (N == 0 || G == 0) return ACTNN_OK;
+  if (!data || !mn || !mx || !bits || !prefix || !scale || !packed) return ACTNN_EINVAL;
+  if (!aligned16(data) || (noise && !aligned16(noise))) return ACTNN_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case ACTNN_F32: return launch_pack<float>(data, mn, mx, bits, prefix, scale, packed, noise, seed, offset, N, G, gs, s);
+    case ACTNN_F16: return launch_pack<__half>(data, mn, mx, bits, prefix, scale, packed, noise, seed, offset, N, G, gs, s);
+    case ACTNN_BF16: return launch_pack<bf16_t>(data, mn, mx, bits, prefix, scale, packed, noise, seed, offset, N, G, gs, s);
+    default: return ACTNN_EDTYPE;
+  }
+}
+
+extern "C" int actnn_unpack_mixed(const int32_t* packed, const int32_t* bits, const int32_t* prefix,
+                                  const void* scale, const void* mn, void* out, int64_t N,
+                                  int64_t G, int64_t gs, int dtype, void* stream) {
+  using namespace actnn;
+  if (N < 0 || G < 0 || gs < 32 || gs > 1024 || gs % 32 != 0) return ACTNN_EINVAL;
+  if (N == 0 || G == 0) return ACTNN_OK;
+  if (!packed || !bits || !prefix || !scale || !mn || !out) return ACTNN_EINVAL;
+  if (!aligned16(out)) return ACTNN_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case ACTNN_F32: return launch_unpack<float>(packed, bits, prefix, scale, mn, out, N, G, gs, s);
+    case ACTNN_F16: return launch_unpack<__half>(packed, bits, prefix, scale, mn, out, N, G, gs, s);
+    case ACTNN_BF16: return launch_unpack<bf16_t>(packed, bits, prefix, scale, mn, out, N, G, gs, s);
+    default: return ACTNN_EDTYPE;
+  }
+}

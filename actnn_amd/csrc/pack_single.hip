@@ -1,0 +1,221 @@
+// Fixed-width pack / unpack (replaces quantization_cuda_kernel.cu:210-405).
+//
+// Stream layout (kept from the reference): byte ((no * G + g) * gs + d) holds the codes of
+// the 8/bits consecutive samples n = no * (8/bits) + ni at bit offset ni * bits.
+//
+// A lane owns 8 consecutive d of one (no, g): it loads 8 elements of each of the 8/bits
+// samples (one 16-byte load per sample for 16-bit types, two for f32), quantises them and
+// writes its 8 output bytes with a single 8-byte store, so a wave writes 512 contiguous bytes.
+// The per-group scale is produced by a small kernel first (N * G values).
+#include "quant_math.h"
+
+namespace actnn {
+namespace {
+
+constexpr int kThreads = 256;
+
+template <typename T, bool DET>
+__global__ __launch_bounds__(kThreads) void scale_single_kernel(const T* __restrict__ mn,
+                                                                const T* __restrict__ mx,
+                                                                T* __restrict__ scale, int bits,
+                                                                int64_t count) {
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i < count) {
+    float mul, sub;
+    Conv<T>::store(scale, i, GroupQuant<T, DET>::prepare(Conv<T>::load(mn, i), Conv<T>::load(mx, i), bits, mul, sub));
+  }
+}
+
+template <typename T, int BITS, bool DET>
+__global__ __launch_bounds__(kThreads) void pack_single_kernel(
+    const T* __restrict__ data, const T* __restrict__ mn, const T* __restrict__ scale,
+    int8_t* __restrict__ packed, const T* __restrict__ noise, uint64_t seed, uint64_t offset,
+    int64_t N, int64_t G, int gs, int64_t units) {
+  constexpr int WPT = 8 / BITS;
+  constexpr float Bf = (float)((1 << BITS) - 1);
+  const int64_t u = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (u >= units) return;
+  const int chunks = gs / 8;
+  const int64_t og = u / chunks;            // no * G + g
+  const int d0 = (int)(u % chunks) * 8;
+  const int64_t no = og / G;
+  const int64_t g = og % G;
+
+  float v[WPT][8];
+  float nz[DET ? WPT : 1][8];
+  float mul[WPT], sub[WPT];
+#pragma unroll
+  for (int ni = 0; ni < WPT; ++ni) {
+    const int64_t n = no * WPT + ni;
+    if (n < N) {
+      const int64_t gi = n * G + g;
+      const int64_t e = gi * gs + d0;
+      load8(data + e, v[ni]);
+      if (DET) load8(noise + e, nz[DET ? ni : 0]);
+      const float sc = Conv<T>::load(scale, gi);
+      const float m = Conv<T>::load(mn, gi);
+      if (DET) {
+        mul[ni] = sc;
+        sub[ni] = Conv<T>::round(m - Conv<T>::round(1e-6f));    // shifted minimum, ops.py:31
+      } else {
+        mul[ni] = sc * 65536.0f;
+        sub[ni] = m;
+      }
+    }
+  }
+  uint32_t lo = 0, hi = 0;   // bytes 0..3 and 4..7
+#pragma unroll
+  for (int ni = 0; ni < WPT; ++ni) {
+    const int64_t n = no * WPT + ni;
+    if (n < N) {
+      uint32_t r16[8];
+      if (!DET) philox_octet((uint64_t)(((n * G + g) * gs + d0) >> 3), seed, offset, r16);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const uint32_t c = DET ? det_code<T>(v[ni][k], nz[DET ? ni : 0][k], mul[ni], sub[ni], Bf)
+                               : rng_code(v[ni][k], r16[k], mul[ni], sub[ni], Bf * 65536.0f);
+        if (k < 4) lo |= c << (8 * k + ni * BITS);
+        else hi |= c << (8 * (k - 4) + ni * BITS);
+      }
+    }
+  }
+  *reinterpret_cast<uint2*>(packed + og * gs + d0) = make_uint2(lo, hi);
+}
+
+template <typename T, int BITS>
+__global__ __launch_bounds__(kThreads) void unpack_single_kernel(
+    const int8_t* __restrict__ packed, const T* __restrict__ scale, const T* __restrict__ mn,
+    T* __restrict__ out, int64_t N, int64_t G, int gs, int64_t units) {
+  constexpr int WPT = 8 / BITS;
+  constexpr uint32_t kMask = (1u << BITS) - 1u;
+  const int64_t u = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (u >= units) return;
+  const int chunks = gs / 8;
+  const int64_t og = u / chunks;
+  const int d0 = (int)(u % chunks) * 8;
+  const int64_t no = og / G;
+  const int64_t g = og % G;
+  const uint2 w = *reinterpret_cast<const uint2*>(packed + og * gs + d0);
+#pragma unroll
+  for (int ni = 0; ni < WPT; ++ni) {
+    const int64_t n = no * WPT + ni;
+    if (n < N) {
+      const int64_t gi = n * G + g;
+      const float sc = Conv<T>::load(scale, gi);
+      const float m = Conv<T>::load(mn, gi);
+      float v[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const uint32_t word = k < 4 ? w.x : w.y;
+        const uint32_t c = (word >> (8 * (k & 3) + ni * BITS)) & kMask;
+        v[k] = Conv<T>::round(Conv<T>::round((float)c / sc) + m);    // .cu:359
+      }
+      store8(out + gi * gs + d0, v);
+    }
+  }
+}
+
+template <typename T, bool DET>
+int launch_pack_bits(int bits, const T* data, const T* mn, const T* scale, int8_t* packed,
+                     const T* noise, uint64_t seed, uint64_t offset, int64_t N, int64_t G, int gs,
+                     hipStream_t s) {
+  const int wpt = 8 / bits;
+  const int64_t units = ((N + wpt - 1) / wpt) * G * (gs / 8);
+  const int64_t blocks = (units + kThreads - 1) / kThreads;
+  if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
+  const dim3 grid((unsigned)blocks), blk(kThreads);
+  switch (bits) {
+    case 1: pack_single_kernel<T, 1, DET><<<grid, blk, 0, s>>>(data, mn, scale, packed, noise, seed, offset, N, G, gs, units); break;
+    case 2: pack_single_kernel<T, 2, DET><<<grid, blk, 0, s>>>(data, mn, scale, packed, noise, seed, offset, N, G, gs, units); break;
+    case 4: pack_single_kernel<T, 4, DET><<<grid, blk, 0, s>>>(data, mn, scale, packed, noise, seed, offset, N, G, gs, units); break;
+    case 8: pack_single_kernel<T, 8, DET><<<grid, blk, 0, s>>>(data, mn, scale, packed, noise, seed, offset, N, G, gs, units); break;
+    default: return ACTNN_EBITS;
+  }
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
+
+template <typename T>
+int launch_pack(const void* data, const void* mn, const void* mx, int bits, void* scale,
+                int8_t* packed, const void* noise, uint64_t seed, uint64_t offset, int64_t N,
+                int64_t G, int64_t gs, hipStream_t s) {
+  const int64_t count = N * G;
+  const int64_t sblocks = (count + kThreads - 1) / kThreads;
+  if (sblocks > 0x7fffffffLL) return ACTNN_EINVAL;
+  const T* lo = static_cast<const T*>(mn);
+  const T* hi = static_cast<const T*>(mx);
+  T* sc = static_cast<T*>(scale);
+  if (noise) scale_single_kernel<T, true><<<dim3((unsigned)sblocks), dim3(kThreads), 0, s>>>(lo, hi, sc, bits, count);
+  else scale_single_kernel<T, false><<<dim3((unsigned)sblocks), dim3(kThreads), 0, s>>>(lo, hi, sc, bits, count);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return (int)e;
+  if (noise)
+    return launch_pack_bits<T, true>(bits, static_cast<const T*>(data), lo, sc, packed,
+                                     static_cast<const T*>(noise), seed, offset, N, G, (int)gs, s);
+  return launch_pack_bits<T, false>(bits, static_cast<const T*>(data), lo, sc, packed, nullptr, seed,
+                                    offset, N, G, (int)gs, s);
+}
+
+template <typename T>
+int launch_unpack(const int8_t* packed, int bits, const void* scale, const void* mn, void* out,
+                  int64_t N, int64_t G, int64_t gs, hipStream_t s) {
+  const int wpt = 8 / bits;
+  const int64_t units = ((N + wpt - 1) / wpt) * G * (gs / 8);
+  const int64_t blocks = (units + kThreads - 1) / kThreads;
+  if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
+  const dim3 grid((unsigned)blocks), blk(kThreads);
+  const T* sc = static_cast<const T*>(scale);
+  const T* lo = static_cast<const T*>(mn);
+  T* o = static_cast<T*>(out);
+  switch (bits) {
+    case 1: unpack_single_kernel<T, 1><<<grid, blk, 0, s>>>(packed, sc, lo, o, N, G, (int)gs, units); break;
+    case 2: unpack_single_kernel<T, 2><<<grid, blk, 0, s>>>(packed, sc, lo, o, N, G, (int)gs, units); break;
+    case 4: unpack_single_kernel<T, 4><<<grid, blk, 0, s>>>(packed, sc, lo, o, N, G, (int)gs, units); break;
+    case 8: unpack_single_kernel<T, 8><<<grid, blk, 0, s>>>(packed, sc, lo, o, N, G, (int)gs, units); break;
+    default: return ACTNN_EBITS;
+  }
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
+
+inline bool single_bits_ok(int bits) { return bits == 1 || bits == 2 || bits == 4 || bits == 8; }
+
+}  // namespace
+}  // namespace actnn
+
+extern "C" int actnn_pack_single(const void* data, const void* mn, const void* mx, int bits,
+                                 void* scale, int8_t* packed, const void* noise, uint64_t seed,
+                                 uint64_t offset, int64_t N, int64_t G, int64_t gs, int dtype,
+                                 void* stream) {
+  using namespace actnn;
+  if (!single_bits_ok(bits)) return ACTNN_EBITS;       // TORCH_CHECK(8 % bits == 0), .cu:272
+  if (N < 0 || G < 0 || gs < 8 || gs % 8 != 0) return ACTNN_EINVAL;
+  if (N == 0 || G == 0) return ACTNN_OK;
+  if (!data || !mn || !mx || !scale || !packed) return ACTNN_EINVAL;
+  if (!aligned16(data) || (noise && !aligned16(noise)) ||
+      (reinterpret_cast<uintptr_t>(packed) & 7u) != 0)
+    return ACTNN_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case ACTNN_F32: return launch_pack<float>(data, mn, mx, bits, scale, packed, noise, seed, offset, N, G, gs, s);
+    case ACTNN_F16: return launch_pack<__half>(data, mn, mx, bits, scale, packed, noise, seed, offset, N, G, gs, s);
+    case ACTNN_BF16: return launch_pack<bf16_t>(data, mn, mx, bits, scale, packed, noise, seed, offset, N, G, gs, s);
+    default: return ACTNN_EDTYPE;
+  }
+}
+
+extern "C" int actnn_unpack_single(const int8_t* packed, int bits, const void* scale,
+                                   const void* mn, void* out, int64_t N, int64_t G, int64_t gs,
+                                   int dtype, void* stream) {
+  using namespace actnn;
+  if (!single_bits_ok(bits)) return ACTNN_EBITS;
+  if (N < 0 || G < 0 || gs < 8 || gs % 8 != 0) return ACTNN_EINVAL;
+  if (N == 0 || G == 0) return ACTNN_OK;
+  if (!packed || !scale || !mn || !out) return ACTNN_EINVAL;
+  if (!aligned16(out) || (reinterpret_cast<uintptr_t>(packed) & 7u) != 0) return ACTNN_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case ACTNN_F32: return launch_unpack<float>(packed, bits, scale, mn, out, N, G, gs, s);
+    case ACTNN_F16: return launch_unpack<__half>(packed, bits, scale, mn, out, N, G, gs, s);
+    case ACTNN_BF16: return launch_unpack<bf16_t>(packed, bits, scale, mn, out, N, G, gs, s);
+    default: return ACTNN_EDTYPE;
+  }
+}

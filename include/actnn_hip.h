@@ -1,0 +1,159 @@
+/*
+ * actnn_hip.h - C ABI of the MI355X (gfx950) activation-compression kernels.
+ *
+ * Every entry point is `extern "C"`, takes plain pointers and sizes, launches on the HIP
+ * stream it is given (`stream` is a hipStream_t passed as void*; NULL = the null stream)
+ * and returns 0 on success, a negative ACTNN_E* code for a rejected argument, or a
+ * positive hipError_t when a launch failed.  Nothing throws and nothing allocates: all
+ * outputs are caller-allocated device buffers.  Unless noted, pointers are device
+ * pointers, tensors are contiguous, and `dtype` is one of ACTNN_F32 / ACTNN_F16 /
+ * ACTNN_BF16 (bf16 is an extension: the reference accepts f32 and f16 only,
+ * actnn/actnn/cpp_extension/ext_common.h:15-19).
+ *
+ * Each declaration cites the reference interface it replaces (paths relative to the
+ * reference tree, actnn/actnn/cpp_extension/).
+ */
+#ifndef ACTNN_HIP_H_
+#define ACTNN_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { ACTNN_F32 = 0, ACTNN_F16 = 1, ACTNN_BF16 = 2 };
+
+enum {
+  ACTNN_OK = 0,
+  ACTNN_EINVAL = -1,   /* bad size / null pointer / unsupported combination */
+  ACTNN_EDTYPE = -2,   /* unknown dtype */
+  ACTNN_EBITS = -3,    /* bit width outside what the operator supports */
+  ACTNN_EALIGN = -4    /* pointer not aligned as the kernel requires (16 bytes) */
+};
+
+/* Human-readable text for a return code of this library (static storage). */
+const char* actnn_strerror(int code);
+
+/* Version string of the library (static storage). */
+const char* actnn_version(void);
+
+/* ---------------------------------------------------------------------------------
+ * minimax: per-row minimum and maximum of data[M, D] -> mn[M], mx[M] (same dtype).
+ * Replaces minimax(Tensor) -> (min, max): minimax.cc:7-11, minimax_cuda_kernel.cu:70-89.
+ * Any D >= 1 is accepted (the reference requires D % 32 == 0 && D > 32).
+ * ------------------------------------------------------------------------------- */
+int actnn_minimax(const void* data, void* mn, void* mx, int64_t M, int64_t D, int dtype,
+                  void* stream);
+
+/* Exclusive prefix sum of the per-sample bit widths: prefix[0] = 0,
+ * prefix[n] = bits[0] + ... + bits[n-1], prefix has N + 1 entries.
+ * Replaces the torch::cumsum calls at quantization_cuda_kernel.cu:97 and :182. */
+int actnn_bits_prefix(const int32_t* bits, int32_t* prefix, int64_t N, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * pack_mixed_precision: quantise data[N, G, gs] with bits[n] in 1..8 bits per sample and
+ * write the int32 bit stream `packed` (ceil(sum(bits) * G * gs / 32) words, reference
+ * layout) and scale[N, G, 1] (dtype of data).
+ * Replaces pack_mixed_precision(data, min, max, bits, stochastic) -> (packed, scale):
+ * quantization.cc:46-57, quantization_cuda_kernel.cu:83-142.
+ *   noise == NULL: in-kernel Philox4x32-10 stochastic rounding keyed by (seed, offset),
+ *                  arithmetic of the reference's CUDA kernel (:32, :65).
+ *   noise != NULL: deterministic mode. noise[N, G, gs] (dtype of data) holds U(-0.5, 0.5)
+ *                  values; codes and scale are bit-identical to the reference's
+ *                  config.simulate quantiser (actnn/actnn/ops.py:23-41) fed the same noise.
+ * gs must be a multiple of 32 and at most 1024.  prefix comes from actnn_bits_prefix.
+ * ------------------------------------------------------------------------------- */
+int actnn_pack_mixed(const void* data, const void* mn, const void* mx, const int32_t* bits,
+                     const int32_t* prefix, void* scale, int32_t* packed, const void* noise,
+                     uint64_t seed, uint64_t offset, int64_t N, int64_t G, int64_t gs,
+                     int dtype, void* stream);
+
+/* unpack_mixed_precision: out[N, G, gs] = code / scale + min (dtype = dtype of scale).
+ * Replaces unpack_mixed_precision(data, bits, scale, min, N, num_groups, group_size):
+ * quantization.cc:59-73, quantization_cuda_kernel.cu:145-205. */
+int actnn_unpack_mixed(const int32_t* packed, const int32_t* bits, const int32_t* prefix,
+                       const void* scale, const void* mn, void* out, int64_t N, int64_t G,
+                       int64_t gs, int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * pack_single_precision: one bit width (1, 2, 4 or 8) for the whole tensor; 8/bits
+ * consecutive samples share a byte.  packed has (bits * N_round * G * gs + 8) / 8 bytes,
+ * N_round = N rounded up to a multiple of 8/bits.
+ * Replaces pack_single_precision(data, min, max, bits, stochastic) -> (packed, scale):
+ * quantization.cc:77-87, quantization_cuda_kernel.cu:261-330.  noise as above.
+ * ------------------------------------------------------------------------------- */
+int actnn_pack_single(const void* data, const void* mn, const void* mx, int bits, void* scale,
+                      int8_t* packed, const void* noise, uint64_t seed, uint64_t offset,
+                      int64_t N, int64_t G, int64_t gs, int dtype, void* stream);
+
+/* Replaces unpack_single_precision(data, bits, scale, min, N, num_groups, group_size):
+ * quantization.cc:89-102, quantization_cuda_kernel.cu:364-405. */
+int actnn_unpack_single(const int8_t* packed, int bits, const void* scale, const void* mn,
+                        void* out, int64_t N, int64_t G, int64_t gs, int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * ReLU with a 1-bit mask.  mask holds 16 int32 words per block of 512 elements,
+ * i.e. ceil(n / 512) * 16 words (equal to the reference's ceil(n / 32) whenever
+ * n % 512 == 0; the reference's tail block writes past its shorter allocation).
+ * Replaces act_quantized_relu_forward_cuda / _backward_cuda:
+ * quantization_cuda_kernel.cu:446-467, :490-508 (quantization.cc:106-124).
+ * ------------------------------------------------------------------------------- */
+int actnn_relu_forward(const void* x, void* y, int32_t* mask, int64_t n, int dtype, void* stream);
+int actnn_relu_backward(const void* grad_out, const int32_t* mask, void* grad_in, int64_t n,
+                        int dtype, void* stream);
+
+/* Dropout with a 1-bit keep mask (same mask layout as ReLU); y = keep ? x / (1 - p) : 0.
+ * keep is drawn from the Philox stream (seed, offset) with probability 1 - p (16-bit
+ * resolution).  Replaces act_quantized_dropout_forward_cuda / _backward_cuda:
+ * quantization_cuda_kernel.cu:555-585, :609-627 (quantization.cc:128-148). */
+int actnn_dropout_forward(const void* x, void* y, int32_t* mask, int64_t n, float p,
+                          uint64_t seed, uint64_t offset, int dtype, void* stream);
+int actnn_dropout_backward(const void* grad_out, const int32_t* mask, void* grad_in, int64_t n,
+                           float p, int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * MaxPool2d keeping the arg-max position inside the window as one int8 per output
+ * element (kh * KW + kw relative to the unclipped window origin; first strict maximum).
+ * KH * KW must be < 16.  Dilation only enters through Ho/Wo, which the caller computes
+ * (quantization_cuda_kernel.cu:679-680); the window itself is undilated, as in the
+ * reference (:649-654).  The backward is a deterministic gather (the reference scatters
+ * with atomicAdd into a zeroed tensor, :723).
+ * Replaces act_quantized_max_pool2d_forward_cuda / _backward_cuda:
+ * quantization_cuda_kernel.cu:672-700, :727-754 (quantization.cc:152-196).
+ * ------------------------------------------------------------------------------- */
+int actnn_max_pool2d_forward(const void* x, void* y, int8_t* idx, int64_t N, int64_t C,
+                             int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH, int KW,
+                             int SH, int SW, int PH, int PW, int dtype, void* stream);
+int actnn_max_pool2d_backward(const void* grad_out, const int8_t* idx, void* grad_in, int64_t N,
+                              int64_t C, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH,
+                              int KW, int SH, int SW, int PH, int PW, int dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------
+ * calc_precision (HOST pointers): greedy bit allocation, mutates b in place.
+ * Replaces calc_precision(b, C, w, target): calc_precision.cc:9-50.
+ * ------------------------------------------------------------------------------- */
+int actnn_calc_precision(int32_t* b, const float* C, const int32_t* w, int64_t N, double target);
+
+/* ---------------------------------------------------------------------------------
+ * Fused QLinear weight gradient: grad_w[O, I] = grad_out[M, O]^T @ dequant(x)[M, I] where x
+ * is held as the pack_single 2-bit stream (4 consecutive rows m per byte) with
+ * scale/min[M, I/256, 1].  The 2-bit tile is unpacked and dequantised to bf16 inside the
+ * LDS loader of a bf16 MFMA GEMM (fp32 accumulation); the full-precision input is never
+ * written to memory.  Replaces dequantize_activation + grad_output.t().mm(input) in
+ * linear.backward, actnn/actnn/ops.py:407-421.
+ * grad_out dtype: f16 or bf16; scale/min dtype = sm_dtype; grad_w dtype = out_dtype
+ * (f32, f16 or bf16).  M % 4 == 0, I % 256 == 0.
+ * ------------------------------------------------------------------------------- */
+int actnn_linear_grad_weight_q2(const void* grad_out, const int8_t* packed, const void* scale,
+                                const void* mn, void* grad_w, int64_t M, int64_t O, int64_t I,
+                                int go_dtype, int sm_dtype, int out_dtype, void* stream);
+
+/* Plain device-to-device streaming copy of `bytes` bytes (16-byte aligned pointers and
+ * size); used by the benchmark to calibrate bandwidth counters.  No reference counterpart. */
+int actnn_stream_copy(const void* src, void* dst, int64_t bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif  /* ACTNN_HIP_H_ */
