@@ -26,6 +26,8 @@ def build(verbose=False):
     from torch.utils import cpp_extension as ce
     os.makedirs(OUT_DIR, exist_ok=True)
     out = os.path.join(OUT_DIR, MOD_NAME + sysconfig.get_config_var("EXT_SUFFIX"))
+    if os.path.exists(out) and os.path.getmtime(out) >= os.path.getmtime(REF_SRC):
+        return out                      # up to date (the torch headers take a minute to compile)
     inc = [f"-I{p}" for p in ce.include_paths()] + [f"-I{sysconfig.get_paths()['include']}"]
     libdir = os.path.join(os.path.dirname(torch.__file__), "lib")
     cmd = ["g++", "-O2", "-std=c++17", "-shared", "-fPIC", f"-DTORCH_EXTENSION_NAME={MOD_NAME}",

@@ -36,9 +36,11 @@ def kernel_scale(mn, mx, bits):
     N = mn.shape[0]
     b = np.broadcast_to(np.asarray(bits, dtype=np.int64), (N,)).reshape(N, 1, 1)
     B = ((1 << b) - 1).astype(np.float64)
-    rng = _round_to(_to_f64(mx) - _to_f64(mn), dtype)          # max - min in scalar_t
+    # max - min in scalar_t: c10::Half arithmetic widens to float, subtracts, narrows again
+    rng = (mx.detach().to(torch.float32) - mn.detach().to(torch.float32)).to(dtype).to(torch.float64).numpy()
     s = B / (rng + 2e-6)                                        # double
-    return torch.from_numpy(s).to(dtype)                        # narrowed on store
+    # narrowed on store: double -> float -> scalar_t (c10::Half is constructed from float)
+    return torch.from_numpy(s).to(torch.float32).to(dtype)
 
 
 def kernel_dequant(codes, scale, mn):

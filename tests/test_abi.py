@@ -1,0 +1,37 @@
+"""The C-ABI library loads and exports every symbol include/actnn_hip.h declares (CPU test:
+no kernel is launched)."""
+import ctypes
+import os
+import re
+
+from actnn_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "actnn_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(actnn_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported(lib):
+    names = _declared()
+    assert len(names) >= 17
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(raw, n), f"{n} declared in include/actnn_hip.h but not exported"
+    assert set(names) == set(_lib.SIGNATURES), "ctypes signature table out of sync with the header"
+
+
+def test_argument_errors_need_no_gpu(lib):
+    # invalid sizes / dtypes are rejected on the host before anything is launched
+    assert lib.actnn_minimax(None, None, None, 4, 0, 0, None) == -1
+    assert lib.actnn_minimax(None, None, None, 0, 256, 0, None) == 0          # empty input
+    assert lib.actnn_pack_mixed(None, None, None, None, None, None, None, None, 0, 0, 4, 4, 100, 0, None) == -1
+    assert lib.actnn_pack_single(None, None, None, 3, None, None, None, 0, 0, 4, 4, 256, 0, None) == -3
+    assert lib.actnn_relu_forward(None, None, None, -1, 0, None) == -1
+    assert lib.actnn_relu_forward(None, None, None, 0, 7, None) == 0
+    assert lib.actnn_max_pool2d_forward(None, None, None, 1, 1, 8, 8, 4, 4, 4, 4, 2, 2, 1, 1, 0, None) == -1
+    assert lib.actnn_strerror(-3) == b"unsupported bit width"
+    assert b"gfx950" in lib.actnn_version()

@@ -1,0 +1,81 @@
+"""ReLU / Dropout with 1-bit masks: values vs torch (exact, as tests/test_act_quantized_ops.py:17-36
+of the reference does for ReLU), mask words vs the oracle's layout."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import actnn_amd.cpp_extension.quantization as ext_q
+from oracle import layouts, philox
+from _util import DEV
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(128, 56, 56, 31), (4, 512), (1, 1), (7,), (3, 171), (2, 8192), (5, 1025)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_relu_forward_backward(dtype, shape):
+    if shape == SHAPES[0] and dtype == torch.bfloat16:
+        pytest.skip("large case covered by f32/f16")
+    torch.manual_seed(len(shape))
+    x = torch.randn(*shape).to(dtype)
+    x.view(-1)[::97] = 0.0
+    xd = x.to(DEV).requires_grad_(True)
+    y = ext_q.act_quantized_relu(xd)
+    ref = F.relu(x.to(DEV))
+    assert torch.equal(y, ref)
+    y.backward(torch.ones_like(y))
+    xr = x.to(DEV).requires_grad_(True)
+    F.relu(xr).backward(torch.ones_like(ref))
+    assert torch.equal(xd.grad, xr.grad)
+    # mask words follow the reference layout, tail block fully materialised
+    _, mask = ext_q.relu_forward(x.to(DEV))
+    exp = layouts.mask_words((x.view(-1) > 0).numpy())
+    assert mask.dtype == torch.int32 and mask.numel() == exp.size
+    assert np.array_equal(mask.cpu().numpy(), exp)
+    # backward with a random upstream gradient
+    g = torch.randn(*shape).to(dtype).to(DEV)
+    gi = ext_q.relu_backward(g, mask)
+    assert torch.equal(gi, torch.where(x.to(DEV) > 0, g, torch.zeros_like(g)))
+
+
+def test_relu_rejects_bad_arguments():
+    with pytest.raises(RuntimeError):
+        ext_q.act_quantized_relu(torch.randn(8))
+    with pytest.raises(RuntimeError):
+        ext_q.act_quantized_relu(torch.randn(8, 8, device=DEV).t())
+    with pytest.raises(RuntimeError):
+        ext_q.act_quantized_relu(torch.zeros(8, dtype=torch.int32, device=DEV))
+    assert ext_q.act_quantized_relu(torch.empty(0, device=DEV)).numel() == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("p", [0.5, 0.1, 0.0, 1.0])
+def test_dropout(dtype, p):
+    n = 1_000_003
+    torch.manual_seed(1)
+    x = (torch.randn(n) + 3.0).to(dtype).to(DEV).requires_grad_(True)
+    torch.cuda.manual_seed(2024)
+    offset = torch.cuda.default_generators[0].get_offset()
+    y = ext_q.act_quantized_dropout(x, p)
+    # keep flags are the oracle's Philox bits: r16 >= round(p * 2^16)
+    r = philox.noise16(np.arange(n, dtype=np.uint64), 2024, offset)
+    keep = r >= np.uint32(min(max(int(p * 65536.0 + 0.5), 0), 65536))
+    keep_t = torch.from_numpy(keep).to(DEV)
+    assert abs(keep.mean() - (1.0 - p)) < 3e-3
+    # reference on the host in numpy: true fp32 division by float(1 - p) (torch's device division by
+    # a python scalar multiplies by the reciprocal, which is not the same rounding)
+    div = np.float32(1.0 - float(np.float32(p)))
+
+    def expect(t):
+        v = t.detach().float().cpu().numpy()
+        with np.errstate(divide="ignore", invalid="ignore"):
+            r_ = np.where(keep, v / div, np.float32(0)).astype(np.float32)
+        return torch.from_numpy(r_).to(dtype)
+
+    assert torch.equal(y.detach().cpu(), expect(x))
+    g = torch.randn(n).to(dtype).to(DEV)
+    y.backward(g)
+    assert torch.equal(x.grad.cpu(), expect(g))

@@ -1,0 +1,58 @@
+"""act_quantized_max_pool2d vs F.max_pool2d forward/backward (reference test:
+tests/test_act_quantized_ops.py:206-232, atol/rtol 1e-4) and vs the oracle's index rule."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import actnn_amd.cpp_extension.quantization as ext_q
+from oracle import pool
+from _util import DEV
+
+pytestmark = pytest.mark.gpu
+
+GEOMS = [((3, 3), (2, 2), (1, 1)), ((2, 2), (2, 2), (0, 0)), ((3, 3), (1, 1), (1, 1)),
+         ((3, 2), (1, 2), (1, 0)), ((1, 1), (1, 1), (0, 0)), ((3, 5), (2, 3), (1, 2))]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("k,s,p", GEOMS)
+@pytest.mark.parametrize("shape", [(4, 8, 28, 28), (2, 3, 13, 17), (1, 1, 5, 5)])
+def test_forward_backward(dtype, k, s, p, shape):
+    torch.manual_seed(sum(shape))
+    x = torch.randn(*shape).to(dtype)
+    xd = x.to(DEV).requires_grad_(True)
+    y = ext_q.act_quantized_max_pool2d(xd, k, s, p, (1, 1), False, False)
+    xr = x.to(DEV).requires_grad_(True)
+    yr = F.max_pool2d(xr, k, s, p)
+    assert torch.equal(y, yr)
+    g = torch.randn_like(yr)
+    y.backward(g)
+    yr.backward(g)
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+    assert torch.allclose(xd.grad.float(), xr.grad.float(), atol=tol, rtol=tol)
+    # index rule against the oracle
+    _, idx = ext_q.max_pool2d_forward(x.to(DEV), k, s, p, (1, 1))
+    out_o, idx_o = pool.max_pool2d_forward(x.float().numpy(), k, s, p)
+    assert idx.dtype == torch.int8 and np.array_equal(idx.cpu().numpy(), idx_o)
+    gin_o = pool.max_pool2d_backward(g.float().cpu().numpy(), idx_o, shape, k, s, p)
+    assert np.allclose(xd.grad.float().cpu().numpy(), gin_o, atol=tol, rtol=tol)
+
+
+def test_ties_take_the_first_position():
+    x = torch.zeros(1, 1, 8, 8, device=DEV)
+    _, idx = ext_q.max_pool2d_forward(x, (3, 3), (2, 2), (1, 1), (1, 1))
+    _, idx_o = pool.max_pool2d_forward(np.zeros((1, 1, 8, 8), np.float32), (3, 3), (2, 2), (1, 1))
+    assert np.array_equal(idx.cpu().numpy(), idx_o)
+
+
+def test_rejected_arguments():
+    x = torch.randn(1, 1, 8, 8, device=DEV)
+    with pytest.raises(RuntimeError):
+        ext_q.act_quantized_max_pool2d(x, (3, 3), (2, 2), (1, 1), (1, 1), True, False)    # ceil_mode
+    with pytest.raises(RuntimeError):
+        ext_q.act_quantized_max_pool2d(x, (3, 3), (2, 2), (1, 1), (1, 1), False, True)    # return_indices
+    with pytest.raises(RuntimeError):
+        ext_q.act_quantized_max_pool2d(x, (4, 4), (2, 2), (1, 1), (1, 1), False, False)   # KH*KW >= 16
+    with pytest.raises(RuntimeError):
+        ext_q.act_quantized_max_pool2d(x, (3,), (2, 2), (1, 1), (1, 1), False, False)
