@@ -16,6 +16,10 @@ struct bf16_t { uint16_t bits; };   // raw bfloat16 storage
 #define ACTNN_DEV __device__ __forceinline__
 
 // ------------------------------------------------------------------ scalar conversions
+// Bit casts go through by-value helpers: __builtin_bit_cast applied directly to a vector
+// element expression (v.y, v[i]) reads element 0 with this compiler.
+ACTNN_DEV float as_float(uint32_t u) { return __builtin_bit_cast(float, u); }
+ACTNN_DEV uint32_t as_uint(float f) { return __builtin_bit_cast(uint32_t, f); }
 ACTNN_DEV float bf16_bits_to_float(uint32_t b) { return __builtin_bit_cast(float, b << 16); }
 ACTNN_DEV uint32_t float_to_bf16_bits(float f) {           // round to nearest even
   uint32_t u = __builtin_bit_cast(uint32_t, f);
@@ -50,15 +54,51 @@ template <> struct Conv<bf16_t> {
   static ACTNN_DEV float round(float v) { return bf16_bits_to_float(float_to_bf16_bits(v)); }
 };
 
+// ------------------------------------------------------------------ 16-byte vector access
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#ifndef ACTNN_NT_LOADS
+#define ACTNN_NT_LOADS 1
+#endif
+#ifndef ACTNN_NT_LOAD8_16
+#define ACTNN_NT_LOAD8_16 0
+#endif
+
+// 16-byte non-temporal load: for data that the kernel reads exactly once AND whose cache
+// lines are consumed whole by one load instruction of the wave (measured: 7.0 vs 6.4 TB/s on
+// a pure read).  Lanes that come back to the same line with a second instruction (the
+// 32-byte-per-lane pattern of fp32 pack) must use the plain load or they fetch the line twice.
+ACTNN_DEV u32x4 load16_nt(const void* p) {
+#if ACTNN_NT_LOADS
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+#else
+  return *reinterpret_cast<const u32x4*>(p);
+#endif
+}
+ACTNN_DEV u32x4 load16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+ACTNN_DEV u32x4 load16_b16(const void* p) {
+#if ACTNN_NT_LOAD8_16
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+#else
+  return *reinterpret_cast<const u32x4*>(p);
+#endif
+}
+ACTNN_DEV void store16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
+
 // ------------------------------------------------------------------ 8 / 16 contiguous elements
 // load8: 8 consecutive elements starting at p (32-byte aligned for f32, 16 for 16-bit types).
 ACTNN_DEV void load8(const float* p, float (&v)[8]) {
-  const float4 a = reinterpret_cast<const float4*>(p)[0];
-  const float4 b = reinterpret_cast<const float4*>(p)[1];
-  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  const u32x4 a = load16(p);
+  const u32x4 b = load16(p + 4);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[i] = as_float(a[i]);
+    v[4 + i] = as_float(b[i]);
+  }
 }
 ACTNN_DEV void load8(const __half* p, float (&v)[8]) {
-  const uint4 a = reinterpret_cast<const uint4*>(p)[0];
+  const u32x4 a = load16_b16(p);
   const uint32_t w[4] = {a.x, a.y, a.z, a.w};
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -67,29 +107,35 @@ ACTNN_DEV void load8(const __half* p, float (&v)[8]) {
   }
 }
 ACTNN_DEV void load8(const bf16_t* p, float (&v)[8]) {
-  const uint4 a = reinterpret_cast<const uint4*>(p)[0];
+  const u32x4 a = load16_b16(p);
   const uint32_t w[4] = {a.x, a.y, a.z, a.w};
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    v[2 * i] = __builtin_bit_cast(float, w[i] << 16);
-    v[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xffff0000u);
+    v[2 * i] = as_float(w[i] << 16);
+    v[2 * i + 1] = as_float(w[i] & 0xffff0000u);
   }
 }
 ACTNN_DEV void store8(float* p, const float (&v)[8]) {
-  reinterpret_cast<float4*>(p)[0] = make_float4(v[0], v[1], v[2], v[3]);
-  reinterpret_cast<float4*>(p)[1] = make_float4(v[4], v[5], v[6], v[7]);
+  u32x4 a, b;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    a[i] = as_uint(v[i]);
+    b[i] = as_uint(v[4 + i]);
+  }
+  store16(p, a);
+  store16(p + 4, b);
 }
 ACTNN_DEV void store8(__half* p, const float (&v)[8]) {
   uint32_t w[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) w[i] = float_to_half_bits(v[2 * i]) | (float_to_half_bits(v[2 * i + 1]) << 16);
-  reinterpret_cast<uint4*>(p)[0] = make_uint4(w[0], w[1], w[2], w[3]);
+  store16(p, (u32x4){w[0], w[1], w[2], w[3]});
 }
 ACTNN_DEV void store8(bf16_t* p, const float (&v)[8]) {
   uint32_t w[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) w[i] = float_to_bf16_bits(v[2 * i]) | (float_to_bf16_bits(v[2 * i + 1]) << 16);
-  reinterpret_cast<uint4*>(p)[0] = make_uint4(w[0], w[1], w[2], w[3]);
+  store16(p, (u32x4){w[0], w[1], w[2], w[3]});
 }
 
 // ------------------------------------------------------------------ cross-lane exchange
@@ -153,13 +199,38 @@ ACTNN_DEV float row16_min(float v) {
   return v;
 }
 
+// Combine the per-row results of row16_min/max across the rows of the wave.  After the call
+// with ROWS == 2 the last row of each 32-lane half holds the half's result; with ROWS == 4
+// the last row of the wave (lanes 48..63) holds the wave's result.
+template <int ROWS> ACTNN_DEV float rows_min(float v) {
+  if (ROWS >= 2)   // row_bcast15 into rows 1 and 3
+    v = fminf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+                     __builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false)));
+  if (ROWS >= 4)   // row_bcast31 into rows 2 and 3
+    v = fminf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+                     __builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false)));
+  return v;
+}
+template <int ROWS> ACTNN_DEV float rows_max(float v) {
+  if (ROWS >= 2)
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+                     __builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false)));
+  if (ROWS >= 4)
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+                     __builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false)));
+  return v;
+}
+
 // ------------------------------------------------------------------ Philox4x32-10
 struct Philox4 { uint32_t x, y, z, w; };
 
+#ifndef ACTNN_PHILOX_ROUNDS
+#define ACTNN_PHILOX_ROUNDS 10    // anything else is for timing experiments only
+#endif
 ACTNN_DEV Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
                                 uint32_t k0, uint32_t k1) {
 #pragma unroll
-  for (int r = 0; r < 10; ++r) {
+  for (int r = 0; r < ACTNN_PHILOX_ROUNDS; ++r) {
     const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
     const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
     const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;

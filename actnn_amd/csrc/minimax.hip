@@ -1,34 +1,44 @@
 // Per-row min/max (replaces minimax_cuda_kernel.cu:23-89 of the reference).
 //
-// HBM-bound streaming read.  A row is reduced by one DPP row (16 lanes): every lane issues
-// independent 16-byte loads (each load instruction of the wave covers four 256-byte
-// contiguous segments), keeps running min/max in registers and the 16 lanes are combined
-// with four DPP steps.  A 256-thread block owns kRowsPerGroup rows per 16-lane group so
-// that many loads are in flight per lane.
+// HBM-bound streaming read.  A row of D elements is reduced by 16, 32 or 64 lanes so that each
+// load instruction of a block covers 4 KiB of consecutive memory (one 16-byte non-temporal
+// load per lane; a 256-element fp32 row is exactly one wave-wide load).  Lanes are combined
+// with DPP steps (quad_perm, row mirrors, row broadcasts).  Small blocks that each sweep a
+// short contiguous run measured faster on MI355X than blocks with many loads in flight per lane;
+// eight rows per lane group (32 KiB per block for fp32 rows of 256) measured best.
 #include "device_utils.h"
 
 namespace actnn {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kRowGroups = kThreads / 16;     // 16-lane groups per block
-constexpr int kRowsPerGroup = 4;              // rows reduced by one 16-lane group
-constexpr int kRowsPerBlock = kRowGroups * kRowsPerGroup;
+constexpr int kRowGroups = kThreads / 16;     // rows per block in the generic kernel
 
-template <typename T> struct Vec16;           // 16-byte vector of T as floats
+#ifndef ACTNN_MM_ROWS
+#define ACTNN_MM_ROWS 8                       // rows per lane group and block (8 measured best)
+#endif
+
+template <typename T> struct Vec16;           // running min/max over one 16-byte vector of T
 template <> struct Vec16<float> {
   static constexpr int kElems = 4;
   static ACTNN_DEV void minmax(const float* p, float& lo, float& hi) {
-    const float4 v = *reinterpret_cast<const float4*>(p);
-    lo = fminf(fminf(lo, v.x), fminf(v.y, fminf(v.z, v.w)));
-    hi = fmaxf(fmaxf(hi, v.x), fmaxf(v.y, fmaxf(v.z, v.w)));
+    const u32x4 u = load16_nt(p);
+    const float a = as_float(u.x), b = as_float(u.y), c = as_float(u.z), d = as_float(u.w);
+    lo = fminf(fminf(lo, a), fminf(b, fminf(c, d)));
+    hi = fmaxf(fmaxf(hi, a), fmaxf(b, fmaxf(c, d)));
   }
 };
 template <> struct Vec16<__half> {
   static constexpr int kElems = 8;
   static ACTNN_DEV void minmax(const __half* p, float& lo, float& hi) {
+    const u32x4 u = load16_nt(p);
+    const uint32_t w[4] = {u.x, u.y, u.z, u.w};
     float v[8];
-    load8(p, v);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = half_bits_to_float(w[i] & 0xffffu);
+      v[2 * i + 1] = half_bits_to_float(w[i] >> 16);
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i) { lo = fminf(lo, v[i]); hi = fmaxf(hi, v[i]); }
   }
@@ -36,63 +46,59 @@ template <> struct Vec16<__half> {
 template <> struct Vec16<bf16_t> {
   static constexpr int kElems = 8;
   static ACTNN_DEV void minmax(const bf16_t* p, float& lo, float& hi) {
+    const u32x4 u = load16_nt(p);
+    const uint32_t w[4] = {u.x, u.y, u.z, u.w};
     float v[8];
-    load8(p, v);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = as_float(w[i] << 16);
+      v[2 * i + 1] = as_float(w[i] & 0xffff0000u);
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i) { lo = fminf(lo, v[i]); hi = fmaxf(hi, v[i]); }
   }
 };
 
-// Fast path: D * sizeof(T) is a multiple of 16 bytes and the base pointer is 16-byte aligned.
-template <typename T, int kVecPerLane>   // kVecPerLane > 0: D == 16 * kVecPerLane * kElems exactly
+// Vector path: a row is D = LPR * kElems * V elements, read by LPR lanes (16, 32 or 64) with V
+// 16-byte loads each, so that every load instruction of a lane group covers LPR * 16
+// contiguous bytes and a block sweeps kThreads * 16 contiguous bytes per instruction.  The
+// base pointer is 16-byte aligned.  V == 0 means "runtime count" (vecs_per_lane).
+template <typename T, int LPR, int V>
 __global__ __launch_bounds__(kThreads) void minimax_vec_kernel(const T* __restrict__ data,
                                                                T* __restrict__ mn,
                                                                T* __restrict__ mx, int64_t M,
-                                                               int64_t D) {
+                                                               int64_t D, int vecs_per_lane) {
   constexpr int E = Vec16<T>::kElems;
-  const int sub = threadIdx.x & 15;
-  const int grp = threadIdx.x >> 4;
-  const int64_t row0 = (int64_t)blockIdx.x * kRowsPerBlock + (int64_t)grp * kRowsPerGroup;
-  float lo[kRowsPerGroup], hi[kRowsPerGroup];
+  constexpr int kSlots = kThreads / LPR;
+  constexpr int R = ACTNN_MM_ROWS;
+  const int sub = threadIdx.x % LPR;
+  const int slot = threadIdx.x / LPR;
+  const int64_t row0 = (int64_t)blockIdx.x * (kSlots * R) + slot;
+  float lo[R], hi[R];
 #pragma unroll
-  for (int r = 0; r < kRowsPerGroup; ++r) { lo[r] = INFINITY; hi[r] = -INFINITY; }
-
-  if (kVecPerLane > 0) {
+  for (int r = 0; r < R; ++r) {
+    lo[r] = INFINITY;
+    hi[r] = -INFINITY;
+    const int64_t row = row0 + r * kSlots;
+    if (row < M) {
+      const T* p = data + row * D + sub * E;
+      if (V > 0) {
 #pragma unroll
-    for (int r = 0; r < kRowsPerGroup; ++r) {
-      const int64_t row = row0 + r;
-      if (row < M) {
-        const T* p = data + row * D + sub * E;
-#pragma unroll
-        for (int i = 0; i < kVecPerLane; ++i) Vec16<T>::minmax(p + i * 16 * E, lo[r], hi[r]);
-      }
-    }
-  } else {
-    const int64_t nvec = D / E;
-#pragma unroll
-    for (int r = 0; r < kRowsPerGroup; ++r) {
-      const int64_t row = row0 + r;
-      if (row < M) {
-        const T* p = data + row * D;
-        for (int64_t v = sub; v < nvec; v += 16) Vec16<T>::minmax(p + v * E, lo[r], hi[r]);
+        for (int i = 0; i < V; ++i) Vec16<T>::minmax(p + i * LPR * E, lo[r], hi[r]);
+      } else {
+        for (int i = 0; i < vecs_per_lane; ++i) Vec16<T>::minmax(p + (int64_t)i * LPR * E, lo[r], hi[r]);
       }
     }
   }
 #pragma unroll
-  for (int r = 0; r < kRowsPerGroup; ++r) {
-    lo[r] = row16_min(lo[r]);
-    hi[r] = row16_max(hi[r]);
-  }
-  // lane r of the group writes row r: four adjacent outputs per group.
-  float wlo = lo[0], whi = hi[0];
-#pragma unroll
-  for (int r = 1; r < kRowsPerGroup; ++r) {
-    if (sub == r) { wlo = lo[r]; whi = hi[r]; }
-  }
-  const int64_t row = row0 + sub;
-  if (sub < kRowsPerGroup && row < M) {
-    Conv<T>::store(mn, row, wlo);
-    Conv<T>::store(mx, row, whi);
+  for (int r = 0; r < R; ++r) {
+    const float l = rows_min<LPR / 16>(row16_min(lo[r]));
+    const float h = rows_max<LPR / 16>(row16_max(hi[r]));
+    const int64_t row = row0 + r * kSlots;
+    if (sub == LPR - 1 && row < M) {      // the last lane of the group holds the combined result
+      Conv<T>::store(mn, row, l);
+      Conv<T>::store(mx, row, h);
+    }
   }
 }
 
@@ -121,27 +127,33 @@ __global__ __launch_bounds__(kThreads) void minimax_generic_kernel(const T* __re
   }
 }
 
+template <typename T, int LPR>
+int launch_vec(const T* d, T* lo, T* hi, int64_t M, int64_t D, int64_t vecs, hipStream_t s) {
+  constexpr int kRows = (kThreads / LPR) * ACTNN_MM_ROWS;
+  const int64_t blocks = (M + kRows - 1) / kRows;
+  if (blocks > 0x7fffffffLL || vecs > 0x7fffffffLL) return ACTNN_EINVAL;
+  const dim3 grid((unsigned)blocks), blk(kThreads);
+  if (vecs == 1) minimax_vec_kernel<T, LPR, 1><<<grid, blk, 0, s>>>(d, lo, hi, M, D, 1);
+  else if (vecs == 2) minimax_vec_kernel<T, LPR, 2><<<grid, blk, 0, s>>>(d, lo, hi, M, D, 2);
+  else minimax_vec_kernel<T, LPR, 0><<<grid, blk, 0, s>>>(d, lo, hi, M, D, (int)vecs);
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
+
 template <typename T>
 int launch_minimax(const void* data, void* mn, void* mx, int64_t M, int64_t D, hipStream_t s) {
   constexpr int E = Vec16<T>::kElems;
   const T* d = static_cast<const T*>(data);
   T* lo = static_cast<T*>(mn);
   T* hi = static_cast<T*>(mx);
-  if (D % E == 0 && aligned16(data)) {
-    const int64_t blocks = (M + kRowsPerBlock - 1) / kRowsPerBlock;
-    if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
-    const int64_t vec_per_lane = (D % (16 * E) == 0) ? D / (16 * E) : 0;
-    if (vec_per_lane == 4)
-      minimax_vec_kernel<T, 4><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(d, lo, hi, M, D);
-    else if (vec_per_lane == 2)
-      minimax_vec_kernel<T, 2><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(d, lo, hi, M, D);
-    else
-      minimax_vec_kernel<T, 0><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(d, lo, hi, M, D);
-  } else {
-    const int64_t blocks = (M + kRowGroups - 1) / kRowGroups;
-    if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
-    minimax_generic_kernel<T><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(d, lo, hi, M, D);
+  if (D % (16 * E) == 0 && aligned16(data)) {
+    const int64_t nvec = D / E;                       // 16-byte vectors per row, a multiple of 16
+    if (nvec % 64 == 0) return launch_vec<T, 64>(d, lo, hi, M, D, nvec / 64, s);
+    if (nvec % 32 == 0) return launch_vec<T, 32>(d, lo, hi, M, D, nvec / 32, s);
+    return launch_vec<T, 16>(d, lo, hi, M, D, nvec / 16, s);
   }
+  const int64_t blocks = (M + kRowGroups - 1) / kRowGroups;
+  if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
+  minimax_generic_kernel<T><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(d, lo, hi, M, D);
   ACTNN_RETURN_LAUNCH_STATUS();
 }
 

@@ -10,9 +10,11 @@
 // elements (one 16-byte load for 16-bit types, two for f32), quantises them and
 // concatenates the 8 codes into 8*b bits of a register (several groups share a register
 // when 8*b <= 16).  One 32x32 bit transpose per register (5 exchange stages) then leaves
-// word p in lane p, which is stored coalesced.  A 256-thread block handles 32 groups of one
-// sample (4 per half-wave, all loads issued before any arithmetic); their 32 scales are
-// computed by the first 32 threads and shared through LDS.
+// word p in lane p, which is stored coalesced.  A 256-thread block handles 16 groups of one
+// sample (2 per half-wave); the element loads are issued first, the block's scales are
+// computed by the first threads and shared through LDS while the loads are in flight.
+// unpack mirrors this; its fp32 stores go through LDS so that each store instruction of a
+// wave writes one whole 1 KiB group.
 //
 // Other group sizes (multiples of 32 up to 1024) take a simple LDS-staged kernel.
 #include "quant_math.h"
@@ -20,44 +22,147 @@
 namespace actnn {
 namespace {
 
+#ifndef ACTNN_PACK_GPH
+#define ACTNN_PACK_GPH 2      // groups per half-wave and block (1, 2 or 4)
+#endif
+#ifndef ACTNN_UNPACK_GPH
+#define ACTNN_UNPACK_GPH 2
+#endif
+
 constexpr int kThreads = 256;
 constexpr int kHalfWaves = kThreads / 32;
-constexpr int kGroupsPerHalf = 4;
-constexpr int kGroupsPerBlock = kHalfWaves * kGroupsPerHalf;   // 32
 constexpr int kGs = 256;
 
-template <int BITS> struct Tile {
+template <int BITS, int GPH> struct Tile {
   static constexpr int kWordsPerGroup = 8 * BITS;
-  static constexpr int kGroupsPerReg = BITS == 1 ? 4 : BITS == 2 ? 2 : 1;   // groups sharing one transpose
+  // consecutive groups that share one register (one transpose): as many as fit in 32 bits
+  static constexpr int kFit = BITS == 1 ? 4 : BITS == 2 ? 2 : 1;
+  static constexpr int kGroupsPerReg = kFit < GPH ? kFit : GPH;
   static constexpr bool kTwoRegs = BITS > 4;                                  // 8*BITS > 32
+  // Group (within the block) that half-wave hw handles in its q-th slot: GPH consecutive groups
+  // per half-wave, whatever the bit width, so that loads can be issued before the width is known.
+  static __device__ __forceinline__ int group_of(int hw, int q) { return hw * GPH + q; }
 };
 
+// fp32: move the 32-byte-per-lane ownership through LDS so that HBM sees whole-line accesses.
+// Measured on MI355X: a clear win for the stores of unpack, a loss for the loads of pack.
+#ifndef ACTNN_PACK_LDS_STAGE
+#define ACTNN_PACK_LDS_STAGE 0
+#endif
+#ifndef ACTNN_PACK_STAGE_OUT
+#define ACTNN_PACK_STAGE_OUT 0     // measured: no gain over direct 4-byte stores
+#endif
+#ifndef ACTNN_UNPACK_LDS_STAGE
+#define ACTNN_UNPACK_LDS_STAGE 1
+#endif
+
+// fp32 groups: a lane owns 32 contiguous bytes, which as direct loads would be two half-used
+// 16-byte accesses per cache line.  Instead each wave reads a whole 1 KiB group per load
+// instruction (64 lanes x 16 bytes, non-temporal), parks it in its private LDS slab and every
+// lane picks up its own 32 bytes from there.  Only lanes of one wave exchange data, so no block
+// barrier is needed: LDS operations of a wave complete in order.
+template <int GPH, typename TL>
+ACTNN_DEV void stage_in_f32(const float* __restrict__ data, int64_t elem_base, int groups_valid,
+                            u32x4* __restrict__ slab, float (&v)[GPH][8]) {
+  const int wl = threadIdx.x & 63;          // lane in the wave
+  const int w = threadIdx.x >> 6;
+  const int h = (threadIdx.x >> 5) & 1;
+  const uint32_t lane = threadIdx.x & 31;
+  u32x4 reg[2 * GPH];
+#pragma unroll
+  for (int i = 0; i < 2 * GPH; ++i) {
+    const int gl = TL::group_of(2 * w + i / GPH, i % GPH);
+    reg[i] = (u32x4){0u, 0u, 0u, 0u};
+    if (gl < groups_valid) reg[i] = load16_nt(data + elem_base + (int64_t)gl * kGs + wl * 4);
+  }
+#pragma unroll
+  for (int i = 0; i < 2 * GPH; ++i) slab[i * 64 + wl] = reg[i];
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int q = 0; q < GPH; ++q) {
+    const u32x4 a = slab[(h * GPH + q) * 64 + 2 * lane];
+    const u32x4 b = slab[(h * GPH + q) * 64 + 2 * lane + 1];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      v[q][k] = as_float(a[k]);
+      v[q][4 + k] = as_float(b[k]);
+    }
+  }
+}
+
+// Mirror image for the fp32 output of unpack: lanes park their 8 values, the wave stores whole
+// 1 KiB groups with one instruction each.
+template <int GPH, typename TL>
+ACTNN_DEV void stage_out_f32(float* __restrict__ out, int64_t elem_base, int groups_valid,
+                             u32x4* __restrict__ slab, const float (&v)[GPH][8]) {
+  const int wl = threadIdx.x & 63;
+  const int w = threadIdx.x >> 6;
+  const int h = (threadIdx.x >> 5) & 1;
+  const uint32_t lane = threadIdx.x & 31;
+#pragma unroll
+  for (int q = 0; q < GPH; ++q) {
+    u32x4 a, b;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      a[k] = as_uint(v[q][k]);
+      b[k] = as_uint(v[q][4 + k]);
+    }
+    slab[(h * GPH + q) * 64 + 2 * lane] = a;
+    slab[(h * GPH + q) * 64 + 2 * lane + 1] = b;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int i = 0; i < 2 * GPH; ++i) {
+    const int gl = TL::group_of(2 * w + i / GPH, i % GPH);
+    if (gl < groups_valid) store16(out + elem_base + (int64_t)gl * kGs + wl * 4, slab[i * 64 + wl]);
+  }
+}
+
+template <typename T> struct IsF32 { static constexpr bool value = false; };
+template <> struct IsF32<float> { static constexpr bool value = true; };
+
 // ---------------------------------------------------------------------------- pack (gs = 256)
+// Issue the loads of this lane's elements (and noise in deterministic mode) for its GPH groups.
+template <typename T, bool DET, int GPH>
+ACTNN_DEV void load_groups(const T* __restrict__ data, const T* __restrict__ noise, int64_t elem_base,
+                           int groups_valid, u32x4* slab, float (&v)[GPH][8],
+                           float (&nz)[DET ? GPH : 1][8]) {
+  using TL = Tile<1, GPH>;
+  const uint32_t lane = threadIdx.x & 31;
+  const int hw = threadIdx.x >> 5;
+  constexpr bool kStage = ACTNN_PACK_LDS_STAGE && IsF32<T>::value;
+  if constexpr (kStage)
+    stage_in_f32<GPH, TL>(reinterpret_cast<const float*>(data), elem_base, groups_valid, slab, v);
+#pragma unroll
+  for (int q = 0; q < GPH; ++q) {
+    const int gl = TL::group_of(hw, q);
+    if (gl < groups_valid) {
+      const int64_t e = elem_base + (int64_t)gl * kGs + lane * 8;
+      if constexpr (!kStage) load8(data + e, v[q]);
+      if (DET) load8(noise + e, nz[DET ? q : 0]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) { if (!kStage) v[q][k] = 0.0f; if (DET) nz[DET ? q : 0][k] = 0.0f; }
+    }
+  }
+}
+
 template <typename T, int BITS, bool DET>
-ACTNN_DEV void pack_groups(const T* __restrict__ data, const T* __restrict__ noise,
+ACTNN_DEV void pack_groups(const float (&v)[ACTNN_PACK_GPH][8], const float (&nz)[DET ? ACTNN_PACK_GPH : 1][8],
                            int32_t* __restrict__ packed, int64_t elem_base, int64_t word_base,
                            int groups_valid, const float* s_mul, const float* s_sub,
-                           uint64_t seed, uint64_t offset) {
-  using TL = Tile<BITS>;
+                           uint64_t seed, uint64_t offset, u32x4* s_out) {
+  constexpr int kGroupsPerHalf = ACTNN_PACK_GPH;
+  using TL = Tile<BITS, kGroupsPerHalf>;
   constexpr int R = TL::kGroupsPerReg;
   constexpr int WPG = TL::kWordsPerGroup;
   constexpr float Bf = (float)((1 << BITS) - 1);
   const uint32_t lane = threadIdx.x & 31;
-  const int gl0 = (threadIdx.x >> 5) * kGroupsPerHalf;
-
-  float v[kGroupsPerHalf][8];
-  float nz[DET ? kGroupsPerHalf : 1][8];
-#pragma unroll
-  for (int q = 0; q < kGroupsPerHalf; ++q) {
-    if (gl0 + q < groups_valid) {
-      const int64_t e = elem_base + (int64_t)(gl0 + q) * kGs + lane * 8;
-      load8(data + e, v[q]);
-      if (DET) load8(noise + e, nz[DET ? q : 0]);
-    } else {
-#pragma unroll
-      for (int k = 0; k < 8; ++k) { v[q][k] = 0.0f; if (DET) nz[DET ? q : 0][k] = 0.0f; }
-    }
-  }
+  const int hw = threadIdx.x >> 5;
 
 #pragma unroll
   for (int q0 = 0; q0 < kGroupsPerHalf; q0 += R) {
@@ -65,10 +170,11 @@ ACTNN_DEV void pack_groups(const T* __restrict__ data, const T* __restrict__ noi
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int q = q0 + r;
-      const float mul = s_mul[gl0 + q];
-      const float sub = s_sub[gl0 + q];
+      const int gl = TL::group_of(hw, q);
+      const float mul = s_mul[gl];
+      const float sub = s_sub[gl];
       uint32_t r16[8];
-      if (!DET) philox_octet((uint64_t)(elem_base >> 3) + (uint64_t)(gl0 + q) * 32 + lane, seed, offset, r16);
+      if (!DET) philox_octet((uint64_t)(elem_base >> 3) + (uint64_t)gl * 32 + lane, seed, offset, r16);
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
         const uint32_t c = DET ? det_code<T>(v[q][k], nz[DET ? q : 0][k], mul, sub, Bf)
@@ -76,18 +182,28 @@ ACTNN_DEV void pack_groups(const T* __restrict__ data, const T* __restrict__ noi
         acc |= (uint64_t)c << (r * WPG + k * BITS);
       }
     }
-    const int64_t tile_words = word_base + (int64_t)(gl0 + q0) * WPG;
+    const int glt = TL::group_of(hw, q0);            // first group of this register tile
+    const int64_t tile_words = word_base + (int64_t)glt * WPG;
     const uint32_t lo = transpose32((uint32_t)acc, lane);
+    // ACTNN_PACK_STAGE_OUT: words go to LDS first and the block writes them as one contiguous
+    // run of 16-byte stores; otherwise each half-wave stores its own 4-byte words.
+    int32_t* dst = ACTNN_PACK_STAGE_OUT ? reinterpret_cast<int32_t*>(s_out) + glt * WPG : packed + tile_words;
     if (TL::kTwoRegs) {
       const uint32_t hi = transpose32((uint32_t)(acc >> 32), lane);
-      if (gl0 + q0 < groups_valid) {
-        packed[tile_words + lane] = (int32_t)lo;
-        if ((int)lane < WPG - 32) packed[tile_words + 32 + lane] = (int32_t)hi;
+      if (glt < groups_valid) {
+        dst[lane] = (int32_t)lo;
+        if ((int)lane < WPG - 32) dst[32 + lane] = (int32_t)hi;
       }
     } else {
-      if ((int)lane < R * WPG && gl0 + q0 + (int)lane / WPG < groups_valid)
-        packed[tile_words + lane] = (int32_t)lo;
+      if ((int)lane < R * WPG && glt + (int)lane / WPG < groups_valid)
+        dst[lane] = (int32_t)lo;
     }
+  }
+  if (ACTNN_PACK_STAGE_OUT) {
+    __syncthreads();
+    const int total_vec = groups_valid * WPG / 4;          // 16-byte vectors of this block's output
+    if ((int)threadIdx.x < total_vec)
+      store16(packed + word_base + threadIdx.x * 4, s_out[threadIdx.x]);
   }
 }
 
@@ -97,13 +213,26 @@ __global__ __launch_bounds__(kThreads) void pack_mixed_kernel(
     const int32_t* __restrict__ bits, const int32_t* __restrict__ prefix, T* __restrict__ scale,
     int32_t* __restrict__ packed, const T* __restrict__ noise, uint64_t seed, uint64_t offset,
     int64_t G, int blocks_per_sample) {
+  constexpr int GPH = ACTNN_PACK_GPH;
+  constexpr int kGroupsPerBlock = kHalfWaves * GPH;
   __shared__ float s_mul[kGroupsPerBlock];
   __shared__ float s_sub[kGroupsPerBlock];
+  constexpr bool kStage = ACTNN_PACK_LDS_STAGE && IsF32<T>::value;
+  __shared__ u32x4 s_slab[kStage ? kGroupsPerBlock * 64 : 1];     // 1 KiB per group
+  u32x4* slab = s_slab + (kStage ? (threadIdx.x >> 6) * (2 * GPH * 64) : 0);
+  __shared__ u32x4 s_out[ACTNN_PACK_STAGE_OUT ? kGroupsPerBlock * 16 : 1];    // up to 64 words per group
   const int64_t n = blockIdx.x / blocks_per_sample;
   const int64_t gb = (int64_t)(blockIdx.x % blocks_per_sample) * kGroupsPerBlock;
-  const int b = bits[n];
   const int groups_valid = (int)((G - gb) < kGroupsPerBlock ? (G - gb) : kGroupsPerBlock);
+  const int64_t elem_base = (n * G + gb) * kGs;
 
+  // The element loads do not depend on the bit width or the scales: get them in flight first,
+  // then compute the block's scales while they travel.
+  float v[GPH][8];
+  float nz[DET ? GPH : 1][8];
+  load_groups<T, DET, GPH>(data, noise, elem_base, groups_valid, slab, v, nz);
+
+  const int b = bits[n];
   if (threadIdx.x < kGroupsPerBlock) {
     float mul = 0.0f, sub = 0.0f;
     if ((int)threadIdx.x < groups_valid) {
@@ -116,13 +245,12 @@ __global__ __launch_bounds__(kThreads) void pack_mixed_kernel(
   }
   __syncthreads();
 
-  const int64_t elem_base = (n * G + gb) * kGs;
   const int64_t word_base = (int64_t)prefix[n] * G * 8 + gb * 8 * b;
   switch (b) {
 #define ACTNN_CASE(B_)                                                                          \
   case B_:                                                                                      \
-    pack_groups<T, B_, DET>(data, noise, packed, elem_base, word_base, groups_valid, s_mul,     \
-                            s_sub, seed, offset);                                               \
+    pack_groups<T, B_, DET>(v, nz, packed, elem_base, word_base, groups_valid, s_mul, s_sub,    \
+                            seed, offset, s_out);                                               \
     break;
     ACTNN_CASE(1) ACTNN_CASE(2) ACTNN_CASE(3) ACTNN_CASE(4)
     ACTNN_CASE(5) ACTNN_CASE(6) ACTNN_CASE(7) ACTNN_CASE(8)
@@ -135,28 +263,31 @@ __global__ __launch_bounds__(kThreads) void pack_mixed_kernel(
 template <typename T, int BITS>
 ACTNN_DEV void unpack_groups(const int32_t* __restrict__ packed, T* __restrict__ out,
                              int64_t elem_base, int64_t word_base, int groups_valid,
-                             const float* s_scale, const float* s_min) {
-  using TL = Tile<BITS>;
+                             const float* s_scale, const float* s_min, u32x4* slab) {
+  constexpr int kGroupsPerHalf = ACTNN_UNPACK_GPH;
+  constexpr bool kStage = ACTNN_UNPACK_LDS_STAGE && IsF32<T>::value;
+  float vs[kStage ? kGroupsPerHalf : 1][8];
+  using TL = Tile<BITS, kGroupsPerHalf>;
   constexpr int R = TL::kGroupsPerReg;
   constexpr int WPG = TL::kWordsPerGroup;
   constexpr uint32_t kMask = (1u << BITS) - 1u;
   const uint32_t lane = threadIdx.x & 31;
-  const int gl0 = (threadIdx.x >> 5) * kGroupsPerHalf;
+  const int hw = threadIdx.x >> 5;
 
   uint32_t wlo[kGroupsPerHalf / R], whi[kGroupsPerHalf / R];
 #pragma unroll
   for (int t = 0; t < kGroupsPerHalf / R; ++t) {
-    const int q0 = t * R;
-    const int64_t tile_words = word_base + (int64_t)(gl0 + q0) * WPG;
+    const int glt = TL::group_of(hw, t * R);
+    const int64_t tile_words = word_base + (int64_t)glt * WPG;
     wlo[t] = 0;
     whi[t] = 0;
     if (TL::kTwoRegs) {
-      if (gl0 + q0 < groups_valid) {
+      if (glt < groups_valid) {
         wlo[t] = (uint32_t)packed[tile_words + lane];
         if ((int)lane < WPG - 32) whi[t] = (uint32_t)packed[tile_words + 32 + lane];
       }
     } else {
-      if ((int)lane < R * WPG && gl0 + q0 + (int)lane / WPG < groups_valid)
+      if ((int)lane < R * WPG && glt + (int)lane / WPG < groups_valid)
         wlo[t] = (uint32_t)packed[tile_words + lane];
     }
   }
@@ -167,10 +298,10 @@ ACTNN_DEV void unpack_groups(const int32_t* __restrict__ packed, T* __restrict__
     if (TL::kTwoRegs) acc |= (uint64_t)transpose32(whi[t], lane) << 32;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const int q = q0 + r;
-      if (gl0 + q < groups_valid) {
-        const float sc = s_scale[gl0 + q];
-        const float m = s_min[gl0 + q];
+      const int gl = TL::group_of(hw, q0 + r);
+      if (gl < groups_valid) {
+        const float sc = s_scale[gl];
+        const float m = s_min[gl];
         float v[8];
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
@@ -178,10 +309,17 @@ ACTNN_DEV void unpack_groups(const int32_t* __restrict__ packed, T* __restrict__
           // (scalar_t)val / scale + min, one rounding per operation (.cu:171)
           v[k] = Conv<T>::round(Conv<T>::round((float)c / sc) + m);
         }
-        store8(out + elem_base + (int64_t)(gl0 + q) * kGs + lane * 8, v);
+        if constexpr (kStage) {
+#pragma unroll
+          for (int k = 0; k < 8; ++k) vs[kStage ? q0 + r : 0][k] = v[k];
+        } else {
+          store8(out + elem_base + (int64_t)gl * kGs + lane * 8, v);
+        }
       }
     }
   }
+  if constexpr (kStage)
+    stage_out_f32<kGroupsPerHalf, TL>(reinterpret_cast<float*>(out), elem_base, groups_valid, slab, vs);
 }
 
 template <typename T>
@@ -189,8 +327,12 @@ __global__ __launch_bounds__(kThreads) void unpack_mixed_kernel(
     const int32_t* __restrict__ packed, const int32_t* __restrict__ bits,
     const int32_t* __restrict__ prefix, const T* __restrict__ scale, const T* __restrict__ mn,
     T* __restrict__ out, int64_t G, int blocks_per_sample) {
+  constexpr int kGroupsPerBlock = kHalfWaves * ACTNN_UNPACK_GPH;
   __shared__ float s_scale[kGroupsPerBlock];
   __shared__ float s_min[kGroupsPerBlock];
+  constexpr bool kStage = ACTNN_UNPACK_LDS_STAGE && IsF32<T>::value;
+  __shared__ u32x4 s_slab[kStage ? kGroupsPerBlock * 64 : 1];
+  u32x4* slab = s_slab + (kStage ? (threadIdx.x >> 6) * (2 * ACTNN_UNPACK_GPH * 64) : 0);
   const int64_t n = blockIdx.x / blocks_per_sample;
   const int64_t gb = (int64_t)(blockIdx.x % blocks_per_sample) * kGroupsPerBlock;
   const int b = bits[n];
@@ -206,7 +348,7 @@ __global__ __launch_bounds__(kThreads) void unpack_mixed_kernel(
   switch (b) {
 #define ACTNN_CASE(B_)                                                                          \
   case B_:                                                                                      \
-    unpack_groups<T, B_>(packed, out, elem_base, word_base, groups_valid, s_scale, s_min);      \
+    unpack_groups<T, B_>(packed, out, elem_base, word_base, groups_valid, s_scale, s_min, slab); \
     break;
     ACTNN_CASE(1) ACTNN_CASE(2) ACTNN_CASE(3) ACTNN_CASE(4)
     ACTNN_CASE(5) ACTNN_CASE(6) ACTNN_CASE(7) ACTNN_CASE(8)
@@ -327,6 +469,7 @@ int launch_pack(const void* data, const void* mn, const void* mx, const int32_t*
   const T* d = static_cast<const T*>(data);
   const T* nz = static_cast<const T*>(noise);
   if (gs == kGs) {
+    constexpr int kGroupsPerBlock = kHalfWaves * ACTNN_PACK_GPH;
     const int64_t bps = (G + kGroupsPerBlock - 1) / kGroupsPerBlock;
     if (N * bps > 0x7fffffffLL) return ACTNN_EINVAL;
     const dim3 grid((unsigned)(N * bps));
@@ -358,6 +501,7 @@ int launch_unpack(const int32_t* packed, const int32_t* bits, const int32_t* pre
                   const void* scale, const void* mn, void* out, int64_t N, int64_t G, int64_t gs,
                   hipStream_t s) {
   if (gs == kGs) {
+    constexpr int kGroupsPerBlock = kHalfWaves * ACTNN_UNPACK_GPH;
     const int64_t bps = (G + kGroupsPerBlock - 1) / kGroupsPerBlock;
     if (N * bps > 0x7fffffffLL) return ACTNN_EINVAL;
     unpack_mixed_kernel<T><<<dim3((unsigned)(N * bps)), dim3(kThreads), 0, s>>>(

@@ -28,7 +28,12 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, then WRITE_SIZE, each scaled by
 # what the same counter reads for actnn_stream_copy of a known size); see profiles/.  None = not
 # measured yet.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # profiles/config2_minimax_pack_unpack_mixed_f32.txt (fetch factor 2.0, write factor 1.0)
+    "minimax": 828817676,
+    "pack_mixed": 883218157,
+    "unpack_mixed": 880260916,
+}
 
 
 def _event_time_ms(fn, reps, warmup=3):
