@@ -1,0 +1,201 @@
+"""Drop-in nn.Module layers that keep their saved activations compressed (behaviour of the
+reference's actnn/actnn/layers.py; conv-transpose and sync-BN variants are not part of this build).
+
+Under torch.autocast the custom autograd functions receive their floating-point arguments already
+cast to the autocast dtype (autocast does not look inside custom Functions); the reference
+predates autocast, this is the one addition here.
+"""
+import warnings
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch.nn.modules.pooling import _AvgPoolNd, _MaxPoolNd
+from torch.nn.modules.utils import _pair, _single, _triple
+
+from .conf import config
+from .cpp_extension import quantization as ext_quantization
+from .ops import batch_norm, conv1d, conv2d, conv3d, linear
+from .qbnscheme import QBNScheme
+from .qscheme import QScheme
+
+
+def _autocast_apply(fn, *args):
+    """Run fn.apply(*args); inside an autocast region cast float tensors to the autocast dtype
+    first and switch autocast off for the call."""
+    if torch.is_autocast_enabled():
+        dt = torch.get_autocast_gpu_dtype()
+        args = tuple(a.to(dt) if isinstance(a, torch.Tensor) and a.is_floating_point() and a.is_cuda else a
+                     for a in args)
+        with torch.autocast(device_type="cuda", enabled=False):
+            return fn.apply(*args)
+    return fn.apply(*args)
+
+
+def _num_locations(kernel_size, dims):
+    if isinstance(kernel_size, int):
+        return kernel_size ** dims
+    n = 1
+    for k in kernel_size[:dims]:
+        n *= k
+    return n
+
+
+class _QConvMixin:
+    """Shared by QConv1d/2d/3d: scheme registration and the training-time dispatch."""
+    _dims = 2
+    _function = conv2d
+    _zero_pad = staticmethod(_pair)
+
+    def _init_scheme(self, kernel_size, groups, group):
+        if config.adaptive_conv_scheme:
+            self.scheme = QScheme(self, num_locations=_num_locations(kernel_size, self._dims), group=group,
+                                  depthwise_groups=groups)
+        else:
+            self.scheme = None
+
+    def forward(self, input):
+        if not config.training:
+            return super().forward(input)
+        if self.padding_mode != "zeros":
+            input = F.pad(input, self._reversed_padding_repeated_twice, mode=self.padding_mode)
+            padding = self._zero_pad(0)
+        else:
+            padding = self.padding
+        return _autocast_apply(self._function, input, self.weight, self.bias, self.stride, padding,
+                               self.dilation, self.groups, self.scheme)
+
+
+class QConv1d(_QConvMixin, nn.Conv1d):
+    _dims, _function, _zero_pad = 1, conv1d, staticmethod(_single)
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
+                 groups=1, bias=True, padding_mode="zeros", group=0):
+        super().__init__(in_channels, out_channels, kernel_size, stride, padding, dilation, groups,
+                         bias, padding_mode)
+        self._init_scheme(kernel_size, groups, group)
+
+
+class QConv2d(_QConvMixin, nn.Conv2d):
+    _dims, _function, _zero_pad = 2, conv2d, staticmethod(_pair)
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
+                 groups=1, bias=True, padding_mode="zeros", group=0):
+        super().__init__(in_channels, out_channels, kernel_size, stride, padding, dilation, groups,
+                         bias, padding_mode)
+        self._init_scheme(kernel_size, groups, group)
+
+
+class QConv3d(_QConvMixin, nn.Conv3d):
+    _dims, _function, _zero_pad = 3, conv3d, staticmethod(_triple)
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
+                 groups=1, bias=True, padding_mode="zeros", group=0):
+        super().__init__(in_channels, out_channels, kernel_size, stride, padding, dilation, groups,
+                         bias, padding_mode)
+        self._init_scheme(kernel_size, groups, group)
+
+
+class QLinear(nn.Linear):
+    num_layers = 0
+
+    def __init__(self, input_features, output_features, bias=True, group=0):
+        super().__init__(input_features, output_features, bias)
+        self.scheme = QScheme(self, group=group) if config.adaptive_conv_scheme else None
+
+    def forward(self, input):
+        if not config.training:
+            return super().forward(input)
+        return _autocast_apply(linear, input, self.weight, self.bias, self.scheme)
+
+
+class _QBatchNormMixin:
+    def _init_scheme(self, group):
+        self.scheme = QBNScheme(group=group) if config.adaptive_bn_scheme else None
+
+    def forward(self, input):
+        if not config.training:
+            return super().forward(input)
+        self._check_input_dim(input)
+        factor = 0.0 if self.momentum is None else self.momentum
+        if self.training and self.track_running_stats and self.num_batches_tracked is not None:
+            self.num_batches_tracked = self.num_batches_tracked + 1
+            factor = 1.0 / float(self.num_batches_tracked) if self.momentum is None else self.momentum
+        # batch statistics in training mode, and in eval mode when there are no running buffers
+        bn_training = True if self.training else (self.running_mean is None and self.running_var is None)
+        keep_buffers = (not self.training) or self.track_running_stats
+        # statistics and affine parameters stay fp32 under autocast (mixed-precision batch norm)
+        return batch_norm.apply(input, self.running_mean if keep_buffers else None,
+                                self.running_var if keep_buffers else None, self.weight, self.bias,
+                                bn_training, factor, self.eps, self.scheme)
+
+
+class QBatchNorm1d(_QBatchNormMixin, nn.BatchNorm1d):
+    def __init__(self, num_features, eps=1e-05, momentum=0.1, affine=True, track_running_stats=True, group=0):
+        super().__init__(num_features, eps, momentum, affine, track_running_stats)
+        self._init_scheme(group)
+
+
+class QBatchNorm2d(_QBatchNormMixin, nn.BatchNorm2d):
+    def __init__(self, num_features, eps=1e-05, momentum=0.1, affine=True, track_running_stats=True, group=0):
+        super().__init__(num_features, eps, momentum, affine, track_running_stats)
+        self._init_scheme(group)
+
+
+class QBatchNorm3d(_QBatchNormMixin, nn.BatchNorm3d):
+    def __init__(self, num_features, eps=1e-05, momentum=0.1, affine=True, track_running_stats=True, group=0):
+        super().__init__(num_features, eps, momentum, affine, track_running_stats)
+        self._init_scheme(group)
+
+
+class QReLU(nn.Module):
+    """ReLU that saves a 1-bit mask; used in training and evaluation alike (layers.py:364-369)."""
+
+    def __init__(self, inplace=False):
+        super().__init__()
+
+    def forward(self, input):
+        return ext_quantization.act_quantized_relu(input)
+
+
+class QDropout(nn.Dropout):
+    def __init__(self, p=0.5):
+        super().__init__(p=p)
+
+    def forward(self, input):
+        if self.training:
+            return ext_quantization.act_quantized_dropout(input, self.p)
+        return super().forward(input)
+
+
+class QMaxPool2d(_MaxPoolNd):
+    def __init__(self, kernel_size, stride=None, padding=0, dilation=1, return_indices=False, ceil_mode=False):
+        super().__init__(kernel_size, stride, padding, dilation, return_indices, ceil_mode)
+        self.kernel_size = _pair(kernel_size)
+        self.stride = _pair(stride if stride is not None else kernel_size)
+        self.padding = _pair(padding)
+        self.dilation = _pair(dilation)
+
+    def forward(self, input):
+        return ext_quantization.act_quantized_max_pool2d(input, self.kernel_size, self.stride, self.padding,
+                                                         self.dilation, self.ceil_mode, self.return_indices)
+
+
+class QAvgPool2d(_AvgPoolNd):
+    """The reference has no average-pool kernel and silently runs max-pool instead
+    (layers.py:506-515); that behaviour is kept, with its warning."""
+
+    def __init__(self, kernel_size, stride=None, padding=0, ceil_mode=False, count_include_pad=True,
+                 divisor_override=None):
+        super().__init__()
+        self.kernel_size = _pair(kernel_size)
+        self.stride = _pair(stride if stride is not None else kernel_size)
+        self.padding = _pair(padding)
+        self.ceil_mode = ceil_mode
+        self.count_include_pad = count_include_pad
+        self.divisor_override = divisor_override
+
+    def forward(self, input):
+        warnings.warn("avg_pool2d is replaced by max_pool2d: no memory-saving average-pool kernel exists.")
+        return ext_quantization.act_quantized_max_pool2d(input, self.kernel_size, self.stride, self.padding,
+                                                         (1, 1), self.ceil_mode, False)

@@ -1,0 +1,283 @@
+"""Autograd functions that keep their input compressed between forward and backward, and the
+quantise / dequantise glue around the kernels (behaviour of the reference's
+actnn/actnn/ops.py:22-502; conv-transpose, sync-BN and adaptive pooling variants are not part
+of this build).
+"""
+import numpy as np
+import torch
+import torch.nn.functional as F
+from torch.autograd.function import Function
+from torch.nn.modules.utils import _pair, _single, _triple
+
+from .conf import config
+from .cpp_extension import backward_func as ext_backward_func
+from .cpp_extension import quantization as ext_quantization
+from .utils import compute_tensor_bytes, empty_cache, get_memory_usage, swap_to_cpu
+
+
+# ------------------------------------------------------------------------------------------
+# quantise / dequantise
+# ------------------------------------------------------------------------------------------
+def quantize_and_pack(data, bits, mn, mx):
+    """data [N,G,gs] -> (packed stream or simulated codes, scale [N,G,1])  (ops.py:22-52)."""
+    if config.simulate:
+        # the reference's pure-torch quantiser, run on the tensor's own device (ops.py:23-41)
+        N = data.shape[0]
+        if isinstance(bits, int):
+            bits = torch.ones(N, dtype=torch.int32, device=data.device) * bits
+        B = (2 ** bits - 1).view(N, 1, 1)
+        mn = mn - 1e-6
+        mx = mx + 1e-6
+        scale = B / (mx - mn)
+        output = (data - mn) * scale
+        if config.stochastic:
+            output.add_(output.new(output.shape).uniform_(-0.5, 0.5))
+        output = F.relu(output)
+        output = torch.min(output, B.float()).round_().int()
+        return output, scale
+    pack = ext_quantization.pack_single_precision if isinstance(bits, int) \
+        else ext_quantization.pack_mixed_precision
+    output, scale = pack(data, mn, mx, bits, config.stochastic)
+    if config.swap:
+        output = swap_to_cpu(output)
+    return output, scale
+
+
+def dequantize_and_unpack(data, shape, bits, scale, mn):
+    """Inverse of quantize_and_pack; returns [N, G, gs] in the dtype of scale (ops.py:55-74)."""
+    if config.simulate:
+        return data / scale + mn
+    if config.swap:
+        data = data.cuda(non_blocking=True)
+    N = shape[0]
+    gs = config.group_size
+    features = int(np.prod(shape[1:]))
+    features = features + (gs - features % gs) % gs
+    unpack = ext_quantization.unpack_single_precision if isinstance(bits, int) \
+        else ext_quantization.unpack_mixed_precision
+    return unpack(data, bits, scale, mn, N, features // gs, gs)
+
+
+def no_scheme_compute_quantization_bits(input):
+    """Fixed width for every sample when no scheme is attached (ops.py:77-96)."""
+    from .qscheme import group_min_max
+    N = input.shape[0]
+    groups, mn, mx, _ = group_min_max(input)
+    return groups, config.activation_compression_bits[0], mn.view(N, -1, 1), mx.view(N, -1, 1)
+
+
+def quantize_activation(input, scheme):
+    """-> (q_input, q_bits, q_scale, q_min); for fp32 activations scale and min are kept as
+    bfloat16 (ops.py:99-118)."""
+    if not config.compress_activation:
+        return (swap_to_cpu(input) if config.swap else input), None, None, None
+    if scheme:
+        groups, q_bits, q_min, mx = scheme.compute_quantization_bits(input)
+    else:
+        groups, q_bits, q_min, mx = no_scheme_compute_quantization_bits(input)
+    q_input, q_scale = quantize_and_pack(groups, q_bits, q_min, mx)
+    if input.dtype == torch.float32:
+        return q_input, q_bits, q_scale.to(torch.bfloat16), q_min.to(torch.bfloat16)
+    return q_input, q_bits, q_scale, q_min
+
+
+def dequantize_activation(quantized, q_input_shape):
+    """Rebuild a tensor of shape q_input_shape (ops.py:121-139)."""
+    if not config.compress_activation:
+        ret = quantized[0]
+        return ret.cuda(non_blocking=True) if config.swap else ret
+    q_input, q_bits, q_scale, q_min = quantized
+    if q_scale.dtype == torch.bfloat16 and _stored_as_bf16(q_input_shape, quantized):
+        q_scale = q_scale.to(torch.float32)
+        q_min = q_min.to(torch.float32)
+    out = dequantize_and_unpack(q_input, q_input_shape, q_bits, q_scale, q_min)
+    N = q_input_shape[0]
+    features = int(np.prod(q_input_shape[1:]))
+    out = out.view(N, -1)[:, :features]
+    return out.reshape(*q_input_shape).contiguous()
+
+
+def _stored_as_bf16(shape, quantized):
+    """True when bf16 scale/min are the compact storage of an fp32 activation (to be widened
+    before unpacking, ops.py:129-131) rather than the native dtype of a bf16 activation - a case
+    the reference, which knows f32/f16 only, never meets.  The saved tuple carries the marker."""
+    return not getattr(quantized, "native_bf16", False)
+
+
+class _Quantized(tuple):
+    """(q_input, q_bits, q_scale, q_min) plus a flag telling bf16 activations apart."""
+    native_bf16 = False
+
+
+def quantize_saved(input, scheme):
+    q = _Quantized(quantize_activation(input, scheme))
+    q.native_bf16 = input.dtype == torch.bfloat16
+    return q
+
+
+# ------------------------------------------------------------------------------------------
+# convolution (1d / 2d / 3d share one implementation, ops.py:145-264)
+# ------------------------------------------------------------------------------------------
+conv_layer_ct = 0
+bn_layer_ct = 0
+total_act_mem = 0
+
+
+def _conv_forward(ctx, forward_op, input, weight, bias, stride, padding, dilation, groups, scheme):
+    quantized = quantize_saved(input, scheme)
+    ctx.scheme = scheme
+    ctx.saved = quantized, weight, bias
+    ctx.other_args = (input.shape, stride, padding, dilation, groups)
+    empty_cache(config.empty_cache_threshold)
+    if config.debug_memory_op_forward:
+        global conv_layer_ct, total_act_mem
+        print("========== conv forward %d ==========" % conv_layer_ct)
+        get_memory_usage(True)
+        conv_layer_ct += 1
+        total_act_mem += compute_tensor_bytes(list(quantized))
+        print("Act mem: %.2f MB" % (total_act_mem / 1024 ** 2))
+    return forward_op(input, weight, bias, stride, padding, dilation, groups)
+
+
+def _conv_backward(ctx, grad_output, bias_reduce_dims, aug):
+    if ctx.scheme:
+        ctx.scheme.set_scale(grad_output)
+    q_input_shape, stride, padding, dilation, groups = ctx.other_args
+    padding, stride, dilation = aug(padding), aug(stride), aug(dilation)
+    quantized, weight, bias = ctx.saved
+    input = dequantize_activation(quantized, q_input_shape)
+    del quantized, ctx.saved
+    empty_cache(config.empty_cache_threshold)
+    grad_output = grad_output.contiguous()
+    need = [ctx.needs_input_grad[0], ctx.needs_input_grad[1]]
+
+    ws_mem = compute_tensor_bytes([grad_output, input, input])
+    if config.pipeline_threshold and ws_mem > config.pipeline_threshold and all(need):
+        # micro-batched backward: grad_input overwrites the dequantised input chunk by chunk so
+        # the transient working set stays bounded (ops.py:202-220)
+        chunks = int((ws_mem + config.pipeline_threshold) // config.pipeline_threshold)
+        grad_weight = None
+        for x_i, g_i in zip(torch.chunk(input, chunks), torch.chunk(grad_output, chunks)):
+            gi, gw = ext_backward_func.cudnn_convolution_backward(
+                x_i, g_i, weight, padding, stride, dilation, groups,
+                config.cudnn_benchmark_conv2d, False, False, need)
+            x_i[:] = gi
+            grad_weight = gw if grad_weight is None else grad_weight.add_(gw)
+        grad_input = input
+    else:
+        grad_input, grad_weight = ext_backward_func.cudnn_convolution_backward(
+            input, grad_output, weight, padding, stride, dilation, groups,
+            config.cudnn_benchmark_conv2d, False, False, need)
+    grad_bias = grad_output.sum(bias_reduce_dims) if bias is not None and ctx.needs_input_grad[2] else None
+    if ctx.scheme:
+        ctx.scheme.if_allocate_perlayer()
+    return grad_input, grad_weight, grad_bias, None, None, None, None, None
+
+
+class conv1d(Function):
+    @staticmethod
+    def forward(ctx, input, weight, bias=None, stride=1, padding=0, dilation=1, groups=1, scheme=None):
+        return _conv_forward(ctx, F.conv1d, input, weight, bias, stride, padding, dilation, groups, scheme)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return _conv_backward(ctx, grad_output, [0, 2], _single)
+
+
+class conv2d(Function):
+    @staticmethod
+    def forward(ctx, input, weight, bias=None, stride=1, padding=0, dilation=1, groups=1, scheme=None):
+        return _conv_forward(ctx, F.conv2d, input, weight, bias, stride, padding, dilation, groups, scheme)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return _conv_backward(ctx, grad_output, [0, 2, 3], _pair)
+
+
+class conv3d(Function):
+    @staticmethod
+    def forward(ctx, input, weight, bias=None, stride=1, padding=0, dilation=1, groups=1, scheme=None):
+        return _conv_forward(ctx, F.conv3d, input, weight, bias, stride, padding, dilation, groups, scheme)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return _conv_backward(ctx, grad_output, [0, 2, 3, 4], _triple)
+
+
+# ------------------------------------------------------------------------------------------
+# linear (ops.py:386-433)
+# ------------------------------------------------------------------------------------------
+class linear(Function):
+    @staticmethod
+    def forward(ctx, input, weight, bias=None, scheme=None):
+        quantized = quantize_saved(input, scheme)
+        empty_cache(config.empty_cache_threshold)
+        ctx.scheme = scheme
+        ctx.saved = quantized, weight, bias
+        ctx.other_args = input.shape
+        return F.linear(input, weight, bias)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        if ctx.scheme:
+            ctx.scheme.set_scale(grad_output)
+        quantized, weight, bias = ctx.saved
+        q_input_shape = ctx.other_args
+        input = dequantize_activation(quantized, q_input_shape)
+        del quantized, ctx.saved
+        empty_cache(config.empty_cache_threshold)
+        go = grad_output.reshape(-1, grad_output.shape[-1])
+        x = input.reshape(-1, input.shape[-1])
+        grad_input = go.mm(weight).view(*q_input_shape) if ctx.needs_input_grad[0] else None
+        grad_weight = go.t().mm(x) if ctx.needs_input_grad[1] else None
+        grad_bias = go.sum(0) if bias is not None and ctx.needs_input_grad[2] else None
+        if ctx.scheme:
+            ctx.scheme.if_allocate_perlayer()
+        return grad_input, grad_weight, grad_bias, None
+
+
+# ------------------------------------------------------------------------------------------
+# batch norm (ops.py:436-502)
+# ------------------------------------------------------------------------------------------
+class batch_norm(Function):
+    @staticmethod
+    def forward(ctx, input, running_mean, running_var, weight, bias, training,
+                exponential_average_factor, eps, scheme):
+        quantized = quantize_saved(input, scheme)
+        empty_cache(config.empty_cache_threshold)
+        if config.debug_memory_op_forward:
+            global bn_layer_ct, total_act_mem
+            print("========== bn forward %d ==========" % bn_layer_ct)
+            get_memory_usage(True)
+            bn_layer_ct += 1
+            total_act_mem += compute_tensor_bytes(list(quantized))
+            print("Act mem: %.2f MB" % (total_act_mem / 1024 ** 2))
+        if training:
+            output, save_mean, save_var, reserve = ext_backward_func.cudnn_batch_norm(
+                input, weight, bias, running_mean, running_var, training, exponential_average_factor, eps)
+        else:
+            output, save_mean, save_var = ext_backward_func.native_batch_norm(
+                input, weight, bias, running_mean, running_var, training, exponential_average_factor, eps)
+            reserve = None
+        ctx.scheme = scheme
+        ctx.other_args = input.shape
+        ctx.saved = (quantized, weight, running_mean, running_var, save_mean, save_var, training, eps, reserve)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        quantized, weight, running_mean, running_var, save_mean, save_var, training, eps, reserve = ctx.saved
+        input = dequantize_activation(quantized, ctx.other_args)
+        del quantized, ctx.saved
+        empty_cache(config.empty_cache_threshold)
+        if training:
+            grad_input, grad_weight, grad_bias = ext_backward_func.cudnn_batch_norm_backward(
+                input.contiguous(), grad_output.contiguous(), weight, running_mean, running_var,
+                save_mean, save_var, eps, reserve)
+        else:
+            grad_input, grad_weight, grad_bias = ext_backward_func.native_batch_norm_backward(
+                grad_output, input, weight, running_mean, running_var, save_mean, save_var, training, eps,
+                [ctx.needs_input_grad[0], ctx.needs_input_grad[3], ctx.needs_input_grad[4]])
+        if ctx.scheme:
+            ctx.scheme.if_allocate_perlayer()
+        return grad_input, None, None, grad_weight, grad_bias, None, None, None, None

@@ -1,0 +1,33 @@
+"""Bit allocation for batch-norm inputs (behaviour of actnn/actnn/qbnscheme.py:9-60): the
+sensitivity is the range term alone and the per-layer budget follows the preceding conv/linear."""
+import torch
+
+from .conf import config
+from .qscheme import QScheme, greedy_bits, group_min_max, range_sqr
+
+
+class QBNScheme(QScheme):
+    layers = []
+
+    def __init__(self, group=0):
+        self.initial_bits = config.initial_bits
+        self.bits = config.activation_compression_bits[group]
+        QBNScheme.layers.append(self)
+        self.prev_linear = QScheme.layers[-1] if len(QScheme.layers) > 0 else None
+
+    def compute_quantization_bits(self, input):
+        self.prev_linear = QScheme.prev_layer
+        N = input.shape[0]
+        groups, mn, mx, num_pixels = group_min_max(input)
+        C = range_sqr(mn, mx, N, num_pixels).to(torch.float32).cpu()       # qbnscheme.py:44-47
+        bits_dev, _ = greedy_bits(C, N, self.initial_bits, self.bits, input.device)
+        return groups, bits_dev, mn.view(N, -1, 1), mx.view(N, -1, 1)
+
+    @staticmethod
+    def allocate_perlayer():
+        for layer in QBNScheme.layers:
+            layer.bits = layer.prev_linear.bits if layer.prev_linear is not None else 8
+
+    @staticmethod
+    def reset():
+        QBNScheme.layers = []

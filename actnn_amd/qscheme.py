@@ -1,0 +1,161 @@
+"""Per-sample / per-layer bit allocation policy for conv and linear inputs
+(behaviour of the reference's actnn/actnn/qscheme.py:9-147, restated for this build).
+
+Sensitivity of sample n:  C_n = num_locations / 4 / depthwise_groups * Range_sqr_n * grad_scale
+with Range_sqr_n = ||max - min||^2 over the sample's groups * (group_size / pixels per channel);
+bits come from the greedy allocation `calc_precision` starting at `initial_bits` down to an
+average of `bits` per sample.
+"""
+import torch
+
+from .conf import config
+from .cpp_extension import calc_precision as ext_calc_precision
+from .cpp_extension import minimax as ext_minimax
+from .cpp_extension.quantization import attach_bits_host
+
+
+def group_min_max(input):
+    """Flatten to [N, -1], zero-pad the feature axis to a multiple of group_size, view as groups
+    and reduce each group (qscheme.py:59-74).  Returns (groups [N,G,gs], mn [N*G], mx [N*G],
+    pixels per channel)."""
+    N = input.shape[0]
+    flat = input.reshape(N, -1)
+    features = flat.shape[1]
+    num_pixels = features // input.shape[1]
+    gs = config.group_size
+    if features % gs != 0:
+        padded = (features // gs + 1) * gs
+        flat = torch.cat([flat, torch.zeros(N, padded - features, dtype=input.dtype, device=input.device)], 1)
+    elif not flat.is_contiguous():
+        flat = flat.contiguous()
+    rows = flat.view(-1, gs)
+    mn, mx = ext_minimax.minimax(rows)
+    if not config.pergroup:                     # one range for the whole tensor (qscheme.py:75-77)
+        mn = torch.ones_like(mn) * mn.min()
+        mx = torch.ones_like(mx) * mx.max()
+    return rows.view(N, -1, gs), mn, mx, num_pixels
+
+
+def range_sqr(mn, mx, N, num_pixels):
+    """G * ||R_n||^2 / I  (qscheme.py:80)."""
+    return torch.norm((mx - mn).view(N, -1), dim=1).float().square() * (config.group_size / num_pixels)
+
+
+def greedy_bits(C_host, N, initial_bits, avg_bits, device):
+    """Per-sample widths: calc_precision(b = initial_bits, C, w = 1, target = int(avg_bits * N)),
+    returned on the device with the host copy attached (qscheme.py:86-94)."""
+    b = torch.ones(N, dtype=torch.int32) * int(initial_bits)
+    w = torch.ones(N, dtype=torch.int32)
+    b = ext_calc_precision.calc_precision(b, C_host, w, int(avg_bits * N))
+    return attach_bits_host(b.to(device, non_blocking=True), b), b
+
+
+class QScheme(object):
+    num_samples = 1        # dataset size, only used with config.use_gradient
+    num_layers = 0
+    batch = None           # dataset indices of the current batch (config.use_gradient)
+    update_scale = True
+    layers = []
+    prev_layer = None
+
+    def __init__(self, layer, group=0, num_locations=1, depthwise_groups=1):
+        self.initial_bits = config.initial_bits
+        self.bits = config.activation_compression_bits[group]
+        if config.use_gradient:
+            assert QScheme.num_samples > 1
+            self.scales = torch.zeros(QScheme.num_samples)
+        else:
+            self.scales = torch.tensor([0.0])
+        QScheme.layers.append(self)
+        self.C = None
+        self.dim = None
+        self.num_locations = num_locations          # kernel positions per output
+        self.depthwise_groups = depthwise_groups
+        self.layer = layer
+        self.group = group
+        self.name = "layer_{}".format(QScheme.num_layers)
+        QScheme.num_layers += 1
+
+    # -- gradient statistics ----------------------------------------------------------------
+    def get_scale(self):
+        if config.use_gradient:
+            assert QScheme.batch is not None
+            scale = self.scales[QScheme.batch].clone()
+            scale[scale == 0] = scale.mean() + 1e-9
+            return scale
+        return self.scales
+
+    def set_scale(self, grad):
+        """Squared gradient norm per sample, kept as a running value (qscheme.py:47-55)."""
+        if not QScheme.update_scale:
+            return
+        sq = grad.reshape(grad.shape[0], -1).float().norm(dim=1).square()
+        if config.use_gradient:
+            assert QScheme.batch is not None
+            self.scales[QScheme.batch] = self.scales[QScheme.batch] * 0.5 + sq.cpu() * 0.5
+        else:
+            self.scales = sq.mean()
+
+    # -- forward-time allocation ------------------------------------------------------------
+    def sensitivity(self, rsq, device):
+        grad_sum = self.get_scale().to(device)
+        return self.num_locations / 4 / self.depthwise_groups * rsq * grad_sum
+
+    def compute_quantization_bits(self, input):
+        QScheme.prev_layer = self
+        N = input.shape[0]
+        groups, mn, mx, num_pixels = group_min_max(input)
+        rsq = range_sqr(mn, mx, N, num_pixels)
+        C = self.sensitivity(rsq, input.device).to(torch.float32).cpu()     # device -> host sync
+        bits_dev, b = greedy_bits(C, N, self.initial_bits, self.bits, input.device)
+        self.C = C
+        self.dim = input.numel() // N
+        self.b = b
+        return groups, bits_dev, mn.view(N, -1, 1), mx.view(N, -1, 1)
+
+    # -- per-layer re-balancing -------------------------------------------------------------
+    @staticmethod
+    def allocate_perlayer():
+        """One greedy pass over all layers of a group (qscheme.py:96-128): either one item per
+        layer (when the group's budget equals initial_bits) or one item per (layer, sample)."""
+        for g, avg in enumerate(config.activation_compression_bits):
+            layers = [l for l in QScheme.layers if l.group == g]
+            L = len(layers)
+            if L == 0:
+                continue
+            if avg == config.initial_bits:
+                C = torch.tensor([float(l.C.sum()) for l in layers])
+                w = torch.tensor([l.dim for l in layers], dtype=torch.int32)
+                b = ext_calc_precision.calc_precision(torch.ones(L, dtype=torch.int32) * 8, C, w,
+                                                      float(w.sum() * avg))
+                for i, l in enumerate(layers):
+                    l.bits = l.initial_bits = b[i]
+            else:
+                N = layers[0].C.shape[0]
+                C = torch.cat([l.C for l in layers], 0)
+                w = torch.cat([torch.ones(N, dtype=torch.int32) * l.dim for l in layers], 0)
+                b = torch.ones(N * L, dtype=torch.int32) * config.initial_bits
+                b = ext_calc_precision.calc_precision(b, C, w, float(w.sum() * avg))
+                for i, l in enumerate(layers):
+                    l.bits = b[i * N:(i + 1) * N].float().mean()
+
+    def if_allocate_perlayer(self):
+        """Called at the end of every layer's backward; the layer whose backward runs last (the
+        first one with a trainable weight) triggers the re-balancing (qscheme.py:130-147)."""
+        if not config.perlayer:
+            return
+        if any(l.C is None for l in QScheme.layers):
+            return
+        first = next((l for l in QScheme.layers if l.layer.weight.requires_grad), None)
+        if config.compress_activation and config.training and self is first:
+            from .qbnscheme import QBNScheme
+            QScheme.allocate_perlayer()
+            QBNScheme.allocate_perlayer()
+
+    @staticmethod
+    def reset():
+        """Forget every registered scheme (build-side helper for tests and repeated model builds)."""
+        QScheme.layers = []
+        QScheme.num_layers = 0
+        QScheme.prev_layer = None
+        QScheme.batch = None

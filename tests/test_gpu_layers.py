@@ -1,0 +1,213 @@
+"""Layer-level behaviour on the GPU: the compressed autograd functions against stock torch layers
+(the reference checks the same things in tests/test_act_quantized_ops.py:318-447 and
+tests/test_linear.py)."""
+import copy
+
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+import actnn_amd
+from actnn_amd import QBNScheme, QModule, QScheme, config, set_optimization_level
+from actnn_amd.ops import dequantize_activation, quantize_saved
+from actnn_amd.resnet import resnet50
+from _util import DEV
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def fresh_config():
+    config.reset()
+    QScheme.reset()
+    QBNScheme.reset()
+    yield
+    config.reset()
+    QScheme.reset()
+    QBNScheme.reset()
+
+
+def _grads(layer, x, g):
+    x = x.clone().requires_grad_(True)
+    y = layer(x)
+    y.backward(g)
+    return y.detach(), x.grad, [p.grad.clone() for p in layer.parameters()]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_conv2d_8bit_close_to_exact(dtype):
+    # per-group 8-bit quantisation of the saved input: gradients within the reference's 8-bit
+    # tolerance of the exact ones (tests/test_act_quantized_ops.py:403-447 uses 1e-1)
+    config.activation_compression_bits = [8]
+    config.initial_bits = 8
+    config.perlayer = False
+    torch.manual_seed(0)
+    N, Cc, H, W = 4, 256, 28, 28
+    q = actnn_amd.QConv2d(Cc, 64, 3, padding=1).to(DEV).to(dtype)
+    ref = nn.Conv2d(Cc, 64, 3, padding=1).to(DEV).to(dtype)
+    ref.load_state_dict(q.state_dict())
+    x = torch.randn(N, Cc, H, W, device=DEV, dtype=dtype)
+    g = torch.randn(N, 64, H, W, device=DEV, dtype=dtype)
+    yq, gxq, gpq = _grads(q, x, g)
+    yr, gxr, gpr = _grads(ref, x, g)
+    # forward is the stock convolution (MIOpen may pick a different algorithm per call)
+    assert torch.allclose(yq.float(), yr.float(), atol=2e-3 if dtype == torch.float32 else 2e-2, rtol=1e-2)
+    tol = 1e-1
+    assert torch.allclose(gxq.float(), gxr.float(), atol=tol, rtol=tol)
+    for a, b in zip(gpq, gpr):
+        rel = (a.float() - b.float()).norm() / b.float().norm()
+        assert rel < 2e-2
+
+
+def test_simulate_and_kernel_paths_agree_statistically():
+    # config.simulate vs the kernels on the same layer (reference: tests/test_act_quantized_ops.py:360-400)
+    config.activation_compression_bits = [8]
+    config.initial_bits = 8
+    config.perlayer = False
+    torch.manual_seed(0)
+    q = actnn_amd.QConv2d(64, 32, 3, padding=1).to(DEV)
+    x = torch.randn(4, 64, 28, 28, device=DEV)
+    g = torch.randn(4, 32, 28, 28, device=DEV)
+    res = []
+    for sim in (True, False):
+        config.simulate = sim
+        q.zero_grad()
+        res.append(_grads(q, x, g))
+    (y0, gx0, gp0), (y1, gx1, gp1) = res
+    assert torch.allclose(y0, y1, atol=2e-3) and torch.allclose(gx0, gx1, atol=2e-3)
+    for a, b in zip(gp0, gp1):
+        assert (a - b).norm() / b.norm() < 2e-2
+
+
+def test_quantize_dequantize_glue_shapes_and_padding():
+    # 300 features per sample -> padded to 512 (2 groups), un-padded on the way back; fp32 keeps
+    # scale/min as bf16 (ops.py:115-116)
+    set_optimization_level("L2")
+    x = torch.randn(6, 3, 10, 10, device=DEV)
+    qd = quantize_saved(x, None)
+    q_input, q_bits, q_scale, q_min = qd
+    assert q_bits == 4 and q_input.dtype == torch.int8
+    assert q_scale.dtype == torch.bfloat16 and q_scale.shape == (6, 2, 1)
+    back = dequantize_activation(qd, x.shape)
+    assert back.shape == x.shape and back.dtype == torch.float32 and back.is_contiguous()
+    rng = (x.view(6, -1).max(1)[0] - x.view(6, -1).min(1)[0]).max()
+    assert (back - x).abs().max() < rng / 15 * 1.1 + 0.05      # one 4-bit step (+ bf16 scale/min rounding)
+
+
+def test_batch_norm_without_compression_matches_torch():
+    config.compress_activation = False
+    torch.manual_seed(0)
+    q = actnn_amd.QBatchNorm2d(16).to(DEV)
+    ref = nn.BatchNorm2d(16).to(DEV)
+    x = torch.randn(8, 16, 14, 14, device=DEV)
+    g = torch.randn_like(x)
+    yq, gxq, gpq = _grads(q, x, g)
+    yr, gxr, gpr = _grads(ref, x, g)
+    assert torch.allclose(yq, yr, atol=1e-3) and torch.allclose(gxq, gxr, atol=1e-3)
+    for a, b in zip(gpq, gpr):
+        assert torch.allclose(a, b, atol=1e-3, rtol=1e-3)
+    assert torch.allclose(q.running_mean, ref.running_mean, atol=1e-5)
+    assert torch.allclose(q.running_var, ref.running_var, atol=1e-5)
+
+
+def test_linear_without_compression_matches_torch():
+    config.compress_activation = False
+    torch.manual_seed(0)
+    q = actnn_amd.QLinear(100, 10).to(DEV)
+    ref = nn.Linear(100, 10).to(DEV)
+    ref.load_state_dict(q.state_dict())
+    x = torch.randn(32, 100, device=DEV)
+    g = torch.randn(32, 10, device=DEV)
+    yq, gxq, gpq = _grads(q, x, g)
+    yr, gxr, gpr = _grads(ref, x, g)
+    assert torch.allclose(yq, yr, atol=1e-5) and torch.allclose(gxq, gxr, atol=1e-5)
+    for a, b in zip(gpq, gpr):
+        assert torch.allclose(a, b, atol=1e-4, rtol=1e-4)
+
+
+def test_l3_first_step_uses_the_degenerate_allocation_then_rebalances():
+    # gradient scale starts at 0 (qscheme.py:24): the first forward gives 8 bits to the first
+    # samples and 1 to the rest; after one backward the scale is positive and bits follow C
+    torch.manual_seed(0)
+    model = QModule(nn.Sequential(nn.Conv2d(8, 8, 3, padding=1), nn.BatchNorm2d(8), nn.ReLU(),
+                                  nn.Conv2d(8, 8, 3, padding=1))).to(DEV)
+    x = torch.randn(16, 8, 16, 16, device=DEV)
+    model(x).square().mean().backward()
+    s0 = QScheme.layers[0]
+    assert s0.b.tolist() == [8, 8, 3] + [1] * 13            # target 32 = 8 + 8 + 3 + 13
+    assert float(s0.scales) > 0
+    budgets = [float(s.bits) for s in QScheme.layers]         # set by the per-layer re-balancing
+    assert abs(sum(budgets) / 2 - 2.0) < 0.26                 # both layers have the same size
+    model(x)
+    assert int(s0.b.sum()) <= int(budgets[0] * 16) and int(s0.b.min()) >= 1
+
+
+def test_small_model_trains_at_l3():
+    # the same toy problem with stock layers and with 2-bit compressed activations: the loss
+    # curves must track each other (the quantisation noise is unbiased)
+    def make():
+        torch.manual_seed(0)
+        return nn.Sequential(nn.Conv2d(3, 16, 3, padding=1), nn.BatchNorm2d(16), nn.ReLU(), nn.MaxPool2d(2),
+                             nn.Conv2d(16, 32, 3, padding=1), nn.BatchNorm2d(32), nn.ReLU(),
+                             nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(32, 10))
+    torch.manual_seed(1)
+    y = torch.randint(0, 10, (64,), device=DEV)
+    pattern = torch.randn(10, 3, 32, 32, device=DEV)
+    x = torch.randn(64, 3, 32, 32, device=DEV) + pattern[y]
+
+    def run(model):
+        model = model.to(DEV)
+        opt = torch.optim.SGD(model.parameters(), lr=0.05, momentum=0.9)
+        losses = []
+        for _ in range(40):
+            opt.zero_grad()
+            loss = F.cross_entropy(model(x), y)
+            loss.backward()
+            opt.step()
+            losses.append(loss.item())
+        return losses
+
+    exact = make()
+    quant = QModule(make())
+    quant.load_state_dict(exact.state_dict())
+    le, lq = run(exact), run(quant)
+    assert lq[-1] < lq[0] - 0.1
+    assert abs(lq[-1] - le[-1]) < 0.05 and max(abs(a - b) for a, b in zip(le, lq)) < 0.1
+
+
+@pytest.mark.parametrize("autocast", [False, True])
+def test_resnet50_step_runs(autocast):
+    torch.manual_seed(0)
+    model = QModule(resnet50()).to(DEV)
+    x = torch.randn(8, 3, 64, 64, device=DEV)
+    y = torch.randint(0, 1000, (8,), device=DEV)
+    for _ in range(2):
+        model.zero_grad()
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+            loss = F.cross_entropy(model(x), y)
+        loss.backward()
+    assert torch.isfinite(loss)
+    grads = [p.grad for p in model.parameters()]
+    assert all(g is not None and torch.isfinite(g).all() for g in grads)
+    assert all(g.dtype == torch.float32 for g in grads)
+
+
+def test_activation_memory_shrinks():
+    # saved-for-backward bytes of one conv+bn+relu stage: L3 (2 bits) vs L0 (masks only)
+    def saved_bytes(level):
+        config.reset(); QScheme.reset(); QBNScheme.reset()
+        set_optimization_level(level)
+        torch.manual_seed(0)
+        model = QModule(nn.Sequential(nn.Conv2d(64, 64, 3, padding=1), nn.BatchNorm2d(64), nn.ReLU(),
+                                      nn.Conv2d(64, 64, 3, padding=1))).to(DEV)
+        x = torch.randn(32, 64, 56, 56, device=DEV)
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_allocated()
+        out = model(x)
+        torch.cuda.synchronize()
+        held = torch.cuda.memory_allocated() - before - out.numel() * 4
+        out.sum().backward()
+        return held
+    full, packed = saved_bytes("L0"), saved_bytes("L3")
+    assert packed < full / 6

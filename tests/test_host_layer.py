@@ -1,0 +1,136 @@
+"""Host-side logic that needs no GPU: configuration levels, model conversion, state-dict
+prefix handling, memory accounting, argument checks of the bindings."""
+import pytest
+import torch
+import torch.nn as nn
+
+import actnn_amd
+from actnn_amd import QBNScheme, QModule, QScheme, config, set_optimization_level
+from actnn_amd.resnet import resnet50
+
+
+@pytest.fixture(autouse=True)
+def fresh_config():
+    config.reset()
+    QScheme.reset()
+    QBNScheme.reset()
+    yield
+    config.reset()
+    QScheme.reset()
+    QBNScheme.reset()
+
+
+def test_defaults_and_levels():
+    assert config.activation_compression_bits == [2, 8, 8] and config.initial_bits == 8
+    assert config.group_size == 256 and config.stochastic and config.compress_activation
+    set_optimization_level("L0")
+    assert not config.compress_activation and not config.adaptive_conv_scheme
+    config.reset()
+    set_optimization_level("L1")
+    assert config.activation_compression_bits == [4] and not config.enable_quantized_bn
+    config.reset()
+    set_optimization_level("L2")
+    assert config.activation_compression_bits == [4] and config.enable_quantized_bn
+    assert not config.adaptive_bn_scheme
+    config.reset()
+    set_optimization_level("L3.1")
+    assert config.pipeline_threshold == 3 * 1024 ** 3 and config.empty_cache_threshold == 0.2
+    config.reset()
+    set_optimization_level("L4")
+    assert config.swap and config.compress_activation
+    config.reset()
+    set_optimization_level("swap")
+    assert config.swap and not config.compress_activation
+    with pytest.raises(ValueError):
+        set_optimization_level("L9")
+
+
+def test_resnet50_conversion_counts():
+    # 53 convs + 1 fc carry a QScheme, 53 batch norms a QBNScheme, 49 ReLU sites, 1 max-pool
+    model = QModule(resnet50())
+    kinds = [type(m).__name__ for m in model.modules()]
+    assert kinds.count("QConv2d") == 53 and kinds.count("QBatchNorm2d") == 53
+    assert kinds.count("QLinear") == 1 and kinds.count("QReLU") == 49 and kinds.count("QMaxPool2d") == 1
+    assert not any(k in ("Conv2d", "BatchNorm2d", "ReLU", "MaxPool2d", "Linear") for k in kinds)
+    assert len(QScheme.layers) == 54 and len(QBNScheme.layers) == 53
+    # kernel positions feed the sensitivity: 7x7 stem, 3x3 and 1x1 convs
+    locs = sorted({s.num_locations for s in QScheme.layers})
+    assert locs == [1, 9, 49]
+    # every BN scheme remembers the conv built just before it
+    assert all(b.prev_linear is not None for b in QBNScheme.layers)
+
+
+def test_l1_leaves_batch_norm_alone():
+    set_optimization_level("L1")
+    model = QModule(nn.Sequential(nn.Conv2d(3, 8, 3), nn.BatchNorm2d(8), nn.ReLU()))
+    kinds = [type(m).__name__ for m in model.model]
+    assert kinds == ["QConv2d", "BatchNorm2d", "QReLU"]
+    assert model.model[0].scheme is None          # no adaptive scheme at L1
+
+
+def test_state_dict_has_no_wrapper_prefix_and_round_trips():
+    plain = nn.Sequential(nn.Conv2d(3, 4, 3), nn.BatchNorm2d(4), nn.ReLU(), nn.Flatten(), nn.Linear(4, 2))
+    keys = list(plain.state_dict().keys())
+    model = QModule(plain)
+    sd = model.state_dict()
+    assert list(sd.keys()) == keys
+    sd = {k: torch.randn_like(v) if v.is_floating_point() else v for k, v in sd.items()}
+    model.load_state_dict(sd)
+    assert torch.equal(model.model[0].weight, sd["0.weight"])
+
+
+def test_train_eval_toggle_config():
+    model = QModule(nn.Sequential(nn.Linear(4, 4)))
+    model.eval()
+    assert not config.training
+    y = model(torch.randn(2, 4))                  # eval path is plain nn.Linear: runs on CPU
+    assert y.shape == (2, 4)
+    model.train()
+    assert config.training
+
+
+def test_compute_tensor_bytes_counts_like_the_reference():
+    ts = [torch.zeros(10), torch.zeros(10, dtype=torch.int32), torch.zeros(10, dtype=torch.bfloat16),
+          torch.zeros(10, dtype=torch.float16), torch.zeros(10, dtype=torch.int8),
+          torch.zeros(10, dtype=torch.float64), None, 4]
+    assert actnn_amd.compute_tensor_bytes(ts) == 40 + 40 + 20 + 20 + 10
+    assert actnn_amd.compute_tensor_bytes(torch.zeros(3, 5)) == 60
+
+
+def test_bindings_reject_host_tensors():
+    import actnn_amd.cpp_extension.minimax as ext_minimax
+    import actnn_amd.cpp_extension.quantization as ext_q
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        ext_minimax.minimax(torch.randn(4, 256))
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        ext_q.act_quantized_relu(torch.randn(4))
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        ext_q.pack_single_precision(torch.randn(2, 2, 256), torch.randn(2, 2, 1), torch.randn(2, 2, 1), 2, True)
+    import actnn_amd.cpp_extension.calc_precision as ext_cp
+    with pytest.raises(RuntimeError):
+        ext_cp.calc_precision(torch.ones(4), torch.ones(4), torch.ones(4, dtype=torch.int32), 8)   # b dtype
+
+
+def test_calc_precision_binding_mutates_and_returns_b():
+    import actnn_amd.cpp_extension.calc_precision as ext_cp
+    b = torch.ones(256, dtype=torch.int32) * 8
+    out = ext_cp.calc_precision(b, torch.zeros(256), torch.ones(256, dtype=torch.int32), 512)
+    assert out is b and int(b.sum()) == 512 and int(b[36]) == 5
+
+
+def test_perlayer_allocation_on_host():
+    # three fake layers with very different sensitivities: bits must follow C, average stays 2
+    class L:
+        weight = nn.Parameter(torch.zeros(1))
+    schemes = [QScheme(L()) for _ in range(3)]
+    N = 16
+    for s, c, d in zip(schemes, (1e-3, 1.0, 1e3), (1000, 1000, 1000)):
+        s.C = torch.full((N,), c)
+        s.dim = d
+    QScheme.allocate_perlayer()
+    bits = [float(s.bits) for s in schemes]
+    assert bits[0] <= bits[1] <= bits[2] and bits[0] < bits[2]
+    assert abs(sum(bits) / 3 - 2.0) < 0.05
+    b1 = QBNScheme()
+    QBNScheme.allocate_perlayer()
+    assert float(b1.bits) == bits[2]              # BN copies the preceding layer's budget
