@@ -1,0 +1,67 @@
+"""Extra benchmark legs used by bench.py: the ResNet-50 training step under QModule at L3
+(BASELINE config 5) with the reference's speed and memory protocols
+(mem_speed_benchmark/train.py:363-397 memory, :422-438 speed)."""
+import time
+
+import torch
+import torch.nn.functional as F
+
+from . import QBNScheme, QModule, QScheme, config, set_optimization_level
+from .resnet import resnet50
+from .utils import compute_tensor_bytes, get_memory_usage
+
+
+def resnet50_step(device, level="L3", batch=512, warmup=3, steps=10, autocast=True):
+    """images/s = batch / median step time over `steps` steps after `warmup`; activation memory =
+    allocated before backward - allocated after the data is loaded - bytes(loss, output)."""
+    config.reset()
+    QScheme.reset()
+    QBNScheme.reset()
+    model = resnet50()
+    if level != "exact":
+        set_optimization_level(level)
+        model = QModule(model)
+    model = model.to(device).train()
+    opt = torch.optim.SGD(model.parameters(), lr=0.1, momentum=0.9, weight_decay=1e-4)
+    g = torch.Generator(device=device).manual_seed(0)
+    images = torch.randn(batch, 3, 224, 224, generator=g, device=device)
+    target = torch.randint(0, 1000, (batch,), generator=g, device=device)
+    times, act_mem, peak = [], None, None
+    for it in range(warmup + steps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        init_mem = get_memory_usage()
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+            output = model(images)
+            loss = F.cross_entropy(output, target)
+        if it == warmup:
+            torch.cuda.synchronize()
+            before_backward = get_memory_usage()
+            act_mem = before_backward - init_mem - compute_tensor_bytes([loss, output])
+        opt.zero_grad(set_to_none=True)
+        loss.backward()
+        opt.step()
+        del loss, output
+        torch.cuda.synchronize()
+        if it >= warmup:
+            times.append(time.perf_counter() - t0)
+    peak = torch.cuda.max_memory_allocated()
+    times.sort()
+    med = times[len(times) // 2]
+    config.reset()
+    QScheme.reset()
+    QBNScheme.reset()
+    return {"images_per_s": round(batch / med, 1), "ms_per_step": round(med * 1e3, 2),
+            "activation_mem_MB": round(act_mem / 2 ** 20, 1), "peak_mem_MB": round(peak / 2 ** 20, 1),
+            "batch": batch, "level": level, "autocast_bf16": autocast, "warmup": warmup, "steps": steps}
+
+
+def run(device):
+    out = {}
+    torch.cuda.reset_peak_memory_stats()
+    out["resnet50_L3"] = resnet50_step(device, "L3")
+    torch.cuda.empty_cache()
+    torch.cuda.reset_peak_memory_stats()
+    out["resnet50_exact"] = resnet50_step(device, "exact")
+    torch.cuda.empty_cache()
+    return out

@@ -23,8 +23,8 @@ from .qscheme import QScheme
 def _autocast_apply(fn, *args):
     """Run fn.apply(*args); inside an autocast region cast float tensors to the autocast dtype
     first and switch autocast off for the call."""
-    if torch.is_autocast_enabled():
-        dt = torch.get_autocast_gpu_dtype()
+    if torch.is_autocast_enabled("cuda"):
+        dt = torch.get_autocast_dtype("cuda")
         args = tuple(a.to(dt) if isinstance(a, torch.Tensor) and a.is_floating_point() and a.is_cuda else a
                      for a in args)
         with torch.autocast(device_type="cuda", enabled=False):

@@ -69,14 +69,31 @@ def no_scheme_compute_quantization_bits(input):
 def quantize_activation(input, scheme):
     """-> (q_input, q_bits, q_scale, q_min); for fp32 activations scale and min are kept as
     bfloat16 (ops.py:99-118)."""
+    return finish_quantize(start_quantize(input, scheme))
+
+
+def start_quantize(input, scheme):
+    """First half of quantize_activation: everything up to the point where the per-sample widths
+    are needed on the host.  The caller may launch other GPU work (the layer's forward) before
+    calling finish_quantize, which hides the device->host round trip of the allocation."""
     if not config.compress_activation:
-        return (swap_to_cpu(input) if config.swap else input), None, None, None
+        return ("raw", input)
     if scheme:
-        groups, q_bits, q_min, mx = scheme.compute_quantization_bits(input)
+        return ("scheme", input.dtype, scheme, scheme.start_quantization_bits(input))
+    return ("fixed", input.dtype, no_scheme_compute_quantization_bits(input))
+
+
+def finish_quantize(started):
+    if started[0] == "raw":
+        input = started[1]
+        return (swap_to_cpu(input) if config.swap else input), None, None, None
+    if started[0] == "scheme":
+        _, dtype, scheme, st = started
+        groups, q_bits, q_min, mx = scheme.finish_quantization_bits(st)
     else:
-        groups, q_bits, q_min, mx = no_scheme_compute_quantization_bits(input)
+        _, dtype, (groups, q_bits, q_min, mx) = started
     q_input, q_scale = quantize_and_pack(groups, q_bits, q_min, mx)
-    if input.dtype == torch.float32:
+    if dtype == torch.float32:
         return q_input, q_bits, q_scale.to(torch.bfloat16), q_min.to(torch.bfloat16)
     return q_input, q_bits, q_scale, q_min
 
@@ -110,8 +127,12 @@ class _Quantized(tuple):
 
 
 def quantize_saved(input, scheme):
-    q = _Quantized(quantize_activation(input, scheme))
-    q.native_bf16 = input.dtype == torch.bfloat16
+    return finish_saved(start_quantize(input, scheme), input.dtype)
+
+
+def finish_saved(started, dtype):
+    q = _Quantized(finish_quantize(started))
+    q.native_bf16 = dtype == torch.bfloat16
     return q
 
 
@@ -124,7 +145,11 @@ total_act_mem = 0
 
 
 def _conv_forward(ctx, forward_op, input, weight, bias, stride, padding, dilation, groups, scheme):
-    quantized = quantize_saved(input, scheme)
+    # min/max and sensitivities first, then the convolution itself, then the allocation and
+    # the pack: the convolution runs while the sensitivities travel to the host
+    started = start_quantize(input, scheme)
+    output = forward_op(input, weight, bias, stride, padding, dilation, groups)
+    quantized = finish_saved(started, input.dtype)
     ctx.scheme = scheme
     ctx.saved = quantized, weight, bias
     ctx.other_args = (input.shape, stride, padding, dilation, groups)
@@ -136,7 +161,7 @@ def _conv_forward(ctx, forward_op, input, weight, bias, stride, padding, dilatio
         conv_layer_ct += 1
         total_act_mem += compute_tensor_bytes(list(quantized))
         print("Act mem: %.2f MB" % (total_act_mem / 1024 ** 2))
-    return forward_op(input, weight, bias, stride, padding, dilation, groups)
+    return output
 
 
 def _conv_backward(ctx, grad_output, bias_reduce_dims, aug):
@@ -210,12 +235,14 @@ class conv3d(Function):
 class linear(Function):
     @staticmethod
     def forward(ctx, input, weight, bias=None, scheme=None):
-        quantized = quantize_saved(input, scheme)
+        started = start_quantize(input, scheme)
+        output = F.linear(input, weight, bias)
+        quantized = finish_saved(started, input.dtype)
         empty_cache(config.empty_cache_threshold)
         ctx.scheme = scheme
         ctx.saved = quantized, weight, bias
         ctx.other_args = input.shape
-        return F.linear(input, weight, bias)
+        return output
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -243,7 +270,15 @@ class batch_norm(Function):
     @staticmethod
     def forward(ctx, input, running_mean, running_var, weight, bias, training,
                 exponential_average_factor, eps, scheme):
-        quantized = quantize_saved(input, scheme)
+        started = start_quantize(input, scheme)
+        if training:
+            output, save_mean, save_var, reserve = ext_backward_func.cudnn_batch_norm(
+                input, weight, bias, running_mean, running_var, training, exponential_average_factor, eps)
+        else:
+            output, save_mean, save_var = ext_backward_func.native_batch_norm(
+                input, weight, bias, running_mean, running_var, training, exponential_average_factor, eps)
+            reserve = None
+        quantized = finish_saved(started, input.dtype)
         empty_cache(config.empty_cache_threshold)
         if config.debug_memory_op_forward:
             global bn_layer_ct, total_act_mem
@@ -252,13 +287,6 @@ class batch_norm(Function):
             bn_layer_ct += 1
             total_act_mem += compute_tensor_bytes(list(quantized))
             print("Act mem: %.2f MB" % (total_act_mem / 1024 ** 2))
-        if training:
-            output, save_mean, save_var, reserve = ext_backward_func.cudnn_batch_norm(
-                input, weight, bias, running_mean, running_var, training, exponential_average_factor, eps)
-        else:
-            output, save_mean, save_var = ext_backward_func.native_batch_norm(
-                input, weight, bias, running_mean, running_var, training, exponential_average_factor, eps)
-            reserve = None
         ctx.scheme = scheme
         ctx.other_args = input.shape
         ctx.saved = (quantized, weight, running_mean, running_var, save_mean, save_var, training, eps, reserve)

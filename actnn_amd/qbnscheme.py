@@ -3,7 +3,7 @@ sensitivity is the range term alone and the per-layer budget follows the precedi
 import torch
 
 from .conf import config
-from .qscheme import QScheme, greedy_bits, group_min_max, range_sqr
+from .qscheme import PendingBits, QScheme, greedy_bits, group_min_max, range_sqr
 
 
 class QBNScheme(QScheme):
@@ -15,12 +15,17 @@ class QBNScheme(QScheme):
         QBNScheme.layers.append(self)
         self.prev_linear = QScheme.layers[-1] if len(QScheme.layers) > 0 else None
 
-    def compute_quantization_bits(self, input):
+    def start_quantization_bits(self, input):
         self.prev_linear = QScheme.prev_layer
         N = input.shape[0]
         groups, mn, mx, num_pixels = group_min_max(input)
-        C = range_sqr(mn, mx, N, num_pixels).to(torch.float32).cpu()       # qbnscheme.py:44-47
-        bits_dev, _ = greedy_bits(C, N, self.initial_bits, self.bits, input.device)
+        pending = PendingBits(range_sqr(mn, mx, N, num_pixels))            # qbnscheme.py:44-47
+        return groups, mn, mx, pending, input.numel() // N
+
+    def finish_quantization_bits(self, started):
+        groups, mn, mx, pending, _ = started
+        N = groups.shape[0]
+        bits_dev, _ = greedy_bits(pending.wait().clone(), N, self.initial_bits, self.bits, groups.device)
         return groups, bits_dev, mn.view(N, -1, 1), mx.view(N, -1, 1)
 
     @staticmethod

@@ -41,6 +41,26 @@ def range_sqr(mn, mx, N, num_pixels):
     return torch.norm((mx - mn).view(N, -1), dim=1).float().square() * (config.group_size / num_pixels)
 
 
+class PendingBits:
+    """Per-sample widths whose sensitivities are still on their way to the host.
+
+    The allocation needs the ranges of every group of a sample on the CPU (greedy heap), which
+    costs one device->host round trip per layer.  `start` queues the copy into pinned memory and
+    records an event; the caller then launches the layer's own forward computation, and `finish`
+    waits for the event only - so the GPU keeps working during the round trip instead of idling
+    as it does with the reference's blocking `.cpu()` (qscheme.py:83-85)."""
+
+    def __init__(self, C_dev):
+        self.host = torch.empty(C_dev.shape, dtype=torch.float32, pin_memory=True)
+        self.host.copy_(C_dev.to(torch.float32), non_blocking=True)
+        self.event = torch.cuda.Event()
+        self.event.record()
+
+    def wait(self):
+        self.event.synchronize()
+        return self.host
+
+
 def greedy_bits(C_host, N, initial_bits, avg_bits, device):
     """Per-sample widths: calc_precision(b = initial_bits, C, w = 1, target = int(avg_bits * N)),
     returned on the device with the host copy attached (qscheme.py:86-94)."""
@@ -89,7 +109,8 @@ class QScheme(object):
         """Squared gradient norm per sample, kept as a running value (qscheme.py:47-55)."""
         if not QScheme.update_scale:
             return
-        sq = grad.reshape(grad.shape[0], -1).float().norm(dim=1).square()
+        # squared L2 norm per sample, accumulated in fp32 without materialising an fp32 copy
+        sq = torch.linalg.vector_norm(grad.reshape(grad.shape[0], -1), dim=1, dtype=torch.float32).square()
         if config.use_gradient:
             assert QScheme.batch is not None
             self.scales[QScheme.batch] = self.scales[QScheme.batch] * 0.5 + sq.cpu() * 0.5
@@ -102,14 +123,26 @@ class QScheme(object):
         return self.num_locations / 4 / self.depthwise_groups * rsq * grad_sum
 
     def compute_quantization_bits(self, input):
+        """-> (groups [N,G,gs], bits on device, mn [N,G,1], mx [N,G,1])  (qscheme.py:57-94)."""
+        return self.finish_quantization_bits(self.start_quantization_bits(input))
+
+    def start_quantization_bits(self, input):
+        """First half: min/max kernel, sensitivities, asynchronous copy to the host."""
         QScheme.prev_layer = self
         N = input.shape[0]
         groups, mn, mx, num_pixels = group_min_max(input)
         rsq = range_sqr(mn, mx, N, num_pixels)
-        C = self.sensitivity(rsq, input.device).to(torch.float32).cpu()     # device -> host sync
-        bits_dev, b = greedy_bits(C, N, self.initial_bits, self.bits, input.device)
+        pending = PendingBits(self.sensitivity(rsq, input.device))
+        return groups, mn, mx, pending, input.numel() // N
+
+    def finish_quantization_bits(self, started):
+        """Second half: wait for the sensitivities, greedy allocation, widths back to the device."""
+        groups, mn, mx, pending, dim = started
+        N = groups.shape[0]
+        C = pending.wait().clone()
+        bits_dev, b = greedy_bits(C, N, self.initial_bits, self.bits, groups.device)
         self.C = C
-        self.dim = input.numel() // N
+        self.dim = dim
         self.b = b
         return groups, bits_dev, mn.view(N, -1, 1), mx.view(N, -1, 1)
 
