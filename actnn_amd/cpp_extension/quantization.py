@@ -169,6 +169,39 @@ def unpack_single_precision(data, bits, scale, min, N, num_groups, group_size):
 
 
 # ------------------------------------------------------------------------------------------
+# fused QLinear weight gradient (no counterpart among the reference's operators: it replaces
+# dequantize + grad_output.t().mm(input) of linear.backward, actnn/actnn/ops.py:407-421)
+# ------------------------------------------------------------------------------------------
+def linear_grad_weight_q2(grad_output, packed, scale, min, in_features, out_dtype=None):
+    """grad_w[O, I] = grad_output[M, O]^T @ dequant(x)[M, I], x given as the pack_single 2-bit
+    stream with scale/min [M, I/256, 1]; the dequantised tile only ever exists in LDS."""
+    g.check_typed(packed, "packed", torch.int8, 1)
+    g.check_float(scale, "scale", 3)
+    g.check_float(min, "min", 3)
+    if not (isinstance(grad_output, torch.Tensor) and grad_output.is_cuda and grad_output.dim() == 2):
+        raise RuntimeError("grad_output must be a 2-d CUDA tensor")
+    if grad_output.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("The type of grad_output is not correct!")
+    grad_output = g.aligned(grad_output.contiguous())
+    M, O = grad_output.shape
+    I = int(in_features)
+    if I % 256 != 0 or M % 4 != 0 or O % 8 != 0:
+        raise RuntimeError("linear_grad_weight_q2 needs M % 4 == 0, in_features % 256 == 0, O % 8 == 0")
+    if scale.numel() != M * (I // 256) or min.numel() != scale.numel() or min.dtype != scale.dtype:
+        raise RuntimeError("linear_grad_weight_q2: scale/min do not match the packed input")
+    if packed.numel() < M * I // 4:
+        raise RuntimeError("linear_grad_weight_q2: packed stream is too short")
+    out_dtype = out_dtype or grad_output.dtype
+    gw = torch.empty(O, I, dtype=out_dtype, device=grad_output.device)
+    with torch.cuda.device(gw.device):
+        check(g.lib().actnn_linear_grad_weight_q2(
+            grad_output.data_ptr(), packed.data_ptr(), scale.data_ptr(), min.data_ptr(), gw.data_ptr(),
+            M, O, I, g.DTYPE_CODE[grad_output.dtype], g.DTYPE_CODE[scale.dtype], g.DTYPE_CODE[out_dtype],
+            g.stream_ptr(gw.device)), "linear_grad_weight_q2")
+    return gw
+
+
+# ------------------------------------------------------------------------------------------
 # ReLU / Dropout with 1-bit masks  (quantization.cc:106-148)
 # ------------------------------------------------------------------------------------------
 def mask_words(n):

@@ -1,6 +1,278 @@
-// placeholder until the fused GEMM lands
+// Fused QLinear weight gradient (replaces dequantize_activation + grad_output.t().mm(input) in
+// linear.backward, actnn/actnn/ops.py:407-421):
+//
+//     grad_w[O, I] = grad_out[M, O]^T @ dequant(x)[M, I]
+//
+// x stays in the 2-bit fixed-width stream (byte ((m/4) * I/256 + g) * 256 + d holds rows
+// 4*(m/4) .. +3 of feature g*256 + d, two bits each) with scale/min[M, I/256].  The full
+// precision input is never written to memory: every k-step the 2-bit tile is unpacked,
+// dequantised (code * (1/scale) + min) and rounded to bf16 straight into the LDS tile that feeds
+// v_mfma_f32_32x32x16_bf16, with fp32 accumulation.
+//
+// Tiling: the reduction runs over the samples m (K of the GEMM).  A 256-thread block owns a
+// 256 (O) x 128 (I) output tile - inside one quantisation group, so a block needs one scale/min
+// per sample - as 4 waves of 64 x 128, each 2 x 4 MFMA tiles of 32 x 32.  Two blocks fit on a
+// CU; they are not synchronised with each other, so one block's unpack/convert work overlaps the
+// other's MFMAs.  Per k-step of 32 samples (LDS tiles are double-buffered, one barrier per step):
+//   * grad_out rows are loaded as they lie in memory (O contiguous, 16-byte vectors), converted
+//     to bf16 if they are fp16, and kept in LDS as [k][o]; the MFMA "A" fragments (8 consecutive
+//     k for one o) are gathered from there with 16-bit LDS reads;
+//   * the packed bytes already hold 4 consecutive k per feature, so a thread unpacks 8 features x
+//     4 samples and writes them k-contiguous: LDS [i][k], "B" fragments are single 16-byte reads.
+// Global loads run two steps ahead of the MFMAs (register prefetch), LDS writes one step ahead.
 #include "device_utils.h"
-extern "C" int actnn_linear_grad_weight_q2(const void*, const int8_t*, const void*, const void*, void*,
-                                           int64_t, int64_t, int64_t, int, int, int, void*) {
-  return ACTNN_EINVAL;
+
+namespace actnn {
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 256;
+constexpr int BM = 256;            // output rows (O) per block
+constexpr int BN = 128;            // output columns (I) per block = half a quantisation group
+constexpr int BK = 32;             // samples per k-step
+constexpr int kPitchA = BM + 8;    // bf16 elements per k-row of the A tile  (528 bytes)
+constexpr int kPitchB = BK + 8;    // bf16 elements per feature row of the B tile (80 bytes)
+constexpr int WM = 64;             // wave tile: 64 (O) x 128 (I) = 2 x 4 MFMA tiles of 32 x 32
+constexpr int NT = BN / 32;        // MFMA tiles per wave along I
+
+template <typename T> ACTNN_DEV float load_as_float(const T* p, int64_t i) { return Conv<T>::load(p, i); }
+
+// two floats -> two bf16 in one word (v_cvt_pk_bf16_f32, round to nearest even)
+ACTNN_DEV uint32_t pack_bf16(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){lo, hi}, bf16x2));
+}
+
+// 8 raw grad_out values (as loaded) -> 8 bf16 (as 4 packed words)
+ACTNN_DEV u32x4 to_bf16x8(u32x4 raw, const __half*) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  u32x4 out;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    out[i] = pack_bf16(half_bits_to_float(w[i] & 0xffffu), half_bits_to_float(w[i] >> 16));
+  return out;
+}
+ACTNN_DEV u32x4 to_bf16x8(u32x4 raw, const bf16_t*) { return raw; }
+
+template <typename T> struct RawScalar;          // a scale/min value exactly as loaded
+template <> struct RawScalar<float> {
+  typedef float type;
+  static ACTNN_DEV float widen(float v) { return v; }
+};
+template <> struct RawScalar<__half> {
+  typedef uint16_t type;
+  static ACTNN_DEV float widen(uint16_t v) { return half_bits_to_float(v); }
+};
+template <> struct RawScalar<bf16_t> {
+  typedef uint16_t type;
+  static ACTNN_DEV float widen(uint16_t v) { return bf16_bits_to_float(v); }
+};
+
+template <typename TG, typename TS, typename TO>
+__global__ __launch_bounds__(kThreads, 2) void linear_gw_q2_kernel(
+    const TG* __restrict__ gout, const uint8_t* __restrict__ packed, const TS* __restrict__ scale,
+    const TS* __restrict__ mn, TO* __restrict__ gw, int M, int O, int I) {
+  __shared__ __attribute__((aligned(16))) uint16_t sA[2][BK * kPitchA];
+  __shared__ __attribute__((aligned(16))) uint16_t sB[2][BN * kPitchB];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wm = (tid >> 6) * WM;            // wave's row offset inside the block tile
+  const int G = I / 256;
+  // blocks that share an O panel are neighbours in launch order
+  const int tiles_n = I / BN;
+  const int tile_m = blockIdx.x / tiles_n;
+  const int tile_n = blockIdx.x % tiles_n;
+  const int o0 = tile_m * BM;
+  const int i0 = tile_n * BN;
+  const int g = i0 / 256;                    // the block's columns lie inside quantisation group g
+  const int d0 = i0 % 256;                   // ... starting at feature d0 of the group
+
+  // A staging: 4 vectors of 8 o's per thread; vector v -> k row v / 32, o offset (v % 32) * 8
+  // B staging: thread -> sample quad br = tid / 32 (4 consecutive k), features (tid % 32) + 32 * e
+  const int br = tid >> 5;
+  const int bi = tid & 31;
+
+  f32x16 acc[2][NT];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < NT; ++b)
+#pragma unroll
+      for (int c = 0; c < 16; ++c) acc[a][b][c] = 0.0f;
+
+  // Registers of the prefetch hold the data exactly as loaded: nothing may consume a load
+  // inside `prefetch`, or the wave would wait out the memory latency there.
+  typedef typename RawScalar<TS>::type raw_t;
+  u32x4 ra[4];
+  uint32_t rb[NT];
+  raw_t rsc[4], rmn[4];
+  bool rvalid = false;
+
+  auto prefetch = [&](int k0) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int v = tid + kThreads * r;
+      const int k = k0 + (v >> 5);
+      const int o = o0 + (v & 31) * 8;
+      ra[r] = (u32x4){0u, 0u, 0u, 0u};
+      if (k < M && o < O) ra[r] = load16(gout + (int64_t)k * O + o);
+    }
+    const int kq = k0 + br * 4;              // first sample of this thread's quad; M % 4 == 0
+    rvalid = kq < M;
+    if (rvalid) {
+#pragma unroll
+      for (int e = 0; e < NT; ++e) rb[e] = packed[((int64_t)(kq >> 2) * G + g) * 256 + d0 + bi + 32 * e];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        rsc[j] = reinterpret_cast<const raw_t*>(scale)[(int64_t)(kq + j) * G + g];
+        rmn[j] = reinterpret_cast<const raw_t*>(mn)[(int64_t)(kq + j) * G + g];
+      }
+    }
+  };
+
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int v = tid + kThreads * r;
+      *reinterpret_cast<u32x4*>(&sA[buf][(v >> 5) * kPitchA + (v & 31) * 8]) =
+          to_bf16x8(ra[r], static_cast<const TG*>(nullptr));
+    }
+    float inv[4], m4[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {            // rows past M dequantise to 0
+      inv[j] = rvalid ? __builtin_amdgcn_rcpf(RawScalar<TS>::widen(rsc[j])) : 0.0f;
+      m4[j] = rvalid ? RawScalar<TS>::widen(rmn[j]) : 0.0f;
+    }
+#pragma unroll
+    for (int e = 0; e < NT; ++e) {
+      const uint32_t by = rvalid ? rb[e] : 0u;
+      const float x0 = fmaf((float)(by & 3u), inv[0], m4[0]);
+      const float x1 = fmaf((float)((by >> 2) & 3u), inv[1], m4[1]);
+      const float x2 = fmaf((float)((by >> 4) & 3u), inv[2], m4[2]);
+      const float x3 = fmaf((float)((by >> 6) & 3u), inv[3], m4[3]);
+      *reinterpret_cast<u32x2*>(&sB[buf][(bi + 32 * e) * kPitchB + br * 4]) =
+          (u32x2){pack_bf16(x0, x1), pack_bf16(x2, x3)};
+    }
+  };
+
+  const int steps = (M + BK - 1) / BK;
+  prefetch(0);
+  if (steps > 0) stage(0);
+  __syncthreads();
+  if (steps > 1) prefetch(BK);
+
+  for (int t = 0; t < steps; ++t) {
+    const int cur = t & 1;
+    // write the tile of step t+1 into the other buffer (its last readers passed the barrier at
+    // the end of step t-1), then get the loads of step t+2 in flight, then multiply step t
+    if (t + 1 < steps) stage(cur ^ 1);
+    if (t + 2 < steps) prefetch((t + 2) * BK);
+
+    // all fragments of the step first (LDS reads return in order, so the MFMAs below can start
+    // as soon as their operands are in), then the 2 x 2 x NT MFMAs
+    bf16x8 fa[BK / 16][2], fb[BK / 16][NT];
+#pragma unroll
+    for (int kb = 0; kb < BK / 16; ++kb) {
+      const int kf = kb * 16 + (lane >> 5) * 8;      // this lane's first k in the step
+#pragma unroll
+      for (int b = 0; b < NT; ++b) {
+        const int n = b * 32 + (lane & 31);
+        const u32x4 bw = *reinterpret_cast<const u32x4*>(&sB[cur][n * kPitchB + kf]);
+        fb[kb][b] = __builtin_bit_cast(bf16x8, bw);
+      }
+#pragma unroll
+      for (int a = 0; a < 2; ++a) {
+        const int o = wm + a * 32 + (lane & 31);
+        uint32_t w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t lo = sA[cur][(kf + 2 * j) * kPitchA + o];
+          const uint32_t hi = sA[cur][(kf + 2 * j + 1) * kPitchA + o];
+          w[j] = lo | (hi << 16);
+        }
+        fa[kb][a] = __builtin_bit_cast(bf16x8, (u32x4){w[0], w[1], w[2], w[3]});
+      }
+    }
+#pragma unroll
+    for (int kb = 0; kb < BK / 16; ++kb)
+#pragma unroll
+      for (int b = 0; b < NT; ++b)
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kb][a], fb[kb][b], acc[a][b], 0, 0, 0);
+    __syncthreads();
+  }
+
+  // 32x32 accumulator layout: register c of a lane is row 8*(c/4) + 4*(lane/32) + c%4, column lane%32
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+#pragma unroll
+    for (int b = 0; b < NT; ++b) {
+      const int col = i0 + b * 32 + (lane & 31);
+#pragma unroll
+      for (int c = 0; c < 16; ++c) {
+        const int row = o0 + wm + a * 32 + 8 * (c >> 2) + 4 * (lane >> 5) + (c & 3);
+        if (row < O) Conv<TO>::store(gw, (int64_t)row * I + col, acc[a][b][c]);
+      }
+    }
+  }
+}
+
+template <typename TG, typename TS, typename TO>
+int launch(const void* gout, const int8_t* packed, const void* scale, const void* mn, void* gw,
+           int64_t M, int64_t O, int64_t I, hipStream_t s) {
+  const int64_t blocks = ((O + BM - 1) / BM) * (I / BN);
+  if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
+  linear_gw_q2_kernel<TG, TS, TO><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+      static_cast<const TG*>(gout), reinterpret_cast<const uint8_t*>(packed),
+      static_cast<const TS*>(scale), static_cast<const TS*>(mn), static_cast<TO*>(gw), (int)M, (int)O,
+      (int)I);
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
+
+template <typename TG, typename TS>
+int launch_out(int out_dtype, const void* gout, const int8_t* packed, const void* scale,
+               const void* mn, void* gw, int64_t M, int64_t O, int64_t I, hipStream_t s) {
+  switch (out_dtype) {
+    case ACTNN_F32: return launch<TG, TS, float>(gout, packed, scale, mn, gw, M, O, I, s);
+    case ACTNN_F16: return launch<TG, TS, __half>(gout, packed, scale, mn, gw, M, O, I, s);
+    case ACTNN_BF16: return launch<TG, TS, bf16_t>(gout, packed, scale, mn, gw, M, O, I, s);
+    default: return ACTNN_EDTYPE;
+  }
+}
+
+template <typename TG>
+int launch_sm(int sm_dtype, int out_dtype, const void* gout, const int8_t* packed, const void* scale,
+              const void* mn, void* gw, int64_t M, int64_t O, int64_t I, hipStream_t s) {
+  switch (sm_dtype) {
+    case ACTNN_F32: return launch_out<TG, float>(out_dtype, gout, packed, scale, mn, gw, M, O, I, s);
+    case ACTNN_F16: return launch_out<TG, __half>(out_dtype, gout, packed, scale, mn, gw, M, O, I, s);
+    case ACTNN_BF16: return launch_out<TG, bf16_t>(out_dtype, gout, packed, scale, mn, gw, M, O, I, s);
+    default: return ACTNN_EDTYPE;
+  }
+}
+
+}  // namespace
+}  // namespace actnn
+
+extern "C" int actnn_linear_grad_weight_q2(const void* grad_out, const int8_t* packed,
+                                           const void* scale, const void* mn, void* grad_w,
+                                           int64_t M, int64_t O, int64_t I, int go_dtype,
+                                           int sm_dtype, int out_dtype, void* stream) {
+  using namespace actnn;
+  if (M < 0 || O < 0 || I < 0 || M % 4 != 0 || I % 256 != 0 || O % 8 != 0) return ACTNN_EINVAL;
+  if (M > 0x7fffffffLL || O > 0x7fffffffLL || I > 0x7fffffffLL) return ACTNN_EINVAL;
+  if (O == 0 || I == 0) return ACTNN_OK;
+  if (!grad_w || (M > 0 && (!grad_out || !packed || !scale || !mn))) return ACTNN_EINVAL;
+  if (M > 0 && !aligned16(grad_out)) return ACTNN_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (go_dtype) {
+    case ACTNN_F16: return launch_sm<__half>(sm_dtype, out_dtype, grad_out, packed, scale, mn, grad_w, M, O, I, s);
+    case ACTNN_BF16: return launch_sm<bf16_t>(sm_dtype, out_dtype, grad_out, packed, scale, mn, grad_w, M, O, I, s);
+    default: return ACTNN_EDTYPE;
+  }
 }

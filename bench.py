@@ -158,6 +158,20 @@ def other_configs(device, reps):
     out["pack_single_2bit_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
     t = _event_time_ms(lambda: ext_q.unpack_single_precision(packed, 2, scale, mn, M, I // 256, 256), reps)
     out["unpack_single_2bit_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
+    # config 4: fused dequant + grad_weight GEMM (MFMA roofline), and the unfused path beside it
+    O = 4096
+    go = torch.randn(M, O, device=device, dtype=torch.float16)
+    flops = 2.0 * M * O * I
+    t = _event_time_ms(lambda: ext_q.linear_grad_weight_q2(go, packed, scale, mn, I), reps)
+    out["linear_grad_weight_q2_fused"] = {"ms": t, "TFLOP/s": flops / t / 1e9,
+                                          "frac_mfma_bf16": flops / t / 1e9 / MFMA_BF16_PEAK_TFLOPS}
+
+    def unfused():
+        x = ext_q.unpack_single_precision(packed, 2, scale, mn, M, I // 256, 256).view(M, I)
+        return go.t().mm(x)
+    t = _event_time_ms(unfused, reps)
+    out["linear_grad_weight_unfused_unpack_plus_mm"] = {"ms": t, "TFLOP/s": flops / t / 1e9,
+                                                        "frac_mfma_bf16": flops / t / 1e9 / MFMA_BF16_PEAK_TFLOPS}
     return {k_: {kk: round(vv, 4) for kk, vv in v.items()} for k_, v in out.items()}
 
 
