@@ -1,10 +1,15 @@
 // MaxPool2d with int8 arg-max-in-window indices (replaces quantization_cuda_kernel.cu:630-754).
 //
-// Forward: one thread per output element scans its clipped window in row-major order and
-// keeps the first strict maximum (index relative to the unclipped window origin).
-// Backward: a gather - one thread per input element sums, in a fixed order, the
-// grad_output of the windows whose stored index points at it.  Unlike the reference's
-// atomicAdd scatter this needs no zero-fill pass and is bit-reproducible.
+// Forward: every output element scans its clipped window in row-major order and keeps the first
+// strict maximum (index relative to the unclipped window origin).
+// Backward: a gather - every input element sums, in a fixed order, the grad_output of the
+// windows whose stored index points at it.  Unlike the reference's atomicAdd scatter this needs no
+// zero-fill pass and is bit-reproducible.
+//
+// Both run tiled through LDS: a block owns a band of rows of one (n, c) plane, copies the rows it
+// needs (a contiguous span of the plane) into LDS with 16-byte loads, and then works out of LDS,
+// so HBM sees each input byte once and all global accesses are coalesced.  Planes too wide for
+// the LDS budget fall back to direct global loads.
 #include "device_utils.h"
 
 namespace actnn {
@@ -78,8 +83,190 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_backward_kernel(const T* 
   Conv<T>::store(gin, id, acc);
 }
 
+
+constexpr int kLdsBudget = 48 * 1024;     // bytes of dynamic LDS a block may use
+
+// Copy the contiguous span [first, first + count) of `src` (element indices into a tensor of
+// `total` elements whose base is 16-byte aligned) into LDS so that element first + i lands at
+// dst[shift + i], shift = first % (16 / sizeof(T)); aligned 16-byte loads wherever they stay
+// inside the tensor.  Returns shift.
+template <typename T>
+ACTNN_DEV int stage_span(const T* __restrict__ src, int64_t first, int count, int64_t total, T* dst) {
+  constexpr int V = 16 / (int)sizeof(T);
+  const int shift = (int)(first % V);
+  const int64_t base = first - shift;                    // aligned element index
+  const int nvec = (shift + count + V - 1) / V;
+  for (int v = threadIdx.x; v < nvec; v += kThreads) {
+    const int64_t e = base + (int64_t)v * V;
+    if (e + V <= total) {
+      *reinterpret_cast<u32x4*>(dst + v * V) = load16(src + e);
+    } else {
+      for (int i = 0; i < V; ++i)
+        if (e + i < total) dst[v * V + i] = src[e + i];
+    }
+  }
+  return shift;
+}
+
+template <typename T> ACTNN_DEV float lds_value(const T* p, int i);
+template <> ACTNN_DEV float lds_value<float>(const float* p, int i) { return p[i]; }
+template <> ACTNN_DEV float lds_value<__half>(const __half* p, int i) { return __half2float(p[i]); }
+template <> ACTNN_DEV float lds_value<bf16_t>(const bf16_t* p, int i) { return bf16_bits_to_float(p[i].bits); }
+
+// Geometry presets: with PRESET != 0 the window parameters are compile-time constants (loops
+// unroll, divisions become shifts); PRESET 0 reads them from the argument.
+//   1: 3x3 stride 2 pad 1 (ResNet stem)   2: 2x2 stride 2 pad 0   3: 3x3 stride 1 pad 1
+template <int PRESET> struct Win {
+  int KH, KW, SH, SW, PH, PW;
+  __device__ __forceinline__ explicit Win(const PoolGeom& g)
+      : KH(PRESET == 1 || PRESET == 3 ? 3 : PRESET == 2 ? 2 : g.KH),
+        KW(PRESET == 1 || PRESET == 3 ? 3 : PRESET == 2 ? 2 : g.KW),
+        SH(PRESET == 1 || PRESET == 2 ? 2 : PRESET == 3 ? 1 : g.SH),
+        SW(PRESET == 1 || PRESET == 2 ? 2 : PRESET == 3 ? 1 : g.SW),
+        PH(PRESET == 1 || PRESET == 3 ? 1 : PRESET == 2 ? 0 : g.PH),
+        PW(PRESET == 1 || PRESET == 3 ? 1 : PRESET == 2 ? 0 : g.PW) {}
+};
+
+inline int preset_of(const PoolGeom& g) {
+  if (g.KH == 3 && g.KW == 3 && g.SH == 2 && g.SW == 2 && g.PH == 1 && g.PW == 1) return 1;
+  if (g.KH == 2 && g.KW == 2 && g.SH == 2 && g.SW == 2 && g.PH == 0 && g.PW == 0) return 2;
+  if (g.KH == 3 && g.KW == 3 && g.SH == 1 && g.SW == 1 && g.PH == 1 && g.PW == 1) return 3;
+  return 0;
+}
+
+template <typename T, int PRESET>
+__global__ __launch_bounds__(kThreads) void max_pool2d_forward_lds_kernel(
+    const T* __restrict__ x, T* __restrict__ y, int8_t* __restrict__ idx, int64_t total_in,
+    PoolGeom g, int rows_per_band, int bands) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  T* s_in = reinterpret_cast<T*>(smem);
+  const Win<PRESET> k(g);
+  const int64_t nc = blockIdx.x / bands;
+  const int ho0 = (int)(blockIdx.x % bands) * rows_per_band;
+  const int rows_out = g.Ho - ho0 < rows_per_band ? g.Ho - ho0 : rows_per_band;
+  int h_lo = ho0 * k.SH - k.PH;
+  h_lo = h_lo > 0 ? h_lo : 0;
+  int h_hi = (ho0 + rows_out - 1) * k.SH - k.PH + k.KH;
+  h_hi = h_hi < g.H ? h_hi : g.H;
+  const int shift = stage_span(x, nc * (int64_t)g.H * g.W + (int64_t)h_lo * g.W, (h_hi - h_lo) * g.W,
+                               total_in, s_in);
+  __syncthreads();
+  const float init = Conv<T>::round(-1e10f);         // as the reference, .cu:656
+  const int lane = threadIdx.x & 63;
+  for (int r = threadIdx.x >> 6; r < rows_out; r += kThreads / 64) {     // one output row per wave
+    const int ho = ho0 + r;
+    const int h_base = ho * k.SH - k.PH;
+    const int64_t orow = (nc * g.Ho + ho) * (int64_t)g.Wo;
+    for (int wo = lane; wo < g.Wo; wo += 64) {
+      const int w_base = wo * k.SW - k.PW;
+      float v = init;
+      int index = 0;
+#pragma unroll
+      for (int a = 0; a < (PRESET ? k.KH : 15); ++a) {
+        if (!PRESET && a >= k.KH) break;
+        const int i = h_base + a;
+        if (i < 0 || i >= g.H) continue;
+        const T* row = s_in + shift + (i - h_lo) * g.W;
+#pragma unroll
+        for (int b = 0; b < (PRESET ? k.KW : 15); ++b) {
+          if (!PRESET && b >= k.KW) break;
+          const int j = w_base + b;
+          if (j < 0 || j >= g.W) continue;
+          const float c = lds_value<T>(row, j);
+          if (c > v) {
+            v = c;
+            index = a * k.KW + b;
+          }
+        }
+      }
+      Conv<T>::store(y, orow + wo, v);
+      idx[orow + wo] = (int8_t)index;
+    }
+  }
+}
+
+template <typename T, int PRESET>
+__global__ __launch_bounds__(kThreads) void max_pool2d_backward_lds_kernel(
+    const T* __restrict__ gout, const int8_t* __restrict__ idx, T* __restrict__ gin,
+    int64_t total_out, PoolGeom g, int rows_per_band, int bands, int max_out_rows) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  // [grad_output rows | index rows], each with room for the alignment shift
+  T* s_g = reinterpret_cast<T*>(smem);
+  int8_t* s_i = reinterpret_cast<int8_t*>(smem + (((size_t)max_out_rows * g.Wo + 16) * sizeof(T) + 15) / 16 * 16);
+  const Win<PRESET> k(g);
+  const int64_t nc = blockIdx.x / bands;
+  const int h0 = (int)(blockIdx.x % bands) * rows_per_band;
+  const int rows_in = g.H - h0 < rows_per_band ? g.H - h0 : rows_per_band;
+  // output rows whose window touches input rows [h0, h0 + rows_in)
+  int ho_lo = h0 + k.PH - k.KH + 1;
+  ho_lo = ho_lo > 0 ? (ho_lo + k.SH - 1) / k.SH : 0;
+  int ho_hi = (h0 + rows_in - 1 + k.PH) / k.SH;
+  ho_hi = ho_hi < g.Ho - 1 ? ho_hi : g.Ho - 1;
+  int shift_g = 0, shift_i = 0;
+  if (ho_hi >= ho_lo) {
+    const int64_t first = (nc * g.Ho + ho_lo) * (int64_t)g.Wo;
+    const int count = (ho_hi - ho_lo + 1) * g.Wo;
+    shift_g = stage_span(gout, first, count, total_out, s_g);
+    shift_i = stage_span(idx, first, count, total_out, s_i);
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63;
+  for (int r = threadIdx.x >> 6; r < rows_in; r += kThreads / 64) {       // one input row per wave
+    const int h = h0 + r;
+    int a_lo = h + k.PH - k.KH + 1;
+    a_lo = a_lo > 0 ? (a_lo + k.SH - 1) / k.SH : 0;
+    int a_hi = (h + k.PH) / k.SH;
+    a_hi = a_hi < g.Ho - 1 ? a_hi : g.Ho - 1;
+    const int64_t irow = (nc * g.H + h) * (int64_t)g.W;
+    for (int w = lane; w < g.W; w += 64) {
+      int b_lo = w + k.PW - k.KW + 1;
+      b_lo = b_lo > 0 ? (b_lo + k.SW - 1) / k.SW : 0;
+      int b_hi = (w + k.PW) / k.SW;
+      b_hi = b_hi < g.Wo - 1 ? b_hi : g.Wo - 1;
+      float acc = 0.0f;
+      for (int ho = a_lo; ho <= a_hi; ++ho) {
+        const int kh = h - (ho * k.SH - k.PH);
+        const int rr = (ho - ho_lo) * g.Wo;
+        for (int wo = b_lo; wo <= b_hi; ++wo) {
+          const int kw = w - (wo * k.SW - k.PW);
+          if ((int)s_i[shift_i + rr + wo] == kh * k.KW + kw) acc += lds_value<T>(s_g, shift_g + rr + wo);
+        }
+      }
+      Conv<T>::store(gin, irow + w, acc);
+    }
+  }
+}
+
+// rows per band so that a block has about `want` elements of work and the LDS need (computed by
+// `bytes(rows)`) fits the budget; 0 if even one row does not fit.
+template <typename F> int pick_rows(int rows_total, int row_elems, int want, F bytes) {
+  int rows = (want + row_elems - 1) / row_elems;
+  rows = rows < 1 ? 1 : (rows > rows_total ? rows_total : rows);
+  while (rows > 1 && bytes(rows) > (size_t)kLdsBudget) --rows;
+  return bytes(rows) <= (size_t)kLdsBudget ? rows : 0;
+}
+
 template <typename T>
 int launch_fwd(const void* x, void* y, int8_t* idx, int64_t total, const PoolGeom& g, hipStream_t s) {
+  const int64_t planes = total / ((int64_t)g.Ho * g.Wo);
+  auto need = [&](int rows) { return ((size_t)((rows - 1) * g.SH + g.KH) * g.W + 16) * sizeof(T); };
+  const int rb = pick_rows(g.Ho, g.Wo, 1024, need);
+  if (rb > 0 && aligned16(x)) {
+    const int bands = (g.Ho + rb - 1) / rb;
+    if (planes * bands <= 0x7fffffffLL) {
+      const dim3 grid((unsigned)(planes * bands)), blk(kThreads);
+      const T* xi = static_cast<const T*>(x);
+      T* yo = static_cast<T*>(y);
+      const int64_t tin = planes * g.H * g.W;
+      switch (preset_of(g)) {
+        case 1: max_pool2d_forward_lds_kernel<T, 1><<<grid, blk, need(rb), s>>>(xi, yo, idx, tin, g, rb, bands); break;
+        case 2: max_pool2d_forward_lds_kernel<T, 2><<<grid, blk, need(rb), s>>>(xi, yo, idx, tin, g, rb, bands); break;
+        case 3: max_pool2d_forward_lds_kernel<T, 3><<<grid, blk, need(rb), s>>>(xi, yo, idx, tin, g, rb, bands); break;
+        default: max_pool2d_forward_lds_kernel<T, 0><<<grid, blk, need(rb), s>>>(xi, yo, idx, tin, g, rb, bands); break;
+      }
+      ACTNN_RETURN_LAUNCH_STATUS();
+    }
+  }
   const int64_t blocks = (total + kThreads - 1) / kThreads;
   if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
   max_pool2d_forward_kernel<T><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
@@ -90,6 +277,31 @@ int launch_fwd(const void* x, void* y, int8_t* idx, int64_t total, const PoolGeo
 template <typename T>
 int launch_bwd(const void* gout, const int8_t* idx, void* gin, int64_t total, const PoolGeom& g,
                hipStream_t s) {
+  const int64_t planes = total / ((int64_t)g.H * g.W);
+  // output rows a band of `rows` input rows can touch
+  auto out_rows = [&](int rows) { return (rows + g.KH - 2) / g.SH + 2; };
+  auto need = [&](int rows) {
+    const size_t elems = (size_t)out_rows(rows) * g.Wo + 16;
+    return (elems * sizeof(T) + 15) / 16 * 16 + elems + 16;
+  };
+  const int rb = pick_rows(g.H, g.W, 2048, need);
+  if (rb > 0 && aligned16(gout) && aligned16(idx)) {
+    const int bands = (g.H + rb - 1) / rb;
+    if (planes * bands <= 0x7fffffffLL) {
+      const dim3 grid((unsigned)(planes * bands)), blk(kThreads);
+      const T* go = static_cast<const T*>(gout);
+      T* gi = static_cast<T*>(gin);
+      const int64_t tout = planes * g.Ho * g.Wo;
+      const int orows = out_rows(rb);
+      switch (preset_of(g)) {
+        case 1: max_pool2d_backward_lds_kernel<T, 1><<<grid, blk, need(rb), s>>>(go, idx, gi, tout, g, rb, bands, orows); break;
+        case 2: max_pool2d_backward_lds_kernel<T, 2><<<grid, blk, need(rb), s>>>(go, idx, gi, tout, g, rb, bands, orows); break;
+        case 3: max_pool2d_backward_lds_kernel<T, 3><<<grid, blk, need(rb), s>>>(go, idx, gi, tout, g, rb, bands, orows); break;
+        default: max_pool2d_backward_lds_kernel<T, 0><<<grid, blk, need(rb), s>>>(go, idx, gi, tout, g, rb, bands, orows); break;
+      }
+      ACTNN_RETURN_LAUNCH_STATUS();
+    }
+  }
   const int64_t blocks = (total + kThreads - 1) / kThreads;
   if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
   max_pool2d_backward_kernel<T><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
