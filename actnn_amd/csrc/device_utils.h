@@ -20,13 +20,14 @@ struct bf16_t { uint16_t bits; };   // raw bfloat16 storage
 // element expression (v.y, v[i]) reads element 0 with this compiler.
 ACTNN_DEV float as_float(uint32_t u) { return __builtin_bit_cast(float, u); }
 ACTNN_DEV uint32_t as_uint(float f) { return __builtin_bit_cast(uint32_t, f); }
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
 ACTNN_DEV float bf16_bits_to_float(uint32_t b) { return __builtin_bit_cast(float, b << 16); }
-ACTNN_DEV uint32_t float_to_bf16_bits(float f) {           // round to nearest even
-  uint32_t u = __builtin_bit_cast(uint32_t, f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;   // quiet NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return u >> 16;
+// two floats -> two bf16 in one word, round to nearest even (one v_cvt_pk_bf16_f32 on gfx950)
+ACTNN_DEV uint32_t pack_bf16x2(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2_t){lo, hi}, bf16x2_t));
 }
+ACTNN_DEV uint32_t float_to_bf16_bits(float f) { return pack_bf16x2(f, 0.0f) & 0xffffu; }
 ACTNN_DEV float half_bits_to_float(uint32_t b) {
   return __half2float(__builtin_bit_cast(__half, (uint16_t)b));
 }
@@ -134,7 +135,7 @@ ACTNN_DEV void store8(__half* p, const float (&v)[8]) {
 ACTNN_DEV void store8(bf16_t* p, const float (&v)[8]) {
   uint32_t w[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) w[i] = float_to_bf16_bits(v[2 * i]) | (float_to_bf16_bits(v[2 * i + 1]) << 16);
+  for (int i = 0; i < 4; ++i) w[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
   store16(p, (u32x4){w[0], w[1], w[2], w[3]});
 }
 

@@ -26,8 +26,6 @@ namespace actnn {
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kThreads = 256;
@@ -41,10 +39,7 @@ constexpr int NT = BN / 32;        // MFMA tiles per wave along I
 
 template <typename T> ACTNN_DEV float load_as_float(const T* p, int64_t i) { return Conv<T>::load(p, i); }
 
-// two floats -> two bf16 in one word (v_cvt_pk_bf16_f32, round to nearest even)
-ACTNN_DEV uint32_t pack_bf16(float lo, float hi) {
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){lo, hi}, bf16x2));
-}
+ACTNN_DEV uint32_t pack_bf16(float lo, float hi) { return pack_bf16x2(lo, hi); }
 
 // 8 raw grad_out values (as loaded) -> 8 bf16 (as 4 packed words)
 ACTNN_DEV u32x4 to_bf16x8(u32x4 raw, const __half*) {

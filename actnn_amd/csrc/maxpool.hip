@@ -161,15 +161,11 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_forward_lds_kernel(
       const int w_base = wo * k.SW - k.PW;
       float v = init;
       int index = 0;
-#pragma unroll
-      for (int a = 0; a < (PRESET ? k.KH : 15); ++a) {
-        if (!PRESET && a >= k.KH) break;
+      for (int a = 0; a < k.KH; ++a) {
         const int i = h_base + a;
         if (i < 0 || i >= g.H) continue;
         const T* row = s_in + shift + (i - h_lo) * g.W;
-#pragma unroll
-        for (int b = 0; b < (PRESET ? k.KW : 15); ++b) {
-          if (!PRESET && b >= k.KW) break;
+        for (int b = 0; b < k.KW; ++b) {
           const int j = w_base + b;
           if (j < 0 || j >= g.W) continue;
           const float c = lds_value<T>(row, j);

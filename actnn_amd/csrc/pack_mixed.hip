@@ -22,12 +22,25 @@
 namespace actnn {
 namespace {
 
+// Groups per half-wave and block (1, 2 or 4).  fp32: 2 measured best (16 KiB of input per block).
+// 16-bit types: a block with 8 KiB of data is dominated by its own latency chain (widths ->
+// scales -> data), so they take 4 (and 8 for unpack, whose chain is longest).
 #ifndef ACTNN_PACK_GPH
-#define ACTNN_PACK_GPH 2      // groups per half-wave and block (1, 2 or 4)
+#define ACTNN_PACK_GPH 2
 #endif
 #ifndef ACTNN_UNPACK_GPH
 #define ACTNN_UNPACK_GPH 2
 #endif
+#ifndef ACTNN_PACK_GPH16
+#define ACTNN_PACK_GPH16 4
+#endif
+#ifndef ACTNN_UNPACK_GPH16
+#define ACTNN_UNPACK_GPH16 4
+#endif
+template <typename T> struct Gph {
+  static constexpr int kPack = sizeof(T) == 2 ? ACTNN_PACK_GPH16 : ACTNN_PACK_GPH;
+  static constexpr int kUnpack = sizeof(T) == 2 ? ACTNN_UNPACK_GPH16 : ACTNN_UNPACK_GPH;
+};
 
 constexpr int kThreads = 256;
 constexpr int kHalfWaves = kThreads / 32;
@@ -152,11 +165,11 @@ ACTNN_DEV void load_groups(const T* __restrict__ data, const T* __restrict__ noi
 }
 
 template <typename T, int BITS, bool DET>
-ACTNN_DEV void pack_groups(const float (&v)[ACTNN_PACK_GPH][8], const float (&nz)[DET ? ACTNN_PACK_GPH : 1][8],
+ACTNN_DEV void pack_groups(const float (&v)[Gph<T>::kPack][8], const float (&nz)[DET ? Gph<T>::kPack : 1][8],
                            int32_t* __restrict__ packed, int64_t elem_base, int64_t word_base,
                            int groups_valid, const float* s_mul, const float* s_sub,
                            uint64_t seed, uint64_t offset, u32x4* s_out) {
-  constexpr int kGroupsPerHalf = ACTNN_PACK_GPH;
+  constexpr int kGroupsPerHalf = Gph<T>::kPack;
   using TL = Tile<BITS, kGroupsPerHalf>;
   constexpr int R = TL::kGroupsPerReg;
   constexpr int WPG = TL::kWordsPerGroup;
@@ -213,7 +226,7 @@ __global__ __launch_bounds__(kThreads) void pack_mixed_kernel(
     const int32_t* __restrict__ bits, const int32_t* __restrict__ prefix, T* __restrict__ scale,
     int32_t* __restrict__ packed, const T* __restrict__ noise, uint64_t seed, uint64_t offset,
     int64_t G, int blocks_per_sample) {
-  constexpr int GPH = ACTNN_PACK_GPH;
+  constexpr int GPH = Gph<T>::kPack;
   constexpr int kGroupsPerBlock = kHalfWaves * GPH;
   __shared__ float s_mul[kGroupsPerBlock];
   __shared__ float s_sub[kGroupsPerBlock];
@@ -263,8 +276,8 @@ __global__ __launch_bounds__(kThreads) void pack_mixed_kernel(
 template <typename T, int BITS>
 ACTNN_DEV void unpack_groups(const int32_t* __restrict__ packed, T* __restrict__ out,
                              int64_t elem_base, int64_t word_base, int groups_valid,
-                             const float* s_scale, const float* s_min, u32x4* slab) {
-  constexpr int kGroupsPerHalf = ACTNN_UNPACK_GPH;
+                             float* s_scale, float* s_min, float my_scale, float my_min, u32x4* slab) {
+  constexpr int kGroupsPerHalf = Gph<T>::kUnpack;
   constexpr bool kStage = ACTNN_UNPACK_LDS_STAGE && IsF32<T>::value;
   float vs[kStage ? kGroupsPerHalf : 1][8];
   using TL = Tile<BITS, kGroupsPerHalf>;
@@ -291,6 +304,13 @@ ACTNN_DEV void unpack_groups(const int32_t* __restrict__ packed, T* __restrict__
         wlo[t] = (uint32_t)packed[tile_words + lane];
     }
   }
+  // the block's scales and minima go to LDS only now, after the word loads have been issued, so
+  // that the two global round trips overlap
+  if ((int)threadIdx.x < groups_valid) {
+    s_scale[threadIdx.x] = my_scale;
+    s_min[threadIdx.x] = my_min;
+  }
+  __syncthreads();
 #pragma unroll
   for (int t = 0; t < kGroupsPerHalf / R; ++t) {
     const int q0 = t * R;
@@ -300,15 +320,10 @@ ACTNN_DEV void unpack_groups(const int32_t* __restrict__ packed, T* __restrict__
     for (int r = 0; r < R; ++r) {
       const int gl = TL::group_of(hw, q0 + r);
       if (gl < groups_valid) {
-        const float sc = s_scale[gl];
-        const float m = s_min[gl];
+        const Dequant<T> dq(s_scale[gl], s_min[gl]);
         float v[8];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
-          const uint32_t c = (uint32_t)(acc >> (r * WPG + k * BITS)) & kMask;
-          // (scalar_t)val / scale + min, one rounding per operation (.cu:171)
-          v[k] = Conv<T>::round(Conv<T>::round((float)c / sc) + m);
-        }
+        for (int k = 0; k < 8; ++k) v[k] = dq((uint32_t)(acc >> (r * WPG + k * BITS)) & kMask);
         if constexpr (kStage) {
 #pragma unroll
           for (int k = 0; k < 8; ++k) vs[kStage ? q0 + r : 0][k] = v[k];
@@ -327,28 +342,29 @@ __global__ __launch_bounds__(kThreads) void unpack_mixed_kernel(
     const int32_t* __restrict__ packed, const int32_t* __restrict__ bits,
     const int32_t* __restrict__ prefix, const T* __restrict__ scale, const T* __restrict__ mn,
     T* __restrict__ out, int64_t G, int blocks_per_sample) {
-  constexpr int kGroupsPerBlock = kHalfWaves * ACTNN_UNPACK_GPH;
+  constexpr int kGroupsPerBlock = kHalfWaves * Gph<T>::kUnpack;
   __shared__ float s_scale[kGroupsPerBlock];
   __shared__ float s_min[kGroupsPerBlock];
   constexpr bool kStage = ACTNN_UNPACK_LDS_STAGE && IsF32<T>::value;
   __shared__ u32x4 s_slab[kStage ? kGroupsPerBlock * 64 : 1];
-  u32x4* slab = s_slab + (kStage ? (threadIdx.x >> 6) * (2 * ACTNN_UNPACK_GPH * 64) : 0);
+  u32x4* slab = s_slab + (kStage ? (threadIdx.x >> 6) * (2 * Gph<T>::kUnpack * 64) : 0);
   const int64_t n = blockIdx.x / blocks_per_sample;
   const int64_t gb = (int64_t)(blockIdx.x % blocks_per_sample) * kGroupsPerBlock;
   const int b = bits[n];
   const int groups_valid = (int)((G - gb) < kGroupsPerBlock ? (G - gb) : kGroupsPerBlock);
+  float my_scale = 0.0f, my_min = 0.0f;
   if ((int)threadIdx.x < groups_valid) {
     const int64_t gi = n * G + gb + threadIdx.x;
-    s_scale[threadIdx.x] = Conv<T>::load(scale, gi);
-    s_min[threadIdx.x] = Conv<T>::load(mn, gi);
+    my_scale = Conv<T>::load(scale, gi);
+    my_min = Conv<T>::load(mn, gi);
   }
-  __syncthreads();
   const int64_t elem_base = (n * G + gb) * kGs;
   const int64_t word_base = (int64_t)prefix[n] * G * 8 + gb * 8 * b;
   switch (b) {
 #define ACTNN_CASE(B_)                                                                          \
   case B_:                                                                                      \
-    unpack_groups<T, B_>(packed, out, elem_base, word_base, groups_valid, s_scale, s_min, slab); \
+    unpack_groups<T, B_>(packed, out, elem_base, word_base, groups_valid, s_scale, s_min,       \
+                         my_scale, my_min, slab);                                               \
     break;
     ACTNN_CASE(1) ACTNN_CASE(2) ACTNN_CASE(3) ACTNN_CASE(4)
     ACTNN_CASE(5) ACTNN_CASE(6) ACTNN_CASE(7) ACTNN_CASE(8)
@@ -426,13 +442,12 @@ __global__ __launch_bounds__(kThreads) void unpack_mixed_generic_kernel(
   for (int w = threadIdx.x; w < L; w += kThreads) s_word[w] = (uint32_t)packed[word_base + w];
   __syncthreads();
   const int64_t gi = n * G + g;
-  const float sc = Conv<T>::load(scale, gi);
-  const float m = Conv<T>::load(mn, gi);
+  const Dequant<T> dq(Conv<T>::load(scale, gi), Conv<T>::load(mn, gi));
   for (int d = threadIdx.x; d < gs; d += kThreads) {
     const int j = d / E, k = d % E;
     uint32_t c = 0;
     for (int i = 0; i < b; ++i) c |= ((s_word[k * b + i] >> j) & 1u) << i;
-    Conv<T>::store(out, gi * gs + d, Conv<T>::round((float)c / sc) + m);
+    Conv<T>::store(out, gi * gs + d, dq(c));
   }
 }
 
@@ -469,7 +484,7 @@ int launch_pack(const void* data, const void* mn, const void* mx, const int32_t*
   const T* d = static_cast<const T*>(data);
   const T* nz = static_cast<const T*>(noise);
   if (gs == kGs) {
-    constexpr int kGroupsPerBlock = kHalfWaves * ACTNN_PACK_GPH;
+    constexpr int kGroupsPerBlock = kHalfWaves * Gph<T>::kPack;
     const int64_t bps = (G + kGroupsPerBlock - 1) / kGroupsPerBlock;
     if (N * bps > 0x7fffffffLL) return ACTNN_EINVAL;
     const dim3 grid((unsigned)(N * bps));
@@ -501,7 +516,7 @@ int launch_unpack(const int32_t* packed, const int32_t* bits, const int32_t* pre
                   const void* scale, const void* mn, void* out, int64_t N, int64_t G, int64_t gs,
                   hipStream_t s) {
   if (gs == kGs) {
-    constexpr int kGroupsPerBlock = kHalfWaves * ACTNN_UNPACK_GPH;
+    constexpr int kGroupsPerBlock = kHalfWaves * Gph<T>::kUnpack;
     const int64_t bps = (G + kGroupsPerBlock - 1) / kGroupsPerBlock;
     if (N * bps > 0x7fffffffLL) return ACTNN_EINVAL;
     unpack_mixed_kernel<T><<<dim3((unsigned)(N * bps)), dim3(kThreads), 0, s>>>(

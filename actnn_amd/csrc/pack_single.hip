@@ -101,14 +101,12 @@ __global__ __launch_bounds__(kThreads) void unpack_single_kernel(
     const int64_t n = no * WPT + ni;
     if (n < N) {
       const int64_t gi = n * G + g;
-      const float sc = Conv<T>::load(scale, gi);
-      const float m = Conv<T>::load(mn, gi);
+      const Dequant<T> dq(Conv<T>::load(scale, gi), Conv<T>::load(mn, gi));
       float v[8];
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
         const uint32_t word = k < 4 ? w.x : w.y;
-        const uint32_t c = (word >> (8 * (k & 3) + ni * BITS)) & kMask;
-        v[k] = Conv<T>::round(Conv<T>::round((float)c / sc) + m);    // .cu:359
+        v[k] = dq((word >> (8 * (k & 3) + ni * BITS)) & kMask);
       }
       store8(out + gi * gs + d0, v);
     }

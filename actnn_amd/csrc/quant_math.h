@@ -54,6 +54,39 @@ template <typename T> ACTNN_DEV uint32_t det_code(float x, float noise, float mu
   return (uint32_t)(int)rintf(t);
 }
 
+// Dequantisation (scalar_t)code / scale + min with one rounding per operation (.cu:171, :359).
+// For fp32 the quotient is the IEEE division.  For 16-bit types the quotient only has to be right
+// after rounding to 8 or 11 significant bits, so it is computed as code * (1/scale) with one
+// Newton step on the reciprocal and one residual correction (Markstein's sequence), which costs 3
+// operations per element instead of ~12; tests/test_gpu_unpack_exhaustive.py checks it against
+// the true division for every 16-bit scale value and every code.  Scales that are not ordinary
+// positive numbers (inf for constant groups in fp16, 0, NaN) take the IEEE path.
+template <typename T> struct Dequant {
+  float sc, m, r;
+  bool fast;
+  ACTNN_DEV Dequant(float scale, float mn) : sc(scale), m(mn), r(0.0f), fast(false) {
+    if (sizeof(T) == 2) {
+      const float a = fabsf(scale);
+      fast = a > 1e-30f && a < 1e30f;           // false for NaN too
+      if (fast) {
+        const float r0 = __builtin_amdgcn_rcpf(scale);
+        r = fmaf(fmaf(-scale, r0, 1.0f), r0, r0);
+      }
+    }
+  }
+  ACTNN_DEV float operator()(uint32_t code) const {
+    const float c = (float)code;
+    float q;
+    if (sizeof(T) == 2 && fast) {
+      const float q0 = c * r;
+      q = fmaf(fmaf(-sc, q0, c), r, q0);
+    } else {
+      q = c / sc;
+    }
+    return Conv<T>::round(Conv<T>::round(q) + m);
+  }
+};
+
 // RNG code: fix = trunc(clamp(fma(x - min, scale * 2^16, 0.5), 0, B * 2^16)); (fix + r16) >> 16.
 ACTNN_DEV uint32_t rng_code(float x, uint32_t r16, float mul, float sub, float Bfix) {
   const float d = x - sub;
