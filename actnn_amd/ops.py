@@ -232,6 +232,20 @@ class conv3d(Function):
 # ------------------------------------------------------------------------------------------
 # linear (ops.py:386-433)
 # ------------------------------------------------------------------------------------------
+def _fused_grad_weight_ok(quantized, shape, go):
+    """The fused kernel applies to a 2-D input saved with the 2-bit fixed-width stream whose rows
+    are whole groups, with 16-bit gradients and native (not bf16-compacted) scale/min."""
+    if not config.compress_activation or config.simulate or config.swap:
+        return False
+    q_input, q_bits, q_scale, q_min = quantized
+    return (isinstance(q_bits, int) and q_bits == 2 and len(shape) == 2
+            and shape[-1] % config.group_size == 0 and config.group_size == 256
+            and shape[0] % 4 == 0 and go.shape[1] % 8 == 0
+            and go.dtype in (torch.float16, torch.bfloat16) and q_scale.dtype == go.dtype
+            and q_input.is_cuda)
+
+
+
 class linear(Function):
     @staticmethod
     def forward(ctx, input, weight, bias=None, scheme=None):
@@ -250,13 +264,22 @@ class linear(Function):
             ctx.scheme.set_scale(grad_output)
         quantized, weight, bias = ctx.saved
         q_input_shape = ctx.other_args
-        input = dequantize_activation(quantized, q_input_shape)
+        go = grad_output.reshape(-1, grad_output.shape[-1])
+        if _fused_grad_weight_ok(quantized, q_input_shape, go):
+            # 2-bit fixed-width input: the weight gradient is computed straight from the packed
+            # stream (dequantised tiles only ever exist in LDS), nothing is materialised
+            q_input, _, q_scale, q_min = quantized
+            grad_weight = ext_quantization.linear_grad_weight_q2(
+                go, q_input, q_scale, q_min, q_input_shape[-1], weight.dtype) \
+                if ctx.needs_input_grad[1] else None
+        else:
+            input = dequantize_activation(quantized, q_input_shape)
+            x = input.reshape(-1, input.shape[-1])
+            grad_weight = go.t().mm(x) if ctx.needs_input_grad[1] else None
+            del input, x
         del quantized, ctx.saved
         empty_cache(config.empty_cache_threshold)
-        go = grad_output.reshape(-1, grad_output.shape[-1])
-        x = input.reshape(-1, input.shape[-1])
         grad_input = go.mm(weight).view(*q_input_shape) if ctx.needs_input_grad[0] else None
-        grad_weight = go.t().mm(x) if ctx.needs_input_grad[1] else None
         grad_bias = go.sum(0) if bias is not None and ctx.needs_input_grad[2] else None
         if ctx.scheme:
             ctx.scheme.if_allocate_perlayer()

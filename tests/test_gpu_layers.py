@@ -126,6 +126,32 @@ def test_linear_without_compression_matches_torch():
         assert torch.allclose(a, b, atol=1e-4, rtol=1e-4)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_qlinear_fused_weight_gradient_path(dtype):
+    # fixed 2-bit width (no adaptive scheme): linear.backward takes the fused GEMM; the result must
+    # agree with the unfused path (unpack + mm) run on the same packed input
+    config.activation_compression_bits = [2]
+    config.adaptive_conv_scheme = False
+    torch.manual_seed(0)
+    q = actnn_amd.QLinear(512, 264).to(DEV).to(dtype)
+    x = torch.randn(64, 512, device=DEV, dtype=dtype)
+    g = torch.randn(64, 264, device=DEV, dtype=dtype)
+    from actnn_amd import ops
+    torch.cuda.manual_seed(7)
+    _, gx_f, gp_f = _grads(q, x, g)
+    q.zero_grad()
+    saved = ops._fused_grad_weight_ok
+    ops._fused_grad_weight_ok = lambda *a: False
+    try:
+        torch.cuda.manual_seed(7)                 # same Philox stream -> same packed input
+        _, gx_u, gp_u = _grads(q, x, g)
+    finally:
+        ops._fused_grad_weight_ok = saved
+    assert torch.equal(gx_f, gx_u)
+    assert (gp_f[0].float() - gp_u[0].float()).norm() / gp_u[0].float().norm() < 1e-2
+    assert torch.equal(gp_f[1], gp_u[1])
+
+
 def test_l3_first_step_uses_the_degenerate_allocation_then_rebalances():
     # gradient scale starts at 0 (qscheme.py:24): the first forward gives 8 bits to the first
     # samples and 1 to the rest; after one backward the scale is positive and bits follow C
