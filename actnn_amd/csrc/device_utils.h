@@ -86,6 +86,7 @@ ACTNN_DEV u32x4 load16_b16(const void* p) {
 #endif
 }
 ACTNN_DEV void store16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
+ACTNN_DEV void store16_nt(void* p, u32x4 v) { __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p)); }
 
 // ------------------------------------------------------------------ 8 / 16 contiguous elements
 // load8: 8 consecutive elements starting at p (32-byte aligned for f32, 16 for 16-bit types).
@@ -116,6 +117,27 @@ ACTNN_DEV void load8(const bf16_t* p, float (&v)[8]) {
     v[2 * i + 1] = as_float(w[i] & 0xffff0000u);
   }
 }
+// Non-temporal variants for streams that are touched once and whose cache lines are covered whole
+// by one instruction of the wave (16 bytes per lane, lanes contiguous).
+ACTNN_DEV void load8_nt(const float* p, float (&v)[8]) { load8(p, v); }   // fp32: 32 bytes per lane, plain
+ACTNN_DEV void load8_nt(const __half* p, float (&v)[8]) {
+  const u32x4 a = load16_nt(p);
+  const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = half_bits_to_float(w[i] & 0xffffu);
+    v[2 * i + 1] = half_bits_to_float(w[i] >> 16);
+  }
+}
+ACTNN_DEV void load8_nt(const bf16_t* p, float (&v)[8]) {
+  const u32x4 a = load16_nt(p);
+  const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = as_float(w[i] << 16);
+    v[2 * i + 1] = as_float(w[i] & 0xffff0000u);
+  }
+}
 ACTNN_DEV void store8(float* p, const float (&v)[8]) {
   u32x4 a, b;
 #pragma unroll
@@ -137,6 +159,20 @@ ACTNN_DEV void store8(bf16_t* p, const float (&v)[8]) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) w[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
   store16(p, (u32x4){w[0], w[1], w[2], w[3]});
+}
+
+ACTNN_DEV void store8_nt(float* p, const float (&v)[8]) { store8(p, v); }  // fp32: 32 bytes per lane, plain
+ACTNN_DEV void store8_nt(__half* p, const float (&v)[8]) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = float_to_half_bits(v[2 * i]) | (float_to_half_bits(v[2 * i + 1]) << 16);
+  store16_nt(p, (u32x4){w[0], w[1], w[2], w[3]});
+}
+ACTNN_DEV void store8_nt(bf16_t* p, const float (&v)[8]) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+  store16_nt(p, (u32x4){w[0], w[1], w[2], w[3]});
 }
 
 // ------------------------------------------------------------------ cross-lane exchange

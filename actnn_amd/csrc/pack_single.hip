@@ -50,7 +50,7 @@ __global__ __launch_bounds__(kThreads) void pack_single_kernel(
     if (n < N) {
       const int64_t gi = n * G + g;
       const int64_t e = gi * gs + d0;
-      load8(data + e, v[ni]);
+      load8_nt(data + e, v[ni]);        // 16-bit types: one whole-line access per wave instruction
       if (DET) load8(noise + e, nz[DET ? ni : 0]);
       const float sc = Conv<T>::load(scale, gi);
       const float m = Conv<T>::load(mn, gi);
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(kThreads) void unpack_single_kernel(
         const uint32_t word = k < 4 ? w.x : w.y;
         v[k] = dq((word >> (8 * (k & 3) + ni * BITS)) & kMask);
       }
-      store8(out + gi * gs + d0, v);
+      store8_nt(out + gi * gs + d0, v);
     }
   }
 }

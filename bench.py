@@ -182,6 +182,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the config-2 hot path")
+    ap.add_argument("--only", choices=["other", "resnet50"], default=None,
+                    help="profiling aid: run just the other single-GPU configs (ReLU, max-pool, "
+                         "fixed-width pack, fused GEMM) or just the ResNet-50 L3 step, print their JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the hot path shards by sample with no exchange step, "
@@ -195,6 +198,13 @@ def main():
 
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.only == "other":
+        print(json.dumps({"other_configs": other_configs(device, max(10, args.steps // 2))}))
+        return
+    if args.only == "resnet50":
+        from actnn_amd import bench_extra
+        print(json.dumps({"resnet50_L3": bench_extra.resnet50_step(device, "L3", warmup=2, steps=3)}))
+        return
     xg, mn, mx, bits, bits_host = make_config2(device)
     N, G, gs = xg.shape
     n = xg.numel()
