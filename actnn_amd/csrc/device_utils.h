@@ -216,6 +216,29 @@ ACTNN_DEV uint32_t transpose32(uint32_t x, uint32_t lane) {
   return x;
 }
 
+// Two interleaved 32x32 bit transposes over the whole wave: the even lanes hold the 32 rows of
+// one matrix (row j in lane 2j), the odd lanes those of another (row j in lane 2j+1).  Afterwards
+// bit j of lane 2p+h is what bit p of lane 2j+h was.  Partner lanes are lane ^ 32, 16, 8, 4, 2.
+template <int S> ACTNN_DEV uint32_t transpose_stage_x2(uint32_t x, uint32_t lane) {
+  constexpr uint32_t M = S == 16 ? 0xFFFF0000u : S == 8 ? 0xFF00FF00u : S == 4 ? 0xF0F0F0F0u
+                       : S == 2 ? 0xCCCCCCCCu : 0xAAAAAAAAu;
+  uint32_t p;
+  if constexpr (S == 16) p = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((lane ^ 32u) << 2), (int)x);   // lane ^ 32
+  else p = lane_xor<2 * S>(x);
+  const bool hi = (lane & (2 * S)) != 0;
+  const uint32_t u = __builtin_amdgcn_alignbit(p, p, hi ? S : 32 - S);
+  const uint32_t sel = hi ? M : ~M;
+  return (x & sel) | (u & ~sel);
+}
+ACTNN_DEV uint32_t transpose32_x2(uint32_t x, uint32_t lane) {
+  x = transpose_stage_x2<16>(x, lane);
+  x = transpose_stage_x2<8>(x, lane);
+  x = transpose_stage_x2<4>(x, lane);
+  x = transpose_stage_x2<2>(x, lane);
+  x = transpose_stage_x2<1>(x, lane);
+  return x;
+}
+
 // Reductions over a DPP row (16 consecutive lanes); every lane ends with the result.
 ACTNN_DEV float row16_max(float v) {
   v = fmaxf(v, __builtin_bit_cast(float, lane_xor<1>(__builtin_bit_cast(uint32_t, v))));

@@ -24,7 +24,7 @@ __global__ __launch_bounds__(kThreads) void mask_forward_kernel(const T* __restr
                                                                 int32_t* __restrict__ mask, int64_t n,
                                                                 int64_t n_mask_blocks, uint32_t thr,
                                                                 float keep_div, uint64_t seed,
-                                                                uint64_t offset) {
+                                                                uint64_t offset, int64_t elem_offset) {
   const uint32_t lane = threadIdx.x & 31;
   const int64_t mb0 = (int64_t)blockIdx.x * kMaskBlocksPerBlock + (threadIdx.x >> 5) * 2;
   uint32_t acc = 0;
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(kThreads) void mask_forward_kernel(const T* __restr
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         uint32_t r16[8];
-        philox_octet((uint64_t)(e0 >> 3) + h, seed, offset, r16);
+        philox_octet((uint64_t)((elem_offset + e0) >> 3) + h, seed, offset, r16);
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
           const bool keep = r16[k] >= thr && e0 + h * 8 + k < n;
@@ -116,25 +116,144 @@ __global__ __launch_bounds__(kThreads) void mask_backward_kernel(const T* __rest
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// 16-bit element types: whole-line streaming variant.  A wave handles 4 mask blocks (2048
+// elements) with four wave-wide 16-byte non-temporal loads and stores, so that HBM sees only whole
+// cache lines.  Lane l then holds elements 8l..8l+7 of each block, i.e. half of the 16 elements a
+// mask row belongs to: lane pairs swap their 8-bit halves (one DPP move) so that the even lanes
+// hold the rows of blocks A|B and the odd lanes those of C|D, two interleaved 32x32 bit
+// transposes turn rows into mask words, and the 64 words leave as one 256-byte store.
+constexpr int kTileElems = 4 * kMaskBlock;        // elements per wave and iteration
+constexpr int kTilesPerBlock = kThreads / 64;
+
+// rows (per lane: 8 keep bits for each of the 4 blocks) -> this lane's transposed mask word
+ACTNN_DEV uint32_t rows_to_word(const uint32_t (&m)[4], uint32_t lane) {
+  const bool odd = lane & 1u;
+  const uint32_t ab = m[0] | (m[1] << 16), cd = m[2] | (m[3] << 16);
+  const uint32_t recv = lane_xor<1>(odd ? ab : cd);           // the half-row the partner computed for me
+  const uint32_t mine = odd ? cd : ab;
+  const uint32_t row = odd ? (recv | (mine << 8)) : (mine | (recv << 8));
+  return transpose32_x2(row, lane);
+}
+// inverse: this lane's mask word -> 8 keep bits for each of the 4 blocks
+ACTNN_DEV void word_to_rows(uint32_t w, uint32_t lane, uint32_t (&m)[4]) {
+  const bool odd = lane & 1u;
+  const uint32_t row = transpose32_x2(w, lane);                // even: row of A|B, odd: row of C|D
+  const uint32_t other = lane_xor<1>(row);
+  const uint32_t ab = odd ? other : row, cd = odd ? row : other;
+  const int sh = odd ? 8 : 0;
+  m[0] = (ab >> sh) & 0xffu;
+  m[1] = (ab >> (16 + sh)) & 0xffu;
+  m[2] = (cd >> sh) & 0xffu;
+  m[3] = (cd >> (16 + sh)) & 0xffu;
+}
+
+template <typename T, Op OP>
+__global__ __launch_bounds__(kThreads) void mask_forward16_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                                  int32_t* __restrict__ mask, int64_t tiles,
+                                                                  uint32_t thr, float keep_div,
+                                                                  uint64_t seed, uint64_t offset) {
+  const uint32_t lane = threadIdx.x & 63;
+  const int64_t tile = (int64_t)blockIdx.x * kTilesPerBlock + (threadIdx.x >> 6);
+  if (tile >= tiles) return;                       // whole waves leave together
+  const int64_t e0 = tile * kTileElems + lane * 8;
+  float v[4][8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) load8_nt(x + e0 + i * kMaskBlock, v[i]);
+  uint32_t m[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    uint32_t r16[8];
+    if (OP == Op::kDropout) philox_octet((uint64_t)((e0 + i * kMaskBlock) >> 3), seed, offset, r16);
+    m[i] = 0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const bool keep = OP == Op::kRelu ? v[i][k] > 0.0f : r16[k] >= thr;
+      v[i][k] = keep ? (OP == Op::kRelu ? v[i][k] : v[i][k] / keep_div) : 0.0f;
+      m[i] |= (uint32_t)keep << k;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) store8_nt(y + e0 + i * kMaskBlock, v[i]);
+  const uint32_t w = rows_to_word(m, lane);
+  // lane 2p+h holds word p % 16 of block 2h + p / 16
+  mask[tile * 64 + (lane & 1u) * 32 + (lane >> 1)] = (int32_t)w;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void mask_backward16_kernel(const T* __restrict__ gout,
+                                                                   const int32_t* __restrict__ mask,
+                                                                   T* __restrict__ gin, int64_t tiles,
+                                                                   float keep_div, bool divide) {
+  const uint32_t lane = threadIdx.x & 63;
+  const int64_t tile = (int64_t)blockIdx.x * kTilesPerBlock + (threadIdx.x >> 6);
+  if (tile >= tiles) return;
+  const int64_t e0 = tile * kTileElems + lane * 8;
+  float v[4][8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) load8_nt(gout + e0 + i * kMaskBlock, v[i]);
+  uint32_t m[4];
+  word_to_rows((uint32_t)mask[tile * 64 + (lane & 1u) * 32 + (lane >> 1)], lane, m);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const bool keep = (m[i] >> k) & 1u;
+      v[i][k] = keep ? (divide ? v[i][k] / keep_div : v[i][k]) : 0.0f;
+    }
+    store8_nt(gin + e0 + i * kMaskBlock, v[i]);
+  }
+}
+
 template <typename T, Op OP>
 int launch_forward(const void* x, void* y, int32_t* mask, int64_t n, uint32_t thr, float keep_div,
                    uint64_t seed, uint64_t offset, hipStream_t s) {
-  const int64_t nmb = (n + kMaskBlock - 1) / kMaskBlock;
-  const int64_t blocks = (nmb + kMaskBlocksPerBlock - 1) / kMaskBlocksPerBlock;
-  if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
-  mask_forward_kernel<T, OP><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
-      static_cast<const T*>(x), static_cast<T*>(y), mask, n, nmb, thr, keep_div, seed, offset);
+  const T* xi = static_cast<const T*>(x);
+  T* yo = static_cast<T*>(y);
+  int64_t done = 0;                               // elements handled by the whole-line kernel
+  if (sizeof(T) == 2) {
+    const int64_t tiles = n / kTileElems;
+    const int64_t tblocks = (tiles + kTilesPerBlock - 1) / kTilesPerBlock;
+    if (tblocks > 0x7fffffffLL) return ACTNN_EINVAL;
+    if (tiles > 0)
+      mask_forward16_kernel<T, OP><<<dim3((unsigned)tblocks), dim3(kThreads), 0, s>>>(
+          xi, yo, mask, tiles, thr, keep_div, seed, offset);
+    done = tiles * kTileElems;
+  }
+  const int64_t rest = n - done;
+  if (rest > 0) {
+    const int64_t nmb = (rest + kMaskBlock - 1) / kMaskBlock;
+    const int64_t blocks = (nmb + kMaskBlocksPerBlock - 1) / kMaskBlocksPerBlock;
+    if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
+    mask_forward_kernel<T, OP><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+        xi + done, yo + done, mask + done / 32, rest, nmb, thr, keep_div, seed, offset, done);
+  }
   ACTNN_RETURN_LAUNCH_STATUS();
 }
 
 template <typename T>
 int launch_backward(const void* gout, const int32_t* mask, void* gin, int64_t n, float keep_div,
                     bool divide, hipStream_t s) {
-  const int64_t nmb = (n + kMaskBlock - 1) / kMaskBlock;
-  const int64_t blocks = (nmb + kMaskBlocksPerBlock - 1) / kMaskBlocksPerBlock;
-  if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
-  mask_backward_kernel<T><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
-      static_cast<const T*>(gout), mask, static_cast<T*>(gin), n, nmb, keep_div, divide);
+  const T* go = static_cast<const T*>(gout);
+  T* gi = static_cast<T*>(gin);
+  int64_t done = 0;
+  if (sizeof(T) == 2) {
+    const int64_t tiles = n / kTileElems;
+    const int64_t tblocks = (tiles + kTilesPerBlock - 1) / kTilesPerBlock;
+    if (tblocks > 0x7fffffffLL) return ACTNN_EINVAL;
+    if (tiles > 0)
+      mask_backward16_kernel<T><<<dim3((unsigned)tblocks), dim3(kThreads), 0, s>>>(go, mask, gi, tiles,
+                                                                                   keep_div, divide);
+    done = tiles * kTileElems;
+  }
+  const int64_t rest = n - done;
+  if (rest > 0) {
+    const int64_t nmb = (rest + kMaskBlock - 1) / kMaskBlock;
+    const int64_t blocks = (nmb + kMaskBlocksPerBlock - 1) / kMaskBlocksPerBlock;
+    if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
+    mask_backward_kernel<T><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+        go + done, mask + done / 32, gi + done, rest, nmb, keep_div, divide);
+  }
   ACTNN_RETURN_LAUNCH_STATUS();
 }
 

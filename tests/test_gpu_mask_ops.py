@@ -11,7 +11,7 @@ from _util import DEV
 
 pytestmark = pytest.mark.gpu
 
-SHAPES = [(128, 56, 56, 31), (4, 512), (1, 1), (7,), (3, 171), (2, 8192), (5, 1025)]
+SHAPES = [(128, 56, 56, 31), (4, 512), (1, 1), (7,), (3, 171), (2, 8192), (5, 1025), (3, 6659)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
@@ -51,7 +51,7 @@ def test_relu_rejects_bad_arguments():
     assert ext_q.act_quantized_relu(torch.empty(0, device=DEV)).numel() == 0
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("p", [0.5, 0.1, 0.0, 1.0])
 def test_dropout(dtype, p):
     n = 1_000_003
