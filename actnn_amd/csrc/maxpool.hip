@@ -233,6 +233,153 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_backward_lds_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Stride-2 fast path (3x3 pad 1 and 2x2 pad 0 with W % 8 == 0, Wo == W / 2, Ho == H / 2): the
+// shapes of every stem / VGG-style pooling layer.  A thread produces 4 adjacent outputs from three
+// 16-byte LDS reads (forward) or 8 adjacent inputs of two rows from a handful of LDS reads
+// (backward), compares against compile-time window positions, and writes 8/16-byte pieces that are
+// contiguous across the wave.  Padding is handled by data, not by branches: the row above the
+// plane is staged as the initial value, out-of-range windows get an index that matches nothing.
+template <typename T> ACTNN_DEV void store4(T* p, const float (&v)[4]);
+template <> ACTNN_DEV void store4<float>(float* p, const float (&v)[4]) {
+  store16(p, (u32x4){as_uint(v[0]), as_uint(v[1]), as_uint(v[2]), as_uint(v[3])});
+}
+template <> ACTNN_DEV void store4<__half>(__half* p, const float (&v)[4]) {
+  *reinterpret_cast<u32x2*>(p) = (u32x2){float_to_half_bits(v[0]) | (float_to_half_bits(v[1]) << 16),
+                                         float_to_half_bits(v[2]) | (float_to_half_bits(v[3]) << 16)};
+}
+template <> ACTNN_DEV void store4<bf16_t>(bf16_t* p, const float (&v)[4]) {
+  *reinterpret_cast<u32x2*>(p) = (u32x2){pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+}
+
+template <typename T, int K, int P>
+__global__ __launch_bounds__(kThreads) void max_pool2d_forward_s2_kernel(
+    const T* __restrict__ x, T* __restrict__ y, int8_t* __restrict__ idx, PoolGeom g, int rows_per_band,
+    int bands) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int V = 16 / (int)sizeof(T);
+  T* s_in = reinterpret_cast<T*>(smem) + 8;             // front pad: column -1 of the first row is addressable
+  const int64_t nc = blockIdx.x / bands;
+  const int ho0 = (int)(blockIdx.x % bands) * rows_per_band;
+  const int rows_out = g.Ho - ho0 < rows_per_band ? g.Ho - ho0 : rows_per_band;
+  const int W = g.W, cpr = g.Wo >> 2;
+  const int i_first = 2 * ho0 - P;                      // -1 for the first band when P == 1
+  const int rows_in = 2 * (rows_out - 1) + K;
+  const int skip = i_first < 0 ? 1 : 0;
+  const float init = Conv<T>::round(-1e10f);            // as the reference, .cu:656
+  {
+    const T* src = x + (nc * g.H + i_first + skip) * (int64_t)W;
+    T* dst = s_in + skip * W;
+    const int nvec = (rows_in - skip) * (W / V);
+    for (int v = threadIdx.x; v < nvec; v += kThreads)
+      *reinterpret_cast<u32x4*>(dst + v * V) = load16_nt(src + (int64_t)v * V);
+    if (skip)
+      for (int v = threadIdx.x; v < W; v += kThreads) Conv<T>::store(s_in, v, init);
+  }
+  __syncthreads();
+  const int items = rows_out * cpr;
+  for (int item = threadIdx.x; item < items; item += kThreads) {
+    const int r = item / cpr, q = item - r * cpr;
+    float cc[K][9];                                     // cc[a][1 + e]: column 8q + e of window row a
+#pragma unroll
+    for (int a = 0; a < K; ++a) {
+      const T* row = s_in + (2 * r + a) * W + 8 * q;
+      load8(row, reinterpret_cast<float(&)[8]>(cc[a][1]));
+      cc[a][0] = init;
+      if (P == 1 && q > 0) cc[a][0] = lds_value<T>(row, -1);
+    }
+    float out[4];
+    uint32_t packed_idx = 0;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      float v = init;
+      uint32_t index = 0;
+#pragma unroll
+      for (int a = 0; a < K; ++a)
+#pragma unroll
+        for (int b = 0; b < K; ++b) {
+          const float c = cc[a][2 * u - P + b + 1];
+          if (c > v) {
+            v = c;
+            index = a * K + b;
+          }
+        }
+      out[u] = v;
+      packed_idx |= index << (8 * u);
+    }
+    const int64_t o = (nc * g.Ho + ho0 + r) * (int64_t)g.Wo + 4 * q;
+    store4<T>(y + o, out);
+    *reinterpret_cast<uint32_t*>(idx + o) = packed_idx;
+  }
+}
+
+template <typename T, int K, int P>
+__global__ __launch_bounds__(kThreads) void max_pool2d_backward_s2_kernel(
+    const T* __restrict__ gout, const int8_t* __restrict__ idx, T* __restrict__ gin, int64_t total_out,
+    PoolGeom g, int pairs_per_band, int bands, int max_out_rows) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int EXTRA = K == 3 ? 1 : 0;                 // windows of the next output row reach odd input rows
+  constexpr int NW = 4 + EXTRA;                         // output columns that touch 8 input columns
+  T* s_g = reinterpret_cast<T*>(smem);
+  int8_t* s_i = reinterpret_cast<int8_t*>(smem + (((size_t)max_out_rows * g.Wo + 16) * sizeof(T) + 15) / 16 * 16);
+  const int64_t nc = blockIdx.x / bands;
+  const int s0 = (int)(blockIdx.x % bands) * pairs_per_band;
+  const int pairs = g.Ho - s0 < pairs_per_band ? g.Ho - s0 : pairs_per_band;
+  const int ho_hi = s0 + pairs - 1 + EXTRA < g.Ho - 1 ? s0 + pairs - 1 + EXTRA : g.Ho - 1;
+  const int64_t first = (nc * g.Ho + s0) * (int64_t)g.Wo;
+  const int count = (ho_hi - s0 + 1) * g.Wo;
+  const int shift_g = stage_span(gout, first, count, total_out, s_g);
+  const int shift_i = stage_span(idx, first, count, total_out, s_i);
+  __syncthreads();
+  const int cpr = g.W >> 3;
+  const int items = pairs * cpr;
+  for (int item = threadIdx.x; item < items; item += kThreads) {
+    const int r = item / cpr, q = item - r * cpr;
+    float gv[1 + EXTRA][NW];
+    int iv[1 + EXTRA][NW];
+#pragma unroll
+    for (int j = 0; j <= EXTRA; ++j) {
+      const int at = (r + j) * g.Wo + 4 * q;
+      const bool row_ok = s0 + r + j < g.Ho;
+#pragma unroll
+      for (int t = 0; t < NW; ++t) {
+        gv[j][t] = lds_value<T>(s_g, shift_g + at + t);
+        const bool ok = row_ok && (t < 4 || q < cpr - 1);
+        iv[j][t] = ok ? (int)s_i[shift_i + at + t] : -1;
+      }
+    }
+#pragma unroll
+    for (int rr = 0; rr < 2; ++rr) {
+      float out[8];
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j <= EXTRA; ++j) {
+          const int kh = rr + P - 2 * j;
+          if (kh < 0 || kh >= K) continue;
+#pragma unroll
+          for (int t = 0; t < NW; ++t) {
+            const int kw = c + P - 2 * t;
+            if (kw < 0 || kw >= K) continue;
+            acc += iv[j][t] == kh * K + kw ? gv[j][t] : 0.0f;
+          }
+        }
+        out[c] = acc;
+      }
+      store8_nt(gin + (nc * g.H + 2 * (s0 + r) + rr) * (int64_t)g.W + 8 * q, out);
+    }
+  }
+}
+
+// the stride-2 kernels' shape requirements; K = 3 (pad 1) or 2 (pad 0)
+inline int s2_kernel_of(const PoolGeom& g) {
+  const int p = preset_of(g);
+  if (p != 1 && p != 2) return 0;
+  if (g.W % 8 != 0 || g.Wo * 2 != g.W || g.Ho * 2 != g.H) return 0;
+  return p == 1 ? 3 : 2;
+}
+
 // rows per band so that a block has about `want` elements of work and the LDS need (computed by
 // `bytes(rows)`) fits the budget; 0 if even one row does not fit.
 template <typename F> int pick_rows(int rows_total, int row_elems, int want, F bytes) {
@@ -242,10 +389,45 @@ template <typename F> int pick_rows(int rows_total, int row_elems, int want, F b
   return bytes(rows) <= (size_t)kLdsBudget ? rows : 0;
 }
 
+// Band height for the stride-2 kernels: `units` rows (or row pairs) of `per_unit` work items each
+// are cut into bands of equal height; a block walks its band in passes of kThreads items.  Picks
+// the height with the fewest idle thread slots among those that fit the LDS budget and need at
+// most 4 passes, preferring taller bands (fewer halo rows) on ties.  0 if nothing fits.
+template <typename F> int pick_band(int units, int per_unit, F bytes) {
+  int best = 0;
+  double best_eff = 0.0;
+  for (int rows = 1; rows <= units; ++rows) {
+    if (bytes(rows) > (size_t)kLdsBudget) break;
+    const int passes = (rows * per_unit + kThreads - 1) / kThreads;
+    if (passes > 4 && best > 0) break;
+    const int full = units / rows, rest = units % rows;
+    const int64_t slots = (int64_t)full * passes * kThreads +
+                          (rest ? (int64_t)((rest * per_unit + kThreads - 1) / kThreads) * kThreads : 0);
+    const double eff = (double)units * per_unit / (double)slots;
+    if (eff >= best_eff) {
+      best_eff = eff;
+      best = rows;
+    }
+  }
+  return best;
+}
+
 template <typename T>
 int launch_fwd(const void* x, void* y, int8_t* idx, int64_t total, const PoolGeom& g, hipStream_t s) {
   const int64_t planes = total / ((int64_t)g.Ho * g.Wo);
   auto need = [&](int rows) { return ((size_t)((rows - 1) * g.SH + g.KH) * g.W + 16) * sizeof(T); };
+  if (const int k = s2_kernel_of(g); k != 0 && aligned16(x) && aligned16(y) && aligned16(idx)) {
+    const int rb = pick_band(g.Ho, g.Wo / 4, need);
+    const int bands = rb > 0 ? (g.Ho + rb - 1) / rb : 0;
+    if (rb > 0 && planes * bands <= 0x7fffffffLL) {
+      const dim3 grid((unsigned)(planes * bands)), blk(kThreads);
+      const T* xi = static_cast<const T*>(x);
+      T* yo = static_cast<T*>(y);
+      if (k == 3) max_pool2d_forward_s2_kernel<T, 3, 1><<<grid, blk, need(rb), s>>>(xi, yo, idx, g, rb, bands);
+      else max_pool2d_forward_s2_kernel<T, 2, 0><<<grid, blk, need(rb), s>>>(xi, yo, idx, g, rb, bands);
+      ACTNN_RETURN_LAUNCH_STATUS();
+    }
+  }
   const int rb = pick_rows(g.Ho, g.Wo, 1024, need);
   if (rb > 0 && aligned16(x)) {
     const int bands = (g.Ho + rb - 1) / rb;
@@ -280,6 +462,24 @@ int launch_bwd(const void* gout, const int8_t* idx, void* gin, int64_t total, co
     const size_t elems = (size_t)out_rows(rows) * g.Wo + 16;
     return (elems * sizeof(T) + 15) / 16 * 16 + elems + 16;
   };
+  if (const int k = s2_kernel_of(g); k != 0 && aligned16(gout) && aligned16(idx) && aligned16(gin)) {
+    // bands of input-row pairs; pair s reads output rows s (and s + 1 for 3x3)
+    auto need2 = [&](int pairs) {
+      const size_t elems = (size_t)(pairs + 2) * g.Wo + 16;
+      return (elems * sizeof(T) + 15) / 16 * 16 + elems + 16;
+    };
+    const int pb = pick_band(g.Ho, g.W / 8, need2);
+    const int bands = pb > 0 ? (g.Ho + pb - 1) / pb : 0;
+    if (pb > 0 && planes * bands <= 0x7fffffffLL) {
+      const dim3 grid((unsigned)(planes * bands)), blk(kThreads);
+      const T* go = static_cast<const T*>(gout);
+      T* gi = static_cast<T*>(gin);
+      const int64_t tout = planes * g.Ho * g.Wo;
+      if (k == 3) max_pool2d_backward_s2_kernel<T, 3, 1><<<grid, blk, need2(pb), s>>>(go, idx, gi, tout, g, pb, bands, pb + 2);
+      else max_pool2d_backward_s2_kernel<T, 2, 0><<<grid, blk, need2(pb), s>>>(go, idx, gi, tout, g, pb, bands, pb + 2);
+      ACTNN_RETURN_LAUNCH_STATUS();
+    }
+  }
   const int rb = pick_rows(g.H, g.W, 2048, need);
   if (rb > 0 && aligned16(gout) && aligned16(idx)) {
     const int bands = (g.H + rb - 1) / rb;

@@ -17,7 +17,8 @@ GEOMS = [((3, 3), (2, 2), (1, 1)), ((2, 2), (2, 2), (0, 0)), ((3, 3), (1, 1), (1
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("k,s,p", GEOMS)
-@pytest.mark.parametrize("shape", [(4, 8, 28, 28), (2, 3, 13, 17), (1, 1, 5, 5)])
+@pytest.mark.parametrize("shape", [(4, 8, 28, 28), (2, 3, 13, 17), (1, 1, 5, 5), (3, 5, 32, 24),
+                                   (2, 3, 16, 8), (1, 2, 224, 224)])
 def test_forward_backward(dtype, k, s, p, shape):
     torch.manual_seed(sum(shape))
     x = torch.randn(*shape).to(dtype)
@@ -44,6 +45,28 @@ def test_ties_take_the_first_position():
     _, idx = ext_q.max_pool2d_forward(x, (3, 3), (2, 2), (1, 1), (1, 1))
     _, idx_o = pool.max_pool2d_forward(np.zeros((1, 1, 8, 8), np.float32), (3, 3), (2, 2), (1, 1))
     assert np.array_equal(idx.cpu().numpy(), idx_o)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("k,s,p", [((3, 3), (2, 2), (1, 1)), ((2, 2), (2, 2), (0, 0))])
+@pytest.mark.parametrize("shape", [(2, 3, 16, 24), (2, 3, 14, 18)])
+def test_special_values_follow_the_strict_compare(dtype, k, s, p, shape):
+    """-inf, NaN, +-0 and values below the -1e10 start never win a strict '>' from the start
+    value: output and index must follow the reference's scan (.cu:656-666) exactly, on the
+    stride-2 kernels (W % 8 == 0) and on the general ones."""
+    rng = np.random.default_rng(7)
+    npdt = np.float32 if dtype == torch.float32 else np.float16
+    x = rng.standard_normal(shape).astype(npdt)
+    special = np.array([-np.inf, np.nan, 0.0, -0.0, -3e10 if npdt == np.float32 else -65504.0, np.inf], npdt)
+    pick = rng.integers(0, 12, size=shape)
+    x = np.where(pick < 6, special[np.minimum(pick, 5)], x)
+    x[0, 0] = -np.inf                                    # whole windows of -inf / NaN
+    x[0, 1] = np.nan
+    y, idx = ext_q.max_pool2d_forward(torch.from_numpy(x).to(DEV), k, s, p, (1, 1))
+    out_o, idx_o = pool.max_pool2d_forward_literal(x, k, s, p)
+    assert np.array_equal(idx.cpu().numpy(), idx_o)
+    assert np.array_equal(y.cpu().numpy(), out_o, equal_nan=True)
+    assert np.array_equal(np.signbit(y.cpu().numpy()), np.signbit(out_o))
 
 
 def test_rejected_arguments():
