@@ -15,7 +15,12 @@
 namespace actnn {
 namespace {
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 256;             // general kernels
+// Stride-2 kernels (measured on 256x64x112x112 f16): the forward likes tall bands and streamed
+// (non-temporal) staging loads; the backward, whose bands share their edge rows and whose cache
+// lines are split between neighbouring blocks, likes short bands and cached loads.
+constexpr int kFwdS2Threads = 256, kFwdS2Passes = 4;
+constexpr int kBwdS2Threads = 128, kBwdS2Passes = 1;
 
 struct PoolGeom {
   int H, W, Ho, Wo, KH, KW, SH, SW, PH, PW;
@@ -90,20 +95,37 @@ constexpr int kLdsBudget = 48 * 1024;     // bytes of dynamic LDS a block may us
 // `total` elements whose base is 16-byte aligned) into LDS so that element first + i lands at
 // dst[shift + i], shift = first % (16 / sizeof(T)); aligned 16-byte loads wherever they stay
 // inside the tensor.  Returns shift.
-template <typename T>
+// Copy nvec 16-byte vectors from global memory (streamed, non-temporal) into LDS.  Loads are issued
+// in batches of 8 per thread before the first LDS write so that several are in flight at once.
+template <int THREADS, bool NT>
+ACTNN_DEV void copy_vectors(const void* __restrict__ src, void* dst, int nvec) {
+  constexpr int U = 8;
+  const u32x4* s = reinterpret_cast<const u32x4*>(src);
+  u32x4* d = reinterpret_cast<u32x4*>(dst);
+  for (int v0 = threadIdx.x; v0 < nvec; v0 += U * THREADS) {
+    u32x4 t[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (v0 + u * THREADS < nvec) t[u] = NT ? load16_nt(s + v0 + u * THREADS) : load16(s + v0 + u * THREADS);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (v0 + u * THREADS < nvec) d[v0 + u * THREADS] = t[u];
+  }
+}
+
+template <typename T, int THREADS = kThreads, bool NT = false>
 ACTNN_DEV int stage_span(const T* __restrict__ src, int64_t first, int count, int64_t total, T* dst) {
   constexpr int V = 16 / (int)sizeof(T);
   const int shift = (int)(first % V);
   const int64_t base = first - shift;                    // aligned element index
   const int nvec = (shift + count + V - 1) / V;
-  for (int v = threadIdx.x; v < nvec; v += kThreads) {
-    const int64_t e = base + (int64_t)v * V;
-    if (e + V <= total) {
-      *reinterpret_cast<u32x4*>(dst + v * V) = load16(src + e);
-    } else {
-      for (int i = 0; i < V; ++i)
-        if (e + i < total) dst[v * V + i] = src[e + i];
-    }
+  // only the last vector can reach past the end of the tensor
+  const bool ragged = base + (int64_t)nvec * V > total;
+  copy_vectors<THREADS, NT>(src + base, dst, ragged ? nvec - 1 : nvec);
+  if (ragged) {
+    const int64_t e = base + (int64_t)(nvec - 1) * V;
+    for (int i = threadIdx.x; i < V; i += THREADS)
+      if (e + i < total) dst[(nvec - 1) * V + i] = src[e + i];
   }
   return shift;
 }
@@ -252,8 +274,26 @@ template <> ACTNN_DEV void store4<bf16_t>(bf16_t* p, const float (&v)[4]) {
   *reinterpret_cast<u32x2*>(p) = (u32x2){pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
 }
 
+// 4 consecutive elements from LDS (8/16-byte aligned)
+ACTNN_DEV void load4(const float* p, float (&v)[4]) {
+  const u32x4 a = *reinterpret_cast<const u32x4*>(p);
+  v[0] = as_float(a.x), v[1] = as_float(a.y), v[2] = as_float(a.z), v[3] = as_float(a.w);
+}
+ACTNN_DEV void load4(const __half* p, float (&v)[4]) {
+  const u32x2 a = *reinterpret_cast<const u32x2*>(p);
+  const uint32_t lo = a.x, hi = a.y;
+  v[0] = half_bits_to_float(lo & 0xffffu), v[1] = half_bits_to_float(lo >> 16);
+  v[2] = half_bits_to_float(hi & 0xffffu), v[3] = half_bits_to_float(hi >> 16);
+}
+ACTNN_DEV void load4(const bf16_t* p, float (&v)[4]) {
+  const u32x2 a = *reinterpret_cast<const u32x2*>(p);
+  const uint32_t lo = a.x, hi = a.y;
+  v[0] = as_float(lo << 16), v[1] = as_float(lo & 0xffff0000u);
+  v[2] = as_float(hi << 16), v[3] = as_float(hi & 0xffff0000u);
+}
+
 template <typename T, int K, int P>
-__global__ __launch_bounds__(kThreads) void max_pool2d_forward_s2_kernel(
+__global__ __launch_bounds__(kFwdS2Threads) void max_pool2d_forward_s2_kernel(
     const T* __restrict__ x, T* __restrict__ y, int8_t* __restrict__ idx, PoolGeom g, int rows_per_band,
     int bands) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -270,23 +310,21 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_forward_s2_kernel(
   {
     const T* src = x + (nc * g.H + i_first + skip) * (int64_t)W;
     T* dst = s_in + skip * W;
-    const int nvec = (rows_in - skip) * (W / V);
-    for (int v = threadIdx.x; v < nvec; v += kThreads)
-      *reinterpret_cast<u32x4*>(dst + v * V) = load16_nt(src + (int64_t)v * V);
+    copy_vectors<kFwdS2Threads, true>(src, dst, (rows_in - skip) * (W / V));
     if (skip)
-      for (int v = threadIdx.x; v < W; v += kThreads) Conv<T>::store(s_in, v, init);
+      for (int v = threadIdx.x; v < W; v += kFwdS2Threads) Conv<T>::store(s_in, v, init);
   }
   __syncthreads();
   const int items = rows_out * cpr;
-  for (int item = threadIdx.x; item < items; item += kThreads) {
+  for (int item = threadIdx.x; item < items; item += kFwdS2Threads) {
     const int r = item / cpr, q = item - r * cpr;
     float cc[K][9];                                     // cc[a][1 + e]: column 8q + e of window row a
 #pragma unroll
     for (int a = 0; a < K; ++a) {
       const T* row = s_in + (2 * r + a) * W + 8 * q;
       load8(row, reinterpret_cast<float(&)[8]>(cc[a][1]));
-      cc[a][0] = init;
-      if (P == 1 && q > 0) cc[a][0] = lds_value<T>(row, -1);
+      const float left = lds_value<T>(row, -1);         // the front pad keeps this inside LDS
+      cc[a][0] = P == 1 && q > 0 ? left : init;
     }
     float out[4];
     uint32_t packed_idx = 0;
@@ -314,7 +352,7 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_forward_s2_kernel(
 }
 
 template <typename T, int K, int P>
-__global__ __launch_bounds__(kThreads) void max_pool2d_backward_s2_kernel(
+__global__ __launch_bounds__(kBwdS2Threads) void max_pool2d_backward_s2_kernel(
     const T* __restrict__ gout, const int8_t* __restrict__ idx, T* __restrict__ gin, int64_t total_out,
     PoolGeom g, int pairs_per_band, int bands, int max_out_rows) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -328,12 +366,12 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_backward_s2_kernel(
   const int ho_hi = s0 + pairs - 1 + EXTRA < g.Ho - 1 ? s0 + pairs - 1 + EXTRA : g.Ho - 1;
   const int64_t first = (nc * g.Ho + s0) * (int64_t)g.Wo;
   const int count = (ho_hi - s0 + 1) * g.Wo;
-  const int shift_g = stage_span(gout, first, count, total_out, s_g);
-  const int shift_i = stage_span(idx, first, count, total_out, s_i);
+  const int shift_g = stage_span<T, kBwdS2Threads, false>(gout, first, count, total_out, s_g);
+  const int shift_i = stage_span<int8_t, kBwdS2Threads, false>(idx, first, count, total_out, s_i);
   __syncthreads();
   const int cpr = g.W >> 3;
   const int items = pairs * cpr;
-  for (int item = threadIdx.x; item < items; item += kThreads) {
+  for (int item = threadIdx.x; item < items; item += kBwdS2Threads) {
     const int r = item / cpr, q = item - r * cpr;
     float gv[1 + EXTRA][NW];
     int iv[1 + EXTRA][NW];
@@ -341,11 +379,14 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_backward_s2_kernel(
     for (int j = 0; j <= EXTRA; ++j) {
       const int at = (r + j) * g.Wo + 4 * q;
       const bool row_ok = s0 + r + j < g.Ho;
+      // Wo % 4 == 0 makes both positions 4-element aligned
+      load4(s_g + shift_g + at, reinterpret_cast<float(&)[4]>(gv[j][0]));
+      const uint32_t i4 = *reinterpret_cast<const uint32_t*>(s_i + shift_i + at);
 #pragma unroll
-      for (int t = 0; t < NW; ++t) {
-        gv[j][t] = lds_value<T>(s_g, shift_g + at + t);
-        const bool ok = row_ok && (t < 4 || q < cpr - 1);
-        iv[j][t] = ok ? (int)s_i[shift_i + at + t] : -1;
+      for (int t = 0; t < 4; ++t) iv[j][t] = row_ok ? (int)((i4 >> (8 * t)) & 0xffu) : -1;
+      if (EXTRA) {
+        gv[j][NW - 1] = lds_value<T>(s_g, shift_g + at + 4);
+        iv[j][NW - 1] = row_ok && q < cpr - 1 ? (int)s_i[shift_i + at + 4] : -1;
       }
     }
 #pragma unroll
@@ -390,19 +431,19 @@ template <typename F> int pick_rows(int rows_total, int row_elems, int want, F b
 }
 
 // Band height for the stride-2 kernels: `units` rows (or row pairs) of `per_unit` work items each
-// are cut into bands of equal height; a block walks its band in passes of kThreads items.  Picks
+// are cut into bands of equal height; a block of `threads` walks its band in passes of `threads` items.  Picks
 // the height with the fewest idle thread slots among those that fit the LDS budget and need at
-// most 4 passes, preferring taller bands (fewer halo rows) on ties.  0 if nothing fits.
-template <typename F> int pick_band(int units, int per_unit, F bytes) {
+// most `max_passes` passes, preferring taller bands (fewer halo rows) on ties.  0 if nothing fits.
+template <typename F> int pick_band(int units, int per_unit, int threads, int max_passes, F bytes) {
   int best = 0;
   double best_eff = 0.0;
   for (int rows = 1; rows <= units; ++rows) {
     if (bytes(rows) > (size_t)kLdsBudget) break;
-    const int passes = (rows * per_unit + kThreads - 1) / kThreads;
-    if (passes > 4 && best > 0) break;
+    const int passes = (rows * per_unit + threads - 1) / threads;
+    if (passes > max_passes && best > 0) break;
     const int full = units / rows, rest = units % rows;
-    const int64_t slots = (int64_t)full * passes * kThreads +
-                          (rest ? (int64_t)((rest * per_unit + kThreads - 1) / kThreads) * kThreads : 0);
+    const int64_t slots = (int64_t)full * passes * threads +
+                          (rest ? (int64_t)((rest * per_unit + threads - 1) / threads) * threads : 0);
     const double eff = (double)units * per_unit / (double)slots;
     if (eff >= best_eff) {
       best_eff = eff;
@@ -417,10 +458,10 @@ int launch_fwd(const void* x, void* y, int8_t* idx, int64_t total, const PoolGeo
   const int64_t planes = total / ((int64_t)g.Ho * g.Wo);
   auto need = [&](int rows) { return ((size_t)((rows - 1) * g.SH + g.KH) * g.W + 16) * sizeof(T); };
   if (const int k = s2_kernel_of(g); k != 0 && aligned16(x) && aligned16(y) && aligned16(idx)) {
-    const int rb = pick_band(g.Ho, g.Wo / 4, need);
+    const int rb = pick_band(g.Ho, g.Wo / 4, kFwdS2Threads, kFwdS2Passes, need);
     const int bands = rb > 0 ? (g.Ho + rb - 1) / rb : 0;
     if (rb > 0 && planes * bands <= 0x7fffffffLL) {
-      const dim3 grid((unsigned)(planes * bands)), blk(kThreads);
+      const dim3 grid((unsigned)(planes * bands)), blk(kFwdS2Threads);
       const T* xi = static_cast<const T*>(x);
       T* yo = static_cast<T*>(y);
       if (k == 3) max_pool2d_forward_s2_kernel<T, 3, 1><<<grid, blk, need(rb), s>>>(xi, yo, idx, g, rb, bands);
@@ -468,10 +509,10 @@ int launch_bwd(const void* gout, const int8_t* idx, void* gin, int64_t total, co
       const size_t elems = (size_t)(pairs + 2) * g.Wo + 16;
       return (elems * sizeof(T) + 15) / 16 * 16 + elems + 16;
     };
-    const int pb = pick_band(g.Ho, g.W / 8, need2);
+    const int pb = pick_band(g.Ho, g.W / 8, kBwdS2Threads, kBwdS2Passes, need2);
     const int bands = pb > 0 ? (g.Ho + pb - 1) / pb : 0;
     if (pb > 0 && planes * bands <= 0x7fffffffLL) {
-      const dim3 grid((unsigned)(planes * bands)), blk(kThreads);
+      const dim3 grid((unsigned)(planes * bands)), blk(kBwdS2Threads);
       const T* go = static_cast<const T*>(gout);
       T* gi = static_cast<T*>(gin);
       const int64_t tout = planes * g.Ho * g.Wo;
