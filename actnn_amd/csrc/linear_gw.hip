@@ -10,16 +10,23 @@
 // v_mfma_f32_32x32x16_bf16 (bf16 gradients) or v_mfma_f32_32x32x16_f16 (fp16 gradients), with
 // fp32 accumulation.
 //
-// Tiling: the reduction runs over the samples m (K of the GEMM).  A 256-thread block owns a
-// 256 (O) x 128 (I) output tile - inside one quantisation group, so a block needs one scale/min
-// per sample - as 4 waves of 64 x 128, each 2 x 4 MFMA tiles of 32 x 32.  Two blocks fit on a
-// CU; they are not synchronised with each other, so one block's unpack/convert work overlaps the
-// other's MFMAs.  Per k-step of 32 samples (LDS tiles are double-buffered, one barrier per step):
-//   * grad_out rows are copied as they lie in memory (O contiguous, 16-byte vectors) into LDS as
-//     [k][o]; the MFMA "A" fragments (8 consecutive k for one o) are gathered from there with
-//     16-bit LDS reads;
-//   * the packed bytes already hold 4 consecutive k per feature, so a thread unpacks 8 features x
-//     4 samples and writes them k-contiguous: LDS [i][k], "B" fragments are single 16-byte reads.
+// Tiling: the reduction runs over the samples m (K of the GEMM).  A 512-thread block (one per CU)
+// owns a 256 (O) x 256 (I) output tile - one whole quantisation group, so a block needs one
+// scale/min per sample - as 8 waves of 64 x 128, each 2 x 4 MFMA tiles of 32 x 32.  The large tile
+// is what keeps the L2 -> CU traffic (grad_out is re-read once per column tile) below what the
+// vector caches deliver.  Per k-step of 64 samples (LDS tiles double-buffered, one barrier a step):
+//   * grad_out lies o-contiguous in memory but MFMA fragments want 8 consecutive k per row, so a
+//     thread loads 4 consecutive k-rows x 8 o's (16-byte vectors, a wave covers whole rows of the
+//     tile), transposes them in registers with 16 byte-permutes and writes 8 rows of 4 k's;
+//   * the packed bytes already hold 4 consecutive k per feature: a thread unpacks 2 x (4 features
+//     x 4 samples) from two 32-bit loads and writes them k-contiguous.  The samples of a thread are
+//     the same for its whole wave: 16 lanes fetch the wave's 8 scales and 8 minima with one load
+//     and v_readlane hands them out (scalar loads of one value per cache line were 40% of the
+//     kernel's time).
+//   Both LDS tiles are [row][k] with a 144-byte pitch, every MFMA fragment is one 16-byte LDS read.
+//   Rows are stored permuted - tile row o at LDS row (o % 8) * 32 + o / 8, tile column i at LDS row
+//   (i % 4) * 64 + i / 4 - which makes the lanes of a staging write hit consecutive LDS rows (no
+//   bank conflicts) and lets the epilogue store 4 consecutive columns per lane.
 // Global loads run two steps ahead of the MFMAs (register prefetch), LDS writes one step ahead.
 #include "device_utils.h"
 
@@ -30,17 +37,17 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int kThreads = 256;
-constexpr int BM = 256;            // output rows (O) per block
-#ifndef GW_BN
-#define GW_BN 128
+#ifndef GW_ABL
+#define GW_ABL 0
 #endif
-constexpr int BN = GW_BN;          // output columns (I) per block: half a quantisation group (or a whole one)
-constexpr int BK = 32;             // samples per k-step
-constexpr int kPitchA = BM + 8;    // 16-bit elements per k-row of the A tile  (528 bytes)
-constexpr int kPitchB = BK + 8;    // 16-bit elements per feature row of the B tile (80 bytes)
-constexpr int WM = 64;             // wave tile: 64 (O) x 128 (I) = 2 x 4 MFMA tiles of 32 x 32
-constexpr int NT = BN / 32;        // MFMA tiles per wave along I
+// tuning aid: bit 0 no MFMA, 1 no fragment reads, 2 no A LDS writes, 3 no B LDS writes, 4 no A loads, 5 no B loads, 6 no dequant
+constexpr int kThreads = 512;
+constexpr int BM = 256;            // output rows (O) per block
+constexpr int BN = 256;            // output columns (I) per block: one quantisation group
+constexpr int BK = 64;             // samples per k-step
+constexpr int kPitch = BK + 8;     // 16-bit elements per row of either LDS tile (144 bytes)
+constexpr int kTile = 256 * kPitch;                 // elements of one operand tile
+constexpr int kLdsBytes = 2 * 2 * kTile * 2;        // two operands, two buffers
 
 // The MFMA runs in the 16-bit format of grad_out, so its rows go to LDS exactly as loaded:
 // bf16 gradients (bf16 autocast) use v_mfma_f32_32x32x16_bf16 and the dequantised activations are
@@ -66,123 +73,201 @@ template <> struct Mma<__half> {
 
 template <typename T> struct RawScalar;          // a scale/min value exactly as loaded
 template <> struct RawScalar<float> {
-  typedef float type;
-  static ACTNN_DEV float widen(float v) { return v; }
+  static ACTNN_DEV uint32_t load(const float* p, int64_t i) { return as_uint(p[i]); }
+  static ACTNN_DEV float widen(uint32_t v) { return as_float(v); }
 };
 template <> struct RawScalar<__half> {
-  typedef uint16_t type;
-  static ACTNN_DEV float widen(uint16_t v) { return half_bits_to_float(v); }
+  static ACTNN_DEV uint32_t load(const __half* p, int64_t i) { return reinterpret_cast<const uint16_t*>(p)[i]; }
+  static ACTNN_DEV float widen(uint32_t v) { return half_bits_to_float(v); }
 };
 template <> struct RawScalar<bf16_t> {
-  typedef uint16_t type;
-  static ACTNN_DEV float widen(uint16_t v) { return bf16_bits_to_float(v); }
+  static ACTNN_DEV uint32_t load(const bf16_t* p, int64_t i) { return p[i].bits; }
+  static ACTNN_DEV float widen(uint32_t v) { return bf16_bits_to_float(v); }
 };
 
+template <typename TO> ACTNN_DEV void store_out4(TO* p, float a, float b, float c, float d);
+template <> ACTNN_DEV void store_out4<float>(float* p, float a, float b, float c, float d) {
+  store16(p, (u32x4){as_uint(a), as_uint(b), as_uint(c), as_uint(d)});
+}
+template <> ACTNN_DEV void store_out4<__half>(__half* p, float a, float b, float c, float d) {
+  *reinterpret_cast<u32x2*>(p) = (u32x2){float_to_half_bits(a) | (float_to_half_bits(b) << 16),
+                                         float_to_half_bits(c) | (float_to_half_bits(d) << 16)};
+}
+template <> ACTNN_DEV void store_out4<bf16_t>(bf16_t* p, float a, float b, float c, float d) {
+  *reinterpret_cast<u32x2*>(p) = (u32x2){pack_bf16x2(a, b), pack_bf16x2(c, d)};
+}
+
 template <typename TG, typename TS, typename TO>
-__global__ __launch_bounds__(kThreads, BN == 128 ? 2 : 1) void linear_gw_q2_kernel(
+__global__ __launch_bounds__(kThreads, 1) void linear_gw_q2_kernel(
     const TG* __restrict__ gout, const uint8_t* __restrict__ packed, const TS* __restrict__ scale,
     const TS* __restrict__ mn, TO* __restrict__ gw, int M, int O, int I) {
-  __shared__ __attribute__((aligned(16))) uint16_t sA[2][BK * kPitchA];
-  __shared__ __attribute__((aligned(16))) uint16_t sB[2][BN * kPitchB];
-  typedef typename RawScalar<TS>::type raw_t;
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  auto tileA = [&](int buf) { return smem + buf * 2 * kTile; };
+  auto tileB = [&](int buf) { return smem + buf * 2 * kTile + kTile; };
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wm = (tid >> 6) * WM;            // wave's row offset inside the block tile
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wr = wave & 3, wn = wave >> 2;   // the wave's 64-row group and 128-column half
   const int G = I / 256;
   // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give every XCD whole
   // panels of grad_out rows (all column tiles of tile_m), so that a panel is pulled into one L2
   // only and reused there by the tiles_n blocks that need it.
-  const int tiles_n = I / BN;
+  const int tiles_n = G;
   const int tiles_m = (O + BM - 1) / BM;
   int tile = blockIdx.x;
+#ifdef GW_RM
+  {  // experiment: XCD x owns a GW_RM x (32 / GW_RM) sub-grid of a 16 x 16 tile grid
+    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    constexpr int RN = 32 / GW_RM;
+    const int subs_n = tiles_n / RN;
+    const int xm = xcd / subs_n, xn = xcd % subs_n;
+    tile = (xm * GW_RM + idx / RN) * tiles_n + xn * RN + idx % RN;
+  }
+#else
   if (tiles_m % 8 == 0) {
     const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
     tile = (xcd * (tiles_m / 8) + idx / tiles_n) * tiles_n + idx % tiles_n;
   }
+#endif
   const int o0 = (tile / tiles_n) * BM;
-  const int i0 = (tile % tiles_n) * BN;
-  const int g = i0 / 256;                    // the block's columns lie inside quantisation group g
-  const int d0 = i0 % 256;                   // ... starting at feature d0 of the group
+  const int g = tile % tiles_n;              // the block's columns are quantisation group g
+  const int i0 = g * 256;
 
-  // A staging: 4 vectors of 8 o's per thread: k rows ar + 8 * r, o offset (tid % 32) * 8
-  // B staging: thread -> sample quad br = tid / 32 (4 consecutive k), features bi + 32 * e
-  const int ar = tid >> 5;
-  const int br = tid >> 5;
-  const int bi = tid & 31;
-  const bool ovalid = o0 + bi * 8 < O;       // O % 8 == 0: a vector is inside or outside as a whole
-  // running pointers, advanced by one k-step per prefetch
-  const TG* pa = gout + (int64_t)ar * O + o0 + bi * 8;
-  const uint8_t* pb = packed + ((int64_t)br * G + g) * 256 + d0 + bi;
-  const raw_t* psc = reinterpret_cast<const raw_t*>(scale) + (int64_t)(br * 4) * G + g;
-  const raw_t* pmn = reinterpret_cast<const raw_t*>(mn) + (int64_t)(br * 4) * G + g;
-  const int64_t a_step = (int64_t)BK * O, a_row8 = (int64_t)8 * O;
-  const int64_t b_step = (int64_t)(BK / 4) * G * 256, s_step = (int64_t)BK * G;
+  // A staging: thread -> k rows 4 * kqa .. + 3 of the step, o offset ao * 8 (a wave: 2 quads x whole rows)
+  // B staging: thread -> features 4 * fi .. + 3, sample quads `wave` and `wave + 8` of the step
+  const int ao = tid & 31, kqa = tid >> 5;
+  const int fi = lane;
+  const bool ovalid = o0 + ao * 8 < O;       // O % 8 == 0: a vector is inside or outside as a whole
+  // running pointers / indices, advanced by one k-step per prefetch
+  const TG* pa = gout + (int64_t)(kqa * 4) * O + o0 + ao * 8;
+  const uint8_t* pb = packed + ((int64_t)wave * G + g) * 256 + fi * 4;
+  int64_t si = (int64_t)(wave * 4) * G + g;  // index of the wave's first sample in scale / min
+  const int64_t a_step = (int64_t)BK * O;
+  const int64_t b_step = (int64_t)(BK / 4) * G * 256, b_half = (int64_t)8 * G * 256;
+  const int64_t s_step = (int64_t)BK * G, s_half = (int64_t)32 * G;
   int k_next = 0;                            // first sample of the step the next prefetch loads
 
-  f32x16 acc[2][NT];
+  f32x16 acc[2][4];
 #pragma unroll
   for (int a = 0; a < 2; ++a)
 #pragma unroll
-    for (int b = 0; b < NT; ++b)
+    for (int b = 0; b < 4; ++b)
 #pragma unroll
       for (int c = 0; c < 16; ++c) acc[a][b][c] = 0.0f;
 
   // Registers of the prefetch hold the data exactly as loaded: nothing may consume a load inside
   // `prefetch`, or the wave would wait out the memory latency there.
   u32x4 ra[4];
-  uint32_t rb[NT];
-  raw_t rsc[4], rmn[4];
-  bool rvalid = false;
+  uint32_t rb[2];
+  uint32_t rsm = 0;                          // lanes 0..15: scale / min of the wave's 8 samples
+  // lane l < 16 fetches for quad half h = l / 8: scale (l % 8 < 4) or min of sample l % 4
+  const int sm_h = (lane >> 3) & 1, sm_j = lane & 3;
+  const TS* sm_base = (lane & 4) ? mn : scale;
 
   auto prefetch = [&]() {
+    const bool avalid = ovalid && k_next + kqa * 4 < M;   // M % 4 == 0: a quad is inside or outside as a whole
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       ra[r] = (u32x4){0u, 0u, 0u, 0u};
-      if (ovalid && k_next + ar + 8 * r < M) ra[r] = load16(pa + r * a_row8);
+      if (avalid && !(GW_ABL & 16)) ra[r] = load16(pa + (int64_t)r * O);
     }
-    rvalid = k_next + br * 4 < M;            // M % 4 == 0: a quad is inside or outside as a whole
-    if (rvalid) {
 #pragma unroll
-      for (int e = 0; e < NT; ++e) rb[e] = pb[32 * e];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        rsc[j] = psc[(int64_t)j * G];
-        rmn[j] = pmn[(int64_t)j * G];
-      }
+    for (int h = 0; h < 2; ++h) {
+      rb[h] = 0u;
+      if (k_next + (wave + 8 * h) * 4 < M && !(GW_ABL & 32))   // wave-uniform
+        rb[h] = *reinterpret_cast<const uint32_t*>(pb + h * b_half);
     }
+    rsm = 0u;
+    if (lane < 16 && k_next + (wave + 8 * sm_h) * 4 < M && !(GW_ABL & 128))
+      rsm = RawScalar<TS>::load(sm_base, si + sm_h * s_half + (int64_t)sm_j * G);
     pa += a_step;
     pb += b_step;
-    psc += s_step;
-    pmn += s_step;
+    si += s_step;
     k_next += BK;
+#ifdef GW_SKEW
+    if (k_next >= M) {   // wrap around (experiment; assumes M % BK == 0)
+      pa -= (int64_t)M * O;
+      pb -= (int64_t)(M / 4) * G * 256;
+      si -= (int64_t)M * G;
+      k_next -= M;
+    }
+#endif
   };
 
-  auto stage = [&](int buf) {
+  // `kfirst` = first sample of the step being staged (rows past M dequantise to 0; their grad_out
+  // rows were loaded as 0)
+  auto stage = [&](int buf, int kfirst) {
+    uint16_t* sA = tileA(buf);
+    uint16_t* sB = tileB(buf);
+    // 4 (k) x 8 (o) -> 8 (o) x 4 (k): word p of ra[r] holds o = 2p (low half) and 2p + 1 (high half)
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-      *reinterpret_cast<u32x4*>(&sA[buf][(ar + 8 * r) * kPitchA + bi * 8]) = ra[r];
-    float inv[4], m4[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {            // rows past M dequantise to 0
-      inv[j] = rvalid ? __builtin_amdgcn_rcpf(RawScalar<TS>::widen(rsc[j])) : 0.0f;
-      m4[j] = rvalid ? RawScalar<TS>::widen(rmn[j]) : 0.0f;
+    for (int p2 = 0; p2 < 4; ++p2) {
+      const uint32_t w0 = ra[0][p2], w1 = ra[1][p2], w2 = ra[2][p2], w3 = ra[3][p2];
+      const u32x2 even = {__builtin_amdgcn_perm(w1, w0, 0x05040100u), __builtin_amdgcn_perm(w3, w2, 0x05040100u)};
+      const u32x2 odd = {__builtin_amdgcn_perm(w1, w0, 0x07060302u), __builtin_amdgcn_perm(w3, w2, 0x07060302u)};
+      if (!(GW_ABL & 4)) {
+      *reinterpret_cast<u32x2*>(&sA[((2 * p2) * 32 + ao) * kPitch + kqa * 4]) = even;
+      *reinterpret_cast<u32x2*>(&sA[((2 * p2 + 1) * 32 + ao) * kPitch + kqa * 4]) = odd;
+      }
     }
 #pragma unroll
-    for (int e = 0; e < NT; ++e) {
-      const uint32_t by = rvalid ? rb[e] : 0u;
-      const float x0 = fmaf((float)(by & 3u), inv[0], m4[0]);
-      const float x1 = fmaf((float)((by >> 2) & 3u), inv[1], m4[1]);
-      const float x2 = fmaf((float)((by >> 4) & 3u), inv[2], m4[2]);
-      const float x3 = fmaf((float)((by >> 6) & 3u), inv[3], m4[3]);
-      *reinterpret_cast<u32x2*>(&sB[buf][(bi + 32 * e) * kPitchB + br * 4]) =
-          (u32x2){Mma<TG>::pack2(x0, x1), Mma<TG>::pack2(x2, x3)};
+    for (int h = 0; h < 2; ++h) {
+      const bool bvalid = kfirst + (wave + 8 * h) * 4 < M;
+      float inv[4], m4[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t sc_raw = (uint32_t)__builtin_amdgcn_readlane((int)rsm, h * 8 + j);
+        const uint32_t mn_raw = (uint32_t)__builtin_amdgcn_readlane((int)rsm, h * 8 + 4 + j);
+        inv[j] = bvalid ? __builtin_amdgcn_rcpf(RawScalar<TS>::widen(sc_raw)) : 0.0f;
+        m4[j] = bvalid ? RawScalar<TS>::widen(mn_raw) : 0.0f;
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t by = rb[h] >> (8 * e);
+        const float x0 = fmaf((float)(by & 3u), inv[0], m4[0]);
+        const float x1 = fmaf((float)((by >> 2) & 3u), inv[1], m4[1]);
+        const float x2 = fmaf((float)((by >> 4) & 3u), inv[2], m4[2]);
+        const float x3 = fmaf((float)((by >> 6) & 3u), inv[3], m4[3]);
+        if (!(GW_ABL & 8))
+        *reinterpret_cast<u32x2*>(&sB[(e * 64 + fi) * kPitch + (wave + 8 * h) * 4]) =
+            (u32x2){Mma<TG>::pack2(x0, x1), Mma<TG>::pack2(x2, x3)};
+      }
+    }
+  };
+
+  auto multiply = [&](int buf) {
+    const uint16_t* sA = tileA(buf) + ((2 * wr) * 32 + (lane & 31)) * kPitch + (lane >> 5) * 8;
+    const uint16_t* sB = tileB(buf) + (wn * 32 + (lane & 31)) * kPitch + (lane >> 5) * 8;
+#pragma unroll
+    for (int kb = 0; kb < ((GW_ABL & 2) ? 0 : BK / 16); ++kb) {
+      u32x4 fa[2], fb[4];
+#pragma unroll
+      for (int a = 0; a < 2; ++a) fa[a] = *reinterpret_cast<const u32x4*>(sA + a * 32 * kPitch + kb * 16);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) fb[e] = *reinterpret_cast<const u32x4*>(sB + e * 64 * kPitch + kb * 16);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+          if (GW_ABL & 1) acc[a][e][0] += as_float(fa[a][0] ^ fb[e][1]);
+          else acc[a][e] = Mma<TG>::mfma(fa[a], fb[e], acc[a][e]);
+        }
     }
   };
 
   const int steps = (M + BK - 1) / BK;
+#ifdef GW_SKEW
+  {
+    const int start = (int)(((int64_t)(tile % tiles_n) * GW_SKEW) % steps);
+    pa += start * a_step;
+    pb += start * b_step;
+    si += start * s_step;
+    k_next = start * BK;
+  }
+#endif
   prefetch();
-  if (steps > 0) stage(0);
+  if (steps > 0) stage(0, 0);
   __syncthreads();
   if (steps > 1) prefetch();
 
@@ -190,48 +275,28 @@ __global__ __launch_bounds__(kThreads, BN == 128 ? 2 : 1) void linear_gw_q2_kern
     const int cur = t & 1;
     // write the tile of step t+1 into the other buffer (its last readers passed the barrier at
     // the end of step t-1), then get the loads of step t+2 in flight, then multiply step t
-    if (t + 1 < steps) stage(cur ^ 1);
+#ifdef GW_SKEW
+    if (t + 1 < steps) stage(cur ^ 1, 0);
+#else
+    if (t + 1 < steps) stage(cur ^ 1, (t + 1) * BK);
+#endif
     if (t + 2 < steps) prefetch();
-
-    // all fragments of the step first (LDS reads return in order, so the MFMAs below can start
-    // as soon as their operands are in), then the 2 x 2 x NT MFMAs
-    u32x4 fa[BK / 16][2], fb[BK / 16][NT];
-#pragma unroll
-    for (int kb = 0; kb < BK / 16; ++kb) {
-      const int kf = kb * 16 + (lane >> 5) * 8;      // this lane's first k in the step
-#pragma unroll
-      for (int b = 0; b < NT; ++b)
-        fb[kb][b] = *reinterpret_cast<const u32x4*>(&sB[cur][(b * 32 + (lane & 31)) * kPitchB + kf]);
-#pragma unroll
-      for (int a = 0; a < 2; ++a) {
-        const uint16_t* col = &sA[cur][kf * kPitchA + wm + a * 32 + (lane & 31)];
-        uint32_t w[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          w[j] = (uint32_t)col[(2 * j) * kPitchA] | ((uint32_t)col[(2 * j + 1) * kPitchA] << 16);
-        fa[kb][a] = (u32x4){w[0], w[1], w[2], w[3]};
-      }
-    }
-#pragma unroll
-    for (int kb = 0; kb < BK / 16; ++kb)
-#pragma unroll
-      for (int b = 0; b < NT; ++b)
-#pragma unroll
-        for (int a = 0; a < 2; ++a) acc[a][b] = Mma<TG>::mfma(fa[kb][a], fb[kb][b], acc[a][b]);
+    multiply(cur);
     __syncthreads();
   }
 
-  // 32x32 accumulator layout: register c of a lane is row 8*(c/4) + 4*(lane/32) + c%4, column lane%32
+  // 32x32 accumulator layout: register c of a lane is fragment row 8*(c/4) + 4*(lane/32) + c%4,
+  // fragment column lane%32.  Fragment row r of A-fragment a is tile row 8*r + 2*wr + a; fragment
+  // column l of B-fragment e is tile column 128*wn + 4*l + e.
 #pragma unroll
   for (int a = 0; a < 2; ++a) {
 #pragma unroll
-    for (int b = 0; b < NT; ++b) {
-      const int col = i0 + b * 32 + (lane & 31);
-#pragma unroll
-      for (int c = 0; c < 16; ++c) {
-        const int row = o0 + wm + a * 32 + 8 * (c >> 2) + 4 * (lane >> 5) + (c & 3);
-        if (row < O) Conv<TO>::store(gw, (int64_t)row * I + col, acc[a][b][c]);
-      }
+    for (int c = 0; c < 16; ++c) {
+      const int r = 8 * (c >> 2) + 4 * (lane >> 5) + (c & 3);
+      const int row = o0 + 8 * r + 2 * wr + a;
+      const int col = i0 + 128 * wn + 4 * (lane & 31);
+      if (row < O)
+        store_out4<TO>(gw + (int64_t)row * I + col, acc[a][0][c], acc[a][1][c], acc[a][2][c], acc[a][3][c]);
     }
   }
 }
@@ -241,7 +306,12 @@ int launch(const void* gout, const int8_t* packed, const void* scale, const void
            int64_t M, int64_t O, int64_t I, hipStream_t s) {
   const int64_t blocks = ((O + BM - 1) / BM) * (I / BN);
   if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
-  linear_gw_q2_kernel<TG, TS, TO><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+  auto kernel = linear_gw_q2_kernel<TG, TS, TO>;
+  // more than the 64 KB a kernel may use without asking
+  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  if (e != hipSuccess) return (int)e;
+  kernel<<<dim3((unsigned)blocks), dim3(kThreads), kLdsBytes, s>>>(
       static_cast<const TG*>(gout), reinterpret_cast<const uint8_t*>(packed),
       static_cast<const TS*>(scale), static_cast<const TS*>(mn), static_cast<TO*>(gw), (int)M, (int)O,
       (int)I);
@@ -282,7 +352,9 @@ extern "C" int actnn_linear_grad_weight_q2(const void* grad_out, const int8_t* p
   if (M > 0x7fffffffLL || O > 0x7fffffffLL || I > 0x7fffffffLL) return ACTNN_EINVAL;
   if (O == 0 || I == 0) return ACTNN_OK;
   if (!grad_w || (M > 0 && (!grad_out || !packed || !scale || !mn))) return ACTNN_EINVAL;
-  if (M > 0 && !aligned16(grad_out)) return ACTNN_EALIGN;
+  if (M > 0 && (!aligned16(grad_out) || !aligned16(grad_w) || reinterpret_cast<uintptr_t>(packed) % 4 != 0 ||
+                reinterpret_cast<uintptr_t>(scale) % 4 != 0 || reinterpret_cast<uintptr_t>(mn) % 4 != 0))
+    return ACTNN_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (go_dtype) {
     case ACTNN_F16: return launch_sm<__half>(sm_dtype, out_dtype, grad_out, packed, scale, mn, grad_w, M, O, I, s);
