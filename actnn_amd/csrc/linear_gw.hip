@@ -27,7 +27,7 @@
 //   Rows are stored permuted - tile row o at LDS row (o % 8) * 32 + o / 8, tile column i at LDS row
 //   (i % 4) * 64 + i / 4 - which makes the lanes of a staging write hit consecutive LDS rows (no
 //   bank conflicts) and lets the epilogue store 4 consecutive columns per lane.
-// Global loads run two steps ahead of the MFMAs (register prefetch), LDS writes one step ahead.
+// Global loads run two steps ahead of the MFMAs (two register sets), LDS writes one step ahead.
 #include "device_utils.h"
 
 namespace actnn {
@@ -37,10 +37,6 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-#ifndef GW_ABL
-#define GW_ABL 0
-#endif
-// tuning aid: bit 0 no MFMA, 1 no fragment reads, 2 no A LDS writes, 3 no B LDS writes, 4 no A loads, 5 no B loads, 6 no dequant
 constexpr int kThreads = 512;
 constexpr int BM = 256;            // output rows (O) per block
 constexpr int BN = 256;            // output columns (I) per block: one quantisation group
@@ -116,20 +112,10 @@ __global__ __launch_bounds__(kThreads, 1) void linear_gw_q2_kernel(
   const int tiles_n = G;
   const int tiles_m = (O + BM - 1) / BM;
   int tile = blockIdx.x;
-#ifdef GW_RM
-  {  // experiment: XCD x owns a GW_RM x (32 / GW_RM) sub-grid of a 16 x 16 tile grid
-    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-    constexpr int RN = 32 / GW_RM;
-    const int subs_n = tiles_n / RN;
-    const int xm = xcd / subs_n, xn = xcd % subs_n;
-    tile = (xm * GW_RM + idx / RN) * tiles_n + xn * RN + idx % RN;
-  }
-#else
   if (tiles_m % 8 == 0) {
     const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
     tile = (xcd * (tiles_m / 8) + idx / tiles_n) * tiles_n + idx % tiles_n;
   }
-#endif
   const int o0 = (tile / tiles_n) * BM;
   const int g = tile % tiles_n;              // the block's columns are quantisation group g
   const int i0 = g * 256;
@@ -146,7 +132,6 @@ __global__ __launch_bounds__(kThreads, 1) void linear_gw_q2_kernel(
   const int64_t a_step = (int64_t)BK * O;
   const int64_t b_step = (int64_t)(BK / 4) * G * 256, b_half = (int64_t)8 * G * 256;
   const int64_t s_step = (int64_t)BK * G, s_half = (int64_t)32 * G;
-  int k_next = 0;                            // first sample of the step the next prefetch loads
 
   f32x16 acc[2][4];
 #pragma unroll
@@ -156,132 +141,134 @@ __global__ __launch_bounds__(kThreads, 1) void linear_gw_q2_kernel(
 #pragma unroll
       for (int c = 0; c < 16; ++c) acc[a][b][c] = 0.0f;
 
-  // Registers of the prefetch hold the data exactly as loaded: nothing may consume a load inside
-  // `prefetch`, or the wave would wait out the memory latency there.
+  // The prefetch registers hold the data of the step after the one being multiplied, exactly as
+  // loaded (nothing may consume a load where it is issued, or the wave would wait out the memory
+  // latency there).  They are refilled as soon as the staging code has read them, most of a
+  // k-step before they are needed again.
   u32x4 ra[4];
   uint32_t rb[2];
-  uint32_t rsm = 0;                          // lanes 0..15: scale / min of the wave's 8 samples
+  uint32_t rsm = 0u;                         // lanes 0..15: scale / min of the wave's 8 samples
   // lane l < 16 fetches for quad half h = l / 8: scale (l % 8 < 4) or min of sample l % 4
   const int sm_h = (lane >> 3) & 1, sm_j = lane & 3;
   const TS* sm_base = (lane & 4) ? mn : scale;
+  int ka_next = 0, kb_next = 0;              // first sample of the step the next prefetch loads
 
-  auto prefetch = [&]() {
-    const bool avalid = ovalid && k_next + kqa * 4 < M;   // M % 4 == 0: a quad is inside or outside as a whole
+  auto prefetch_a = [&]() {
+    const bool avalid = ovalid && ka_next + kqa * 4 < M;   // M % 4 == 0: a quad is inside or outside as a whole
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       ra[r] = (u32x4){0u, 0u, 0u, 0u};
-      if (avalid && !(GW_ABL & 16)) ra[r] = load16(pa + (int64_t)r * O);
+      if (avalid) ra[r] = load16(pa + (int64_t)r * O);
     }
+    pa += a_step;
+    ka_next += BK;
+  };
+  auto prefetch_b = [&]() {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       rb[h] = 0u;
-      if (k_next + (wave + 8 * h) * 4 < M && !(GW_ABL & 32))   // wave-uniform
+      if (kb_next + (wave + 8 * h) * 4 < M)   // wave-uniform
         rb[h] = *reinterpret_cast<const uint32_t*>(pb + h * b_half);
     }
     rsm = 0u;
-    if (lane < 16 && k_next + (wave + 8 * sm_h) * 4 < M && !(GW_ABL & 128))
+    if (lane < 16 && kb_next + (wave + 8 * sm_h) * 4 < M)
       rsm = RawScalar<TS>::load(sm_base, si + sm_h * s_half + (int64_t)sm_j * G);
-    pa += a_step;
     pb += b_step;
     si += s_step;
-    k_next += BK;
-#ifdef GW_SKEW
-    if (k_next >= M) {   // wrap around (experiment; assumes M % BK == 0)
-      pa -= (int64_t)M * O;
-      pb -= (int64_t)(M / 4) * G * 256;
-      si -= (int64_t)M * G;
-      k_next -= M;
-    }
-#endif
+    kb_next += BK;
   };
 
-  // `kfirst` = first sample of the step being staged (rows past M dequantise to 0; their grad_out
-  // rows were loaded as 0)
-  auto stage = [&](int buf, int kfirst) {
+  // 4 (k) x 8 (o) -> 8 (o) x 4 (k): word p of ra[r] holds o = 2p (low half) and 2p + 1 (high half)
+  auto stage_a = [&](int buf) {
     uint16_t* sA = tileA(buf);
-    uint16_t* sB = tileB(buf);
-    // 4 (k) x 8 (o) -> 8 (o) x 4 (k): word p of ra[r] holds o = 2p (low half) and 2p + 1 (high half)
 #pragma unroll
     for (int p2 = 0; p2 < 4; ++p2) {
       const uint32_t w0 = ra[0][p2], w1 = ra[1][p2], w2 = ra[2][p2], w3 = ra[3][p2];
       const u32x2 even = {__builtin_amdgcn_perm(w1, w0, 0x05040100u), __builtin_amdgcn_perm(w3, w2, 0x05040100u)};
       const u32x2 odd = {__builtin_amdgcn_perm(w1, w0, 0x07060302u), __builtin_amdgcn_perm(w3, w2, 0x07060302u)};
-      if (!(GW_ABL & 4)) {
       *reinterpret_cast<u32x2*>(&sA[((2 * p2) * 32 + ao) * kPitch + kqa * 4]) = even;
       *reinterpret_cast<u32x2*>(&sA[((2 * p2 + 1) * 32 + ao) * kPitch + kqa * 4]) = odd;
-      }
+    }
+  };
+  // quad half h of the step whose first sample is kfirst (rows past M dequantise to 0; their
+  // grad_out rows were loaded as 0)
+  auto stage_b = [&](int buf, int kfirst, int h) {
+    uint16_t* sB = tileB(buf);
+    const bool bvalid = kfirst + (wave + 8 * h) * 4 < M;
+    float inv[4], m4[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t sc_raw = (uint32_t)__builtin_amdgcn_readlane((int)rsm, h * 8 + j);
+      const uint32_t mn_raw = (uint32_t)__builtin_amdgcn_readlane((int)rsm, h * 8 + 4 + j);
+      inv[j] = bvalid ? __builtin_amdgcn_rcpf(RawScalar<TS>::widen(sc_raw)) : 0.0f;
+      m4[j] = bvalid ? RawScalar<TS>::widen(mn_raw) : 0.0f;
     }
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const bool bvalid = kfirst + (wave + 8 * h) * 4 < M;
-      float inv[4], m4[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint32_t sc_raw = (uint32_t)__builtin_amdgcn_readlane((int)rsm, h * 8 + j);
-        const uint32_t mn_raw = (uint32_t)__builtin_amdgcn_readlane((int)rsm, h * 8 + 4 + j);
-        inv[j] = bvalid ? __builtin_amdgcn_rcpf(RawScalar<TS>::widen(sc_raw)) : 0.0f;
-        m4[j] = bvalid ? RawScalar<TS>::widen(mn_raw) : 0.0f;
-      }
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const uint32_t by = rb[h] >> (8 * e);
-        const float x0 = fmaf((float)(by & 3u), inv[0], m4[0]);
-        const float x1 = fmaf((float)((by >> 2) & 3u), inv[1], m4[1]);
-        const float x2 = fmaf((float)((by >> 4) & 3u), inv[2], m4[2]);
-        const float x3 = fmaf((float)((by >> 6) & 3u), inv[3], m4[3]);
-        if (!(GW_ABL & 8))
-        *reinterpret_cast<u32x2*>(&sB[(e * 64 + fi) * kPitch + (wave + 8 * h) * 4]) =
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t by = rb[h] >> (8 * e);
+      const float x0 = fmaf((float)(by & 3u), inv[0], m4[0]);
+      const float x1 = fmaf((float)((by >> 2) & 3u), inv[1], m4[1]);
+      const float x2 = fmaf((float)((by >> 4) & 3u), inv[2], m4[2]);
+      const float x3 = fmaf((float)((by >> 6) & 3u), inv[3], m4[3]);
+      *reinterpret_cast<u32x2*>(&sB[(e * 64 + fi) * kPitch + (wave + 8 * h) * 4]) =
             (u32x2){Mma<TG>::pack2(x0, x1), Mma<TG>::pack2(x2, x3)};
-      }
     }
   };
 
-  auto multiply = [&](int buf) {
+  u32x4 fa[2], fb[4];
+  auto fragments = [&](int buf, int kb) {
     const uint16_t* sA = tileA(buf) + ((2 * wr) * 32 + (lane & 31)) * kPitch + (lane >> 5) * 8;
     const uint16_t* sB = tileB(buf) + (wn * 32 + (lane & 31)) * kPitch + (lane >> 5) * 8;
 #pragma unroll
-    for (int kb = 0; kb < ((GW_ABL & 2) ? 0 : BK / 16); ++kb) {
-      u32x4 fa[2], fb[4];
+    for (int a = 0; a < 2; ++a) fa[a] = *reinterpret_cast<const u32x4*>(sA + a * 32 * kPitch + kb * 16);
 #pragma unroll
-      for (int a = 0; a < 2; ++a) fa[a] = *reinterpret_cast<const u32x4*>(sA + a * 32 * kPitch + kb * 16);
+    for (int e = 0; e < 4; ++e) fb[e] = *reinterpret_cast<const u32x4*>(sB + e * 64 * kPitch + kb * 16);
+  };
+  auto mfmas = [&]() {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) fb[e] = *reinterpret_cast<const u32x4*>(sB + e * 64 * kPitch + kb * 16);
+    for (int e = 0; e < 4; ++e)
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-#pragma unroll
-        for (int a = 0; a < 2; ++a) {
-          if (GW_ABL & 1) acc[a][e][0] += as_float(fa[a][0] ^ fb[e][1]);
-          else acc[a][e] = Mma<TG>::mfma(fa[a], fb[e], acc[a][e]);
-        }
-    }
+      for (int a = 0; a < 2; ++a) {
+        acc[a][e] = Mma<TG>::mfma(fa[a], fb[e], acc[a][e]);
+      }
   };
 
+  // One k-step: multiply step t out of LDS buffer PAR while the tile of step t+1 is written into
+  // the other buffer - its last readers passed the barrier at the end of step t-1 - and the loads
+  // of step t+2 are issued.  The staging work is cut into three pieces placed between the four
+  // MFMA groups; each piece's registers are reloaded right after it.
   const int steps = (M + BK - 1) / BK;
-#ifdef GW_SKEW
-  {
-    const int start = (int)(((int64_t)(tile % tiles_n) * GW_SKEW) % steps);
-    pa += start * a_step;
-    pb += start * b_step;
-    si += start * s_step;
-    k_next = start * BK;
+  prefetch_a();
+  prefetch_b();
+  if (steps > 0) {
+    stage_a(0);
+    stage_b(0, 0, 0);
+    stage_b(0, 0, 1);
   }
-#endif
-  prefetch();
-  if (steps > 0) stage(0, 0);
   __syncthreads();
-  if (steps > 1) prefetch();
+  if (steps > 1) {
+    prefetch_a();
+    prefetch_b();
+  }
 
   for (int t = 0; t < steps; ++t) {
     const int cur = t & 1;
     // write the tile of step t+1 into the other buffer (its last readers passed the barrier at
     // the end of step t-1), then get the loads of step t+2 in flight, then multiply step t
-#ifdef GW_SKEW
-    if (t + 1 < steps) stage(cur ^ 1, 0);
-#else
-    if (t + 1 < steps) stage(cur ^ 1, (t + 1) * BK);
-#endif
-    if (t + 2 < steps) prefetch();
-    multiply(cur);
+    if (t + 1 < steps) {
+      stage_a(cur ^ 1);
+      stage_b(cur ^ 1, (t + 1) * BK, 0);
+      stage_b(cur ^ 1, (t + 1) * BK, 1);
+    }
+    if (t + 2 < steps) {
+      prefetch_a();
+      prefetch_b();
+    }
+#pragma unroll
+    for (int kb = 0; kb < BK / 16; ++kb) {
+      fragments(cur, kb);
+      mfmas();
+    }
     __syncthreads();
   }
 
