@@ -19,14 +19,14 @@
 //     thread loads 4 consecutive k-rows x 8 o's (16-byte vectors, a wave covers whole rows of the
 //     tile), transposes them in registers with 16 byte-permutes and writes 8 rows of 4 k's;
 //   * the packed bytes already hold 4 consecutive k per feature: a thread unpacks 2 x (4 features
-//     x 4 samples) from two 32-bit loads and writes them k-contiguous.  The samples of a thread are
-//     the same for its whole wave: 16 lanes fetch the wave's 8 scales and 8 minima with one load
-//     and v_readlane hands them out (scalar loads of one value per cache line were 40% of the
-//     kernel's time).
+//     x 4 samples) from two 32-bit loads and writes them k-contiguous.  A wave works on 8
+//     consecutive samples: 16 lanes fetch their 8 scales and 8 minima with one load and v_readlane
+//     hands them out (scalar loads of one value per cache line were 40% of the kernel's time).
 //   Both LDS tiles are [row][k] with a 144-byte pitch, every MFMA fragment is one 16-byte LDS read.
 //   Rows are stored permuted - tile row o at LDS row (o % 8) * 32 + o / 8, tile column i at LDS row
-//   (i % 4) * 64 + i / 4 - which makes the lanes of a staging write hit consecutive LDS rows (no
-//   bank conflicts) and lets the epilogue store 4 consecutive columns per lane.
+//   (i % 4) * 64 + i / 4 - which makes lane pairs of a staging write fill 16 contiguous bytes of
+//   consecutive LDS rows (no bank conflicts) and lets the epilogue store 4 consecutive columns
+//   per lane.
 // Global loads run two steps ahead of the MFMAs (two register sets), LDS writes one step ahead.
 #include "device_utils.h"
 
@@ -120,18 +120,22 @@ __global__ __launch_bounds__(kThreads, 1) void linear_gw_q2_kernel(
   const int g = tile % tiles_n;              // the block's columns are quantisation group g
   const int i0 = g * 256;
 
-  // A staging: thread -> k rows 4 * kqa .. + 3 of the step, o offset ao * 8 (a wave: 2 quads x whole rows)
-  // B staging: thread -> features 4 * fi .. + 3, sample quads `wave` and `wave + 8` of the step
-  const int ao = tid & 31, kqa = tid >> 5;
-  const int fi = lane;
+  // A wave stages the sample quads 2 * wave and 2 * wave + 1 (8 consecutive samples) of a step.
+  // Neighbouring lanes take the two quads of the same row, so that the 32 lanes served by one LDS
+  // cycle write 16 rows x 16 contiguous bytes: no bank conflicts with the 144-byte pitch.
+  // A staging: thread -> k rows 4 * quad .. + 3, o offset ao * 8 (a wave: 2 quads x whole rows)
+  // B staging: thread -> the same quad, features 4 * fl .. + 3 and 128 + 4 * fl .. + 3
+  const int par = lane & 1;
+  const int quad = 2 * wave + par;
+  const int ao = lane >> 1, fl = lane >> 1;
   const bool ovalid = o0 + ao * 8 < O;       // O % 8 == 0: a vector is inside or outside as a whole
   // running pointers / indices, advanced by one k-step per prefetch
-  const TG* pa = gout + (int64_t)(kqa * 4) * O + o0 + ao * 8;
-  const uint8_t* pb = packed + ((int64_t)wave * G + g) * 256 + fi * 4;
-  int64_t si = (int64_t)(wave * 4) * G + g;  // index of the wave's first sample in scale / min
+  const TG* pa = gout + (int64_t)(quad * 4) * O + o0 + ao * 8;
+  const uint8_t* pb = packed + ((int64_t)quad * G + g) * 256 + fl * 4;
+  int64_t si = (int64_t)(wave * 8) * G + g;  // index of the wave's first sample in scale / min
   const int64_t a_step = (int64_t)BK * O;
-  const int64_t b_step = (int64_t)(BK / 4) * G * 256, b_half = (int64_t)8 * G * 256;
-  const int64_t s_step = (int64_t)BK * G, s_half = (int64_t)32 * G;
+  const int64_t b_step = (int64_t)(BK / 4) * G * 256;
+  const int64_t s_step = (int64_t)BK * G;
 
   f32x16 acc[2][4];
 #pragma unroll
@@ -148,13 +152,13 @@ __global__ __launch_bounds__(kThreads, 1) void linear_gw_q2_kernel(
   u32x4 ra[4];
   uint32_t rb[2];
   uint32_t rsm = 0u;                         // lanes 0..15: scale / min of the wave's 8 samples
-  // lane l < 16 fetches for quad half h = l / 8: scale (l % 8 < 4) or min of sample l % 4
+  // lane l < 16 fetches for quad 2 * wave + l / 8: scale (l % 8 < 4) or min of its sample l % 4
   const int sm_h = (lane >> 3) & 1, sm_j = lane & 3;
   const TS* sm_base = (lane & 4) ? mn : scale;
   int ka_next = 0, kb_next = 0;              // first sample of the step the next prefetch loads
 
   auto prefetch_a = [&]() {
-    const bool avalid = ovalid && ka_next + kqa * 4 < M;   // M % 4 == 0: a quad is inside or outside as a whole
+    const bool avalid = ovalid && ka_next + quad * 4 < M;   // M % 4 == 0: a quad is inside or outside as a whole
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       ra[r] = (u32x4){0u, 0u, 0u, 0u};
@@ -164,15 +168,14 @@ __global__ __launch_bounds__(kThreads, 1) void linear_gw_q2_kernel(
     ka_next += BK;
   };
   auto prefetch_b = [&]() {
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      rb[h] = 0u;
-      if (kb_next + (wave + 8 * h) * 4 < M)   // wave-uniform
-        rb[h] = *reinterpret_cast<const uint32_t*>(pb + h * b_half);
+    rb[0] = rb[1] = 0u;
+    if (kb_next + quad * 4 < M) {
+      rb[0] = *reinterpret_cast<const uint32_t*>(pb);
+      rb[1] = *reinterpret_cast<const uint32_t*>(pb + 128);
     }
     rsm = 0u;
-    if (lane < 16 && kb_next + (wave + 8 * sm_h) * 4 < M)
-      rsm = RawScalar<TS>::load(sm_base, si + sm_h * s_half + (int64_t)sm_j * G);
+    if (lane < 16 && kb_next + (2 * wave + sm_h) * 4 < M)
+      rsm = RawScalar<TS>::load(sm_base, si + (int64_t)(4 * sm_h + sm_j) * G);
     pb += b_step;
     si += s_step;
     kb_next += BK;
@@ -186,89 +189,86 @@ __global__ __launch_bounds__(kThreads, 1) void linear_gw_q2_kernel(
       const uint32_t w0 = ra[0][p2], w1 = ra[1][p2], w2 = ra[2][p2], w3 = ra[3][p2];
       const u32x2 even = {__builtin_amdgcn_perm(w1, w0, 0x05040100u), __builtin_amdgcn_perm(w3, w2, 0x05040100u)};
       const u32x2 odd = {__builtin_amdgcn_perm(w1, w0, 0x07060302u), __builtin_amdgcn_perm(w3, w2, 0x07060302u)};
-      *reinterpret_cast<u32x2*>(&sA[((2 * p2) * 32 + ao) * kPitch + kqa * 4]) = even;
-      *reinterpret_cast<u32x2*>(&sA[((2 * p2 + 1) * 32 + ao) * kPitch + kqa * 4]) = odd;
+      *reinterpret_cast<u32x2*>(&sA[((2 * p2) * 32 + ao) * kPitch + quad * 4]) = even;
+      *reinterpret_cast<u32x2*>(&sA[((2 * p2 + 1) * 32 + ao) * kPitch + quad * 4]) = odd;
     }
   };
-  // quad half h of the step whose first sample is kfirst (rows past M dequantise to 0; their
-  // grad_out rows were loaded as 0)
-  auto stage_b = [&](int buf, int kfirst, int h) {
+  // the step whose first sample is kfirst (rows past M dequantise to 0; their grad_out rows were
+  // loaded as 0)
+  auto stage_b = [&](int buf, int kfirst) {
     uint16_t* sB = tileB(buf);
-    const bool bvalid = kfirst + (wave + 8 * h) * 4 < M;
+    const bool bvalid = kfirst + quad * 4 < M;
     float inv[4], m4[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint32_t sc_raw = (uint32_t)__builtin_amdgcn_readlane((int)rsm, h * 8 + j);
-      const uint32_t mn_raw = (uint32_t)__builtin_amdgcn_readlane((int)rsm, h * 8 + 4 + j);
-      inv[j] = bvalid ? __builtin_amdgcn_rcpf(RawScalar<TS>::widen(sc_raw)) : 0.0f;
-      m4[j] = bvalid ? RawScalar<TS>::widen(mn_raw) : 0.0f;
+      const uint32_t sc0 = (uint32_t)__builtin_amdgcn_readlane((int)rsm, j);
+      const uint32_t mn0 = (uint32_t)__builtin_amdgcn_readlane((int)rsm, 4 + j);
+      const uint32_t sc1 = (uint32_t)__builtin_amdgcn_readlane((int)rsm, 8 + j);
+      const uint32_t mn1 = (uint32_t)__builtin_amdgcn_readlane((int)rsm, 12 + j);
+      inv[j] = bvalid ? __builtin_amdgcn_rcpf(RawScalar<TS>::widen(par ? sc1 : sc0)) : 0.0f;
+      m4[j] = bvalid ? RawScalar<TS>::widen(par ? mn1 : mn0) : 0.0f;
     }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const uint32_t by = rb[h] >> (8 * e);
-      const float x0 = fmaf((float)(by & 3u), inv[0], m4[0]);
-      const float x1 = fmaf((float)((by >> 2) & 3u), inv[1], m4[1]);
-      const float x2 = fmaf((float)((by >> 4) & 3u), inv[2], m4[2]);
-      const float x3 = fmaf((float)((by >> 6) & 3u), inv[3], m4[3]);
-      *reinterpret_cast<u32x2*>(&sB[(e * 64 + fi) * kPitch + (wave + 8 * h) * 4]) =
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t by = rb[h] >> (8 * e);
+        const float x0 = fmaf((float)(by & 3u), inv[0], m4[0]);
+        const float x1 = fmaf((float)((by >> 2) & 3u), inv[1], m4[1]);
+        const float x2 = fmaf((float)((by >> 4) & 3u), inv[2], m4[2]);
+        const float x3 = fmaf((float)((by >> 6) & 3u), inv[3], m4[3]);
+        *reinterpret_cast<u32x2*>(&sB[(e * 64 + 32 * h + fl) * kPitch + quad * 4]) =
             (u32x2){Mma<TG>::pack2(x0, x1), Mma<TG>::pack2(x2, x3)};
+      }
     }
   };
 
-  u32x4 fa[2], fb[4];
+  // Fragments are double-buffered in registers: those of k-block kb+1 are requested before the
+  // MFMAs of k-block kb are issued, so the matrix pipe does not wait for LDS inside a step.
+  u32x4 fa[2][2], fb[2][4];
   auto fragments = [&](int buf, int kb) {
     const uint16_t* sA = tileA(buf) + ((2 * wr) * 32 + (lane & 31)) * kPitch + (lane >> 5) * 8;
     const uint16_t* sB = tileB(buf) + (wn * 32 + (lane & 31)) * kPitch + (lane >> 5) * 8;
 #pragma unroll
-    for (int a = 0; a < 2; ++a) fa[a] = *reinterpret_cast<const u32x4*>(sA + a * 32 * kPitch + kb * 16);
+    for (int a = 0; a < 2; ++a) fa[kb & 1][a] = *reinterpret_cast<const u32x4*>(sA + a * 32 * kPitch + kb * 16);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) fb[e] = *reinterpret_cast<const u32x4*>(sB + e * 64 * kPitch + kb * 16);
+    for (int e = 0; e < 4; ++e) fb[kb & 1][e] = *reinterpret_cast<const u32x4*>(sB + e * 64 * kPitch + kb * 16);
   };
-  auto mfmas = [&]() {
+  auto mfmas = [&](int kb) {
 #pragma unroll
     for (int e = 0; e < 4; ++e)
 #pragma unroll
-      for (int a = 0; a < 2; ++a) {
-        acc[a][e] = Mma<TG>::mfma(fa[a], fb[e], acc[a][e]);
-      }
+      for (int a = 0; a < 2; ++a) acc[a][e] = Mma<TG>::mfma(fa[kb & 1][a], fb[kb & 1][e], acc[a][e]);
+  };
+  auto multiply_step = [&](int buf) {
+    fragments(buf, 0);
+#pragma unroll
+    for (int kb = 0; kb < BK / 16; ++kb) {
+      // keep the compiler from sinking the reads of kb+1 below the MFMAs of kb
+      __builtin_amdgcn_sched_barrier(0);
+      if (kb + 1 < BK / 16) fragments(buf, kb + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      mfmas(kb);
+    }
+  };
+  auto stage_step = [&](int j) {             // write tile j, then get the loads of tile j+1 in flight
+    stage_a(j & 1);
+    stage_b(j & 1, j * BK);
+    prefetch_a();
+    prefetch_b();
   };
 
-  // One k-step: multiply step t out of LDS buffer PAR while the tile of step t+1 is written into
-  // the other buffer - its last readers passed the barrier at the end of step t-1 - and the loads
-  // of step t+2 are issued.  The staging work is cut into three pieces placed between the four
-  // MFMA groups; each piece's registers are reloaded right after it.
+  // Step t is multiplied out of LDS buffer t % 2 while the tile of step t+1 is written into the
+  // other buffer (its last readers passed the barrier at the end of step t-1) and the loads of
+  // step t+2 are issued: one barrier per step.
   const int steps = (M + BK - 1) / BK;
   prefetch_a();
   prefetch_b();
-  if (steps > 0) {
-    stage_a(0);
-    stage_b(0, 0, 0);
-    stage_b(0, 0, 1);
-  }
+  if (steps > 0) stage_step(0);
   __syncthreads();
-  if (steps > 1) {
-    prefetch_a();
-    prefetch_b();
-  }
-
   for (int t = 0; t < steps; ++t) {
-    const int cur = t & 1;
-    // write the tile of step t+1 into the other buffer (its last readers passed the barrier at
-    // the end of step t-1), then get the loads of step t+2 in flight, then multiply step t
-    if (t + 1 < steps) {
-      stage_a(cur ^ 1);
-      stage_b(cur ^ 1, (t + 1) * BK, 0);
-      stage_b(cur ^ 1, (t + 1) * BK, 1);
-    }
-    if (t + 2 < steps) {
-      prefetch_a();
-      prefetch_b();
-    }
-#pragma unroll
-    for (int kb = 0; kb < BK / 16; ++kb) {
-      fragments(cur, kb);
-      mfmas();
-    }
+    if (t + 1 < steps) stage_step(t + 1);
+    multiply_step(t & 1);
     __syncthreads();
   }
 
