@@ -30,9 +30,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 # measured yet.
 MEASURED_TRAFFIC_BYTES = {
     # profiles/config2_minimax_pack_unpack_mixed_f32.txt (fetch factor 2.0, write factor 1.0)
-    "minimax": 828817676,
-    "pack_mixed": 883218157,
-    "unpack_mixed": 880260916,
+    "minimax": 828540312,
+    "pack_mixed": 889626116,
+    "unpack_mixed": 886690445,
 }
 
 

@@ -138,12 +138,13 @@ int actnn_calc_precision(int32_t* b, const float* C, const int32_t* w, int64_t N
 /* ---------------------------------------------------------------------------------
  * Fused QLinear weight gradient: grad_w[O, I] = grad_out[M, O]^T @ dequant(x)[M, I] where x
  * is held as the pack_single 2-bit stream (4 consecutive rows m per byte) with
- * scale/min[M, I/256, 1].  The 2-bit tile is unpacked and dequantised to bf16 inside the
- * LDS loader of a bf16 MFMA GEMM (fp32 accumulation); the full-precision input is never
- * written to memory.  Replaces dequantize_activation + grad_output.t().mm(input) in
+ * scale/min[M, I/256, 1].  The 2-bit tile is unpacked and dequantised to the 16-bit format of
+ * grad_out inside the LDS loader of an MFMA GEMM (fp32 accumulation); the full-precision input
+ * is never written to memory.  Replaces dequantize_activation + grad_output.t().mm(input) in
  * linear.backward, actnn/actnn/ops.py:407-421.
  * grad_out dtype: f16 or bf16; scale/min dtype = sm_dtype; grad_w dtype = out_dtype
- * (f32, f16 or bf16).  M % 4 == 0, I % 256 == 0.
+ * (f32, f16 or bf16).  M % 4 == 0, I % 256 == 0, O % 8 == 0; grad_out and grad_w 16-byte,
+ * packed, scale and min 4-byte aligned.
  * ------------------------------------------------------------------------------- */
 int actnn_linear_grad_weight_q2(const void* grad_out, const int8_t* packed, const void* scale,
                                 const void* mn, void* grad_w, int64_t M, int64_t O, int64_t I,
