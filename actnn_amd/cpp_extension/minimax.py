@@ -17,3 +17,27 @@ def minimax(data):
         check(g.lib().actnn_minimax(data.data_ptr(), mn.data_ptr(), mx.data_ptr(), M, D,
                                     g.DTYPE_CODE[data.dtype], g.stream_ptr(data.device)), "minimax")
     return mn, mx
+
+
+def range_sqr(mn, mx, N, factor=1.0, mult=None):
+    """fp32 [N]: factor * mult * sum over the groups of sample n of (mx - mn)^2, in one kernel
+    (reference: the tensor expression of qscheme.py:80-82).  mn / mx: the [N * G] outputs of
+    ``minimax``; mult: None, a 0-dim fp32 device tensor or an fp32 device tensor of N values."""
+    g.check_float(mn, "min")
+    if mx.dtype != mn.dtype or mx.shape != mn.shape or mn.numel() % max(N, 1) != 0:
+        raise RuntimeError("range_sqr: min and max do not match")
+    mn = mn.contiguous()
+    mx = mx.contiguous()
+    G = mn.numel() // N if N else 0
+    out = torch.empty(N, dtype=torch.float32, device=mn.device)
+    mult_ptr, per_sample = None, 0
+    if mult is not None:
+        if mult.dtype != torch.float32 or mult.device != mn.device or mult.numel() not in (1, N):
+            raise RuntimeError("range_sqr: mult must be fp32 on the same device with 1 or N values")
+        mult = mult.contiguous()
+        mult_ptr, per_sample = mult.data_ptr(), int(mult.numel() == N and N != 1)
+    with torch.cuda.device(mn.device):
+        check(g.lib().actnn_range_sqr(mn.data_ptr(), mx.data_ptr(), out.data_ptr(), N, G, float(factor),
+                                      mult_ptr, per_sample, g.DTYPE_CODE[mn.dtype], g.stream_ptr(mn.device)),
+              "range_sqr")
+    return out

@@ -157,8 +157,65 @@ int launch_minimax(const void* data, void* mn, void* mx, int64_t M, int64_t D, h
   ACTNN_RETURN_LAUNCH_STATUS();
 }
 
+// Per-sample sensitivity of the bit allocation: out[n] = factor * mult * sum_g (mx[n,g] - mn[n,g])^2
+// (the difference rounded to T, as the tensor subtraction of qscheme.py:80 rounds it; the sum is
+// kept in fp32 in a fixed order).  mult: nothing, one device scalar or one value per sample.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void range_sqr_kernel(const T* __restrict__ mn,
+                                                             const T* __restrict__ mx,
+                                                             float* __restrict__ out, int64_t G,
+                                                             float factor, const float* __restrict__ mult,
+                                                             int mult_stride) {
+  __shared__ float s_part[kThreads];
+  const int64_t n = blockIdx.x;
+  float acc = 0.0f;
+  for (int64_t g = threadIdx.x; g < G; g += kThreads) {
+    const float d = Conv<T>::round(Conv<T>::load(mx, n * G + g) - Conv<T>::load(mn, n * G + g));
+    acc = fmaf(d, d, acc);
+  }
+  s_part[threadIdx.x] = acc;
+  __syncthreads();
+  for (int w = kThreads / 2; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) s_part[threadIdx.x] += s_part[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    float v = s_part[0] * factor;
+    if (mult) v *= mult[n * mult_stride];
+    out[n] = v;
+  }
+}
+
 }  // namespace
 }  // namespace actnn
+
+extern "C" int actnn_range_sqr(const void* mn, const void* mx, float* out, int64_t N, int64_t G,
+                               float factor, const float* mult, int mult_per_sample, int dtype,
+                               void* stream) {
+  using namespace actnn;
+  if (N < 0 || G < 0 || N > 0x7fffffffLL) return ACTNN_EINVAL;
+  if (N == 0) return ACTNN_OK;
+  if (!out || (G > 0 && (!mn || !mx))) return ACTNN_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)N), blk(kThreads);
+  const int stride = mult_per_sample ? 1 : 0;
+  switch (dtype) {
+    case ACTNN_F32:
+      range_sqr_kernel<float><<<grid, blk, 0, s>>>(static_cast<const float*>(mn), static_cast<const float*>(mx),
+                                                   out, G, factor, mult, stride);
+      break;
+    case ACTNN_F16:
+      range_sqr_kernel<__half><<<grid, blk, 0, s>>>(static_cast<const __half*>(mn), static_cast<const __half*>(mx),
+                                                    out, G, factor, mult, stride);
+      break;
+    case ACTNN_BF16:
+      range_sqr_kernel<bf16_t><<<grid, blk, 0, s>>>(static_cast<const bf16_t*>(mn), static_cast<const bf16_t*>(mx),
+                                                    out, G, factor, mult, stride);
+      break;
+    default: return ACTNN_EDTYPE;
+  }
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
 
 extern "C" int actnn_minimax(const void* data, void* mn, void* mx, int64_t M, int64_t D, int dtype,
                              void* stream) {

@@ -36,9 +36,9 @@ def group_min_max(input):
     return rows.view(N, -1, gs), mn, mx, num_pixels
 
 
-def range_sqr(mn, mx, N, num_pixels):
-    """G * ||R_n||^2 / I  (qscheme.py:80)."""
-    return torch.norm((mx - mn).view(N, -1), dim=1).float().square() * (config.group_size / num_pixels)
+def range_sqr(mn, mx, N, num_pixels, factor=1.0, mult=None):
+    """fp32 [N]: factor * mult * G * ||R_n||^2 / I  (qscheme.py:80-82), one kernel per call."""
+    return ext_minimax.range_sqr(mn, mx, N, factor * config.group_size / num_pixels, mult)
 
 
 class PendingBits:
@@ -52,7 +52,7 @@ class PendingBits:
 
     def __init__(self, C_dev):
         self.host = torch.empty(C_dev.shape, dtype=torch.float32, pin_memory=True)
-        self.host.copy_(C_dev.to(torch.float32), non_blocking=True)
+        self.host.copy_(C_dev if C_dev.dtype == torch.float32 else C_dev.to(torch.float32), non_blocking=True)
         self.event = torch.cuda.Event()
         self.event.record()
 
@@ -118,9 +118,10 @@ class QScheme(object):
             self.scales = sq.mean()
 
     # -- forward-time allocation ------------------------------------------------------------
-    def sensitivity(self, rsq, device):
-        grad_sum = self.get_scale().to(device)
-        return self.num_locations / 4 / self.depthwise_groups * rsq * grad_sum
+    def sensitivity(self, mn, mx, N, num_pixels):
+        """C_n = num_locations / 4 / depthwise_groups * Range_sqr_n * grad_sum_n  (qscheme.py:80-82)."""
+        grad_sum = self.get_scale().to(device=mn.device, dtype=torch.float32)
+        return range_sqr(mn, mx, N, num_pixels, self.num_locations / 4 / self.depthwise_groups, grad_sum)
 
     def compute_quantization_bits(self, input):
         """-> (groups [N,G,gs], bits on device, mn [N,G,1], mx [N,G,1])  (qscheme.py:57-94)."""
@@ -131,8 +132,7 @@ class QScheme(object):
         QScheme.prev_layer = self
         N = input.shape[0]
         groups, mn, mx, num_pixels = group_min_max(input)
-        rsq = range_sqr(mn, mx, N, num_pixels)
-        pending = PendingBits(self.sensitivity(rsq, input.device))
+        pending = PendingBits(self.sensitivity(mn, mx, N, num_pixels))
         return groups, mn, mx, pending, input.numel() // N
 
     def finish_quantization_bits(self, started):

@@ -46,6 +46,18 @@ const char* actnn_version(void);
 int actnn_minimax(const void* data, void* mn, void* mx, int64_t M, int64_t D, int dtype,
                   void* stream);
 
+/* ---------------------------------------------------------------------------------
+ * Per-sample sensitivity of the bit allocation from the group ranges:
+ *   out[n] = factor * mult * sum_g (mx[n, g] - mn[n, g])^2        (out: fp32[N], device)
+ * mult: NULL, one fp32 device scalar (mult_per_sample == 0) or fp32[N] (mult_per_sample != 0).
+ * Replaces the chain of tensor ops behind Range_sqr and C in QScheme.compute_quantization_bits,
+ * actnn/actnn/qscheme.py:80-82 (norm over the groups of a sample, squared, scaled by
+ * group_size / num_pixels, by num_locations / 4 / depthwise_groups and by the gradient scale);
+ * the squared norm is accumulated directly in fp32.
+ * ------------------------------------------------------------------------------- */
+int actnn_range_sqr(const void* mn, const void* mx, float* out, int64_t N, int64_t G, float factor,
+                    const float* mult, int mult_per_sample, int dtype, void* stream);
+
 /* Exclusive prefix sum of the per-sample bit widths: prefix[0] = 0,
  * prefix[n] = bits[0] + ... + bits[n-1], prefix has N + 1 entries.
  * Replaces the torch::cumsum calls at quantization_cuda_kernel.cu:97 and :182. */

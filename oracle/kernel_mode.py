@@ -85,3 +85,19 @@ def code_variance(data, mn, scale, bits):
     ActNN's bound R^2/(4 B^2) per element is its maximum, qscheme.py:84)."""
     f = (rng_fixed_point(data, mn, scale, bits) & np.uint32(0xFFFF)).astype(np.float64) / 65536.0
     return f * (1.0 - f)
+
+
+def range_sqr(mn, mx, factor=1.0, mult=None):
+    """Per-sample sensitivity term: factor * mult * sum_g (mx - mn)^2 for mn, mx of shape [N, G]
+    (numpy arrays of the activation dtype's values).  Follows actnn/actnn/qscheme.py:80-82
+    (``torch.norm((mx - mn).view(N, -1), dim=1).float().square() * (group_size / num_pixels)``,
+    then ``num_locations / 4 / depthwise_groups * Range_sqr * grad_sum``): the subtraction rounds
+    to the tensor dtype; the square root and re-squaring of the reference are the identity up to
+    rounding and are not repeated, the sum is taken in float64 here.  Pinned by the closed form for
+    constant ranges (tests/test_oracle_simulate.py) and by torch's own expression on random data."""
+    import numpy as np
+    d = (np.asarray(mx) - np.asarray(mn)).astype(np.asarray(mn).dtype)      # rounds like the tensor op
+    v = (d.astype(np.float64) ** 2).sum(axis=1) * float(factor)
+    if mult is not None:
+        v = v * np.asarray(mult, dtype=np.float64)
+    return v

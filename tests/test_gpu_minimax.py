@@ -39,3 +39,41 @@ def test_minimax_rejects_bad_arguments():
         ext_minimax.minimax(torch.zeros(4, 256, dtype=torch.int32, device=DEV))
     mn, mx = ext_minimax.minimax(torch.empty(0, 256, device=DEV))
     assert mn.numel() == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,G", [(1, 1), (3, 7), (16, 784), (5, 3136)])
+def test_range_sqr_matches_the_oracle(dtype, N, G):
+    """Fused sensitivity kernel vs the oracle (float64 sum of the dtype-rounded differences), with
+    no multiplier, a device scalar and one value per sample; fp32 summation order differs: 1e-5."""
+    import numpy as np
+    from oracle import kernel_mode
+    g = torch.Generator().manual_seed(N * 1000 + G)
+    mn = torch.randn(N * G, generator=g).to(dtype)
+    mx = (mn.float() + torch.rand(N * G, generator=g) * 4).to(dtype)
+    per = torch.rand(N, generator=g) + 0.5
+    for mult in (None, per[:1].clone().view(()), per):
+        out = ext_minimax.range_sqr(mn.to(DEV), mx.to(DEV), N, 0.37,
+                                    None if mult is None else mult.to(DEV))
+        assert out.dtype == torch.float32 and out.shape == (N,)
+        to_np = (lambda t: t.numpy()) if dtype != torch.bfloat16 else None
+        if dtype == torch.bfloat16:        # numpy has no bf16: round the difference with torch instead
+            d = (mx - mn).float().numpy().astype(np.float64).reshape(N, G)
+            exp = (d ** 2).sum(1) * 0.37
+            if mult is not None:
+                exp = exp * mult.numpy().astype(np.float64)
+        else:
+            exp = kernel_mode.range_sqr(to_np(mn).reshape(N, G), to_np(mx).reshape(N, G), 0.37,
+                                        None if mult is None else mult.numpy())
+        assert np.allclose(out.cpu().numpy(), exp, rtol=1e-5, atol=0)
+
+
+def test_range_sqr_rejects_bad_arguments():
+    mn = torch.zeros(8, device=DEV)
+    with pytest.raises(RuntimeError):
+        ext_minimax.range_sqr(mn, torch.zeros(9, device=DEV), 2)
+    with pytest.raises(RuntimeError):
+        ext_minimax.range_sqr(mn, mn, 2, 1.0, torch.ones(3, device=DEV))
+    with pytest.raises(RuntimeError):
+        ext_minimax.range_sqr(mn.int(), mn.int(), 2)
+    assert ext_minimax.range_sqr(mn[:0], mn[:0], 0).numel() == 0

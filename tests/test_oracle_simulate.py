@@ -111,3 +111,25 @@ def test_minimax_is_rowwise():
     mn, mx = simulate.minimax(x)
     assert torch.equal(mn, torch.from_numpy(x.numpy().min(axis=1)))
     assert torch.equal(mx, torch.from_numpy(x.numpy().max(axis=1)))
+
+
+def test_range_sqr_closed_form_and_torch_expression():
+    """oracle.kernel_mode.range_sqr: a constant range r over G groups gives G * r^2 * factor, and on
+    random fp32 data it agrees with the reference's tensor expression (qscheme.py:80) evaluated
+    by torch on the CPU; 16-bit inputs round the subtraction to the tensor dtype first."""
+    from oracle import kernel_mode
+    N, G = 5, 37
+    mn = np.full((N, G), -0.25, np.float32)
+    mx = np.full((N, G), 1.25, np.float32)
+    assert np.allclose(kernel_mode.range_sqr(mn, mx, 0.5), G * 1.5 ** 2 * 0.5, rtol=0, atol=1e-12)
+    rng = np.random.default_rng(0)
+    mn = rng.standard_normal((N, G)).astype(np.float32)
+    mx = mn + rng.random((N, G)).astype(np.float32) * 3
+    ref = torch.norm((torch.from_numpy(mx) - torch.from_numpy(mn)).view(N, -1), dim=1).float().square() * (256 / 49)
+    mult = rng.random(N).astype(np.float32) + 0.5
+    got = kernel_mode.range_sqr(mn, mx, 256 / 49, mult)
+    assert np.allclose(got, ref.numpy().astype(np.float64) * mult, rtol=1e-5)
+    # 16-bit inputs: the subtraction rounds to the tensor dtype (numpy float16 stands for it here)
+    mnh, mxh = mn.astype(np.float16), mx.astype(np.float16)
+    d = (torch.from_numpy(mxh) - torch.from_numpy(mnh)).float().numpy().astype(np.float64)
+    assert np.allclose(kernel_mode.range_sqr(mnh, mxh), (d ** 2).sum(1), rtol=1e-12)
