@@ -180,16 +180,16 @@ ACTNN_DEV void store8_nt(bf16_t* p, const float (&v)[8]) {
 // through ds_swizzle (LDS crossbar, no memory), so they do not take a VALU slot.
 template <int D> ACTNN_DEV uint32_t lane_xor(uint32_t x);
 template <> ACTNN_DEV uint32_t lane_xor<1>(uint32_t x) {
-  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, false);   // quad_perm [1,0,3,2]
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
 }
 template <> ACTNN_DEV uint32_t lane_xor<2>(uint32_t x) {
-  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, false);   // quad_perm [2,3,0,1]
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
 }
 template <> ACTNN_DEV uint32_t lane_xor<4>(uint32_t x) {
   return (uint32_t)__builtin_amdgcn_ds_swizzle((int)x, 0x101F);                      // xor 4
 }
 template <> ACTNN_DEV uint32_t lane_xor<8>(uint32_t x) {
-  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x128, 0xF, 0xF, false);  // row_ror:8
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, 0x128, 0xF, 0xF, true);  // row_ror:8
 }
 template <> ACTNN_DEV uint32_t lane_xor<16>(uint32_t x) {
   return (uint32_t)__builtin_amdgcn_ds_swizzle((int)x, 0x401F);                      // xor 16
