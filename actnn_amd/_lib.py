@@ -12,7 +12,7 @@ CSRC = os.path.join(_HERE, "csrc")
 # ACTNN_HIP_LIB points at another build of the same library (kernel tuning experiments)
 LIB_PATH = os.environ.get("ACTNN_HIP_LIB") or os.path.join(_HERE, "libactnn_hip.so")
 SOURCES = ["minimax.hip", "pack_mixed.hip", "pack_single.hip", "mask_ops.hip", "maxpool.hip",
-           "linear_gw.hip", "misc.hip", "calc_precision.cpp"]
+           "linear_gw.hip", "misc.hip", "calc_precision.cpp", "calc_precision_dev.hip"]
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-ffp-contract=off",                      # bit-exact quantiser: no implicit FMA
@@ -27,6 +27,7 @@ SIGNATURES = {
     "actnn_strerror": [c_i32],
     "actnn_version": [],
     "actnn_minimax": [c_vp, c_vp, c_vp, c_i64, c_i64, c_i32, c_vp],
+    "actnn_calc_precision_device": [c_vp, c_vp, c_i64, c_i32, c_i64, c_vp],
     "actnn_range_sqr": [c_vp, c_vp, c_vp, c_i64, c_i64, ctypes.c_float, c_vp, c_i32, c_i32, c_vp],
     "actnn_bits_prefix": [c_vp, c_vp, c_i64, c_vp],
     "actnn_pack_mixed": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u64, c_u64,

@@ -27,6 +27,7 @@ class QuantizationConfig:
         self.adaptive_bn_scheme = True
         self.simulate = False                          # pure-torch quantiser instead of the kernels
         self.enable_quantized_bn = True
+        self.device_allocation = True                  # per-sample widths computed on the GPU when the batch fits
         # memory management (conf.py:54-58)
         self.empty_cache_threshold = None
         self.pipeline_threshold = None

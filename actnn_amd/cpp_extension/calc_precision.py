@@ -1,6 +1,8 @@
 """``calc_precision(b, C, w, target) -> b``: greedy bit allocation on CPU tensors; ``b`` is
 modified in place and returned (reference: cpp_extension/calc_precision.cc:9-50).
-``calc_precision_dp`` of the reference has no Python caller and is not provided."""
+``calc_precision_dp`` of the reference has no Python caller and is not provided.
+``calc_precision_device`` runs the same allocation on the GPU for uniform start widths and unit
+weights (what every layer asks for at every step), so that no host round trip is needed."""
 import torch
 
 from . import _glue as g
@@ -20,3 +22,27 @@ def calc_precision(b, C, w, target):
     check(g.lib().actnn_calc_precision(b.data_ptr(), C.data_ptr(), w.data_ptr(), b.numel(),
                                        float(target)), "calc_precision")
     return b
+
+
+DEVICE_MAX_CANDIDATES = 8192
+
+
+def device_allocation_fits(N, initial_bits):
+    return 1 <= int(initial_bits) <= 8 and N * (int(initial_bits) - 1) <= DEVICE_MAX_CANDIDATES
+
+
+def calc_precision_device(C, initial_bits, target):
+    """int32 device tensor [N]: the widths ``calc_precision(ones(N) * initial_bits, C, ones(N),
+    target)`` would return, computed on the device of ``C`` (fp32 [N])."""
+    if not (isinstance(C, torch.Tensor) and C.is_cuda and C.dtype == torch.float32 and C.dim() == 1):
+        raise RuntimeError("C must be a 1-D fp32 device tensor!")
+    N = C.numel()
+    if not device_allocation_fits(N, initial_bits):
+        raise RuntimeError("calc_precision_device: N * (initial_bits - 1) must be <= %d, initial_bits in 1..8"
+                           % DEVICE_MAX_CANDIDATES)
+    C = C.contiguous()
+    bits = torch.empty(N, dtype=torch.int32, device=C.device)
+    with torch.cuda.device(C.device):
+        check(g.lib().actnn_calc_precision_device(C.data_ptr(), bits.data_ptr(), N, int(initial_bits),
+                                                  int(target), g.stream_ptr(C.device)), "calc_precision_device")
+    return bits

@@ -22,17 +22,26 @@ def attach_bits_host(bits_dev, bits_host):
     return bits_dev
 
 
+def attach_bits_total(bits_dev, total):
+    """For widths computed on the device (no host copy): remember their sum, which the caller
+    knows from the budget, so that the packed stream can be sized without a sync."""
+    bits_dev._actnn_total = int(total)
+    return bits_dev
+
+
 def _bits_info(bits):
     """(sum(bits), device exclusive prefix [N+1]) of an int32 device tensor, cached on it."""
     cached = getattr(bits, "_actnn_info", None)
     if cached is not None:
         return cached
-    host = getattr(bits, "_actnn_host", None)
-    if host is None:
-        host = bits.cpu()                              # sync, like the reference's .item() calls
-    if host.numel() and (int(host.min()) < 1 or int(host.max()) > 8):
-        raise RuntimeError("pack_mixed_precision supports 1..8 bits per sample")
-    total = int(host.sum())
+    total = getattr(bits, "_actnn_total", None)        # widths made on the device: only their sum is known
+    if total is None:
+        host = getattr(bits, "_actnn_host", None)
+        if host is None:
+            host = bits.cpu()                          # sync, like the reference's .item() calls
+        if host.numel() and (int(host.min()) < 1 or int(host.max()) > 8):
+            raise RuntimeError("pack_mixed_precision supports 1..8 bits per sample")
+        total = int(host.sum())
     N = bits.numel()
     prefix = torch.empty(N + 1, dtype=torch.int32, device=bits.device)
     with torch.cuda.device(bits.device):

@@ -3,7 +3,8 @@ sensitivity is the range term alone and the per-layer budget follows the precedi
 import torch
 
 from .conf import config
-from .qscheme import PendingBits, QScheme, greedy_bits, group_min_max, range_sqr
+from .qscheme import (PendingBits, QScheme, allocate_on_device, greedy_bits, greedy_bits_device,
+                      group_min_max, range_sqr)
 
 
 class QBNScheme(QScheme):
@@ -19,13 +20,16 @@ class QBNScheme(QScheme):
         self.prev_linear = QScheme.prev_layer
         N = input.shape[0]
         groups, mn, mx, num_pixels = group_min_max(input)
-        pending = PendingBits(range_sqr(mn, mx, N, num_pixels))            # qbnscheme.py:44-47
-        return groups, mn, mx, pending, input.numel() // N
+        C_dev = range_sqr(mn, mx, N, num_pixels)                           # qbnscheme.py:44-47
+        if allocate_on_device(N, self.initial_bits):
+            return groups, mn, mx, None, input.numel() // N, greedy_bits_device(C_dev, N, self.initial_bits, self.bits)
+        return groups, mn, mx, PendingBits(C_dev), input.numel() // N, None
 
     def finish_quantization_bits(self, started):
-        groups, mn, mx, pending, _ = started
+        groups, mn, mx, pending, _, bits_dev = started
         N = groups.shape[0]
-        bits_dev, _ = greedy_bits(pending.wait().clone(), N, self.initial_bits, self.bits, groups.device)
+        if bits_dev is None:
+            bits_dev, _ = greedy_bits(pending.wait().clone(), N, self.initial_bits, self.bits, groups.device)
         return groups, bits_dev, mn.view(N, -1, 1), mx.view(N, -1, 1)
 
     @staticmethod

@@ -11,7 +11,7 @@ import torch
 from .conf import config
 from .cpp_extension import calc_precision as ext_calc_precision
 from .cpp_extension import minimax as ext_minimax
-from .cpp_extension.quantization import attach_bits_host
+from .cpp_extension.quantization import attach_bits_host, attach_bits_total
 
 
 def group_min_max(input):
@@ -70,7 +70,48 @@ def greedy_bits(C_host, N, initial_bits, avg_bits, device):
     return attach_bits_host(b.to(device, non_blocking=True), b), b
 
 
-class QScheme(object):
+def greedy_bits_device(C_dev, N, initial_bits, avg_bits):
+    """The same widths computed on the device (no round trip): only their sum - fixed by the
+    budget - is known on the host, which is all pack / unpack need to size the stream."""
+    initial = int(initial_bits)
+    target = int(avg_bits * N)
+    bits = ext_calc_precision.calc_precision_device(C_dev, initial, target)
+    taken = min(max(N * initial - target, 0), N * (initial - 1))
+    return attach_bits_total(bits, N * initial - taken)
+
+
+def allocate_on_device(N, initial_bits):
+    return config.device_allocation and ext_calc_precision.device_allocation_fits(N, initial_bits)
+
+
+class _LazyHost:
+    """Attribute pair for values whose host copy may still be in flight: `C` (sensitivities, wanted
+    by the per-layer re-balancing at the end of the step) and `b` (widths, wanted by tests)."""
+
+    def _get_C(self):
+        pending = getattr(self, "_pending_C", None)
+        if pending is not None:
+            self._C = pending.wait().clone()
+            self._pending_C = None
+        return getattr(self, "_C", None)
+
+    def _set_C(self, value):
+        self._pending_C = None
+        self._C = value
+
+    C = property(_get_C, _set_C)
+
+    def _get_b(self):
+        b = getattr(self, "_b", None)
+        return b.cpu() if isinstance(b, torch.Tensor) and b.is_cuda else b
+
+    def _set_b(self, value):
+        self._b = value
+
+    b = property(_get_b, _set_b)
+
+
+class QScheme(_LazyHost):
     num_samples = 1        # dataset size, only used with config.use_gradient
     num_layers = 0
     batch = None           # dataset indices of the current batch (config.use_gradient)
@@ -88,6 +129,7 @@ class QScheme(object):
             self.scales = torch.tensor([0.0])
         QScheme.layers.append(self)
         self.C = None
+        self.b = None
         self.dim = None
         self.num_locations = num_locations          # kernel positions per output
         self.depthwise_groups = depthwise_groups
@@ -132,18 +174,28 @@ class QScheme(object):
         QScheme.prev_layer = self
         N = input.shape[0]
         groups, mn, mx, num_pixels = group_min_max(input)
-        pending = PendingBits(self.sensitivity(mn, mx, N, num_pixels))
-        return groups, mn, mx, pending, input.numel() // N
+        C_dev = self.sensitivity(mn, mx, N, num_pixels)
+        bits_dev = None
+        if allocate_on_device(N, self.initial_bits):
+            bits_dev = greedy_bits_device(C_dev, N, self.initial_bits, self.bits)
+        pending = PendingBits(C_dev)
+        return groups, mn, mx, pending, input.numel() // N, bits_dev
 
     def finish_quantization_bits(self, started):
-        """Second half: wait for the sensitivities, greedy allocation, widths back to the device."""
-        groups, mn, mx, pending, dim = started
+        """Second half.  Widths made on the device: nothing to wait for (the host copy of the
+        sensitivities is picked up when the per-layer re-balancing asks for it).  Otherwise: wait
+        for the sensitivities, greedy allocation on the host, widths back to the device."""
+        groups, mn, mx, pending, dim, bits_dev = started
         N = groups.shape[0]
-        C = pending.wait().clone()
-        bits_dev, b = greedy_bits(C, N, self.initial_bits, self.bits, groups.device)
-        self.C = C
         self.dim = dim
-        self.b = b
+        if bits_dev is not None:
+            self._pending_C = pending
+            self.b = bits_dev
+        else:
+            C = pending.wait().clone()
+            bits_dev, b = greedy_bits(C, N, self.initial_bits, self.bits, groups.device)
+            self.C = C
+            self.b = b
         return groups, bits_dev, mn.view(N, -1, 1), mx.view(N, -1, 1)
 
     # -- per-layer re-balancing -------------------------------------------------------------

@@ -147,6 +147,15 @@ int actnn_max_pool2d_backward(const void* grad_out, const int8_t* idx, void* gra
  * ------------------------------------------------------------------------------- */
 int actnn_calc_precision(int32_t* b, const float* C, const int32_t* w, int64_t N, double target);
 
+/* Same allocation on the DEVICE for the case every layer uses at every step: all N items start
+ * at initial_bits (1..8) with weight 1 and `target` is the bit budget, so exactly
+ * N * initial_bits - target widths are taken away (clamped to [0, N * (initial_bits - 1)]).
+ * C: fp32[N] device, bits: int32[N] device (output).  Bit-identical to actnn_calc_precision on
+ * the same inputs; N * (initial_bits - 1) <= 8192, otherwise ACTNN_EINVAL (use the host routine).
+ * Replaces the device -> host -> device round trip of qscheme.py:83-94. */
+int actnn_calc_precision_device(const float* C, int32_t* bits, int64_t N, int initial_bits,
+                                int64_t target, void* stream);
+
 /* ---------------------------------------------------------------------------------
  * Fused QLinear weight gradient: grad_w[O, I] = grad_out[M, O]^T @ dequant(x)[M, I] where x
  * is held as the pack_single 2-bit stream (4 consecutive rows m per byte) with

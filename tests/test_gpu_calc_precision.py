@@ -1,0 +1,60 @@
+"""Greedy allocation on the device vs the host routine (itself pinned against the oracle, brute
+force and the reference's own calc_precision.cc in tests/test_oracle_calc_precision.py): the
+widths must be identical, ties and zero sensitivities included."""
+import numpy as np
+import pytest
+import torch
+
+import actnn_amd.cpp_extension.calc_precision as ext_cp
+from _util import DEV
+
+pytestmark = pytest.mark.gpu
+
+
+def _host(C, initial, target):
+    N = C.numel()
+    b = torch.ones(N, dtype=torch.int32) * initial
+    return ext_cp.calc_precision(b, C.clone(), torch.ones(N, dtype=torch.int32), float(target))
+
+
+def _cases():
+    g = torch.Generator().manual_seed(0)
+    yield "lognormal", torch.exp(3 * torch.randn(512, generator=g)), 8, 2 * 512
+    yield "uniform", torch.rand(300, generator=g), 8, int(2.5 * 300)
+    yield "all_zero", torch.zeros(16), 8, 32                  # first training step: every delta is -0
+    yield "some_zero", torch.cat([torch.zeros(7), torch.rand(9, generator=g)]), 8, 40
+    yield "duplicates", torch.tensor([1.0, 2.0, 1.0, 2.0, 1.0, 0.5, 0.5, 4.0] * 8), 8, 3 * 64
+    yield "one_item", torch.tensor([3.0]), 8, 2
+    yield "nothing_to_take", torch.rand(10, generator=g), 4, 40
+    yield "over_budget", torch.rand(10, generator=g), 4, 50
+    yield "everything_taken", torch.rand(10, generator=g), 8, 10
+    yield "below_floor", torch.rand(10, generator=g), 8, 3    # cannot go below one bit each
+    yield "initial_2", torch.rand(100, generator=g), 2, 150
+    yield "huge_range", torch.tensor([1e-30, 1e30, 1.0, 1e-10, 1e10] * 20), 8, 250
+    yield "max_candidates", torch.exp(torch.randn(1170, generator=g)), 8, 2 * 1170
+    for seed in range(20):
+        gg = torch.Generator().manual_seed(100 + seed)
+        N = int(torch.randint(1, 600, (1,), generator=gg))
+        initial = int(torch.randint(2, 9, (1,), generator=gg))
+        avg = float(torch.rand(1, generator=gg)) * (initial - 1) + 1
+        C = torch.exp(2 * torch.randn(N, generator=gg)).round(decimals=int(seed % 3))   # coarse values: ties
+        yield f"random{seed}", C, initial, int(avg * N)
+
+
+@pytest.mark.parametrize("name,C,initial,target", list(_cases()), ids=lambda v: v if isinstance(v, str) else "")
+def test_device_allocation_equals_host(name, C, initial, target):
+    C = C.float().contiguous()
+    exp = _host(C, initial, target)
+    got = ext_cp.calc_precision_device(C.to(DEV), initial, target)
+    assert got.dtype == torch.int32 and got.is_cuda
+    assert np.array_equal(got.cpu().numpy(), exp.numpy()), name
+
+
+def test_device_allocation_rejects_what_does_not_fit():
+    with pytest.raises(RuntimeError):
+        ext_cp.calc_precision_device(torch.rand(1171, device=DEV), 8, 2000)      # 8197 candidates
+    with pytest.raises(RuntimeError):
+        ext_cp.calc_precision_device(torch.rand(8, device=DEV), 9, 16)
+    with pytest.raises(RuntimeError):
+        ext_cp.calc_precision_device(torch.rand(8), 8, 16)                        # host tensor
+    assert ext_cp.calc_precision_device(torch.rand(0, device=DEV), 8, 0).numel() == 0
