@@ -30,6 +30,7 @@ def _cases():
     yield "everything_taken", torch.rand(10, generator=g), 8, 10
     yield "below_floor", torch.rand(10, generator=g), 8, 3    # cannot go below one bit each
     yield "initial_2", torch.rand(100, generator=g), 2, 150
+    yield "initial_1", torch.rand(9, generator=g), 1, 9
     yield "huge_range", torch.tensor([1e-30, 1e30, 1.0, 1e-10, 1e10] * 20), 8, 250
     yield "max_candidates", torch.exp(torch.randn(1170, generator=g)), 8, 2 * 1170
     for seed in range(20):
