@@ -45,11 +45,22 @@ __global__ __launch_bounds__(kThreads) void calc_precision_device_kernel(
       bits[item0 + threadIdx.x] = K <= 0 ? initial : 1;
     return;
   }
-  for (int c = threadIdx.x; c < total; c += kThreads) {
-    const int i = c / L, l = c - i * L, b = initial - l;
+  // 1/(2^b - 1)^2 - 1/(2^(b-1) - 1)^2 for the L steps: held in the tail of the key array until the
+  // keys that would overwrite it are built (total < kMaxCand leaves room; otherwise per key)
+  const bool shared_factors = total + 8 <= kMaxCand;
+  double* factors = reinterpret_cast<double*>(keys + kMaxCand - 8);
+  auto factor_of = [&](int l) {
+    const int b = initial - l;
     const int64_t full = ((int64_t)1 << b) - 1, less = ((int64_t)1 << (b - 1)) - 1;
-    const double factor = 1.0 / (double)(full * full) - 1.0 / (double)(less * less);
-    keys[c] = step_key(C[i], factor, i, l);
+    return 1.0 / (double)(full * full) - 1.0 / (double)(less * less);
+  };
+  if (shared_factors) {
+    if ((int)threadIdx.x < L) factors[threadIdx.x] = factor_of(threadIdx.x);
+    __syncthreads();
+  }
+  for (int c = threadIdx.x; c < total; c += kThreads) {
+    const int i = c / L, l = c - i * L;
+    keys[c] = step_key(C[i], shared_factors ? factors[l] : factor_of(l), i, l);
   }
   __syncthreads();
   // thread -> (slot = candidate of this block, seg = which 16th of the keys it counts over)
