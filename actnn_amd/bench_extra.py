@@ -1,5 +1,5 @@
 """Extra benchmark legs used by bench.py: the ResNet-50 training step under QModule at L3
-(BASELINE config 5) with the reference's speed and memory protocols
+(benchmark config 5) with the reference's speed and memory protocols
 (mem_speed_benchmark/train.py:363-397 memory, :422-438 speed)."""
 import time
 

@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-One step = one pass of the hot path over BASELINE config 2: minimax -> pack_mixed_precision
+One step = one pass of the hot path over benchmark config 2: minimax -> pack_mixed_precision
 (in-kernel Philox) -> unpack_mixed_precision on a resident fp32 activation [256,256,56,56]
 (ResNet-50 layer1), per-sample bits from the greedy allocation at an average of 2.0 bits,
 groups of 256.  `value` is algorithmic bytes per step / time per step.  The JSON line also
@@ -54,7 +54,7 @@ def _event_time_ms(fn, reps, warmup=3):
 
 
 def make_config2(device, N=256, C=256, H=56, W=56, seed=0):
-    """fp32 activation of BASELINE config 2 and its per-sample bits (greedy at avg 2.0 bits)."""
+    """fp32 activation of benchmark config 2 and its per-sample bits (greedy at avg 2.0 bits)."""
     import torch
     import actnn_amd.cpp_extension.calc_precision as ext_cp
     import actnn_amd.cpp_extension.minimax as ext_minimax
@@ -91,7 +91,7 @@ def algorithmic_bytes(n, esize, avg_bits, gs=256):
 
 def cpu_baseline(budget_s=15.0):
     """The oracle's restatement of the reference's config.simulate quantise+dequantise
-    (actnn/actnn/ops.py:22-41,55-57) on BASELINE config 1, all host cores."""
+    (actnn/actnn/ops.py:22-41,55-57) on benchmark config 1, all host cores."""
     import torch
     from oracle import simulate
     cores = os.cpu_count() or 1

@@ -21,7 +21,7 @@ def make_groups(N, G, gs, dtype, seed, kind="relu", scale=1.0):
     x = torch.randn(N, G, gs, generator=g) * scale
     if kind == "relu":
         x = torch.relu(x)
-    elif kind == "chan":       # per-group log-normal scale, like BASELINE config 2
+    elif kind == "chan":       # per-group log-normal scale, like benchmark config 2
         x = torch.relu(x) * torch.exp(torch.randn(1, G, 1, generator=g))
     elif kind == "shift":      # large offset relative to the range
         x = x + 100.0

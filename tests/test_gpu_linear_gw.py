@@ -1,5 +1,5 @@
 """Fused 2-bit QLinear weight gradient vs torch's bf16 GEMM on the dequantised input
-(BASELINE config 4 tolerance: rtol 2e-2)."""
+(benchmark config 4 tolerance: rtol 2e-2)."""
 import pytest
 import torch
 

@@ -38,7 +38,7 @@ def _det_case(x, noise, bits_list):
 
 
 def test_config1_fp32_uniform_2bit_bit_exact():
-    # BASELINE config 1: relu(randn(32,64,56,56)) -> [32,784,256], 2 bits, seeded noise
+    # benchmark config 1: relu(randn(32,64,56,56)) -> [32,784,256], 2 bits, seeded noise
     torch.manual_seed(0)
     x = torch.relu(torch.randn(32, 64, 56, 56)).view(32, 784, 256)
     noise = torch.rand(32, 784, 256, generator=torch.Generator().manual_seed(1)) - 0.5
