@@ -12,7 +12,7 @@ CSRC = os.path.join(_HERE, "csrc")
 # ACTNN_HIP_LIB points at another build of the same library (kernel tuning experiments)
 LIB_PATH = os.environ.get("ACTNN_HIP_LIB") or os.path.join(_HERE, "libactnn_hip.so")
 SOURCES = ["minimax.hip", "pack_mixed.hip", "pack_single.hip", "mask_ops.hip", "maxpool.hip",
-           "linear_gw.hip", "misc.hip", "calc_precision.cpp", "calc_precision_dev.hip"]
+           "linear_gw.hip", "misc.hip", "calc_precision.cpp", "calc_precision_dev.hip", "batch_norm.hip"]
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-ffp-contract=off",                      # bit-exact quantiser: no implicit FMA
@@ -48,8 +48,14 @@ SIGNATURES = {
     "actnn_linear_grad_weight_q2": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64,
                                     c_i32, c_i32, c_i32, c_vp],
     "actnn_stream_copy": [c_vp, c_vp, c_i64, c_vp],
+    "actnn_batch_norm_workspace_bytes": [c_i64, c_i64, c_i64, c_i32],
+    "actnn_batch_norm_forward": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,
+                                 c_i64, c_i64, c_i64, ctypes.c_double, ctypes.c_double, c_i32, c_vp],
+    "actnn_batch_norm_backward": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,
+                                  c_i64, c_i64, c_i64, c_i32, c_vp],
 }
-_RESTYPES = {"actnn_strerror": ctypes.c_char_p, "actnn_version": ctypes.c_char_p}
+_RESTYPES = {"actnn_strerror": ctypes.c_char_p, "actnn_version": ctypes.c_char_p,
+             "actnn_batch_norm_workspace_bytes": ctypes.c_int64}
 
 _lib = None
 

@@ -1,12 +1,83 @@
 """Backward ATen entry points the reference re-exports (cpp_extension/backward_func.cc:81-91),
-mapped onto the ATen ops that exist on PyTorch-ROCm (MIOpen behind them).  No new kernels:
-this module only keeps the reference's names and argument order.
+under the reference's names and argument order.  The convolutions map onto the ATen ops that
+exist on PyTorch-ROCm (MIOpen behind them); training-mode batch norm runs this library's own
+kernels (actnn_batch_norm_forward / _backward) whenever the shape qualifies and falls back to
+ATen's miopen_batch_norm otherwise.
 
 The three layer-norm exports of the reference have no Python caller and are not provided.
 """
 import torch
 
+from . import _glue
+
 _aten = torch.ops.aten
+
+
+def _bn_geometry(input):
+    """(N, C, HW) when the library's batch-norm kernels take this tensor, else None."""
+    if not (isinstance(input, torch.Tensor) and input.is_cuda and input.dim() >= 2
+            and input.dtype in _glue.DTYPE_CODE and input.is_contiguous() and input.numel() > 0):
+        return None
+    N, C = input.shape[0], input.shape[1]
+    HW = input.numel() // (N * C)
+    if _glue.lib().actnn_batch_norm_workspace_bytes(N, C, HW, _glue.DTYPE_CODE[input.dtype]) < 0:
+        return None
+    return N, C, HW
+
+
+def _f32_or_none(t):
+    return t is None or (t.dtype == torch.float32 and t.is_cuda and t.is_contiguous())
+
+
+def hip_batch_norm_applies(input, weight, bias, running_mean, running_var):
+    return (_bn_geometry(input) is not None and input.data_ptr() % 16 == 0
+            and all(_f32_or_none(t) for t in (weight, bias, running_mean, running_var)))
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def hip_batch_norm_forward(input, weight, bias, running_mean, running_var, momentum, eps, minmax=False):
+    """-> (output, save_mean, save_invstd, mn, mx): training-mode batch norm; with `minmax` the
+    minimum and maximum of every group of 256 consecutive elements of a sample come out of the
+    same pass over the input (None, None otherwise)."""
+    N, C, HW = _bn_geometry(input)
+    lib = _glue.lib()
+    code = _glue.DTYPE_CODE[input.dtype]
+    ws_bytes = lib.actnn_batch_norm_workspace_bytes(N, C, HW, code)
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=input.device)
+    out = torch.empty_like(input)
+    save_mean = torch.empty(C, dtype=torch.float32, device=input.device)
+    save_invstd = torch.empty(C, dtype=torch.float32, device=input.device)
+    mn = mx = None
+    if minmax:
+        groups = N * C * HW // 256
+        mn = torch.empty(groups, dtype=input.dtype, device=input.device)
+        mx = torch.empty(groups, dtype=input.dtype, device=input.device)
+    _glue._lib.check(lib.actnn_batch_norm_forward(
+        input.data_ptr(), _ptr(weight), _ptr(bias), _ptr(running_mean), _ptr(running_var),
+        out.data_ptr(), save_mean.data_ptr(), save_invstd.data_ptr(), _ptr(mn), _ptr(mx),
+        ws.data_ptr(), ws_bytes, N, C, HW, float(momentum), float(eps), code,
+        _glue.stream_ptr(input.device)), "batch_norm_forward")
+    return out, save_mean, save_invstd, mn, mx
+
+
+def hip_batch_norm_backward(input, grad_output, weight, save_mean, save_invstd):
+    """-> (grad_input, grad_weight, grad_bias) of training-mode batch norm."""
+    N, C, HW = _bn_geometry(input)
+    lib = _glue.lib()
+    code = _glue.DTYPE_CODE[input.dtype]
+    ws_bytes = lib.actnn_batch_norm_workspace_bytes(N, C, HW, code)
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=input.device)
+    grad_input = torch.empty_like(input)
+    grad_weight = torch.empty(C, dtype=torch.float32, device=input.device)
+    grad_bias = torch.empty(C, dtype=torch.float32, device=input.device)
+    _glue._lib.check(lib.actnn_batch_norm_backward(
+        input.data_ptr(), grad_output.data_ptr(), _ptr(weight), save_mean.data_ptr(),
+        save_invstd.data_ptr(), grad_input.data_ptr(), grad_weight.data_ptr(), grad_bias.data_ptr(),
+        ws.data_ptr(), ws_bytes, N, C, HW, code, _glue.stream_ptr(input.device)), "batch_norm_backward")
+    return grad_input, grad_weight, grad_bias
 
 
 def cudnn_convolution_backward(input, grad_output, weight, padding, stride, dilation, groups,
@@ -32,7 +103,12 @@ def cudnn_convolution_transpose_backward(input, grad_output, weight, padding, ou
 def cudnn_batch_norm(input, weight, bias, running_mean, running_var, training,
                      exponential_average_factor, epsilon):
     """-> (output, save_mean, save_var, reserve).  at::native::cudnn_batch_norm
-    (backward_func.cc:87) -> miopen_batch_norm; `reserve` is an empty placeholder."""
+    (backward_func.cc:87); save_var holds the inverse standard deviation, as cuDNN's and
+    MIOpen's do; `reserve` is an empty placeholder."""
+    if training and hip_batch_norm_applies(input, weight, bias, running_mean, running_var):
+        out, save_mean, save_invstd, _, _ = hip_batch_norm_forward(
+            input, weight, bias, running_mean, running_var, exponential_average_factor, epsilon)
+        return out, save_mean, save_invstd, input.new_empty(0, dtype=torch.uint8)
     out, save_mean, save_var = _aten.miopen_batch_norm(
         input, weight, bias, running_mean, running_var, training, exponential_average_factor, epsilon)
     return out, save_mean, save_var, input.new_empty(0, dtype=torch.uint8)
@@ -41,7 +117,11 @@ def cudnn_batch_norm(input, weight, bias, running_mean, running_var, training,
 def cudnn_batch_norm_backward(input, grad_output, weight, running_mean, running_var, save_mean,
                               save_var, epsilon, reserve):
     """-> (grad_input, grad_weight, grad_bias).  at::native::cudnn_batch_norm_backward
-    (backward_func.cc:88) -> miopen_batch_norm_backward."""
+    (backward_func.cc:88)."""
+    if (hip_batch_norm_applies(input, weight, None, save_mean, save_var)
+            and grad_output.dtype == input.dtype and grad_output.shape == input.shape
+            and grad_output.is_contiguous() and grad_output.data_ptr() % 16 == 0):
+        return hip_batch_norm_backward(input, grad_output, weight, save_mean, save_var)
     return _aten.miopen_batch_norm_backward(input, grad_output, weight, running_mean, running_var,
                                             save_mean, save_var, epsilon)
 

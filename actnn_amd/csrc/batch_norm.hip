@@ -1,0 +1,505 @@
+// Training-mode batch normalisation over contiguous [N, C, HW] tensors, forward and backward
+// (the work the reference hands to cuDNN through cudnn_batch_norm / cudnn_batch_norm_backward,
+// cpp_extension/backward_func.cc:87-88, called from ops.py:448-449 and ops.py:479-481).
+//
+// All four passes are HBM-bound streams and share one thread-to-data mapping.  A sample is a row
+// of F = C*HW elements; a block owns a span of kThreads 16-byte chunks of that row and walks down
+// the batch, so a thread meets the same offsets - hence the same one or two channels - in every
+// sample.  Everything that depends on the channel (accumulators, coefficients, the position of a
+// channel boundary inside the chunk) lives in registers for the whole loop, the loads are
+// 16 bytes wide and contiguous across the block, and no per-element division or table lookup is
+// needed.  Reductions finish once per block: lanes of one channel are combined with a segmented
+// shuffle reduction, the per-wave results are added in a fixed order and written to a table of
+// partial sums that a small second kernel folds per channel in double precision (no atomics: the
+// result does not depend on the schedule).
+//
+// The statistics pass can also produce the per-group minimum and maximum of the activation
+// quantiser (groups of 256 consecutive elements of the row) from the registers it already holds,
+// which saves the quantiser's own read of the tensor.
+#include "device_utils.h"
+
+namespace actnn {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / 64;
+constexpr int kUnroll = 4;            // samples in flight per thread
+
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+
+// Arithmetic on the dwords of a 16-byte chunk.  16-bit types use the two-element dot product
+// instructions, whose products are exact in fp32.
+template <typename T> struct Chunk;
+template <> struct Chunk<float> {
+  static constexpr int kElems = 4, kPerDword = 1;
+  static ACTNN_DEV void add(uint32_t a, float& s) { s += as_float(a); }
+  static ACTNN_DEV void dot(uint32_t a, uint32_t b, float& s) { s = fmaf(as_float(a), as_float(b), s); }
+  static ACTNN_DEV void widen(uint32_t a, float* v) { v[0] = as_float(a); }
+  static ACTNN_DEV uint32_t narrow(const float* v) { return as_uint(v[0]); }
+};
+template <> struct Chunk<__half> {
+  static constexpr int kElems = 8, kPerDword = 2;
+  static ACTNN_DEV void add(uint32_t a, float& s) {
+    s = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, a), __builtin_bit_cast(f16x2_t, 0x3c003c00u), s, false);
+  }
+  static ACTNN_DEV void dot(uint32_t a, uint32_t b, float& s) {
+    s = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, a), __builtin_bit_cast(f16x2_t, b), s, false);
+  }
+  static ACTNN_DEV void widen(uint32_t a, float* v) {
+    v[0] = half_bits_to_float(a & 0xffffu);
+    v[1] = half_bits_to_float(a >> 16);
+  }
+  static ACTNN_DEV uint32_t narrow(const float* v) {
+    return float_to_half_bits(v[0]) | (float_to_half_bits(v[1]) << 16);
+  }
+};
+template <> struct Chunk<bf16_t> {
+  static constexpr int kElems = 8, kPerDword = 2;
+  static ACTNN_DEV void add(uint32_t a, float& s) {
+    s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), s, false);
+  }
+  static ACTNN_DEV void dot(uint32_t a, uint32_t b, float& s) {
+    s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), s, false);
+  }
+  static ACTNN_DEV void widen(uint32_t a, float* v) {
+    v[0] = as_float(a << 16);
+    v[1] = as_float(a & 0xffff0000u);
+  }
+  static ACTNN_DEV uint32_t narrow(const float* v) { return pack_bf16x2(v[0], v[1]); }
+};
+
+// Where a thread's chunk lies: the channel of its first element, how many of its elements belong
+// to that channel (>= kElems when the chunk does not cross a boundary; the rest belong to the
+// next channel - HW >= kElems is a precondition), and whether the chunk exists at all.
+struct Place {
+  int64_t elem;        // offset of the chunk in the row
+  int64_t channel;     // channel of the first element
+  int head;            // elements of the chunk in `channel`, clamped to kElems
+  bool active;
+};
+template <int E> ACTNN_DEV Place place_of(int64_t F, int64_t HW) {
+  Place p;
+  p.elem = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * E;
+  p.active = p.elem < F;
+  if (!p.active) p.elem = (int64_t)blockIdx.x * kThreads * E;       // a valid address; results dropped
+  p.channel = p.elem / HW;
+  const int64_t left = (p.channel + 1) * HW - p.elem;
+  p.head = left >= E ? E : (int)left;
+  return p;
+}
+
+// Dword masks that keep the elements of the chunk's first channel.
+template <typename T> ACTNN_DEV void head_masks(int head, uint32_t (&m)[4]) {
+  constexpr int PD = Chunk<T>::kPerDword;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int k = head - j * PD;
+    m[j] = k <= 0 ? 0u : (PD == 2 && k == 1) ? 0x0000ffffu : 0xffffffffu;
+  }
+}
+
+// Sum over the lanes of a run of equal keys (runs are contiguous); the first lane of a run
+// ends with the run's total.
+ACTNN_DEV void run_sums(int key, float& a, float& b) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int k2 = __shfl_down(key, d);
+    const float a2 = __shfl_down(a, d), b2 = __shfl_down(b, d);
+    if (lane + d < 64 && k2 == key) { a += a2; b += b2; }
+  }
+}
+
+// Adds the block's per-thread sums into the table of partial sums.  (head0, head1) belong to the
+// chunk's first channel, (tail0, tail1) to the next one (chunks that cross a boundary only).
+// `s_acc` holds kWaves * (slots + 1) pairs; slot `slots` absorbs the chunks that do not exist.
+// Within one instruction the lanes that write touch distinct slots (one lane per run of equal
+// channels, one lane per channel boundary), and a wave's instructions reach LDS in order, so
+// plain read-modify-write is enough and the order of the additions is fixed.
+template <int E>
+ACTNN_DEV void fold_block(float* s_acc, int slots, const Place& p, int64_t first_channel,
+                          float head0, float head1, float tail0, float tail1,
+                          float* __restrict__ part) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float* acc = s_acc + (size_t)wave * (slots + 1) * 2;
+  for (int i = threadIdx.x; i < kWaves * (slots + 1) * 2; i += kThreads) s_acc[i] = 0.0f;
+  __syncthreads();
+  const int key = p.active ? (int)(p.channel - first_channel) : slots;
+  if (!p.active) { head0 = 0.0f; head1 = 0.0f; }
+  run_sums(key, head0, head1);
+  const int prev = __shfl_up(key, 1);
+  if (lane == 0 || prev != key) {
+    acc[2 * key] += head0;
+    acc[2 * key + 1] += head1;
+  }
+  if (p.active && p.head < E) {
+    acc[2 * (key + 1)] += tail0;
+    acc[2 * (key + 1) + 1] += tail1;
+  }
+  __syncthreads();
+  const int64_t base = ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * slots * 2;
+  for (int i = threadIdx.x; i < slots * 2; i += kThreads) {
+    float v = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) v += s_acc[(size_t)w * (slots + 1) * 2 + i];
+    part[base + i] = v;
+  }
+}
+
+// Pass 1 of either direction.  Forward: per-channel sum(x) and sum(x*x) (+ per-group min/max of
+// x when MINMAX).  Backward: per-channel sum(dy) and sum(x*dy).
+template <typename T, bool SPLIT, bool BWD, bool MINMAX>
+__global__ __launch_bounds__(kThreads) void bn_reduce_kernel(
+    const T* __restrict__ x, const T* __restrict__ dy, float* __restrict__ part,
+    T* __restrict__ mn, T* __restrict__ mx, int64_t N, int64_t F, int64_t HW, int per_block, int slots) {
+  constexpr int E = Chunk<T>::kElems;
+  extern __shared__ float s_acc[];
+  const Place p = place_of<E>(F, HW);
+  uint32_t m[4];
+  head_masks<T>(p.head, m);
+  const int64_t n0 = (int64_t)blockIdx.y * per_block;
+  const int64_t n1 = n0 + per_block < N ? n0 + per_block : N;
+  float t0 = 0.0f, t1 = 0.0f, h0 = 0.0f, h1 = 0.0f;
+
+  auto accumulate = [&](const u32x4& ux, const u32x4& ud, int64_t n) {
+    const uint32_t w[4] = {ux.x, ux.y, ux.z, ux.w};
+    const uint32_t d[4] = {ud.x, ud.y, ud.z, ud.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t a = BWD ? d[j] : w[j];
+      Chunk<T>::add(a, t0);
+      Chunk<T>::dot(w[j], a, t1);
+      if (SPLIT) {
+        const uint32_t am = a & m[j];
+        Chunk<T>::add(am, h0);
+        Chunk<T>::dot(w[j], am, h1);
+      }
+    }
+    if (MINMAX) {
+      constexpr int PD = Chunk<T>::kPerDword;
+      constexpr int LPG = 256 / E;                      // lanes per quantisation group
+      float v[E];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) Chunk<T>::widen(w[j], v + j * PD);
+      float lo = v[0], hi = v[0];
+#pragma unroll
+      for (int i = 1; i < E; ++i) { lo = fminf(lo, v[i]); hi = fmaxf(hi, v[i]); }
+      lo = rows_min<LPG / 16>(row16_min(lo));
+      hi = rows_max<LPG / 16>(row16_max(hi));
+      if ((threadIdx.x & (LPG - 1)) == LPG - 1 && p.active) {
+        const int64_t g = n * (F >> 8) + (p.elem >> 8);
+        Conv<T>::store(mn, g, lo);
+        Conv<T>::store(mx, g, hi);
+      }
+    }
+  };
+
+  const T* px = x + n0 * F + p.elem;
+  const T* pd = BWD ? dy + n0 * F + p.elem : nullptr;
+  int64_t n = n0;
+  for (; n + kUnroll <= n1; n += kUnroll) {
+    u32x4 ux[kUnroll], ud[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      ux[u] = load16(px + u * F);
+      ud[u] = BWD ? load16(pd + u * F) : ux[u];
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) accumulate(ux[u], ud[u], n + u);
+    px += kUnroll * F;
+    if (BWD) pd += kUnroll * F;
+  }
+  for (; n < n1; ++n) {
+    const u32x4 ux = load16(px);
+    const u32x4 ud = BWD ? load16(pd) : ux;
+    accumulate(ux, ud, n);
+    px += F;
+    if (BWD) pd += F;
+  }
+  const int64_t first_channel = ((int64_t)blockIdx.x * kThreads * E) / HW;
+  fold_block<E>(s_acc, slots, p, first_channel, SPLIT ? h0 : t0, SPLIT ? h1 : t1,
+                SPLIT ? t0 - h0 : 0.0f, SPLIT ? t1 - h1 : 0.0f, part);
+}
+
+// Folds the table of partial sums of channel c in double precision, in a fixed order.
+ACTNN_DEV void channel_totals(const float* __restrict__ part, int64_t c, int64_t HW, int64_t L,
+                              int nsplit, int slots, double& s0, double& s1) {
+  const int64_t j0 = (c * HW) / L, j1 = ((c + 1) * HW - 1) / L;
+  s0 = 0.0;
+  s1 = 0.0;
+  for (int64_t j = j0; j <= j1; ++j) {
+    const int64_t slot = c - (j * L) / HW;
+    const float* q = part + ((j * nsplit) * slots + slot) * 2;
+    for (int y = 0; y < nsplit; ++y, q += (int64_t)slots * 2) {
+      s0 += (double)q[0];
+      s1 += (double)q[1];
+    }
+  }
+}
+
+// mean / inverse standard deviation of the batch, the running estimates (unbiased variance, as
+// torch's batch norm keeps them) and the per-channel coefficients of y = a*x + b.
+__global__ __launch_bounds__(kThreads) void bn_forward_finalize_kernel(
+    const float* __restrict__ part, const float* __restrict__ weight, const float* __restrict__ bias,
+    float* __restrict__ running_mean, float* __restrict__ running_var, float* __restrict__ save_mean,
+    float* __restrict__ save_invstd, float* __restrict__ coef, int64_t N, int64_t C, int64_t HW,
+    int64_t L, int nsplit, int slots, double momentum, double eps) {
+  const int64_t c = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (c >= C) return;
+  double S, Q;
+  channel_totals(part, c, HW, L, nsplit, slots, S, Q);
+  const double M = (double)N * (double)HW;
+  const double mean = S / M;
+  double var = Q / M - mean * mean;
+  if (!(var > 0.0)) var = 0.0;
+  const double invstd = 1.0 / sqrt(var + eps);
+  save_mean[c] = (float)mean;
+  save_invstd[c] = (float)invstd;
+  if (running_mean) running_mean[c] = (float)((1.0 - momentum) * running_mean[c] + momentum * mean);
+  if (running_var) {
+    const double unbiased = M > 1.0 ? var * (M / (M - 1.0)) : var;
+    running_var[c] = (float)((1.0 - momentum) * running_var[c] + momentum * unbiased);
+  }
+  const double a = (weight ? (double)weight[c] : 1.0) * invstd;
+  coef[2 * c] = (float)a;
+  coef[2 * c + 1] = (float)((bias ? (double)bias[c] : 0.0) - mean * a);
+}
+
+// grad_weight, grad_bias and the per-channel coefficients of dx = A*dy + B*x + K, from
+// dx = w*r*(dy - mean(dy) - xhat*mean(dy*xhat)) with xhat = (x - mean)*r.
+__global__ __launch_bounds__(kThreads) void bn_backward_finalize_kernel(
+    const float* __restrict__ part, const float* __restrict__ weight, const float* __restrict__ save_mean,
+    const float* __restrict__ save_invstd, float* __restrict__ dweight, float* __restrict__ dbias,
+    float* __restrict__ coef, int64_t N, int64_t C, int64_t HW, int64_t L, int nsplit, int slots) {
+  const int64_t c = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (c >= C) return;
+  double S, Q;                                   // sum(dy), sum(x*dy)
+  channel_totals(part, c, HW, L, nsplit, slots, S, Q);
+  const double M = (double)N * (double)HW;
+  const double mean = save_mean[c], r = save_invstd[c];
+  const double w = weight ? (double)weight[c] : 1.0;
+  const double dot = (Q - mean * S) * r;         // sum(dy * xhat)
+  if (dweight) dweight[c] = (float)dot;
+  if (dbias) dbias[c] = (float)S;
+  const double A = w * r;
+  const double B = -w * r * r * (dot / M);
+  coef[3 * c] = (float)A;
+  coef[3 * c + 1] = (float)B;
+  coef[3 * c + 2] = (float)(-A * (S / M) - B * mean);
+}
+
+// Pass 2 of either direction.  Forward: y = a*x + b.  Backward: dx = A*dy + B*x + K.
+template <typename T, bool SPLIT, bool BWD>
+__global__ __launch_bounds__(kThreads) void bn_apply_kernel(
+    const T* __restrict__ x, const T* __restrict__ dy, const float* __restrict__ coef,
+    T* __restrict__ out, int64_t N, int64_t F, int64_t HW, int per_block) {
+  constexpr int E = Chunk<T>::kElems;
+  constexpr int PD = Chunk<T>::kPerDword;
+  constexpr int NC = BWD ? 3 : 2;
+  const Place p = place_of<E>(F, HW);
+  if (!p.active) return;
+  float k0[NC], k1[NC];
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    k0[i] = coef[NC * p.channel + i];
+    k1[i] = (SPLIT && p.head < E) ? coef[NC * (p.channel + 1) + i] : k0[i];
+  }
+  float ka[E], kb[E], kc[E];
+#pragma unroll
+  for (int i = 0; i < E; ++i) {
+    const bool first = !SPLIT || i < p.head;
+    ka[i] = first ? k0[0] : k1[0];
+    kb[i] = first ? k0[1] : k1[1];
+    kc[i] = BWD ? (first ? k0[NC - 1] : k1[NC - 1]) : 0.0f;
+  }
+  const int64_t n0 = (int64_t)blockIdx.y * per_block;
+  const int64_t n1 = n0 + per_block < N ? n0 + per_block : N;
+
+  auto apply = [&](const u32x4& ux, const u32x4& ud) -> u32x4 {
+    const uint32_t w[4] = {ux.x, ux.y, ux.z, ux.w};
+    const uint32_t d[4] = {ud.x, ud.y, ud.z, ud.w};
+    uint32_t r[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float v[PD], g[PD], o[PD];
+      Chunk<T>::widen(w[j], v);
+      if (BWD) Chunk<T>::widen(d[j], g);
+#pragma unroll
+      for (int i = 0; i < PD; ++i) {
+        const int e = j * PD + i;
+        o[i] = BWD ? fmaf(g[i], ka[e], fmaf(v[i], kb[e], kc[e])) : fmaf(v[i], ka[e], kb[e]);
+      }
+      r[j] = Chunk<T>::narrow(o);
+    }
+    return u32x4{r[0], r[1], r[2], r[3]};
+  };
+
+  const T* px = x + n0 * F + p.elem;
+  const T* pd = BWD ? dy + n0 * F + p.elem : nullptr;
+  T* po = out + n0 * F + p.elem;
+  int64_t n = n0;
+  for (; n + kUnroll <= n1; n += kUnroll) {
+    u32x4 ux[kUnroll], ud[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      ux[u] = load16(px + u * F);
+      ud[u] = BWD ? load16(pd + u * F) : ux[u];
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) store16(po + u * F, apply(ux[u], ud[u]));
+    px += kUnroll * F;
+    po += kUnroll * F;
+    if (BWD) pd += kUnroll * F;
+  }
+  for (; n < n1; ++n) {
+    const u32x4 ux = load16(px);
+    const u32x4 ud = BWD ? load16(pd) : ux;
+    store16(po, apply(ux, ud));
+    px += F;
+    po += F;
+    if (BWD) pd += F;
+  }
+}
+
+// Launch geometry shared by the passes of one call.
+struct Plan {
+  int elems;           // elements per 16-byte chunk
+  int64_t F, L, spans;
+  int per_block, nsplit, slots;
+  bool split;
+  int64_t part_floats;
+};
+bool make_plan(int64_t N, int64_t C, int64_t HW, int dtype, Plan& pl) {
+  if (N <= 0 || C <= 0 || HW <= 0 || dtype < 0 || dtype > 2) return false;
+  pl.elems = dtype == ACTNN_F32 ? 4 : 8;
+  if (HW < pl.elems || C > ((int64_t)1 << 40) / HW) return false;
+  pl.F = C * HW;
+  if (pl.F % pl.elems != 0 || N > ((int64_t)1 << 62) / pl.F) return false;
+  pl.L = (int64_t)kThreads * pl.elems;
+  pl.spans = (pl.F + pl.L - 1) / pl.L;
+  if (pl.spans > 0x7fffffffLL) return false;
+  int64_t want = (2048 + pl.spans - 1) / pl.spans;       // enough blocks to fill the chip
+  if (want > 65535) want = 65535;
+  int64_t per_block = (N + want - 1) / want;
+  if (per_block < 8) per_block = 8;
+  if (per_block > N) per_block = N;
+  const int64_t nsplit = (N + per_block - 1) / per_block;
+  if (nsplit > 65535 || per_block > 0x7fffffffLL) return false;
+  pl.per_block = (int)per_block;
+  pl.nsplit = (int)nsplit;
+  int64_t slots = (pl.L - 1) / HW + 2;                    // channels one span can touch
+  if (slots > C) slots = C;
+  pl.slots = (int)slots;
+  pl.split = HW % pl.elems != 0;
+  pl.part_floats = pl.spans * nsplit * slots * 2;
+  return true;
+}
+int64_t workspace_floats(const Plan& pl, int64_t C) { return pl.part_floats + 3 * C; }
+
+template <typename T, bool BWD, bool MINMAX>
+void launch_reduce(const Plan& pl, const void* x, const void* dy, float* part, void* mn, void* mx,
+                   int64_t N, int64_t HW, hipStream_t s) {
+  const dim3 grid((unsigned)pl.spans, (unsigned)pl.nsplit), blk(kThreads);
+  const size_t lds = (size_t)kWaves * (pl.slots + 1) * 2 * sizeof(float);
+  const T* px = static_cast<const T*>(x);
+  const T* pd = static_cast<const T*>(dy);
+  T* lo = static_cast<T*>(mn);
+  T* hi = static_cast<T*>(mx);
+  if (pl.split)
+    bn_reduce_kernel<T, true, BWD, MINMAX><<<grid, blk, lds, s>>>(px, pd, part, lo, hi, N, pl.F, HW, pl.per_block, pl.slots);
+  else
+    bn_reduce_kernel<T, false, BWD, MINMAX><<<grid, blk, lds, s>>>(px, pd, part, lo, hi, N, pl.F, HW, pl.per_block, pl.slots);
+}
+
+template <typename T, bool BWD>
+void launch_apply(const Plan& pl, const void* x, const void* dy, const float* coef, void* out,
+                  int64_t N, int64_t HW, hipStream_t s) {
+  const dim3 grid((unsigned)pl.spans, (unsigned)pl.nsplit), blk(kThreads);
+  const T* px = static_cast<const T*>(x);
+  const T* pd = static_cast<const T*>(dy);
+  T* po = static_cast<T*>(out);
+  if (pl.split)
+    bn_apply_kernel<T, true, BWD><<<grid, blk, 0, s>>>(px, pd, coef, po, N, pl.F, HW, pl.per_block);
+  else
+    bn_apply_kernel<T, false, BWD><<<grid, blk, 0, s>>>(px, pd, coef, po, N, pl.F, HW, pl.per_block);
+}
+
+template <typename T>
+int forward_t(const Plan& pl, const void* x, const float* weight, const float* bias, float* running_mean,
+              float* running_var, void* y, float* save_mean, float* save_invstd, void* mn, void* mx,
+              float* ws, int64_t N, int64_t C, int64_t HW, double momentum, double eps, hipStream_t s) {
+  float* part = ws;
+  float* coef = ws + pl.part_floats;
+  if (mn) launch_reduce<T, false, true>(pl, x, nullptr, part, mn, mx, N, HW, s);
+  else launch_reduce<T, false, false>(pl, x, nullptr, part, nullptr, nullptr, N, HW, s);
+  bn_forward_finalize_kernel<<<dim3((unsigned)((C + kThreads - 1) / kThreads)), dim3(kThreads), 0, s>>>(
+      part, weight, bias, running_mean, running_var, save_mean, save_invstd, coef, N, C, HW, pl.L,
+      pl.nsplit, pl.slots, momentum, eps);
+  launch_apply<T, false>(pl, x, nullptr, coef, y, N, HW, s);
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
+
+template <typename T>
+int backward_t(const Plan& pl, const void* x, const void* dy, const float* weight, const float* save_mean,
+               const float* save_invstd, void* dx, float* dweight, float* dbias, float* ws, int64_t N,
+               int64_t C, int64_t HW, hipStream_t s) {
+  float* part = ws;
+  float* coef = ws + pl.part_floats;
+  launch_reduce<T, true, false>(pl, x, dy, part, nullptr, nullptr, N, HW, s);
+  bn_backward_finalize_kernel<<<dim3((unsigned)((C + kThreads - 1) / kThreads)), dim3(kThreads), 0, s>>>(
+      part, weight, save_mean, save_invstd, dweight, dbias, coef, N, C, HW, pl.L, pl.nsplit, pl.slots);
+  if (dx) launch_apply<T, true>(pl, x, dy, coef, dx, N, HW, s);
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
+
+}  // namespace
+}  // namespace actnn
+
+extern "C" int64_t actnn_batch_norm_workspace_bytes(int64_t N, int64_t C, int64_t HW, int dtype) {
+  actnn::Plan pl;
+  if (!actnn::make_plan(N, C, HW, dtype, pl)) return -1;
+  return actnn::workspace_floats(pl, C) * (int64_t)sizeof(float);
+}
+
+extern "C" int actnn_batch_norm_forward(const void* x, const float* weight, const float* bias,
+                                        float* running_mean, float* running_var, void* y,
+                                        float* save_mean, float* save_invstd, void* mn, void* mx,
+                                        void* workspace, int64_t workspace_bytes, int64_t N, int64_t C,
+                                        int64_t HW, double momentum, double eps, int dtype, void* stream) {
+  using namespace actnn;
+  if (dtype < 0 || dtype > 2) return ACTNN_EDTYPE;
+  Plan pl;
+  if (!make_plan(N, C, HW, dtype, pl)) return ACTNN_EINVAL;
+  if (!x || !y || !save_mean || !save_invstd || !workspace || (mn == nullptr) != (mx == nullptr)) return ACTNN_EINVAL;
+  if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
+  if (mn && pl.F % 256 != 0) return ACTNN_EINVAL;
+  if (!aligned16(x) || !aligned16(y) || !aligned16(workspace)) return ACTNN_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float* ws = static_cast<float*>(workspace);
+  switch (dtype) {
+    case ACTNN_F32: return forward_t<float>(pl, x, weight, bias, running_mean, running_var, y, save_mean, save_invstd, mn, mx, ws, N, C, HW, momentum, eps, s);
+    case ACTNN_F16: return forward_t<__half>(pl, x, weight, bias, running_mean, running_var, y, save_mean, save_invstd, mn, mx, ws, N, C, HW, momentum, eps, s);
+    default: return forward_t<bf16_t>(pl, x, weight, bias, running_mean, running_var, y, save_mean, save_invstd, mn, mx, ws, N, C, HW, momentum, eps, s);
+  }
+}
+
+extern "C" int actnn_batch_norm_backward(const void* x, const void* dy, const float* weight,
+                                         const float* save_mean, const float* save_invstd, void* dx,
+                                         float* dweight, float* dbias, void* workspace,
+                                         int64_t workspace_bytes, int64_t N, int64_t C, int64_t HW,
+                                         int dtype, void* stream) {
+  using namespace actnn;
+  if (dtype < 0 || dtype > 2) return ACTNN_EDTYPE;
+  Plan pl;
+  if (!make_plan(N, C, HW, dtype, pl)) return ACTNN_EINVAL;
+  if (!x || !dy || !save_mean || !save_invstd || !workspace) return ACTNN_EINVAL;
+  if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
+  if (!aligned16(x) || !aligned16(dy) || (dx && !aligned16(dx)) || !aligned16(workspace)) return ACTNN_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float* ws = static_cast<float*>(workspace);
+  switch (dtype) {
+    case ACTNN_F32: return backward_t<float>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+    case ACTNN_F16: return backward_t<__half>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+    default: return backward_t<bf16_t>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+  }
+}

@@ -1,0 +1,123 @@
+"""The library's training-mode batch norm (actnn_batch_norm_forward / _backward) against the
+float64 restatement and against torch's own batch norm.  Floating point: the tolerances below are
+a few units of the output type's rounding (fp32: 2^-19 of |y| + 4, the rounding of a*x + b on inputs a few standard deviations from a mean of order 1; 16-bit types one
+rounding step of the result, 2^-8 for bf16 and 2^-11 for fp16, plus the fp32 error)."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import actnn_amd.cpp_extension.backward_func as ext_bf
+import actnn_amd.cpp_extension.minimax as ext_minimax
+from oracle import batch_norm as o_bn
+from _util import DEV
+
+pytestmark = pytest.mark.gpu
+
+# (N, C, spatial): ResNet-50 planes (112^2 ... 7^2), channel boundaries inside a 16-byte chunk
+# (49, 196, 12, 10), several spans per channel, one span over many channels, ragged batch splits
+SHAPES = [(8, 64, (112, 112)), (8, 16, (56, 56)), (5, 32, (28, 28)), (37, 24, (14, 14)),
+          (16, 256, (7, 7)), (3, 6, (4, 3)), (9, 4, (10,)), (2, 8, (3, 4, 5)), (70, 8, (8, 8)),
+          (4, 2048, (7, 7)), (1, 8, (16, 16))]
+RND = {torch.float32: 2.0 ** -19, torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}
+
+
+def _inputs(N, C, spatial, dtype, seed):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    x = torch.randn(N, C, *spatial, generator=g, device=DEV)
+    x = x * (0.5 + torch.rand(1, C, *([1] * len(spatial)), generator=g, device=DEV) * 2)
+    x = (x + torch.randn(1, C, *([1] * len(spatial)), generator=g, device=DEV)).to(dtype)
+    w = torch.rand(C, generator=g, device=DEV) + 0.5
+    b = torch.randn(C, generator=g, device=DEV)
+    rm = torch.randn(C, generator=g, device=DEV)
+    rv = torch.rand(C, generator=g, device=DEV) + 0.5
+    dy = torch.randn(N, C, *spatial, generator=g, device=DEV).to(dtype)
+    return x, w, b, rm, rv, dy
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,C,spatial", SHAPES)
+def test_forward_backward_against_float64(N, C, spatial, dtype):
+    x, w, b, rm, rv, dy = _inputs(N, C, spatial, dtype, N * 1000 + C)
+    assert ext_bf.hip_batch_norm_applies(x, w, b, rm, rv)
+    rm0, rv0 = rm.clone(), rv.clone()
+    y, mean, invstd, _ = ext_bf.cudnn_batch_norm(x, w, b, rm, rv, True, 0.1, 1e-5)
+    yo, mean_o, invstd_o, rm_o, rv_o = o_bn.forward(
+        x.double().cpu().numpy(), w.cpu().numpy(), b.cpu().numpy(), rm0.cpu().numpy(), rv0.cpu().numpy(), 0.1, 1e-5)
+    assert y.dtype == dtype and y.shape == x.shape
+    assert np.allclose(mean.cpu().numpy(), mean_o, rtol=1e-5, atol=1e-6)
+    assert np.allclose(invstd.cpu().numpy(), invstd_o, rtol=2e-5)
+    assert np.allclose(rm.cpu().numpy(), rm_o, rtol=1e-5, atol=1e-6)
+    assert np.allclose(rv.cpu().numpy(), rv_o, rtol=2e-5)
+    err = np.abs(y.double().cpu().numpy() - yo)
+    assert (err <= RND[dtype] * (np.abs(yo) + 4.0)).all(), float(err.max())
+
+    gi, gw, gb = ext_bf.cudnn_batch_norm_backward(x, dy, w, rm, rv, mean, invstd, 1e-5, None)
+    gi_o, gw_o, gb_o = o_bn.backward(x.double().cpu().numpy(), dy.double().cpu().numpy(), w.cpu().numpy(), 1e-5)
+    count = x.numel() / C
+    scale = np.sqrt(count)                       # sums of `count` terms of order 1
+    assert np.allclose(gb.cpu().numpy(), gb_o, rtol=1e-5, atol=2e-5 * scale)
+    assert np.allclose(gw.cpu().numpy(), gw_o, rtol=1e-5, atol=4e-5 * scale)
+    err = np.abs(gi.double().cpu().numpy() - gi_o)
+    assert (err <= RND[dtype] * (np.abs(gi_o) + 4.0)).all(), float(err.max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_against_torch_batch_norm_and_autograd(dtype):
+    x, w, b, rm, rv, dy = _inputs(16, 64, (28, 28), dtype, 5)
+    rm_t, rv_t = rm.clone(), rv.clone()
+    xt = x.clone().requires_grad_(True)
+    wt, bt = w.clone().requires_grad_(True), b.clone().requires_grad_(True)
+    yt = F.batch_norm(xt, rm_t, rv_t, wt, bt, True, 0.1, 1e-5)
+    yt.backward(dy)
+    y, mean, invstd, _ = ext_bf.cudnn_batch_norm(x, w, b, rm, rv, True, 0.1, 1e-5)
+    gi, gw, gb = ext_bf.cudnn_batch_norm_backward(x, dy, w, rm, rv, mean, invstd, 1e-5, None)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert torch.allclose(y.float(), yt.float(), rtol=tol, atol=tol)
+    assert torch.allclose(rm, rm_t, rtol=1e-5, atol=1e-6) and torch.allclose(rv, rv_t, rtol=1e-5)
+    assert torch.allclose(gi.float(), xt.grad.float(), rtol=tol, atol=tol)
+    assert torch.allclose(gw, wt.grad, rtol=1e-3, atol=1e-2) and torch.allclose(gb, bt.grad, rtol=1e-3, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,C,spatial", [(8, 64, (56, 56)), (5, 256, (7, 7)), (9, 64, (14, 14)), (3, 8, (8, 4))])
+def test_group_min_max_from_the_statistics_pass(N, C, spatial, dtype):
+    x, w, b, rm, rv, _ = _inputs(N, C, spatial, dtype, 11)
+    y0, m0, i0, _, _ = ext_bf.hip_batch_norm_forward(x, w, b, rm.clone(), rv.clone(), 0.1, 1e-5)
+    y, m, i, mn, mx = ext_bf.hip_batch_norm_forward(x, w, b, rm.clone(), rv.clone(), 0.1, 1e-5, minmax=True)
+    mn_ref, mx_ref = ext_minimax.minimax(x.view(-1, 256))
+    assert torch.equal(mn, mn_ref.view(-1)) and torch.equal(mx, mx_ref.view(-1))
+    assert torch.equal(y, y0) and torch.equal(m, m0) and torch.equal(i, i0)     # and nothing else changes
+
+
+def test_results_do_not_depend_on_the_schedule():
+    x, w, b, rm, rv, dy = _inputs(64, 128, (14, 14), torch.bfloat16, 3)
+    first = None
+    for _ in range(3):
+        y, mean, invstd, _, _ = ext_bf.hip_batch_norm_forward(x, w, b, None, None, 0.1, 1e-5)
+        gi, gw, gb = ext_bf.hip_batch_norm_backward(x, dy, w, mean, invstd)
+        cur = (y, mean, invstd, gi, gw, gb)
+        if first is None:
+            first = cur
+        else:
+            assert all(torch.equal(a, c) for a, c in zip(first, cur))
+
+
+def test_no_affine_no_running_stats_and_fallback_shapes():
+    x, _, _, _, _, dy = _inputs(6, 16, (8, 8), torch.float32, 4)
+    y, mean, invstd, _ = ext_bf.cudnn_batch_norm(x, None, None, None, None, True, 0.1, 1e-5)
+    yo, mean_o, invstd_o, _, _ = o_bn.forward(x.double().cpu().numpy(), None, None, None, None, 0.1, 1e-5)
+    assert np.allclose(y.cpu().numpy(), yo, rtol=1e-5, atol=1e-5)
+    gi, gw, gb = ext_bf.cudnn_batch_norm_backward(x, dy, None, None, None, mean, invstd, 1e-5, None)
+    gi_o, _, gb_o = o_bn.backward(x.double().cpu().numpy(), dy.double().cpu().numpy(), None, 1e-5)
+    assert np.allclose(gi.cpu().numpy(), gi_o, rtol=1e-4, atol=1e-5)
+    # shapes the kernels do not take ([N, C] rows, C*HW not a multiple of the chunk) go to ATen
+    for shape in ((32, 10), (4, 3, 7, 7)):
+        xs = torch.randn(*shape, device=DEV)
+        assert not ext_bf.hip_batch_norm_applies(xs, None, None, None, None)
+        w = torch.ones(shape[1], device=DEV)
+        b = torch.zeros(shape[1], device=DEV)
+        rm, rv = torch.zeros(shape[1], device=DEV), torch.ones(shape[1], device=DEV)
+        ys = ext_bf.cudnn_batch_norm(xs, w, b, rm, rv, True, 0.1, 1e-5)[0]
+        ref = o_bn.forward(xs.double().cpu().numpy(), None, None, None, None, 0.1, 1e-5)[0]
+        assert np.allclose(ys.cpu().numpy(), ref, rtol=1e-4, atol=1e-4)
