@@ -58,11 +58,11 @@ def dequantize_and_unpack(data, shape, bits, scale, mn):
     return unpack(data, bits, scale, mn, N, features // gs, gs)
 
 
-def no_scheme_compute_quantization_bits(input):
+def no_scheme_compute_quantization_bits(input, known_minmax=None):
     """Fixed width for every sample when no scheme is attached (ops.py:77-96)."""
     from .qscheme import group_min_max
     N = input.shape[0]
-    groups, mn, mx, _ = group_min_max(input)
+    groups, mn, mx, _ = group_min_max(input, known_minmax)
     return groups, config.activation_compression_bits[0], mn.view(N, -1, 1), mx.view(N, -1, 1)
 
 
@@ -72,15 +72,16 @@ def quantize_activation(input, scheme):
     return finish_quantize(start_quantize(input, scheme))
 
 
-def start_quantize(input, scheme):
+def start_quantize(input, scheme, known_minmax=None):
     """First half of quantize_activation: everything up to the point where the per-sample widths
     are needed on the host.  The caller may launch other GPU work (the layer's forward) before
-    calling finish_quantize, which hides the device->host round trip of the allocation."""
+    calling finish_quantize, which hides the device->host round trip of the allocation.
+    `known_minmax`: per-group (mn, mx) of `input` when another kernel has produced them already."""
     if not config.compress_activation:
         return ("raw", input)
     if scheme:
-        return ("scheme", input.dtype, scheme, scheme.start_quantization_bits(input))
-    return ("fixed", input.dtype, no_scheme_compute_quantization_bits(input))
+        return ("scheme", input.dtype, scheme, scheme.start_quantization_bits(input, known_minmax))
+    return ("fixed", input.dtype, no_scheme_compute_quantization_bits(input, known_minmax))
 
 
 def finish_quantize(started):
@@ -289,15 +290,30 @@ class linear(Function):
 # ------------------------------------------------------------------------------------------
 # batch norm (ops.py:436-502)
 # ------------------------------------------------------------------------------------------
+def _bn_shares_min_max(input, weight, bias, running_mean, running_var, training):
+    features = input.numel() // max(input.shape[0], 1)
+    return (training and config.compress_activation and not config.simulate
+            and config.group_size == 256 and features % 256 == 0
+            and ext_backward_func.hip_batch_norm_applies(input, weight, bias, running_mean, running_var))
+
+
 class batch_norm(Function):
     @staticmethod
     def forward(ctx, input, running_mean, running_var, weight, bias, training,
                 exponential_average_factor, eps, scheme):
-        started = start_quantize(input, scheme)
-        if training:
+        if _bn_shares_min_max(input, weight, bias, running_mean, running_var, training):
+            # the statistics pass of the library's batch norm also yields the per-group min/max
+            # the quantiser needs: one read of the input less
+            output, save_mean, save_var, mn, mx = ext_backward_func.hip_batch_norm_forward(
+                input, weight, bias, running_mean, running_var, exponential_average_factor, eps, minmax=True)
+            reserve = None
+            started = start_quantize(input, scheme, (mn, mx))
+        elif training:
+            started = start_quantize(input, scheme)
             output, save_mean, save_var, reserve = ext_backward_func.cudnn_batch_norm(
                 input, weight, bias, running_mean, running_var, training, exponential_average_factor, eps)
         else:
+            started = start_quantize(input, scheme)
             output, save_mean, save_var = ext_backward_func.native_batch_norm(
                 input, weight, bias, running_mean, running_var, training, exponential_average_factor, eps)
             reserve = None

@@ -16,10 +16,10 @@ class QBNScheme(QScheme):
         QBNScheme.layers.append(self)
         self.prev_linear = QScheme.layers[-1] if len(QScheme.layers) > 0 else None
 
-    def start_quantization_bits(self, input):
+    def start_quantization_bits(self, input, known_minmax=None):
         self.prev_linear = QScheme.prev_layer
         N = input.shape[0]
-        groups, mn, mx, num_pixels = group_min_max(input)
+        groups, mn, mx, num_pixels = group_min_max(input, known_minmax)
         C_dev = range_sqr(mn, mx, N, num_pixels)                           # qbnscheme.py:44-47
         if allocate_on_device(N, self.initial_bits):
             return groups, mn, mx, None, input.numel() // N, greedy_bits_device(C_dev, N, self.initial_bits, self.bits)

@@ -14,10 +14,11 @@ from .cpp_extension import minimax as ext_minimax
 from .cpp_extension.quantization import attach_bits_host, attach_bits_total
 
 
-def group_min_max(input):
+def group_min_max(input, known=None):
     """Flatten to [N, -1], zero-pad the feature axis to a multiple of group_size, view as groups
     and reduce each group (qscheme.py:59-74).  Returns (groups [N,G,gs], mn [N*G], mx [N*G],
-    pixels per channel)."""
+    pixels per channel).  `known` = (mn, mx) already produced by another pass over the same
+    tensor (the batch-norm statistics kernel); only given when no padding is needed."""
     N = input.shape[0]
     flat = input.reshape(N, -1)
     features = flat.shape[1]
@@ -29,7 +30,7 @@ def group_min_max(input):
     elif not flat.is_contiguous():
         flat = flat.contiguous()
     rows = flat.view(-1, gs)
-    mn, mx = ext_minimax.minimax(rows)
+    mn, mx = known if known is not None else ext_minimax.minimax(rows)
     if not config.pergroup:                     # one range for the whole tensor (qscheme.py:75-77)
         mn = torch.ones_like(mn) * mn.min()
         mx = torch.ones_like(mx) * mx.max()
@@ -169,11 +170,11 @@ class QScheme(_LazyHost):
         """-> (groups [N,G,gs], bits on device, mn [N,G,1], mx [N,G,1])  (qscheme.py:57-94)."""
         return self.finish_quantization_bits(self.start_quantization_bits(input))
 
-    def start_quantization_bits(self, input):
+    def start_quantization_bits(self, input, known_minmax=None):
         """First half: min/max kernel, sensitivities, asynchronous copy to the host."""
         QScheme.prev_layer = self
         N = input.shape[0]
-        groups, mn, mx, num_pixels = group_min_max(input)
+        groups, mn, mx, num_pixels = group_min_max(input, known_minmax)
         C_dev = self.sensitivity(mn, mx, N, num_pixels)
         bits_dev = None
         if allocate_on_device(N, self.initial_bits):
