@@ -13,16 +13,23 @@ from . import _glue
 _aten = torch.ops.aten
 
 
-def _bn_geometry(input):
-    """(N, C, HW) when the library's batch-norm kernels take this tensor, else None."""
-    if not (isinstance(input, torch.Tensor) and input.is_cuda and input.dim() >= 2
-            and input.dtype in _glue.DTYPE_CODE and input.is_contiguous() and input.numel() > 0):
+def _shape_geometry(shape, dtype):
+    """(N, C, HW) when the library's batch-norm kernels take a tensor of this shape, else None."""
+    if len(shape) < 2 or dtype not in _glue.DTYPE_CODE:
         return None
-    N, C = input.shape[0], input.shape[1]
-    HW = input.numel() // (N * C)
-    if _glue.lib().actnn_batch_norm_workspace_bytes(N, C, HW, _glue.DTYPE_CODE[input.dtype]) < 0:
+    N, C = int(shape[0]), int(shape[1])
+    HW = 1
+    for d in shape[2:]:
+        HW *= int(d)
+    if N * C * HW == 0 or _glue.lib().actnn_batch_norm_workspace_bytes(N, C, HW, _glue.DTYPE_CODE[dtype]) < 0:
         return None
     return N, C, HW
+
+
+def _bn_geometry(input):
+    if not (isinstance(input, torch.Tensor) and input.is_cuda and input.is_contiguous()):
+        return None
+    return _shape_geometry(input.shape, input.dtype)
 
 
 def _f32_or_none(t):
@@ -55,11 +62,12 @@ def hip_batch_norm_forward(input, weight, bias, running_mean, running_var, momen
         groups = N * C * HW // 256
         mn = torch.empty(groups, dtype=input.dtype, device=input.device)
         mx = torch.empty(groups, dtype=input.dtype, device=input.device)
-    _glue._lib.check(lib.actnn_batch_norm_forward(
-        input.data_ptr(), _ptr(weight), _ptr(bias), _ptr(running_mean), _ptr(running_var),
-        out.data_ptr(), save_mean.data_ptr(), save_invstd.data_ptr(), _ptr(mn), _ptr(mx),
-        ws.data_ptr(), ws_bytes, N, C, HW, float(momentum), float(eps), code,
-        _glue.stream_ptr(input.device)), "batch_norm_forward")
+    with torch.cuda.device(input.device):
+        _glue._lib.check(lib.actnn_batch_norm_forward(
+            input.data_ptr(), _ptr(weight), _ptr(bias), _ptr(running_mean), _ptr(running_var),
+            out.data_ptr(), save_mean.data_ptr(), save_invstd.data_ptr(), _ptr(mn), _ptr(mx),
+            ws.data_ptr(), ws_bytes, N, C, HW, float(momentum), float(eps), code,
+            _glue.stream_ptr(input.device)), "batch_norm_forward")
     return out, save_mean, save_invstd, mn, mx
 
 
@@ -73,10 +81,52 @@ def hip_batch_norm_backward(input, grad_output, weight, save_mean, save_invstd):
     grad_input = torch.empty_like(input)
     grad_weight = torch.empty(C, dtype=torch.float32, device=input.device)
     grad_bias = torch.empty(C, dtype=torch.float32, device=input.device)
-    _glue._lib.check(lib.actnn_batch_norm_backward(
-        input.data_ptr(), grad_output.data_ptr(), _ptr(weight), save_mean.data_ptr(),
-        save_invstd.data_ptr(), grad_input.data_ptr(), grad_weight.data_ptr(), grad_bias.data_ptr(),
-        ws.data_ptr(), ws_bytes, N, C, HW, code, _glue.stream_ptr(input.device)), "batch_norm_backward")
+    with torch.cuda.device(input.device):
+        _glue._lib.check(lib.actnn_batch_norm_backward(
+            input.data_ptr(), grad_output.data_ptr(), _ptr(weight), save_mean.data_ptr(),
+            save_invstd.data_ptr(), grad_input.data_ptr(), grad_weight.data_ptr(), grad_bias.data_ptr(),
+            ws.data_ptr(), ws_bytes, N, C, HW, code, _glue.stream_ptr(input.device)), "batch_norm_backward")
+    return grad_input, grad_weight, grad_bias
+
+
+def hip_batch_norm_backward_packed_applies(shape, quantized, grad_output, weight, save_mean, save_invstd):
+    """True when the batch-norm backward kernels can read the saved input straight from its
+    mixed-precision stream: 16-bit activation with scale/min in its own dtype, whole groups of 256."""
+    q_input, q_bits, q_scale, q_min = quantized
+    dtype = grad_output.dtype
+    geo = _shape_geometry(shape, dtype)
+    return (geo is not None and dtype in (torch.float16, torch.bfloat16)
+            and (geo[1] * geo[2]) % 256 == 0 and isinstance(q_bits, torch.Tensor)
+            and isinstance(q_input, torch.Tensor) and q_input.is_cuda and q_input.dtype == torch.int32
+            and q_scale.dtype == dtype and q_min.dtype == dtype
+            and q_scale.is_contiguous() and q_min.is_contiguous()
+            and tuple(grad_output.shape) == tuple(shape) and grad_output.is_contiguous()
+            and grad_output.data_ptr() % 16 == 0
+            and all(_f32_or_none(t) for t in (weight, save_mean, save_invstd)))
+
+
+def hip_batch_norm_backward_packed(shape, quantized, grad_output, weight, save_mean, save_invstd):
+    """-> (grad_input, grad_weight, grad_bias); the saved input is decoded inside the kernels."""
+    from .quantization import _bits_info
+    q_input, q_bits, q_scale, q_min = quantized
+    N, C, HW = _shape_geometry(shape, grad_output.dtype)
+    lib = _glue.lib()
+    code = _glue.DTYPE_CODE[grad_output.dtype]
+    total, prefix = _bits_info(q_bits)
+    if q_input.numel() < total * (C * HW // 256) * 8:
+        raise RuntimeError("batch_norm_backward_packed: packed stream is too short")
+    ws_bytes = lib.actnn_batch_norm_workspace_bytes(N, C, HW, code)
+    dev = grad_output.device
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dev)
+    grad_input = torch.empty_like(grad_output)
+    grad_weight = torch.empty(C, dtype=torch.float32, device=dev)
+    grad_bias = torch.empty(C, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _glue._lib.check(lib.actnn_batch_norm_backward_packed(
+            q_input.data_ptr(), q_bits.data_ptr(), prefix.data_ptr(), q_scale.data_ptr(), q_min.data_ptr(),
+            grad_output.data_ptr(), _ptr(weight), save_mean.data_ptr(), save_invstd.data_ptr(),
+            grad_input.data_ptr(), grad_weight.data_ptr(), grad_bias.data_ptr(), ws.data_ptr(), ws_bytes,
+            N, C, HW, code, _glue.stream_ptr(dev)), "batch_norm_backward_packed")
     return grad_input, grad_weight, grad_bias
 
 

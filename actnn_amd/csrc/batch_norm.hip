@@ -17,6 +17,7 @@
 // quantiser (groups of 256 consecutive elements of the row) from the registers it already holds,
 // which saves the quantiser's own read of the tensor.
 #include "device_utils.h"
+#include "quant_math.h"
 
 namespace actnn {
 namespace {
@@ -146,15 +147,85 @@ ACTNN_DEV void fold_block(float* s_acc, int slots, const Place& p, int64_t first
   }
 }
 
+// Where the input x of the backward passes comes from.  Both sources hand out the chunk of this
+// thread for sample n in two steps, so that the loads of several samples can be in flight before
+// the first one is used.
+template <typename T> struct PlainInput {
+  const T* p;            // already offset to the thread's chunk of sample 0
+  int64_t F;
+  struct Raw { u32x4 v; };
+  ACTNN_DEV Raw fetch(int64_t n) const { return Raw{load16(p + n * F)}; }
+  ACTNN_DEV u32x4 decode(const Raw& r) const { return r.v; }
+};
+
+// x kept as the mixed-precision bit stream of the activation quantiser (pack_mixed layout: sample
+// n owns bits[n] * G * 8 words from prefix[n] * G * 8 on; in a group of 256 elements bit i of the
+// code of element 8j + k is bit j of word k * bits + i).  The 32 lanes that own a group here are
+// the 32 lanes of that layout - lane j holds elements 8j .. 8j+7 - so a half-wave loads the group's
+// words, transposes them (32x32 bits) and every lane finds its 8 codes in its own register.
+// Values are rebuilt exactly as actnn_unpack_mixed rebuilds them.  16-bit types only.
+template <typename T> struct PackedInput {
+  const int32_t* words;
+  const int32_t* bits;
+  const int32_t* prefix;
+  const T* scale;
+  const T* mn;
+  int64_t G, g;          // groups per sample, this thread's group
+  uint32_t lane32;
+  bool active;
+  struct Raw { uint32_t lo, hi; float sc, m; int b; };
+  ACTNN_DEV Raw fetch(int64_t n) const {
+    Raw r{0u, 0u, 1.0f, 0.0f, 1};
+    if (active) {
+      r.b = bits[n];
+      const int32_t* w = words + ((int64_t)prefix[n] * G + g * r.b) * 8;
+      if ((int)lane32 < 8 * r.b) r.lo = (uint32_t)w[lane32];
+      if ((int)lane32 + 32 < 8 * r.b) r.hi = (uint32_t)w[lane32 + 32];
+      r.sc = Conv<T>::load(scale, n * G + g);
+      r.m = Conv<T>::load(mn, n * G + g);
+    }
+    return r;
+  }
+  template <int BITS> ACTNN_DEV u32x4 decode_bits(const Raw& r) const {
+    uint64_t acc = transpose32(r.lo, lane32);
+    if (BITS > 4) acc |= (uint64_t)transpose32(r.hi, lane32) << 32;
+    const Dequant<T> dq(r.sc, r.m);
+    float v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = dq((uint32_t)(acc >> (k * BITS)) & ((1u << BITS) - 1u));
+    return u32x4{Chunk<T>::narrow(v), Chunk<T>::narrow(v + 2), Chunk<T>::narrow(v + 4), Chunk<T>::narrow(v + 6)};
+  }
+  ACTNN_DEV u32x4 decode(const Raw& r) const {
+    switch (r.b) {                       // uniform over the block: one sample, one width
+      case 1: return decode_bits<1>(r);
+      case 2: return decode_bits<2>(r);
+      case 3: return decode_bits<3>(r);
+      case 4: return decode_bits<4>(r);
+      case 5: return decode_bits<5>(r);
+      case 6: return decode_bits<6>(r);
+      case 7: return decode_bits<7>(r);
+      default: return decode_bits<8>(r);
+    }
+  }
+};
+
+template <typename T> ACTNN_DEV void bind_input(PlainInput<T>& xs, const Place& p) { xs.p += p.elem; }
+template <typename T> ACTNN_DEV void bind_input(PackedInput<T>& xs, const Place& p) {
+  xs.g = p.elem >> 8;
+  xs.lane32 = threadIdx.x & 31;
+  xs.active = p.active;
+}
+
 // Pass 1 of either direction.  Forward: per-channel sum(x) and sum(x*x) (+ per-group min/max of
 // x when MINMAX).  Backward: per-channel sum(dy) and sum(x*dy).
-template <typename T, bool SPLIT, bool BWD, bool MINMAX>
+template <typename T, bool SPLIT, bool BWD, bool MINMAX, typename XS>
 __global__ __launch_bounds__(kThreads) void bn_reduce_kernel(
-    const T* __restrict__ x, const T* __restrict__ dy, float* __restrict__ part,
+    XS xs, const T* __restrict__ dy, float* __restrict__ part,
     T* __restrict__ mn, T* __restrict__ mx, int64_t N, int64_t F, int64_t HW, int per_block, int slots) {
   constexpr int E = Chunk<T>::kElems;
   extern __shared__ float s_acc[];
   const Place p = place_of<E>(F, HW);
+  bind_input(xs, p);
   uint32_t m[4];
   head_masks<T>(p.head, m);
   const int64_t n0 = (int64_t)blockIdx.y * per_block;
@@ -194,46 +265,53 @@ __global__ __launch_bounds__(kThreads) void bn_reduce_kernel(
     }
   };
 
-  const T* px = x + n0 * F + p.elem;
-  const T* pd = BWD ? dy + n0 * F + p.elem : nullptr;
+  const T* pd = BWD ? dy + p.elem : nullptr;
   int64_t n = n0;
   for (; n + kUnroll <= n1; n += kUnroll) {
-    u32x4 ux[kUnroll], ud[kUnroll];
+    typename XS::Raw rx[kUnroll];
+    u32x4 ud[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
-      ux[u] = load16(px + u * F);
-      ud[u] = BWD ? load16(pd + u * F) : ux[u];
+      rx[u] = xs.fetch(n + u);
+      if (BWD) ud[u] = load16(pd + (n + u) * F);
     }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) accumulate(ux[u], ud[u], n + u);
-    px += kUnroll * F;
-    if (BWD) pd += kUnroll * F;
+    for (int u = 0; u < kUnroll; ++u) {
+      const u32x4 ux = xs.decode(rx[u]);
+      accumulate(ux, BWD ? ud[u] : ux, n + u);
+    }
   }
   for (; n < n1; ++n) {
-    const u32x4 ux = load16(px);
-    const u32x4 ud = BWD ? load16(pd) : ux;
-    accumulate(ux, ud, n);
-    px += F;
-    if (BWD) pd += F;
+    const typename XS::Raw rx = xs.fetch(n);
+    const u32x4 ux = xs.decode(rx);
+    accumulate(ux, BWD ? load16(pd + n * F) : ux, n);
   }
   const int64_t first_channel = ((int64_t)blockIdx.x * kThreads * E) / HW;
   fold_block<E>(s_acc, slots, p, first_channel, SPLIT ? h0 : t0, SPLIT ? h1 : t1,
                 SPLIT ? t0 - h0 : 0.0f, SPLIT ? t1 - h1 : 0.0f, part);
 }
 
-// Folds the table of partial sums of channel c in double precision, in a fixed order.
+// Folds the table of partial sums of channel c in double precision: the wave's lanes take the
+// (span, batch split) entries of the channel in a fixed assignment and are combined by a butterfly,
+// so every lane ends with the same totals and the order of the additions is fixed.
 ACTNN_DEV void channel_totals(const float* __restrict__ part, int64_t c, int64_t HW, int64_t L,
                               int nsplit, int slots, double& s0, double& s1) {
+  const int lane = threadIdx.x & 63;
   const int64_t j0 = (c * HW) / L, j1 = ((c + 1) * HW - 1) / L;
+  const int64_t count = (j1 - j0 + 1) * nsplit;
   s0 = 0.0;
   s1 = 0.0;
-  for (int64_t j = j0; j <= j1; ++j) {
+  for (int64_t i = lane; i < count; i += 64) {
+    const int64_t j = j0 + i / nsplit, y = i % nsplit;
     const int64_t slot = c - (j * L) / HW;
-    const float* q = part + ((j * nsplit) * slots + slot) * 2;
-    for (int y = 0; y < nsplit; ++y, q += (int64_t)slots * 2) {
-      s0 += (double)q[0];
-      s1 += (double)q[1];
-    }
+    const float* q = part + ((j * nsplit + y) * slots + slot) * 2;
+    s0 += (double)q[0];
+    s1 += (double)q[1];
+  }
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) {
+    s0 += __shfl_xor(s0, d);
+    s1 += __shfl_xor(s1, d);
   }
 }
 
@@ -244,10 +322,11 @@ __global__ __launch_bounds__(kThreads) void bn_forward_finalize_kernel(
     float* __restrict__ running_mean, float* __restrict__ running_var, float* __restrict__ save_mean,
     float* __restrict__ save_invstd, float* __restrict__ coef, int64_t N, int64_t C, int64_t HW,
     int64_t L, int nsplit, int slots, double momentum, double eps) {
-  const int64_t c = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const int64_t c = (int64_t)blockIdx.x * kWaves + (threadIdx.x >> 6);     // one wave per channel
   if (c >= C) return;
   double S, Q;
   channel_totals(part, c, HW, L, nsplit, slots, S, Q);
+  if ((threadIdx.x & 63) != 0) return;
   const double M = (double)N * (double)HW;
   const double mean = S / M;
   double var = Q / M - mean * mean;
@@ -271,10 +350,11 @@ __global__ __launch_bounds__(kThreads) void bn_backward_finalize_kernel(
     const float* __restrict__ part, const float* __restrict__ weight, const float* __restrict__ save_mean,
     const float* __restrict__ save_invstd, float* __restrict__ dweight, float* __restrict__ dbias,
     float* __restrict__ coef, int64_t N, int64_t C, int64_t HW, int64_t L, int nsplit, int slots) {
-  const int64_t c = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const int64_t c = (int64_t)blockIdx.x * kWaves + (threadIdx.x >> 6);     // one wave per channel
   if (c >= C) return;
   double S, Q;                                   // sum(dy), sum(x*dy)
   channel_totals(part, c, HW, L, nsplit, slots, S, Q);
+  if ((threadIdx.x & 63) != 0) return;
   const double M = (double)N * (double)HW;
   const double mean = save_mean[c], r = save_invstd[c];
   const double w = weight ? (double)weight[c] : 1.0;
@@ -289,15 +369,16 @@ __global__ __launch_bounds__(kThreads) void bn_backward_finalize_kernel(
 }
 
 // Pass 2 of either direction.  Forward: y = a*x + b.  Backward: dx = A*dy + B*x + K.
-template <typename T, bool SPLIT, bool BWD>
+template <typename T, bool SPLIT, bool BWD, typename XS>
 __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
-    const T* __restrict__ x, const T* __restrict__ dy, const float* __restrict__ coef,
+    XS xs, const T* __restrict__ dy, const float* __restrict__ coef,
     T* __restrict__ out, int64_t N, int64_t F, int64_t HW, int per_block) {
   constexpr int E = Chunk<T>::kElems;
   constexpr int PD = Chunk<T>::kPerDword;
   constexpr int NC = BWD ? 3 : 2;
   const Place p = place_of<E>(F, HW);
-  if (!p.active) return;
+  if (!p.active) return;               // whole quantisation groups (32 lanes) leave together
+  bind_input(xs, p);
   float k0[NC], k1[NC];
 #pragma unroll
   for (int i = 0; i < NC; ++i) {
@@ -334,30 +415,27 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
     return u32x4{r[0], r[1], r[2], r[3]};
   };
 
-  const T* px = x + n0 * F + p.elem;
-  const T* pd = BWD ? dy + n0 * F + p.elem : nullptr;
-  T* po = out + n0 * F + p.elem;
+  const T* pd = BWD ? dy + p.elem : nullptr;
+  T* po = out + p.elem;
   int64_t n = n0;
   for (; n + kUnroll <= n1; n += kUnroll) {
-    u32x4 ux[kUnroll], ud[kUnroll];
+    typename XS::Raw rx[kUnroll];
+    u32x4 ud[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
-      ux[u] = load16(px + u * F);
-      ud[u] = BWD ? load16(pd + u * F) : ux[u];
+      rx[u] = xs.fetch(n + u);
+      if (BWD) ud[u] = load16(pd + (n + u) * F);
     }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) store16(po + u * F, apply(ux[u], ud[u]));
-    px += kUnroll * F;
-    po += kUnroll * F;
-    if (BWD) pd += kUnroll * F;
+    for (int u = 0; u < kUnroll; ++u) {
+      const u32x4 ux = xs.decode(rx[u]);
+      store16(po + (n + u) * F, apply(ux, BWD ? ud[u] : ux));
+    }
   }
   for (; n < n1; ++n) {
-    const u32x4 ux = load16(px);
-    const u32x4 ud = BWD ? load16(pd) : ux;
-    store16(po, apply(ux, ud));
-    px += F;
-    po += F;
-    if (BWD) pd += F;
+    const typename XS::Raw rx = xs.fetch(n);
+    const u32x4 ux = xs.decode(rx);
+    store16(po + n * F, apply(ux, BWD ? load16(pd + n * F) : ux));
   }
 }
 
@@ -372,7 +450,7 @@ struct Plan {
 bool make_plan(int64_t N, int64_t C, int64_t HW, int dtype, Plan& pl) {
   if (N <= 0 || C <= 0 || HW <= 0 || dtype < 0 || dtype > 2) return false;
   pl.elems = dtype == ACTNN_F32 ? 4 : 8;
-  if (HW < pl.elems || C > ((int64_t)1 << 40) / HW) return false;
+  if (HW < pl.elems || C > 0x7fffffffLL || C > ((int64_t)1 << 40) / HW) return false;
   pl.F = C * HW;
   if (pl.F % pl.elems != 0 || N > ((int64_t)1 << 62) / pl.F) return false;
   pl.L = (int64_t)kThreads * pl.elems;
@@ -396,32 +474,30 @@ bool make_plan(int64_t N, int64_t C, int64_t HW, int dtype, Plan& pl) {
 }
 int64_t workspace_floats(const Plan& pl, int64_t C) { return pl.part_floats + 3 * C; }
 
-template <typename T, bool BWD, bool MINMAX>
-void launch_reduce(const Plan& pl, const void* x, const void* dy, float* part, void* mn, void* mx,
+template <typename T, bool BWD, bool MINMAX, typename XS>
+void launch_reduce(const Plan& pl, const XS& xs, const void* dy, float* part, void* mn, void* mx,
                    int64_t N, int64_t HW, hipStream_t s) {
   const dim3 grid((unsigned)pl.spans, (unsigned)pl.nsplit), blk(kThreads);
   const size_t lds = (size_t)kWaves * (pl.slots + 1) * 2 * sizeof(float);
-  const T* px = static_cast<const T*>(x);
   const T* pd = static_cast<const T*>(dy);
   T* lo = static_cast<T*>(mn);
   T* hi = static_cast<T*>(mx);
   if (pl.split)
-    bn_reduce_kernel<T, true, BWD, MINMAX><<<grid, blk, lds, s>>>(px, pd, part, lo, hi, N, pl.F, HW, pl.per_block, pl.slots);
+    bn_reduce_kernel<T, true, BWD, MINMAX, XS><<<grid, blk, lds, s>>>(xs, pd, part, lo, hi, N, pl.F, HW, pl.per_block, pl.slots);
   else
-    bn_reduce_kernel<T, false, BWD, MINMAX><<<grid, blk, lds, s>>>(px, pd, part, lo, hi, N, pl.F, HW, pl.per_block, pl.slots);
+    bn_reduce_kernel<T, false, BWD, MINMAX, XS><<<grid, blk, lds, s>>>(xs, pd, part, lo, hi, N, pl.F, HW, pl.per_block, pl.slots);
 }
 
-template <typename T, bool BWD>
-void launch_apply(const Plan& pl, const void* x, const void* dy, const float* coef, void* out,
+template <typename T, bool BWD, typename XS>
+void launch_apply(const Plan& pl, const XS& xs, const void* dy, const float* coef, void* out,
                   int64_t N, int64_t HW, hipStream_t s) {
   const dim3 grid((unsigned)pl.spans, (unsigned)pl.nsplit), blk(kThreads);
-  const T* px = static_cast<const T*>(x);
   const T* pd = static_cast<const T*>(dy);
   T* po = static_cast<T*>(out);
   if (pl.split)
-    bn_apply_kernel<T, true, BWD><<<grid, blk, 0, s>>>(px, pd, coef, po, N, pl.F, HW, pl.per_block);
+    bn_apply_kernel<T, true, BWD, XS><<<grid, blk, 0, s>>>(xs, pd, coef, po, N, pl.F, HW, pl.per_block);
   else
-    bn_apply_kernel<T, false, BWD><<<grid, blk, 0, s>>>(px, pd, coef, po, N, pl.F, HW, pl.per_block);
+    bn_apply_kernel<T, false, BWD, XS><<<grid, blk, 0, s>>>(xs, pd, coef, po, N, pl.F, HW, pl.per_block);
 }
 
 template <typename T>
@@ -430,26 +506,45 @@ int forward_t(const Plan& pl, const void* x, const float* weight, const float* b
               float* ws, int64_t N, int64_t C, int64_t HW, double momentum, double eps, hipStream_t s) {
   float* part = ws;
   float* coef = ws + pl.part_floats;
-  if (mn) launch_reduce<T, false, true>(pl, x, nullptr, part, mn, mx, N, HW, s);
-  else launch_reduce<T, false, false>(pl, x, nullptr, part, nullptr, nullptr, N, HW, s);
-  bn_forward_finalize_kernel<<<dim3((unsigned)((C + kThreads - 1) / kThreads)), dim3(kThreads), 0, s>>>(
+  const PlainInput<T> xs{static_cast<const T*>(x), pl.F};
+  if (mn) launch_reduce<T, false, true>(pl, xs, nullptr, part, mn, mx, N, HW, s);
+  else launch_reduce<T, false, false>(pl, xs, nullptr, part, nullptr, nullptr, N, HW, s);
+  bn_forward_finalize_kernel<<<dim3((unsigned)((C + kWaves - 1) / kWaves)), dim3(kThreads), 0, s>>>(
       part, weight, bias, running_mean, running_var, save_mean, save_invstd, coef, N, C, HW, pl.L,
       pl.nsplit, pl.slots, momentum, eps);
-  launch_apply<T, false>(pl, x, nullptr, coef, y, N, HW, s);
+  launch_apply<T, false>(pl, xs, nullptr, coef, y, N, HW, s);
   ACTNN_RETURN_LAUNCH_STATUS();
 }
 
-template <typename T>
-int backward_t(const Plan& pl, const void* x, const void* dy, const float* weight, const float* save_mean,
+template <typename T, typename XS>
+int backward_t(const Plan& pl, const XS& xs, const void* dy, const float* weight, const float* save_mean,
                const float* save_invstd, void* dx, float* dweight, float* dbias, float* ws, int64_t N,
                int64_t C, int64_t HW, hipStream_t s) {
   float* part = ws;
   float* coef = ws + pl.part_floats;
-  launch_reduce<T, true, false>(pl, x, dy, part, nullptr, nullptr, N, HW, s);
-  bn_backward_finalize_kernel<<<dim3((unsigned)((C + kThreads - 1) / kThreads)), dim3(kThreads), 0, s>>>(
+  launch_reduce<T, true, false>(pl, xs, dy, part, nullptr, nullptr, N, HW, s);
+  bn_backward_finalize_kernel<<<dim3((unsigned)((C + kWaves - 1) / kWaves)), dim3(kThreads), 0, s>>>(
       part, weight, save_mean, save_invstd, dweight, dbias, coef, N, C, HW, pl.L, pl.nsplit, pl.slots);
-  if (dx) launch_apply<T, true>(pl, x, dy, coef, dx, N, HW, s);
+  if (dx) launch_apply<T, true>(pl, xs, dy, coef, dx, N, HW, s);
   ACTNN_RETURN_LAUNCH_STATUS();
+}
+
+template <typename T>
+int backward_plain(const Plan& pl, const void* x, const void* dy, const float* weight, const float* save_mean,
+                   const float* save_invstd, void* dx, float* dweight, float* dbias, float* ws, int64_t N,
+                   int64_t C, int64_t HW, hipStream_t s) {
+  const PlainInput<T> xs{static_cast<const T*>(x), pl.F};
+  return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+}
+
+template <typename T>
+int backward_packed(const Plan& pl, const int32_t* packed, const int32_t* bits, const int32_t* prefix,
+                    const void* scale, const void* mn, const void* dy, const float* weight,
+                    const float* save_mean, const float* save_invstd, void* dx, float* dweight,
+                    float* dbias, float* ws, int64_t N, int64_t C, int64_t HW, hipStream_t s) {
+  const PackedInput<T> xs{packed, bits, prefix, static_cast<const T*>(scale), static_cast<const T*>(mn),
+                          pl.F / 256, 0, 0u, false};
+  return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
 }
 
 }  // namespace
@@ -498,8 +593,29 @@ extern "C" int actnn_batch_norm_backward(const void* x, const void* dy, const fl
   hipStream_t s = static_cast<hipStream_t>(stream);
   float* ws = static_cast<float*>(workspace);
   switch (dtype) {
-    case ACTNN_F32: return backward_t<float>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
-    case ACTNN_F16: return backward_t<__half>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
-    default: return backward_t<bf16_t>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+    case ACTNN_F32: return backward_plain<float>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+    case ACTNN_F16: return backward_plain<__half>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+    default: return backward_plain<bf16_t>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
   }
+}
+
+extern "C" int actnn_batch_norm_backward_packed(const int32_t* packed, const int32_t* bits,
+                                                const int32_t* prefix, const void* scale, const void* mn,
+                                                const void* dy, const float* weight,
+                                                const float* save_mean, const float* save_invstd,
+                                                void* dx, float* dweight, float* dbias, void* workspace,
+                                                int64_t workspace_bytes, int64_t N, int64_t C,
+                                                int64_t HW, int dtype, void* stream) {
+  using namespace actnn;
+  if (dtype != ACTNN_F16 && dtype != ACTNN_BF16) return ACTNN_EDTYPE;
+  Plan pl;
+  if (!make_plan(N, C, HW, dtype, pl) || pl.F % 256 != 0) return ACTNN_EINVAL;
+  if (!packed || !bits || !prefix || !scale || !mn || !dy || !save_mean || !save_invstd || !workspace) return ACTNN_EINVAL;
+  if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
+  if (!aligned16(dy) || (dx && !aligned16(dx)) || !aligned16(workspace)) return ACTNN_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float* ws = static_cast<float*>(workspace);
+  if (dtype == ACTNN_F16)
+    return backward_packed<__half>(pl, packed, bits, prefix, scale, mn, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+  return backward_packed<bf16_t>(pl, packed, bits, prefix, scale, mn, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
 }

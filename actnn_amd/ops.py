@@ -334,6 +334,18 @@ class batch_norm(Function):
     @staticmethod
     def backward(ctx, grad_output):
         quantized, weight, running_mean, running_var, save_mean, save_var, training, eps, reserve = ctx.saved
+        if (training and config.compress_activation and not config.simulate and not config.swap
+                and config.group_size == 256 and config.fused_bn_backward):
+            grad_output = grad_output.contiguous()
+            if ext_backward_func.hip_batch_norm_backward_packed_applies(
+                    ctx.other_args, quantized, grad_output, weight, save_mean, save_var):
+                # the kernels decode the saved input from its bit stream: no full-precision copy
+                grads = ext_backward_func.hip_batch_norm_backward_packed(
+                    ctx.other_args, quantized, grad_output, weight, save_mean, save_var)
+                del quantized, ctx.saved
+                if ctx.scheme:
+                    ctx.scheme.if_allocate_perlayer()
+                return grads[0], None, None, grads[1], grads[2], None, None, None, None
         input = dequantize_activation(quantized, ctx.other_args)
         del quantized, ctx.saved
         empty_cache(config.empty_cache_threshold)

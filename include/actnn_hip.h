@@ -199,6 +199,18 @@ int actnn_batch_norm_backward(const void* x, const void* dy, const float* weight
                               int64_t workspace_bytes, int64_t N, int64_t C, int64_t HW, int dtype,
                               void* stream);
 
+/* The same backward pass with x held as the mixed-precision stream of actnn_pack_mixed (group
+ * size 256, C*HW % 256 == 0, 16-bit dtype; bits / prefix / scale / mn as for actnn_unpack_mixed):
+ * both passes rebuild x in registers, bit for bit what actnn_unpack_mixed would write, so the
+ * full-precision copy of x that ops.py:478 (dequantize_activation before
+ * cudnn_batch_norm_backward) materialises never exists. */
+int actnn_batch_norm_backward_packed(const int32_t* packed, const int32_t* bits,
+                                     const int32_t* prefix, const void* scale, const void* mn,
+                                     const void* dy, const float* weight, const float* save_mean,
+                                     const float* save_invstd, void* dx, float* dweight,
+                                     float* dbias, void* workspace, int64_t workspace_bytes,
+                                     int64_t N, int64_t C, int64_t HW, int dtype, void* stream);
+
 /* Plain device-to-device streaming copy of `bytes` bytes (16-byte aligned pointers and
  * size); used by the benchmark to calibrate bandwidth counters.  No reference counterpart. */
 int actnn_stream_copy(const void* src, void* dst, int64_t bytes, void* stream);

@@ -121,3 +121,29 @@ def test_no_affine_no_running_stats_and_fallback_shapes():
         ys = ext_bf.cudnn_batch_norm(xs, w, b, rm, rv, True, 0.1, 1e-5)[0]
         ref = o_bn.forward(xs.double().cpu().numpy(), None, None, None, None, 0.1, 1e-5)[0]
         assert np.allclose(ys.cpu().numpy(), ref, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,C,spatial", [(8, 64, (56, 56)), (16, 256, (7, 7)), (37, 64, (14, 14)),
+                                         (9, 32, (4, 2)), (12, 128, (28, 28))])
+def test_backward_from_the_packed_stream_equals_unpack_then_backward(N, C, spatial, dtype):
+    """The fused pass rebuilds x exactly as unpack_mixed_precision does, so every output is
+    bit-identical to the two-step path, for every width 1..8 in one batch."""
+    import actnn_amd.cpp_extension.quantization as ext_q
+    from _util import bits_tensor
+    x, w, b, rm, rv, dy = _inputs(N, C, spatial, dtype, 21)
+    G = x[0].numel() // 256
+    groups = x.view(N, G, 256)
+    mn, mx = ext_minimax.minimax(groups.view(-1, 256))
+    mn, mx = mn.view(N, G, 1), mx.view(N, G, 1)
+    bits_dev, _ = bits_tensor([1 + (3 * i + i // 8) % 8 for i in range(N)])
+    torch.cuda.manual_seed(5)
+    packed, scale = ext_q.pack_mixed_precision(groups, mn, mx, bits_dev, True)
+    _, mean, invstd, _, _ = ext_bf.hip_batch_norm_forward(x, w, b, None, None, 0.1, 1e-5)
+    xq = ext_q.unpack_mixed_precision(packed, bits_dev, scale, mn, N, G, 256).view_as(x)
+    ref = ext_bf.hip_batch_norm_backward(xq, dy, w, mean, invstd)
+    quantized = (packed, bits_dev, scale, mn)
+    assert ext_bf.hip_batch_norm_backward_packed_applies(x.shape, quantized, dy, w, mean, invstd)
+    got = ext_bf.hip_batch_norm_backward_packed(x.shape, quantized, dy, w, mean, invstd)
+    for a, r in zip(got, ref):
+        assert torch.equal(a, r)
