@@ -11,7 +11,7 @@ from .resnet import resnet50
 from .utils import compute_tensor_bytes, get_memory_usage
 
 
-def resnet50_step(device, level="L3", batch=512, warmup=3, steps=10, autocast=True):
+def resnet50_step(device, level="L3", batch=512, warmup=3, steps=10, autocast=True, channels_last=False):
     """images/s = batch / median step time over `steps` steps after `warmup`; activation memory =
     allocated before backward - allocated after the data is loaded - bytes(loss, output)."""
     config.reset()
@@ -22,9 +22,13 @@ def resnet50_step(device, level="L3", batch=512, warmup=3, steps=10, autocast=Tr
         set_optimization_level(level)
         model = QModule(model)
     model = model.to(device).train()
+    if channels_last:
+        model = model.to(memory_format=torch.channels_last)
     opt = torch.optim.SGD(model.parameters(), lr=0.1, momentum=0.9, weight_decay=1e-4)
     g = torch.Generator(device=device).manual_seed(0)
     images = torch.randn(batch, 3, 224, 224, generator=g, device=device)
+    if channels_last:
+        images = images.contiguous(memory_format=torch.channels_last)
     target = torch.randint(0, 1000, (batch,), generator=g, device=device)
     times, act_mem, peak = [], None, None
     for it in range(warmup + steps):
@@ -53,7 +57,8 @@ def resnet50_step(device, level="L3", batch=512, warmup=3, steps=10, autocast=Tr
     QBNScheme.reset()
     return {"images_per_s": round(batch / med, 1), "ms_per_step": round(med * 1e3, 2),
             "activation_mem_MB": round(act_mem / 2 ** 20, 1), "peak_mem_MB": round(peak / 2 ** 20, 1),
-            "batch": batch, "level": level, "autocast_bf16": autocast, "warmup": warmup, "steps": steps}
+            "batch": batch, "level": level, "autocast_bf16": autocast,
+            "memory_format": "channels_last" if channels_last else "contiguous", "warmup": warmup, "steps": steps}
 
 
 def run(device):

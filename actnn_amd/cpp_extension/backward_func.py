@@ -150,6 +150,12 @@ def cudnn_convolution_transpose_backward(input, grad_output, weight, padding, ou
     return gi, gw
 
 
+def _miopen_takes(input, weight, bias):
+    """MIOpen's batch norm wants fp32 affine parameters (and wants them to exist); other
+    combinations go to ATen's native kernels, which save the same (mean, invstd) pair."""
+    return all(t is not None and t.dtype == torch.float32 for t in (weight, bias))
+
+
 def cudnn_batch_norm(input, weight, bias, running_mean, running_var, training,
                      exponential_average_factor, epsilon):
     """-> (output, save_mean, save_var, reserve).  at::native::cudnn_batch_norm
@@ -159,6 +165,10 @@ def cudnn_batch_norm(input, weight, bias, running_mean, running_var, training,
         out, save_mean, save_invstd, _, _ = hip_batch_norm_forward(
             input, weight, bias, running_mean, running_var, exponential_average_factor, epsilon)
         return out, save_mean, save_invstd, input.new_empty(0, dtype=torch.uint8)
+    if not _miopen_takes(input, weight, bias):
+        out, save_mean, save_var = _aten.native_batch_norm(
+            input, weight, bias, running_mean, running_var, training, exponential_average_factor, epsilon)
+        return out, save_mean, save_var, input.new_empty(0, dtype=torch.uint8)
     out, save_mean, save_var = _aten.miopen_batch_norm(
         input, weight, bias, running_mean, running_var, training, exponential_average_factor, epsilon)
     return out, save_mean, save_var, input.new_empty(0, dtype=torch.uint8)
@@ -172,6 +182,9 @@ def cudnn_batch_norm_backward(input, grad_output, weight, running_mean, running_
             and grad_output.dtype == input.dtype and grad_output.shape == input.shape
             and grad_output.is_contiguous() and grad_output.data_ptr() % 16 == 0):
         return hip_batch_norm_backward(input, grad_output, weight, save_mean, save_var)
+    if not _miopen_takes(input, weight, weight):
+        return _aten.native_batch_norm_backward(grad_output, input, weight, running_mean, running_var,
+                                                save_mean, save_var, True, epsilon, [True, True, True])
     return _aten.miopen_batch_norm_backward(input, grad_output, weight, running_mean, running_var,
                                             save_mean, save_var, epsilon)
 

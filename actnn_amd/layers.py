@@ -18,6 +18,7 @@ from .cpp_extension import quantization as ext_quantization
 from .ops import batch_norm, conv1d, conv2d, conv3d, linear
 from .qbnscheme import QBNScheme
 from .qscheme import QScheme
+from .utils import channels_last_format, logical_order, memory_order
 
 
 def _autocast_apply(fn, *args):
@@ -155,6 +156,10 @@ class QReLU(nn.Module):
         super().__init__()
 
     def forward(self, input):
+        # the mask follows memory order, so a channels-last activation needs no transposition
+        fmt = channels_last_format(input)
+        if fmt is not None:
+            return logical_order(ext_quantization.act_quantized_relu(memory_order(input)), fmt)
         return ext_quantization.act_quantized_relu(input)
 
 
@@ -164,6 +169,9 @@ class QDropout(nn.Dropout):
 
     def forward(self, input):
         if self.training:
+            fmt = channels_last_format(input)
+            if fmt is not None:
+                return logical_order(ext_quantization.act_quantized_dropout(memory_order(input), self.p), fmt)
             return ext_quantization.act_quantized_dropout(input, self.p)
         return super().forward(input)
 
@@ -177,6 +185,12 @@ class QMaxPool2d(_MaxPoolNd):
         self.dilation = _pair(dilation)
 
     def forward(self, input):
+        if channels_last_format(input) is not None:
+            # the pooling kernels are NCHW: transpose in and out so that the model stays channels-last
+            out = ext_quantization.act_quantized_max_pool2d(
+                input.contiguous(), self.kernel_size, self.stride, self.padding, self.dilation,
+                self.ceil_mode, self.return_indices)
+            return out.contiguous(memory_format=torch.channels_last)
         return ext_quantization.act_quantized_max_pool2d(input, self.kernel_size, self.stride, self.padding,
                                                          self.dilation, self.ceil_mode, self.return_indices)
 

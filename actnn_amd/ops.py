@@ -12,7 +12,8 @@ from torch.nn.modules.utils import _pair, _single, _triple
 from .conf import config
 from .cpp_extension import backward_func as ext_backward_func
 from .cpp_extension import quantization as ext_quantization
-from .utils import compute_tensor_bytes, empty_cache, get_memory_usage, swap_to_cpu
+from .utils import (channels_last_format, compute_tensor_bytes, empty_cache, get_memory_usage,
+                    logical_order, swap_to_cpu)
 
 
 # ------------------------------------------------------------------------------------------
@@ -112,6 +113,11 @@ def dequantize_activation(quantized, q_input_shape):
     N = q_input_shape[0]
     features = int(np.prod(q_input_shape[1:]))
     out = out.view(N, -1)[:, :features]
+    memory_format = getattr(quantized, "memory_format", None)
+    if memory_format is not None:
+        # saved in channels-last order: rebuild [N, ..., C] and hand out the channels-last view
+        out = out.reshape(N, *q_input_shape[2:], q_input_shape[1])
+        return logical_order(out.contiguous(), memory_format)
     return out.reshape(*q_input_shape).contiguous()
 
 
@@ -123,17 +129,20 @@ def _stored_as_bf16(shape, quantized):
 
 
 class _Quantized(tuple):
-    """(q_input, q_bits, q_scale, q_min) plus a flag telling bf16 activations apart."""
+    """(q_input, q_bits, q_scale, q_min) plus what the tuple cannot say: whether bf16 scale/min
+    are the activation's own dtype, and the memory format the activation was compressed in."""
     native_bf16 = False
+    memory_format = None
 
 
 def quantize_saved(input, scheme):
-    return finish_saved(start_quantize(input, scheme), input.dtype)
+    return finish_saved(start_quantize(input, scheme), input)
 
 
-def finish_saved(started, dtype):
+def finish_saved(started, input):
     q = _Quantized(finish_quantize(started))
-    q.native_bf16 = dtype == torch.bfloat16
+    q.native_bf16 = input.dtype == torch.bfloat16
+    q.memory_format = channels_last_format(input)
     return q
 
 
@@ -150,7 +159,7 @@ def _conv_forward(ctx, forward_op, input, weight, bias, stride, padding, dilatio
     # the pack: the convolution runs while the sensitivities travel to the host
     started = start_quantize(input, scheme)
     output = forward_op(input, weight, bias, stride, padding, dilation, groups)
-    quantized = finish_saved(started, input.dtype)
+    quantized = finish_saved(started, input)
     ctx.scheme = scheme
     ctx.saved = quantized, weight, bias
     ctx.other_args = (input.shape, stride, padding, dilation, groups)
@@ -172,9 +181,10 @@ def _conv_backward(ctx, grad_output, bias_reduce_dims, aug):
     padding, stride, dilation = aug(padding), aug(stride), aug(dilation)
     quantized, weight, bias = ctx.saved
     input = dequantize_activation(quantized, q_input_shape)
+    memory_format = getattr(quantized, "memory_format", None) or torch.contiguous_format
     del quantized, ctx.saved
     empty_cache(config.empty_cache_threshold)
-    grad_output = grad_output.contiguous()
+    grad_output = grad_output.contiguous(memory_format=memory_format)
     need = [ctx.needs_input_grad[0], ctx.needs_input_grad[1]]
 
     ws_mem = compute_tensor_bytes([grad_output, input, input])
@@ -252,7 +262,7 @@ class linear(Function):
     def forward(ctx, input, weight, bias=None, scheme=None):
         started = start_quantize(input, scheme)
         output = F.linear(input, weight, bias)
-        quantized = finish_saved(started, input.dtype)
+        quantized = finish_saved(started, input)
         empty_cache(config.empty_cache_threshold)
         ctx.scheme = scheme
         ctx.saved = quantized, weight, bias
@@ -317,7 +327,7 @@ class batch_norm(Function):
             output, save_mean, save_var = ext_backward_func.native_batch_norm(
                 input, weight, bias, running_mean, running_var, training, exponential_average_factor, eps)
             reserve = None
-        quantized = finish_saved(started, input.dtype)
+        quantized = finish_saved(started, input)
         empty_cache(config.empty_cache_threshold)
         if config.debug_memory_op_forward:
             global bn_layer_ct, total_act_mem
@@ -335,7 +345,8 @@ class batch_norm(Function):
     def backward(ctx, grad_output):
         quantized, weight, running_mean, running_var, save_mean, save_var, training, eps, reserve = ctx.saved
         if (training and config.compress_activation and not config.simulate and not config.swap
-                and config.group_size == 256 and config.fused_bn_backward):
+                and config.group_size == 256 and config.fused_bn_backward
+                and getattr(quantized, "memory_format", None) is None):
             grad_output = grad_output.contiguous()
             if ext_backward_func.hip_batch_norm_backward_packed_applies(
                     ctx.other_args, quantized, grad_output, weight, save_mean, save_var):
@@ -347,11 +358,13 @@ class batch_norm(Function):
                     ctx.scheme.if_allocate_perlayer()
                 return grads[0], None, None, grads[1], grads[2], None, None, None, None
         input = dequantize_activation(quantized, ctx.other_args)
+        memory_format = getattr(quantized, "memory_format", None) or torch.contiguous_format
         del quantized, ctx.saved
         empty_cache(config.empty_cache_threshold)
         if training:
             grad_input, grad_weight, grad_bias = ext_backward_func.cudnn_batch_norm_backward(
-                input.contiguous(), grad_output.contiguous(), weight, running_mean, running_var,
+                input.contiguous(memory_format=memory_format),
+                grad_output.contiguous(memory_format=memory_format), weight, running_mean, running_var,
                 save_mean, save_var, eps, reserve)
         else:
             grad_input, grad_weight, grad_bias = ext_backward_func.native_batch_norm_backward(

@@ -12,6 +12,7 @@ from .conf import config
 from .cpp_extension import calc_precision as ext_calc_precision
 from .cpp_extension import minimax as ext_minimax
 from .cpp_extension.quantization import attach_bits_host, attach_bits_total
+from .utils import memory_order
 
 
 def group_min_max(input, known=None):
@@ -20,7 +21,7 @@ def group_min_max(input, known=None):
     pixels per channel).  `known` = (mn, mx) already produced by another pass over the same
     tensor (the batch-norm statistics kernel); only given when no padding is needed."""
     N = input.shape[0]
-    flat = input.reshape(N, -1)
+    flat = memory_order(input).reshape(N, -1)            # a view for default and channels-last layouts
     features = flat.shape[1]
     num_pixels = features // input.shape[1]
     gs = config.group_size
@@ -153,7 +154,8 @@ class QScheme(_LazyHost):
         if not QScheme.update_scale:
             return
         # squared L2 norm per sample, accumulated in fp32 without materialising an fp32 copy
-        sq = torch.linalg.vector_norm(grad.reshape(grad.shape[0], -1), dim=1, dtype=torch.float32).square()
+        sq = torch.linalg.vector_norm(memory_order(grad).reshape(grad.shape[0], -1), dim=1,
+                                      dtype=torch.float32).square()
         if config.use_gradient:
             assert QScheme.batch is not None
             self.scales[QScheme.batch] = self.scales[QScheme.batch] * 0.5 + sq.cpu() * 0.5

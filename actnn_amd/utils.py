@@ -13,6 +13,35 @@ def swap_to_cpu(tensor):
     return host
 
 
+def channels_last_format(t):
+    """torch.channels_last / channels_last_3d when `t` is dense in that order and not in the
+    default one, else None.  Tensors whose two orders coincide (C == 1 or no spatial extent)
+    count as default."""
+    if t.dim() == 4 and not t.is_contiguous() and t.is_contiguous(memory_format=torch.channels_last):
+        return torch.channels_last
+    if t.dim() == 5 and not t.is_contiguous() and t.is_contiguous(memory_format=torch.channels_last_3d):
+        return torch.channels_last_3d
+    return None
+
+
+def memory_order(t):
+    """`t` with its axes arranged as they lie in memory: a channels-last tensor [N, C, ...]
+    comes back as the contiguous view [N, ..., C], everything else unchanged.  On MI355X the
+    convolution kernels are channels-last natively, so activations of a channels-last model are
+    compressed in that order instead of being transposed first: groups of 256 elements that are
+    consecutive in memory, whatever the logical axis order."""
+    if channels_last_format(t) is None:
+        return t
+    return t.permute(0, *range(2, t.dim()), 1)
+
+
+def logical_order(t_mem, memory_format):
+    """Inverse of memory_order for a tensor laid out [N, ..., C] in memory."""
+    if memory_format is None:
+        return t_mem
+    return t_mem.permute(0, t_mem.dim() - 1, *range(1, t_mem.dim() - 1))
+
+
 def get_memory_usage(print_info=False):
     """Bytes currently allocated by torch's caching allocator on device 0 - the reference's
     memory metric (utils.py:16-23; explicitly not the driver's view)."""

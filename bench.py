@@ -145,7 +145,33 @@ def other_configs(device, reps):
     out["max_pool2d_forward_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
     t = _event_time_ms(lambda: ext_q.max_pool2d_backward(gp, idx, x.shape, k, s, p), reps)
     out["max_pool2d_backward_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
-    del x, g, y, mask, yp, idx, gp
+    del y, mask, yp, idx, gp
+    # training-mode batch norm on the same tensor: forward (statistics + normalise, with and without
+    # the quantiser's group min/max from the statistics pass), backward from the full-precision
+    # input and backward straight from the 2-bit stream
+    import actnn_amd.cpp_extension.backward_func as ext_bf
+    C = x.shape[1]
+    w = torch.rand(C, device=device) + 0.5
+    bias = torch.randn(C, device=device)
+    b = 3 * 2 * n
+    t = _event_time_ms(lambda: ext_bf.hip_batch_norm_forward(x, w, bias, None, None, 0.1, 1e-5), reps)
+    out["batch_norm_forward_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
+    b = 3 * 2 * n + 2 * 2 * n / 256
+    t = _event_time_ms(lambda: ext_bf.hip_batch_norm_forward(x, w, bias, None, None, 0.1, 1e-5, minmax=True), reps)
+    out["batch_norm_forward_with_group_minmax_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
+    _, mean, invstd, lo, hi = ext_bf.hip_batch_norm_forward(x, w, bias, None, None, 0.1, 1e-5, minmax=True)
+    b = 5 * 2 * n
+    t = _event_time_ms(lambda: ext_bf.hip_batch_norm_backward(x, g, w, mean, invstd), reps)
+    out["batch_norm_backward_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
+    Nb, Gb = x.shape[0], n // x.shape[0] // 256
+    host_bits = torch.full((Nb,), 2, dtype=torch.int32)
+    bits2 = ext_q.attach_bits_host(host_bits.to(device), host_bits)
+    q_in, q_scale = ext_q.pack_mixed_precision(x.view(Nb, Gb, 256), lo.view(Nb, Gb, 1), hi.view(Nb, Gb, 1), bits2, True)
+    quantized = (q_in, bits2, q_scale, lo.view(Nb, Gb, 1))
+    b = 3 * 2 * n + 2 * (2 * n / 8 + 2 * 2 * n / 256)       # dy twice, dx once; stream, scale, min twice
+    t = _event_time_ms(lambda: ext_bf.hip_batch_norm_backward_packed(x.shape, quantized, g, w, mean, invstd), reps)
+    out["batch_norm_backward_from_2bit_stream_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
+    del x, g, q_in, q_scale, quantized, lo, hi
     # config 4 input through the fixed-width path (2 bits)
     M, I = 8192, 4096
     xs = torch.randn(M, I // 256, 256, device=device, dtype=torch.float16)
@@ -182,7 +208,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the config-2 hot path")
-    ap.add_argument("--only", choices=["other", "resnet50"], default=None,
+    ap.add_argument("--only", choices=["other", "resnet50", "resnet50_channels_last"], default=None,
                     help="profiling aid: run just the other single-GPU configs (ReLU, max-pool, "
                          "fixed-width pack, fused GEMM) or just the ResNet-50 L3 step, print their JSON")
     args = ap.parse_args()
@@ -204,6 +230,11 @@ def main():
     if args.only == "resnet50":
         from actnn_amd import bench_extra
         print(json.dumps({"resnet50_L3": bench_extra.resnet50_step(device, "L3", warmup=2, steps=3)}))
+        return
+    if args.only == "resnet50_channels_last":
+        from actnn_amd import bench_extra
+        print(json.dumps({"resnet50_L3_channels_last": bench_extra.resnet50_step(
+            device, "L3", warmup=2, steps=3, channels_last=True)}))
         return
     xg, mn, mx, bits, bits_host = make_config2(device)
     N, G, gs = xg.shape

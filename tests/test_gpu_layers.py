@@ -237,3 +237,76 @@ def test_activation_memory_shrinks():
         return held
     full, packed = saved_bytes("L0"), saved_bytes("L3")
     assert packed < full / 6
+
+
+def _cl(model):
+    return model.to(DEV).to(memory_format=torch.channels_last)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_channels_last_block_8bit_close_to_exact_and_stays_channels_last(dtype):
+    """A channels-last model is compressed in memory order (no transposes): with 8 bits the
+    gradients of conv + BN + ReLU + max-pool + conv match the exact ones as in the default layout,
+    and activations and gradients keep the channels-last strides throughout."""
+    config.activation_compression_bits = [8]
+    config.initial_bits = 8
+    config.perlayer = False
+
+    def make():
+        torch.manual_seed(0)
+        return nn.Sequential(nn.Conv2d(16, 32, 3, padding=1, bias=False), nn.BatchNorm2d(32), nn.ReLU(),
+                             nn.MaxPool2d(3, 2, 1), nn.Conv2d(32, 64, 3, padding=1, bias=False),
+                             nn.BatchNorm2d(64), nn.ReLU(), nn.Dropout(0.0))
+    exact = _cl(make()).to(dtype)
+    quant = _cl(QModule(make())).to(dtype)
+    quant.load_state_dict(exact.state_dict())
+    x = torch.randn(8, 16, 32, 32, device=DEV, dtype=dtype).contiguous(memory_format=torch.channels_last)
+    g = torch.randn(8, 64, 16, 16, device=DEV, dtype=dtype).contiguous(memory_format=torch.channels_last)
+    res = []
+    for model in (exact, quant):
+        xi = x.clone(memory_format=torch.preserve_format).requires_grad_(True)
+        y = model(xi)
+        assert y.is_contiguous(memory_format=torch.channels_last)
+        y.backward(g)
+        assert xi.grad.is_contiguous(memory_format=torch.channels_last)
+        res.append((y.detach().float(), xi.grad.float(), [p.grad.float() for p in model.parameters()]))
+    (ye, gxe, gpe), (yq, gxq, gpq) = res
+    tol = 2e-3 if dtype == torch.float32 else 6e-2
+    assert torch.allclose(yq, ye, atol=tol, rtol=tol)
+    assert (gxq - gxe).norm() / gxe.norm() < 3e-2
+    for a, b in zip(gpq, gpe):
+        assert (a - b).norm() / (b.norm() + 1e-6) < 3e-2
+
+
+def test_channels_last_saved_activation_round_trip():
+    """quantize_saved / dequantize_activation on a channels-last tensor: groups follow memory
+    order, the rebuilt tensor has the logical shape, channels-last strides and 8-bit accuracy;
+    the packed stream equals the one of the same memory seen as a default-layout tensor."""
+    config.activation_compression_bits = [8]
+    torch.manual_seed(0)
+    x = torch.randn(4, 64, 12, 8, device=DEV).contiguous(memory_format=torch.channels_last)
+    torch.cuda.manual_seed(3)
+    q = quantize_saved(x, None)
+    assert q.memory_format == torch.channels_last
+    back = dequantize_activation(q, x.shape)
+    assert back.shape == x.shape and back.is_contiguous(memory_format=torch.channels_last)
+    # one 8-bit step, plus the bfloat16 rounding of the stored scale / minimum of an fp32 activation
+    assert (back - x).abs().max() < (x.max() - x.min()) / 255 + 2.0 ** -6 * x.abs().max()
+    torch.cuda.manual_seed(3)
+    q2 = quantize_saved(x.permute(0, 2, 3, 1).contiguous(), None)       # same memory, default layout
+    # (the fixed-width stream ends in one spare byte that no kernel writes, .cu:268)
+    assert torch.equal(q[0][:-1], q2[0][:-1]) and torch.equal(q[2], q2[2])
+
+
+def test_resnet50_channels_last_step_runs():
+    torch.manual_seed(0)
+    model = _cl(QModule(resnet50()))
+    x = torch.randn(8, 3, 64, 64, device=DEV).contiguous(memory_format=torch.channels_last)
+    y = torch.randint(0, 1000, (8,), device=DEV)
+    for _ in range(2):
+        model.zero_grad()
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            loss = F.cross_entropy(model(x), y)
+        loss.backward()
+    assert torch.isfinite(loss)
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in model.parameters())
