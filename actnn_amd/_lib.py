@@ -48,13 +48,13 @@ SIGNATURES = {
     "actnn_linear_grad_weight_q2": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64,
                                     c_i32, c_i32, c_i32, c_vp],
     "actnn_stream_copy": [c_vp, c_vp, c_i64, c_vp],
-    "actnn_batch_norm_workspace_bytes": [c_i64, c_i64, c_i64, c_i32],
+    "actnn_batch_norm_workspace_bytes": [c_i64, c_i64, c_i64, c_i32, c_i32],
     "actnn_batch_norm_forward": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,
-                                 c_i64, c_i64, c_i64, ctypes.c_double, ctypes.c_double, c_i32, c_vp],
+                                 c_i64, c_i64, c_i64, ctypes.c_double, ctypes.c_double, c_i32, c_i32, c_vp],
     "actnn_batch_norm_backward_packed": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp,
-                                         c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i32, c_vp],
+                                         c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
     "actnn_batch_norm_backward": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,
-                                  c_i64, c_i64, c_i64, c_i32, c_vp],
+                                  c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
 }
 _RESTYPES = {"actnn_strerror": ctypes.c_char_p, "actnn_version": ctypes.c_char_p,
              "actnn_batch_norm_workspace_bytes": ctypes.c_int64}

@@ -9,11 +9,12 @@ The three layer-norm exports of the reference have no Python caller and are not 
 import torch
 
 from . import _glue
+from ..utils import channels_last_format
 
 _aten = torch.ops.aten
 
 
-def _shape_geometry(shape, dtype):
+def _shape_geometry(shape, dtype, channels_last):
     """(N, C, HW) when the library's batch-norm kernels take a tensor of this shape, else None."""
     if len(shape) < 2 or dtype not in _glue.DTYPE_CODE:
         return None
@@ -21,15 +22,21 @@ def _shape_geometry(shape, dtype):
     HW = 1
     for d in shape[2:]:
         HW *= int(d)
-    if N * C * HW == 0 or _glue.lib().actnn_batch_norm_workspace_bytes(N, C, HW, _glue.DTYPE_CODE[dtype]) < 0:
+    if N * C * HW == 0 or _glue.lib().actnn_batch_norm_workspace_bytes(
+            N, C, HW, _glue.DTYPE_CODE[dtype], int(channels_last)) < 0:
         return None
     return N, C, HW
 
 
 def _bn_geometry(input):
-    if not (isinstance(input, torch.Tensor) and input.is_cuda and input.is_contiguous()):
+    """(N, C, HW, channels_last) of a dense tensor in the default or the channels-last layout."""
+    if not (isinstance(input, torch.Tensor) and input.is_cuda):
         return None
-    return _shape_geometry(input.shape, input.dtype)
+    channels_last = channels_last_format(input) is not None
+    if not channels_last and not input.is_contiguous():
+        return None
+    geo = _shape_geometry(input.shape, input.dtype, channels_last)
+    return None if geo is None else geo + (channels_last,)
 
 
 def _f32_or_none(t):
@@ -41,20 +48,33 @@ def hip_batch_norm_applies(input, weight, bias, running_mean, running_var):
             and all(_f32_or_none(t) for t in (weight, bias, running_mean, running_var)))
 
 
+def _groups_align(C, HW, channels_last):
+    """Groups of 256 elements (in memory order) coincide with runs of threads of the kernels."""
+    return (C * HW) % 256 == 0 and (not channels_last or C % 256 == 0 or 256 % C == 0)
+
+
+def hip_batch_norm_minmax_applies(input, weight, bias, running_mean, running_var):
+    """True when the forward pass can also return the quantiser's per-group min/max."""
+    if not hip_batch_norm_applies(input, weight, bias, running_mean, running_var):
+        return False
+    _, C, HW, channels_last = _bn_geometry(input)
+    return _groups_align(C, HW, channels_last)
+
+
 def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
 def hip_batch_norm_forward(input, weight, bias, running_mean, running_var, momentum, eps, minmax=False):
     """-> (output, save_mean, save_invstd, mn, mx): training-mode batch norm; with `minmax` the
-    minimum and maximum of every group of 256 consecutive elements of a sample come out of the
-    same pass over the input (None, None otherwise)."""
-    N, C, HW = _bn_geometry(input)
+    minimum and maximum of every group of 256 elements of a sample that are consecutive in memory
+    come out of the same pass over the input (None, None otherwise)."""
+    N, C, HW, channels_last = _bn_geometry(input)
     lib = _glue.lib()
     code = _glue.DTYPE_CODE[input.dtype]
-    ws_bytes = lib.actnn_batch_norm_workspace_bytes(N, C, HW, code)
+    ws_bytes = lib.actnn_batch_norm_workspace_bytes(N, C, HW, code, int(channels_last))
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=input.device)
-    out = torch.empty_like(input)
+    out = torch.empty_like(input)                       # same strides as the input
     save_mean = torch.empty(C, dtype=torch.float32, device=input.device)
     save_invstd = torch.empty(C, dtype=torch.float32, device=input.device)
     mn = mx = None
@@ -66,17 +86,18 @@ def hip_batch_norm_forward(input, weight, bias, running_mean, running_var, momen
         _glue._lib.check(lib.actnn_batch_norm_forward(
             input.data_ptr(), _ptr(weight), _ptr(bias), _ptr(running_mean), _ptr(running_var),
             out.data_ptr(), save_mean.data_ptr(), save_invstd.data_ptr(), _ptr(mn), _ptr(mx),
-            ws.data_ptr(), ws_bytes, N, C, HW, float(momentum), float(eps), code,
+            ws.data_ptr(), ws_bytes, N, C, HW, float(momentum), float(eps), code, int(channels_last),
             _glue.stream_ptr(input.device)), "batch_norm_forward")
     return out, save_mean, save_invstd, mn, mx
 
 
 def hip_batch_norm_backward(input, grad_output, weight, save_mean, save_invstd):
-    """-> (grad_input, grad_weight, grad_bias) of training-mode batch norm."""
-    N, C, HW = _bn_geometry(input)
+    """-> (grad_input, grad_weight, grad_bias) of training-mode batch norm; `grad_output` has the
+    strides of `input`."""
+    N, C, HW, channels_last = _bn_geometry(input)
     lib = _glue.lib()
     code = _glue.DTYPE_CODE[input.dtype]
-    ws_bytes = lib.actnn_batch_norm_workspace_bytes(N, C, HW, code)
+    ws_bytes = lib.actnn_batch_norm_workspace_bytes(N, C, HW, code, int(channels_last))
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=input.device)
     grad_input = torch.empty_like(input)
     grad_weight = torch.empty(C, dtype=torch.float32, device=input.device)
@@ -85,22 +106,28 @@ def hip_batch_norm_backward(input, grad_output, weight, save_mean, save_invstd):
         _glue._lib.check(lib.actnn_batch_norm_backward(
             input.data_ptr(), grad_output.data_ptr(), _ptr(weight), save_mean.data_ptr(),
             save_invstd.data_ptr(), grad_input.data_ptr(), grad_weight.data_ptr(), grad_bias.data_ptr(),
-            ws.data_ptr(), ws_bytes, N, C, HW, code, _glue.stream_ptr(input.device)), "batch_norm_backward")
+            ws.data_ptr(), ws_bytes, N, C, HW, code, int(channels_last),
+            _glue.stream_ptr(input.device)), "batch_norm_backward")
     return grad_input, grad_weight, grad_bias
 
 
 def hip_batch_norm_backward_packed_applies(shape, quantized, grad_output, weight, save_mean, save_invstd):
     """True when the batch-norm backward kernels can read the saved input straight from its
-    mixed-precision stream: 16-bit activation with scale/min in its own dtype, whole groups of 256."""
+    mixed-precision stream: 16-bit activation with scale/min in its own dtype, whole groups of
+    256, and a gradient laid out like the activation was when it was compressed."""
     q_input, q_bits, q_scale, q_min = quantized
     dtype = grad_output.dtype
-    geo = _shape_geometry(shape, dtype)
+    memory_format = getattr(quantized, "memory_format", None)
+    channels_last = memory_format is not None
+    geo = _shape_geometry(shape, dtype, channels_last)
     return (geo is not None and dtype in (torch.float16, torch.bfloat16)
-            and (geo[1] * geo[2]) % 256 == 0 and isinstance(q_bits, torch.Tensor)
+            and _groups_align(geo[1], geo[2], channels_last) and isinstance(q_bits, torch.Tensor)
             and isinstance(q_input, torch.Tensor) and q_input.is_cuda and q_input.dtype == torch.int32
             and q_scale.dtype == dtype and q_min.dtype == dtype
             and q_scale.is_contiguous() and q_min.is_contiguous()
-            and tuple(grad_output.shape) == tuple(shape) and grad_output.is_contiguous()
+            and tuple(grad_output.shape) == tuple(shape)
+            and grad_output.is_contiguous(memory_format=memory_format or torch.contiguous_format)
+            and (not channels_last or geo[0] * geo[2] < 2 ** 31)
             and grad_output.data_ptr() % 16 == 0
             and all(_f32_or_none(t) for t in (weight, save_mean, save_invstd)))
 
@@ -109,13 +136,14 @@ def hip_batch_norm_backward_packed(shape, quantized, grad_output, weight, save_m
     """-> (grad_input, grad_weight, grad_bias); the saved input is decoded inside the kernels."""
     from .quantization import _bits_info
     q_input, q_bits, q_scale, q_min = quantized
-    N, C, HW = _shape_geometry(shape, grad_output.dtype)
+    channels_last = getattr(quantized, "memory_format", None) is not None
+    N, C, HW = _shape_geometry(shape, grad_output.dtype, channels_last)
     lib = _glue.lib()
     code = _glue.DTYPE_CODE[grad_output.dtype]
     total, prefix = _bits_info(q_bits)
     if q_input.numel() < total * (C * HW // 256) * 8:
         raise RuntimeError("batch_norm_backward_packed: packed stream is too short")
-    ws_bytes = lib.actnn_batch_norm_workspace_bytes(N, C, HW, code)
+    ws_bytes = lib.actnn_batch_norm_workspace_bytes(N, C, HW, code, int(channels_last))
     dev = grad_output.device
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dev)
     grad_input = torch.empty_like(grad_output)
@@ -126,7 +154,7 @@ def hip_batch_norm_backward_packed(shape, quantized, grad_output, weight, save_m
             q_input.data_ptr(), q_bits.data_ptr(), prefix.data_ptr(), q_scale.data_ptr(), q_min.data_ptr(),
             grad_output.data_ptr(), _ptr(weight), save_mean.data_ptr(), save_invstd.data_ptr(),
             grad_input.data_ptr(), grad_weight.data_ptr(), grad_bias.data_ptr(), ws.data_ptr(), ws_bytes,
-            N, C, HW, code, _glue.stream_ptr(dev)), "batch_norm_backward_packed")
+            N, C, HW, code, int(channels_last), _glue.stream_ptr(dev)), "batch_norm_backward_packed")
     return grad_input, grad_weight, grad_bias
 
 
@@ -180,7 +208,7 @@ def cudnn_batch_norm_backward(input, grad_output, weight, running_mean, running_
     (backward_func.cc:88)."""
     if (hip_batch_norm_applies(input, weight, None, save_mean, save_var)
             and grad_output.dtype == input.dtype and grad_output.shape == input.shape
-            and grad_output.is_contiguous() and grad_output.data_ptr() % 16 == 0):
+            and grad_output.stride() == input.stride() and grad_output.data_ptr() % 16 == 0):
         return hip_batch_norm_backward(input, grad_output, weight, save_mean, save_var)
     if not _miopen_takes(input, weight, weight):
         return _aten.native_batch_norm_backward(grad_output, input, weight, running_mean, running_var,

@@ -158,6 +158,7 @@ ACTNN_DEV void fold_block(float* s_acc, int slots, const Place& p, int64_t first
 // thread for sample n in two steps, so that the loads of several samples can be in flight before
 // the first one is used.
 template <typename T> struct PlainInput {
+  static constexpr bool kRows = false;
   static constexpr int kInFlight = 4;      // samples whose loads are issued before the first is used
   const T* p;            // already offset to the thread's chunk of sample 0
   int64_t F;
@@ -173,6 +174,7 @@ template <typename T> struct PlainInput {
 // words, transposes them (32x32 bits) and every lane finds its 8 codes in its own register.
 // Values are rebuilt exactly as actnn_unpack_mixed rebuilds them.  16-bit types only.
 template <typename T> struct PackedInput {
+  static constexpr bool kRows = false;
   static constexpr int kInFlight = 2;      // the decode needs registers: 2 measured faster than 4
   const int32_t* words;
   const int32_t* bits;
@@ -183,18 +185,19 @@ template <typename T> struct PackedInput {
   uint32_t lane32;
   bool active;
   struct Raw { uint32_t lo, hi; float sc, m; int b; };
-  ACTNN_DEV Raw fetch(int64_t n) const {
+  ACTNN_DEV Raw fetch_group(int64_t n, int64_t grp) const {
     Raw r{0u, 0u, 1.0f, 0.0f, 1};
     if (active) {
       r.b = bits[n];
-      const int32_t* w = words + ((int64_t)prefix[n] * G + g * r.b) * 8;
+      const int32_t* w = words + ((int64_t)prefix[n] * G + grp * r.b) * 8;
       if ((int)lane32 < 8 * r.b) r.lo = (uint32_t)w[lane32];
       if ((int)lane32 + 32 < 8 * r.b) r.hi = (uint32_t)w[lane32 + 32];
-      r.sc = Conv<T>::load(scale, n * G + g);
-      r.m = Conv<T>::load(mn, n * G + g);
+      r.sc = Conv<T>::load(scale, n * G + grp);
+      r.m = Conv<T>::load(mn, n * G + grp);
     }
     return r;
   }
+  ACTNN_DEV Raw fetch(int64_t n) const { return fetch_group(n, g); }
   template <int BITS> ACTNN_DEV u32x4 decode_bits(const Raw& r) const {
     uint64_t acc = transpose32(r.lo, lane32);
     if (BITS > 4) acc |= (uint64_t)transpose32(r.hi, lane32) << 32;
@@ -304,19 +307,29 @@ __global__ __launch_bounds__(kThreads) void bn_reduce_kernel(
 // Folds the table of partial sums of channel c in double precision: the wave's lanes take the
 // (span, batch split) entries of the channel in a fixed assignment and are combined by a butterfly,
 // so every lane ends with the same totals and the order of the additions is fixed.
+// (channels-last tables, slots == 0, hold nsplit consecutive values per channel and sum.)
 ACTNN_DEV void channel_totals(const float* __restrict__ part, int64_t c, int64_t HW, int64_t L,
                               int nsplit, int slots, double& s0, double& s1) {
   const int lane = threadIdx.x & 63;
-  const int64_t j0 = (c * HW) / L, j1 = ((c + 1) * HW - 1) / L;
-  const int64_t count = (j1 - j0 + 1) * nsplit;
   s0 = 0.0;
   s1 = 0.0;
-  for (int64_t i = lane; i < count; i += 64) {
-    const int64_t j = j0 + i / nsplit, y = i % nsplit;
-    const int64_t slot = c - (j * L) / HW;
-    const float* q = part + ((j * nsplit + y) * slots + slot) * 2;
-    s0 += (double)q[0];
-    s1 += (double)q[1];
+  if (slots == 0) {
+    const float* q0 = part + (c * 2) * (int64_t)nsplit;
+    const float* q1 = q0 + nsplit;
+    for (int i = lane; i < nsplit; i += 64) {
+      s0 += (double)q0[i];
+      s1 += (double)q1[i];
+    }
+  } else {
+    const int64_t j0 = (c * HW) / L, j1 = ((c + 1) * HW - 1) / L;
+    const int64_t count = (j1 - j0 + 1) * nsplit;
+    for (int64_t i = lane; i < count; i += 64) {
+      const int64_t j = j0 + i / nsplit, y = i % nsplit;
+      const int64_t slot = c - (j * L) / HW;
+      const float* q = part + ((j * nsplit + y) * slots + slot) * 2;
+      s0 += (double)q[0];
+      s1 += (double)q[1];
+    }
   }
 #pragma unroll
   for (int d = 32; d > 0; d >>= 1) {
@@ -450,6 +463,211 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
   }
 }
 
+// ------------------------------------------------------------------ channels-last tensors
+// [N, HW, C] in memory: a matrix of P = N * HW rows (pixels) by C columns (channels), the layout
+// the convolution kernels of this GPU work in.  A block owns a tile of up to 256 columns and a run
+// of consecutive rows; its threads form R rows of `tpr` chunks, thread (r, j) keeps the same E
+// channels for the whole run, so the per-channel sums and coefficients again live in registers.
+// For C <= 256 a block reads one contiguous stretch of memory; for wider tensors a row segment is
+// 512 bytes.  With C % 256 == 0 or 256 % C == 0 a quantisation group (256 consecutive elements)
+// is an aligned run of 256 / E threads, as in the default layout, so the group min/max and the
+// decoding of a packed input carry over unchanged.
+template <typename T> struct PlainRows {
+  static constexpr bool kRows = true;
+  static constexpr int kInFlight = 4;
+  const T* p;            // offset to the thread's columns of row 0 once bound
+  int64_t C;
+  struct Raw { u32x4 v; };
+  ACTNN_DEV void bind(int64_t col, int64_t) { p += col; }
+  ACTNN_DEV Raw fetch(int64_t row) const { return Raw{load16(p + row * C)}; }
+  ACTNN_DEV u32x4 decode(const Raw& r) const { return r.v; }
+};
+template <typename T> struct PackedRows {
+  static constexpr bool kRows = true;
+  static constexpr int kInFlight = 2;
+  PackedInput<T> in;     // G = groups per sample
+  int64_t C, col;
+  uint32_t HW;
+  using Raw = typename PackedInput<T>::Raw;
+  ACTNN_DEV void bind(int64_t column, int64_t) {
+    col = column;
+    in.lane32 = threadIdx.x & 31;
+    in.active = true;
+  }
+  ACTNN_DEV Raw fetch(int64_t row) const {
+    const uint32_t n = (uint32_t)row / HW;                 // rows < 2^31 (checked by the launcher)
+    const int64_t grp = ((row * C + col) >> 8) - (int64_t)n * in.G;
+    return in.fetch_group(n, grp);
+  }
+  ACTNN_DEV u32x4 decode(const Raw& r) const { return in.decode(r); }
+};
+
+struct RowTile {
+  int64_t col;           // first channel of the thread's chunk
+  int r;                 // row of the thread inside one iteration
+  bool active;
+};
+template <int E> ACTNN_DEV RowTile row_tile(int64_t C, int tpr, int R) {
+  RowTile t;
+  const int j = threadIdx.x % tpr;
+  t.r = threadIdx.x / tpr;
+  t.col = (int64_t)blockIdx.x * 256 + (int64_t)j * E;
+  t.active = t.r < R && t.col < C && j * E < 256;
+  if (!t.active) t.col = 0;
+  return t;
+}
+
+template <typename T, bool BWD, bool MINMAX, typename XS>
+__global__ __launch_bounds__(kThreads) void bn_cl_reduce_kernel(
+    XS xs, const T* __restrict__ dy, float* __restrict__ part, T* __restrict__ mn, T* __restrict__ mx,
+    int64_t P, int64_t C, int tpr, int R, int64_t ppb) {
+  constexpr int E = Chunk<T>::kElems;
+  constexpr int PD = Chunk<T>::kPerDword;
+  constexpr int U = XS::kInFlight;
+  __shared__ float s_part[kThreads * 2 * E];
+  const RowTile t = row_tile<E>(C, tpr, R);
+  xs.bind(t.col, C);
+  const T* pd = BWD ? dy + t.col : nullptr;
+  const int64_t p0 = (int64_t)blockIdx.y * ppb;
+  const int64_t p1 = p0 + ppb < P ? p0 + ppb : P;
+  float s[E], q[E];
+#pragma unroll
+  for (int i = 0; i < E; ++i) { s[i] = 0.0f; q[i] = 0.0f; }
+
+  auto accumulate = [&](const u32x4& ux, const u32x4& ud, int64_t row) {
+    const uint32_t w[4] = {ux.x, ux.y, ux.z, ux.w};
+    const uint32_t d[4] = {ud.x, ud.y, ud.z, ud.w};
+    float v[E], g[E];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      Chunk<T>::widen(w[k], v + k * PD);
+      if (BWD) Chunk<T>::widen(d[k], g + k * PD);
+    }
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      const float a = BWD ? g[i] : v[i];
+      s[i] += a;
+      q[i] = fmaf(v[i], a, q[i]);
+    }
+    if (MINMAX) {
+      constexpr int LPG = 256 / E;
+      float lo = v[0], hi = v[0];
+#pragma unroll
+      for (int i = 1; i < E; ++i) { lo = fminf(lo, v[i]); hi = fmaxf(hi, v[i]); }
+      lo = rows_min<LPG / 16>(row16_min(lo));
+      hi = rows_max<LPG / 16>(row16_max(hi));
+      if ((threadIdx.x & (LPG - 1)) == LPG - 1) {
+        const int64_t g_index = (row * C + t.col) >> 8;
+        Conv<T>::store(mn, g_index, lo);
+        Conv<T>::store(mx, g_index, hi);
+      }
+    }
+  };
+
+  if (t.active) {
+    int64_t row = p0 + t.r;
+    for (; row + (int64_t)(U - 1) * R < p1; row += (int64_t)U * R) {
+      typename XS::Raw rx[U];
+      u32x4 ud[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        rx[u] = xs.fetch(row + (int64_t)u * R);
+        if (BWD) ud[u] = load16(pd + (row + (int64_t)u * R) * C);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const u32x4 ux = xs.decode(rx[u]);
+        accumulate(ux, BWD ? ud[u] : ux, row + (int64_t)u * R);
+      }
+    }
+    for (; row < p1; row += R) {
+      const typename XS::Raw rx = xs.fetch(row);
+      const u32x4 ux = xs.decode(rx);
+      accumulate(ux, BWD ? load16(pd + row * C) : ux, row);
+    }
+  }
+  // rows of the tile are folded in a fixed order; table: [channel][sum][block row]
+#pragma unroll
+  for (int i = 0; i < E; ++i) {
+    s_part[threadIdx.x * 2 * E + i] = t.active ? s[i] : 0.0f;
+    s_part[threadIdx.x * 2 * E + E + i] = t.active ? q[i] : 0.0f;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < tpr * 2 * E; i += kThreads) {
+    const int j = i / (2 * E), k = i % (2 * E);
+    const int64_t channel = (int64_t)blockIdx.x * 256 + j * E + k % E;
+    if (j * E < 256 && channel < C) {
+      float v = 0.0f;
+      for (int rr = 0; rr < R; ++rr) v += s_part[(rr * tpr + j) * 2 * E + k];
+      part[(channel * 2 + k / E) * gridDim.y + blockIdx.y] = v;
+    }
+  }
+}
+
+template <typename T, bool BWD, typename XS>
+__global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
+    XS xs, const T* __restrict__ dy, const float* __restrict__ coef, T* __restrict__ out,
+    int64_t P, int64_t C, int tpr, int R, int64_t ppb) {
+  constexpr int E = Chunk<T>::kElems;
+  constexpr int PD = Chunk<T>::kPerDword;
+  constexpr int NC = BWD ? 3 : 2;
+  constexpr int U = XS::kInFlight;
+  const RowTile t = row_tile<E>(C, tpr, R);
+  if (!t.active) return;               // whole quantisation groups leave together
+  xs.bind(t.col, C);
+  float ka[E], kb[E], kc[E];
+#pragma unroll
+  for (int i = 0; i < E; ++i) {
+    ka[i] = coef[NC * (t.col + i)];
+    kb[i] = coef[NC * (t.col + i) + 1];
+    kc[i] = BWD ? coef[NC * (t.col + i) + 2] : 0.0f;
+  }
+  const int64_t p0 = (int64_t)blockIdx.y * ppb;
+  const int64_t p1 = p0 + ppb < P ? p0 + ppb : P;
+
+  auto apply = [&](const u32x4& ux, const u32x4& ud) -> u32x4 {
+    const uint32_t w[4] = {ux.x, ux.y, ux.z, ux.w};
+    const uint32_t d[4] = {ud.x, ud.y, ud.z, ud.w};
+    uint32_t r[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float v[PD], g[PD], o[PD];
+      Chunk<T>::widen(w[k], v);
+      if (BWD) Chunk<T>::widen(d[k], g);
+#pragma unroll
+      for (int i = 0; i < PD; ++i) {
+        const int e = k * PD + i;
+        o[i] = BWD ? fmaf(g[i], ka[e], fmaf(v[i], kb[e], kc[e])) : fmaf(v[i], ka[e], kb[e]);
+      }
+      r[k] = Chunk<T>::narrow(o);
+    }
+    return u32x4{r[0], r[1], r[2], r[3]};
+  };
+
+  const T* pd = BWD ? dy + t.col : nullptr;
+  T* po = out + t.col;
+  int64_t row = p0 + t.r;
+  for (; row + (int64_t)(U - 1) * R < p1; row += (int64_t)U * R) {
+    typename XS::Raw rx[U];
+    u32x4 ud[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      rx[u] = xs.fetch(row + (int64_t)u * R);
+      if (BWD) ud[u] = load_last(pd + (row + (int64_t)u * R) * C);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const u32x4 ux = xs.decode(rx[u]);
+      store_out(po + (row + (int64_t)u * R) * C, apply(ux, BWD ? ud[u] : ux));
+    }
+  }
+  for (; row < p1; row += R) {
+    const typename XS::Raw rx = xs.fetch(row);
+    const u32x4 ux = xs.decode(rx);
+    store_out(po + row * C, apply(ux, BWD ? load_last(pd + row * C) : ux));
+  }
+}
+
 // Launch geometry shared by the passes of one call.
 struct Plan {
   int elems;           // elements per 16-byte chunk
@@ -457,9 +675,44 @@ struct Plan {
   int per_block, nsplit, slots;
   bool split;
   int64_t part_floats;
+  // channels-last: P rows, column tiles of 256, tpr threads per row, R rows per iteration,
+  // ppb rows per block, nsplit blocks along the rows (slots == 0 marks this table layout)
+  bool channels_last;
+  int64_t P, ppb;
+  int tiles, tpr, R;
+  bool groups_align;   // quantisation groups are aligned runs of threads
 };
+bool make_plan_cl(int64_t N, int64_t C, int64_t HW, int dtype, Plan& pl) {
+  if (N <= 0 || C <= 0 || HW <= 0 || dtype < 0 || dtype > 2) return false;
+  pl.channels_last = true;
+  pl.elems = dtype == ACTNN_F32 ? 4 : 8;
+  if (C % pl.elems != 0 || C > 0x7fffffffLL || HW > 0x7fffffffLL || N > ((int64_t)1 << 62) / (C * HW)) return false;
+  pl.F = C * HW;
+  pl.P = N * HW;
+  pl.tiles = (int)((C + 255) / 256);
+  pl.tpr = (int)((C < 256 ? C : 256) / pl.elems);
+  pl.R = kThreads / pl.tpr;
+  // One round of blocks (2048 fit on the chip at once) measured best here: the block's final
+  // reduction over its R rows is dearer than in the default layout.  At least 128 rows per block
+  // keep the table of partial sums below 3 % of the data.
+  constexpr int64_t target = 2048, min_ppb = 128;
+  const int64_t want = (target + pl.tiles - 1) / pl.tiles;
+  int64_t ppb = (pl.P + want - 1) / want;
+  if (ppb < min_ppb) ppb = min_ppb;
+  if (ppb < (pl.P + 65534) / 65535) ppb = (pl.P + 65534) / 65535;
+  ppb = (ppb + pl.R - 1) / pl.R * pl.R;
+  pl.ppb = ppb;
+  pl.nsplit = (int)((pl.P + ppb - 1) / ppb);
+  pl.slots = 0;
+  pl.split = false;
+  pl.part_floats = C * 2 * pl.nsplit;
+  pl.groups_align = pl.F % 256 == 0 && (C % 256 == 0 || 256 % C == 0);
+  pl.L = 0; pl.spans = 0; pl.per_block = 0;
+  return true;
+}
 bool make_plan(int64_t N, int64_t C, int64_t HW, int dtype, Plan& pl) {
   if (N <= 0 || C <= 0 || HW <= 0 || dtype < 0 || dtype > 2) return false;
+  pl.channels_last = false;
   pl.elems = dtype == ACTNN_F32 ? 4 : 8;
   if (HW < pl.elems || C > 0x7fffffffLL || C > ((int64_t)1 << 40) / HW) return false;
   pl.F = C * HW;
@@ -485,7 +738,11 @@ bool make_plan(int64_t N, int64_t C, int64_t HW, int dtype, Plan& pl) {
   pl.slots = (int)slots;
   pl.split = HW % pl.elems != 0;
   pl.part_floats = pl.spans * nsplit * slots * 2;
+  pl.groups_align = pl.F % 256 == 0;
   return true;
+}
+bool make_plan(int64_t N, int64_t C, int64_t HW, int dtype, int channels_last, Plan& pl) {
+  return channels_last ? make_plan_cl(N, C, HW, dtype, pl) : make_plan(N, C, HW, dtype, pl);
 }
 int64_t workspace_floats(const Plan& pl, int64_t C) { return pl.part_floats + 3 * C; }
 
@@ -515,18 +772,44 @@ void launch_apply(const Plan& pl, const XS& xs, const void* dy, const float* coe
     bn_apply_kernel<T, false, BWD, XS><<<grid, blk, 0, s>>>(xs, pd, coef, po, N, pl.F, HW, pl.per_block);
 }
 
+template <typename T, bool BWD, bool MINMAX, typename XS>
+void launch_cl_reduce(const Plan& pl, const XS& xs, const void* dy, float* part, void* mn, void* mx,
+                      int64_t C, hipStream_t s) {
+  const dim3 grid((unsigned)pl.tiles, (unsigned)pl.nsplit), blk(kThreads);
+  bn_cl_reduce_kernel<T, BWD, MINMAX, XS><<<grid, blk, 0, s>>>(
+      xs, static_cast<const T*>(dy), part, static_cast<T*>(mn), static_cast<T*>(mx), pl.P, C, pl.tpr, pl.R, pl.ppb);
+}
+template <typename T, bool BWD, typename XS>
+void launch_cl_apply(const Plan& pl, const XS& xs, const void* dy, const float* coef, void* out, int64_t C,
+                     hipStream_t s) {
+  const dim3 grid((unsigned)pl.tiles, (unsigned)pl.nsplit), blk(kThreads);
+  bn_cl_apply_kernel<T, BWD, XS><<<grid, blk, 0, s>>>(xs, static_cast<const T*>(dy), coef,
+                                                      static_cast<T*>(out), pl.P, C, pl.tpr, pl.R, pl.ppb);
+}
+
 template <typename T>
 int forward_t(const Plan& pl, const void* x, const float* weight, const float* bias, float* running_mean,
               float* running_var, void* y, float* save_mean, float* save_invstd, void* mn, void* mx,
               float* ws, int64_t N, int64_t C, int64_t HW, double momentum, double eps, hipStream_t s) {
   float* part = ws;
   float* coef = ws + pl.part_floats;
+  const dim3 fin((unsigned)((C + kWaves - 1) / kWaves)), blk(kThreads);
+  if (pl.channels_last) {
+    const PlainRows<T> xs{static_cast<const T*>(x), C};
+    if (mn) launch_cl_reduce<T, false, true>(pl, xs, nullptr, part, mn, mx, C, s);
+    else launch_cl_reduce<T, false, false>(pl, xs, nullptr, part, nullptr, nullptr, C, s);
+    bn_forward_finalize_kernel<<<fin, blk, 0, s>>>(part, weight, bias, running_mean, running_var, save_mean,
+                                                   save_invstd, coef, N, C, HW, pl.L, pl.nsplit, pl.slots,
+                                                   momentum, eps);
+    launch_cl_apply<T, false>(pl, xs, nullptr, coef, y, C, s);
+    ACTNN_RETURN_LAUNCH_STATUS();
+  }
   const PlainInput<T> xs{static_cast<const T*>(x), pl.F};
   if (mn) launch_reduce<T, false, true>(pl, xs, nullptr, part, mn, mx, N, HW, s);
   else launch_reduce<T, false, false>(pl, xs, nullptr, part, nullptr, nullptr, N, HW, s);
-  bn_forward_finalize_kernel<<<dim3((unsigned)((C + kWaves - 1) / kWaves)), dim3(kThreads), 0, s>>>(
-      part, weight, bias, running_mean, running_var, save_mean, save_invstd, coef, N, C, HW, pl.L,
-      pl.nsplit, pl.slots, momentum, eps);
+  bn_forward_finalize_kernel<<<fin, blk, 0, s>>>(part, weight, bias, running_mean, running_var, save_mean,
+                                                 save_invstd, coef, N, C, HW, pl.L, pl.nsplit, pl.slots,
+                                                 momentum, eps);
   launch_apply<T, false>(pl, xs, nullptr, coef, y, N, HW, s);
   ACTNN_RETURN_LAUNCH_STATUS();
 }
@@ -537,10 +820,14 @@ int backward_t(const Plan& pl, const XS& xs, const void* dy, const float* weight
                int64_t C, int64_t HW, hipStream_t s) {
   float* part = ws;
   float* coef = ws + pl.part_floats;
-  launch_reduce<T, true, false>(pl, xs, dy, part, nullptr, nullptr, N, HW, s);
+  if constexpr (XS::kRows) launch_cl_reduce<T, true, false>(pl, xs, dy, part, nullptr, nullptr, C, s);
+  else launch_reduce<T, true, false>(pl, xs, dy, part, nullptr, nullptr, N, HW, s);
   bn_backward_finalize_kernel<<<dim3((unsigned)((C + kWaves - 1) / kWaves)), dim3(kThreads), 0, s>>>(
       part, weight, save_mean, save_invstd, dweight, dbias, coef, N, C, HW, pl.L, pl.nsplit, pl.slots);
-  if (dx) launch_apply<T, true>(pl, xs, dy, coef, dx, N, HW, s);
+  if (dx) {
+    if constexpr (XS::kRows) launch_cl_apply<T, true>(pl, xs, dy, coef, dx, C, s);
+    else launch_apply<T, true>(pl, xs, dy, coef, dx, N, HW, s);
+  }
   ACTNN_RETURN_LAUNCH_STATUS();
 }
 
@@ -548,6 +835,10 @@ template <typename T>
 int backward_plain(const Plan& pl, const void* x, const void* dy, const float* weight, const float* save_mean,
                    const float* save_invstd, void* dx, float* dweight, float* dbias, float* ws, int64_t N,
                    int64_t C, int64_t HW, hipStream_t s) {
+  if (pl.channels_last) {
+    const PlainRows<T> xs{static_cast<const T*>(x), C};
+    return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+  }
   const PlainInput<T> xs{static_cast<const T*>(x), pl.F};
   return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
 }
@@ -557,17 +848,22 @@ int backward_packed(const Plan& pl, const int32_t* packed, const int32_t* bits, 
                     const void* scale, const void* mn, const void* dy, const float* weight,
                     const float* save_mean, const float* save_invstd, void* dx, float* dweight,
                     float* dbias, float* ws, int64_t N, int64_t C, int64_t HW, hipStream_t s) {
-  const PackedInput<T> xs{packed, bits, prefix, static_cast<const T*>(scale), static_cast<const T*>(mn),
+  const PackedInput<T> in{packed, bits, prefix, static_cast<const T*>(scale), static_cast<const T*>(mn),
                           pl.F / 256, 0, 0u, false};
-  return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+  if (pl.channels_last) {
+    const PackedRows<T> xs{in, C, 0, (uint32_t)HW};
+    return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+  }
+  return backward_t<T>(pl, in, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
 }
 
 }  // namespace
 }  // namespace actnn
 
-extern "C" int64_t actnn_batch_norm_workspace_bytes(int64_t N, int64_t C, int64_t HW, int dtype) {
+extern "C" int64_t actnn_batch_norm_workspace_bytes(int64_t N, int64_t C, int64_t HW, int dtype,
+                                                    int channels_last) {
   actnn::Plan pl;
-  if (!actnn::make_plan(N, C, HW, dtype, pl)) return -1;
+  if (!actnn::make_plan(N, C, HW, dtype, channels_last, pl)) return -1;
   return actnn::workspace_floats(pl, C) * (int64_t)sizeof(float);
 }
 
@@ -575,14 +871,15 @@ extern "C" int actnn_batch_norm_forward(const void* x, const float* weight, cons
                                         float* running_mean, float* running_var, void* y,
                                         float* save_mean, float* save_invstd, void* mn, void* mx,
                                         void* workspace, int64_t workspace_bytes, int64_t N, int64_t C,
-                                        int64_t HW, double momentum, double eps, int dtype, void* stream) {
+                                        int64_t HW, double momentum, double eps, int dtype,
+                                        int channels_last, void* stream) {
   using namespace actnn;
   if (dtype < 0 || dtype > 2) return ACTNN_EDTYPE;
   Plan pl;
-  if (!make_plan(N, C, HW, dtype, pl)) return ACTNN_EINVAL;
+  if (!make_plan(N, C, HW, dtype, channels_last, pl)) return ACTNN_EINVAL;
   if (!x || !y || !save_mean || !save_invstd || !workspace || (mn == nullptr) != (mx == nullptr)) return ACTNN_EINVAL;
   if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
-  if (mn && pl.F % 256 != 0) return ACTNN_EINVAL;
+  if (mn && !pl.groups_align) return ACTNN_EINVAL;
   if (!aligned16(x) || !aligned16(y) || !aligned16(workspace)) return ACTNN_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   float* ws = static_cast<float*>(workspace);
@@ -597,11 +894,11 @@ extern "C" int actnn_batch_norm_backward(const void* x, const void* dy, const fl
                                          const float* save_mean, const float* save_invstd, void* dx,
                                          float* dweight, float* dbias, void* workspace,
                                          int64_t workspace_bytes, int64_t N, int64_t C, int64_t HW,
-                                         int dtype, void* stream) {
+                                         int dtype, int channels_last, void* stream) {
   using namespace actnn;
   if (dtype < 0 || dtype > 2) return ACTNN_EDTYPE;
   Plan pl;
-  if (!make_plan(N, C, HW, dtype, pl)) return ACTNN_EINVAL;
+  if (!make_plan(N, C, HW, dtype, channels_last, pl)) return ACTNN_EINVAL;
   if (!x || !dy || !save_mean || !save_invstd || !workspace) return ACTNN_EINVAL;
   if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
   if (!aligned16(x) || !aligned16(dy) || (dx && !aligned16(dx)) || !aligned16(workspace)) return ACTNN_EALIGN;
@@ -620,11 +917,13 @@ extern "C" int actnn_batch_norm_backward_packed(const int32_t* packed, const int
                                                 const float* save_mean, const float* save_invstd,
                                                 void* dx, float* dweight, float* dbias, void* workspace,
                                                 int64_t workspace_bytes, int64_t N, int64_t C,
-                                                int64_t HW, int dtype, void* stream) {
+                                                int64_t HW, int dtype, int channels_last,
+                                                void* stream) {
   using namespace actnn;
   if (dtype != ACTNN_F16 && dtype != ACTNN_BF16) return ACTNN_EDTYPE;
   Plan pl;
-  if (!make_plan(N, C, HW, dtype, pl) || pl.F % 256 != 0) return ACTNN_EINVAL;
+  if (!make_plan(N, C, HW, dtype, channels_last, pl) || !pl.groups_align) return ACTNN_EINVAL;
+  if (channels_last && pl.P > 0x7fffffffLL) return ACTNN_EINVAL;
   if (!packed || !bits || !prefix || !scale || !mn || !dy || !save_mean || !save_invstd || !workspace) return ACTNN_EINVAL;
   if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
   if (!aligned16(dy) || (dx && !aligned16(dx)) || !aligned16(workspace)) return ACTNN_EALIGN;

@@ -301,10 +301,8 @@ class linear(Function):
 # batch norm (ops.py:436-502)
 # ------------------------------------------------------------------------------------------
 def _bn_shares_min_max(input, weight, bias, running_mean, running_var, training):
-    features = input.numel() // max(input.shape[0], 1)
-    return (training and config.compress_activation and not config.simulate
-            and config.group_size == 256 and features % 256 == 0
-            and ext_backward_func.hip_batch_norm_applies(input, weight, bias, running_mean, running_var))
+    return (training and config.compress_activation and not config.simulate and config.group_size == 256
+            and ext_backward_func.hip_batch_norm_minmax_applies(input, weight, bias, running_mean, running_var))
 
 
 class batch_norm(Function):
@@ -345,9 +343,9 @@ class batch_norm(Function):
     def backward(ctx, grad_output):
         quantized, weight, running_mean, running_var, save_mean, save_var, training, eps, reserve = ctx.saved
         if (training and config.compress_activation and not config.simulate and not config.swap
-                and config.group_size == 256 and config.fused_bn_backward
-                and getattr(quantized, "memory_format", None) is None):
-            grad_output = grad_output.contiguous()
+                and config.group_size == 256 and config.fused_bn_backward):
+            grad_output = grad_output.contiguous(
+                memory_format=getattr(quantized, "memory_format", None) or torch.contiguous_format)
             if ext_backward_func.hip_batch_norm_backward_packed_applies(
                     ctx.other_args, quantized, grad_output, weight, save_mean, save_var):
                 # the kernels decode the saved input from its bit stream: no full-precision copy

@@ -172,35 +172,40 @@ int actnn_linear_grad_weight_q2(const void* grad_out, const int8_t* packed, cons
                                 int go_dtype, int sm_dtype, int out_dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------
- * Training-mode batch normalisation over a contiguous [N, C, HW] tensor (HW = 1 for [N, C]
- * inputs is not covered: HW >= 4 for f32, >= 8 for 16-bit types, and C*HW a multiple of that).
+ * Training-mode batch normalisation over a dense tensor of N samples, C channels and HW
+ * positions, laid out [N, C, HW] (channels_last = 0; HW >= 4 for f32, >= 8 for 16-bit types and
+ * C*HW a multiple of that - [N, C] inputs with HW = 1 are not covered) or [N, HW, C]
+ * (channels_last = 1, the layout of this GPU's convolution kernels; C a multiple of 4 / 8).
  * Replaces the two cuDNN calls the reference re-exports, at::cudnn_batch_norm and
  * at::cudnn_batch_norm_backward (cpp_extension/backward_func.cc:87-88; callers ops.py:448-449
  * and ops.py:479-481).  weight/bias (may be null = 1/0), running_* (may be null), save_* and
  * the gradients of weight/bias are fp32[C]; x, y, dy, dx are `dtype`.
  * forward: batch mean and biased variance per channel, y = (x - mean) * invstd * weight + bias,
  * running_mean/var updated in place with `momentum` (variance unbiased), save_mean/save_invstd
- * written.  When mn/mx are given (both or neither; needs C*HW % 256 == 0) the per-group minimum
+ * written.  When mn/mx are given (both or neither; needs C*HW % 256 == 0, and for channels_last
+ * C % 256 == 0 or 256 % C == 0) the per-group minimum
  * and maximum of x over groups of 256 consecutive elements of a sample - what actnn_minimax
  * returns for x viewed as [N*C*HW/256, 256] - are written as well, from the same read of x.
  * backward: dx, dweight, dbias from x, dy and the saved statistics (dx may be null).
  * `workspace`: device scratch of actnn_batch_norm_workspace_bytes(...) bytes (16-byte aligned;
  * -1 = shape not supported), contents undefined before and after.
  * ------------------------------------------------------------------------------- */
-int64_t actnn_batch_norm_workspace_bytes(int64_t N, int64_t C, int64_t HW, int dtype);
+int64_t actnn_batch_norm_workspace_bytes(int64_t N, int64_t C, int64_t HW, int dtype,
+                                         int channels_last);
 int actnn_batch_norm_forward(const void* x, const float* weight, const float* bias,
                              float* running_mean, float* running_var, void* y, float* save_mean,
                              float* save_invstd, void* mn, void* mx, void* workspace,
                              int64_t workspace_bytes, int64_t N, int64_t C, int64_t HW,
-                             double momentum, double eps, int dtype, void* stream);
+                             double momentum, double eps, int dtype, int channels_last,
+                             void* stream);
 int actnn_batch_norm_backward(const void* x, const void* dy, const float* weight,
                               const float* save_mean, const float* save_invstd, void* dx,
                               float* dweight, float* dbias, void* workspace,
                               int64_t workspace_bytes, int64_t N, int64_t C, int64_t HW, int dtype,
-                              void* stream);
+                              int channels_last, void* stream);
 
 /* The same backward pass with x held as the mixed-precision stream of actnn_pack_mixed (group
- * size 256, C*HW % 256 == 0, 16-bit dtype; bits / prefix / scale / mn as for actnn_unpack_mixed):
+ * size 256 over the sample in memory order, the conditions of mn/mx above, 16-bit dtype; bits / prefix / scale / mn as for actnn_unpack_mixed):
  * both passes rebuild x in registers, bit for bit what actnn_unpack_mixed would write, so the
  * full-precision copy of x that ops.py:478 (dequantize_activation before
  * cudnn_batch_norm_backward) materialises never exists. */
@@ -209,7 +214,8 @@ int actnn_batch_norm_backward_packed(const int32_t* packed, const int32_t* bits,
                                      const void* dy, const float* weight, const float* save_mean,
                                      const float* save_invstd, void* dx, float* dweight,
                                      float* dbias, void* workspace, int64_t workspace_bytes,
-                                     int64_t N, int64_t C, int64_t HW, int dtype, void* stream);
+                                     int64_t N, int64_t C, int64_t HW, int dtype,
+                                     int channels_last, void* stream);
 
 /* Plain device-to-device streaming copy of `bytes` bytes (16-byte aligned pointers and
  * size); used by the benchmark to calibrate bandwidth counters.  No reference counterpart. */

@@ -147,3 +147,86 @@ def test_backward_from_the_packed_stream_equals_unpack_then_backward(N, C, spati
     got = ext_bf.hip_batch_norm_backward_packed(x.shape, quantized, dy, w, mean, invstd)
     for a, r in zip(got, ref):
         assert torch.equal(a, r)
+
+
+# ------------------------------------------------------------------------------------------
+# channels-last tensors ([N, HW, C] in memory)
+# ------------------------------------------------------------------------------------------
+def _cl(t):
+    return t.contiguous(memory_format=torch.channels_last if t.dim() == 4 else torch.channels_last_3d)
+
+
+CL_SHAPES = [(8, 64, (56, 56)), (16, 256, (7, 7)), (5, 32, (28, 28)), (37, 24, (14, 14)),
+             (4, 2048, (7, 7)), (3, 320, (5, 5)), (2, 16, (3, 4, 5)), (70, 8, (8, 8)), (2, 512, (28, 28))]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,C,spatial", CL_SHAPES)
+def test_channels_last_forward_backward_against_float64(N, C, spatial, dtype):
+    x, w, b, rm, rv, dy = _inputs(N, C, spatial, dtype, N * 1000 + C + 1)
+    x, dy = _cl(x), _cl(dy)
+    assert ext_bf.hip_batch_norm_applies(x, w, b, rm, rv)
+    rm0, rv0 = rm.clone(), rv.clone()
+    y, mean, invstd, _ = ext_bf.cudnn_batch_norm(x, w, b, rm, rv, True, 0.1, 1e-5)
+    assert y.stride() == x.stride()
+    yo, mean_o, invstd_o, rm_o, rv_o = o_bn.forward(
+        x.double().cpu().numpy(), w.cpu().numpy(), b.cpu().numpy(), rm0.cpu().numpy(), rv0.cpu().numpy(), 0.1, 1e-5)
+    assert np.allclose(mean.cpu().numpy(), mean_o, rtol=1e-5, atol=1e-6)
+    assert np.allclose(invstd.cpu().numpy(), invstd_o, rtol=2e-5)
+    assert np.allclose(rm.cpu().numpy(), rm_o, rtol=1e-5, atol=1e-6)
+    assert np.allclose(rv.cpu().numpy(), rv_o, rtol=2e-5)
+    err = np.abs(y.double().cpu().numpy() - yo)
+    assert (err <= RND[dtype] * (np.abs(yo) + 4.0)).all(), float(err.max())
+    gi, gw, gb = ext_bf.cudnn_batch_norm_backward(x, dy, w, rm, rv, mean, invstd, 1e-5, None)
+    assert gi.stride() == x.stride()
+    gi_o, gw_o, gb_o = o_bn.backward(x.double().cpu().numpy(), dy.double().cpu().numpy(), w.cpu().numpy(), 1e-5)
+    scale = np.sqrt(x.numel() / C)
+    assert np.allclose(gb.cpu().numpy(), gb_o, rtol=1e-5, atol=2e-5 * scale)
+    assert np.allclose(gw.cpu().numpy(), gw_o, rtol=1e-5, atol=4e-5 * scale)
+    err = np.abs(gi.double().cpu().numpy() - gi_o)
+    assert (err <= RND[dtype] * (np.abs(gi_o) + 4.0)).all(), float(err.max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,C,spatial", [(8, 64, (56, 56)), (5, 256, (7, 7)), (9, 128, (14, 14)),
+                                         (3, 8, (8, 4)), (2, 512, (6, 6)), (3, 2048, (7, 7))])
+def test_channels_last_group_min_max(N, C, spatial, dtype):
+    from actnn_amd.utils import memory_order
+    x, w, b, rm, rv, _ = _inputs(N, C, spatial, dtype, 12)
+    x = _cl(x)
+    assert ext_bf.hip_batch_norm_minmax_applies(x, w, b, rm, rv)
+    y0, m0, i0, _, _ = ext_bf.hip_batch_norm_forward(x, w, b, rm.clone(), rv.clone(), 0.1, 1e-5)
+    y, m, i, mn, mx = ext_bf.hip_batch_norm_forward(x, w, b, rm.clone(), rv.clone(), 0.1, 1e-5, minmax=True)
+    mn_ref, mx_ref = ext_minimax.minimax(memory_order(x).reshape(-1, 256))
+    assert torch.equal(mn, mn_ref.view(-1)) and torch.equal(mx, mx_ref.view(-1))
+    assert torch.equal(y, y0) and torch.equal(m, m0) and torch.equal(i, i0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,C,spatial", [(8, 64, (56, 56)), (16, 256, (7, 7)), (37, 128, (14, 14)),
+                                         (9, 32, (4, 2)), (5, 1024, (6, 6))])
+def test_channels_last_backward_from_the_packed_stream(N, C, spatial, dtype):
+    import actnn_amd.cpp_extension.quantization as ext_q
+    from actnn_amd.ops import _Quantized
+    from actnn_amd.utils import logical_order, memory_order
+    from _util import bits_tensor
+    x, w, b, rm, rv, dy = _inputs(N, C, spatial, dtype, 22)
+    x, dy = _cl(x), _cl(dy)
+    G = x[0].numel() // 256
+    groups = memory_order(x).reshape(N, G, 256)
+    mn, mx = ext_minimax.minimax(groups.view(-1, 256))
+    mn, mx = mn.view(N, G, 1), mx.view(N, G, 1)
+    bits_dev, _ = bits_tensor([1 + (3 * i + i // 8) % 8 for i in range(N)])
+    torch.cuda.manual_seed(5)
+    packed, scale = ext_q.pack_mixed_precision(groups, mn, mx, bits_dev, True)
+    _, mean, invstd, _, _ = ext_bf.hip_batch_norm_forward(x, w, b, None, None, 0.1, 1e-5)
+    xq = ext_q.unpack_mixed_precision(packed, bits_dev, scale, mn, N, G, 256)
+    xq = logical_order(xq.view(N, *spatial, C), torch.channels_last)
+    ref = ext_bf.hip_batch_norm_backward(xq, dy, w, mean, invstd)
+    quantized = _Quantized((packed, bits_dev, scale, mn))
+    quantized.memory_format = torch.channels_last
+    assert ext_bf.hip_batch_norm_backward_packed_applies(x.shape, quantized, dy, w, mean, invstd)
+    got = ext_bf.hip_batch_norm_backward_packed(x.shape, quantized, dy, w, mean, invstd)
+    assert got[0].stride() == x.stride()
+    for a, r in zip(got, ref):
+        assert torch.equal(a, r)
