@@ -8,6 +8,7 @@ from torch.autograd import Function
 
 from . import _glue as g
 from .._lib import check
+from ..utils import channels_last_format
 
 MASK_BLOCK = 512
 
@@ -315,15 +316,27 @@ def _pair_check(v, name):
     return v
 
 
+def pool_takes_channels_last(x):
+    """True for a channels-last tensor the [N, H, W, C] kernels take (whole 16-byte chunks of channels)."""
+    return (channels_last_format(x) is not None and x.shape[1] % (16 // x.element_size()) == 0
+            and x.data_ptr() % 16 == 0)
+
+
 def max_pool2d_forward(x, kernel_size, stride, padding, dilation):
+    """-> (y, idx) in the memory format of x (default or channels-last)."""
     N, C, H, W = x.shape
     KH, KW = kernel_size
     Ho = (H + 2 * padding[0] - dilation[0] * (KH - 1) - 1) // stride[0] + 1       # .cu:679
     Wo = (W + 2 * padding[1] - dilation[1] * (KW - 1) - 1) // stride[1] + 1       # .cu:680
-    y = torch.empty(N, C, Ho, Wo, dtype=x.dtype, device=x.device)
-    idx = torch.empty(N, C, Ho, Wo, dtype=torch.int8, device=x.device)
+    channels_last = pool_takes_channels_last(x)
+    fmt = torch.channels_last if channels_last else torch.contiguous_format
+    if not channels_last:
+        x = x.contiguous()
+    y = torch.empty((N, C, Ho, Wo), dtype=x.dtype, device=x.device, memory_format=fmt)
+    idx = torch.empty((N, C, Ho, Wo), dtype=torch.int8, device=x.device, memory_format=fmt)
+    fn = g.lib().actnn_max_pool2d_forward_cl if channels_last else g.lib().actnn_max_pool2d_forward
     with torch.cuda.device(x.device):
-        check(g.lib().actnn_max_pool2d_forward(
+        check(fn(
             x.data_ptr(), y.data_ptr(), idx.data_ptr(), N, C, H, W, Ho, Wo, KH, KW, stride[0],
             stride[1], padding[0], padding[1], g.DTYPE_CODE[x.dtype], g.stream_ptr(x.device)),
             "max_pool2d_forward")
@@ -331,12 +344,16 @@ def max_pool2d_forward(x, kernel_size, stride, padding, dilation):
 
 
 def max_pool2d_backward(grad_output, idx, input_shape, kernel_size, stride, padding):
-    grad_output = grad_output.contiguous()
+    """The gradient comes back in the memory format of `idx` (the format of the forward input)."""
+    channels_last = channels_last_format(idx) is not None
+    fmt = torch.channels_last if channels_last else torch.contiguous_format
+    grad_output = grad_output.contiguous(memory_format=fmt)
     N, C, H, W = input_shape
     Ho, Wo = grad_output.shape[2], grad_output.shape[3]
-    gin = torch.empty(N, C, H, W, dtype=grad_output.dtype, device=grad_output.device)
+    gin = torch.empty((N, C, H, W), dtype=grad_output.dtype, device=grad_output.device, memory_format=fmt)
+    fn = g.lib().actnn_max_pool2d_backward_cl if channels_last else g.lib().actnn_max_pool2d_backward
     with torch.cuda.device(gin.device):
-        check(g.lib().actnn_max_pool2d_backward(
+        check(fn(
             grad_output.data_ptr(), idx.data_ptr(), gin.data_ptr(), N, C, H, W, Ho, Wo,
             kernel_size[0], kernel_size[1], stride[0], stride[1], padding[0], padding[1],
             g.DTYPE_CODE[gin.dtype], g.stream_ptr(gin.device)), "max_pool2d_backward")
@@ -374,6 +391,7 @@ class ActQuantizedMaxPool2d(Function):
 
 
 def act_quantized_max_pool2d(input, kernel_size, stride, padding, dilation, ceil_mode, return_indices):
-    g.check_float(input, "input")                                                  # quantization.cc:194
+    if not (isinstance(input, torch.Tensor) and input.is_cuda and input.dim() == 4 and pool_takes_channels_last(input)):
+        g.check_float(input, "input")                                              # quantization.cc:194
     return ActQuantizedMaxPool2d.apply(input, kernel_size, stride, padding, dilation, ceil_mode,
                                        return_indices)

@@ -546,6 +546,138 @@ int launch_bwd(const void* gout, const int8_t* idx, void* gin, int64_t total, co
   ACTNN_RETURN_LAUNCH_STATUS();
 }
 
+// ------------------------------------------------------------------ channels-last ([N, H, W, C])
+// A thread owns one 16-byte chunk of channels of one pixel; consecutive threads take consecutive
+// chunks, then the next pixel, so every access of a wave is a run of whole cache lines and the
+// overlap between neighbouring windows is served by the caches.  Same scan order and strict
+// compare as the default-layout kernels, hence the same values and indices.
+template <typename T> struct PoolChunk;
+template <> struct PoolChunk<float> { static constexpr int kElems = 4; };
+template <> struct PoolChunk<__half> { static constexpr int kElems = 8; };
+template <> struct PoolChunk<bf16_t> { static constexpr int kElems = 8; };
+
+template <typename T, int E> ACTNN_DEV void widen_chunk(const T* p, float (&v)[E]) {
+  if constexpr (E == 4) {
+    const u32x4 u = load16(p);
+    v[0] = as_float(u.x); v[1] = as_float(u.y); v[2] = as_float(u.z); v[3] = as_float(u.w);
+  } else {
+    load8(p, v);
+  }
+}
+template <typename T, int E> ACTNN_DEV void narrow_chunk(T* p, const float (&v)[E]) {
+  if constexpr (E == 4) store16(p, u32x4{as_uint(v[0]), as_uint(v[1]), as_uint(v[2]), as_uint(v[3])});
+  else store8(p, v);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void max_pool2d_forward_cl_kernel(
+    const T* __restrict__ x, T* __restrict__ y, int8_t* __restrict__ idx, int64_t chunks, int cpp /* chunks per pixel */,
+    int64_t C, PoolGeom g) {
+  constexpr int E = PoolChunk<T>::kElems;
+  const int64_t id = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (id >= chunks) return;
+  const int c = (int)(id % cpp) * E;
+  const int64_t pix = id / cpp;
+  const int w = (int)(pix % g.Wo);
+  const int h = (int)((pix / g.Wo) % g.Ho);
+  const int64_t n = pix / ((int64_t)g.Wo * g.Ho);
+  const int h_base = h * g.SH - g.PH, w_base = w * g.SW - g.PW;
+  const int h_start = h_base > 0 ? h_base : 0, h_end = h_base + g.KH < g.H ? h_base + g.KH : g.H;
+  const int w_start = w_base > 0 ? w_base : 0, w_end = w_base + g.KW < g.W ? w_base + g.KW : g.W;
+  float best[E];
+  int where[E];
+  const float init = Conv<T>::round(-1e10f);      // .cu:656, narrowed to the element type
+#pragma unroll
+  for (int e = 0; e < E; ++e) { best[e] = init; where[e] = 0; }
+  const T* img = x + n * (int64_t)g.H * g.W * C + c;
+  for (int i = h_start; i < h_end; ++i) {
+    for (int j = w_start; j < w_end; ++j) {
+      float v[E];
+      widen_chunk<T, E>(img + ((int64_t)i * g.W + j) * C, v);
+      const int k = (i - h_base) * g.KW + (j - w_base);
+#pragma unroll
+      for (int e = 0; e < E; ++e)
+        if (v[e] > best[e]) { best[e] = v[e]; where[e] = k; }
+    }
+  }
+  narrow_chunk<T, E>(y + pix * C + c, best);
+  uint32_t packed[E / 4];
+#pragma unroll
+  for (int q = 0; q < E / 4; ++q)
+    packed[q] = (uint32_t)where[4 * q] | ((uint32_t)where[4 * q + 1] << 8) | ((uint32_t)where[4 * q + 2] << 16) |
+                ((uint32_t)where[4 * q + 3] << 24);
+  uint32_t* out = reinterpret_cast<uint32_t*>(idx + pix * C + c);
+#pragma unroll
+  for (int q = 0; q < E / 4; ++q) out[q] = packed[q];
+}
+
+// Gather form of the backward pass: every input position sums the gradients of the windows that
+// chose it, in a fixed order (no atomics, no zero fill).
+template <typename T>
+__global__ __launch_bounds__(kThreads) void max_pool2d_backward_cl_kernel(
+    const T* __restrict__ gout, const int8_t* __restrict__ idx, T* __restrict__ gin, int64_t chunks, int cpp,
+    int64_t C, PoolGeom g) {
+  constexpr int E = PoolChunk<T>::kElems;
+  const int64_t id = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (id >= chunks) return;
+  const int c = (int)(id % cpp) * E;
+  const int64_t pix = id / cpp;
+  const int w = (int)(pix % g.W);
+  const int h = (int)((pix / g.W) % g.H);
+  const int64_t n = pix / ((int64_t)g.W * g.H);
+  int ho_lo = h + g.PH - g.KH + 1;
+  ho_lo = ho_lo > 0 ? (ho_lo + g.SH - 1) / g.SH : 0;
+  int ho_hi = (h + g.PH) / g.SH;
+  ho_hi = ho_hi < g.Ho - 1 ? ho_hi : g.Ho - 1;
+  int wo_lo = w + g.PW - g.KW + 1;
+  wo_lo = wo_lo > 0 ? (wo_lo + g.SW - 1) / g.SW : 0;
+  int wo_hi = (w + g.PW) / g.SW;
+  wo_hi = wo_hi < g.Wo - 1 ? wo_hi : g.Wo - 1;
+  float acc[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) acc[e] = 0.0f;
+  const int64_t obase = n * (int64_t)g.Ho * g.Wo;
+  for (int ho = ho_lo; ho <= ho_hi; ++ho) {
+    const int kh = h - (ho * g.SH - g.PH);
+    for (int wo = wo_lo; wo <= wo_hi; ++wo) {
+      const int k = kh * g.KW + (w - (wo * g.SW - g.PW));
+      const int64_t o = (obase + (int64_t)ho * g.Wo + wo) * C + c;
+      float v[E];
+      widen_chunk<T, E>(gout + o, v);
+      const uint32_t* pi = reinterpret_cast<const uint32_t*>(idx + o);
+#pragma unroll
+      for (int q = 0; q < E / 4; ++q) {
+        const uint32_t word = pi[q];
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          if ((int)((word >> (8 * b)) & 0xffu) == k) acc[4 * q + b] += v[4 * q + b];
+      }
+    }
+  }
+  narrow_chunk<T, E>(gin + pix * C + c, acc);
+}
+
+template <typename T>
+int launch_cl(bool forward, const void* a, const int8_t* idx_in, int8_t* idx_out, void* out, int64_t N, int64_t C,
+              const PoolGeom& g, hipStream_t s) {
+  constexpr int E = PoolChunk<T>::kElems;
+  if (C % E != 0 || C / E > 0x7fffffffLL) return ACTNN_EINVAL;
+  if (!aligned16(a) || !aligned16(out)) return ACTNN_EALIGN;
+  const int cpp = (int)(C / E);
+  const int64_t pixels = forward ? N * g.Ho * g.Wo : N * (int64_t)g.H * g.W;
+  const int64_t chunks = pixels * cpp;
+  const int64_t blocks = (chunks + kThreads - 1) / kThreads;
+  if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
+  if (blocks == 0) return ACTNN_OK;
+  if (forward)
+    max_pool2d_forward_cl_kernel<T><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+        static_cast<const T*>(a), static_cast<T*>(out), idx_out, chunks, cpp, C, g);
+  else
+    max_pool2d_backward_cl_kernel<T><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+        static_cast<const T*>(a), idx_in, static_cast<T*>(out), chunks, cpp, C, g);
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
+
 int check_geom(int64_t N, int64_t C, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH, int KW,
                int SH, int SW, int PH, int PW) {
   if (N < 0 || C < 0 || H < 1 || W < 1 || Ho < 0 || Wo < 0) return ACTNN_EINVAL;
@@ -596,6 +728,43 @@ extern "C" int actnn_max_pool2d_backward(const void* grad_out, const int8_t* idx
     case ACTNN_F32: return launch_bwd<float>(grad_out, idx, grad_in, total, g, s);
     case ACTNN_F16: return launch_bwd<__half>(grad_out, idx, grad_in, total, g, s);
     case ACTNN_BF16: return launch_bwd<bf16_t>(grad_out, idx, grad_in, total, g, s);
+    default: return ACTNN_EDTYPE;
+  }
+}
+
+extern "C" int actnn_max_pool2d_forward_cl(const void* x, void* y, int8_t* idx, int64_t N, int64_t C,
+                                           int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH, int KW,
+                                           int SH, int SW, int PH, int PW, int dtype, void* stream) {
+  using namespace actnn;
+  const int rc = check_geom(N, C, H, W, Ho, Wo, KH, KW, SH, SW, PH, PW);
+  if (rc != ACTNN_OK) return rc;
+  if (N * C * Ho * Wo == 0) return ACTNN_OK;
+  if (!x || !y || !idx) return ACTNN_EINVAL;
+  const PoolGeom g{(int)H, (int)W, (int)Ho, (int)Wo, KH, KW, SH, SW, PH, PW};
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case ACTNN_F32: return launch_cl<float>(true, x, nullptr, idx, y, N, C, g, s);
+    case ACTNN_F16: return launch_cl<__half>(true, x, nullptr, idx, y, N, C, g, s);
+    case ACTNN_BF16: return launch_cl<bf16_t>(true, x, nullptr, idx, y, N, C, g, s);
+    default: return ACTNN_EDTYPE;
+  }
+}
+
+extern "C" int actnn_max_pool2d_backward_cl(const void* grad_out, const int8_t* idx, void* grad_in,
+                                            int64_t N, int64_t C, int64_t H, int64_t W, int64_t Ho,
+                                            int64_t Wo, int KH, int KW, int SH, int SW, int PH, int PW,
+                                            int dtype, void* stream) {
+  using namespace actnn;
+  const int rc = check_geom(N, C, H, W, Ho, Wo, KH, KW, SH, SW, PH, PW);
+  if (rc != ACTNN_OK) return rc;
+  if (N * C * H * W == 0) return ACTNN_OK;
+  if (!grad_out || !grad_in || !idx) return ACTNN_EINVAL;
+  const PoolGeom g{(int)H, (int)W, (int)Ho, (int)Wo, KH, KW, SH, SW, PH, PW};
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case ACTNN_F32: return launch_cl<float>(false, grad_out, idx, nullptr, grad_in, N, C, g, s);
+    case ACTNN_F16: return launch_cl<__half>(false, grad_out, idx, nullptr, grad_in, N, C, g, s);
+    case ACTNN_BF16: return launch_cl<bf16_t>(false, grad_out, idx, nullptr, grad_in, N, C, g, s);
     default: return ACTNN_EDTYPE;
   }
 }

@@ -185,8 +185,9 @@ class QMaxPool2d(_MaxPoolNd):
         self.dilation = _pair(dilation)
 
     def forward(self, input):
-        if channels_last_format(input) is not None:
-            # the pooling kernels are NCHW: transpose in and out so that the model stays channels-last
+        if channels_last_format(input) is not None and not ext_quantization.pool_takes_channels_last(input):
+            # channel counts the channels-last kernels do not take: transpose in and out so that
+            # the model stays channels-last
             out = ext_quantization.act_quantized_max_pool2d(
                 input.contiguous(), self.kernel_size, self.stride, self.padding, self.dilation,
                 self.ceil_mode, self.return_indices)

@@ -140,6 +140,16 @@ int actnn_max_pool2d_forward(const void* x, void* y, int8_t* idx, int64_t N, int
 int actnn_max_pool2d_backward(const void* grad_out, const int8_t* idx, void* grad_in, int64_t N,
                               int64_t C, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH,
                               int KW, int SH, int SW, int PH, int PW, int dtype, void* stream);
+/* The same two operators on channels-last tensors: x, y, idx and the gradients are laid out
+ * [N, H, W, C] / [N, Ho, Wo, C] (C a multiple of 4 for f32, 8 for 16-bit types; 16-byte aligned
+ * pointers).  Values and indices equal those of the default-layout operators on the transposed
+ * tensors. */
+int actnn_max_pool2d_forward_cl(const void* x, void* y, int8_t* idx, int64_t N, int64_t C,
+                                int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH, int KW,
+                                int SH, int SW, int PH, int PW, int dtype, void* stream);
+int actnn_max_pool2d_backward_cl(const void* grad_out, const int8_t* idx, void* grad_in, int64_t N,
+                                 int64_t C, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH,
+                                 int KW, int SH, int SW, int PH, int PW, int dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------
  * calc_precision (HOST pointers): greedy bit allocation, mutates b in place.

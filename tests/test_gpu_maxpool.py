@@ -79,3 +79,46 @@ def test_rejected_arguments():
         ext_q.act_quantized_max_pool2d(x, (4, 4), (2, 2), (1, 1), (1, 1), False, False)   # KH*KW >= 16
     with pytest.raises(RuntimeError):
         ext_q.act_quantized_max_pool2d(x, (3,), (2, 2), (1, 1), (1, 1), False, False)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("k,s,p", GEOMS)
+@pytest.mark.parametrize("shape", [(4, 8, 28, 28), (2, 16, 13, 17), (1, 64, 5, 5), (3, 24, 32, 24), (2, 8, 224, 224)])
+def test_channels_last_equals_default_layout(dtype, k, s, p, shape):
+    """[N, H, W, C] kernels: values, indices and gradients are those of the default-layout kernels
+    on the same logical tensor; outputs keep the channels-last strides."""
+    torch.manual_seed(sum(shape) + 1)
+    x = torch.randn(*shape).to(dtype).to(DEV)
+    x_cl = x.contiguous(memory_format=torch.channels_last)
+    assert ext_q.pool_takes_channels_last(x_cl)
+    y, idx = ext_q.max_pool2d_forward(x, k, s, p, (1, 1))
+    y_cl, idx_cl = ext_q.max_pool2d_forward(x_cl, k, s, p, (1, 1))
+    assert y_cl.is_contiguous(memory_format=torch.channels_last) and idx_cl.is_contiguous(memory_format=torch.channels_last)
+    assert torch.equal(y_cl, y) and torch.equal(idx_cl, idx)
+    g = torch.randn_like(y)
+    gin = ext_q.max_pool2d_backward(g, idx, x.shape, k, s, p)
+    gin_cl = ext_q.max_pool2d_backward(g.contiguous(memory_format=torch.channels_last), idx_cl, x.shape, k, s, p)
+    assert gin_cl.is_contiguous(memory_format=torch.channels_last)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2          # the two kernels add overlapping windows in the same order
+    assert torch.allclose(gin_cl.float(), gin.float(), atol=tol, rtol=tol)
+    # and through autograd, against torch's own channels-last max-pool
+    xa = x_cl.clone(memory_format=torch.preserve_format).requires_grad_(True)
+    ya = ext_q.act_quantized_max_pool2d(xa, k, s, p, (1, 1), False, False)
+    ya.backward(g)
+    xr = x.clone().requires_grad_(True)
+    F.max_pool2d(xr, k, s, p).backward(g)
+    assert torch.equal(ya, F.max_pool2d(x, k, s, p))
+    assert torch.allclose(xa.grad.float(), xr.grad.float(), atol=tol if dtype != torch.float32 else 1e-4, rtol=tol)
+
+
+def test_channels_last_special_values():
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((2, 16, 14, 18)).astype(np.float16)
+    special = np.array([-np.inf, np.nan, 0.0, -0.0, -65504.0, np.inf], np.float16)
+    pick = rng.integers(0, 12, size=x.shape)
+    x = np.where(pick < 6, special[np.minimum(pick, 5)], x)
+    xt = torch.from_numpy(x).to(DEV).contiguous(memory_format=torch.channels_last)
+    y, idx = ext_q.max_pool2d_forward(xt, (3, 3), (2, 2), (1, 1), (1, 1))
+    out_o, idx_o = pool.max_pool2d_forward_literal(x, (3, 3), (2, 2), (1, 1))
+    assert np.array_equal(idx.cpu().numpy(), idx_o)
+    assert np.array_equal(y.cpu().numpy(), out_o, equal_nan=True)
