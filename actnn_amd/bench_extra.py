@@ -62,11 +62,15 @@ def resnet50_step(device, level="L3", batch=512, warmup=3, steps=10, autocast=Tr
 
 
 def run(device):
+    """ResNet-50, batch 512, bf16 autocast: L3 and the unquantised model, in the channels-last
+    layout (what this GPU's convolution kernels work in natively) and in the default one."""
     out = {}
-    torch.cuda.reset_peak_memory_stats()
-    out["resnet50_L3"] = resnet50_step(device, "L3")
-    torch.cuda.empty_cache()
-    torch.cuda.reset_peak_memory_stats()
-    out["resnet50_exact"] = resnet50_step(device, "exact")
+    for key, level, channels_last in (("resnet50_L3_channels_last", "L3", True),
+                                      ("resnet50_exact_channels_last", "exact", True),
+                                      ("resnet50_L3", "L3", False),
+                                      ("resnet50_exact", "exact", False)):
+        torch.cuda.empty_cache()
+        torch.cuda.reset_peak_memory_stats()
+        out[key] = resnet50_step(device, level, channels_last=channels_last)
     torch.cuda.empty_cache()
     return out

@@ -201,7 +201,21 @@ def other_configs(device, reps):
     return {k_: {kk: round(vv, 4) for kk, vv in v.items()} for k_, v in out.items()}
 
 
+def _heartbeat(period=30.0):
+    """Progress lines on stderr while the long legs run (MIOpen's solver search during the first
+    ResNet-50 step is silent for minutes); stdout stays the single JSON line."""
+    import threading
+    t0 = time.time()
+
+    def beat():
+        while True:
+            time.sleep(period)
+            print(f"[bench] running, {time.time() - t0:.0f} s", file=sys.stderr, flush=True)
+    threading.Thread(target=beat, daemon=True).start()
+
+
 def main():
+    _heartbeat()
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
