@@ -4,6 +4,7 @@ import torch
 
 from . import _glue as g
 from .._lib import check
+from ..utils import channels_last_format
 
 
 def minimax(data):
@@ -41,3 +42,21 @@ def range_sqr(mn, mx, N, factor=1.0, mult=None):
                                       mult_ptr, per_sample, g.DTYPE_CODE[mn.dtype], g.stream_ptr(mn.device)),
               "range_sqr")
     return out
+
+
+def sample_sqnorm(x):
+    """fp32 [N]: squared L2 norm of every sample of a dense tensor (any layout: the sum does not
+    care about the order), one pass at memory speed."""
+    N = x.shape[0]
+    F = x.numel() // max(N, 1)
+    elems = 16 // x.element_size()
+    dense = x.is_contiguous() or channels_last_format(x) is not None
+    if (N == 0 or N > 65535 or F % elems != 0 or x.dtype not in g.DTYPE_CODE or not x.is_cuda
+            or not dense or x.data_ptr() % 16 != 0):
+        return torch.linalg.vector_norm(x.reshape(N, -1), dim=1, dtype=torch.float32).square()
+    slices = max(1, min(64, F // 8192))
+    part = torch.empty(N, slices, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        check(g.lib().actnn_sample_sqnorm(x.data_ptr(), part.data_ptr(), N, F, slices,
+                                          g.DTYPE_CODE[x.dtype], g.stream_ptr(x.device)), "sample_sqnorm")
+    return part.sum(1) if slices > 1 else part.view(N)

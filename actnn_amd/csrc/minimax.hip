@@ -186,6 +186,61 @@ __global__ __launch_bounds__(kThreads) void range_sqr_kernel(const T* __restrict
   }
 }
 
+// Squared L2 norm of every sample (the gradient statistic of the bit allocation, qscheme.py:47-55):
+// part[n * B + b] = sum of squares over slice b of row n, fp32, in a fixed order; the caller adds
+// the B slices.  Rows are read with 16-byte non-temporal loads; 16-bit types use the dot-product
+// instructions (exact products, fp32 accumulation).
+template <typename T> ACTNN_DEV float square_sum16(const T* p);
+template <> ACTNN_DEV float square_sum16<float>(const float* p) {
+  const u32x4 u = load16_nt(p);
+  const float a = as_float(u.x), b = as_float(u.y), c = as_float(u.z), d = as_float(u.w);
+  return fmaf(a, a, fmaf(b, b, fmaf(c, c, d * d)));
+}
+typedef _Float16 f16x2_mm __attribute__((ext_vector_type(2)));
+template <> ACTNN_DEV float square_sum16<__half>(const __half* p) {
+  const u32x4 u = load16_nt(p);
+  float q = 0.0f;
+  const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    q = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_mm, w[i]), __builtin_bit_cast(f16x2_mm, w[i]), q, false);
+  return q;
+}
+template <> ACTNN_DEV float square_sum16<bf16_t>(const bf16_t* p) {
+  const u32x4 u = load16_nt(p);
+  float q = 0.0f;
+  const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    q = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[i]), __builtin_bit_cast(bf16x2_t, w[i]), q, false);
+  return q;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void sample_sqnorm_kernel(const T* __restrict__ x, float* __restrict__ part,
+                                                                int64_t F, int64_t slice) {
+  constexpr int E = Vec16<T>::kElems;
+  __shared__ float s_part[kThreads];
+  const int64_t n = blockIdx.y;
+  const int64_t lo = (int64_t)blockIdx.x * slice;
+  const int64_t hi = lo + slice < F ? lo + slice : F;
+  const T* row = x + n * F;
+  float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  int64_t i = lo + (int64_t)threadIdx.x * E;
+  for (; i + 3 * (int64_t)kThreads * E < hi; i += 4 * (int64_t)kThreads * E) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc[u] += square_sum16<T>(row + i + (int64_t)u * kThreads * E);
+  }
+  for (; i < hi; i += (int64_t)kThreads * E) acc[0] += square_sum16<T>(row + i);
+  s_part[threadIdx.x] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+  __syncthreads();
+  for (int w = kThreads / 2; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) s_part[threadIdx.x] += s_part[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) part[n * gridDim.x + blockIdx.x] = s_part[0];
+}
+
 }  // namespace
 }  // namespace actnn
 
@@ -230,4 +285,26 @@ extern "C" int actnn_minimax(const void* data, void* mn, void* mx, int64_t M, in
     case ACTNN_BF16: return launch_minimax<bf16_t>(data, mn, mx, M, D, s);
     default: return ACTNN_EDTYPE;
   }
+}
+
+extern "C" int actnn_sample_sqnorm(const void* x, float* part, int64_t N, int64_t F, int slices, int dtype,
+                                   void* stream) {
+  using namespace actnn;
+  if (N < 0 || F < 0 || slices < 1 || slices > 65535 || N > 65535) return ACTNN_EINVAL;
+  if (N == 0) return ACTNN_OK;
+  if (!x || !part) return ACTNN_EINVAL;
+  const int elems = dtype == ACTNN_F32 ? 4 : 8;
+  if (F % elems != 0) return ACTNN_EINVAL;
+  if (!aligned16(x)) return ACTNN_EALIGN;
+  int64_t slice = (F + slices - 1) / slices;
+  slice = (slice + elems - 1) / elems * elems;                 // whole 16-byte vectors
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)slices, (unsigned)N), blk(kThreads);
+  switch (dtype) {
+    case ACTNN_F32: sample_sqnorm_kernel<float><<<grid, blk, 0, s>>>(static_cast<const float*>(x), part, F, slice); break;
+    case ACTNN_F16: sample_sqnorm_kernel<__half><<<grid, blk, 0, s>>>(static_cast<const __half*>(x), part, F, slice); break;
+    case ACTNN_BF16: sample_sqnorm_kernel<bf16_t><<<grid, blk, 0, s>>>(static_cast<const bf16_t*>(x), part, F, slice); break;
+    default: return ACTNN_EDTYPE;
+  }
+  ACTNN_RETURN_LAUNCH_STATUS();
 }

@@ -153,9 +153,8 @@ class QScheme(_LazyHost):
         """Squared gradient norm per sample, kept as a running value (qscheme.py:47-55)."""
         if not QScheme.update_scale:
             return
-        # squared L2 norm per sample, accumulated in fp32 without materialising an fp32 copy
-        sq = torch.linalg.vector_norm(memory_order(grad).reshape(grad.shape[0], -1), dim=1,
-                                      dtype=torch.float32).square()
+        # squared L2 norm per sample, accumulated in fp32 in one pass over the gradient
+        sq = ext_minimax.sample_sqnorm(grad)
         if config.use_gradient:
             assert QScheme.batch is not None
             self.scales[QScheme.batch] = self.scales[QScheme.batch] * 0.5 + sq.cpu() * 0.5

@@ -157,6 +157,13 @@ int actnn_max_pool2d_backward_cl(const void* grad_out, const int8_t* idx, void* 
  * ------------------------------------------------------------------------------- */
 int actnn_calc_precision(int32_t* b, const float* C, const int32_t* w, int64_t N, double target);
 
+/* Squared L2 norm per sample of x[N, F] (the per-sample gradient statistic of the bit allocation,
+ * qscheme.py:47-55, where the reference chains square / sum over a full-size temporary):
+ * part[n * slices + b] = sum of squares of slice b of row n (fp32, fixed order); the caller adds the
+ * `slices` values of a row.  F a multiple of 4 (f32) or 8 (16-bit types), N <= 65535, x 16-byte aligned. */
+int actnn_sample_sqnorm(const void* x, float* part, int64_t N, int64_t F, int slices, int dtype,
+                        void* stream);
+
 /* Same allocation on the DEVICE for the case every layer uses at every step: all N items start
  * at initial_bits (1..8) with weight 1 and `target` is the bit budget, so exactly
  * N * initial_bits - target widths are taken away (clamped to [0, N * (initial_bits - 1)]).

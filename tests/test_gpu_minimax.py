@@ -77,3 +77,19 @@ def test_range_sqr_rejects_bad_arguments():
     with pytest.raises(RuntimeError):
         ext_minimax.range_sqr(mn.int(), mn.int(), 2)
     assert ext_minimax.range_sqr(mn[:0], mn[:0], 0).numel() == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(4, 64, 56, 56), (3, 8, 5, 7), (16, 4096), (2, 3, 5, 5), (1, 16, 300, 301), (5, 24, 14, 14)])
+def test_sample_sqnorm(dtype, shape):
+    """Per-sample sum of squares against a float64 sum (fp32 accumulation: 1e-5 relative), for the
+    default and the channels-last layout, and the ATen fallback for shapes without whole vectors."""
+    g = torch.Generator(device=DEV).manual_seed(sum(shape))
+    x = (torch.randn(*shape, generator=g, device=DEV) * 3).to(dtype)
+    ref = x.double().reshape(shape[0], -1).square().sum(1)
+    got = ext_minimax.sample_sqnorm(x)
+    assert got.dtype == torch.float32 and got.shape == (shape[0],)
+    assert torch.allclose(got.double(), ref, rtol=1e-5)
+    if len(shape) == 4:
+        got_cl = ext_minimax.sample_sqnorm(x.contiguous(memory_format=torch.channels_last))
+        assert torch.allclose(got_cl.double(), ref, rtol=1e-5)
