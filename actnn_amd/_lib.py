@@ -56,6 +56,10 @@ SIGNATURES = {
     "actnn_batch_norm_workspace_bytes": [c_i64, c_i64, c_i64, c_i32, c_i32],
     "actnn_batch_norm_forward": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,
                                  c_i64, c_i64, c_i64, ctypes.c_double, ctypes.c_double, c_i32, c_i32, c_vp],
+    "actnn_batch_norm_forward_stats": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,
+                                       c_i64, c_i64, c_i64, ctypes.c_double, ctypes.c_double, c_i32, c_i32, c_vp],
+    "actnn_batch_norm_forward_apply": [c_vp, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u64, c_u64,
+                                       c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
     "actnn_batch_norm_backward_packed": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp,
                                          c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
     "actnn_batch_norm_backward": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,

@@ -91,6 +91,65 @@ def hip_batch_norm_forward(input, weight, bias, running_mean, running_var, momen
     return out, save_mean, save_invstd, mn, mx
 
 
+def hip_batch_norm_forward_stats(input, weight, bias, running_mean, running_var, momentum, eps, minmax=True):
+    """First half of the forward pass -> (workspace, save_mean, save_invstd, mn, mx); the workspace
+    carries the per-channel coefficients to hip_batch_norm_forward_apply."""
+    N, C, HW, channels_last = _bn_geometry(input)
+    lib = _glue.lib()
+    code = _glue.DTYPE_CODE[input.dtype]
+    ws_bytes = lib.actnn_batch_norm_workspace_bytes(N, C, HW, code, int(channels_last))
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=input.device)
+    save_mean = torch.empty(C, dtype=torch.float32, device=input.device)
+    save_invstd = torch.empty(C, dtype=torch.float32, device=input.device)
+    mn = mx = None
+    if minmax:
+        groups = N * C * HW // 256
+        mn = torch.empty(groups, dtype=input.dtype, device=input.device)
+        mx = torch.empty(groups, dtype=input.dtype, device=input.device)
+    with torch.cuda.device(input.device):
+        _glue._lib.check(lib.actnn_batch_norm_forward_stats(
+            input.data_ptr(), _ptr(weight), _ptr(bias), _ptr(running_mean), _ptr(running_var),
+            save_mean.data_ptr(), save_invstd.data_ptr(), _ptr(mn), _ptr(mx), ws.data_ptr(), ws_bytes,
+            N, C, HW, float(momentum), float(eps), code, int(channels_last),
+            _glue.stream_ptr(input.device)), "batch_norm_forward_stats")
+    return ws, save_mean, save_invstd, mn, mx
+
+
+def hip_batch_norm_forward_apply(input, workspace, bits=None, mn=None, mx=None):
+    """Second half -> (output, packed, scale).  With `bits` (int32 [N] on the device) and the group
+    min/max, the pass also quantises the input: `packed` and `scale` are what
+    pack_mixed_precision(groups of input, mn, mx, bits, True) returns for the same generator state."""
+    from .quantization import _bits_info
+    N, C, HW, channels_last = _bn_geometry(input)
+    lib = _glue.lib()
+    code = _glue.DTYPE_CODE[input.dtype]
+    out = torch.empty_like(input)
+    packed = scale = prefix = None
+    seed = offset = 0
+    if bits is not None:
+        G = C * HW // 256
+        total, prefix = _bits_info(bits)
+        packed = torch.empty(total * G * 8, dtype=torch.int32, device=input.device)
+        scale = torch.empty(N, G, 1, dtype=input.dtype, device=input.device)
+        seed, offset = _glue.philox_args(input.device)
+    with torch.cuda.device(input.device):
+        _glue._lib.check(lib.actnn_batch_norm_forward_apply(
+            input.data_ptr(), out.data_ptr(), workspace.data_ptr(), workspace.numel() * 4, _ptr(bits),
+            _ptr(prefix), _ptr(mn), _ptr(mx), _ptr(scale), _ptr(packed), seed, offset, N, C, HW, code,
+            int(channels_last), _glue.stream_ptr(input.device)), "batch_norm_forward_apply")
+    return out, packed, scale
+
+
+def hip_batch_norm_pack_applies(input, weight, bias, running_mean, running_var):
+    """True when the forward pass can also write the packed copy of its input."""
+    if input.dtype not in (torch.float16, torch.bfloat16):
+        return False
+    if not hip_batch_norm_minmax_applies(input, weight, bias, running_mean, running_var):
+        return False
+    N, C, HW, channels_last = _bn_geometry(input)
+    return not channels_last or N * HW < 2 ** 31
+
+
 def hip_batch_norm_backward(input, grad_output, weight, save_mean, save_invstd):
     """-> (grad_input, grad_weight, grad_bias) of training-mode batch norm; `grad_output` has the
     strides of `input`."""

@@ -221,6 +221,68 @@ template <typename T> struct PackedInput {
   }
 };
 
+// Where the forward apply pass can leave the activation quantiser's output: the chunk a lane holds
+// is its share of one quantisation group (32 lanes per group, 16-bit types), so the codes are made
+// from the registers the normalisation reads anyway - same arithmetic, same Philox counters (the
+// index of the 8-element chunk in the tensor as it lies in memory) and same stream layout as
+// actnn_pack_mixed, hence the same bits.
+struct PackSink {
+  const int32_t* bits;
+  const int32_t* prefix;
+  const void* mn;
+  const void* mx;
+  void* scale;
+  int32_t* packed;
+  uint64_t seed, offset;
+  int64_t G;             // groups per sample
+};
+
+template <int BITS>
+ACTNN_DEV void pack_chunk_bits(const float (&v)[8], const uint32_t (&r16)[8], float mul, float sub,
+                               uint32_t lane32, int32_t* __restrict__ dst) {
+  constexpr float kBfix = (float)((1 << BITS) - 1) * 65536.0f;
+  uint64_t acc = 0;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) acc |= (uint64_t)rng_code(v[k], r16[k], mul, sub, kBfix) << (k * BITS);
+  const uint32_t lo = transpose32((uint32_t)acc, lane32);
+  if ((int)lane32 < 8 * BITS) __builtin_nontemporal_store((int32_t)lo, dst + lane32);
+  if (BITS > 4) {
+    const uint32_t hi = transpose32((uint32_t)(acc >> 32), lane32);
+    if ((int)lane32 < 8 * BITS - 32) __builtin_nontemporal_store((int32_t)hi, dst + 32 + lane32);
+  }
+}
+
+template <typename T>
+ACTNN_DEV void pack_chunk(const PackSink& ps, const u32x4& ux, int64_t n, int64_t grp, int64_t octet) {
+  constexpr int PD = Chunk<T>::kPerDword;
+  static_assert(Chunk<T>::kElems == 8, "16-bit types only");
+  const uint32_t lane32 = threadIdx.x & 31;
+  const int b = ps.bits[n];
+  const int64_t gi = n * ps.G + grp;
+  float mul, sub;
+  const float sc = GroupQuant<T, false>::prepare(Conv<T>::load(static_cast<const T*>(ps.mn), gi),
+                                                 Conv<T>::load(static_cast<const T*>(ps.mx), gi), b, mul, sub);
+  if (lane32 == 0) Conv<T>::store(static_cast<T*>(ps.scale), gi, sc);
+  const uint32_t w[4] = {ux.x, ux.y, ux.z, ux.w};
+  float v[8];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) Chunk<T>::widen(w[k], v + k * PD);
+  uint32_t r16[8];
+  philox_octet((uint64_t)octet, ps.seed, ps.offset, r16);
+  int32_t* dst = ps.packed + ((int64_t)ps.prefix[n] * ps.G + grp * b) * 8;
+  switch (b) {                           // uniform over the half-wave: one sample, one width
+    case 1: pack_chunk_bits<1>(v, r16, mul, sub, lane32, dst); break;
+    case 2: pack_chunk_bits<2>(v, r16, mul, sub, lane32, dst); break;
+    case 3: pack_chunk_bits<3>(v, r16, mul, sub, lane32, dst); break;
+    case 4: pack_chunk_bits<4>(v, r16, mul, sub, lane32, dst); break;
+    case 5: pack_chunk_bits<5>(v, r16, mul, sub, lane32, dst); break;
+    case 6: pack_chunk_bits<6>(v, r16, mul, sub, lane32, dst); break;
+    case 7: pack_chunk_bits<7>(v, r16, mul, sub, lane32, dst); break;
+    case 8: pack_chunk_bits<8>(v, r16, mul, sub, lane32, dst); break;
+    default: break;
+  }
+}
+
 template <typename T> ACTNN_DEV void bind_input(PlainInput<T>& xs, const Place& p) { xs.p += p.elem; }
 template <typename T> ACTNN_DEV void bind_input(PackedInput<T>& xs, const Place& p) {
   xs.g = p.elem >> 8;
@@ -392,14 +454,14 @@ __global__ __launch_bounds__(kThreads) void bn_backward_finalize_kernel(
 }
 
 // Pass 2 of either direction.  Forward: y = a*x + b.  Backward: dx = A*dy + B*x + K.
-template <typename T, bool SPLIT, bool BWD, typename XS>
+template <typename T, bool SPLIT, bool BWD, bool PACK, typename XS>
 __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
     XS xs, const T* __restrict__ dy, const float* __restrict__ coef,
-    T* __restrict__ out, int64_t N, int64_t F, int64_t HW, int per_block) {
+    T* __restrict__ out, int64_t N, int64_t F, int64_t HW, int per_block, PackSink ps) {
   constexpr int E = Chunk<T>::kElems;
   constexpr int PD = Chunk<T>::kPerDword;
   constexpr int NC = BWD ? 3 : 2;
-  constexpr int kUnroll = XS::kInFlight;
+  constexpr int kUnroll = PACK ? 2 : XS::kInFlight;
   const Place p = place_of<E>(F, HW);
   if (!p.active) return;               // whole quantisation groups (32 lanes) leave together
   bind_input(xs, p);
@@ -454,12 +516,14 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
     for (int u = 0; u < kUnroll; ++u) {
       const u32x4 ux = xs.decode(rx[u]);
       store_out(po + (n + u) * F, apply(ux, BWD ? ud[u] : ux));
+      if constexpr (PACK) pack_chunk<T>(ps, ux, n + u, p.elem >> 8, ((n + u) * F + p.elem) >> 3);
     }
   }
   for (; n < n1; ++n) {
     const typename XS::Raw rx = xs.fetch(n);
     const u32x4 ux = xs.decode(rx);
     store_out(po + n * F, apply(ux, BWD ? load_last(pd + n * F) : ux));
+    if constexpr (PACK) pack_chunk<T>(ps, ux, n, p.elem >> 8, (n * F + p.elem) >> 3);
   }
 }
 
@@ -604,14 +668,21 @@ __global__ __launch_bounds__(kThreads) void bn_cl_reduce_kernel(
   }
 }
 
-template <typename T, bool BWD, typename XS>
+template <typename T, bool BWD, bool PACK, typename XS>
 __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
     XS xs, const T* __restrict__ dy, const float* __restrict__ coef, T* __restrict__ out,
-    int64_t P, int64_t C, int tpr, int R, int64_t ppb) {
+    int64_t P, int64_t C, int tpr, int R, int64_t ppb, PackSink ps, uint32_t HW) {
   constexpr int E = Chunk<T>::kElems;
   constexpr int PD = Chunk<T>::kPerDword;
   constexpr int NC = BWD ? 3 : 2;
-  constexpr int U = XS::kInFlight;
+  constexpr int U = PACK ? 2 : XS::kInFlight;
+  auto pack_row = [&](const u32x4& ux, int64_t row, int64_t col) {
+    if constexpr (PACK) {
+      const uint32_t n = (uint32_t)row / HW;               // rows < 2^31 (checked by the launcher)
+      const int64_t flat = row * C + col;
+      pack_chunk<T>(ps, ux, n, (flat >> 8) - (int64_t)n * ps.G, flat >> 3);
+    }
+  };
   const RowTile t = row_tile<E>(C, tpr, R);
   if (!t.active) return;               // whole quantisation groups leave together
   xs.bind(t.col, C);
@@ -659,12 +730,14 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
     for (int u = 0; u < U; ++u) {
       const u32x4 ux = xs.decode(rx[u]);
       store_out(po + (row + (int64_t)u * R) * C, apply(ux, BWD ? ud[u] : ux));
+      pack_row(ux, row + (int64_t)u * R, t.col);
     }
   }
   for (; row < p1; row += R) {
     const typename XS::Raw rx = xs.fetch(row);
     const u32x4 ux = xs.decode(rx);
     store_out(po + row * C, apply(ux, BWD ? load_last(pd + row * C) : ux));
+    pack_row(ux, row, t.col);
   }
 }
 
@@ -760,16 +833,16 @@ void launch_reduce(const Plan& pl, const XS& xs, const void* dy, float* part, vo
     bn_reduce_kernel<T, false, BWD, MINMAX, XS><<<grid, blk, lds, s>>>(xs, pd, part, lo, hi, N, pl.F, HW, pl.per_block, pl.slots);
 }
 
-template <typename T, bool BWD, typename XS>
+template <typename T, bool BWD, bool PACK, typename XS>
 void launch_apply(const Plan& pl, const XS& xs, const void* dy, const float* coef, void* out,
-                  int64_t N, int64_t HW, hipStream_t s) {
+                  int64_t N, int64_t HW, const PackSink& ps, hipStream_t s) {
   const dim3 grid((unsigned)pl.spans, (unsigned)pl.nsplit), blk(kThreads);
   const T* pd = static_cast<const T*>(dy);
   T* po = static_cast<T*>(out);
   if (pl.split)
-    bn_apply_kernel<T, true, BWD, XS><<<grid, blk, 0, s>>>(xs, pd, coef, po, N, pl.F, HW, pl.per_block);
+    bn_apply_kernel<T, true, BWD, PACK, XS><<<grid, blk, 0, s>>>(xs, pd, coef, po, N, pl.F, HW, pl.per_block, ps);
   else
-    bn_apply_kernel<T, false, BWD, XS><<<grid, blk, 0, s>>>(xs, pd, coef, po, N, pl.F, HW, pl.per_block);
+    bn_apply_kernel<T, false, BWD, PACK, XS><<<grid, blk, 0, s>>>(xs, pd, coef, po, N, pl.F, HW, pl.per_block, ps);
 }
 
 template <typename T, bool BWD, bool MINMAX, typename XS>
@@ -779,38 +852,56 @@ void launch_cl_reduce(const Plan& pl, const XS& xs, const void* dy, float* part,
   bn_cl_reduce_kernel<T, BWD, MINMAX, XS><<<grid, blk, 0, s>>>(
       xs, static_cast<const T*>(dy), part, static_cast<T*>(mn), static_cast<T*>(mx), pl.P, C, pl.tpr, pl.R, pl.ppb);
 }
-template <typename T, bool BWD, typename XS>
+template <typename T, bool BWD, bool PACK, typename XS>
 void launch_cl_apply(const Plan& pl, const XS& xs, const void* dy, const float* coef, void* out, int64_t C,
-                     hipStream_t s) {
+                     const PackSink& ps, hipStream_t s) {
   const dim3 grid((unsigned)pl.tiles, (unsigned)pl.nsplit), blk(kThreads);
-  bn_cl_apply_kernel<T, BWD, XS><<<grid, blk, 0, s>>>(xs, static_cast<const T*>(dy), coef,
-                                                      static_cast<T*>(out), pl.P, C, pl.tpr, pl.R, pl.ppb);
+  bn_cl_apply_kernel<T, BWD, PACK, XS><<<grid, blk, 0, s>>>(
+      xs, static_cast<const T*>(dy), coef, static_cast<T*>(out), pl.P, C, pl.tpr, pl.R, pl.ppb, ps,
+      (uint32_t)(pl.F / C));
 }
 
 template <typename T>
-int forward_t(const Plan& pl, const void* x, const float* weight, const float* bias, float* running_mean,
-              float* running_var, void* y, float* save_mean, float* save_invstd, void* mn, void* mx,
-              float* ws, int64_t N, int64_t C, int64_t HW, double momentum, double eps, hipStream_t s) {
+int forward_stats_t(const Plan& pl, const void* x, const float* weight, const float* bias, float* running_mean,
+                    float* running_var, float* save_mean, float* save_invstd, void* mn, void* mx, float* ws,
+                    int64_t N, int64_t C, int64_t HW, double momentum, double eps, hipStream_t s) {
   float* part = ws;
   float* coef = ws + pl.part_floats;
-  const dim3 fin((unsigned)((C + kWaves - 1) / kWaves)), blk(kThreads);
   if (pl.channels_last) {
     const PlainRows<T> xs{static_cast<const T*>(x), C};
     if (mn) launch_cl_reduce<T, false, true>(pl, xs, nullptr, part, mn, mx, C, s);
     else launch_cl_reduce<T, false, false>(pl, xs, nullptr, part, nullptr, nullptr, C, s);
-    bn_forward_finalize_kernel<<<fin, blk, 0, s>>>(part, weight, bias, running_mean, running_var, save_mean,
-                                                   save_invstd, coef, N, C, HW, pl.L, pl.nsplit, pl.slots,
-                                                   momentum, eps);
-    launch_cl_apply<T, false>(pl, xs, nullptr, coef, y, C, s);
-    ACTNN_RETURN_LAUNCH_STATUS();
+  } else {
+    const PlainInput<T> xs{static_cast<const T*>(x), pl.F};
+    if (mn) launch_reduce<T, false, true>(pl, xs, nullptr, part, mn, mx, N, HW, s);
+    else launch_reduce<T, false, false>(pl, xs, nullptr, part, nullptr, nullptr, N, HW, s);
   }
-  const PlainInput<T> xs{static_cast<const T*>(x), pl.F};
-  if (mn) launch_reduce<T, false, true>(pl, xs, nullptr, part, mn, mx, N, HW, s);
-  else launch_reduce<T, false, false>(pl, xs, nullptr, part, nullptr, nullptr, N, HW, s);
-  bn_forward_finalize_kernel<<<fin, blk, 0, s>>>(part, weight, bias, running_mean, running_var, save_mean,
-                                                 save_invstd, coef, N, C, HW, pl.L, pl.nsplit, pl.slots,
-                                                 momentum, eps);
-  launch_apply<T, false>(pl, xs, nullptr, coef, y, N, HW, s);
+  bn_forward_finalize_kernel<<<dim3((unsigned)((C + kWaves - 1) / kWaves)), dim3(kThreads), 0, s>>>(
+      part, weight, bias, running_mean, running_var, save_mean, save_invstd, coef, N, C, HW, pl.L, pl.nsplit,
+      pl.slots, momentum, eps);
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
+
+// y = a*x + b from the coefficients the statistics step left in the workspace; with a sink the
+// same pass also writes the packed copy of x (16-bit types).
+template <typename T>
+int forward_apply_t(const Plan& pl, const void* x, void* y, const float* ws, const PackSink* sink, int64_t N,
+                    int64_t C, int64_t HW, hipStream_t s) {
+  const float* coef = ws + pl.part_floats;
+  const PackSink none{};
+  if (pl.channels_last) {
+    const PlainRows<T> xs{static_cast<const T*>(x), C};
+    if constexpr (sizeof(T) == 2) {
+      if (sink) { launch_cl_apply<T, false, true>(pl, xs, nullptr, coef, y, C, *sink, s); ACTNN_RETURN_LAUNCH_STATUS(); }
+    }
+    launch_cl_apply<T, false, false>(pl, xs, nullptr, coef, y, C, none, s);
+  } else {
+    const PlainInput<T> xs{static_cast<const T*>(x), pl.F};
+    if constexpr (sizeof(T) == 2) {
+      if (sink) { launch_apply<T, false, true>(pl, xs, nullptr, coef, y, N, HW, *sink, s); ACTNN_RETURN_LAUNCH_STATUS(); }
+    }
+    launch_apply<T, false, false>(pl, xs, nullptr, coef, y, N, HW, none, s);
+  }
   ACTNN_RETURN_LAUNCH_STATUS();
 }
 
@@ -825,8 +916,9 @@ int backward_t(const Plan& pl, const XS& xs, const void* dy, const float* weight
   bn_backward_finalize_kernel<<<dim3((unsigned)((C + kWaves - 1) / kWaves)), dim3(kThreads), 0, s>>>(
       part, weight, save_mean, save_invstd, dweight, dbias, coef, N, C, HW, pl.L, pl.nsplit, pl.slots);
   if (dx) {
-    if constexpr (XS::kRows) launch_cl_apply<T, true>(pl, xs, dy, coef, dx, C, s);
-    else launch_apply<T, true>(pl, xs, dy, coef, dx, N, HW, s);
+    const PackSink none{};
+    if constexpr (XS::kRows) launch_cl_apply<T, true, false>(pl, xs, dy, coef, dx, C, none, s);
+    else launch_apply<T, true, false>(pl, xs, dy, coef, dx, N, HW, none, s);
   }
   ACTNN_RETURN_LAUNCH_STATUS();
 }
@@ -867,27 +959,70 @@ extern "C" int64_t actnn_batch_norm_workspace_bytes(int64_t N, int64_t C, int64_
   return actnn::workspace_floats(pl, C) * (int64_t)sizeof(float);
 }
 
+extern "C" int actnn_batch_norm_forward_stats(const void* x, const float* weight, const float* bias,
+                                              float* running_mean, float* running_var, float* save_mean,
+                                              float* save_invstd, void* mn, void* mx, void* workspace,
+                                              int64_t workspace_bytes, int64_t N, int64_t C, int64_t HW,
+                                              double momentum, double eps, int dtype, int channels_last,
+                                              void* stream) {
+  using namespace actnn;
+  if (dtype < 0 || dtype > 2) return ACTNN_EDTYPE;
+  Plan pl;
+  if (!make_plan(N, C, HW, dtype, channels_last, pl)) return ACTNN_EINVAL;
+  if (!x || !save_mean || !save_invstd || !workspace || (mn == nullptr) != (mx == nullptr)) return ACTNN_EINVAL;
+  if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
+  if (mn && !pl.groups_align) return ACTNN_EINVAL;
+  if (!aligned16(x) || !aligned16(workspace)) return ACTNN_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float* ws = static_cast<float*>(workspace);
+  switch (dtype) {
+    case ACTNN_F32: return forward_stats_t<float>(pl, x, weight, bias, running_mean, running_var, save_mean, save_invstd, mn, mx, ws, N, C, HW, momentum, eps, s);
+    case ACTNN_F16: return forward_stats_t<__half>(pl, x, weight, bias, running_mean, running_var, save_mean, save_invstd, mn, mx, ws, N, C, HW, momentum, eps, s);
+    default: return forward_stats_t<bf16_t>(pl, x, weight, bias, running_mean, running_var, save_mean, save_invstd, mn, mx, ws, N, C, HW, momentum, eps, s);
+  }
+}
+
+extern "C" int actnn_batch_norm_forward_apply(const void* x, void* y, const void* workspace,
+                                              int64_t workspace_bytes, const int32_t* bits,
+                                              const int32_t* prefix, const void* mn, const void* mx,
+                                              void* scale, int32_t* packed, uint64_t seed, uint64_t offset,
+                                              int64_t N, int64_t C, int64_t HW, int dtype, int channels_last,
+                                              void* stream) {
+  using namespace actnn;
+  if (dtype < 0 || dtype > 2) return ACTNN_EDTYPE;
+  Plan pl;
+  if (!make_plan(N, C, HW, dtype, channels_last, pl)) return ACTNN_EINVAL;
+  if (!x || !y || !workspace) return ACTNN_EINVAL;
+  if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
+  if (!aligned16(x) || !aligned16(y) || !aligned16(workspace)) return ACTNN_EALIGN;
+  PackSink sink{bits, prefix, mn, mx, scale, packed, seed, offset, pl.F / 256};
+  const bool pack = bits != nullptr;
+  if (pack) {
+    if (dtype == ACTNN_F32 || !pl.groups_align || !prefix || !mn || !mx || !scale || !packed) return ACTNN_EINVAL;
+    if (channels_last && pl.P > 0x7fffffffLL) return ACTNN_EINVAL;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const float* ws = static_cast<const float*>(workspace);
+  switch (dtype) {
+    case ACTNN_F32: return forward_apply_t<float>(pl, x, y, ws, nullptr, N, C, HW, s);
+    case ACTNN_F16: return forward_apply_t<__half>(pl, x, y, ws, pack ? &sink : nullptr, N, C, HW, s);
+    default: return forward_apply_t<bf16_t>(pl, x, y, ws, pack ? &sink : nullptr, N, C, HW, s);
+  }
+}
+
 extern "C" int actnn_batch_norm_forward(const void* x, const float* weight, const float* bias,
                                         float* running_mean, float* running_var, void* y,
                                         float* save_mean, float* save_invstd, void* mn, void* mx,
                                         void* workspace, int64_t workspace_bytes, int64_t N, int64_t C,
                                         int64_t HW, double momentum, double eps, int dtype,
                                         int channels_last, void* stream) {
-  using namespace actnn;
-  if (dtype < 0 || dtype > 2) return ACTNN_EDTYPE;
-  Plan pl;
-  if (!make_plan(N, C, HW, dtype, channels_last, pl)) return ACTNN_EINVAL;
-  if (!x || !y || !save_mean || !save_invstd || !workspace || (mn == nullptr) != (mx == nullptr)) return ACTNN_EINVAL;
-  if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
-  if (mn && !pl.groups_align) return ACTNN_EINVAL;
-  if (!aligned16(x) || !aligned16(y) || !aligned16(workspace)) return ACTNN_EALIGN;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  float* ws = static_cast<float*>(workspace);
-  switch (dtype) {
-    case ACTNN_F32: return forward_t<float>(pl, x, weight, bias, running_mean, running_var, y, save_mean, save_invstd, mn, mx, ws, N, C, HW, momentum, eps, s);
-    case ACTNN_F16: return forward_t<__half>(pl, x, weight, bias, running_mean, running_var, y, save_mean, save_invstd, mn, mx, ws, N, C, HW, momentum, eps, s);
-    default: return forward_t<bf16_t>(pl, x, weight, bias, running_mean, running_var, y, save_mean, save_invstd, mn, mx, ws, N, C, HW, momentum, eps, s);
-  }
+  if (!y) return ACTNN_EINVAL;
+  const int rc = actnn_batch_norm_forward_stats(x, weight, bias, running_mean, running_var, save_mean,
+                                                save_invstd, mn, mx, workspace, workspace_bytes, N, C, HW,
+                                                momentum, eps, dtype, channels_last, stream);
+  if (rc != ACTNN_OK) return rc;
+  return actnn_batch_norm_forward_apply(x, y, workspace, workspace_bytes, nullptr, nullptr, nullptr, nullptr,
+                                        nullptr, nullptr, 0, 0, N, C, HW, dtype, channels_last, stream);
 }
 
 extern "C" int actnn_batch_norm_backward(const void* x, const void* dy, const float* weight,

@@ -139,11 +139,14 @@ def quantize_saved(input, scheme):
     return finish_saved(start_quantize(input, scheme), input)
 
 
-def finish_saved(started, input):
-    q = _Quantized(finish_quantize(started))
+def _mark_saved(q, input):
     q.native_bf16 = input.dtype == torch.bfloat16
     q.memory_format = channels_last_format(input)
     return q
+
+
+def finish_saved(started, input):
+    return _mark_saved(_Quantized(finish_quantize(started)), input)
 
 
 # ------------------------------------------------------------------------------------------
@@ -309,7 +312,21 @@ class batch_norm(Function):
     @staticmethod
     def forward(ctx, input, running_mean, running_var, weight, bias, training,
                 exponential_average_factor, eps, scheme):
-        if _bn_shares_min_max(input, weight, bias, running_mean, running_var, training):
+        if (scheme and config.fused_bn_pack and not config.swap
+                and _bn_shares_min_max(input, weight, bias, running_mean, running_var, training)
+                and ext_backward_func.hip_batch_norm_pack_applies(input, weight, bias, running_mean, running_var)):
+            # two reads of the input in total: the statistics pass also yields the quantiser's
+            # per-group min/max, the widths are allocated from them, and the normalising pass
+            # writes the packed copy of the input next to the output
+            ws, save_mean, save_var, mn, mx = ext_backward_func.hip_batch_norm_forward_stats(
+                input, weight, bias, running_mean, running_var, exponential_average_factor, eps)
+            _, q_bits, q_min, q_max = scheme.finish_quantization_bits(
+                scheme.start_quantization_bits(input, (mn, mx)))
+            output, q_input, q_scale = ext_backward_func.hip_batch_norm_forward_apply(
+                input, ws, q_bits, q_min, q_max)
+            reserve = None
+            started = ("done", _mark_saved(_Quantized((q_input, q_bits, q_scale, q_min)), input))
+        elif _bn_shares_min_max(input, weight, bias, running_mean, running_var, training):
             # the statistics pass of the library's batch norm also yields the per-group min/max
             # the quantiser needs: one read of the input less
             output, save_mean, save_var, mn, mx = ext_backward_func.hip_batch_norm_forward(
@@ -325,7 +342,7 @@ class batch_norm(Function):
             output, save_mean, save_var = ext_backward_func.native_batch_norm(
                 input, weight, bias, running_mean, running_var, training, exponential_average_factor, eps)
             reserve = None
-        quantized = finish_saved(started, input)
+        quantized = started[1] if started[0] == "done" else finish_saved(started, input)
         empty_cache(config.empty_cache_threshold)
         if config.debug_memory_op_forward:
             global bn_layer_ct, total_act_mem

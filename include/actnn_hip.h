@@ -221,6 +221,25 @@ int actnn_batch_norm_backward(const void* x, const void* dy, const float* weight
                               int64_t workspace_bytes, int64_t N, int64_t C, int64_t HW, int dtype,
                               int channels_last, void* stream);
 
+/* The forward pass in two steps, for callers that want the quantiser's output from the same read
+ * of x: _stats runs the statistics pass (save_mean/save_invstd, running estimates, optional group
+ * min/max) and leaves the per-channel coefficients in `workspace`; the caller may then derive the
+ * per-sample bit widths from mn/mx; _apply writes y from x and the same workspace and, when `bits`
+ * is given (16-bit dtypes, the alignment conditions of mn/mx), also scale[N*G] and the packed
+ * stream - bit for bit what actnn_pack_mixed(x, mn, mx, bits, prefix, ..., seed, offset) writes in
+ * its in-kernel Philox mode.  actnn_batch_norm_forward is _stats followed by _apply without bits. */
+int actnn_batch_norm_forward_stats(const void* x, const float* weight, const float* bias,
+                                   float* running_mean, float* running_var, float* save_mean,
+                                   float* save_invstd, void* mn, void* mx, void* workspace,
+                                   int64_t workspace_bytes, int64_t N, int64_t C, int64_t HW,
+                                   double momentum, double eps, int dtype, int channels_last,
+                                   void* stream);
+int actnn_batch_norm_forward_apply(const void* x, void* y, const void* workspace,
+                                   int64_t workspace_bytes, const int32_t* bits,
+                                   const int32_t* prefix, const void* mn, const void* mx, void* scale,
+                                   int32_t* packed, uint64_t seed, uint64_t offset, int64_t N,
+                                   int64_t C, int64_t HW, int dtype, int channels_last, void* stream);
+
 /* The same backward pass with x held as the mixed-precision stream of actnn_pack_mixed (group
  * size 256 over the sample in memory order, the conditions of mn/mx above, 16-bit dtype; bits / prefix / scale / mn as for actnn_unpack_mixed):
  * both passes rebuild x in registers, bit for bit what actnn_unpack_mixed would write, so the

@@ -230,3 +230,36 @@ def test_channels_last_backward_from_the_packed_stream(N, C, spatial, dtype):
     assert got[0].stride() == x.stride()
     for a, r in zip(got, ref):
         assert torch.equal(a, r)
+
+
+@pytest.mark.parametrize("channels_last", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,C,spatial", [(8, 64, (56, 56)), (16, 256, (7, 7)), (37, 128, (14, 14)),
+                                         (9, 32, (4, 2)), (5, 1024, (6, 6))])
+def test_forward_with_packed_copy_equals_forward_then_pack(N, C, spatial, dtype, channels_last):
+    """The normalising pass that also packs its input: output equal to the plain forward pass,
+    stream and scales equal to pack_mixed_precision with the same generator state (every width)."""
+    import actnn_amd.cpp_extension.quantization as ext_q
+    from actnn_amd.utils import memory_order
+    from _util import bits_tensor
+    x, w, b, rm, rv, _ = _inputs(N, C, spatial, dtype, 31)
+    if channels_last:
+        x = _cl(x)
+    assert ext_bf.hip_batch_norm_pack_applies(x, w, b, rm, rv)
+    G = x[0].numel() // 256
+    bits_dev, _ = bits_tensor([1 + (5 * i + i // 8) % 8 for i in range(N)])
+    y_ref, mean_ref, invstd_ref, mn_ref, mx_ref = ext_bf.hip_batch_norm_forward(
+        x, w, b, rm.clone(), rv.clone(), 0.1, 1e-5, minmax=True)
+    torch.cuda.manual_seed(9)
+    packed_ref, scale_ref = ext_q.pack_mixed_precision(
+        memory_order(x).reshape(N, G, 256), mn_ref.view(N, G, 1), mx_ref.view(N, G, 1), bits_dev, True)
+    ws, mean, invstd, mn, mx = ext_bf.hip_batch_norm_forward_stats(x, w, b, rm.clone(), rv.clone(), 0.1, 1e-5)
+    torch.cuda.manual_seed(9)
+    y, packed, scale = ext_bf.hip_batch_norm_forward_apply(x, ws, bits_dev, mn.view(N, G, 1), mx.view(N, G, 1))
+    assert torch.equal(y, y_ref) and y.stride() == x.stride()
+    assert torch.equal(mean, mean_ref) and torch.equal(invstd, invstd_ref)
+    assert torch.equal(mn, mn_ref) and torch.equal(mx, mx_ref)
+    assert torch.equal(scale, scale_ref)
+    assert torch.equal(packed, packed_ref)
+    y2, none1, none2 = ext_bf.hip_batch_norm_forward_apply(x, ws)
+    assert torch.equal(y2, y_ref) and none1 is None and none2 is None
