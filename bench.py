@@ -28,12 +28,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, then WRITE_SIZE, each scaled by
 # what the same counter reads for actnn_stream_copy of a known size); see profiles/.  None = not
 # measured yet.
-MEASURED_TRAFFIC_BYTES = {
-    # profiles/config2_minimax_pack_unpack_mixed_f32.txt (fetch factor 2.0, write factor 1.0)
-    "minimax": 828540312,
-    "pack_mixed": 889626116,
-    "unpack_mixed": 886690445,
-}
+MEASURED_TRAFFIC_BYTES = {"minimax": 828538264, "pack_mixed": 889626321, "unpack_mixed": 886644877}
 
 
 def _event_time_ms(fn, reps, warmup=3):
