@@ -378,6 +378,7 @@ ACTNN_DEV void channel_totals(const float* __restrict__ part, int64_t c, int64_t
   if (slots == 0) {
     const float* q0 = part + (c * 2) * (int64_t)nsplit;
     const float* q1 = q0 + nsplit;
+#pragma unroll 8
     for (int i = lane; i < nsplit; i += 64) {
       s0 += (double)q0[i];
       s1 += (double)q1[i];
@@ -765,10 +766,10 @@ bool make_plan_cl(int64_t N, int64_t C, int64_t HW, int dtype, Plan& pl) {
   pl.tiles = (int)((C + 255) / 256);
   pl.tpr = (int)((C < 256 ? C : 256) / pl.elems);
   pl.R = kThreads / pl.tpr;
-  // One round of blocks (2048 fit on the chip at once) measured best here: the block's final
-  // reduction over its R rows is dearer than in the default layout.  At least 128 rows per block
-  // keep the table of partial sums below 3 % of the data.
-  constexpr int64_t target = 2048, min_ppb = 128;
+  // One or two rounds of blocks (2048 fit on the chip at once) measured best here: the block's
+  // final reduction over its R rows is dearer than in the default layout.  At least 64 rows per
+  // block keep the table of partial sums below 6 % of the data.
+  constexpr int64_t target = 4096, min_ppb = 64;
   const int64_t want = (target + pl.tiles - 1) / pl.tiles;
   int64_t ppb = (pl.P + want - 1) / want;
   if (ppb < min_ppb) ppb = min_ppb;

@@ -1,5 +1,5 @@
 """Drop-in nn.Module layers that keep their saved activations compressed (behaviour of the
-reference's actnn/actnn/layers.py; conv-transpose and sync-BN variants are not part of this build).
+reference's actnn/actnn/layers.py; the sync-BN variant is not part of this build).
 
 Under torch.autocast the custom autograd functions receive their floating-point arguments already
 cast to the autocast dtype (autocast does not look inside custom Functions); the reference
@@ -15,7 +15,8 @@ from torch.nn.modules.utils import _pair, _single, _triple
 
 from .conf import config
 from .cpp_extension import quantization as ext_quantization
-from .ops import batch_norm, conv1d, conv2d, conv3d, linear
+from .ops import (batch_norm, conv1d, conv2d, conv3d, conv_transpose1d, conv_transpose2d, conv_transpose3d,
+                  linear)
 from .qbnscheme import QBNScheme
 from .qscheme import QScheme
 from .utils import channels_last_format, logical_order, memory_order
@@ -94,6 +95,59 @@ class QConv3d(_QConvMixin, nn.Conv3d):
                  groups=1, bias=True, padding_mode="zeros", group=0):
         super().__init__(in_channels, out_channels, kernel_size, stride, padding, dilation, groups,
                          bias, padding_mode)
+        self._init_scheme(kernel_size, groups, group)
+
+
+class _QConvTransposeMixin:
+    """Shared by QConvTranspose1d/2d/3d (layers.py:101-191)."""
+    _dims = 2
+    _function = conv_transpose2d
+
+    def _init_scheme(self, kernel_size, groups, group):
+        if config.adaptive_conv_scheme:
+            self.scheme = QScheme(self, num_locations=_num_locations(kernel_size, self._dims), group=group,
+                                  depthwise_groups=groups)
+        else:
+            self.scheme = None
+
+    def forward(self, input, output_size=None):
+        if not config.training:
+            return super().forward(input, output_size)
+        if self.padding_mode != "zeros":
+            raise ValueError("Only `zeros` padding mode is supported for %s" % type(self).__name__)
+        output_padding = self._output_padding(input, output_size, self.stride, self.padding, self.kernel_size,
+                                              self._dims, self.dilation)
+        return _autocast_apply(self._function, input, self.weight, self.bias, self.stride, self.padding,
+                               output_padding, self.groups, self.dilation, self.scheme)
+
+
+class QConvTranspose1d(_QConvTransposeMixin, nn.ConvTranspose1d):
+    _dims, _function = 1, conv_transpose1d
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, output_padding=0,
+                 groups=1, bias=True, dilation=1, padding_mode="zeros", group=0):
+        super().__init__(in_channels, out_channels, kernel_size, stride, padding, output_padding, groups,
+                         bias, dilation, padding_mode)
+        self._init_scheme(kernel_size, groups, group)
+
+
+class QConvTranspose2d(_QConvTransposeMixin, nn.ConvTranspose2d):
+    _dims, _function = 2, conv_transpose2d
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, output_padding=0,
+                 groups=1, bias=True, dilation=1, padding_mode="zeros", group=0):
+        super().__init__(in_channels, out_channels, kernel_size, stride, padding, output_padding, groups,
+                         bias, dilation, padding_mode)
+        self._init_scheme(kernel_size, groups, group)
+
+
+class QConvTranspose3d(_QConvTransposeMixin, nn.ConvTranspose3d):
+    _dims, _function = 3, conv_transpose3d
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, output_padding=0,
+                 groups=1, bias=True, dilation=1, padding_mode="zeros", group=0):
+        super().__init__(in_channels, out_channels, kernel_size, stride, padding, output_padding, groups,
+                         bias, dilation, padding_mode)
         self._init_scheme(kernel_size, groups, group)
 
 

@@ -6,9 +6,10 @@ import torch.nn as nn
 
 from .conf import config
 from .layers import (QAvgPool2d, QBatchNorm1d, QBatchNorm2d, QBatchNorm3d, QConv1d, QConv2d, QConv3d,
-                     QDropout, QLinear, QMaxPool2d, QReLU)
+                     QConvTranspose1d, QConvTranspose2d, QConvTranspose3d, QDropout, QLinear, QMaxPool2d,
+                     QReLU)
 
-_Q_TYPES = (QConv1d, QConv2d, QConv3d, QBatchNorm1d, QBatchNorm2d, QBatchNorm3d, QReLU, QDropout,
+_Q_TYPES = (QConv1d, QConv2d, QConv3d, QConvTranspose1d, QConvTranspose2d, QConvTranspose3d, QBatchNorm1d, QBatchNorm2d, QBatchNorm3d, QReLU, QDropout,
             QLinear, QMaxPool2d, QAvgPool2d)
 
 
@@ -20,6 +21,12 @@ def _convert(child):
             return qconv(child.in_channels, child.out_channels, child.kernel_size, child.stride,
                          child.padding, child.dilation, child.groups, child.bias is not None,
                          child.padding_mode)
+    for conv, qconv in ((nn.ConvTranspose1d, QConvTranspose1d), (nn.ConvTranspose2d, QConvTranspose2d),
+                        (nn.ConvTranspose3d, QConvTranspose3d)):
+        if isinstance(child, conv):
+            return qconv(child.in_channels, child.out_channels, child.kernel_size, child.stride,
+                         child.padding, child.output_padding, child.groups, child.bias is not None,
+                         child.dilation, child.padding_mode)
     if config.enable_quantized_bn:
         for bn, qbn in ((nn.BatchNorm1d, QBatchNorm1d), (nn.BatchNorm2d, QBatchNorm2d),
                         (nn.BatchNorm3d, QBatchNorm3d)):

@@ -1,7 +1,6 @@
 """Autograd functions that keep their input compressed between forward and backward, and the
 quantise / dequantise glue around the kernels (behaviour of the reference's
-actnn/actnn/ops.py:22-502; conv-transpose, sync-BN and adaptive pooling variants are not part
-of this build).
+actnn/actnn/ops.py:22-502; sync-BN and adaptive pooling variants are not part of this build).
 """
 import numpy as np
 import torch
@@ -241,6 +240,76 @@ class conv3d(Function):
     @staticmethod
     def backward(ctx, grad_output):
         return _conv_backward(ctx, grad_output, [0, 2, 3, 4], _triple)
+
+
+# ------------------------------------------------------------------------------------------
+# transposed convolution (ops.py:267-383): same saved-input handling, other backward call
+# ------------------------------------------------------------------------------------------
+def _conv_transpose_forward(ctx, forward_op, input, weight, bias, stride, padding, output_padding, groups,
+                            dilation, scheme):
+    started = start_quantize(input, scheme)
+    output = forward_op(input, weight, bias, stride, padding, output_padding, groups, dilation)
+    ctx.scheme = scheme
+    ctx.saved = finish_saved(started, input), weight, bias
+    ctx.other_args = (input.shape, stride, padding, output_padding, dilation, groups)
+    empty_cache(config.empty_cache_threshold)
+    return output
+
+
+def _conv_transpose_backward(ctx, grad_output, bias_reduce_dims, aug):
+    if ctx.scheme:
+        ctx.scheme.set_scale(grad_output)
+    q_input_shape, stride, padding, output_padding, dilation, groups = ctx.other_args
+    padding, output_padding, stride, dilation = aug(padding), aug(output_padding), aug(stride), aug(dilation)
+    quantized, weight, bias = ctx.saved
+    input = dequantize_activation(quantized, q_input_shape)
+    memory_format = getattr(quantized, "memory_format", None) or torch.contiguous_format
+    del quantized, ctx.saved
+    empty_cache(config.empty_cache_threshold)
+    grad_output = grad_output.contiguous(memory_format=memory_format)
+    grad_input, grad_weight = ext_backward_func.cudnn_convolution_transpose_backward(
+        input, grad_output, weight, padding, output_padding, stride, dilation, groups,
+        config.cudnn_benchmark_conv2d, False, False, [ctx.needs_input_grad[0], ctx.needs_input_grad[1]])
+    grad_bias = grad_output.sum(bias_reduce_dims) if bias is not None and ctx.needs_input_grad[2] else None
+    if ctx.scheme:
+        ctx.scheme.if_allocate_perlayer()
+    return grad_input, grad_weight, grad_bias, None, None, None, None, None, None
+
+
+class conv_transpose1d(Function):
+    @staticmethod
+    def forward(ctx, input, weight, bias=None, stride=1, padding=0, output_padding=0, groups=1, dilation=1,
+                scheme=None):
+        return _conv_transpose_forward(ctx, F.conv_transpose1d, input, weight, bias, stride, padding,
+                                       output_padding, groups, dilation, scheme)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return _conv_transpose_backward(ctx, grad_output, [0, 2], _single)
+
+
+class conv_transpose2d(Function):
+    @staticmethod
+    def forward(ctx, input, weight, bias=None, stride=1, padding=0, output_padding=0, groups=1, dilation=1,
+                scheme=None):
+        return _conv_transpose_forward(ctx, F.conv_transpose2d, input, weight, bias, stride, padding,
+                                       output_padding, groups, dilation, scheme)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return _conv_transpose_backward(ctx, grad_output, [0, 2, 3], _pair)
+
+
+class conv_transpose3d(Function):
+    @staticmethod
+    def forward(ctx, input, weight, bias=None, stride=1, padding=0, output_padding=0, groups=1, dilation=1,
+                scheme=None):
+        return _conv_transpose_forward(ctx, F.conv_transpose3d, input, weight, bias, stride, padding,
+                                       output_padding, groups, dilation, scheme)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return _conv_transpose_backward(ctx, grad_output, [0, 2, 3, 4], _triple)
 
 
 # ------------------------------------------------------------------------------------------

@@ -141,31 +141,41 @@ def other_configs(device, reps):
     t = _event_time_ms(lambda: ext_q.max_pool2d_backward(gp, idx, x.shape, k, s, p), reps)
     out["max_pool2d_backward_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
     del y, mask, yp, idx, gp
-    # training-mode batch norm on the same tensor: forward (statistics + normalise, with and without
-    # the quantiser's group min/max from the statistics pass), backward from the full-precision
-    # input and backward straight from the 2-bit stream
+    # training-mode batch norm on the same tensor, in both layouts: forward (statistics + normalise;
+    # with the quantiser's group min/max from the statistics pass; with the 2-bit pack in the
+    # normalising pass), backward from the full-precision input and straight from the 2-bit stream
     import actnn_amd.cpp_extension.backward_func as ext_bf
+    from actnn_amd.ops import _Quantized
+    from actnn_amd.utils import memory_order
     C = x.shape[1]
     w = torch.rand(C, device=device) + 0.5
     bias = torch.randn(C, device=device)
-    b = 3 * 2 * n
-    t = _event_time_ms(lambda: ext_bf.hip_batch_norm_forward(x, w, bias, None, None, 0.1, 1e-5), reps)
-    out["batch_norm_forward_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
-    b = 3 * 2 * n + 2 * 2 * n / 256
-    t = _event_time_ms(lambda: ext_bf.hip_batch_norm_forward(x, w, bias, None, None, 0.1, 1e-5, minmax=True), reps)
-    out["batch_norm_forward_with_group_minmax_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
-    _, mean, invstd, lo, hi = ext_bf.hip_batch_norm_forward(x, w, bias, None, None, 0.1, 1e-5, minmax=True)
-    b = 5 * 2 * n
-    t = _event_time_ms(lambda: ext_bf.hip_batch_norm_backward(x, g, w, mean, invstd), reps)
-    out["batch_norm_backward_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
     Nb, Gb = x.shape[0], n // x.shape[0] // 256
     host_bits = torch.full((Nb,), 2, dtype=torch.int32)
     bits2 = ext_q.attach_bits_host(host_bits.to(device), host_bits)
-    q_in, q_scale = ext_q.pack_mixed_precision(x.view(Nb, Gb, 256), lo.view(Nb, Gb, 1), hi.view(Nb, Gb, 1), bits2, True)
-    quantized = (q_in, bits2, q_scale, lo.view(Nb, Gb, 1))
-    b = 3 * 2 * n + 2 * (2 * n / 8 + 2 * 2 * n / 256)       # dy twice, dx once; stream, scale, min twice
-    t = _event_time_ms(lambda: ext_bf.hip_batch_norm_backward_packed(x.shape, quantized, g, w, mean, invstd), reps)
-    out["batch_norm_backward_from_2bit_stream_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
+    for tag, fmt in (("", torch.contiguous_format), ("_channels_last", torch.channels_last)):
+        xb, gb = x.contiguous(memory_format=fmt), g.contiguous(memory_format=fmt)
+
+        def rate(name, nbytes, fn):
+            t = _event_time_ms(fn, reps)
+            out[name + tag + "_f16"] = {"ms": t, "GB/s": nbytes / t / 1e6, "frac": nbytes / t / 1e6 / HBM_PEAK_GBS}
+        rate("batch_norm_forward", 3 * 2 * n, lambda: ext_bf.hip_batch_norm_forward(xb, w, bias, None, None, 0.1, 1e-5))
+        rate("batch_norm_forward_with_group_minmax", 3 * 2 * n + 2 * 2 * n / 256,
+             lambda: ext_bf.hip_batch_norm_forward(xb, w, bias, None, None, 0.1, 1e-5, minmax=True))
+        ws, mean, invstd, lo, hi = ext_bf.hip_batch_norm_forward_stats(xb, w, bias, None, None, 0.1, 1e-5)
+        lo3, hi3 = lo.view(Nb, Gb, 1), hi.view(Nb, Gb, 1)
+        # statistics + min/max, then normalise + 2-bit pack: x twice, y, stream, min/max/scale
+        rate("batch_norm_forward_with_pack", 3 * 2 * n + 2 * n / 8 + 5 * 2 * n / 256,
+             lambda: ext_bf.hip_batch_norm_forward_apply(
+                 xb, ext_bf.hip_batch_norm_forward_stats(xb, w, bias, None, None, 0.1, 1e-5)[0], bits2, lo3, hi3))
+        rate("batch_norm_backward", 5 * 2 * n, lambda: ext_bf.hip_batch_norm_backward(xb, gb, w, mean, invstd))
+        q_in, q_scale = ext_q.pack_mixed_precision(memory_order(xb).reshape(Nb, Gb, 256), lo3, hi3, bits2, True)
+        quantized = _Quantized((q_in, bits2, q_scale, lo3))
+        quantized.memory_format = None if fmt == torch.contiguous_format else fmt
+        # dy twice, dx once; stream, scale, min twice
+        rate("batch_norm_backward_from_2bit_stream", 3 * 2 * n + 2 * (2 * n / 8 + 2 * 2 * n / 256),
+             lambda: ext_bf.hip_batch_norm_backward_packed(xb.shape, quantized, gb, w, mean, invstd))
+        del xb, gb
     del x, g, q_in, q_scale, quantized, lo, hi
     # config 4 input through the fixed-width path (2 bits)
     M, I = 8192, 4096

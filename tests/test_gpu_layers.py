@@ -310,3 +310,30 @@ def test_resnet50_channels_last_step_runs():
         loss.backward()
     assert torch.isfinite(loss)
     assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in model.parameters())
+
+
+@pytest.mark.parametrize("dims", [1, 2, 3])
+def test_conv_transpose_8bit_close_to_exact(dims):
+    """QConvTranspose1d/2d/3d (layers.py:101-191 of the reference): forward is the stock operator,
+    gradients from the 8-bit saved input are within the reference's 8-bit tolerance of the exact
+    ones; QModule converts the stock layers."""
+    config.activation_compression_bits = [8]
+    config.initial_bits = 8
+    config.perlayer = False
+    torch.manual_seed(dims)
+    stock = {1: nn.ConvTranspose1d, 2: nn.ConvTranspose2d, 3: nn.ConvTranspose3d}[dims]
+    quant = {1: actnn_amd.QConvTranspose1d, 2: actnn_amd.QConvTranspose2d, 3: actnn_amd.QConvTranspose3d}[dims]
+    spatial = {1: (64,), 2: (16, 16), 3: (4, 8, 8)}[dims]
+    ref = stock(32, 16, 3, stride=2, padding=1, output_padding=1).to(DEV)
+    q = quant(32, 16, 3, stride=2, padding=1, output_padding=1).to(DEV)
+    q.load_state_dict(ref.state_dict())
+    wrapped = QModule(nn.Sequential(stock(32, 16, 3, stride=2, padding=1, output_padding=1)))
+    assert isinstance(wrapped.model[0], quant)
+    x = torch.randn(4, 32, *spatial, device=DEV)
+    g = torch.randn(4, 16, *[2 * s for s in spatial], device=DEV)
+    yq, gxq, gpq = _grads(q, x, g)
+    yr, gxr, gpr = _grads(ref, x, g)
+    assert torch.allclose(yq, yr, atol=2e-3, rtol=1e-2)
+    assert torch.allclose(gxq, gxr, atol=1e-1, rtol=1e-1)
+    for a, b in zip(gpq, gpr):
+        assert (a - b).norm() / b.norm() < 2e-2
