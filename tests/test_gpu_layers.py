@@ -337,3 +337,39 @@ def test_conv_transpose_8bit_close_to_exact(dims):
     assert torch.allclose(gxq, gxr, atol=1e-1, rtol=1e-1)
     for a, b in zip(gpq, gpr):
         assert (a - b).norm() / b.norm() < 2e-2
+
+
+@pytest.mark.parametrize("channels_last", [False, True])
+def test_batch_norm_fused_and_unfused_paths_save_the_same_stream(channels_last):
+    """QBatchNorm2d at L3: the fused sequence (statistics + min/max, allocation, normalise + pack;
+    backward from the stream) and the reference's sequence (minimax, pack, library batch norm;
+    unpack + backward) save bit-identical tuples for the same generator state, with the widths
+    allocated on the device or on the host, and give matching outputs and gradients."""
+    def run(fused, device_allocation):
+        config.reset(); QScheme.reset(); QBNScheme.reset()
+        config.fused_bn_pack = config.fused_bn_backward = fused
+        config.device_allocation = device_allocation
+        config.perlayer = False
+        torch.manual_seed(0)
+        conv = actnn_amd.QConv2d(16, 64, 3, padding=1).to(DEV)        # gives the BN scheme its predecessor
+        bn = actnn_amd.QBatchNorm2d(64).to(DEV)
+        x = torch.randn(24, 16, 16, 16, device=DEV)
+        if channels_last:
+            conv, bn = conv.to(memory_format=torch.channels_last), bn.to(memory_format=torch.channels_last)
+            x = x.contiguous(memory_format=torch.channels_last)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            h = conv(x)
+            torch.cuda.manual_seed(11)
+            y = bn(h)
+        saved = y.grad_fn.saved[0]
+        g = torch.randn_like(y)
+        gh, gw = torch.autograd.grad(y, [h, bn.weight], g)        # the saved tuple is released by backward
+        return y, saved, gh, gw
+    ref = run(False, False)
+    for fused, dev_alloc in ((True, True), (True, False), (False, True)):
+        y, saved, gh, gw = run(fused, dev_alloc)
+        assert torch.equal(saved[1].cpu(), ref[1][1].cpu())                       # widths
+        assert torch.equal(saved[0], ref[1][0]) and torch.equal(saved[2], ref[1][2]) and torch.equal(saved[3], ref[1][3])
+        assert torch.allclose(y.float(), ref[0].float(), atol=2e-2, rtol=2e-2)
+        assert torch.allclose(gh.float(), ref[2].float(), atol=3e-2, rtol=3e-2)
+        assert torch.allclose(gw, ref[3], rtol=2e-2, atol=2e-1)
