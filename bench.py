@@ -58,6 +58,9 @@ def make_config2(device, N=256, C=256, H=56, W=56, seed=0):
     s_c = torch.exp(torch.randn(C, generator=g, device=device))
     x = torch.randn(N, C, H, W, generator=g, device=device)
     x = torch.relu_(x).mul_(s_c.view(1, C, 1, 1))
+    # samples differ in range (LogNormal(0, 0.7) per sample): with identically distributed samples
+    # the greedy allocation hands every sample the same width and the mixed-width path is not used
+    x.mul_(torch.exp(0.7 * torch.randn(N, generator=g, device=device)).view(N, 1, 1, 1))
     gs = 256
     G = C * H * W // gs
     xg = x.view(N, G, gs)
