@@ -2,6 +2,7 @@
 (behaviour of the reference's actnn/actnn/module.py:14-100)."""
 from collections import OrderedDict
 
+import torch
 import torch.nn as nn
 
 from .conf import config
@@ -49,10 +50,16 @@ def _convert(child):
 
 
 class QModule(nn.Module):
-    def __init__(self, model):
+    def __init__(self, model, channels_last=False):
+        """`channels_last=True` (an addition to the reference's signature) keeps 4-D parameters
+        and inputs in the channels-last layout, the one this GPU's convolution kernels work in; the
+        Q-layers then compress activations in memory order without transposes."""
         super().__init__()
         self.model = model
+        self.channels_last = bool(channels_last)
         QModule.convert_layers(model)
+        if self.channels_last:
+            self.model.to(memory_format=torch.channels_last)
 
     @staticmethod
     def convert_layers(module):
@@ -66,7 +73,19 @@ class QModule(nn.Module):
                 setattr(module, name, new)
 
     def forward(self, *args, **kwargs):
+        if self.channels_last:
+            args = tuple(a.contiguous(memory_format=torch.channels_last)
+                         if isinstance(a, torch.Tensor) and a.dim() == 4 else a for a in args)
         return self.model(*args, **kwargs)
+
+    def _apply(self, fn, recurse=True):
+        # .to(device) / .half() of the wrapper must not undo the layout of the parameters
+        ret = super()._apply(fn, recurse)
+        if getattr(self, "channels_last", False):
+            for p in self.model.parameters():
+                if p.dim() == 4 and not p.is_contiguous(memory_format=torch.channels_last):
+                    p.data = p.data.contiguous(memory_format=torch.channels_last)
+        return ret
 
     def train(self, mode=True):
         config.training = mode

@@ -373,3 +373,47 @@ def test_batch_norm_fused_and_unfused_paths_save_the_same_stream(channels_last):
         assert torch.allclose(y.float(), ref[0].float(), atol=2e-2, rtol=2e-2)
         assert torch.allclose(gh.float(), ref[2].float(), atol=3e-2, rtol=3e-2)
         assert torch.allclose(gw, ref[3], rtol=2e-2, atol=2e-1)
+
+
+@pytest.mark.parametrize("channels_last", [False, True])
+@pytest.mark.parametrize("level", ["L0", "L1", "L2", "L3", "L3.1", "L4", "swap"])
+def test_every_optimization_level_trains_a_step(level, channels_last):
+    """All levels of set_optimization_level (conf.py:5-36) run two training steps of a small
+    conv / BN / ReLU / max-pool / dropout / linear model in both memory layouts, with finite
+    gradients close to the exact model's at the levels that keep 4 bits or more."""
+    def make():
+        torch.manual_seed(0)
+        return nn.Sequential(nn.Conv2d(8, 32, 3, padding=1, bias=False), nn.BatchNorm2d(32), nn.ReLU(),
+                             nn.MaxPool2d(3, 2, 1), nn.Conv2d(32, 64, 1), nn.BatchNorm2d(64), nn.ReLU(),
+                             nn.Dropout(0.0), nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(64, 10))
+    set_optimization_level(level)
+    if level == "L3.1":
+        config.pipeline_threshold = 1 << 16                 # force the micro-batched conv backward
+    exact = make().to(DEV)
+    quant = QModule(make()).to(DEV)
+    quant.load_state_dict(exact.state_dict())
+    x = torch.randn(16, 8, 32, 32, device=DEV)
+    if channels_last:
+        exact, quant = exact.to(memory_format=torch.channels_last), quant.to(memory_format=torch.channels_last)
+        x = x.contiguous(memory_format=torch.channels_last)
+    y = torch.randint(0, 10, (16,), device=DEV)
+    for model in (exact, quant):
+        for _ in range(2):
+            model.zero_grad()
+            F.cross_entropy(model(x), y).backward()
+    for (name, p), q in zip(exact.named_parameters(), quant.parameters()):
+        assert q.grad is not None and torch.isfinite(q.grad).all(), name
+        if level in ("L0", "L1", "L2", "swap"):
+            assert (q.grad - p.grad).norm() <= 0.25 * p.grad.norm() + 1e-3, name
+
+
+def test_qmodule_channels_last_option():
+    torch.manual_seed(0)
+    net = nn.Sequential(nn.Conv2d(8, 32, 3, padding=1), nn.BatchNorm2d(32), nn.ReLU(), nn.Conv2d(32, 16, 1))
+    model = QModule(net, channels_last=True).to(DEV)
+    assert all(p.is_contiguous(memory_format=torch.channels_last) for p in model.parameters() if p.dim() == 4)
+    x = torch.randn(4, 8, 16, 16, device=DEV, requires_grad=True)          # default-layout input
+    y = model(x)
+    assert y.is_contiguous(memory_format=torch.channels_last)
+    y.sum().backward()
+    assert x.grad.shape == x.shape and torch.isfinite(x.grad).all()
