@@ -175,7 +175,7 @@ template <typename T> struct PlainInput {
 // Values are rebuilt exactly as actnn_unpack_mixed rebuilds them.  16-bit types only.
 template <typename T> struct PackedInput {
   static constexpr bool kRows = false;
-  static constexpr int kInFlight = 2;      // the decode needs registers: 2 measured faster than 4
+  static constexpr int kInFlight = 2;      // the decode needs registers: 2 measured faster than 1 and 4
   const int32_t* words;
   const int32_t* bits;
   const int32_t* prefix;
@@ -185,23 +185,50 @@ template <typename T> struct PackedInput {
   uint32_t lane32;
   bool active;
   struct Raw { uint32_t lo, hi; float sc, m; int b; };
-  ACTNN_DEV Raw fetch_group(int64_t n, int64_t grp) const {
-    Raw r{0u, 0u, 1.0f, 0.0f, 1};
+  // group `grp` of sample n, whose width b and first word (prefix[n] * G * 8) the caller knows
+  ACTNN_DEV Raw fetch_known(int64_t n, int64_t grp, int b, int64_t first_word) const {
+    Raw r{0u, 0u, 1.0f, 0.0f, b};
     if (active) {
-      r.b = bits[n];
-      const int32_t* w = words + ((int64_t)prefix[n] * G + grp * r.b) * 8;
-      if ((int)lane32 < 8 * r.b) r.lo = (uint32_t)w[lane32];
-      if ((int)lane32 + 32 < 8 * r.b) r.hi = (uint32_t)w[lane32 + 32];
+      const int32_t* w = words + first_word + grp * b * 8;
+      if ((int)lane32 < 8 * b) r.lo = (uint32_t)w[lane32];
+      if ((int)lane32 + 32 < 8 * b) r.hi = (uint32_t)w[lane32 + 32];
       r.sc = Conv<T>::load(scale, n * G + grp);
       r.m = Conv<T>::load(mn, n * G + grp);
     }
     return r;
   }
-  ACTNN_DEV Raw fetch(int64_t n) const { return fetch_group(n, g); }
+  ACTNN_DEV Raw fetch(int64_t n) const {
+    return fetch_known(n, g, active ? bits[n] : 1, active ? (int64_t)prefix[n] * G * 8 : 0);
+  }
   template <int BITS> ACTNN_DEV u32x4 decode_bits(const Raw& r) const {
     uint64_t acc = transpose32(r.lo, lane32);
     if (BITS > 4) acc |= (uint64_t)transpose32(r.hi, lane32) << 32;
     const Dequant<T> dq(r.sc, r.m);
+    if constexpr (BITS <= 2) {
+      // A group at 1 or 2 bits has at most four distinct values.  Lane l evaluates level l & 3
+      // (11 operations once instead of once per element), the four lanes of a quad exchange them
+      // (DPP quad_perm broadcasts) into an 8-byte table, and every pair of elements is one byte
+      // permute of that table.  Same arithmetic per level, hence the same bits.
+      const float mine = dq(lane32 & 3u);
+      const float pair[2] = {mine, mine};
+      const int h = (int)(Chunk<T>::narrow(pair) & 0xffffu);
+      const uint32_t l0 = (uint32_t)__builtin_amdgcn_update_dpp(0, h, 0x00, 0xF, 0xF, true);   // quad_perm [0,0,0,0]
+      const uint32_t l1 = (uint32_t)__builtin_amdgcn_update_dpp(0, h, 0x55, 0xF, 0xF, true);   // [1,1,1,1]
+      const uint32_t l2 = (uint32_t)__builtin_amdgcn_update_dpp(0, h, 0xAA, 0xF, 0xF, true);   // [2,2,2,2]
+      const uint32_t l3 = (uint32_t)__builtin_amdgcn_update_dpp(0, h, 0xFF, 0xF, 0xF, true);   // [3,3,3,3]
+      const uint32_t lut_lo = l0 | (l1 << 16), lut_hi = l2 | (l3 << 16);
+      const uint32_t a = (uint32_t)acc;
+      uint32_t out[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t c0 = (a >> (2 * j * BITS)) & ((1u << BITS) - 1u);
+        const uint32_t c1 = (a >> ((2 * j + 1) * BITS)) & ((1u << BITS) - 1u);
+        // bytes 2c, 2c+1 of the table for each of the two elements
+        const uint32_t sel = (c0 * 0x0202u + 0x0100u) | ((c1 * 0x0202u + 0x0100u) << 16);
+        out[j] = __builtin_amdgcn_perm(lut_hi, lut_lo, sel);
+      }
+      return u32x4{out[0], out[1], out[2], out[3]};
+    }
     float v[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) v[k] = dq((uint32_t)(acc >> (k * BITS)) & ((1u << BITS) - 1u));
@@ -252,12 +279,13 @@ ACTNN_DEV void pack_chunk_bits(const float (&v)[8], const uint32_t (&r16)[8], fl
   }
 }
 
+// b = bits[n], first_word = prefix[n] * G * 8: looked up by the caller, who knows how often n changes
 template <typename T>
-ACTNN_DEV void pack_chunk(const PackSink& ps, const u32x4& ux, int64_t n, int64_t grp, int64_t octet) {
+ACTNN_DEV void pack_chunk(const PackSink& ps, const u32x4& ux, int64_t n, int64_t grp, int64_t octet, int b,
+                          int64_t first_word) {
   constexpr int PD = Chunk<T>::kPerDword;
   static_assert(Chunk<T>::kElems == 8, "16-bit types only");
   const uint32_t lane32 = threadIdx.x & 31;
-  const int b = ps.bits[n];
   const int64_t gi = n * ps.G + grp;
   float mul, sub;
   const float sc = GroupQuant<T, false>::prepare(Conv<T>::load(static_cast<const T*>(ps.mn), gi),
@@ -269,7 +297,7 @@ ACTNN_DEV void pack_chunk(const PackSink& ps, const u32x4& ux, int64_t n, int64_
   for (int k = 0; k < 4; ++k) Chunk<T>::widen(w[k], v + k * PD);
   uint32_t r16[8];
   philox_octet((uint64_t)octet, ps.seed, ps.offset, r16);
-  int32_t* dst = ps.packed + ((int64_t)ps.prefix[n] * ps.G + grp * b) * 8;
+  int32_t* dst = ps.packed + first_word + grp * b * 8;
   switch (b) {                           // uniform over the half-wave: one sample, one width
     case 1: pack_chunk_bits<1>(v, r16, mul, sub, lane32, dst); break;
     case 2: pack_chunk_bits<2>(v, r16, mul, sub, lane32, dst); break;
@@ -462,7 +490,7 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
   constexpr int E = Chunk<T>::kElems;
   constexpr int PD = Chunk<T>::kPerDword;
   constexpr int NC = BWD ? 3 : 2;
-  constexpr int kUnroll = PACK ? 2 : XS::kInFlight;
+  constexpr int kUnroll = PACK ? 2 : XS::kInFlight;      // measured: 2 beats 1 and 4 with the pack
   const Place p = place_of<E>(F, HW);
   if (!p.active) return;               // whole quantisation groups (32 lanes) leave together
   bind_input(xs, p);
@@ -517,14 +545,17 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
     for (int u = 0; u < kUnroll; ++u) {
       const u32x4 ux = xs.decode(rx[u]);
       store_out(po + (n + u) * F, apply(ux, BWD ? ud[u] : ux));
-      if constexpr (PACK) pack_chunk<T>(ps, ux, n + u, p.elem >> 8, ((n + u) * F + p.elem) >> 3);
+      if constexpr (PACK)
+        pack_chunk<T>(ps, ux, n + u, p.elem >> 8, ((n + u) * F + p.elem) >> 3, ps.bits[n + u],
+                      (int64_t)ps.prefix[n + u] * ps.G * 8);
     }
   }
   for (; n < n1; ++n) {
     const typename XS::Raw rx = xs.fetch(n);
     const u32x4 ux = xs.decode(rx);
     store_out(po + n * F, apply(ux, BWD ? load_last(pd + n * F) : ux));
-    if constexpr (PACK) pack_chunk<T>(ps, ux, n, p.elem >> 8, (n * F + p.elem) >> 3);
+    if constexpr (PACK)
+      pack_chunk<T>(ps, ux, n, p.elem >> 8, (n * F + p.elem) >> 3, ps.bits[n], (int64_t)ps.prefix[n] * ps.G * 8);
   }
 }
 
@@ -558,11 +589,23 @@ template <typename T> struct PackedRows {
     col = column;
     in.lane32 = threadIdx.x & 31;
     in.active = true;
+    cur_n = 0xffffffffu;
   }
-  ACTNN_DEV Raw fetch(int64_t row) const {
+  // A thread stays inside one sample for many rows: the sample's width and first word are kept
+  // in registers and reloaded only when the row moves on to the next sample, which takes two
+  // dependent loads off the path of every fetch.
+  uint32_t cur_n;
+  int cur_b;
+  int64_t cur_first;
+  ACTNN_DEV Raw fetch(int64_t row) {
     const uint32_t n = (uint32_t)row / HW;                 // rows < 2^31 (checked by the launcher)
+    if (n != cur_n) {
+      cur_n = n;
+      cur_b = in.bits[n];
+      cur_first = (int64_t)in.prefix[n] * in.G * 8;
+    }
     const int64_t grp = ((row * C + col) >> 8) - (int64_t)n * in.G;
-    return in.fetch_group(n, grp);
+    return in.fetch_known(n, grp, cur_b, cur_first);
   }
   ACTNN_DEV u32x4 decode(const Raw& r) const { return in.decode(r); }
 };
@@ -676,12 +719,20 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
   constexpr int E = Chunk<T>::kElems;
   constexpr int PD = Chunk<T>::kPerDword;
   constexpr int NC = BWD ? 3 : 2;
-  constexpr int U = PACK ? 2 : XS::kInFlight;
+  constexpr int U = PACK ? 1 : XS::kInFlight;            // measured: 1 beats 2 and 4 with the pack here
+  uint32_t cur_n = 0xffffffffu;          // the sample whose width and first word are held below
+  int cur_b = 1;
+  int64_t cur_first = 0;
   auto pack_row = [&](const u32x4& ux, int64_t row, int64_t col) {
     if constexpr (PACK) {
       const uint32_t n = (uint32_t)row / HW;               // rows < 2^31 (checked by the launcher)
+      if (n != cur_n) {
+        cur_n = n;
+        cur_b = ps.bits[n];
+        cur_first = (int64_t)ps.prefix[n] * ps.G * 8;
+      }
       const int64_t flat = row * C + col;
-      pack_chunk<T>(ps, ux, n, (flat >> 8) - (int64_t)n * ps.G, flat >> 3);
+      pack_chunk<T>(ps, ux, n, (flat >> 8) - (int64_t)n * ps.G, flat >> 3, cur_b, cur_first);
     }
   };
   const RowTile t = row_tile<E>(C, tpr, R);
@@ -944,7 +995,7 @@ int backward_packed(const Plan& pl, const int32_t* packed, const int32_t* bits, 
   const PackedInput<T> in{packed, bits, prefix, static_cast<const T*>(scale), static_cast<const T*>(mn),
                           pl.F / 256, 0, 0u, false};
   if (pl.channels_last) {
-    const PackedRows<T> xs{in, C, 0, (uint32_t)HW};
+    const PackedRows<T> xs{in, C, 0, (uint32_t)HW, 0xffffffffu, 1, 0};
     return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
   }
   return backward_t<T>(pl, in, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
