@@ -589,23 +589,23 @@ template <typename T> struct PackedRows {
     col = column;
     in.lane32 = threadIdx.x & 31;
     in.active = true;
-    cur_n = 0xffffffffu;
+    cur_row0 = -(int64_t)HW - 1;                           // no row is inside: the first fetch looks up
   }
   // A thread stays inside one sample for many rows: the sample's width and first word are kept
   // in registers and reloaded only when the row moves on to the next sample, which takes two
   // dependent loads off the path of every fetch.
-  uint32_t cur_n;
+  uint32_t cur_n;        // sample of the last fetch; cur_row0 = cur_n * HW
   int cur_b;
-  int64_t cur_first;
+  int64_t cur_first, cur_row0;
   ACTNN_DEV Raw fetch(int64_t row) {
-    const uint32_t n = (uint32_t)row / HW;                 // rows < 2^31 (checked by the launcher)
-    if (n != cur_n) {
-      cur_n = n;
-      cur_b = in.bits[n];
-      cur_first = (int64_t)in.prefix[n] * in.G * 8;
+    if ((uint64_t)(row - cur_row0) >= HW) {                // left the sample (or the first fetch)
+      cur_n = (uint32_t)row / HW;                          // rows < 2^31 (checked by the launcher)
+      cur_row0 = (int64_t)cur_n * HW;
+      cur_b = in.bits[cur_n];
+      cur_first = (int64_t)in.prefix[cur_n] * in.G * 8;
     }
-    const int64_t grp = ((row * C + col) >> 8) - (int64_t)n * in.G;
-    return in.fetch_known(n, grp, cur_b, cur_first);
+    const int64_t grp = ((row * C + col) >> 8) - (int64_t)cur_n * in.G;
+    return in.fetch_known(cur_n, grp, cur_b, cur_first);
   }
   ACTNN_DEV u32x4 decode(const Raw& r) const { return in.decode(r); }
 };
@@ -720,19 +720,19 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
   constexpr int PD = Chunk<T>::kPerDword;
   constexpr int NC = BWD ? 3 : 2;
   constexpr int U = PACK ? 1 : XS::kInFlight;            // measured: 1 beats 2 and 4 with the pack here
-  uint32_t cur_n = 0xffffffffu;          // the sample whose width and first word are held below
+  uint32_t cur_n = 0;                    // the sample whose width and first word are held below
   int cur_b = 1;
-  int64_t cur_first = 0;
+  int64_t cur_first = 0, cur_row0 = -(int64_t)HW - 1;
   auto pack_row = [&](const u32x4& ux, int64_t row, int64_t col) {
     if constexpr (PACK) {
-      const uint32_t n = (uint32_t)row / HW;               // rows < 2^31 (checked by the launcher)
-      if (n != cur_n) {
-        cur_n = n;
-        cur_b = ps.bits[n];
-        cur_first = (int64_t)ps.prefix[n] * ps.G * 8;
+      if ((uint64_t)(row - cur_row0) >= HW) {              // left the sample (or the first row)
+        cur_n = (uint32_t)row / HW;                        // rows < 2^31 (checked by the launcher)
+        cur_row0 = (int64_t)cur_n * HW;
+        cur_b = ps.bits[cur_n];
+        cur_first = (int64_t)ps.prefix[cur_n] * ps.G * 8;
       }
       const int64_t flat = row * C + col;
-      pack_chunk<T>(ps, ux, n, (flat >> 8) - (int64_t)n * ps.G, flat >> 3, cur_b, cur_first);
+      pack_chunk<T>(ps, ux, cur_n, (flat >> 8) - (int64_t)cur_n * ps.G, flat >> 3, cur_b, cur_first);
     }
   };
   const RowTile t = row_tile<E>(C, tpr, R);
@@ -995,7 +995,7 @@ int backward_packed(const Plan& pl, const int32_t* packed, const int32_t* bits, 
   const PackedInput<T> in{packed, bits, prefix, static_cast<const T*>(scale), static_cast<const T*>(mn),
                           pl.F / 256, 0, 0u, false};
   if (pl.channels_last) {
-    const PackedRows<T> xs{in, C, 0, (uint32_t)HW, 0xffffffffu, 1, 0};
+    const PackedRows<T> xs{in, C, 0, (uint32_t)HW, 0u, 1, 0, 0};
     return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
   }
   return backward_t<T>(pl, in, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
