@@ -12,7 +12,7 @@ from .conf import config
 from .cpp_extension import backward_func as ext_backward_func
 from .cpp_extension import quantization as ext_quantization
 from .utils import (channels_last_format, compute_tensor_bytes, empty_cache, get_memory_usage,
-                    logical_order, swap_to_cpu)
+                    logical_order, swap_to_cpu, swap_to_device)
 
 
 # ------------------------------------------------------------------------------------------
@@ -48,7 +48,7 @@ def dequantize_and_unpack(data, shape, bits, scale, mn):
     if config.simulate:
         return data / scale + mn
     if config.swap:
-        data = data.cuda(non_blocking=True)
+        data = swap_to_device(data)
     N = shape[0]
     gs = config.group_size
     features = int(np.prod(shape[1:]))
@@ -103,7 +103,7 @@ def dequantize_activation(quantized, q_input_shape):
     """Rebuild a tensor of shape q_input_shape (ops.py:121-139)."""
     if not config.compress_activation:
         ret = quantized[0]
-        return ret.cuda(non_blocking=True) if config.swap else ret
+        return swap_to_device(ret) if config.swap else ret
     q_input, q_bits, q_scale, q_min = quantized
     if q_scale.dtype == torch.bfloat16 and _stored_as_bf16(q_input_shape, quantized):
         q_scale = q_scale.to(torch.float32)
@@ -381,7 +381,7 @@ class batch_norm(Function):
     @staticmethod
     def forward(ctx, input, running_mean, running_var, weight, bias, training,
                 exponential_average_factor, eps, scheme):
-        if (scheme and config.fused_bn_pack and not config.swap
+        if (scheme and config.fused_bn_pack
                 and _bn_shares_min_max(input, weight, bias, running_mean, running_var, training)
                 and ext_backward_func.hip_batch_norm_pack_applies(input, weight, bias, running_mean, running_var)):
             # two reads of the input in total: the statistics pass also yields the quantiser's
@@ -393,6 +393,8 @@ class batch_norm(Function):
                 scheme.start_quantization_bits(input, (mn, mx)))
             output, q_input, q_scale = ext_backward_func.hip_batch_norm_forward_apply(
                 input, ws, q_bits, q_min, q_max)
+            if config.swap:
+                q_input = swap_to_cpu(q_input)
             reserve = None
             started = ("done", _mark_saved(_Quantized((q_input, q_bits, q_scale, q_min)), input))
         elif _bn_shares_min_max(input, weight, bias, running_mean, running_var, training):
@@ -428,8 +430,12 @@ class batch_norm(Function):
     @staticmethod
     def backward(ctx, grad_output):
         quantized, weight, running_mean, running_var, save_mean, save_var, training, eps, reserve = ctx.saved
-        if (training and config.compress_activation and not config.simulate and not config.swap
+        if (training and config.compress_activation and not config.simulate
                 and config.group_size == 256 and config.fused_bn_backward):
+            if config.swap and isinstance(quantized[0], torch.Tensor) and not quantized[0].is_cuda:
+                back = _Quantized((swap_to_device(quantized[0]),) + tuple(quantized[1:]))
+                back.native_bf16, back.memory_format = quantized.native_bf16, quantized.memory_format
+                quantized = back
             grad_output = grad_output.contiguous(
                 memory_format=getattr(quantized, "memory_format", None) or torch.contiguous_format)
             if ext_backward_func.hip_batch_norm_backward_packed_applies(

@@ -1,16 +1,95 @@
 """Memory accounting and small helpers (reference: actnn/actnn/utils.py:10-80)."""
 import json
+import weakref
 from collections import OrderedDict
 
 import numpy as np
 import torch
 
 
+class _SwapSpace:
+    """Host parking for saved tensors (levels L4 / swap; the reference copies with
+    `non_blocking=True` on the compute stream, utils.py:10-13, and copies back the same way,
+    ops.py:59-60, so every transfer sits in the path of the kernels around it).
+
+    Here a separate copy stream (default priority) carries both directions: a tensor is parked as
+    soon as the compute stream has produced it, while the forward pass goes on; in the backward
+    pass, asking for a tensor also starts the transfers of the `depth` tensors parked before it -
+    the ones the backward pass will ask for next - so that they arrive while the current layer
+    computes.  Events order the two streams; `record_stream` keeps every buffer alive until the
+    other stream is done with it."""
+    depth = 3
+
+    def __init__(self):
+        self.streams = {}
+        self.parked = []                      # weak references to the host tensors, in parking order
+
+    def _stream(self, device):
+        key = torch.device(device).index or 0
+        if key not in self.streams:
+            self.streams[key] = torch.cuda.Stream(device=device)
+        return self.streams[key]
+
+    def park(self, tensor):
+        device = tensor.device
+        copy = self._stream(device)
+        host = torch.empty(tensor.shape, dtype=tensor.dtype, device="cpu", pin_memory=True)
+        copy.wait_stream(torch.cuda.current_stream(device))       # the tensor is complete by then
+        with torch.cuda.stream(copy):
+            host.copy_(tensor, non_blocking=True)
+            done = torch.cuda.Event()
+            done.record(copy)
+        tensor.record_stream(copy)                                 # not reused before the copy has run
+        host._actnn_swap = {"done": done, "device": device, "ahead": None}
+        if len(self.parked) > 4096:                                # forward-only use: forget the dead ones
+            self.parked = [r for r in self.parked if r() is not None]
+        self.parked.append(weakref.ref(host))
+        return host
+
+    def _start(self, host):
+        meta = host._actnn_swap
+        if meta["ahead"] is None:
+            copy = self._stream(meta["device"])
+            with torch.cuda.stream(copy):                          # same stream as the parking copy: ordered
+                dev = host.to(meta["device"], non_blocking=True)
+                arrived = torch.cuda.Event()
+                arrived.record(copy)
+            meta["ahead"] = (dev, arrived)
+
+    def fetch(self, host):
+        meta = getattr(host, "_actnn_swap", None)
+        if meta is None:                                           # not parked by this class
+            return host.cuda(non_blocking=True)
+        compute = torch.cuda.current_stream(meta["device"])
+        self._start(host)
+        dev, arrived = meta["ahead"]
+        compute.wait_event(arrived)
+        dev.record_stream(compute)
+        # the backward pass walks the parked tensors last-in first-out: get the next ones moving
+        i = next((k for k in range(len(self.parked) - 1, -1, -1) if self.parked[k]() is host), None)
+        if i is not None:
+            del self.parked[i:]                                    # later ones have been consumed or dropped
+            for ref in self.parked[max(0, i - self.depth):i]:
+                prev = ref()
+                if prev is not None:
+                    self._start(prev)
+        return dev
+
+    def reset(self):
+        self.parked.clear()
+
+
+swap_space = _SwapSpace()
+
+
 def swap_to_cpu(tensor):
-    """Asynchronous copy into freshly allocated pinned host memory (utils.py:10-13)."""
-    host = torch.empty(tensor.shape, dtype=tensor.dtype, device="cpu", pin_memory=True)
-    host.copy_(tensor, non_blocking=True)
-    return host
+    """Park a device tensor in pinned host memory (utils.py:10-13); asynchronous, on the copy stream."""
+    return swap_space.park(tensor)
+
+
+def swap_to_device(host):
+    """The device copy of a parked tensor, ordered after its transfer on the current stream."""
+    return swap_space.fetch(host)
 
 
 def channels_last_format(t):

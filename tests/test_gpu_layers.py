@@ -417,3 +417,25 @@ def test_qmodule_channels_last_option():
     assert y.is_contiguous(memory_format=torch.channels_last)
     y.sum().backward()
     assert x.grad.shape == x.shape and torch.isfinite(x.grad).all()
+
+
+def test_swap_space_round_trip_and_prefetch():
+    """Tensors parked on the host come back bit-identical in last-in first-out order (the order of
+    the backward pass), whether they were transferred ahead of time or on demand."""
+    from actnn_amd.utils import swap_space, swap_to_cpu, swap_to_device
+    swap_space.reset()
+    g = torch.Generator(device=DEV).manual_seed(0)
+    originals = [torch.randint(-2 ** 31, 2 ** 31 - 1, (1 << (12 + i % 5),), generator=g, device=DEV, dtype=torch.int64).int()
+                 for i in range(12)]
+    hosts = [swap_to_cpu(t) for t in originals]
+    assert all(h.device.type == "cpu" and h.is_pinned() for h in hosts)
+    for k in range(11, -1, -1):
+        back = swap_to_device(hosts[k])
+        assert back.is_cuda and torch.equal(back, originals[k])
+        if k >= 1:
+            assert hosts[k - 1]._actnn_swap["ahead"] is not None          # already on its way
+    assert swap_space.parked == []
+    # on demand, out of order
+    hosts = [swap_to_cpu(t) for t in originals[:4]]
+    for k in (2, 0, 3, 1):
+        assert torch.equal(swap_to_device(hosts[k]), originals[k])
