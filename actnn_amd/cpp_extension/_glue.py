@@ -37,7 +37,35 @@ def check_typed(t, name, dtype, dim=None):
 
 
 def stream_ptr(device):
-    return torch.cuda.current_stream(device).cuda_stream
+    """The current HIP stream of `device` as an integer (one C call; the Stream object that
+    torch.cuda.current_stream builds costs several microseconds per kernel launch)."""
+    index = device.index
+    if index is None:
+        index = torch.cuda.current_device()
+    return torch._C._cuda_getCurrentRawStream(index)
+
+
+class on_device:
+    """`with on_device(t.device):` - makes the tensor's device current for the launch, like
+    torch.cuda.device, but does nothing at all in the usual case that it already is."""
+    __slots__ = ("index", "previous")
+
+    def __init__(self, device):
+        self.index = device.index
+        self.previous = -1
+
+    def __enter__(self):
+        if self.index is not None:
+            current = torch._C._cuda_getDevice()
+            if current != self.index:
+                self.previous = current
+                torch.cuda.set_device(self.index)
+        return self
+
+    def __exit__(self, *exc):
+        if self.previous >= 0:
+            torch.cuda.set_device(self.previous)
+        return False
 
 
 def aligned(t):

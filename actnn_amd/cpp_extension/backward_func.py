@@ -6,6 +6,8 @@ ATen's miopen_batch_norm otherwise.
 
 The three layer-norm exports of the reference have no Python caller and are not provided.
 """
+import functools
+
 import torch
 
 from . import _glue
@@ -16,16 +18,26 @@ _aten = torch.ops.aten
 
 def _shape_geometry(shape, dtype, channels_last):
     """(N, C, HW) when the library's batch-norm kernels take a tensor of this shape, else None."""
+    return _geometry_of(tuple(int(d) for d in shape), dtype, bool(channels_last))
+
+
+@functools.lru_cache(maxsize=4096)
+def _geometry_of(shape, dtype, channels_last):
+    # asked several times per layer and step with the same few shapes: remembered
     if len(shape) < 2 or dtype not in _glue.DTYPE_CODE:
         return None
-    N, C = int(shape[0]), int(shape[1])
+    N, C = shape[0], shape[1]
     HW = 1
     for d in shape[2:]:
-        HW *= int(d)
-    if N * C * HW == 0 or _glue.lib().actnn_batch_norm_workspace_bytes(
-            N, C, HW, _glue.DTYPE_CODE[dtype], int(channels_last)) < 0:
+        HW *= d
+    if N * C * HW == 0 or _workspace_bytes(N, C, HW, _glue.DTYPE_CODE[dtype], int(channels_last)) < 0:
         return None
     return N, C, HW
+
+
+@functools.lru_cache(maxsize=4096)
+def _workspace_bytes(N, C, HW, code, channels_last):
+    return _glue.lib().actnn_batch_norm_workspace_bytes(N, C, HW, code, channels_last)
 
 
 def _bn_geometry(input):
@@ -72,7 +84,7 @@ def hip_batch_norm_forward(input, weight, bias, running_mean, running_var, momen
     N, C, HW, channels_last = _bn_geometry(input)
     lib = _glue.lib()
     code = _glue.DTYPE_CODE[input.dtype]
-    ws_bytes = lib.actnn_batch_norm_workspace_bytes(N, C, HW, code, int(channels_last))
+    ws_bytes = _workspace_bytes(N, C, HW, code, int(channels_last))
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=input.device)
     out = torch.empty_like(input)                       # same strides as the input
     save_mean = torch.empty(C, dtype=torch.float32, device=input.device)
@@ -82,7 +94,7 @@ def hip_batch_norm_forward(input, weight, bias, running_mean, running_var, momen
         groups = N * C * HW // 256
         mn = torch.empty(groups, dtype=input.dtype, device=input.device)
         mx = torch.empty(groups, dtype=input.dtype, device=input.device)
-    with torch.cuda.device(input.device):
+    with _glue.on_device(input.device):
         _glue._lib.check(lib.actnn_batch_norm_forward(
             input.data_ptr(), _ptr(weight), _ptr(bias), _ptr(running_mean), _ptr(running_var),
             out.data_ptr(), save_mean.data_ptr(), save_invstd.data_ptr(), _ptr(mn), _ptr(mx),
@@ -97,7 +109,7 @@ def hip_batch_norm_forward_stats(input, weight, bias, running_mean, running_var,
     N, C, HW, channels_last = _bn_geometry(input)
     lib = _glue.lib()
     code = _glue.DTYPE_CODE[input.dtype]
-    ws_bytes = lib.actnn_batch_norm_workspace_bytes(N, C, HW, code, int(channels_last))
+    ws_bytes = _workspace_bytes(N, C, HW, code, int(channels_last))
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=input.device)
     save_mean = torch.empty(C, dtype=torch.float32, device=input.device)
     save_invstd = torch.empty(C, dtype=torch.float32, device=input.device)
@@ -106,7 +118,7 @@ def hip_batch_norm_forward_stats(input, weight, bias, running_mean, running_var,
         groups = N * C * HW // 256
         mn = torch.empty(groups, dtype=input.dtype, device=input.device)
         mx = torch.empty(groups, dtype=input.dtype, device=input.device)
-    with torch.cuda.device(input.device):
+    with _glue.on_device(input.device):
         _glue._lib.check(lib.actnn_batch_norm_forward_stats(
             input.data_ptr(), _ptr(weight), _ptr(bias), _ptr(running_mean), _ptr(running_var),
             save_mean.data_ptr(), save_invstd.data_ptr(), _ptr(mn), _ptr(mx), ws.data_ptr(), ws_bytes,
@@ -132,7 +144,7 @@ def hip_batch_norm_forward_apply(input, workspace, bits=None, mn=None, mx=None):
         packed = torch.empty(total * G * 8, dtype=torch.int32, device=input.device)
         scale = torch.empty(N, G, 1, dtype=input.dtype, device=input.device)
         seed, offset = _glue.philox_args(input.device)
-    with torch.cuda.device(input.device):
+    with _glue.on_device(input.device):
         _glue._lib.check(lib.actnn_batch_norm_forward_apply(
             input.data_ptr(), out.data_ptr(), workspace.data_ptr(), workspace.numel() * 4, _ptr(bits),
             _ptr(prefix), _ptr(mn), _ptr(mx), _ptr(scale), _ptr(packed), seed, offset, N, C, HW, code,
@@ -156,12 +168,12 @@ def hip_batch_norm_backward(input, grad_output, weight, save_mean, save_invstd):
     N, C, HW, channels_last = _bn_geometry(input)
     lib = _glue.lib()
     code = _glue.DTYPE_CODE[input.dtype]
-    ws_bytes = lib.actnn_batch_norm_workspace_bytes(N, C, HW, code, int(channels_last))
+    ws_bytes = _workspace_bytes(N, C, HW, code, int(channels_last))
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=input.device)
     grad_input = torch.empty_like(input)
     grad_weight = torch.empty(C, dtype=torch.float32, device=input.device)
     grad_bias = torch.empty(C, dtype=torch.float32, device=input.device)
-    with torch.cuda.device(input.device):
+    with _glue.on_device(input.device):
         _glue._lib.check(lib.actnn_batch_norm_backward(
             input.data_ptr(), grad_output.data_ptr(), _ptr(weight), save_mean.data_ptr(),
             save_invstd.data_ptr(), grad_input.data_ptr(), grad_weight.data_ptr(), grad_bias.data_ptr(),
@@ -202,13 +214,13 @@ def hip_batch_norm_backward_packed(shape, quantized, grad_output, weight, save_m
     total, prefix = _bits_info(q_bits)
     if q_input.numel() < total * (C * HW // 256) * 8:
         raise RuntimeError("batch_norm_backward_packed: packed stream is too short")
-    ws_bytes = lib.actnn_batch_norm_workspace_bytes(N, C, HW, code, int(channels_last))
+    ws_bytes = _workspace_bytes(N, C, HW, code, int(channels_last))
     dev = grad_output.device
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dev)
     grad_input = torch.empty_like(grad_output)
     grad_weight = torch.empty(C, dtype=torch.float32, device=dev)
     grad_bias = torch.empty(C, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _glue.on_device(dev):
         _glue._lib.check(lib.actnn_batch_norm_backward_packed(
             q_input.data_ptr(), q_bits.data_ptr(), prefix.data_ptr(), q_scale.data_ptr(), q_min.data_ptr(),
             grad_output.data_ptr(), _ptr(weight), save_mean.data_ptr(), save_invstd.data_ptr(),

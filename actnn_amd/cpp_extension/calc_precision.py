@@ -42,7 +42,7 @@ def calc_precision_device(C, initial_bits, target):
                            % DEVICE_MAX_CANDIDATES)
     C = C.contiguous()
     bits = torch.empty(N, dtype=torch.int32, device=C.device)
-    with torch.cuda.device(C.device):
+    with g.on_device(C.device):
         check(g.lib().actnn_calc_precision_device(C.data_ptr(), bits.data_ptr(), N, int(initial_bits),
                                                   int(target), g.stream_ptr(C.device)), "calc_precision_device")
     return bits

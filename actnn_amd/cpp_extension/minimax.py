@@ -14,7 +14,7 @@ def minimax(data):
     M, D = data.shape
     mn = torch.empty(M, dtype=data.dtype, device=data.device)
     mx = torch.empty(M, dtype=data.dtype, device=data.device)
-    with torch.cuda.device(data.device):
+    with g.on_device(data.device):
         check(g.lib().actnn_minimax(data.data_ptr(), mn.data_ptr(), mx.data_ptr(), M, D,
                                     g.DTYPE_CODE[data.dtype], g.stream_ptr(data.device)), "minimax")
     return mn, mx
@@ -37,7 +37,7 @@ def range_sqr(mn, mx, N, factor=1.0, mult=None):
             raise RuntimeError("range_sqr: mult must be fp32 on the same device with 1 or N values")
         mult = mult.contiguous()
         mult_ptr, per_sample = mult.data_ptr(), int(mult.numel() == N and N != 1)
-    with torch.cuda.device(mn.device):
+    with g.on_device(mn.device):
         check(g.lib().actnn_range_sqr(mn.data_ptr(), mx.data_ptr(), out.data_ptr(), N, G, float(factor),
                                       mult_ptr, per_sample, g.DTYPE_CODE[mn.dtype], g.stream_ptr(mn.device)),
               "range_sqr")
@@ -56,7 +56,7 @@ def sample_sqnorm(x):
         return torch.linalg.vector_norm(x.reshape(N, -1), dim=1, dtype=torch.float32).square()
     slices = max(1, min(64, F // 8192))
     part = torch.empty(N, slices, dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with g.on_device(x.device):
         check(g.lib().actnn_sample_sqnorm(x.data_ptr(), part.data_ptr(), N, F, slices,
                                           g.DTYPE_CODE[x.dtype], g.stream_ptr(x.device)), "sample_sqnorm")
     return part.sum(1) if slices > 1 else part.view(N)

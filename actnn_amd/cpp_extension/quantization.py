@@ -45,7 +45,7 @@ def _bits_info(bits):
         total = int(host.sum())
     N = bits.numel()
     prefix = torch.empty(N + 1, dtype=torch.int32, device=bits.device)
-    with torch.cuda.device(bits.device):
+    with g.on_device(bits.device):
         check(g.lib().actnn_bits_prefix(bits.data_ptr(), prefix.data_ptr(), N,
                                         g.stream_ptr(bits.device)), "bits_prefix")
     bits._actnn_info = (total, prefix)
@@ -80,7 +80,7 @@ def pack_mixed_precision(data, min, max, bits, stochastic, *, noise=None):
     packed = torch.empty(n_words, dtype=torch.int32, device=data.device)
     scale = torch.empty(N, G, 1, dtype=data.dtype, device=data.device)
     seed, offset = (0, 0) if noise is not None else g.philox_args(data.device)
-    with torch.cuda.device(data.device):
+    with g.on_device(data.device):
         check(g.lib().actnn_pack_mixed(
             data.data_ptr(), min.data_ptr(), max.data_ptr(), bits.data_ptr(), prefix.data_ptr(),
             scale.data_ptr(), packed.data_ptr(), noise.data_ptr() if noise is not None else None,
@@ -104,7 +104,7 @@ def unpack_mixed_precision(data, bits, scale, min, N, num_groups, group_size):
     if data.numel() < (total * num_groups * group_size + 31) // 32:
         raise RuntimeError("unpack_mixed_precision: packed stream is too short")
     out = torch.empty(N, num_groups, group_size, dtype=scale.dtype, device=data.device)
-    with torch.cuda.device(data.device):
+    with g.on_device(data.device):
         check(g.lib().actnn_unpack_mixed(
             data.data_ptr(), bits.data_ptr(), prefix.data_ptr(), scale.data_ptr(), min.data_ptr(),
             out.data_ptr(), N, num_groups, group_size, g.DTYPE_CODE[scale.dtype],
@@ -147,7 +147,7 @@ def pack_single_precision(data, min, max, bits, stochastic, *, noise=None):
     scale = torch.empty(N, G, 1, dtype=data.dtype, device=data.device)
     wpt = 8 // bits
     seed, offset = (0, 0) if noise is not None else g.philox_args(data.device)
-    with torch.cuda.device(data.device):
+    with g.on_device(data.device):
         check(g.lib().actnn_pack_single(
             data.data_ptr(), min.data_ptr(), max.data_ptr(), bits, scale.data_ptr(),
             packed.data_ptr(), noise.data_ptr() if noise is not None else None, seed, offset,
@@ -170,7 +170,7 @@ def unpack_single_precision(data, bits, scale, min, N, num_groups, group_size):
     if data.numel() < single_packed_bytes(N, num_groups, group_size, bits) - 1:
         raise RuntimeError("unpack_single_precision: packed stream is too short")
     out = torch.empty(N, num_groups, group_size, dtype=scale.dtype, device=data.device)
-    with torch.cuda.device(data.device):
+    with g.on_device(data.device):
         check(g.lib().actnn_unpack_single(
             data.data_ptr(), bits, scale.data_ptr(), min.data_ptr(), out.data_ptr(), N, num_groups,
             group_size, g.DTYPE_CODE[scale.dtype], g.stream_ptr(data.device)),
@@ -203,7 +203,7 @@ def linear_grad_weight_q2(grad_output, packed, scale, min, in_features, out_dtyp
         raise RuntimeError("linear_grad_weight_q2: packed stream is too short")
     out_dtype = out_dtype or grad_output.dtype
     gw = torch.empty(O, I, dtype=out_dtype, device=grad_output.device)
-    with torch.cuda.device(gw.device):
+    with g.on_device(gw.device):
         check(g.lib().actnn_linear_grad_weight_q2(
             grad_output.data_ptr(), packed.data_ptr(), scale.data_ptr(), min.data_ptr(), gw.data_ptr(),
             M, O, I, g.DTYPE_CODE[grad_output.dtype], g.DTYPE_CODE[scale.dtype], g.DTYPE_CODE[out_dtype],
@@ -226,7 +226,7 @@ def relu_forward(x):
     n = x.numel()
     y = torch.empty_like(x)
     mask = torch.empty(mask_words(n), dtype=torch.int32, device=x.device)
-    with torch.cuda.device(x.device):
+    with g.on_device(x.device):
         check(g.lib().actnn_relu_forward(x.data_ptr(), y.data_ptr(), mask.data_ptr(), n,
                                          g.DTYPE_CODE[x.dtype], g.stream_ptr(x.device)), "relu_forward")
     return y, mask
@@ -235,7 +235,7 @@ def relu_forward(x):
 def relu_backward(grad_output, mask):
     grad_output = g.aligned(grad_output.contiguous())
     gin = torch.empty_like(grad_output)
-    with torch.cuda.device(gin.device):
+    with g.on_device(gin.device):
         check(g.lib().actnn_relu_backward(grad_output.data_ptr(), mask.data_ptr(), gin.data_ptr(),
                                           gin.numel(), g.DTYPE_CODE[gin.dtype],
                                           g.stream_ptr(gin.device)), "relu_backward")
@@ -268,7 +268,7 @@ def dropout_forward(x, p):
     y = torch.empty_like(x)
     mask = torch.empty(mask_words(n), dtype=torch.int32, device=x.device)
     seed, offset = g.philox_args(x.device)
-    with torch.cuda.device(x.device):
+    with g.on_device(x.device):
         check(g.lib().actnn_dropout_forward(x.data_ptr(), y.data_ptr(), mask.data_ptr(), n, float(p),
                                             seed, offset, g.DTYPE_CODE[x.dtype],
                                             g.stream_ptr(x.device)), "dropout_forward")
@@ -278,7 +278,7 @@ def dropout_forward(x, p):
 def dropout_backward(grad_output, mask, p):
     grad_output = g.aligned(grad_output.contiguous())
     gin = torch.empty_like(grad_output)
-    with torch.cuda.device(gin.device):
+    with g.on_device(gin.device):
         check(g.lib().actnn_dropout_backward(grad_output.data_ptr(), mask.data_ptr(), gin.data_ptr(),
                                              gin.numel(), float(p), g.DTYPE_CODE[gin.dtype],
                                              g.stream_ptr(gin.device)), "dropout_backward")
@@ -335,7 +335,7 @@ def max_pool2d_forward(x, kernel_size, stride, padding, dilation):
     y = torch.empty((N, C, Ho, Wo), dtype=x.dtype, device=x.device, memory_format=fmt)
     idx = torch.empty((N, C, Ho, Wo), dtype=torch.int8, device=x.device, memory_format=fmt)
     fn = g.lib().actnn_max_pool2d_forward_cl if channels_last else g.lib().actnn_max_pool2d_forward
-    with torch.cuda.device(x.device):
+    with g.on_device(x.device):
         check(fn(
             x.data_ptr(), y.data_ptr(), idx.data_ptr(), N, C, H, W, Ho, Wo, KH, KW, stride[0],
             stride[1], padding[0], padding[1], g.DTYPE_CODE[x.dtype], g.stream_ptr(x.device)),
@@ -352,7 +352,7 @@ def max_pool2d_backward(grad_output, idx, input_shape, kernel_size, stride, padd
     Ho, Wo = grad_output.shape[2], grad_output.shape[3]
     gin = torch.empty((N, C, H, W), dtype=grad_output.dtype, device=grad_output.device, memory_format=fmt)
     fn = g.lib().actnn_max_pool2d_backward_cl if channels_last else g.lib().actnn_max_pool2d_backward
-    with torch.cuda.device(gin.device):
+    with g.on_device(gin.device):
         check(fn(
             grad_output.data_ptr(), idx.data_ptr(), gin.data_ptr(), N, C, H, W, Ho, Wo,
             kernel_size[0], kernel_size[1], stride[0], stride[1], padding[0], padding[1],
