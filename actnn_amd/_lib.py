@@ -30,6 +30,8 @@ SIGNATURES = {
     "actnn_calc_precision_device": [c_vp, c_vp, c_i64, c_i32, c_i64, c_vp],
     "actnn_range_sqr": [c_vp, c_vp, c_vp, c_i64, c_i64, ctypes.c_float, c_vp, c_i32, c_i32, c_vp],
     "actnn_sample_sqnorm": [c_vp, c_vp, c_i64, c_i64, c_i32, c_i32, c_vp],
+    "actnn_allocate_bits_device": [c_vp, c_vp, ctypes.c_float, c_vp, c_i32, c_vp, c_vp, c_vp, c_i64, c_i64, c_i32,
+                                   c_i64, c_i32, c_vp],
     "actnn_bits_prefix": [c_vp, c_vp, c_i64, c_vp],
     "actnn_pack_mixed": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u64, c_u64,
                          c_i64, c_i64, c_i64, c_i32, c_vp],

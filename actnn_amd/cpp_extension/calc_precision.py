@@ -46,3 +46,25 @@ def calc_precision_device(C, initial_bits, target):
         check(g.lib().actnn_calc_precision_device(C.data_ptr(), bits.data_ptr(), N, int(initial_bits),
                                                   int(target), g.stream_ptr(C.device)), "calc_precision_device")
     return bits
+
+
+def allocate_bits_device(mn, mx, N, factor, mult, initial_bits, target):
+    """-> (sensitivity fp32 [N], bits int32 [N], prefix int32 [N + 1]) on the device of mn:
+    ``range_sqr`` -> ``calc_precision_device`` -> exclusive prefix of the widths, in one call."""
+    G = mn.numel() // N
+    dev = mn.device
+    sens = torch.empty(N, dtype=torch.float32, device=dev)
+    bits = torch.empty(N, dtype=torch.int32, device=dev)
+    prefix = torch.empty(N + 1, dtype=torch.int32, device=dev)
+    mult_ptr, per_sample = None, 0
+    if mult is not None:
+        if mult.dtype != torch.float32 or mult.device != dev or mult.numel() not in (1, N):
+            raise RuntimeError("allocate_bits_device: mult must be fp32 on the same device with 1 or N values")
+        mult = mult.contiguous()
+        mult_ptr, per_sample = mult.data_ptr(), int(mult.numel() == N and N != 1)
+    with g.on_device(dev):
+        check(g.lib().actnn_allocate_bits_device(
+            mn.data_ptr(), mx.data_ptr(), float(factor), mult_ptr, per_sample, sens.data_ptr(), bits.data_ptr(),
+            prefix.data_ptr(), N, G, int(initial_bits), int(target), g.DTYPE_CODE[mn.dtype], g.stream_ptr(dev)),
+            "allocate_bits_device")
+    return sens, bits, prefix

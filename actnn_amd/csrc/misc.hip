@@ -35,6 +35,25 @@ extern "C" int actnn_stream_copy(const void* src, void* dst, int64_t bytes, void
   ACTNN_RETURN_LAUNCH_STATUS();
 }
 
+// The three allocation steps of a layer in one call (one crossing of the language boundary instead
+// of three): sensitivities, greedy widths on the device, exclusive prefix of the widths.
+extern "C" int actnn_range_sqr(const void* mn, const void* mx, float* out, int64_t N, int64_t G, float factor,
+                               const float* mult, int mult_per_sample, int dtype, void* stream);
+extern "C" int actnn_calc_precision_device(const float* C, int32_t* bits, int64_t N, int initial_bits,
+                                           int64_t target, void* stream);
+extern "C" int actnn_bits_prefix(const int32_t* bits, int32_t* prefix, int64_t N, void* stream);
+
+extern "C" int actnn_allocate_bits_device(const void* mn, const void* mx, float factor, const float* mult,
+                                          int mult_per_sample, float* sensitivity, int32_t* bits,
+                                          int32_t* prefix, int64_t N, int64_t G, int initial_bits,
+                                          int64_t target, int dtype, void* stream) {
+  int rc = actnn_range_sqr(mn, mx, sensitivity, N, G, factor, mult, mult_per_sample, dtype, stream);
+  if (rc != ACTNN_OK) return rc;
+  rc = actnn_calc_precision_device(sensitivity, bits, N, initial_bits, target, stream);
+  if (rc != ACTNN_OK) return rc;
+  return actnn_bits_prefix(bits, prefix, N, stream);
+}
+
 extern "C" const char* actnn_strerror(int code) {
   switch (code) {
     case ACTNN_OK: return "success";

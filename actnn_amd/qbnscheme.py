@@ -3,7 +3,7 @@ sensitivity is the range term alone and the per-layer budget follows the precedi
 import torch
 
 from .conf import config
-from .qscheme import (PendingBits, QScheme, allocate_on_device, greedy_bits, greedy_bits_device,
+from .qscheme import (PendingBits, QScheme, allocate_bits_on_device, allocate_on_device, greedy_bits,
                       group_min_max, range_sqr)
 
 
@@ -20,9 +20,10 @@ class QBNScheme(QScheme):
         self.prev_linear = QScheme.prev_layer
         N = input.shape[0]
         groups, mn, mx, num_pixels = group_min_max(input, known_minmax)
+        if allocate_on_device(N, self.initial_bits) and mn.is_contiguous() and mx.is_contiguous():
+            _, bits_dev = allocate_bits_on_device(mn, mx, N, num_pixels, 1.0, None, self.initial_bits, self.bits)
+            return groups, mn, mx, None, input.numel() // N, bits_dev
         C_dev = range_sqr(mn, mx, N, num_pixels)                           # qbnscheme.py:44-47
-        if allocate_on_device(N, self.initial_bits):
-            return groups, mn, mx, None, input.numel() // N, greedy_bits_device(C_dev, N, self.initial_bits, self.bits)
         return groups, mn, mx, PendingBits(C_dev), input.numel() // N, None
 
     def finish_quantization_bits(self, started):

@@ -82,6 +82,19 @@ def greedy_bits_device(C_dev, N, initial_bits, avg_bits):
     return attach_bits_total(bits, N * initial - taken)
 
 
+def allocate_bits_on_device(mn, mx, N, num_pixels, factor, mult, initial_bits, avg_bits):
+    """Sensitivities, widths and the prefix of the widths in one call -> (C on the device, bits
+    with their sum and prefix attached)."""
+    initial = int(initial_bits)
+    target = int(avg_bits * N)
+    C_dev, bits, prefix = ext_calc_precision.allocate_bits_device(
+        mn, mx, N, factor * config.group_size / num_pixels, mult, initial, target)
+    taken = min(max(N * initial - target, 0), N * (initial - 1))
+    bits = attach_bits_total(bits, N * initial - taken)
+    bits._actnn_info = (bits._actnn_total, prefix)
+    return C_dev, bits
+
+
 def allocate_on_device(N, initial_bits):
     return config.device_allocation and ext_calc_precision.device_allocation_fits(N, initial_bits)
 
@@ -176,10 +189,14 @@ class QScheme(_LazyHost):
         QScheme.prev_layer = self
         N = input.shape[0]
         groups, mn, mx, num_pixels = group_min_max(input, known_minmax)
-        C_dev = self.sensitivity(mn, mx, N, num_pixels)
         bits_dev = None
-        if allocate_on_device(N, self.initial_bits):
-            bits_dev = greedy_bits_device(C_dev, N, self.initial_bits, self.bits)
+        if allocate_on_device(N, self.initial_bits) and mn.is_contiguous() and mx.is_contiguous():
+            grad_sum = self.get_scale().to(device=mn.device, dtype=torch.float32)
+            C_dev, bits_dev = allocate_bits_on_device(
+                mn, mx, N, num_pixels, self.num_locations / 4 / self.depthwise_groups, grad_sum,
+                self.initial_bits, self.bits)
+        else:
+            C_dev = self.sensitivity(mn, mx, N, num_pixels)
         pending = PendingBits(C_dev)
         return groups, mn, mx, pending, input.numel() // N, bits_dev
 

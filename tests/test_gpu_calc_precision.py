@@ -59,3 +59,21 @@ def test_device_allocation_rejects_what_does_not_fit():
     with pytest.raises(RuntimeError):
         ext_cp.calc_precision_device(torch.rand(8), 8, 16)                        # host tensor
     assert ext_cp.calc_precision_device(torch.rand(0, device=DEV), 8, 0).numel() == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("N,G", [(512, 49), (37, 3136), (8, 1)])
+def test_allocation_in_one_call_equals_the_three_calls(N, G, dtype):
+    import actnn_amd.cpp_extension.minimax as ext_minimax
+    from actnn_amd.cpp_extension.quantization import _bits_info
+    g = torch.Generator(device=DEV).manual_seed(N + G)
+    mn = -torch.rand(N * G, generator=g, device=DEV).to(dtype)
+    mx = (torch.rand(N * G, generator=g, device=DEV) * torch.exp(torch.randn(N, 1, generator=g, device=DEV)).expand(N, G).reshape(-1)).to(dtype)
+    mult = torch.rand(N, generator=g, device=DEV) + 0.5
+    for m in (None, mult, mult[:1].reshape(())):
+        sens, bits, prefix = ext_cp.allocate_bits_device(mn, mx, N, 0.37, m, 8, 2 * N)
+        sens_ref = ext_minimax.range_sqr(mn, mx, N, 0.37, m)
+        bits_ref = ext_cp.calc_precision_device(sens_ref, 8, 2 * N)
+        assert torch.equal(sens, sens_ref) and torch.equal(bits, bits_ref)
+        assert torch.equal(prefix, _bits_info(bits_ref)[1])
+        assert int(prefix[-1]) == int(bits.sum()) == 2 * N
