@@ -232,6 +232,26 @@ def relu_forward(x):
     return y, mask
 
 
+def relu_forward_minmax(x):
+    """-> (y, mask, mn, mx): ReLU whose pass also yields the min / max of every group of 256
+    consecutive outputs (16-bit tensors of whole 2048-element tiles)."""
+    n = x.numel()
+    y = torch.empty_like(x)
+    mask = torch.empty(mask_words(n), dtype=torch.int32, device=x.device)
+    mn = torch.empty(n // 256, dtype=x.dtype, device=x.device)
+    mx = torch.empty(n // 256, dtype=x.dtype, device=x.device)
+    with g.on_device(x.device):
+        check(g.lib().actnn_relu_forward_minmax(x.data_ptr(), y.data_ptr(), mask.data_ptr(), mn.data_ptr(),
+                                                mx.data_ptr(), n, g.DTYPE_CODE[x.dtype],
+                                                g.stream_ptr(x.device)), "relu_forward_minmax")
+    return y, mask, mn, mx
+
+
+def relu_minmax_applies(x):
+    return (x.is_cuda and x.dtype in (torch.float16, torch.bfloat16) and x.is_contiguous()
+            and x.numel() > 0 and x.numel() % 2048 == 0 and x.data_ptr() % 16 == 0)
+
+
 def relu_backward(grad_output, mask):
     grad_output = g.aligned(grad_output.contiguous())
     gin = torch.empty_like(grad_output)
@@ -253,6 +273,23 @@ class ActQuantizedReLU(Function):
 
     @staticmethod
     def backward(ctx, grad_output):
+        (mask,) = ctx.saved_tensors
+        return relu_backward(grad_output, mask)
+
+
+class ActQuantizedReLUMinMax(Function):
+    """The same operator, additionally returning the group min / max of its output (not
+    differentiable) for the layer that compresses this output next."""
+
+    @staticmethod
+    def forward(ctx, input):
+        output, mask, mn, mx = relu_forward_minmax(input)
+        ctx.save_for_backward(mask)
+        ctx.mark_non_differentiable(mn, mx)
+        return output, mn, mx
+
+    @staticmethod
+    def backward(ctx, grad_output, _grad_mn, _grad_mx):
         (mask,) = ctx.saved_tensors
         return relu_backward(grad_output, mask)
 

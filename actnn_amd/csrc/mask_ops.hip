@@ -148,11 +148,16 @@ ACTNN_DEV void word_to_rows(uint32_t w, uint32_t lane, uint32_t (&m)[4]) {
   m[3] = (cd >> (16 + sh)) & 0xffu;
 }
 
-template <typename T, Op OP>
+// MINMAX: also write the minimum and maximum of every group of 256 consecutive outputs (the lower
+// and upper 32 lanes of each load own one group each) - what actnn_minimax returns for the output
+// viewed as rows of 256, for a consumer that quantises it next.
+template <typename T, Op OP, bool MINMAX = false>
 __global__ __launch_bounds__(kThreads) void mask_forward16_kernel(const T* __restrict__ x, T* __restrict__ y,
                                                                   int32_t* __restrict__ mask, int64_t tiles,
                                                                   uint32_t thr, float keep_div,
-                                                                  uint64_t seed, uint64_t offset) {
+                                                                  uint64_t seed, uint64_t offset,
+                                                                  T* __restrict__ mn = nullptr,
+                                                                  T* __restrict__ mx = nullptr) {
   const uint32_t lane = threadIdx.x & 63;
   const int64_t tile = (int64_t)blockIdx.x * kTilesPerBlock + (threadIdx.x >> 6);
   if (tile >= tiles) return;                       // whole waves leave together
@@ -175,6 +180,21 @@ __global__ __launch_bounds__(kThreads) void mask_forward16_kernel(const T* __res
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) store8_nt(y + e0 + i * kMaskBlock, v[i]);
+  if (MINMAX) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float lo = v[i][0], hi = v[i][0];
+#pragma unroll
+      for (int k = 1; k < 8; ++k) { lo = fminf(lo, v[i][k]); hi = fmaxf(hi, v[i][k]); }
+      lo = rows_min<2>(row16_min(lo));
+      hi = rows_max<2>(row16_max(hi));
+      if ((lane & 31u) == 31u) {
+        const int64_t g = tile * (kTileElems / 256) + i * (kMaskBlock / 256) + (lane >> 5);
+        Conv<T>::store(mn, g, lo);
+        Conv<T>::store(mx, g, hi);
+      }
+    }
+  }
   const uint32_t w = rows_to_word(m, lane);
   // lane 2p+h holds word p % 16 of block 2h + p / 16
   mask[tile * 64 + (lane & 1u) * 32 + (lane >> 1)] = (int32_t)w;
@@ -301,6 +321,30 @@ inline uint32_t dropout_threshold(float p) {
 extern "C" int actnn_relu_forward(const void* x, void* y, int32_t* mask, int64_t n, int dtype,
                                   void* stream) {
   return actnn::dispatch_forward<actnn::Op::kRelu>(x, y, mask, n, 0u, 1.0f, 0, 0, dtype, stream);
+}
+
+extern "C" int actnn_relu_forward_minmax(const void* x, void* y, int32_t* mask, void* mn, void* mx,
+                                         int64_t n, int dtype, void* stream) {
+  using namespace actnn;
+  if (n < 0 || n % kTileElems != 0) return ACTNN_EINVAL;       // whole tiles of 2048 elements only
+  if (dtype != ACTNN_F16 && dtype != ACTNN_BF16) return ACTNN_EDTYPE;
+  if (n == 0) return ACTNN_OK;
+  if (!x || !y || !mask || !mn || !mx) return ACTNN_EINVAL;
+  if (!aligned16(x) || !aligned16(y)) return ACTNN_EALIGN;
+  const int64_t tiles = n / kTileElems;
+  const int64_t blocks = (tiles + kTilesPerBlock - 1) / kTilesPerBlock;
+  if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)blocks), blk(kThreads);
+  if (dtype == ACTNN_F16)
+    mask_forward16_kernel<__half, Op::kRelu, true><<<grid, blk, 0, s>>>(
+        static_cast<const __half*>(x), static_cast<__half*>(y), mask, tiles, 0u, 1.0f, 0, 0,
+        static_cast<__half*>(mn), static_cast<__half*>(mx));
+  else
+    mask_forward16_kernel<bf16_t, Op::kRelu, true><<<grid, blk, 0, s>>>(
+        static_cast<const bf16_t*>(x), static_cast<bf16_t*>(y), mask, tiles, 0u, 1.0f, 0, 0,
+        static_cast<bf16_t*>(mn), static_cast<bf16_t*>(mx));
+  ACTNN_RETURN_LAUNCH_STATUS();
 }
 
 extern "C" int actnn_relu_backward(const void* grad_out, const int32_t* mask, void* grad_in,

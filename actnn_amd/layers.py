@@ -34,6 +34,21 @@ def _autocast_apply(fn, *args):
     return fn.apply(*args)
 
 
+def _relu_shares_min_max(x):
+    return (config.share_relu_min_max and config.training and config.compress_activation and config.pergroup
+            and not config.simulate and config.group_size == 256 and x.dim() >= 2
+            and (x.numel() // max(x.shape[0], 1)) % 256 == 0 and ext_quantization.relu_minmax_applies(x))
+
+
+def known_group_minmax(input):
+    """(mn, mx) left on `input` by the layer that produced it, if they still describe it."""
+    known = getattr(input, "_actnn_group_minmax", None)
+    if known is None or known[2] != input._version or known[0].dtype != input.dtype \
+            or known[0].numel() * 256 != input.numel():
+        return None
+    return known[0], known[1]
+
+
 def _num_locations(kernel_size, dims):
     if isinstance(kernel_size, int):
         return kernel_size ** dims
@@ -65,7 +80,7 @@ class _QConvMixin:
         else:
             padding = self.padding
         return _autocast_apply(self._function, input, self.weight, self.bias, self.stride, padding,
-                               self.dilation, self.groups, self.scheme)
+                               self.dilation, self.groups, self.scheme, known_group_minmax(input))
 
 
 class QConv1d(_QConvMixin, nn.Conv1d):
@@ -212,9 +227,16 @@ class QReLU(nn.Module):
     def forward(self, input):
         # the mask follows memory order, so a channels-last activation needs no transposition
         fmt = channels_last_format(input)
-        if fmt is not None:
-            return logical_order(ext_quantization.act_quantized_relu(memory_order(input)), fmt)
-        return ext_quantization.act_quantized_relu(input)
+        x = memory_order(input) if fmt is not None else input
+        if _relu_shares_min_max(x):
+            # the layer that compresses this output next (a convolution) finds the group min / max
+            # on the tensor instead of reading it once more for them
+            out, mn, mx = ext_quantization.ActQuantizedReLUMinMax.apply(x)
+            out = logical_order(out, fmt) if fmt is not None else out
+            out._actnn_group_minmax = (mn, mx, out._version)
+            return out
+        out = ext_quantization.act_quantized_relu(x)
+        return logical_order(out, fmt) if fmt is not None else out
 
 
 class QDropout(nn.Dropout):

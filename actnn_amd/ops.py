@@ -156,10 +156,14 @@ bn_layer_ct = 0
 total_act_mem = 0
 
 
-def _conv_forward(ctx, forward_op, input, weight, bias, stride, padding, dilation, groups, scheme):
+def _conv_forward(ctx, forward_op, input, weight, bias, stride, padding, dilation, groups, scheme,
+                  known_minmax=None):
     # min/max and sensitivities first, then the convolution itself, then the allocation and
     # the pack: the convolution runs while the sensitivities travel to the host
-    started = start_quantize(input, scheme)
+    if known_minmax is not None and (known_minmax[0].dtype != input.dtype
+                                     or known_minmax[0].numel() * config.group_size != input.numel()):
+        known_minmax = None                  # e.g. the input was cast on its way here
+    started = start_quantize(input, scheme, known_minmax)
     output = forward_op(input, weight, bias, stride, padding, dilation, groups)
     quantized = finish_saved(started, input)
     ctx.scheme = scheme
@@ -209,13 +213,15 @@ def _conv_backward(ctx, grad_output, bias_reduce_dims, aug):
     grad_bias = grad_output.sum(bias_reduce_dims) if bias is not None and ctx.needs_input_grad[2] else None
     if ctx.scheme:
         ctx.scheme.if_allocate_perlayer()
-    return grad_input, grad_weight, grad_bias, None, None, None, None, None
+    return grad_input, grad_weight, grad_bias, None, None, None, None, None, None
 
 
 class conv1d(Function):
     @staticmethod
-    def forward(ctx, input, weight, bias=None, stride=1, padding=0, dilation=1, groups=1, scheme=None):
-        return _conv_forward(ctx, F.conv1d, input, weight, bias, stride, padding, dilation, groups, scheme)
+    def forward(ctx, input, weight, bias=None, stride=1, padding=0, dilation=1, groups=1, scheme=None,
+                known_minmax=None):
+        return _conv_forward(ctx, F.conv1d, input, weight, bias, stride, padding, dilation, groups, scheme,
+                             known_minmax)
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -224,8 +230,10 @@ class conv1d(Function):
 
 class conv2d(Function):
     @staticmethod
-    def forward(ctx, input, weight, bias=None, stride=1, padding=0, dilation=1, groups=1, scheme=None):
-        return _conv_forward(ctx, F.conv2d, input, weight, bias, stride, padding, dilation, groups, scheme)
+    def forward(ctx, input, weight, bias=None, stride=1, padding=0, dilation=1, groups=1, scheme=None,
+                known_minmax=None):
+        return _conv_forward(ctx, F.conv2d, input, weight, bias, stride, padding, dilation, groups, scheme,
+                             known_minmax)
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -234,8 +242,10 @@ class conv2d(Function):
 
 class conv3d(Function):
     @staticmethod
-    def forward(ctx, input, weight, bias=None, stride=1, padding=0, dilation=1, groups=1, scheme=None):
-        return _conv_forward(ctx, F.conv3d, input, weight, bias, stride, padding, dilation, groups, scheme)
+    def forward(ctx, input, weight, bias=None, stride=1, padding=0, dilation=1, groups=1, scheme=None,
+                known_minmax=None):
+        return _conv_forward(ctx, F.conv3d, input, weight, bias, stride, padding, dilation, groups, scheme,
+                             known_minmax)
 
     @staticmethod
     def backward(ctx, grad_output):

@@ -112,6 +112,12 @@ int actnn_unpack_single(const int8_t* packed, int bits, const void* scale, const
  * quantization_cuda_kernel.cu:446-467, :490-508 (quantization.cc:106-124).
  * ------------------------------------------------------------------------------- */
 int actnn_relu_forward(const void* x, void* y, int32_t* mask, int64_t n, int dtype, void* stream);
+/* ReLU forward that also writes the per-group minimum and maximum of its OUTPUT (groups of 256
+ * consecutive elements; mn/mx[n / 256] in `dtype`) - what actnn_minimax returns for y viewed as
+ * rows of 256 - so that a layer which quantises y next need not read it again.  16-bit dtypes,
+ * n a multiple of 2048. */
+int actnn_relu_forward_minmax(const void* x, void* y, int32_t* mask, void* mn, void* mx, int64_t n,
+                              int dtype, void* stream);
 int actnn_relu_backward(const void* grad_out, const int32_t* mask, void* grad_in, int64_t n,
                         int dtype, void* stream);
 

@@ -439,3 +439,37 @@ def test_swap_space_round_trip_and_prefetch():
     hosts = [swap_to_cpu(t) for t in originals[:4]]
     for k in (2, 0, 3, 1):
         assert torch.equal(swap_to_device(hosts[k]), originals[k])
+
+
+@pytest.mark.parametrize("channels_last", [False, True])
+def test_relu_hands_group_min_max_to_the_next_convolution(channels_last):
+    """QReLU -> QConv2d: with the hand-off the convolution saves the same stream, widths, scales
+    and minima as when it reduces its input itself; a tensor changed in place after the ReLU, or a
+    cast one, is not trusted."""
+    from actnn_amd.layers import known_group_minmax
+    def run(share):
+        config.reset(); QScheme.reset(); QBNScheme.reset()
+        config.share_relu_min_max = share
+        config.perlayer = False
+        torch.manual_seed(0)
+        relu, conv = actnn_amd.QReLU(), actnn_amd.QConv2d(64, 32, 3, padding=1).to(DEV)
+        x = torch.randn(16, 64, 16, 16, device=DEV).bfloat16()
+        if channels_last:
+            conv = conv.to(memory_format=torch.channels_last)
+            x = x.contiguous(memory_format=torch.channels_last)
+        x.requires_grad_(True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            h = relu(x)
+            assert (known_group_minmax(h) is not None) == share
+            torch.cuda.manual_seed(4)
+            y = conv(h)
+        saved = y.grad_fn.saved[0]
+        (gx,) = torch.autograd.grad(y, x, torch.ones_like(y))
+        return h, saved, gx
+    h0, s0, g0 = run(False)
+    h1, s1, g1 = run(True)
+    assert torch.equal(h0, h1) and torch.equal(g0, g1)
+    assert all(torch.equal(a, b) for a, b in zip(s0, s1))
+    h1.add_(1.0)
+    assert known_group_minmax(h1) is None                    # changed in place: the version moved on
+    assert known_group_minmax(h0.float()) is None

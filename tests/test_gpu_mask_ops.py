@@ -79,3 +79,22 @@ def test_dropout(dtype, p):
     g = torch.randn(n).to(dtype).to(DEV)
     y.backward(g)
     assert torch.equal(x.grad.cpu(), expect(g))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n", [2048, 2048 * 37, 8 * 64 * 56 * 56])
+def test_relu_forward_with_group_min_max(dtype, n):
+    """The ReLU pass that also reduces its output per group of 256: output and mask as the plain
+    operator, min / max bit-identical to minimax on the output."""
+    import actnn_amd.cpp_extension.minimax as ext_minimax
+    g = torch.Generator(device=DEV).manual_seed(n)
+    x = (torch.randn(n, generator=g, device=DEV) * 2 - 0.3).to(dtype)
+    x[:256] = -1.0                                                  # a group that is all zero after ReLU
+    x[256:512] = torch.linspace(0.5, 3, 256, device=DEV).to(dtype)     # a group without zeros
+    assert ext_q.relu_minmax_applies(x)
+    y0, mask0 = ext_q.relu_forward(x)
+    y, mask, mn, mx = ext_q.relu_forward_minmax(x)
+    assert torch.equal(y, y0) and torch.equal(mask, mask0)
+    mn_ref, mx_ref = ext_minimax.minimax(y.view(-1, 256))
+    assert torch.equal(mn, mn_ref) and torch.equal(mx, mx_ref)
+    assert not ext_q.relu_minmax_applies(x[:1024]) and not ext_q.relu_minmax_applies(x.float())
