@@ -169,9 +169,10 @@ def test_l3_first_step_uses_the_degenerate_allocation_then_rebalances():
     assert int(s0.b.sum()) <= int(budgets[0] * 16) and int(s0.b.min()) >= 1
 
 
-def test_small_model_trains_at_l3():
+@pytest.mark.parametrize("channels_last", [False, True])
+def test_small_model_trains_at_l3(channels_last):
     # the same toy problem with stock layers and with 2-bit compressed activations: the loss
-    # curves must track each other (the quantisation noise is unbiased)
+    # curves must track each other (the quantisation noise is unbiased), in both memory layouts
     def make():
         torch.manual_seed(0)
         return nn.Sequential(nn.Conv2d(3, 16, 3, padding=1), nn.BatchNorm2d(16), nn.ReLU(), nn.MaxPool2d(2),
@@ -182,8 +183,13 @@ def test_small_model_trains_at_l3():
     pattern = torch.randn(10, 3, 32, 32, device=DEV)
     x = torch.randn(64, 3, 32, 32, device=DEV) + pattern[y]
 
+    if channels_last:
+        x = x.contiguous(memory_format=torch.channels_last)
+
     def run(model):
         model = model.to(DEV)
+        if channels_last:
+            model = model.to(memory_format=torch.channels_last)
         opt = torch.optim.SGD(model.parameters(), lr=0.05, momentum=0.9)
         losses = []
         for _ in range(40):
