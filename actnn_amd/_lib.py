@@ -64,12 +64,14 @@ SIGNATURES = {
     "actnn_batch_norm_forward_apply": [c_vp, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u64, c_u64,
                                        c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
     "actnn_batch_norm_backward_packed": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp,
-                                         c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
-    "actnn_batch_norm_backward": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,
+                                         c_vp, c_vp, c_i64, c_vp, c_i64, c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
+    "actnn_batch_norm_backward": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_vp, c_i64,
                                   c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
+    "actnn_batch_norm_backward_sumsq_entries": [c_i64, c_i64, c_i64, c_i32, c_i32],
 }
 _RESTYPES = {"actnn_strerror": ctypes.c_char_p, "actnn_version": ctypes.c_char_p,
-             "actnn_batch_norm_workspace_bytes": ctypes.c_int64}
+             "actnn_batch_norm_workspace_bytes": ctypes.c_int64,
+             "actnn_batch_norm_backward_sumsq_entries": ctypes.c_int64}
 
 _lib = None
 

@@ -30,6 +30,7 @@ class QuantizationConfig:
         self.device_allocation = True                  # per-sample widths computed on the GPU when the batch fits
         self.fused_bn_backward = True                  # batch-norm backward reads the packed input directly
         self.share_relu_min_max = True                 # ReLU leaves its output's group min/max for the next layer
+        self.share_grad_sqnorm = True                  # batch-norm backward leaves sum(dx^2) for the conv's set_scale
         self.fused_bn_pack = True                      # batch-norm forward writes the packed copy of its input
         # memory management (conf.py:54-58)
         self.empty_cache_threshold = None

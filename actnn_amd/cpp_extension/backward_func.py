@@ -40,6 +40,25 @@ def _workspace_bytes(N, C, HW, code, channels_last):
     return _glue.lib().actnn_batch_norm_workspace_bytes(N, C, HW, code, channels_last)
 
 
+@functools.lru_cache(maxsize=4096)
+def _sumsq_entries(N, C, HW, code, channels_last):
+    return _glue.lib().actnn_batch_norm_backward_sumsq_entries(N, C, HW, code, channels_last)
+
+
+def _leave_sumsq(grad_input, table):
+    """Attach the partial sums of grad_input^2 that the backward pass left, for the layer that
+    receives this gradient next (QScheme.set_scale); the version pins them to these contents."""
+    grad_input._actnn_sumsq = (table, grad_input._version)
+
+
+def known_sumsq(grad):
+    """Total of grad^2 as a 0-d fp32 tensor if the kernel that wrote `grad` left it, else None."""
+    left = getattr(grad, "_actnn_sumsq", None)
+    if left is None or left[1] != grad._version:
+        return None
+    return left[0].sum()
+
+
 def _bn_geometry(input):
     """(N, C, HW, channels_last) of a dense tensor in the default or the channels-last layout."""
     if not (isinstance(input, torch.Tensor) and input.is_cuda):
@@ -162,14 +181,16 @@ def hip_batch_norm_pack_applies(input, weight, bias, running_mean, running_var):
     return not channels_last or N * HW < 2 ** 31
 
 
-def hip_batch_norm_backward(input, grad_output, weight, save_mean, save_invstd):
+def hip_batch_norm_backward(input, grad_output, weight, save_mean, save_invstd, sumsq=False):
     """-> (grad_input, grad_weight, grad_bias) of training-mode batch norm; `grad_output` has the
-    strides of `input`."""
+    strides of `input`.  With `sumsq` the pass also leaves the partial sums of grad_input^2 on
+    grad_input (see known_sumsq)."""
     N, C, HW, channels_last = _bn_geometry(input)
     lib = _glue.lib()
     code = _glue.DTYPE_CODE[input.dtype]
     ws_bytes = _workspace_bytes(N, C, HW, code, int(channels_last))
-    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=input.device)
+    entries = _sumsq_entries(N, C, HW, code, int(channels_last)) if sumsq else 0
+    ws = torch.empty(ws_bytes // 4 + entries, dtype=torch.float32, device=input.device)
     grad_input = torch.empty_like(input)
     grad_weight = torch.empty(C, dtype=torch.float32, device=input.device)
     grad_bias = torch.empty(C, dtype=torch.float32, device=input.device)
@@ -177,8 +198,10 @@ def hip_batch_norm_backward(input, grad_output, weight, save_mean, save_invstd):
         _glue._lib.check(lib.actnn_batch_norm_backward(
             input.data_ptr(), grad_output.data_ptr(), _ptr(weight), save_mean.data_ptr(),
             save_invstd.data_ptr(), grad_input.data_ptr(), grad_weight.data_ptr(), grad_bias.data_ptr(),
-            ws.data_ptr(), ws_bytes, N, C, HW, code, int(channels_last),
-            _glue.stream_ptr(input.device)), "batch_norm_backward")
+            ws.data_ptr(), ws_bytes, ws.data_ptr() + ws_bytes if entries else None, entries,
+            N, C, HW, code, int(channels_last), _glue.stream_ptr(input.device)), "batch_norm_backward")
+    if entries:
+        _leave_sumsq(grad_input, ws[ws_bytes // 4:])
     return grad_input, grad_weight, grad_bias
 
 
@@ -203,8 +226,9 @@ def hip_batch_norm_backward_packed_applies(shape, quantized, grad_output, weight
             and all(_f32_or_none(t) for t in (weight, save_mean, save_invstd)))
 
 
-def hip_batch_norm_backward_packed(shape, quantized, grad_output, weight, save_mean, save_invstd):
-    """-> (grad_input, grad_weight, grad_bias); the saved input is decoded inside the kernels."""
+def hip_batch_norm_backward_packed(shape, quantized, grad_output, weight, save_mean, save_invstd, sumsq=False):
+    """-> (grad_input, grad_weight, grad_bias); the saved input is decoded inside the kernels.
+    `sumsq` as in hip_batch_norm_backward."""
     from .quantization import _bits_info
     q_input, q_bits, q_scale, q_min = quantized
     channels_last = getattr(quantized, "memory_format", None) is not None
@@ -216,7 +240,8 @@ def hip_batch_norm_backward_packed(shape, quantized, grad_output, weight, save_m
         raise RuntimeError("batch_norm_backward_packed: packed stream is too short")
     ws_bytes = _workspace_bytes(N, C, HW, code, int(channels_last))
     dev = grad_output.device
-    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dev)
+    entries = _sumsq_entries(N, C, HW, code, int(channels_last)) if sumsq else 0
+    ws = torch.empty(ws_bytes // 4 + entries, dtype=torch.float32, device=dev)
     grad_input = torch.empty_like(grad_output)
     grad_weight = torch.empty(C, dtype=torch.float32, device=dev)
     grad_bias = torch.empty(C, dtype=torch.float32, device=dev)
@@ -225,7 +250,10 @@ def hip_batch_norm_backward_packed(shape, quantized, grad_output, weight, save_m
             q_input.data_ptr(), q_bits.data_ptr(), prefix.data_ptr(), q_scale.data_ptr(), q_min.data_ptr(),
             grad_output.data_ptr(), _ptr(weight), save_mean.data_ptr(), save_invstd.data_ptr(),
             grad_input.data_ptr(), grad_weight.data_ptr(), grad_bias.data_ptr(), ws.data_ptr(), ws_bytes,
+            ws.data_ptr() + ws_bytes if entries else None, entries,
             N, C, HW, code, int(channels_last), _glue.stream_ptr(dev)), "batch_norm_backward_packed")
+    if entries:
+        _leave_sumsq(grad_input, ws[ws_bytes // 4:])
     return grad_input, grad_weight, grad_bias
 
 
@@ -274,13 +302,13 @@ def cudnn_batch_norm(input, weight, bias, running_mean, running_var, training,
 
 
 def cudnn_batch_norm_backward(input, grad_output, weight, running_mean, running_var, save_mean,
-                              save_var, epsilon, reserve):
+                              save_var, epsilon, reserve, sumsq=False):
     """-> (grad_input, grad_weight, grad_bias).  at::native::cudnn_batch_norm_backward
-    (backward_func.cc:88)."""
+    (backward_func.cc:88).  `sumsq` (an addition): see hip_batch_norm_backward."""
     if (hip_batch_norm_applies(input, weight, None, save_mean, save_var)
             and grad_output.dtype == input.dtype and grad_output.shape == input.shape
             and grad_output.stride() == input.stride() and grad_output.data_ptr() % 16 == 0):
-        return hip_batch_norm_backward(input, grad_output, weight, save_mean, save_var)
+        return hip_batch_norm_backward(input, grad_output, weight, save_mean, save_var, sumsq)
     if not _miopen_takes(input, weight, weight):
         return _aten.native_batch_norm_backward(grad_output, input, weight, running_mean, running_var,
                                                 save_mean, save_var, True, epsilon, [True, True, True])

@@ -262,7 +262,18 @@ struct PackSink {
   int32_t* packed;
   uint64_t seed, offset;
   int64_t G;             // groups per sample
+  // backward apply only: when set, every wave leaves the sum of the squares of the gradient values
+  // it wrote (as stored, i.e. rounded to T) in sumsq[(blockIdx.y * gridDim.x + blockIdx.x) * kWaves +
+  // wave] - the gradient-norm statistic of the layer that receives this gradient, for free
+  float* sumsq;
 };
+
+ACTNN_DEV void leave_wave_sum(float* table, float v) {
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) v += __shfl_xor(v, d);
+  if ((threadIdx.x & 63) == 0)
+    table[((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * kWaves + (threadIdx.x >> 6)] = v;
+}
 
 template <int BITS>
 ACTNN_DEV void pack_chunk_bits(const float (&v)[8], const uint32_t (&r16)[8], float mul, float sub,
@@ -492,7 +503,9 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
   constexpr int NC = BWD ? 3 : 2;
   constexpr int kUnroll = PACK ? 2 : XS::kInFlight;      // measured: 2 beats 1 and 4 with the pack
   const Place p = place_of<E>(F, HW);
-  if (!p.active) return;               // whole quantisation groups (32 lanes) leave together
+  float sumsq = 0.0f;
+  if (!BWD && !p.active) return;       // whole quantisation groups (32 lanes) leave together
+  if (p.active) {                      // (backward: the lanes meet again for the wave's sum below)
   bind_input(xs, p);
   float k0[NC], k1[NC];
 #pragma unroll
@@ -526,6 +539,7 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
         o[i] = BWD ? fmaf(g[i], ka[e], fmaf(v[i], kb[e], kc[e])) : fmaf(v[i], ka[e], kb[e]);
       }
       r[j] = Chunk<T>::narrow(o);
+      if (BWD) Chunk<T>::dot(r[j], r[j], sumsq);
     }
     return u32x4{r[0], r[1], r[2], r[3]};
   };
@@ -557,6 +571,8 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
     if constexpr (PACK)
       pack_chunk<T>(ps, ux, n, p.elem >> 8, (n * F + p.elem) >> 3, ps.bits[n], (int64_t)ps.prefix[n] * ps.G * 8);
   }
+  }
+  if (BWD && ps.sumsq) leave_wave_sum(ps.sumsq, sumsq);
 }
 
 // ------------------------------------------------------------------ channels-last tensors
@@ -736,7 +752,9 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
     }
   };
   const RowTile t = row_tile<E>(C, tpr, R);
-  if (!t.active) return;               // whole quantisation groups leave together
+  float sumsq = 0.0f;
+  if (!BWD && !t.active) return;       // whole quantisation groups leave together
+  if (t.active) {                      // (backward: the lanes meet again for the wave's sum below)
   xs.bind(t.col, C);
   float ka[E], kb[E], kc[E];
 #pragma unroll
@@ -763,6 +781,7 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
         o[i] = BWD ? fmaf(g[i], ka[e], fmaf(v[i], kb[e], kc[e])) : fmaf(v[i], ka[e], kb[e]);
       }
       r[k] = Chunk<T>::narrow(o);
+      if (BWD) Chunk<T>::dot(r[k], r[k], sumsq);
     }
     return u32x4{r[0], r[1], r[2], r[3]};
   };
@@ -791,6 +810,8 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
     store_out(po + row * C, apply(ux, BWD ? load_last(pd + row * C) : ux));
     pack_row(ux, row, t.col);
   }
+  }
+  if (BWD && ps.sumsq) leave_wave_sum(ps.sumsq, sumsq);
 }
 
 // Launch geometry shared by the passes of one call.
@@ -870,6 +891,9 @@ bool make_plan(int64_t N, int64_t C, int64_t HW, int dtype, int channels_last, P
   return channels_last ? make_plan_cl(N, C, HW, dtype, pl) : make_plan(N, C, HW, dtype, pl);
 }
 int64_t workspace_floats(const Plan& pl, int64_t C) { return pl.part_floats + 3 * C; }
+int64_t apply_waves(const Plan& pl) {      // entries of the sum-of-squares table of the backward apply pass
+  return (pl.channels_last ? (int64_t)pl.tiles : pl.spans) * pl.nsplit * kWaves;
+}
 
 template <typename T, bool BWD, bool MINMAX, typename XS>
 void launch_reduce(const Plan& pl, const XS& xs, const void* dy, float* part, void* mn, void* mx,
@@ -960,7 +984,7 @@ int forward_apply_t(const Plan& pl, const void* x, void* y, const float* ws, con
 template <typename T, typename XS>
 int backward_t(const Plan& pl, const XS& xs, const void* dy, const float* weight, const float* save_mean,
                const float* save_invstd, void* dx, float* dweight, float* dbias, float* ws, int64_t N,
-               int64_t C, int64_t HW, hipStream_t s) {
+               int64_t C, int64_t HW, float* sumsq, hipStream_t s) {
   float* part = ws;
   float* coef = ws + pl.part_floats;
   if constexpr (XS::kRows) launch_cl_reduce<T, true, false>(pl, xs, dy, part, nullptr, nullptr, C, s);
@@ -968,9 +992,10 @@ int backward_t(const Plan& pl, const XS& xs, const void* dy, const float* weight
   bn_backward_finalize_kernel<<<dim3((unsigned)((C + kWaves - 1) / kWaves)), dim3(kThreads), 0, s>>>(
       part, weight, save_mean, save_invstd, dweight, dbias, coef, N, C, HW, pl.L, pl.nsplit, pl.slots);
   if (dx) {
-    const PackSink none{};
-    if constexpr (XS::kRows) launch_cl_apply<T, true, false>(pl, xs, dy, coef, dx, C, none, s);
-    else launch_apply<T, true, false>(pl, xs, dy, coef, dx, N, HW, none, s);
+    PackSink extra{};
+    extra.sumsq = sumsq;
+    if constexpr (XS::kRows) launch_cl_apply<T, true, false>(pl, xs, dy, coef, dx, C, extra, s);
+    else launch_apply<T, true, false>(pl, xs, dy, coef, dx, N, HW, extra, s);
   }
   ACTNN_RETURN_LAUNCH_STATUS();
 }
@@ -978,27 +1003,27 @@ int backward_t(const Plan& pl, const XS& xs, const void* dy, const float* weight
 template <typename T>
 int backward_plain(const Plan& pl, const void* x, const void* dy, const float* weight, const float* save_mean,
                    const float* save_invstd, void* dx, float* dweight, float* dbias, float* ws, int64_t N,
-                   int64_t C, int64_t HW, hipStream_t s) {
+                   int64_t C, int64_t HW, float* sumsq, hipStream_t s) {
   if (pl.channels_last) {
     const PlainRows<T> xs{static_cast<const T*>(x), C};
-    return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+    return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
   }
   const PlainInput<T> xs{static_cast<const T*>(x), pl.F};
-  return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+  return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
 }
 
 template <typename T>
 int backward_packed(const Plan& pl, const int32_t* packed, const int32_t* bits, const int32_t* prefix,
                     const void* scale, const void* mn, const void* dy, const float* weight,
                     const float* save_mean, const float* save_invstd, void* dx, float* dweight,
-                    float* dbias, float* ws, int64_t N, int64_t C, int64_t HW, hipStream_t s) {
+                    float* dbias, float* ws, int64_t N, int64_t C, int64_t HW, float* sumsq, hipStream_t s) {
   const PackedInput<T> in{packed, bits, prefix, static_cast<const T*>(scale), static_cast<const T*>(mn),
                           pl.F / 256, 0, 0u, false};
   if (pl.channels_last) {
     const PackedRows<T> xs{in, C, 0, (uint32_t)HW, 0u, 1, 0, 0};
-    return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+    return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
   }
-  return backward_t<T>(pl, in, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+  return backward_t<T>(pl, in, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
 }
 
 }  // namespace
@@ -1009,6 +1034,13 @@ extern "C" int64_t actnn_batch_norm_workspace_bytes(int64_t N, int64_t C, int64_
   actnn::Plan pl;
   if (!actnn::make_plan(N, C, HW, dtype, channels_last, pl)) return -1;
   return actnn::workspace_floats(pl, C) * (int64_t)sizeof(float);
+}
+
+extern "C" int64_t actnn_batch_norm_backward_sumsq_entries(int64_t N, int64_t C, int64_t HW, int dtype,
+                                                           int channels_last) {
+  actnn::Plan pl;
+  if (!actnn::make_plan(N, C, HW, dtype, channels_last, pl)) return -1;
+  return actnn::apply_waves(pl);
 }
 
 extern "C" int actnn_batch_norm_forward_stats(const void* x, const float* weight, const float* bias,
@@ -1080,21 +1112,23 @@ extern "C" int actnn_batch_norm_forward(const void* x, const float* weight, cons
 extern "C" int actnn_batch_norm_backward(const void* x, const void* dy, const float* weight,
                                          const float* save_mean, const float* save_invstd, void* dx,
                                          float* dweight, float* dbias, void* workspace,
-                                         int64_t workspace_bytes, int64_t N, int64_t C, int64_t HW,
-                                         int dtype, int channels_last, void* stream) {
+                                         int64_t workspace_bytes, float* sumsq, int64_t sumsq_entries,
+                                         int64_t N, int64_t C, int64_t HW, int dtype, int channels_last,
+                                         void* stream) {
   using namespace actnn;
   if (dtype < 0 || dtype > 2) return ACTNN_EDTYPE;
   Plan pl;
   if (!make_plan(N, C, HW, dtype, channels_last, pl)) return ACTNN_EINVAL;
   if (!x || !dy || !save_mean || !save_invstd || !workspace) return ACTNN_EINVAL;
+  if (sumsq && (!dx || sumsq_entries < apply_waves(pl))) return ACTNN_EINVAL;
   if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
   if (!aligned16(x) || !aligned16(dy) || (dx && !aligned16(dx)) || !aligned16(workspace)) return ACTNN_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   float* ws = static_cast<float*>(workspace);
   switch (dtype) {
-    case ACTNN_F32: return backward_plain<float>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
-    case ACTNN_F16: return backward_plain<__half>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
-    default: return backward_plain<bf16_t>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+    case ACTNN_F32: return backward_plain<float>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
+    case ACTNN_F16: return backward_plain<__half>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
+    default: return backward_plain<bf16_t>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
   }
 }
 
@@ -1103,7 +1137,8 @@ extern "C" int actnn_batch_norm_backward_packed(const int32_t* packed, const int
                                                 const void* dy, const float* weight,
                                                 const float* save_mean, const float* save_invstd,
                                                 void* dx, float* dweight, float* dbias, void* workspace,
-                                                int64_t workspace_bytes, int64_t N, int64_t C,
+                                                int64_t workspace_bytes, float* sumsq,
+                                                int64_t sumsq_entries, int64_t N, int64_t C,
                                                 int64_t HW, int dtype, int channels_last,
                                                 void* stream) {
   using namespace actnn;
@@ -1111,12 +1146,13 @@ extern "C" int actnn_batch_norm_backward_packed(const int32_t* packed, const int
   Plan pl;
   if (!make_plan(N, C, HW, dtype, channels_last, pl) || !pl.groups_align) return ACTNN_EINVAL;
   if (channels_last && pl.P > 0x7fffffffLL) return ACTNN_EINVAL;
+  if (sumsq && (!dx || sumsq_entries < apply_waves(pl))) return ACTNN_EINVAL;
   if (!packed || !bits || !prefix || !scale || !mn || !dy || !save_mean || !save_invstd || !workspace) return ACTNN_EINVAL;
   if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
   if (!aligned16(dy) || (dx && !aligned16(dx)) || !aligned16(workspace)) return ACTNN_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   float* ws = static_cast<float*>(workspace);
   if (dtype == ACTNN_F16)
-    return backward_packed<__half>(pl, packed, bits, prefix, scale, mn, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
-  return backward_packed<bf16_t>(pl, packed, bits, prefix, scale, mn, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s);
+    return backward_packed<__half>(pl, packed, bits, prefix, scale, mn, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
+  return backward_packed<bf16_t>(pl, packed, bits, prefix, scale, mn, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
 }

@@ -382,6 +382,14 @@ class linear(Function):
 # ------------------------------------------------------------------------------------------
 # batch norm (ops.py:436-502)
 # ------------------------------------------------------------------------------------------
+def _leaves_grad_sqnorm():
+    """Batch-norm backward leaves the squared norm of its input gradient for the set_scale of the
+    convolution before it (the statistic is one number per layer unless gradients are tracked per
+    sample)."""
+    from .qscheme import QScheme
+    return config.share_grad_sqnorm and QScheme.update_scale and not config.use_gradient
+
+
 def _bn_shares_min_max(input, weight, bias, running_mean, running_var, training):
     return (training and config.compress_activation and not config.simulate and config.group_size == 256
             and ext_backward_func.hip_batch_norm_minmax_applies(input, weight, bias, running_mean, running_var))
@@ -452,7 +460,8 @@ class batch_norm(Function):
                     ctx.other_args, quantized, grad_output, weight, save_mean, save_var):
                 # the kernels decode the saved input from its bit stream: no full-precision copy
                 grads = ext_backward_func.hip_batch_norm_backward_packed(
-                    ctx.other_args, quantized, grad_output, weight, save_mean, save_var)
+                    ctx.other_args, quantized, grad_output, weight, save_mean, save_var,
+                    sumsq=_leaves_grad_sqnorm())
                 del quantized, ctx.saved
                 if ctx.scheme:
                     ctx.scheme.if_allocate_perlayer()
@@ -465,7 +474,7 @@ class batch_norm(Function):
             grad_input, grad_weight, grad_bias = ext_backward_func.cudnn_batch_norm_backward(
                 input.contiguous(memory_format=memory_format),
                 grad_output.contiguous(memory_format=memory_format), weight, running_mean, running_var,
-                save_mean, save_var, eps, reserve)
+                save_mean, save_var, eps, reserve, sumsq=_leaves_grad_sqnorm())
         else:
             grad_input, grad_weight, grad_bias = ext_backward_func.native_batch_norm_backward(
                 grad_output, input, weight, running_mean, running_var, save_mean, save_var, training, eps,

@@ -9,6 +9,7 @@ average of `bits` per sample.
 import torch
 
 from .conf import config
+from .cpp_extension import backward_func as ext_backward_func
 from .cpp_extension import calc_precision as ext_calc_precision
 from .cpp_extension import minimax as ext_minimax
 from .cpp_extension.quantization import attach_bits_host, attach_bits_total
@@ -166,6 +167,11 @@ class QScheme(_LazyHost):
         """Squared gradient norm per sample, kept as a running value (qscheme.py:47-55)."""
         if not QScheme.update_scale:
             return
+        if not config.use_gradient and config.share_grad_sqnorm:
+            total = ext_backward_func.known_sumsq(grad)     # left by the kernel that wrote `grad`
+            if total is not None:
+                self.scales = total / grad.shape[0]
+                return
         # squared L2 norm per sample, accumulated in fp32 in one pass over the gradient
         sq = ext_minimax.sample_sqnorm(grad)
         if config.use_gradient:

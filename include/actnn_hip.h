@@ -232,8 +232,15 @@ int actnn_batch_norm_forward(const void* x, const float* weight, const float* bi
 int actnn_batch_norm_backward(const void* x, const void* dy, const float* weight,
                               const float* save_mean, const float* save_invstd, void* dx,
                               float* dweight, float* dbias, void* workspace,
-                              int64_t workspace_bytes, int64_t N, int64_t C, int64_t HW, int dtype,
-                              int channels_last, void* stream);
+                              int64_t workspace_bytes, float* sumsq, int64_t sumsq_entries,
+                              int64_t N, int64_t C, int64_t HW, int dtype, int channels_last,
+                              void* stream);
+/* `sumsq` (may be null) of the two backward entry points: a table of
+ * actnn_batch_norm_backward_sumsq_entries(...) floats that receives partial sums of dx^2 (the values
+ * as stored in dx); their total is the squared norm of the gradient the preceding layer receives -
+ * the statistic of qscheme.py:47-55 - without another pass over dx. */
+int64_t actnn_batch_norm_backward_sumsq_entries(int64_t N, int64_t C, int64_t HW, int dtype,
+                                                int channels_last);
 
 /* The forward pass in two steps, for callers that want the quantiser's output from the same read
  * of x: _stats runs the statistics pass (save_mean/save_invstd, running estimates, optional group
@@ -264,8 +271,8 @@ int actnn_batch_norm_backward_packed(const int32_t* packed, const int32_t* bits,
                                      const void* dy, const float* weight, const float* save_mean,
                                      const float* save_invstd, void* dx, float* dweight,
                                      float* dbias, void* workspace, int64_t workspace_bytes,
-                                     int64_t N, int64_t C, int64_t HW, int dtype,
-                                     int channels_last, void* stream);
+                                     float* sumsq, int64_t sumsq_entries, int64_t N, int64_t C,
+                                     int64_t HW, int dtype, int channels_last, void* stream);
 
 /* Plain device-to-device streaming copy of `bytes` bytes (16-byte aligned pointers and
  * size); used by the benchmark to calibrate bandwidth counters.  No reference counterpart. */

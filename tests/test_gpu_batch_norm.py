@@ -147,6 +147,26 @@ def test_backward_from_the_packed_stream_equals_unpack_then_backward(N, C, spati
     got = ext_bf.hip_batch_norm_backward_packed(x.shape, quantized, dy, w, mean, invstd)
     for a, r in zip(got, ref):
         assert torch.equal(a, r)
+    _check_sumsq(lambda: ext_bf.hip_batch_norm_backward_packed(x.shape, quantized, dy, w, mean, invstd, sumsq=True),
+                 lambda: ext_bf.hip_batch_norm_backward(xq, dy, w, mean, invstd, sumsq=True), ref)
+
+
+def _check_sumsq(*args):
+    """Both backward passes, asked for it, leave sum(dx^2) of the dx they store (float64 sum of the
+    stored values, rtol 1e-5: fp32 partial sums of at most a few thousand products each) and
+    change nothing else; the statistic lapses when dx is written to afterwards."""
+    *passes, ref = args
+    for run in passes:
+        got = run()
+        for a, r in zip(got, ref):
+            assert torch.equal(a, r)
+        total = ext_bf.known_sumsq(got[0])
+        want = got[0].double().square().sum()
+        assert total is not None and total.dtype == torch.float32
+        assert abs(total.double().item() - want.item()) <= 1e-5 * want.item() + 1e-30
+        got[0].mul_(2.0)
+        assert ext_bf.known_sumsq(got[0]) is None
+    assert ext_bf.known_sumsq(ref[0]) is None
 
 
 # ------------------------------------------------------------------------------------------
@@ -230,6 +250,8 @@ def test_channels_last_backward_from_the_packed_stream(N, C, spatial, dtype):
     assert got[0].stride() == x.stride()
     for a, r in zip(got, ref):
         assert torch.equal(a, r)
+    _check_sumsq(lambda: ext_bf.hip_batch_norm_backward_packed(x.shape, quantized, dy, w, mean, invstd, sumsq=True),
+                 lambda: ext_bf.hip_batch_norm_backward(xq, dy, w, mean, invstd, sumsq=True), ref)
 
 
 @pytest.mark.parametrize("channels_last", [False, True])

@@ -479,3 +479,43 @@ def test_relu_hands_group_min_max_to_the_next_convolution(channels_last):
     h1.add_(1.0)
     assert known_group_minmax(h1) is None                    # changed in place: the version moved on
     assert known_group_minmax(h0.float()) is None
+
+
+@pytest.mark.parametrize("channels_last", [False, True])
+def test_batch_norm_backward_hands_the_gradient_norm_to_the_convolution(channels_last):
+    """QConv2d -> QBatchNorm2d: the convolution's running gradient statistic (qscheme.py:47-55) is
+    the same whether batch-norm backward leaves sum(dx^2) or the convolution reduces its incoming
+    gradient itself (fp32 sums in different orders: rtol 1e-5), and the gradients are identical."""
+    def run(share):
+        config.reset(); QScheme.reset(); QBNScheme.reset()
+        config.share_grad_sqnorm = share
+        config.perlayer = False
+        torch.manual_seed(0)
+        conv = actnn_amd.QConv2d(16, 64, 3, padding=1, bias=False).to(DEV)
+        bn = actnn_amd.QBatchNorm2d(64).to(DEV)
+        x = torch.randn(16, 16, 16, 16, device=DEV).bfloat16()
+        if channels_last:
+            conv, bn = conv.to(memory_format=torch.channels_last), bn.to(memory_format=torch.channels_last)
+            x = x.contiguous(memory_format=torch.channels_last)
+        x.requires_grad_(True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            torch.cuda.manual_seed(4)
+            y = bn(conv(x))
+        g = torch.randn_like(y)
+        grads = torch.autograd.grad(y, [x, conv.weight, bn.weight], g)
+        return conv.scheme.scales, grads
+    s0, g0 = run(False)
+    s1, g1 = run(True)
+    assert all(torch.equal(a, b) for a, b in zip(g0, g1))
+    s0, s1 = float(s0), float(s1)
+    assert s0 > 0 and abs(s0 - s1) <= 1e-5 * s0
+    # the statistic really came from the hand-off: without the attribute set_scale reduces itself
+    import actnn_amd.cpp_extension.backward_func as ext_bf
+    seen = []
+    original = ext_bf.known_sumsq
+    ext_bf.known_sumsq = lambda grad: seen.append(original(grad)) or seen[-1]
+    try:
+        run(True)
+    finally:
+        ext_bf.known_sumsq = original
+    assert len(seen) == 1 and seen[0] is not None
