@@ -1,9 +1,9 @@
 """actnn_amd: MI355X-native activation-compressed training layers.
 
-Same public names as the reference package (actnn/actnn/__init__.py:1-10) minus its DataLoader
-fork; the kernels live in libactnn_hip.so (include/actnn_hip.h) and there is no CPU fallback.
+Same public names as the reference package (actnn/actnn/__init__.py:1-10); the kernels live in
+libactnn_hip.so (include/actnn_hip.h) and there is no CPU fallback.
 """
-from . import ops  # noqa: F401
+from . import dataloader, ops  # noqa: F401
 from .conf import config, set_optimization_level
 from .layers import (QAvgPool2d, QBatchNorm1d, QBatchNorm2d, QBatchNorm3d, QConv1d, QConv2d, QConv3d,
                      QConvTranspose1d, QConvTranspose2d, QConvTranspose3d, QDropout, QLinear, QMaxPool2d,
@@ -15,4 +15,5 @@ from .utils import compute_tensor_bytes, exp_recorder, get_memory_usage
 
 __all__ = ["config", "set_optimization_level", "QModule", "QScheme", "QBNScheme", "QConv1d", "QConv2d",
            "QConv3d", "QConvTranspose1d", "QConvTranspose2d", "QConvTranspose3d", "QLinear", "QBatchNorm1d", "QBatchNorm2d", "QBatchNorm3d", "QReLU", "QDropout",
-           "QMaxPool2d", "QAvgPool2d", "get_memory_usage", "compute_tensor_bytes", "exp_recorder", "ops"]
+           "QMaxPool2d", "QAvgPool2d", "get_memory_usage", "compute_tensor_bytes", "exp_recorder", "ops",
+           "dataloader"]

@@ -155,12 +155,28 @@ class QScheme(_LazyHost):
         QScheme.num_layers += 1
 
     # -- gradient statistics ----------------------------------------------------------------
-    def get_scale(self):
+    _batch_index_cache = None
+
+    @staticmethod
+    def batch_index(device):
+        """QScheme.batch as an int64 index tensor on `device`, converted once per batch and device
+        (the list object is held, so a new batch is a new object)."""
+        cached = QScheme._batch_index_cache
+        if cached is None or cached[0] is not QScheme.batch or cached[1] != device:
+            index = torch.as_tensor(QScheme.batch, dtype=torch.long).to(device)
+            QScheme._batch_index_cache = cached = (QScheme.batch, device, index)
+        return cached[2]
+
+    def get_scale(self, device=None):
+        """Gradient statistic of the current batch (qscheme.py:37-45).  With config.use_gradient the
+        per-sample table moves to `device` on first use and stays there: looking up and updating a
+        batch's entries are indexed device operations, without a host round trip per layer."""
         if config.use_gradient:
             assert QScheme.batch is not None
-            scale = self.scales[QScheme.batch].clone()
-            scale[scale == 0] = scale.mean() + 1e-9
-            return scale
+            if device is not None and self.scales.device != device:
+                self.scales = self.scales.to(device)
+            scale = self.scales[QScheme.batch_index(self.scales.device)]
+            return torch.where(scale == 0, scale.mean() + 1e-9, scale)     # samples not seen yet
         return self.scales
 
     def set_scale(self, grad):
@@ -176,14 +192,17 @@ class QScheme(_LazyHost):
         sq = ext_minimax.sample_sqnorm(grad)
         if config.use_gradient:
             assert QScheme.batch is not None
-            self.scales[QScheme.batch] = self.scales[QScheme.batch] * 0.5 + sq.cpu() * 0.5
+            if self.scales.device != sq.device:
+                self.scales = self.scales.to(sq.device)
+            index = QScheme.batch_index(sq.device)
+            self.scales[index] = self.scales[index] * 0.5 + sq * 0.5
         else:
             self.scales = sq.mean()
 
     # -- forward-time allocation ------------------------------------------------------------
     def sensitivity(self, mn, mx, N, num_pixels):
         """C_n = num_locations / 4 / depthwise_groups * Range_sqr_n * grad_sum_n  (qscheme.py:80-82)."""
-        grad_sum = self.get_scale().to(device=mn.device, dtype=torch.float32)
+        grad_sum = self.get_scale(mn.device).to(device=mn.device, dtype=torch.float32)
         return range_sqr(mn, mx, N, num_pixels, self.num_locations / 4 / self.depthwise_groups, grad_sum)
 
     def compute_quantization_bits(self, input):
@@ -197,7 +216,7 @@ class QScheme(_LazyHost):
         groups, mn, mx, num_pixels = group_min_max(input, known_minmax)
         bits_dev = None
         if allocate_on_device(N, self.initial_bits) and mn.is_contiguous() and mx.is_contiguous():
-            grad_sum = self.get_scale().to(device=mn.device, dtype=torch.float32)
+            grad_sum = self.get_scale(mn.device).to(device=mn.device, dtype=torch.float32)
             C_dev, bits_dev = allocate_bits_on_device(
                 mn, mx, N, num_pixels, self.num_locations / 4 / self.depthwise_groups, grad_sum,
                 self.initial_bits, self.bits)
@@ -269,3 +288,4 @@ class QScheme(_LazyHost):
         QScheme.num_layers = 0
         QScheme.prev_layer = None
         QScheme.batch = None
+        QScheme._batch_index_cache = None

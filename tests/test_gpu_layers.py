@@ -519,3 +519,51 @@ def test_batch_norm_backward_hands_the_gradient_norm_to_the_convolution(channels
     finally:
         ext_bf.known_sumsq = original
     assert len(seen) == 1 and seen[0] is not None
+
+
+def test_per_sample_gradient_statistics_with_the_index_yielding_loader():
+    """config.use_gradient (qscheme.py:20-22,37-55): every layer keeps one running squared gradient
+    norm per dataset entry; the loader supplies the entries of each batch.  The table lives on the
+    device, holds 0.5 * ||grad_n||^2 after an entry's first visit (running value from 0), leaves
+    entries not yet visited at zero, and entries not yet visited borrow the batch mean when the
+    widths are allocated."""
+    from torch.utils.data import TensorDataset
+    from actnn_amd.dataloader import DataLoader
+    torch.manual_seed(0)
+    data = TensorDataset(torch.randn(48, 8, 16, 16) * torch.linspace(0.2, 3.0, 48).view(48, 1, 1, 1),
+                         torch.randint(0, 4, (48,)))
+    config.use_gradient = True
+    QScheme.num_samples = len(data)
+    model = QModule(nn.Sequential(nn.Conv2d(8, 8, 3, padding=1), nn.BatchNorm2d(8), nn.ReLU(),
+                                  nn.Conv2d(8, 4, 3, padding=1), nn.AdaptiveAvgPool2d(1), nn.Flatten())).to(DEV)
+    first, last = QScheme.layers[0], QScheme.layers[1]
+    assert first.scales.shape == (48,)
+    grads = {}
+    model.model[3].register_full_backward_hook(lambda m, gi, go: grads.__setitem__("last", go[0].detach().clone()))
+    loader = DataLoader(data, batch_size=16, shuffle=True, generator=torch.Generator().manual_seed(1))
+    seen = []
+    for step, (indices, (x, y)) in enumerate(loader):
+        QScheme.batch = indices
+        F.cross_entropy(model(x.to(DEV)), y.to(DEV)).backward()
+        seen += indices
+        assert last.scales.is_cuda and first.scales.is_cuda
+        want = 0.5 * grads["last"].double().flatten(1).square().sum(1)
+        got = last.scales[torch.tensor(indices, device=DEV)].double()
+        assert torch.allclose(got, want, rtol=1e-5, atol=0)
+        rest = sorted(set(range(48)) - set(seen))
+        assert (last.scales[torch.tensor(rest, device=DEV, dtype=torch.long)] == 0).all()
+        if step == 1:
+            break
+    # second visit: running value, and a batch with unseen entries borrows the mean for them
+    QScheme.batch = seen[:8] + rest[:8]
+    scale = last.get_scale(torch.device(DEV))
+    table = last.scales[torch.tensor(QScheme.batch, device=DEV)]
+    assert torch.equal(scale[:8], table[:8]) and (table[8:] == 0).all()
+    assert torch.allclose(scale[8:], (table.mean() + 1e-9).expand(8))
+    before = last.scales.clone()
+    x, y = data[QScheme.batch]
+    F.cross_entropy(model(x.to(DEV)), y.to(DEV)).backward()
+    want = 0.5 * before[torch.tensor(QScheme.batch, device=DEV)].double() \
+        + 0.5 * grads["last"].double().flatten(1).square().sum(1)
+    assert torch.allclose(last.scales[torch.tensor(QScheme.batch, device=DEV)].double(), want, rtol=1e-5, atol=0)
+    assert int(last.b.min()) >= 1 and int(last.b.sum()) <= int(last.bits * 16) and len(set(last.b.tolist())) > 1
