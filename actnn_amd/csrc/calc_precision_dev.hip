@@ -6,17 +6,17 @@
 // priority queue and pushes the popped item's next step.  The steps of one item get strictly more
 // expensive (delta more negative) as its width shrinks - or stay equal when C is 0 - so the popped
 // set is exactly the K largest of all N * (initial - 1) candidate steps under the order
-// (delta, index, earlier step first).  Every block builds the keys of all candidates in LDS with
-// the reference's arithmetic (delta evaluated in double, narrowed to float) and ranks the steps of
-// a few items by counting the keys above each of them - 16 threads per step, each over a 16th of
-// the keys - so the whole allocation is one launch of independent blocks: no sort, no atomics.
+// (delta, index, earlier step first).  Every block builds the keys of all candidates with the
+// reference's arithmetic (delta evaluated in double, narrowed to float) - each thread a 256th of
+// them, in registers - and ranks the steps of a few items by counting the keys above each of
+// them, so the whole allocation is one launch of independent blocks: no sort, no atomics.
 #include "device_utils.h"
 
 namespace actnn {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kMaxCand = 8192;           // 64 KiB of keys: all a kernel gets without asking
+constexpr int kMaxCand = 8192;           // a thread counts at most 32 keys per candidate (8-bit counters)
 constexpr int kSlots = 16;               // candidate steps ranked per block (16 threads each)
 
 // Key of step `l` (width initial - l -> initial - l - 1) of item i: larger key = popped earlier.
@@ -35,51 +35,80 @@ __global__ __launch_bounds__(kThreads) void fill_kernel(int32_t* __restrict__ ou
 
 __global__ __launch_bounds__(kThreads) void calc_precision_device_kernel(
     const float* __restrict__ C, int32_t* __restrict__ bits, int N, int initial, int64_t K) {
-  __shared__ uint64_t keys[kMaxCand];
+  constexpr int kWaves = kThreads / 64;
+  __shared__ double factors[8];
+  __shared__ float C_s[kMaxCand];                      // N <= kMaxCand / L
+  __shared__ uint64_t mine_s[kSlots];
+  __shared__ int above_s[kWaves][kSlots];
+  __shared__ int taken[kSlots];
   const int L = initial - 1;
   const int total = N * L;
   const int items_per_block = kSlots / L;
+  const int nslot = items_per_block * L;
   const int item0 = blockIdx.x * items_per_block;
   if (K <= 0 || K >= total) {                          // nothing to take, or everything
     if ((int)threadIdx.x < items_per_block && item0 + (int)threadIdx.x < N)
       bits[item0 + threadIdx.x] = K <= 0 ? initial : 1;
     return;
   }
-  // 1/(2^b - 1)^2 - 1/(2^(b-1) - 1)^2 for the L steps: held in the tail of the key array until the
-  // keys that would overwrite it are built (total < kMaxCand leaves room; otherwise per key)
-  const bool shared_factors = total + 8 <= kMaxCand;
-  double* factors = reinterpret_cast<double*>(keys + kMaxCand - 8);
-  auto factor_of = [&](int l) {
-    const int b = initial - l;
+  for (int n = threadIdx.x; n < N; n += kThreads) C_s[n] = C[n];      // one trip to memory for all keys
+  // 1/(2^b - 1)^2 - 1/(2^(b-1) - 1)^2 for the L steps
+  if ((int)threadIdx.x < L) {
+    const int b = initial - (int)threadIdx.x;
     const int64_t full = ((int64_t)1 << b) - 1, less = ((int64_t)1 << (b - 1)) - 1;
-    return 1.0 / (double)(full * full) - 1.0 / (double)(less * less);
-  };
-  if (shared_factors) {
-    if ((int)threadIdx.x < L) factors[threadIdx.x] = factor_of(threadIdx.x);
-    __syncthreads();
-  }
-  for (int c = threadIdx.x; c < total; c += kThreads) {
-    const int i = c / L, l = c - i * L;
-    keys[c] = step_key(C[i], shared_factors ? factors[l] : factor_of(l), i, l);
+    factors[threadIdx.x] = 1.0 / (double)(full * full) - 1.0 / (double)(less * less);
   }
   __syncthreads();
-  // thread -> (slot = candidate of this block, seg = which 16th of the keys it counts over)
-  const int slot = threadIdx.x >> 4, seg = threadIdx.x & 15;
-  const int cand = item0 * L + slot;
-  const bool live = slot < items_per_block * L && cand < total;
-  const uint64_t mine = live ? keys[cand] : ~0ull;
-  int above = 0;
-  for (int m = seg; m < total; m += 16) above += keys[m] > mine ? 1 : 0;
-  above += __shfl_xor(above, 1);
-  above += __shfl_xor(above, 2);
-  above += __shfl_xor(above, 4);
-  above += __shfl_xor(above, 8);                       // the 16 threads of a slot are 16 consecutive lanes
-  __shared__ int taken[kSlots];
-  if (seg == 0) taken[slot] = live && above < K ? 1 : 0;
+  // the block's own candidates: steps item0 * L + slot
+  if ((int)threadIdx.x < kSlots) {
+    const int slot = threadIdx.x, cand = item0 * L + slot;
+    uint64_t key = ~0ull;                              // nothing ranks above a dead slot
+    if (slot < nslot && cand < total) {
+      const int i = cand / L, l = cand - i * L;
+      key = step_key(C_s[i], factors[l], i, l);
+    }
+    mine_s[slot] = key;
+  }
+  __syncthreads();
+  uint64_t mine[kSlots];
+#pragma unroll
+  for (int sl = 0; sl < kSlots; ++sl) mine[sl] = mine_s[sl];
+  // every thread builds a 256th of all keys in registers and counts, for each of the block's
+  // candidates, the keys above it (the counts of a thread stay below 256: four to a register)
+  uint32_t packed[kSlots / 4];
+#pragma unroll
+  for (int q = 0; q < kSlots / 4; ++q) packed[q] = 0u;
+  int i = (int)threadIdx.x / L, l = (int)threadIdx.x - i * L;
+  const int di = kThreads / L, dl = kThreads - di * L;
+  for (int c = threadIdx.x; c < total; c += kThreads) {
+    const uint64_t key = step_key(C_s[i], factors[l], i, l);
+#pragma unroll
+    for (int sl = 0; sl < kSlots; ++sl) packed[sl / 4] += (key > mine[sl] ? 1u : 0u) << (8 * (sl % 4));
+    i += di;
+    l += dl;
+    if (l >= L) { l -= L; ++i; }
+  }
+  // counts of the block: butterfly inside each wave, then across the waves through LDS
+#pragma unroll
+  for (int sl = 0; sl < kSlots; ++sl) {
+    int v = (int)((packed[sl / 4] >> (8 * (sl % 4))) & 0xffu);
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) v += __shfl_xor(v, d);
+    if ((threadIdx.x & 63) == 0) above_s[threadIdx.x >> 6][sl] = v;
+  }
+  __syncthreads();
+  if ((int)threadIdx.x < kSlots) {
+    const int slot = threadIdx.x;
+    int above = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) above += above_s[w][slot];
+    const bool live = slot < nslot && item0 * L + slot < total;
+    taken[slot] = live && above < K ? 1 : 0;
+  }
   __syncthreads();
   if ((int)threadIdx.x < items_per_block && item0 + (int)threadIdx.x < N) {
     int t = 0;
-    for (int l = 0; l < L; ++l) t += taken[threadIdx.x * L + l];
+    for (int k = 0; k < L; ++k) t += taken[threadIdx.x * L + k];
     bits[item0 + threadIdx.x] = initial - t;
   }
 }
