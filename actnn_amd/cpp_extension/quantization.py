@@ -286,10 +286,13 @@ class ActQuantizedReLUMinMax(Function):
         output, mask, mn, mx = relu_forward_minmax(input)
         ctx.save_for_backward(mask)
         ctx.mark_non_differentiable(mn, mx)
+        ctx.set_materialize_grads(False)          # no zero tensors for the two statistics
         return output, mn, mx
 
     @staticmethod
     def backward(ctx, grad_output, _grad_mn, _grad_mx):
+        if grad_output is None:
+            return None
         (mask,) = ctx.saved_tensors
         return relu_backward(grad_output, mask)
 

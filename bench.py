@@ -28,7 +28,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, then WRITE_SIZE, each scaled by
 # what the same counter reads for actnn_stream_copy of a known size); see profiles/.  None = not
 # measured yet.
-MEASURED_TRAFFIC_BYTES = {"minimax": 828537445, "pack_mixed": 892279188, "unpack_mixed": 886739578}
+MEASURED_TRAFFIC_BYTES = {"minimax": 828536830, "pack_mixed": 892254308, "unpack_mixed": 886732426}
 
 
 def _event_time_ms(fn, reps, warmup=3):
