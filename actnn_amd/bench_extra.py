@@ -74,3 +74,57 @@ def run(device):
         out[key] = resnet50_step(device, level, channels_last=channels_last)
     torch.cuda.empty_cache()
     return out
+
+
+# ResNet-50's batch-norm inputs: (channels, height = width, how many layers have this shape)
+RESNET50_BN_SHAPES = [(64, 112, 1), (64, 56, 6), (256, 56, 4), (128, 56, 1), (128, 28, 7), (512, 28, 5),
+                      (256, 28, 1), (256, 14, 11), (1024, 14, 7), (512, 14, 1), (512, 7, 5), (2048, 7, 4)]
+
+
+def batch_norm_shapes(device, channels_last=True, batch=512, reps=10):
+    """The three fused batch-norm steps of an L3 training step (statistics + group min/max;
+    normalise + 2-bit pack; backward from the packed input with the gradient norm), timed with
+    events on every batch-norm shape of ResNet-50 in bf16: ms and GB/s of algorithmic bytes per
+    shape, and the totals weighted by the number of layers."""
+    import actnn_amd.cpp_extension.backward_func as bf
+    from .cpp_extension.quantization import attach_bits_total
+    from .ops import _Quantized
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize(device)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(reps):
+            fn()
+        stop.record()
+        torch.cuda.synchronize(device)
+        return start.elapsed_time(stop) / reps
+
+    rows, totals = [], [0.0, 0.0, 0.0]
+    for C, H, count in RESNET50_BN_SHAPES:
+        x = torch.randn(batch, C, H, H, device=device, dtype=torch.bfloat16)
+        dy = torch.randn_like(x)
+        if channels_last:
+            x = x.contiguous(memory_format=torch.channels_last)
+            dy = dy.contiguous(memory_format=torch.channels_last)
+        w, b = torch.rand(C, device=device) + 0.5, torch.randn(C, device=device)
+        n = x.numel()
+        bits = attach_bits_total(torch.full((batch,), 2, dtype=torch.int32, device=device), 2 * batch)
+        ws, mean, invstd, mn, mx = bf.hip_batch_norm_forward_stats(x, w, b, None, None, 0.1, 1e-5)
+        _, packed, scale = bf.hip_batch_norm_forward_apply(x, ws, bits, mn, mx)
+        quantized = _Quantized((packed, bits, scale, mn.view(batch, -1, 1)))
+        quantized.native_bf16 = True
+        quantized.memory_format = torch.channels_last if channels_last else None
+        t = [timed(lambda: bf.hip_batch_norm_forward_stats(x, w, b, None, None, 0.1, 1e-5)),
+             timed(lambda: bf.hip_batch_norm_forward_apply(x, ws, bits, mn, mx)),
+             timed(lambda: bf.hip_batch_norm_backward_packed(x.shape, quantized, dy, w, mean, invstd, sumsq=True))]
+        nbytes = [2 * n + 4 * n / 256, 4 * n + n / 4 + 2 * n / 256, 3 * 2 * n + 2 * (n / 4 + 4 * n / 256)]
+        rows.append({"shape": [C, H, H], "layers": count, "ms": [round(v, 4) for v in t],
+                     "GB/s": [round(nb / v / 1e6) for nb, v in zip(nbytes, t)]})
+        for k in range(3):
+            totals[k] += count * t[k]
+    return {"steps": ["statistics+minmax", "normalise+pack", "backward_from_2bit_stream"], "batch": batch,
+            "memory_format": "channels_last" if channels_last else "contiguous", "shapes": rows,
+            "ms_per_training_step": [round(v, 3) for v in totals]}

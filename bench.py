@@ -230,9 +230,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the config-2 hot path")
-    ap.add_argument("--only", choices=["other", "resnet50", "resnet50_channels_last"], default=None,
+    ap.add_argument("--only", choices=["other", "resnet50", "resnet50_channels_last", "batch_norm_shapes"],
+                    default=None,
                     help="profiling aid: run just the other single-GPU configs (ReLU, max-pool, "
-                         "fixed-width pack, fused GEMM) or just the ResNet-50 L3 step, print their JSON")
+                         "fixed-width pack, fused GEMM), just the ResNet-50 L3 step, or the fused "
+                         "batch-norm passes on every batch-norm shape of ResNet-50; print their JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the hot path shards by sample with no exchange step, "
@@ -257,6 +259,11 @@ def main():
         from actnn_amd import bench_extra
         print(json.dumps({"resnet50_L3_channels_last": bench_extra.resnet50_step(
             device, "L3", warmup=2, steps=3, channels_last=True)}))
+        return
+    if args.only == "batch_norm_shapes":
+        from actnn_amd import bench_extra
+        print(json.dumps({"batch_norm_shapes": [bench_extra.batch_norm_shapes(device, channels_last=cl)
+                                                for cl in (True, False)]}))
         return
     xg, mn, mx, bits, bits_host = make_config2(device)
     N, G, gs = xg.shape

@@ -474,8 +474,12 @@ def test_relu_hands_group_min_max_to_the_next_convolution(channels_last):
         return h, saved, gx
     h0, s0, g0 = run(False)
     h1, s1, g1 = run(True)
-    assert torch.equal(h0, h1) and torch.equal(g0, g1)
+    assert torch.equal(h0, h1)
     assert all(torch.equal(a, b) for a, b in zip(s0, s1))
+    # the gradient passes through MIOpen's backward-data kernel, which may add in no fixed order
+    # before rounding to bf16: one rounding step of slack
+    a, b = g0.float(), g1.float()
+    assert ((a - b).abs() <= 2.0 ** -7 * torch.maximum(a.abs(), b.abs()) + 1e-3 * a.abs().max()).all()
     h1.add_(1.0)
     assert known_group_minmax(h1) is None                    # changed in place: the version moved on
     assert known_group_minmax(h0.float()) is None
@@ -485,7 +489,7 @@ def test_relu_hands_group_min_max_to_the_next_convolution(channels_last):
 def test_batch_norm_backward_hands_the_gradient_norm_to_the_convolution(channels_last):
     """QConv2d -> QBatchNorm2d: the convolution's running gradient statistic (qscheme.py:47-55) is
     the same whether batch-norm backward leaves sum(dx^2) or the convolution reduces its incoming
-    gradient itself (fp32 sums in different orders: rtol 1e-5), and the gradients are identical."""
+    gradient itself (fp32 sums in different orders: rtol 1e-5), and the gradients agree."""
     def run(share):
         config.reset(); QScheme.reset(); QBNScheme.reset()
         config.share_grad_sqnorm = share
@@ -506,7 +510,11 @@ def test_batch_norm_backward_hands_the_gradient_norm_to_the_convolution(channels
         return conv.scheme.scales, grads
     s0, g0 = run(False)
     s1, g1 = run(True)
-    assert all(torch.equal(a, b) for a, b in zip(g0, g1))
+    assert torch.equal(g0[2], g1[2])                # batch norm's own weight gradient: same kernels, same bits
+    for a, b in zip(g0[:2], g1[:2]):                # through MIOpen's convolution backward, whose split-K
+        a, b = a.float(), b.float()                 # kernels add in no fixed order before the result is
+        bound = 2.0 ** -7 * torch.maximum(a.abs(), b.abs()) + 1e-3 * a.abs().max()    # rounded to bf16
+        assert ((a - b).abs() <= bound).all()
     s0, s1 = float(s0), float(s1)
     assert s0 > 0 and abs(s0 - s1) <= 1e-5 * s0
     # the statistic really came from the hand-off: without the attribute set_scale reduces itself
