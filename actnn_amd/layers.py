@@ -218,6 +218,30 @@ class QBatchNorm3d(_QBatchNormMixin, nn.BatchNorm3d):
         self._init_scheme(group)
 
 
+class QSyncBatchNorm(_QBatchNormMixin, nn.SyncBatchNorm):
+    """nn.SyncBatchNorm with a compressed saved input (layers.py:383-462).  The statistics of one
+    process need no exchange, and that is the case built here: without an initialised process
+    group, or in a group of one rank, the layer is QBatchNorm on its own batch - the path the
+    reference takes for world_size == 1 (layers.py:444-455).  Across ranks the reference gathers
+    [mean, invstd, count] and reduces the two gradient sums (ops.py:519-526,585-588); this build
+    runs on one GPU and raises instead of normalising with local statistics only."""
+
+    def __init__(self, num_features, eps=1e-05, momentum=0.1, affine=True, track_running_stats=True,
+                 process_group=None, group=0):
+        super().__init__(num_features, eps, momentum, affine, track_running_stats, process_group)
+        self._init_scheme(group)
+
+    def forward(self, input):
+        if not input.is_cuda:
+            raise ValueError("SyncBatchNorm expected input tensor to be on GPU")
+        uses_batch_statistics = self.training or (self.running_mean is None and self.running_var is None)
+        if uses_batch_statistics and torch.distributed.is_available() and torch.distributed.is_initialized():
+            group = self.process_group or torch.distributed.group.WORLD
+            if torch.distributed.get_world_size(group) > 1:
+                raise NotImplementedError("QSyncBatchNorm across ranks is not part of this single-GPU build")
+        return super().forward(input)
+
+
 class QReLU(nn.Module):
     """ReLU that saves a 1-bit mask; used in training and evaluation alike (layers.py:364-369)."""
 

@@ -8,10 +8,10 @@ import torch.nn as nn
 from .conf import config
 from .layers import (QAvgPool2d, QBatchNorm1d, QBatchNorm2d, QBatchNorm3d, QConv1d, QConv2d, QConv3d,
                      QConvTranspose1d, QConvTranspose2d, QConvTranspose3d, QDropout, QLinear, QMaxPool2d,
-                     QReLU)
+                     QReLU, QSyncBatchNorm)
 
-_Q_TYPES = (QConv1d, QConv2d, QConv3d, QConvTranspose1d, QConvTranspose2d, QConvTranspose3d, QBatchNorm1d, QBatchNorm2d, QBatchNorm3d, QReLU, QDropout,
-            QLinear, QMaxPool2d, QAvgPool2d)
+_Q_TYPES = (QConv1d, QConv2d, QConv3d, QConvTranspose1d, QConvTranspose2d, QConvTranspose3d, QBatchNorm1d,
+            QBatchNorm2d, QBatchNorm3d, QSyncBatchNorm, QReLU, QDropout, QLinear, QMaxPool2d, QAvgPool2d)
 
 
 def _convert(child):

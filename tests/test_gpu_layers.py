@@ -575,3 +575,37 @@ def test_per_sample_gradient_statistics_with_the_index_yielding_loader():
         + 0.5 * grads["last"].double().flatten(1).square().sum(1)
     assert torch.allclose(last.scales[torch.tensor(QScheme.batch, device=DEV)].double(), want, rtol=1e-5, atol=0)
     assert int(last.b.min()) >= 1 and int(last.b.sum()) <= int(last.bits * 16) and len(set(last.b.tolist())) > 1
+
+
+def test_sync_batch_norm_of_one_process_is_batch_norm(monkeypatch):
+    """QSyncBatchNorm without peers (no process group, or a group of one rank) takes the path of
+    QBatchNorm2d (layers.py:444-455): same output, gradients and saved stream; with peers it
+    refuses, since the statistics exchange is not part of this build."""
+    import torch.distributed as dist
+    def run(cls):
+        config.reset(); QScheme.reset(); QBNScheme.reset()
+        torch.manual_seed(0)
+        bn = cls(64).to(DEV)
+        x = torch.randn(8, 64, 16, 16, device=DEV, requires_grad=True)
+        torch.cuda.manual_seed(3)
+        y = bn(x)
+        saved = y.grad_fn.saved[0]
+        grads = torch.autograd.grad(y, [x, bn.weight, bn.bias], torch.ones_like(y) * x.detach())
+        return y, saved, grads, bn
+    y0, s0, g0, _ = run(actnn_amd.QBatchNorm2d)
+    y1, s1, g1, bn = run(actnn_amd.QSyncBatchNorm)
+    assert torch.equal(y0, y1) and all(torch.equal(a, b) for a, b in zip(g0, g1))
+    assert all(torch.equal(a, b) for a, b in zip(s0, s1))
+    assert int(bn.num_batches_tracked) == 1 and isinstance(bn, nn.SyncBatchNorm)
+    with pytest.raises(ValueError):
+        bn(torch.randn(8, 64, 4, 4))                                   # host tensor, as the reference
+    bn.eval()
+    assert torch.allclose(bn(y0.detach()), F.batch_norm(y0.detach(), bn.running_mean, bn.running_var,
+                                                        bn.weight, bn.bias, False, 0.1, bn.eps), atol=1e-5)
+    bn.train()
+    monkeypatch.setattr(dist, "is_initialized", lambda: True)
+    monkeypatch.setattr(dist, "get_world_size", lambda group=None: 1)
+    assert torch.equal(bn(y0.detach()), actnn_amd.QSyncBatchNorm(64).to(DEV)(y0.detach()))
+    monkeypatch.setattr(dist, "get_world_size", lambda group=None: 2)
+    with pytest.raises(NotImplementedError):
+        bn(y0.detach())
