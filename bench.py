@@ -135,6 +135,12 @@ def other_configs(device, reps):
     out["relu_forward_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
     t = _event_time_ms(lambda: ext_q.relu_backward(g, mask), reps)
     out["relu_backward_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
+    _, keep = ext_q.dropout_forward(x, 0.25)
+    t = _event_time_ms(lambda: ext_q.dropout_forward(x, 0.25), reps)
+    out["dropout_forward_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
+    t = _event_time_ms(lambda: ext_q.dropout_backward(g, keep, 0.25), reps)
+    out["dropout_backward_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
+    del keep
     k, s, p = (3, 3), (2, 2), (1, 1)
     yp, idx = ext_q.max_pool2d_forward(x, k, s, p, (1, 1))
     gp = torch.randn_like(yp)
