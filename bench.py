@@ -236,10 +236,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the config-2 hot path")
-    ap.add_argument("--only", choices=["other", "resnet50", "resnet50_channels_last", "batch_norm_shapes"],
+    ap.add_argument("--only", choices=["other", "resnet50", "resnet50_channels_last", "resnet50_fp32", "batch_norm_shapes"],
                     default=None,
                     help="profiling aid: run just the other single-GPU configs (ReLU, max-pool, "
-                         "fixed-width pack, fused GEMM), just the ResNet-50 L3 step, or the fused "
+                         "fixed-width pack, fused GEMM), just the ResNet-50 L3 step, the fp32 "
+                         "(no autocast) ResNet-50 pair of the reference's own protocol, or the fused "
                          "batch-norm passes on every batch-norm shape of ResNet-50; print their JSON")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -265,6 +266,17 @@ def main():
         from actnn_amd import bench_extra
         print(json.dumps({"resnet50_L3_channels_last": bench_extra.resnet50_step(
             device, "L3", warmup=2, steps=3, channels_last=True)}))
+        return
+    if args.only == "resnet50_fp32":
+        from actnn_amd import bench_extra
+        out = {}
+        for key, level, cl in (("resnet50_fp32_exact", "exact", False), ("resnet50_fp32_L3", "L3", False),
+                               ("resnet50_fp32_exact_channels_last", "exact", True),
+                               ("resnet50_fp32_L3_channels_last", "L3", True)):
+            torch.cuda.empty_cache()
+            torch.cuda.reset_peak_memory_stats()
+            out[key] = bench_extra.resnet50_step(device, level, warmup=2, steps=5, autocast=False, channels_last=cl)
+        print(json.dumps(out))
         return
     if args.only == "batch_norm_shapes":
         from actnn_amd import bench_extra
