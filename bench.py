@@ -236,11 +236,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the config-2 hot path")
-    ap.add_argument("--only", choices=["other", "resnet50", "resnet50_channels_last", "resnet50_fp32", "batch_norm_shapes"],
+    ap.add_argument("--only", choices=["other", "resnet50", "resnet50_channels_last", "resnet50_fp32", "resnet50_levels", "batch_norm_shapes"],
                     default=None,
                     help="profiling aid: run just the other single-GPU configs (ReLU, max-pool, "
                          "fixed-width pack, fused GEMM), just the ResNet-50 L3 step, the fp32 "
-                         "(no autocast) ResNet-50 pair of the reference's own protocol, or the fused "
+                         "(no autocast) ResNet-50 pair of the reference's own protocol, every "
+                         "optimisation level (channels-last, bf16), or the fused "
                          "batch-norm passes on every batch-norm shape of ResNet-50; print their JSON")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -276,6 +277,16 @@ def main():
             torch.cuda.empty_cache()
             torch.cuda.reset_peak_memory_stats()
             out[key] = bench_extra.resnet50_step(device, level, warmup=2, steps=5, autocast=False, channels_last=cl)
+        print(json.dumps(out))
+        return
+    if args.only == "resnet50_levels":
+        from actnn_amd import bench_extra
+        out = {}
+        for level in ("exact", "L0", "L1", "L2", "L3", "L3.1", "L4", "swap"):
+            torch.cuda.empty_cache()
+            torch.cuda.reset_peak_memory_stats()
+            out["resnet50_" + level] = bench_extra.resnet50_step(device, level, warmup=2, steps=5, channels_last=True)
+            print("[bench] %s done" % level, file=sys.stderr, flush=True)
         print(json.dumps(out))
         return
     if args.only == "batch_norm_shapes":
