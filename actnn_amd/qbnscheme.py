@@ -1,7 +1,5 @@
 """Bit allocation for batch-norm inputs (behaviour of actnn/actnn/qbnscheme.py:9-60): the
 sensitivity is the range term alone and the per-layer budget follows the preceding conv/linear."""
-import torch
-
 from .conf import config
 from .qscheme import (PendingBits, QScheme, allocate_bits_on_device, allocate_on_device, greedy_bits,
                       group_min_max, range_sqr)

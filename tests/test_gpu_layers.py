@@ -1,8 +1,6 @@
 """Layer-level behaviour on the GPU: the compressed autograd functions against stock torch layers
 (the reference checks the same things in tests/test_act_quantized_ops.py:318-447 and
 tests/test_linear.py)."""
-import copy
-
 import pytest
 import torch
 import torch.nn as nn
