@@ -53,10 +53,15 @@ class PendingBits:
     waits for the event only - so the GPU keeps working during the round trip instead of idling
     as it does with the reference's blocking `.cpu()` (qscheme.py:83-85)."""
 
-    def __init__(self, C_dev):
-        self.host = torch.empty(C_dev.shape, dtype=torch.float32, pin_memory=True)
+    def __init__(self, C_dev, previous=None):
+        # `previous`: the same layer's object of the step before, whose pinned buffer and event are
+        # taken over (its values were picked up at the end of that step, or never will be)
+        if previous is not None and previous.host.shape == C_dev.shape:
+            self.host, self.event = previous.host, previous.event
+        else:
+            self.host = torch.empty(C_dev.shape, dtype=torch.float32, pin_memory=True)
+            self.event = torch.cuda.Event()
         self.host.copy_(C_dev if C_dev.dtype == torch.float32 else C_dev.to(torch.float32), non_blocking=True)
-        self.event = torch.cuda.Event()
         self.event.record()
 
     def wait(self):
@@ -222,7 +227,7 @@ class QScheme(_LazyHost):
                 self.initial_bits, self.bits)
         else:
             C_dev = self.sensitivity(mn, mx, N, num_pixels)
-        pending = PendingBits(C_dev)
+        pending = self._last_pending = PendingBits(C_dev, getattr(self, "_last_pending", None))
         return groups, mn, mx, pending, input.numel() // N, bits_dev
 
     def finish_quantization_bits(self, started):
@@ -271,15 +276,14 @@ class QScheme(_LazyHost):
     def if_allocate_perlayer(self):
         """Called at the end of every layer's backward; the layer whose backward runs last (the
         first one with a trainable weight) triggers the re-balancing (qscheme.py:130-147)."""
-        if not config.perlayer:
-            return
-        if any(l.C is None for l in QScheme.layers):
+        if not (config.perlayer and config.compress_activation and config.training):
             return
         first = next((l for l in QScheme.layers if l.layer.weight.requires_grad), None)
-        if config.compress_activation and config.training and self is first:
-            from .qbnscheme import QBNScheme
-            QScheme.allocate_perlayer()
-            QBNScheme.allocate_perlayer()
+        if self is not first or any(l.C is None for l in QScheme.layers):
+            return
+        from .qbnscheme import QBNScheme
+        QScheme.allocate_perlayer()
+        QBNScheme.allocate_perlayer()
 
     @staticmethod
     def reset():
