@@ -27,6 +27,7 @@ SIGNATURES = {
     "actnn_strerror": [c_i32],
     "actnn_version": [],
     "actnn_minimax": [c_vp, c_vp, c_vp, c_i64, c_i64, c_i32, c_vp],
+    "actnn_calc_precision_dp": [c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_vp, c_vp],
     "actnn_calc_precision_device": [c_vp, c_vp, c_i64, c_i32, c_i64, c_vp],
     "actnn_range_sqr": [c_vp, c_vp, c_vp, c_i64, c_i64, ctypes.c_float, c_vp, c_i32, c_i32, c_vp],
     "actnn_sample_sqnorm": [c_vp, c_vp, c_i64, c_i64, c_i32, c_i32, c_vp],

@@ -1,6 +1,8 @@
 """``calc_precision(b, C, w, target) -> b``: greedy bit allocation on CPU tensors; ``b`` is
 modified in place and returned (reference: cpp_extension/calc_precision.cc:9-50).
-``calc_precision_dp`` of the reference has no Python caller and is not provided.
+``calc_precision_dp(A, C, max_b, target, states) -> (b, p)``: the reference's second export
+(calc_precision.cc:58-125, no caller in its Python), a dynamic programme over widths and keep
+probabilities.
 ``calc_precision_device`` runs the same allocation on the GPU for uniform start widths and unit
 weights (what every layer asks for at every step), so that no host round trip is needed."""
 import torch
@@ -22,6 +24,24 @@ def calc_precision(b, C, w, target):
     check(g.lib().actnn_calc_precision(b.data_ptr(), C.data_ptr(), w.data_ptr(), b.numel(),
                                        float(target)), "calc_precision")
     return b
+
+
+def calc_precision_dp(A, C, max_b, target, states):
+    for t, name in ((A, "A"), (C, "C")):
+        if not (isinstance(t, torch.Tensor) and t.device.type == "cpu"):
+            raise RuntimeError(f"{name} must be a CPU tensor!")           # calc_precision.cc:61-64
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous!")
+    if A.dtype != torch.float32 or C.dtype != torch.float32 or A.numel() != C.numel():
+        raise RuntimeError("calc_precision_dp expects A and C as float32 of the same length")
+    b_vec, p_vec = torch.zeros_like(A), torch.zeros_like(A)
+    rc = g.lib().actnn_calc_precision_dp(A.data_ptr(), C.data_ptr(), A.numel(), int(max_b), int(target),
+                                         int(states), b_vec.data_ptr(), p_vec.data_ptr())
+    if rc != 0:
+        raise RuntimeError("DP Failed: no path to initial state!" if A.numel() and 0 < int(max_b) <= 30
+                           and 0 < int(states) and int(max_b) * int(states) <= 255 and int(target) >= 0
+                           else "calc_precision_dp: argument out of range")
+    return b_vec, p_vec
 
 
 DEVICE_MAX_CANDIDATES = 8192

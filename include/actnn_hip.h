@@ -163,6 +163,14 @@ int actnn_max_pool2d_backward_cl(const void* grad_out, const int8_t* idx, void* 
  * ------------------------------------------------------------------------------- */
 int actnn_calc_precision(int32_t* b, const float* C, const int32_t* w, int64_t N, double target);
 
+/* calc_precision_dp (HOST pointers): widths b_i in 1..max_b and keep probabilities p_i in
+ * {1/states..1} minimising sum (1-p_i)/p_i*A_i + C_i/(p_i*(2^b_i-1)^2) with
+ * sum b_i*p_i*states == target*N*states, by dynamic programming; b_out, p_out: fp32[N].
+ * ACTNN_EINVAL when no assignment meets the budget (the reference raises "DP Failed").
+ * Replaces calc_precision_dp(A, C, max_b, target, states): calc_precision.cc:58-125. */
+int actnn_calc_precision_dp(const float* A, const float* C, int64_t N, int max_b, int target,
+                            int states, float* b_out, float* p_out);
+
 /* Squared L2 norm per sample of x[N, F] (the per-sample gradient statistic of the bit allocation,
  * qscheme.py:47-55, where the reference chains square / sum over a full-size temporary):
  * part[n * slices + b] = sum of squares of slice b of row n (fp32, fixed order); the caller adds the

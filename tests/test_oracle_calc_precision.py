@@ -80,3 +80,68 @@ def test_against_compiled_reference():
         target = float(rng.uniform(1.0, 8.0) * w.sum())
         got = ref.calc_precision(torch.from_numpy(b0.copy()), torch.from_numpy(C), torch.from_numpy(w), target)
         assert np.array_equal(got.numpy(), cp.calc_precision(b0, C, w, target))
+
+
+# ------------------------------------------------------------------------------------------
+# calc_precision_dp (calc_precision.cc:58-125)
+# ------------------------------------------------------------------------------------------
+def _dp_inputs(rng, N):
+    A = rng.lognormal(0, 1, N).astype(np.float32)
+    C = rng.lognormal(1, 2, N).astype(np.float32)
+    return A, C
+
+
+def test_dp_restatement_is_optimal_on_tiny_inputs():
+    """The objective is separable and the budget an equality: brute force over every (b, p)
+    assignment gives the same minimum (float64 objective of the float32 DP's choice)."""
+    rng = np.random.default_rng(3)
+    for N, max_b, target, states in ((3, 3, 2, 2), (4, 2, 1, 2), (2, 4, 3, 1), (3, 2, 2, 3)):
+        A, C = _dp_inputs(rng, N)
+        b, p = cp.calc_precision_dp(A, C, max_b, target, states)
+        assert np.isclose(sum(b * p * states), target * N * states)
+        assert ((b >= 1) & (b <= max_b) & (p > 0) & (p <= 1)).all()
+        best = cp.dp_brute_force(A, C, max_b, target, states)
+        assert cp.dp_objective(b, p, A, C) <= best * (1 + 1e-5)
+
+
+def test_dp_known_cases():
+    # one state, budget = max_b: every item keeps all its bits, p = 1
+    b, p = cp.calc_precision_dp(np.ones(5, np.float32), np.ones(5, np.float32), 4, 4, 1)
+    assert (b == 4).all() and (p == 1).all()
+    # budget of one unit per item and state: the only way is b = 1, p = 1/states ... or b*p = states
+    b, p = cp.calc_precision_dp(np.zeros(3, np.float32), np.array([1, 100, 1], np.float32), 2, 1, 1)
+    assert (b == 1).all() and (p == 1).all()
+    # an unreachable budget fails like the reference's TORCH_CHECK
+    with pytest.raises(ValueError):
+        cp.calc_precision_dp(np.ones(2, np.float32), np.ones(2, np.float32), 1, 3, 1)
+
+
+def test_dp_library_routine_matches_the_restatement_and_the_compiled_reference():
+    import actnn_amd.cpp_extension.calc_precision as ext
+    ref = build_ref.load()
+    rng = np.random.default_rng(11)
+    for trial in range(12):
+        N = int(rng.integers(1, 24))
+        max_b, target, states = int(rng.integers(1, 5)), int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        A, C = _dp_inputs(rng, N)
+        if trial % 4 == 0:
+            C[rng.random(N) < 0.4] = 0.0                  # equal costs: the tie rule decides
+        if target > max_b:                                # no assignment can spend that much
+            with pytest.raises(RuntimeError):
+                ext.calc_precision_dp(torch.from_numpy(A), torch.from_numpy(C), max_b, target, states)
+            continue
+        want_b, want_p = cp.calc_precision_dp(A, C, max_b, target, states)
+        got_b, got_p = ext.calc_precision_dp(torch.from_numpy(A), torch.from_numpy(C), max_b, target, states)
+        assert np.array_equal(got_b.numpy(), want_b) and np.array_equal(got_p.numpy(), want_p)
+        if ref is not None:
+            ref_b, ref_p = ref.calc_precision_dp(torch.from_numpy(A), torch.from_numpy(C), max_b, target, states)
+            assert np.array_equal(ref_b.numpy(), want_b) and np.array_equal(ref_p.numpy(), want_p)
+    with pytest.raises(RuntimeError):
+        ext.calc_precision_dp(torch.ones(3, dtype=torch.float64), torch.ones(3), 2, 1, 1)
+    # the reference's own sizing (N = 128, b = 2, s = 2: calc_precision.cc:73) in well under a second
+    A, C = _dp_inputs(rng, 128)
+    got_b, got_p = ext.calc_precision_dp(torch.from_numpy(A), torch.from_numpy(C), 8, 2, 2)
+    assert float((got_b * got_p * 2).sum()) == 2 * 128 * 2
+    if ref is not None:
+        ref_b, ref_p = ref.calc_precision_dp(torch.from_numpy(A), torch.from_numpy(C), 8, 2, 2)
+        assert torch.equal(ref_b, got_b) and torch.equal(ref_p, got_p)
