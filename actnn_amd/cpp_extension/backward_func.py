@@ -326,3 +326,48 @@ def native_batch_norm_backward(grad_out, input, weight, running_mean, running_va
     """at::native_batch_norm_backward (backward_func.cc:90)."""
     return _aten.native_batch_norm_backward(grad_out, input, weight, running_mean, running_var,
                                             save_mean, save_invstd, train, eps, list(output_mask))
+
+
+def prepare_layer_norm_inputs(input, normalized_shape, weight, bias):
+    """-> (X, gamma, beta, M, N): contiguous operands and the [M, N] geometry of a layer norm
+    over the trailing `normalized_shape` (backward_func.cc:14-72, re-exported at :83; no caller
+    in the reference's Python)."""
+    normalized_shape = tuple(int(d) for d in normalized_shape)
+    if len(normalized_shape) < 1:
+        raise RuntimeError("Expected normalized_shape to be at least 1-dimensional")
+    for t, name in ((weight, "weight"), (bias, "bias")):
+        if t is not None and tuple(t.shape) != normalized_shape:
+            raise RuntimeError(f"Expected {name} to be of same shape as normalized_shape, but got {name} of "
+                               f"shape {tuple(t.shape)} and normalized_shape = {normalized_shape}")
+    lead = input.dim() - len(normalized_shape)
+    if lead < 0 or tuple(input.shape[lead:]) != normalized_shape:
+        raise RuntimeError(f"Given normalized_shape={normalized_shape}, expected input with shape "
+                           f"[*, {', '.join(map(str, normalized_shape))}], but got input of size {tuple(input.shape)}")
+    M = 1
+    for d in input.shape[:lead]:
+        M *= d
+    N = 1
+    for d in normalized_shape:
+        N *= d
+    return (input.contiguous(), None if weight is None else weight.contiguous(),
+            None if bias is None else bias.contiguous(), M, N)
+
+
+def layer_norm_cuda(X, gamma, beta, M, N, eps):
+    """-> (Y, mean [M], rstd [M]) of the [M, N] problem (at::native::layer_norm_cuda,
+    backward_func.cc:84); ATen's kernel through its current name."""
+    Y, mean, rstd = _aten.native_layer_norm(X.reshape(M, N), [N], None if gamma is None else gamma.reshape(N),
+                                            None if beta is None else beta.reshape(N), eps)
+    return Y.view_as(X), mean.reshape(M), rstd.reshape(M)
+
+
+def layer_norm_backward_cuda(dY, X, mean, rstd, gamma, M, N, grad_input_mask):
+    """-> (dX, dgamma, dbeta) (at::native::layer_norm_backward_cuda, backward_func.cc:85)."""
+    flat = None if gamma is None else gamma.reshape(N)
+    # ATen's current entry also takes the bias, of which only the shape matters: gamma stands in
+    dX, dgamma, dbeta = _aten.native_layer_norm_backward(
+        dY.reshape(M, N), X.reshape(M, N), [N], mean.reshape(M, 1), rstd.reshape(M, 1), flat, flat,
+        list(grad_input_mask))
+    shape = None if gamma is None else gamma.shape
+    return (None if dX is None else dX.view_as(X), None if dgamma is None or shape is None else dgamma.view(shape),
+            None if dbeta is None or shape is None else dbeta.view(shape))

@@ -607,3 +607,28 @@ def test_sync_batch_norm_of_one_process_is_batch_norm(monkeypatch):
     monkeypatch.setattr(dist, "get_world_size", lambda group=None: 2)
     with pytest.raises(NotImplementedError):
         bn(y0.detach())
+
+
+def test_layer_norm_re_exports_against_torch():
+    """backward_func's three layer-norm names (backward_func.cc:83-85) against F.layer_norm and
+    autograd."""
+    import actnn_amd.cpp_extension.backward_func as ext_bf
+    torch.manual_seed(0)
+    x = torch.randn(6, 5, 32, 8, device=DEV, requires_grad=True)
+    w = (torch.rand(32, 8, device=DEV) + 0.5).requires_grad_(True)
+    b = torch.randn(32, 8, device=DEV, requires_grad=True)
+    X, gamma, beta, M, N = ext_bf.prepare_layer_norm_inputs(x.detach(), (32, 8), w.detach(), b.detach())
+    assert (M, N) == (30, 256)
+    Y, mean, rstd = ext_bf.layer_norm_cuda(X, gamma, beta, M, N, 1e-5)
+    ref = F.layer_norm(x, (32, 8), w, b, 1e-5)
+    assert torch.allclose(Y, ref, atol=1e-5)
+    assert torch.allclose(mean, x.detach().reshape(30, 256).mean(1), atol=1e-5)
+    dY = torch.randn_like(ref)
+    gx, gw, gb = torch.autograd.grad(ref, [x, w, b], dY)
+    dX, dgamma, dbeta = ext_bf.layer_norm_backward_cuda(dY, X, mean, rstd, gamma, M, N, [True, True, True])
+    assert torch.allclose(dX, gx, atol=1e-4) and torch.allclose(dgamma, gw, atol=1e-4)
+    assert torch.allclose(dbeta, gb, atol=1e-4)
+    with pytest.raises(RuntimeError):
+        ext_bf.prepare_layer_norm_inputs(x.detach(), (8,), w.detach(), None)      # weight shape
+    with pytest.raises(RuntimeError):
+        ext_bf.prepare_layer_norm_inputs(x.detach(), (16, 8), None, None)         # trailing dims
