@@ -482,3 +482,20 @@ class batch_norm(Function):
         if ctx.scheme:
             ctx.scheme.if_allocate_perlayer()
         return grad_input, None, None, grad_weight, grad_bias, None, None, None, None
+
+
+class adaptive_avg_pool2d(Function):
+    """Global average pool that keeps only the input's shape for the backward pass
+    (ops.py:617-629); output size (1, 1) only, as there."""
+
+    @staticmethod
+    def forward(ctx, input, output_size):
+        if tuple(output_size) != (1, 1):
+            raise AssertionError("adaptive_avg_pool2d supports output_size (1, 1) only")
+        ctx.saved = input.shape
+        return torch.mean(input, dim=[2, 3], keepdim=True)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        shape = ctx.saved
+        return (grad_output / (shape[2] * shape[3])).expand(shape), None

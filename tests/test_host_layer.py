@@ -134,3 +134,18 @@ def test_perlayer_allocation_on_host():
     b1 = QBNScheme()
     QBNScheme.allocate_perlayer()
     assert float(b1.bits) == bits[2]              # BN copies the preceding layer's budget
+
+
+def test_adaptive_avg_pool2d_keeps_only_the_shape():
+    import torch.nn.functional as F
+    from actnn_amd.ops import adaptive_avg_pool2d
+    x = torch.randn(3, 5, 7, 4, dtype=torch.float64, requires_grad=True)
+    y = adaptive_avg_pool2d.apply(x, (1, 1))
+    ref = F.adaptive_avg_pool2d(x, (1, 1))
+    assert torch.allclose(y, ref)
+    g = torch.randn_like(ref)
+    (gx,) = torch.autograd.grad(y, x, g)
+    (gr,) = torch.autograd.grad(ref, x, g)
+    assert torch.allclose(gx, gr) and y.grad_fn.saved == x.shape
+    with pytest.raises(AssertionError):
+        adaptive_avg_pool2d.apply(x, (2, 2))
