@@ -1,7 +1,9 @@
 """Autograd functions that keep their input compressed between forward and backward, and the
 quantise / dequantise glue around the kernels (behaviour of the reference's
-actnn/actnn/ops.py:22-502; sync-BN and adaptive pooling variants are not part of this build).
+actnn/actnn/ops.py:22-629; sync_batch_norm across ranks is not part of this build).
 """
+import functools
+
 import numpy as np
 import torch
 import torch.nn.functional as F
@@ -395,11 +397,24 @@ def _bn_shares_min_max(input, weight, bias, running_mean, running_var, training)
             and ext_backward_func.hip_batch_norm_minmax_applies(input, weight, bias, running_mean, running_var))
 
 
+@functools.lru_cache(maxsize=64)
+def _uniform_bits(N, bits, device):
+    """int32 [N] on `device`, every sample `bits` wide, with its sum and prefix attached: the
+    fixed-width schemes as a special case of the per-sample stream the fused kernels write."""
+    q_bits = torch.full((N,), bits, dtype=torch.int32, device=device)
+    ext_quantization.attach_bits_host(q_bits, torch.full((N,), bits, dtype=torch.int32))
+    ext_quantization._bits_info(q_bits)
+    return q_bits
+
+
 class batch_norm(Function):
     @staticmethod
     def forward(ctx, input, running_mean, running_var, weight, bias, training,
                 exponential_average_factor, eps, scheme):
-        if (scheme and config.fused_bn_pack
+        fixed_width = (not scheme and config.compress_activation and not config.simulate
+                       and isinstance(config.activation_compression_bits[0], int)
+                       and 1 <= config.activation_compression_bits[0] <= 8)
+        if ((scheme or fixed_width) and config.fused_bn_pack
                 and _bn_shares_min_max(input, weight, bias, running_mean, running_var, training)
                 and ext_backward_func.hip_batch_norm_pack_applies(input, weight, bias, running_mean, running_var)):
             # two reads of the input in total: the statistics pass also yields the quantiser's
@@ -407,8 +422,14 @@ class batch_norm(Function):
             # writes the packed copy of the input next to the output
             ws, save_mean, save_var, mn, mx = ext_backward_func.hip_batch_norm_forward_stats(
                 input, weight, bias, running_mean, running_var, exponential_average_factor, eps)
-            _, q_bits, q_min, q_max = scheme.finish_quantization_bits(
-                scheme.start_quantization_bits(input, (mn, mx)))
+            if scheme:
+                _, q_bits, q_min, q_max = scheme.finish_quantization_bits(
+                    scheme.start_quantization_bits(input, (mn, mx)))
+            else:
+                # no per-sample allocation (levels L1/L2): the same stream at one width for all
+                N = input.shape[0]
+                q_bits = _uniform_bits(N, config.activation_compression_bits[0], input.device)
+                q_min, q_max = mn.view(N, -1, 1), mx.view(N, -1, 1)
             output, q_input, q_scale = ext_backward_func.hip_batch_norm_forward_apply(
                 input, ws, q_bits, q_min, q_max)
             if config.swap:

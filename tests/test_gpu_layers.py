@@ -632,3 +632,50 @@ def test_layer_norm_re_exports_against_torch():
         ext_bf.prepare_layer_norm_inputs(x.detach(), (8,), w.detach(), None)      # weight shape
     with pytest.raises(RuntimeError):
         ext_bf.prepare_layer_norm_inputs(x.detach(), (16, 8), None, None)         # trailing dims
+
+
+@pytest.mark.parametrize("channels_last", [False, True])
+def test_fixed_width_batch_norm_takes_the_fused_passes(channels_last):
+    """Levels without per-sample allocation (L2: 4 bits everywhere, no scheme): batch norm still
+    writes the packed copy of its input in its normalising pass - the per-sample stream at one
+    width - and reads it back in the backward kernels.  Output identical to the unfused sequence,
+    saved input within one quantisation step, gradients those of the dequantised input."""
+    def run(fused):
+        config.reset(); QScheme.reset(); QBNScheme.reset()
+        set_optimization_level("L2")
+        config.fused_bn_pack = fused
+        config.fused_bn_backward = fused
+        torch.manual_seed(0)
+        bn = actnn_amd.QBatchNorm2d(64).to(DEV)
+        assert bn.scheme is None
+        x = torch.randn(16, 64, 14, 14, device=DEV).bfloat16()
+        if channels_last:
+            bn = bn.to(memory_format=torch.channels_last)
+            x = x.contiguous(memory_format=torch.channels_last)
+        x.requires_grad_(True)
+        torch.cuda.manual_seed(2)
+        y = bn(x)
+        quantized, _, _, _, save_mean, save_invstd = y.grad_fn.saved[:6]
+        back = dequantize_activation(quantized, x.shape)
+        g = torch.randn_like(y)
+        grads = torch.autograd.grad(y, [x, bn.weight, bn.bias], g)
+        return x, y, quantized, back, g, grads, (bn.weight.detach(), save_mean, save_invstd)
+    x, y1, q1, back1, g, grads1, stats = run(True)
+    _, y0, q0, back0, _, grads0, _ = run(False)
+    assert isinstance(q1[1], torch.Tensor) and q1[1].tolist() == [4] * 16 and isinstance(q0[1], int)
+    assert q1[0].numel() * 4 == x.numel() * 4 // 8                       # int32 words: 4 bits per element
+    assert torch.equal(y0, y1)
+    span = (x.detach().float().max() - x.detach().float().min()).item()
+    for back in (back0, back1):
+        assert back.shape == x.shape and (back.float() - x.detach().float()).abs().max().item() <= span / 15 + 0.05
+    # the backward kernels rebuild x exactly as the unpack kernel does: same gradients, bit for bit,
+    # as the plain backward pass on the dequantised tensor
+    import actnn_amd.cpp_extension.backward_func as ext_bf
+    want = ext_bf.hip_batch_norm_backward(back1, g, *stats)
+    assert all(torch.equal(a, b) for a, b in zip(grads1, want))
+    assert torch.equal(grads1[2], grads0[2])                             # the bias gradient never sees x
+    # and the quantisation noise is unbiased: the input gradient stays close to the exact layer's
+    ref = nn.BatchNorm2d(64).to(DEV)
+    xr = x.detach().float().requires_grad_(True)
+    (gx,) = torch.autograd.grad(ref(xr), xr, g.float())
+    assert (grads1[0].float() - gx).abs().max() <= 0.05 * gx.abs().max() + 0.05
