@@ -9,8 +9,7 @@ import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
-# ACTNN_HIP_LIB points at another build of the same library (kernel tuning experiments)
-LIB_PATH = os.environ.get("ACTNN_HIP_LIB") or os.path.join(_HERE, "libactnn_hip.so")
+LIB_PATH = os.path.join(_HERE, "libactnn_hip.so")
 SOURCES = ["minimax.hip", "pack_mixed.hip", "pack_single.hip", "mask_ops.hip", "maxpool.hip",
            "linear_gw.hip", "misc.hip", "calc_precision.cpp", "calc_precision_dev.hip", "batch_norm.hip"]
 HIPCC_FLAGS = [

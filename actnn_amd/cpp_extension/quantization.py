@@ -18,26 +18,40 @@ MASK_BLOCK = 512
 # ------------------------------------------------------------------------------------------
 def attach_bits_host(bits_dev, bits_host):
     """Remember the host copy of a device ``bits`` tensor so that pack/unpack need no
-    device->host sync (the reference syncs twice per pack: .cu:92, :98)."""
-    bits_dev._actnn_host = bits_host
+    device->host sync (the reference syncs twice per pack: .cu:92, :98).  The hand-off is tied to
+    the tensor's version counter: after an in-place change of ``bits_dev`` it is ignored."""
+    bits_dev._actnn_host = (bits_dev._version, bits_host)
+    bits_dev._actnn_info = None
     return bits_dev
 
 
-def attach_bits_total(bits_dev, total):
+def attach_bits_total(bits_dev, total, prefix=None):
     """For widths computed on the device (no host copy): remember their sum, which the caller
-    knows from the budget, so that the packed stream can be sized without a sync."""
-    bits_dev._actnn_total = int(total)
+    knows from the budget, so that the packed stream can be sized without a sync; `prefix` is the
+    device exclusive prefix sum [N+1] when the caller has it already."""
+    bits_dev._actnn_total = (bits_dev._version, int(total))
+    bits_dev._actnn_info = None if prefix is None else (bits_dev._version, int(total), prefix)
     return bits_dev
+
+
+def _fresh(bits, name):
+    """Value attached to `bits` under `name`, or None when `bits` has been written since."""
+    tagged = getattr(bits, name, None)
+    if tagged is None or tagged[0] != bits._version:
+        return None
+    return tagged[1] if len(tagged) == 2 else tagged[1:]
 
 
 def _bits_info(bits):
-    """(sum(bits), device exclusive prefix [N+1]) of an int32 device tensor, cached on it."""
-    cached = getattr(bits, "_actnn_info", None)
+    """(sum(bits), device exclusive prefix [N+1]) of an int32 device tensor, cached on it together
+    with the tensor's version counter: an in-place change of `bits` invalidates the cache (and the
+    attached host copy / total), and the widths are then read back and range-checked again."""
+    cached = _fresh(bits, "_actnn_info")
     if cached is not None:
         return cached
-    total = getattr(bits, "_actnn_total", None)        # widths made on the device: only their sum is known
+    total = _fresh(bits, "_actnn_total")               # widths made on the device: only their sum is known
     if total is None:
-        host = getattr(bits, "_actnn_host", None)
+        host = _fresh(bits, "_actnn_host")
         if host is None:
             host = bits.cpu()                          # sync, like the reference's .item() calls
         if host.numel() and (int(host.min()) < 1 or int(host.max()) > 8):
@@ -48,8 +62,8 @@ def _bits_info(bits):
     with g.on_device(bits.device):
         check(g.lib().actnn_bits_prefix(bits.data_ptr(), prefix.data_ptr(), N,
                                         g.stream_ptr(bits.device)), "bits_prefix")
-    bits._actnn_info = (total, prefix)
-    return bits._actnn_info
+    bits._actnn_info = (bits._version, total, prefix)
+    return total, prefix
 
 
 # ------------------------------------------------------------------------------------------

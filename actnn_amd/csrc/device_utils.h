@@ -59,32 +59,14 @@ template <> struct Conv<bf16_t> {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-#ifndef ACTNN_NT_LOADS
-#define ACTNN_NT_LOADS 1
-#endif
-#ifndef ACTNN_NT_LOAD8_16
-#define ACTNN_NT_LOAD8_16 0
-#endif
-
 // 16-byte non-temporal load: for data that the kernel reads exactly once AND whose cache
 // lines are consumed whole by one load instruction of the wave (measured: 7.0 vs 6.4 TB/s on
 // a pure read).  Lanes that come back to the same line with a second instruction (the
 // 32-byte-per-lane pattern of fp32 pack) must use the plain load or they fetch the line twice.
 ACTNN_DEV u32x4 load16_nt(const void* p) {
-#if ACTNN_NT_LOADS
   return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
-#else
-  return *reinterpret_cast<const u32x4*>(p);
-#endif
 }
 ACTNN_DEV u32x4 load16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
-ACTNN_DEV u32x4 load16_b16(const void* p) {
-#if ACTNN_NT_LOAD8_16
-  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
-#else
-  return *reinterpret_cast<const u32x4*>(p);
-#endif
-}
 ACTNN_DEV void store16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
 ACTNN_DEV void store16_nt(void* p, u32x4 v) { __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p)); }
 
@@ -100,7 +82,7 @@ ACTNN_DEV void load8(const float* p, float (&v)[8]) {
   }
 }
 ACTNN_DEV void load8(const __half* p, float (&v)[8]) {
-  const u32x4 a = load16_b16(p);
+  const u32x4 a = load16(p);
   const uint32_t w[4] = {a.x, a.y, a.z, a.w};
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -109,7 +91,7 @@ ACTNN_DEV void load8(const __half* p, float (&v)[8]) {
   }
 }
 ACTNN_DEV void load8(const bf16_t* p, float (&v)[8]) {
-  const u32x4 a = load16_b16(p);
+  const u32x4 a = load16(p);
   const uint32_t w[4] = {a.x, a.y, a.z, a.w};
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -284,13 +266,10 @@ template <int ROWS> ACTNN_DEV float rows_max(float v) {
 // ------------------------------------------------------------------ Philox4x32-10
 struct Philox4 { uint32_t x, y, z, w; };
 
-#ifndef ACTNN_PHILOX_ROUNDS
-#define ACTNN_PHILOX_ROUNDS 10    // anything else is for timing experiments only
-#endif
 ACTNN_DEV Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
                                 uint32_t k0, uint32_t k1) {
 #pragma unroll
-  for (int r = 0; r < ACTNN_PHILOX_ROUNDS; ++r) {
+  for (int r = 0; r < 10; ++r) {
     const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
     const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
     // three-input xor in one instruction (v_bitop3_b32, truth table 0x96)

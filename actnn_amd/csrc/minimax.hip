@@ -14,9 +14,7 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kRowGroups = kThreads / 16;     // rows per block in the generic kernel
 
-#ifndef ACTNN_MM_ROWS
-#define ACTNN_MM_ROWS 8                       // rows per lane group and block (8 measured best)
-#endif
+constexpr int kRowsPerLaneGroup = 8;          // rows per lane group and block (8 measured best)
 
 template <typename T> struct Vec16;           // running min/max over one 16-byte vector of T
 template <> struct Vec16<float> {
@@ -70,7 +68,7 @@ __global__ __launch_bounds__(kThreads) void minimax_vec_kernel(const T* __restri
                                                                int64_t D, int vecs_per_lane) {
   constexpr int E = Vec16<T>::kElems;
   constexpr int kSlots = kThreads / LPR;
-  constexpr int R = ACTNN_MM_ROWS;
+  constexpr int R = kRowsPerLaneGroup;
   const int sub = threadIdx.x % LPR;
   const int slot = threadIdx.x / LPR;
   const int64_t row0 = (int64_t)blockIdx.x * (kSlots * R) + slot;
@@ -129,7 +127,7 @@ __global__ __launch_bounds__(kThreads) void minimax_generic_kernel(const T* __re
 
 template <typename T, int LPR>
 int launch_vec(const T* d, T* lo, T* hi, int64_t M, int64_t D, int64_t vecs, hipStream_t s) {
-  constexpr int kRows = (kThreads / LPR) * ACTNN_MM_ROWS;
+  constexpr int kRows = (kThreads / LPR) * kRowsPerLaneGroup;
   const int64_t blocks = (M + kRows - 1) / kRows;
   if (blocks > 0x7fffffffLL || vecs > 0x7fffffffLL) return ACTNN_EINVAL;
   const dim3 grid((unsigned)blocks), blk(kThreads);

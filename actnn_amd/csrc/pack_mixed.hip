@@ -22,24 +22,12 @@
 namespace actnn {
 namespace {
 
-// Groups per half-wave and block (1, 2 or 4).  fp32: 2 measured best (16 KiB of input per block).
+// Groups per half-wave and block.  fp32: 2 measured best (16 KiB of input per block).
 // 16-bit types: a block with 8 KiB of data is dominated by its own latency chain (widths ->
-// scales -> data), so they take 4 (and 8 for unpack, whose chain is longest).
-#ifndef ACTNN_PACK_GPH
-#define ACTNN_PACK_GPH 2
-#endif
-#ifndef ACTNN_UNPACK_GPH
-#define ACTNN_UNPACK_GPH 2
-#endif
-#ifndef ACTNN_PACK_GPH16
-#define ACTNN_PACK_GPH16 4
-#endif
-#ifndef ACTNN_UNPACK_GPH16
-#define ACTNN_UNPACK_GPH16 4
-#endif
+// scales -> data), so they take 4.
 template <typename T> struct Gph {
-  static constexpr int kPack = sizeof(T) == 2 ? ACTNN_PACK_GPH16 : ACTNN_PACK_GPH;
-  static constexpr int kUnpack = sizeof(T) == 2 ? ACTNN_UNPACK_GPH16 : ACTNN_UNPACK_GPH;
+  static constexpr int kPack = sizeof(T) == 2 ? 4 : 2;
+  static constexpr int kUnpack = sizeof(T) == 2 ? 4 : 2;
 };
 
 constexpr int kThreads = 256;
@@ -57,69 +45,12 @@ template <int BITS, int GPH> struct Tile {
   static __device__ __forceinline__ int group_of(int hw, int q) { return hw * GPH + q; }
 };
 
-// fp32: move the 32-byte-per-lane ownership through LDS so that HBM sees whole-line accesses.
-// Measured on MI355X: a clear win for the stores of unpack, a loss for the loads of pack.
-#ifndef ACTNN_PACK_LDS_STAGE
-#define ACTNN_PACK_LDS_STAGE 0
-#endif
-#ifndef ACTNN_PACK_STAGE_OUT
-#define ACTNN_PACK_STAGE_OUT 0     // measured: no gain over direct 4-byte stores
-#endif
-// Non-temporal stores for the unpacked output: with whole-line stores 6.9 instead of 5.3 TB/s
-// (and no dirty lines left behind for the next kernel to wait on).
-#ifndef ACTNN_UNPACK_NT_STORE
-#define ACTNN_UNPACK_NT_STORE 1
-#endif
-#ifndef ACTNN_PACK_NT_LOAD16
-#define ACTNN_PACK_NT_LOAD16 1
-#endif
-// Non-temporal stores for the packed words (a half-wave writes whole 128-byte lines): 3 % faster,
-// and no dirty lines are left behind for the next kernel.
-#ifndef ACTNN_PACK_NT_STORE
-#define ACTNN_PACK_NT_STORE 1
-#endif
-#ifndef ACTNN_UNPACK_LDS_STAGE
-#define ACTNN_UNPACK_LDS_STAGE 1
-#endif
-
-// fp32 groups: a lane owns 32 contiguous bytes, which as direct loads would be two half-used
-// 16-byte accesses per cache line.  Instead each wave reads a whole 1 KiB group per load
-// instruction (64 lanes x 16 bytes, non-temporal), parks it in its private LDS slab and every
-// lane picks up its own 32 bytes from there.  Only lanes of one wave exchange data, so no block
-// barrier is needed: LDS operations of a wave complete in order.
-template <int GPH, typename TL>
-ACTNN_DEV void stage_in_f32(const float* __restrict__ data, int64_t elem_base, int groups_valid,
-                            u32x4* __restrict__ slab, float (&v)[GPH][8]) {
-  const int wl = threadIdx.x & 63;          // lane in the wave
-  const int w = threadIdx.x >> 6;
-  const int h = (threadIdx.x >> 5) & 1;
-  const uint32_t lane = threadIdx.x & 31;
-  u32x4 reg[2 * GPH];
-#pragma unroll
-  for (int i = 0; i < 2 * GPH; ++i) {
-    const int gl = TL::group_of(2 * w + i / GPH, i % GPH);
-    reg[i] = (u32x4){0u, 0u, 0u, 0u};
-    if (gl < groups_valid) reg[i] = load16_nt(data + elem_base + (int64_t)gl * kGs + wl * 4);
-  }
-#pragma unroll
-  for (int i = 0; i < 2 * GPH; ++i) slab[i * 64 + wl] = reg[i];
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-  for (int q = 0; q < GPH; ++q) {
-    const u32x4 a = slab[(h * GPH + q) * 64 + 2 * lane];
-    const u32x4 b = slab[(h * GPH + q) * 64 + 2 * lane + 1];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      v[q][k] = as_float(a[k]);
-      v[q][4 + k] = as_float(b[k]);
-    }
-  }
-}
-
-// Mirror image for the fp32 output of unpack: lanes park their 8 values, the wave stores whole
-// 1 KiB groups with one instruction each.
+// fp32 output of unpack: a lane owns 32 contiguous bytes, which as direct stores would be two
+// half-used 16-byte accesses per cache line.  Instead lanes park their 8 values in the wave's
+// private LDS slab and the wave stores whole 1 KiB groups with one non-temporal instruction each
+// (measured 6.9 instead of 5.3 TB/s, and no dirty lines are left for the next kernel to wait on).
+// Only lanes of one wave exchange data, so no block barrier is needed: LDS operations of a wave
+// complete in order.  (The same staging for the fp32 loads of pack was measured slower.)
 template <int GPH, typename TL>
 ACTNN_DEV void stage_out_f32(float* __restrict__ out, int64_t elem_base, int groups_valid,
                              u32x4* __restrict__ slab, const float (&v)[GPH][8]) {
@@ -145,11 +76,7 @@ ACTNN_DEV void stage_out_f32(float* __restrict__ out, int64_t elem_base, int gro
   for (int i = 0; i < 2 * GPH; ++i) {
     const int gl = TL::group_of(2 * w + i / GPH, i % GPH);
     if (gl < groups_valid) {
-#if ACTNN_UNPACK_NT_STORE
       store16_nt(out + elem_base + (int64_t)gl * kGs + wl * 4, slab[i * 64 + wl]);
-#else
-      store16(out + elem_base + (int64_t)gl * kGs + wl * 4, slab[i * 64 + wl]);
-#endif
     }
   }
 }
@@ -161,26 +88,20 @@ template <> struct IsF32<float> { static constexpr bool value = true; };
 // Issue the loads of this lane's elements (and noise in deterministic mode) for its GPH groups.
 template <typename T, bool DET, int GPH>
 ACTNN_DEV void load_groups(const T* __restrict__ data, const T* __restrict__ noise, int64_t elem_base,
-                           int groups_valid, u32x4* slab, float (&v)[GPH][8],
-                           float (&nz)[DET ? GPH : 1][8]) {
+                           int groups_valid, float (&v)[GPH][8], float (&nz)[DET ? GPH : 1][8]) {
   using TL = Tile<1, GPH>;
   const uint32_t lane = threadIdx.x & 31;
   const int hw = threadIdx.x >> 5;
-  constexpr bool kStage = ACTNN_PACK_LDS_STAGE && IsF32<T>::value;
-  if constexpr (kStage)
-    stage_in_f32<GPH, TL>(reinterpret_cast<const float*>(data), elem_base, groups_valid, slab, v);
 #pragma unroll
   for (int q = 0; q < GPH; ++q) {
     const int gl = TL::group_of(hw, q);
     if (gl < groups_valid) {
       const int64_t e = elem_base + (int64_t)gl * kGs + lane * 8;
-      if constexpr (!kStage) {
-        if (ACTNN_PACK_NT_LOAD16) load8_nt(data + e, v[q]); else load8(data + e, v[q]);
-      }
+      load8_nt(data + e, v[q]);      // non-temporal for 16-bit types only (one instruction per line)
       if (DET) load8(noise + e, nz[DET ? q : 0]);
     } else {
 #pragma unroll
-      for (int k = 0; k < 8; ++k) { if (!kStage) v[q][k] = 0.0f; if (DET) nz[DET ? q : 0][k] = 0.0f; }
+      for (int k = 0; k < 8; ++k) { v[q][k] = 0.0f; if (DET) nz[DET ? q : 0][k] = 0.0f; }
     }
   }
 }
@@ -189,7 +110,7 @@ template <typename T, int BITS, bool DET>
 ACTNN_DEV void pack_groups(const float (&v)[Gph<T>::kPack][8], const float (&nz)[DET ? Gph<T>::kPack : 1][8],
                            int32_t* __restrict__ packed, int64_t elem_base, int64_t word_base,
                            int groups_valid, const float* s_mul, const float* s_sub,
-                           uint64_t seed, uint64_t offset, u32x4* s_out) {
+                           uint64_t seed, uint64_t offset) {
   constexpr int kGroupsPerHalf = Gph<T>::kPack;
   using TL = Tile<BITS, kGroupsPerHalf>;
   constexpr int R = TL::kGroupsPerReg;
@@ -219,32 +140,19 @@ ACTNN_DEV void pack_groups(const float (&v)[Gph<T>::kPack][8], const float (&nz)
     const int glt = TL::group_of(hw, q0);            // first group of this register tile
     const int64_t tile_words = word_base + (int64_t)glt * WPG;
     const uint32_t lo = transpose32((uint32_t)acc, lane);
-    // ACTNN_PACK_STAGE_OUT: words go to LDS first and the block writes them as one contiguous
-    // run of 16-byte stores; otherwise each half-wave stores its own 4-byte words.
-    int32_t* dst = ACTNN_PACK_STAGE_OUT ? reinterpret_cast<int32_t*>(s_out) + glt * WPG : packed + tile_words;
+    // each half-wave stores its own 4-byte words (whole 128-byte lines), non-temporally: 3 % faster
+    // than plain stores, and no dirty lines are left behind for the next kernel
+    int32_t* dst = packed + tile_words;
     if (TL::kTwoRegs) {
       const uint32_t hi = transpose32((uint32_t)(acc >> 32), lane);
       if (glt < groups_valid) {
-        if (ACTNN_PACK_NT_STORE && !ACTNN_PACK_STAGE_OUT) {
-          __builtin_nontemporal_store((int32_t)lo, dst + lane);
-          if ((int)lane < WPG - 32) __builtin_nontemporal_store((int32_t)hi, dst + 32 + lane);
-        } else {
-          dst[lane] = (int32_t)lo;
-          if ((int)lane < WPG - 32) dst[32 + lane] = (int32_t)hi;
-        }
+        __builtin_nontemporal_store((int32_t)lo, dst + lane);
+        if ((int)lane < WPG - 32) __builtin_nontemporal_store((int32_t)hi, dst + 32 + lane);
       }
     } else {
-      if ((int)lane < R * WPG && glt + (int)lane / WPG < groups_valid) {
-        if (ACTNN_PACK_NT_STORE && !ACTNN_PACK_STAGE_OUT) __builtin_nontemporal_store((int32_t)lo, dst + lane);
-        else dst[lane] = (int32_t)lo;
-      }
+      if ((int)lane < R * WPG && glt + (int)lane / WPG < groups_valid)
+        __builtin_nontemporal_store((int32_t)lo, dst + lane);
     }
-  }
-  if (ACTNN_PACK_STAGE_OUT) {
-    __syncthreads();
-    const int total_vec = groups_valid * WPG / 4;          // 16-byte vectors of this block's output
-    if ((int)threadIdx.x < total_vec)
-      store16(packed + word_base + threadIdx.x * 4, s_out[threadIdx.x]);
   }
 }
 
@@ -258,10 +166,6 @@ __global__ __launch_bounds__(kThreads) void pack_mixed_kernel(
   constexpr int kGroupsPerBlock = kHalfWaves * GPH;
   __shared__ float s_mul[kGroupsPerBlock];
   __shared__ float s_sub[kGroupsPerBlock];
-  constexpr bool kStage = ACTNN_PACK_LDS_STAGE && IsF32<T>::value;
-  __shared__ u32x4 s_slab[kStage ? kGroupsPerBlock * 64 : 1];     // 1 KiB per group
-  u32x4* slab = s_slab + (kStage ? (threadIdx.x >> 6) * (2 * GPH * 64) : 0);
-  __shared__ u32x4 s_out[ACTNN_PACK_STAGE_OUT ? kGroupsPerBlock * 16 : 1];    // up to 64 words per group
   const int64_t n = blockIdx.x / blocks_per_sample;
   const int64_t gb = (int64_t)(blockIdx.x % blocks_per_sample) * kGroupsPerBlock;
   const int groups_valid = (int)((G - gb) < kGroupsPerBlock ? (G - gb) : kGroupsPerBlock);
@@ -271,7 +175,7 @@ __global__ __launch_bounds__(kThreads) void pack_mixed_kernel(
   // then compute the block's scales while they travel.
   float v[GPH][8];
   float nz[DET ? GPH : 1][8];
-  load_groups<T, DET, GPH>(data, noise, elem_base, groups_valid, slab, v, nz);
+  load_groups<T, DET, GPH>(data, noise, elem_base, groups_valid, v, nz);
 
   const int b = bits[n];
   if (threadIdx.x < kGroupsPerBlock) {
@@ -291,7 +195,7 @@ __global__ __launch_bounds__(kThreads) void pack_mixed_kernel(
 #define ACTNN_CASE(B_)                                                                          \
   case B_:                                                                                      \
     pack_groups<T, B_, DET>(v, nz, packed, elem_base, word_base, groups_valid, s_mul, s_sub,    \
-                            seed, offset, s_out);                                               \
+                            seed, offset);                                                      \
     break;
     ACTNN_CASE(1) ACTNN_CASE(2) ACTNN_CASE(3) ACTNN_CASE(4)
     ACTNN_CASE(5) ACTNN_CASE(6) ACTNN_CASE(7) ACTNN_CASE(8)
@@ -306,7 +210,7 @@ ACTNN_DEV void unpack_groups(const int32_t* __restrict__ packed, T* __restrict__
                              int64_t elem_base, int64_t word_base, int groups_valid,
                              float* s_scale, float* s_min, float my_scale, float my_min, u32x4* slab) {
   constexpr int kGroupsPerHalf = Gph<T>::kUnpack;
-  constexpr bool kStage = ACTNN_UNPACK_LDS_STAGE && IsF32<T>::value;
+  constexpr bool kStage = IsF32<T>::value;
   float vs[kStage ? kGroupsPerHalf : 1][8];
   using TL = Tile<BITS, kGroupsPerHalf>;
   constexpr int R = TL::kGroupsPerReg;
@@ -356,8 +260,7 @@ ACTNN_DEV void unpack_groups(const int32_t* __restrict__ packed, T* __restrict__
 #pragma unroll
           for (int k = 0; k < 8; ++k) vs[kStage ? q0 + r : 0][k] = v[k];
         } else {
-          if (ACTNN_UNPACK_NT_STORE) store8_nt(out + elem_base + (int64_t)gl * kGs + lane * 8, v);
-          else store8(out + elem_base + (int64_t)gl * kGs + lane * 8, v);
+          store8_nt(out + elem_base + (int64_t)gl * kGs + lane * 8, v);
         }
       }
     }
@@ -374,7 +277,7 @@ __global__ __launch_bounds__(kThreads) void unpack_mixed_kernel(
   constexpr int kGroupsPerBlock = kHalfWaves * Gph<T>::kUnpack;
   __shared__ float s_scale[kGroupsPerBlock];
   __shared__ float s_min[kGroupsPerBlock];
-  constexpr bool kStage = ACTNN_UNPACK_LDS_STAGE && IsF32<T>::value;
+  constexpr bool kStage = IsF32<T>::value;
   __shared__ u32x4 s_slab[kStage ? kGroupsPerBlock * 64 : 1];
   u32x4* slab = s_slab + (kStage ? (threadIdx.x >> 6) * (2 * Gph<T>::kUnpack * 64) : 0);
   const int64_t n = blockIdx.x / blocks_per_sample;

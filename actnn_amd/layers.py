@@ -77,6 +77,18 @@ class _QConvMixin:
         if self.padding_mode != "zeros":
             input = F.pad(input, self._reversed_padding_repeated_twice, mode=self.padding_mode)
             padding = self._zero_pad(0)
+        elif isinstance(self.padding, str):
+            # 'valid' / 'same': the backward operator wants integers.  nn.Conv*d has worked the
+            # string out per side (last dimension first); a symmetric amount is passed on as the
+            # convolution's own padding, an asymmetric one ('same' with an even extent) is applied
+            # to the input beforehand, as torch's own convolution does.
+            sides = self._reversed_padding_repeated_twice
+            pairs = [(sides[2 * i], sides[2 * i + 1]) for i in range(self._dims)]
+            if all(left == right for left, right in pairs):
+                padding = tuple(left for left, _ in reversed(pairs))
+            else:
+                input = F.pad(input, sides)
+                padding = self._zero_pad(0)
         else:
             padding = self.padding
         return _autocast_apply(self._function, input, self.weight, self.bias, self.stride, padding,

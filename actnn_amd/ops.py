@@ -61,10 +61,11 @@ def dequantize_and_unpack(data, shape, bits, scale, mn):
 
 
 def no_scheme_compute_quantization_bits(input, known_minmax=None):
-    """Fixed width for every sample when no scheme is attached (ops.py:77-96)."""
+    """Fixed width for every sample when no scheme is attached (ops.py:77-96).  Always per-group
+    ranges: `config.pergroup` is a rule of the schemes, this path of the reference never reads it."""
     from .qscheme import group_min_max
     N = input.shape[0]
-    groups, mn, mx, _ = group_min_max(input, known_minmax)
+    groups, mn, mx, _ = group_min_max(input, known_minmax, whole_tensor_range=False)
     return groups, config.activation_compression_bits[0], mn.view(N, -1, 1), mx.view(N, -1, 1)
 
 
@@ -414,7 +415,9 @@ class batch_norm(Function):
         fixed_width = (not scheme and config.compress_activation and not config.simulate
                        and isinstance(config.activation_compression_bits[0], int)
                        and 1 <= config.activation_compression_bits[0] <= 8)
-        if ((scheme or fixed_width) and config.fused_bn_pack
+        # (the pass rounds stochastically, like pack_*; with config.stochastic off the unfused
+        # sequence below is taken and pack_* refuses, as in the reference)
+        if ((scheme or fixed_width) and config.fused_bn_pack and config.stochastic
                 and _bn_shares_min_max(input, weight, bias, running_mean, running_var, training)
                 and ext_backward_func.hip_batch_norm_pack_applies(input, weight, bias, running_mean, running_var)):
             # two reads of the input in total: the statistics pass also yields the quantiser's

@@ -16,11 +16,13 @@ from .cpp_extension.quantization import attach_bits_host, attach_bits_total
 from .utils import memory_order
 
 
-def group_min_max(input, known=None):
+def group_min_max(input, known=None, whole_tensor_range=None):
     """Flatten to [N, -1], zero-pad the feature axis to a multiple of group_size, view as groups
     and reduce each group (qscheme.py:59-74).  Returns (groups [N,G,gs], mn [N*G], mx [N*G],
     pixels per channel).  `known` = (mn, mx) already produced by another pass over the same
-    tensor (the batch-norm statistics kernel); only given when no padding is needed."""
+    tensor (the batch-norm statistics kernel); only given when no padding is needed.
+    `whole_tensor_range`: replace the group ranges by the tensor's (default: `not config.pergroup`,
+    the scheme's rule, qscheme.py:75-77)."""
     N = input.shape[0]
     flat = memory_order(input).reshape(N, -1)            # a view for default and channels-last layouts
     features = flat.shape[1]
@@ -33,7 +35,9 @@ def group_min_max(input, known=None):
         flat = flat.contiguous()
     rows = flat.view(-1, gs)
     mn, mx = known if known is not None else ext_minimax.minimax(rows)
-    if not config.pergroup:                     # one range for the whole tensor (qscheme.py:75-77)
+    if whole_tensor_range is None:
+        whole_tensor_range = not config.pergroup
+    if whole_tensor_range:                      # one range for the whole tensor (qscheme.py:75-77)
         mn = torch.ones_like(mn) * mn.min()
         mx = torch.ones_like(mx) * mx.max()
     return rows.view(N, -1, gs), mn, mx, num_pixels
@@ -96,9 +100,7 @@ def allocate_bits_on_device(mn, mx, N, num_pixels, factor, mult, initial_bits, a
     C_dev, bits, prefix = ext_calc_precision.allocate_bits_device(
         mn, mx, N, factor * config.group_size / num_pixels, mult, initial, target)
     taken = min(max(N * initial - target, 0), N * (initial - 1))
-    bits = attach_bits_total(bits, N * initial - taken)
-    bits._actnn_info = (bits._actnn_total, prefix)
-    return C_dev, bits
+    return C_dev, attach_bits_total(bits, N * initial - taken, prefix)
 
 
 def allocate_on_device(N, initial_bits):

@@ -260,16 +260,16 @@ def main():
         print(json.dumps({"other_configs": other_configs(device, max(10, args.steps // 2))}))
         return
     if args.only == "resnet50":
-        from actnn_amd import bench_extra
+        import bench_extra
         print(json.dumps({"resnet50_L3": bench_extra.resnet50_step(device, "L3", warmup=2, steps=3)}))
         return
     if args.only == "resnet50_channels_last":
-        from actnn_amd import bench_extra
+        import bench_extra
         print(json.dumps({"resnet50_L3_channels_last": bench_extra.resnet50_step(
             device, "L3", warmup=2, steps=3, channels_last=True)}))
         return
     if args.only == "resnet50_fp32":
-        from actnn_amd import bench_extra
+        import bench_extra
         out = {}
         for key, level, cl in (("resnet50_fp32_exact", "exact", False), ("resnet50_fp32_L3", "L3", False),
                                ("resnet50_fp32_exact_channels_last", "exact", True),
@@ -280,7 +280,7 @@ def main():
         print(json.dumps(out))
         return
     if args.only == "resnet50_levels":
-        from actnn_amd import bench_extra
+        import bench_extra
         out = {}
         for level in ("exact", "L0", "L1", "L2", "L3", "L3.1", "L4", "swap"):
             torch.cuda.empty_cache()
@@ -290,7 +290,7 @@ def main():
         print(json.dumps(out))
         return
     if args.only == "batch_norm_shapes":
-        from actnn_amd import bench_extra
+        import bench_extra
         print(json.dumps({"batch_norm_shapes": [bench_extra.batch_norm_shapes(device, channels_last=cl)
                                                 for cl in (True, False)]}))
         return
@@ -366,7 +366,7 @@ def main():
         except Exception as e:                       # keep the headline line even if an extra fails
             result["other_configs"] = {"error": repr(e)}
         try:
-            from actnn_amd import bench_extra
+            import bench_extra
             result.update(bench_extra.run(device))
         except ImportError:
             pass

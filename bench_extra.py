@@ -6,9 +6,9 @@ import time
 import torch
 import torch.nn.functional as F
 
-from . import QBNScheme, QModule, QScheme, config, set_optimization_level
-from .resnet import resnet50
-from .utils import compute_tensor_bytes, get_memory_usage
+from actnn_amd import QBNScheme, QModule, QScheme, config, set_optimization_level
+from actnn_amd.resnet import resnet50
+from actnn_amd.utils import compute_tensor_bytes, get_memory_usage
 
 
 def resnet50_step(device, level="L3", batch=512, warmup=3, steps=10, autocast=True, channels_last=False):
@@ -87,8 +87,8 @@ def batch_norm_shapes(device, channels_last=True, batch=512, reps=10):
     events on every batch-norm shape of ResNet-50 in bf16: ms and GB/s of algorithmic bytes per
     shape, and the totals weighted by the number of layers."""
     import actnn_amd.cpp_extension.backward_func as bf
-    from .cpp_extension.quantization import attach_bits_total
-    from .ops import _Quantized
+    from actnn_amd.cpp_extension.quantization import attach_bits_total
+    from actnn_amd.ops import _Quantized
 
     def timed(fn):
         for _ in range(3):

@@ -20,8 +20,13 @@ Pinning status (what fixes each function besides its own formula):
 * ``calc_precision.calc_precision`` - brute-force optimality on tiny inputs, the
   hand-derived degenerate allocation (C == 0) and, where it builds, the reference's own
   calc_precision.cc compiled into ``oracle/_ref`` (see ``oracle/build_ref.py``).
-* ``kernel_mode.*`` (arithmetic of the reference's CUDA kernels, which differs from
-  ``config.simulate``) - values are only pinned statistically (unbiasedness, closed-form
-  variance) because the reference's RNG stream (cuRAND) is not reproducible here:
-  the *stream values* are parity unpinned, the distribution is pinned.
+* ``kernel_mode.kernel_scale`` / ``kernel_dequant`` (arithmetic of the reference's CUDA
+  kernels, which differs from ``config.simulate``) - pinned on the CPU by
+  tests/test_oracle_kernel_mode.py: known answers where evaluating the scale in float instead
+  of double, or narrowing double -> half directly, would store another value; an exact
+  rational-arithmetic model of the rounding chain; constant groups (+inf in fp16) and B = 255.
+* ``kernel_mode.rng_codes`` and the rest of the in-kernel-RNG model - values are only pinned
+  statistically (unbiasedness, closed-form variance) because the reference's RNG stream
+  (cuRAND) is not reproducible here: the *stream values* are parity unpinned, the
+  distribution is pinned.
 """

@@ -149,3 +149,77 @@ def test_adaptive_avg_pool2d_keeps_only_the_shape():
     assert torch.allclose(gx, gr) and y.grad_fn.saved == x.shape
     with pytest.raises(AssertionError):
         adaptive_avg_pool2d.apply(x, (2, 2))
+
+
+class _FakeLib:
+    """Stands in for the C-ABI library where a test only needs to see which calls are made."""
+
+    def __init__(self):
+        self.prefix_calls = 0
+
+    def actnn_bits_prefix(self, bits_ptr, prefix_ptr, N, stream):
+        self.prefix_calls += 1
+        return 0
+
+
+def test_bits_cache_follows_the_version_counter(monkeypatch):
+    # the sum / prefix / host copy attached to a `bits` tensor must not outlive an in-place change
+    import actnn_amd.cpp_extension._glue as glue
+    import actnn_amd.cpp_extension.quantization as ext_q
+    fake = _FakeLib()
+    monkeypatch.setattr(glue, "lib", lambda: fake)
+    monkeypatch.setattr(glue, "stream_ptr", lambda device: 0)
+    host = torch.tensor([2, 2, 3, 1], dtype=torch.int32)
+    bits = ext_q.attach_bits_host(host.clone(), host)
+    total, prefix = ext_q._bits_info(bits)
+    assert total == 8 and fake.prefix_calls == 1
+    assert ext_q._bits_info(bits)[1] is prefix and fake.prefix_calls == 1        # cache hit
+    bits[0] = 8                                                                  # in-place: version moves on
+    total2, prefix2 = ext_q._bits_info(bits)
+    assert total2 == 14 and prefix2 is not prefix and fake.prefix_calls == 2      # re-read, not the stale sum
+    bits[1] = 9                                                                  # out of range now
+    with pytest.raises(RuntimeError, match="1..8 bits"):
+        ext_q._bits_info(bits)
+    # a total attached by the device allocation is dropped the same way
+    b2 = ext_q.attach_bits_total(torch.full((4,), 2, dtype=torch.int32), 8, prefix=torch.zeros(5, dtype=torch.int32))
+    assert ext_q._bits_info(b2)[0] == 8 and fake.prefix_calls == 2               # prefix came attached
+    b2.fill_(4)
+    assert ext_q._bits_info(b2)[0] == 16 and fake.prefix_calls == 3
+
+
+@pytest.mark.parametrize("padding,kernel", [("same", 3), ("same", 4), ("valid", 3), (1, 3)])
+def test_qconv_string_padding_matches_torch(padding, kernel):
+    # with compression off the Q-layer's training path (custom Function, explicit backward
+    # operator) runs on the CPU: outputs and all three gradients must equal nn.Conv2d's
+    from actnn_amd.layers import QConv2d
+    set_optimization_level("L0")
+    torch.manual_seed(0)
+    ref = nn.Conv2d(3, 5, kernel, padding=padding)
+    q = QModule(nn.Sequential(nn.Conv2d(3, 5, kernel, padding=padding)))
+    assert isinstance(q.model[0], QConv2d) and q.model[0].padding == ref.padding
+    q.model[0].load_state_dict(ref.state_dict())
+    x = torch.randn(2, 3, 9, 8, requires_grad=True)
+    xr = x.detach().clone().requires_grad_(True)
+    y, yr = q(x), ref(xr)
+    assert torch.allclose(y, yr, atol=1e-6)
+    g = torch.randn_like(yr)
+    y.backward(g)
+    yr.backward(g)
+    assert torch.allclose(x.grad, xr.grad, atol=1e-5)
+    assert torch.allclose(q.model[0].weight.grad, ref.weight.grad, atol=1e-5)
+    assert torch.allclose(q.model[0].bias.grad, ref.bias.grad, atol=1e-5)
+
+
+def test_no_scheme_path_keeps_group_ranges_whatever_pergroup_says():
+    # the reference's fixed-width path (ops.py:77-96) never reads config.pergroup
+    from actnn_amd.ops import no_scheme_compute_quantization_bits
+    from actnn_amd.qscheme import group_min_max
+    x = torch.randn(2, 4, 8, 16)                     # 512 features: two groups per sample
+    rows = x.view(-1, 256)
+    known = (rows.min(1)[0], rows.max(1)[0])
+    config.pergroup = False
+    config.activation_compression_bits = [4]
+    groups, bits, mn, mx = no_scheme_compute_quantization_bits(x, known)
+    assert bits == 4 and torch.equal(mn.view(-1), known[0]) and torch.equal(mx.view(-1), known[1])
+    _, mn_s, mx_s, _ = group_min_max(x, known)        # the schemes' rule: one range for the tensor
+    assert bool((mn_s == x.min()).all()) and bool((mx_s == x.max()).all())
