@@ -25,10 +25,24 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, then WRITE_SIZE, each scaled by
-# what the same counter reads for actnn_stream_copy of a known size); see profiles/.  None = not
-# measured yet.
-MEASURED_TRAFFIC_BYTES = {"minimax": 828536830, "pack_mixed": 892254308, "unpack_mixed": 886732426}
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "config2_minimax_pack_unpack_mixed_f32.txt")
+
+
+def measured_traffic(kernel_name, path=TRAFFIC_SUMMARY):
+    """HBM bytes per launch of `kernel_name` as measured with rocprofv3 --pmc (FETCH_SIZE, then
+    WRITE_SIZE, each scaled by what the same counter reads for actnn_stream_copy of a known size):
+    read from the table of the committed summary (columns: kernel, FETCH_SIZE, WRITE_SIZE, HBM
+    bytes, algorithmic bytes, ratio).  -> (bytes or None, algorithmic bytes the measurement was
+    taken against or None)."""
+    try:
+        with open(path) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) == 6 and parts[0] == kernel_name:
+                    return int(parts[3]), int(parts[4])
+    except (OSError, ValueError):
+        pass
+    return None, None
 
 
 def _event_time_ms(fn, reps, warmup=3):
@@ -48,8 +62,12 @@ def _event_time_ms(fn, reps, warmup=3):
     return start.elapsed_time(stop) / reps
 
 
-def make_config2(device, N=256, C=256, H=56, W=56, seed=0):
-    """fp32 activation of benchmark config 2 and its per-sample bits (greedy at avg 2.0 bits)."""
+def make_config2(device, N=256, C=256, H=56, W=56, seed=0, sample_spread=0.0, dtype=None):
+    """Activation of benchmark config 2 - ReLU(N(0,1)) times a per-channel LogNormal(0,1) scale,
+    fp32 unless `dtype` says otherwise - and its per-sample bits (greedy at avg 2.0 bits).
+    `sample_spread` > 0 additionally multiplies every sample by LogNormal(0, sample_spread): with
+    identically distributed samples the greedy allocation hands (almost) every sample the same
+    width, the spread makes it use many widths.  Same bytes, same average width."""
     import torch
     import actnn_amd.cpp_extension.calc_precision as ext_cp
     import actnn_amd.cpp_extension.minimax as ext_minimax
@@ -58,9 +76,10 @@ def make_config2(device, N=256, C=256, H=56, W=56, seed=0):
     s_c = torch.exp(torch.randn(C, generator=g, device=device))
     x = torch.randn(N, C, H, W, generator=g, device=device)
     x = torch.relu_(x).mul_(s_c.view(1, C, 1, 1))
-    # samples differ in range (LogNormal(0, 0.7) per sample): with identically distributed samples
-    # the greedy allocation hands every sample the same width and the mixed-width path is not used
-    x.mul_(torch.exp(0.7 * torch.randn(N, generator=g, device=device)).view(N, 1, 1, 1))
+    if sample_spread > 0:
+        x.mul_(torch.exp(sample_spread * torch.randn(N, generator=g, device=device)).view(N, 1, 1, 1))
+    if dtype is not None:
+        x = x.to(dtype)
     gs = 256
     G = C * H * W // gs
     xg = x.view(N, G, gs)
@@ -87,9 +106,12 @@ def algorithmic_bytes(n, esize, avg_bits, gs=256):
     }
 
 
-def cpu_baseline(budget_s=15.0):
+def cpu_baseline(budget_s=15.0, device=None):
     """The oracle's restatement of the reference's config.simulate quantise+dequantise
-    (actnn/actnn/ops.py:22-41,55-57) on benchmark config 1, all host cores."""
+    (actnn/actnn/ops.py:22-41,55-57) on benchmark config 1, all host cores.  With `device` the
+    same tensors then go through the HIP kernels' deterministic mode (explicit noise tensor) and
+    the packed words, scales and dequantised values are compared bit for bit with the CPU result
+    (`hip_deterministic_bit_exact`); the oracle is only the checker here."""
     import torch
     from oracle import simulate
     cores = os.cpu_count() or 1
@@ -101,7 +123,7 @@ def cpu_baseline(budget_s=15.0):
 
     def run():
         q, s = simulate.quantize_simulate(x.clone(), 2, mn, mx, noise)
-        return simulate.dequantize_simulate(q, s, mn)
+        return q, s, simulate.dequantize_simulate(q, s, mn)
 
     for _ in range(3):
         run()
@@ -109,15 +131,40 @@ def cpu_baseline(budget_s=15.0):
     t_end = time.perf_counter() + budget_s
     while len(times) < 10 or (time.perf_counter() < t_end and len(times) < 200):
         t0 = time.perf_counter()
-        run()
+        codes, scale, deq = run()
         times.append(time.perf_counter() - t0)
     times.sort()
     med = times[len(times) // 2]
     n = x.numel()
-    return {"value": round(4 * n / med / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
-            "kind": "port", "elements_per_s": round(n / med, 1), "median_ms": round(med * 1e3, 3),
-            "sample": f"config.simulate quantise+dequantise of fp32 [32,64,56,56] (n={n}), 2 bits, "
-                      f"median of {len(times)} repetitions; GB/s over 4n input bytes"}
+    out = {"value": round(4 * n / med / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+           "kind": "port", "elements_per_s": round(n / med, 1), "median_ms": round(med * 1e3, 3),
+           "sample": f"config.simulate quantise+dequantise of fp32 [32,64,56,56] (n={n}), 2 bits, "
+                     f"median of {len(times)} repetitions; GB/s over 4n input bytes"}
+    if device is not None:
+        import numpy as np
+        import actnn_amd.cpp_extension.minimax as ext_minimax
+        import actnn_amd.cpp_extension.quantization as ext_q
+        from oracle import layouts
+        N, G, gs = x.shape
+        xd = x.to(device)
+        lo, hi = ext_minimax.minimax(xd.view(-1, gs))
+        lo, hi = lo.view(N, G, 1), hi.view(N, G, 1)
+        host_bits = torch.full((N,), 2, dtype=torch.int32)
+        bits = ext_q.attach_bits_host(host_bits.to(device), host_bits)
+        packed, sc = ext_q.pack_mixed_precision(xd, lo, hi, bits, True, noise=noise.to(device))
+        back = ext_q.unpack_mixed_precision(packed, bits, sc, lo, N, G, gs)
+        packed1, sc1 = ext_q.pack_single_precision(xd, lo, hi, 2, True, noise=noise.to(device))
+        back1 = ext_q.unpack_single_precision(packed1, 2, sc1, lo, N, G, gs)
+        torch.cuda.synchronize()
+        want_single = layouts.pack_single(codes.numpy(), 2)
+        nbytes = N // 4 * G * gs                    # the stream proper (one spare byte follows it)
+        out["hip_deterministic_bit_exact"] = bool(
+            torch.equal(lo.cpu(), mn) and torch.equal(hi.cpu(), mx)
+            and np.array_equal(packed.cpu().numpy(), layouts.pack_mixed(codes.numpy(), host_bits.numpy()))
+            and torch.equal(sc.cpu(), scale) and torch.equal(back.cpu(), deq)
+            and np.array_equal(packed1.cpu().numpy()[:nbytes], want_single[:nbytes])
+            and torch.equal(sc1.cpu(), scale) and torch.equal(back1.cpu(), deq))
+    return out
 
 
 def other_configs(device, reps):
@@ -186,9 +233,34 @@ def other_configs(device, reps):
              lambda: ext_bf.hip_batch_norm_backward_packed(xb.shape, quantized, gb, w, mean, invstd))
         del xb, gb
     del x, g, q_in, q_scale, quantized, lo, hi
-    # config 4 input through the fixed-width path (2 bits)
+    # the 16-bit streaming kernels at the size that carries the ResNet-50 step (config 5): bf16
+    # [512,256,56,56], config 2's distribution, greedy widths at an average of 2 bits; and the
+    # fixed-width pack at 4 bits (levels L1/L2) on the same tensor
+    xb16, lo16, hi16, bits16, bits16_host = make_config2(device, N=512, dtype=torch.bfloat16)
+    Nb, Gb, _ = xb16.shape
+    nb = xb16.numel()
+    ab16 = algorithmic_bytes(nb, 2, float(bits16_host.float().mean()))
+    k16, pair16 = config2_kernel_times(xb16, lo16, hi16, bits16, ab16, reps)
+    for name, v in k16.items():
+        out[name + "_bf16_512x256x56x56"] = {"ms": v["ms"], "GB/s": v["GB/s"], "frac": v["frac"]}
+    out["minimax_plus_pack_mixed_bf16_512x256x56x56"] = pair16
+    p4, s4 = ext_q.pack_single_precision(xb16, lo16, hi16, 4, True)
+    b = 2 * nb + 3 * 2 * nb / 256 + nb / 2
+    t = _event_time_ms(lambda: ext_q.pack_single_precision(xb16, lo16, hi16, 4, True), reps)
+    out["pack_single_4bit_bf16_512x256x56x56"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
+    t = _event_time_ms(lambda: ext_q.unpack_single_precision(p4, 4, s4, lo16, Nb, Gb, 256), reps)
+    out["unpack_single_4bit_bf16_512x256x56x56"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
+    del xb16, lo16, hi16, bits16, p4, s4
+    torch.cuda.empty_cache()
+    # config 4: fp16 [8192,4096], Student-t(nu=3) heavy tails with a per-feature scale, through the
+    # fixed-width path (2 bits per row group of 256)
     M, I = 8192, 4096
-    xs = torch.randn(M, I // 256, 256, device=device, dtype=torch.float16)
+    gen = torch.Generator(device=device).manual_seed(4)
+    z = torch.randn(M, I, generator=gen, device=device)
+    chi = torch.randn(3, M, I, generator=gen, device=device).square_().sum(0).div_(3)
+    xs = (z / chi.sqrt_() * torch.exp(torch.randn(1, I, generator=gen, device=device))).to(torch.float16)
+    xs = xs.view(M, I // 256, 256)
+    del z, chi
     mn, mx = ext_minimax.minimax(xs.view(-1, 256))
     mn, mx = mn.view(M, -1, 1), mx.view(M, -1, 1)
     packed, scale = ext_q.pack_single_precision(xs, mn, mx, 2, True)
@@ -200,7 +272,7 @@ def other_configs(device, reps):
     out["unpack_single_2bit_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
     # config 4: fused dequant + grad_weight GEMM (MFMA roofline), and the unfused path beside it
     O = 4096
-    go = torch.randn(M, O, device=device, dtype=torch.float16)
+    go = torch.randn(M, O, generator=gen, device=device).to(torch.float16)
     flops = 2.0 * M * O * I
     t = _event_time_ms(lambda: ext_q.linear_grad_weight_q2(go, packed, scale, mn, I), reps)
     out["linear_grad_weight_q2_fused"] = {"ms": t, "TFLOP/s": flops / t / 1e9,
@@ -213,6 +285,35 @@ def other_configs(device, reps):
     out["linear_grad_weight_unfused_unpack_plus_mm"] = {"ms": t, "TFLOP/s": flops / t / 1e9,
                                                         "frac_mfma_bf16": flops / t / 1e9 / MFMA_BF16_PEAK_TFLOPS}
     return {k_: {kk: round(vv, 4) for kk, vv in v.items()} for k_, v in out.items()}
+
+
+def _width_histogram(bits_host):
+    """'1:12 2:200 ...' - how many samples got each width."""
+    import torch
+    counts = torch.bincount(bits_host.to(torch.int64), minlength=9)
+    return " ".join(f"{b}:{int(c)}" for b, c in enumerate(counts) if c)
+
+
+def config2_kernel_times(xg, mn, mx, bits, ab, reps):
+    """HIP-event time, GB/s of algorithmic bytes and fraction of the HBM peak for minimax,
+    pack_mixed (in-kernel Philox) and unpack_mixed on the given groups -> (kernels, minimax+pack)."""
+    import actnn_amd.cpp_extension.minimax as ext_minimax
+    import actnn_amd.cpp_extension.quantization as ext_q
+    N, G, gs = xg.shape
+    packed, scale = ext_q.pack_mixed_precision(xg, mn, mx, bits, True)
+    kern = {
+        "minimax": _event_time_ms(lambda: ext_minimax.minimax(xg.view(-1, gs)), reps),
+        "pack_mixed": _event_time_ms(lambda: ext_q.pack_mixed_precision(xg, mn, mx, bits, True), reps),
+        "unpack_mixed": _event_time_ms(lambda: ext_q.unpack_mixed_precision(packed, bits, scale, mn, N, G, gs), reps),
+    }
+    kernels = {k: {"ms": round(v, 4), "GB/s": round(ab[k] / v / 1e6, 1),
+                   "frac": round(ab[k] / v / 1e6 / HBM_PEAK_GBS, 4), "algorithmic_bytes": int(ab[k])}
+               for k, v in kern.items()}
+    pair_ms = kern["minimax"] + kern["pack_mixed"]
+    pair_bytes = ab["minimax"] + ab["pack_mixed"]
+    pair = {"ms": round(pair_ms, 4), "GB/s": round(pair_bytes / pair_ms / 1e6, 1),
+            "frac": round(pair_bytes / pair_ms / 1e6 / HBM_PEAK_GBS, 4)}
+    return kernels, pair
 
 
 def _heartbeat(period=30.0):
@@ -318,30 +419,21 @@ def main():
 
     # per-kernel timing (HIP events on the launch stream)
     reps = max(20, args.steps)
-    packed, scale = ext_q.pack_mixed_precision(xg, mn, mx, bits, True)
-    kern = {
-        "minimax": _event_time_ms(lambda: ext_minimax.minimax(xg.view(-1, gs)), reps),
-        "pack_mixed": _event_time_ms(lambda: ext_q.pack_mixed_precision(xg, mn, mx, bits, True), reps),
-        "unpack_mixed": _event_time_ms(lambda: ext_q.unpack_mixed_precision(packed, bits, scale, mn, N, G, gs), reps),
-    }
+    kernels, pair = config2_kernel_times(xg, mn, mx, bits, ab, reps)
     # plain copy of the same footprint: what a streaming kernel reaches on this box
     dst = torch.empty_like(xg)
     copy_ms = _event_time_ms(lambda: _lib.check(lib.actnn_stream_copy(
         xg.data_ptr(), dst.data_ptr(), n * 4, torch.cuda.current_stream().cuda_stream), "copy"), reps)
     del dst
-    kernels = {k: {"ms": round(v, 4), "GB/s": round(ab[k] / v / 1e6, 1),
-                   "frac": round(ab[k] / v / 1e6 / HBM_PEAK_GBS, 4), "algorithmic_bytes": int(ab[k])}
-               for k, v in kern.items()}
     kernels["stream_copy"] = {"ms": round(copy_ms, 4), "GB/s": round(2 * n * 4 / copy_ms / 1e6, 1),
                               "frac": round(2 * n * 4 / copy_ms / 1e6 / HBM_PEAK_GBS, 4)}
-    pair_ms = kern["minimax"] + kern["pack_mixed"]
-    pair = {"ms": round(pair_ms, 4), "GB/s": round((ab["minimax"] + ab["pack_mixed"]) / pair_ms / 1e6, 1),
-            "frac": round((ab["minimax"] + ab["pack_mixed"]) / pair_ms / 1e6 / HBM_PEAK_GBS, 4)}
 
     dom = "pack_mixed"
+    traffic, traffic_alg = measured_traffic("pack_mixed_kernel")
     roofline = {"bound": "hbm", "kernel": dom, "achieved": kernels[dom]["GB/s"], "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": kernels[dom]["frac"],
-                "traffic": MEASURED_TRAFFIC_BYTES.get(dom)}
+                "unit": "GB/s", "frac": kernels[dom]["frac"], "traffic": traffic,
+                "traffic_source": "profiles/" + os.path.basename(TRAFFIC_SUMMARY) +
+                                  (f" (measured against {traffic_alg} algorithmic bytes)" if traffic_alg else "")}
 
     result = {
         "metric": "pack+unpack GB/s & % HBM peak at avg 2-bit; R50 L3 train images/sec",
@@ -349,18 +441,27 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: minimax + pack_mixed_precision + unpack_mixed_precision, "
-                               "fp32 [256,256,56,56], group 256, greedy bits at avg "
-                               f"{avg_bits:.3f} (min {int(bits_host.min())}, max {int(bits_host.max())}), "
-                               "in-kernel Philox",
+                               "fp32 [256,256,56,56] = ReLU(N(0,1)) x per-channel LogNormal(0,1), group 256, "
+                               f"greedy bits at avg {avg_bits:.3f} ({_width_histogram(bits_host)}), "
+                               "in-kernel Philox; `kernels_mixed_spread` repeats the kernels with an extra "
+                               "per-sample LogNormal(0,0.7) factor that configs[1] does not have, so that "
+                               "the allocation uses many widths",
                    "bytes_per_step": int(step_bytes)},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "roofline": roofline,
         "kernels": kernels,
         "minimax_plus_pack": pair,
     }
+    del xg, mn, mx, bits
+    torch.cuda.empty_cache()
+    xs, mns, mxs, bits_s, bits_s_host = make_config2(device, sample_spread=0.7)
+    avg_s = float(bits_s_host.float().mean())
+    ks, pair_s = config2_kernel_times(xs, mns, mxs, bits_s, algorithmic_bytes(n, 4, avg_s), reps)
+    result["kernels_mixed_spread"] = {"widths": _width_histogram(bits_s_host), "avg_bits": round(avg_s, 3),
+                                      "kernels": ks, "minimax_plus_pack": pair_s}
+    del xs, mns, mxs, bits_s
+    torch.cuda.empty_cache()
     if not args.skip_extra:
-        del packed, scale
-        torch.cuda.empty_cache()
         try:
             result["other_configs"] = other_configs(device, max(10, args.steps // 2))
         except Exception as e:                       # keep the headline line even if an extra fails
@@ -373,7 +474,7 @@ def main():
         except Exception as e:
             result["extra_error"] = repr(e)
     if not args.skip_cpu:
-        result["cpu_baseline"] = cpu_baseline()
+        result["cpu_baseline"] = cpu_baseline(device=device)
     print(json.dumps(result))
 
 
