@@ -59,6 +59,9 @@ SIGNATURES = {
     "actnn_batch_norm_workspace_bytes": [c_i64, c_i64, c_i64, c_i32, c_i32],
     "actnn_batch_norm_forward": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,
                                  c_i64, c_i64, c_i64, ctypes.c_double, ctypes.c_double, c_i32, c_i32, c_vp],
+    "actnn_batch_norm_forward_static_limit": [],
+    "actnn_batch_norm_forward_static": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64,
+                                        c_i64, ctypes.c_double, ctypes.c_double, c_i32, c_i32, c_vp],
     "actnn_batch_norm_forward_stats": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,
                                        c_i64, c_i64, c_i64, ctypes.c_double, ctypes.c_double, c_i32, c_i32, c_vp],
     "actnn_batch_norm_forward_apply": [c_vp, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u64, c_u64,
@@ -71,6 +74,7 @@ SIGNATURES = {
 }
 _RESTYPES = {"actnn_strerror": ctypes.c_char_p, "actnn_version": ctypes.c_char_p,
              "actnn_batch_norm_workspace_bytes": ctypes.c_int64,
+             "actnn_batch_norm_forward_static_limit": ctypes.c_int64,
              "actnn_batch_norm_backward_sumsq_entries": ctypes.c_int64}
 
 _lib = None

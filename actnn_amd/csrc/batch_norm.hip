@@ -16,6 +16,8 @@
 // The statistics pass can also produce the per-group minimum and maximum of the activation
 // quantiser (groups of 256 consecutive elements of the row) from the registers it already holds,
 // which saves the quantiser's own read of the tensor.
+#include <mutex>
+
 #include "device_utils.h"
 #include "quant_math.h"
 
@@ -1102,6 +1104,64 @@ extern "C" int actnn_batch_norm_forward(const void* x, const float* weight, cons
   if (rc != ACTNN_OK) return rc;
   return actnn_batch_norm_forward_apply(x, y, workspace, workspace_bytes, nullptr, nullptr, nullptr, nullptr,
                                         nullptr, nullptr, 0, 0, N, C, HW, dtype, channels_last, stream);
+}
+
+// ------------------------------------------------------------------------------------------
+// The forward pass for callers that cannot allocate and have no workspace to hand over: the partial
+// sums and coefficients live in a fixed array in device memory instead of a workspace argument.
+// Every GPU the library runs on holds its own copy of the array, at its own address, until the
+// process ends.  In host code the array's name is only a stand-in for the symbol, not a device
+// address: the address of this device's copy is asked for once per device, with that device
+// current, and that pointer is what the kernels are given.
+namespace actnn {
+namespace {
+constexpr int64_t kStaticScratchBytes = (int64_t)16 << 20;
+static __device__ __align__(256) float scratch[kStaticScratchBytes / sizeof(float)];
+
+constexpr int kMaxDevices = 64;
+float* g_scratch_of_device[kMaxDevices];          // device address of `scratch`, per device
+std::mutex g_scratch_mutex;
+
+// -> ACTNN_OK and *out = this device's copy of the array, or an error code
+int static_scratch(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return ACTNN_EINVAL;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_of_device[dev]) {
+    float* ptr = nullptr;
+    e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!ptr) return ACTNN_EINVAL;
+    g_scratch_of_device[dev] = ptr;
+  }
+  *out = g_scratch_of_device[dev];
+  return ACTNN_OK;
+}
+}  // namespace
+}  // namespace actnn
+
+extern "C" int64_t actnn_batch_norm_forward_static_limit(void) { return actnn::kStaticScratchBytes; }
+
+extern "C" int actnn_batch_norm_forward_static(const void* x, const float* weight, const float* bias,
+                                               float* running_mean, float* running_var, void* y,
+                                               float* save_mean, float* save_invstd, void* mn, void* mx,
+                                               int64_t N, int64_t C, int64_t HW, double momentum,
+                                               double eps, int dtype, int channels_last, void* stream) {
+  using namespace actnn;
+  if (dtype < 0 || dtype > 2) return ACTNN_EDTYPE;
+  Plan pl;
+  if (!make_plan(N, C, HW, dtype, channels_last, pl)) return ACTNN_EINVAL;
+  const int64_t need = workspace_floats(pl, C) * (int64_t)sizeof(float);
+  if (need > kStaticScratchBytes) return ACTNN_ETOOBIG;
+  float* ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc != ACTNN_OK) return rc;
+  // every partial sum and coefficient the second kernel reads is written by the first ones in this
+  // call: nothing in the array has to start at zero
+  return actnn_batch_norm_forward(x, weight, bias, running_mean, running_var, y, save_mean, save_invstd, mn,
+                                  mx, ws, need, N, C, HW, momentum, eps, dtype, channels_last, stream);
 }
 
 extern "C" int actnn_batch_norm_backward(const void* x, const void* dy, const float* weight,

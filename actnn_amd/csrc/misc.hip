@@ -61,6 +61,7 @@ extern "C" const char* actnn_strerror(int code) {
     case ACTNN_EDTYPE: return "unknown dtype";
     case ACTNN_EBITS: return "unsupported bit width";
     case ACTNN_EALIGN: return "pointer is not aligned as required (16 bytes)";
+    case ACTNN_ETOOBIG: return "the problem needs more scratch memory than the library's fixed buffer holds";
     default: return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "unknown error";
   }
 }

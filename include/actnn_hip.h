@@ -29,7 +29,8 @@ enum {
   ACTNN_EINVAL = -1,   /* bad size / null pointer / unsupported combination */
   ACTNN_EDTYPE = -2,   /* unknown dtype */
   ACTNN_EBITS = -3,    /* bit width outside what the operator supports */
-  ACTNN_EALIGN = -4    /* pointer not aligned as the kernel requires (16 bytes) */
+  ACTNN_EALIGN = -4,   /* pointer not aligned as the kernel requires (16 bytes) */
+  ACTNN_ETOOBIG = -5   /* problem needs more scratch memory than the library's fixed buffer holds */
 };
 
 /* Human-readable text for a return code of this library (static storage). */
@@ -249,6 +250,23 @@ int actnn_batch_norm_backward(const void* x, const void* dy, const float* weight
  * the statistic of qscheme.py:47-55 - without another pass over dx. */
 int64_t actnn_batch_norm_backward_sumsq_entries(int64_t N, int64_t C, int64_t HW, int dtype,
                                                 int channels_last);
+
+/* actnn_batch_norm_forward without the workspace arguments, for callers that cannot allocate
+ * device memory and have no workspace to pass: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference.  The partial sums and
+ * coefficients live in a fixed device array inside the library (one copy per GPU, held until the
+ * process ends) of actnn_batch_norm_forward_static_limit() bytes (16 MiB: ResNet-50's batch norms up
+ * to batch 1024 in either layout need at most 8.4 MB); a shape whose
+ * actnn_batch_norm_workspace_bytes exceeds it is rejected with ACTNN_ETOOBIG.  Calls no hipMalloc,
+ * hipFree or other allocating routine.  Results are bit-identical to actnn_batch_norm_forward.
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different
+ * streams or threads) race; calls on one stream are ordered and safe. */
+int64_t actnn_batch_norm_forward_static_limit(void);
+int actnn_batch_norm_forward_static(const void* x, const float* weight, const float* bias,
+                                    float* running_mean, float* running_var, void* y,
+                                    float* save_mean, float* save_invstd, void* mn, void* mx,
+                                    int64_t N, int64_t C, int64_t HW, double momentum, double eps,
+                                    int dtype, int channels_last, void* stream);
 
 /* The forward pass in two steps, for callers that want the quantiser's output from the same read
  * of x: _stats runs the statistics pass (save_mean/save_invstd, running estimates, optional group
