@@ -53,6 +53,8 @@ SIGNATURES = {
     "actnn_max_pool2d_backward_cl": [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
                                      c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
     "actnn_calc_precision": [c_vp, c_vp, c_vp, c_i64, ctypes.c_double],
+    "actnn_linear_grad_weight": [c_vp, c_vp, c_vp, c_vp, c_i32, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64,
+                                 c_i32, c_i32, c_i32, c_vp],
     "actnn_linear_grad_weight_q2": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64,
                                     c_i32, c_i32, c_i32, c_vp],
     "actnn_stream_copy": [c_vp, c_vp, c_i64, c_vp],

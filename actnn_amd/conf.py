@@ -32,6 +32,7 @@ class QuantizationConfig:
         self.share_relu_min_max = True                 # ReLU leaves its output's group min/max for the next layer
         self.share_grad_sqnorm = True                  # batch-norm backward leaves sum(dx^2) for the conv's set_scale
         self.fused_bn_pack = True                      # batch-norm forward writes the packed copy of its input
+        self.fused_linear_grad_weight = True           # QLinear's weight gradient straight from the packed input
         # memory management (conf.py:54-58)
         self.empty_cache_threshold = None
         self.pipeline_threshold = None

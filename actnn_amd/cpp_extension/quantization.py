@@ -196,10 +196,13 @@ def unpack_single_precision(data, bits, scale, min, N, num_groups, group_size):
 # fused QLinear weight gradient (no counterpart among the reference's operators: it replaces
 # dequantize + grad_output.t().mm(input) of linear.backward, actnn/actnn/ops.py:407-421)
 # ------------------------------------------------------------------------------------------
-def linear_grad_weight_q2(grad_output, packed, scale, min, in_features, out_dtype=None):
-    """grad_w[O, I] = grad_output[M, O]^T @ dequant(x)[M, I], x given as the pack_single 2-bit
-    stream with scale/min [M, I/256, 1]; the dequantised tile only ever exists in LDS."""
-    g.check_typed(packed, "packed", torch.int8, 1)
+def linear_grad_weight(grad_output, packed, bits, scale, min, in_features, out_dtype=None):
+    """grad_w[O, I] = grad_output[M, O]^T @ dequant(x)[M, I] with x given as it was saved: `bits`
+    an int (the fixed-width stream of pack_single_precision, int8) or an int32 tensor [M] (the
+    mixed-width stream of pack_mixed_precision, int32), scale/min [M, I/256, 1].  The dequantised
+    tile only ever exists in LDS."""
+    mixed = isinstance(bits, torch.Tensor)
+    g.check_typed(packed, "packed", torch.int32 if mixed else torch.int8, 1)
     g.check_float(scale, "scale", 3)
     g.check_float(min, "min", 3)
     if not (isinstance(grad_output, torch.Tensor) and grad_output.is_cuda and grad_output.dim() == 2):
@@ -209,20 +212,41 @@ def linear_grad_weight_q2(grad_output, packed, scale, min, in_features, out_dtyp
     grad_output = g.aligned(grad_output.contiguous())
     M, O = grad_output.shape
     I = int(in_features)
-    if I % 256 != 0 or M % 4 != 0 or O % 8 != 0:
-        raise RuntimeError("linear_grad_weight_q2 needs M % 4 == 0, in_features % 256 == 0, O % 8 == 0")
-    if scale.numel() != M * (I // 256) or min.numel() != scale.numel() or min.dtype != scale.dtype:
-        raise RuntimeError("linear_grad_weight_q2: scale/min do not match the packed input")
-    if packed.numel() < M * I // 4:
-        raise RuntimeError("linear_grad_weight_q2: packed stream is too short")
+    if I % 256 != 0 or O % 8 != 0:
+        raise RuntimeError("linear_grad_weight needs in_features % 256 == 0 and out_features % 8 == 0")
+    G = I // 256
+    if scale.numel() != M * G or min.numel() != scale.numel() or min.dtype != scale.dtype:
+        raise RuntimeError("linear_grad_weight: scale/min do not match the packed input")
+    if mixed:
+        g.check_typed(bits, "bits", torch.int32, 1)
+        if bits.numel() != M:
+            raise RuntimeError("linear_grad_weight: one width per row expected")
+        total, prefix = _bits_info(bits)
+        if packed.numel() < (total * G * 256 + 31) // 32:
+            raise RuntimeError("linear_grad_weight: packed stream is too short")
+        bits_ptr, prefix_ptr, fixed = bits.data_ptr(), prefix.data_ptr(), 0
+    else:
+        fixed = int(bits)
+        if fixed not in (1, 2, 4, 8):
+            raise RuntimeError("linear_grad_weight: 8 % bits must be 0")
+        if packed.numel() < single_packed_bytes(M, G, 256, fixed) - 1:
+            raise RuntimeError("linear_grad_weight: packed stream is too short")
+        bits_ptr = prefix_ptr = None
     out_dtype = out_dtype or grad_output.dtype
     gw = torch.empty(O, I, dtype=out_dtype, device=grad_output.device)
     with g.on_device(gw.device):
-        check(g.lib().actnn_linear_grad_weight_q2(
-            grad_output.data_ptr(), packed.data_ptr(), scale.data_ptr(), min.data_ptr(), gw.data_ptr(),
-            M, O, I, g.DTYPE_CODE[grad_output.dtype], g.DTYPE_CODE[scale.dtype], g.DTYPE_CODE[out_dtype],
-            g.stream_ptr(gw.device)), "linear_grad_weight_q2")
+        check(g.lib().actnn_linear_grad_weight(
+            grad_output.data_ptr(), packed.data_ptr(), bits_ptr, prefix_ptr, fixed, scale.data_ptr(),
+            min.data_ptr(), gw.data_ptr(), M, O, I, g.DTYPE_CODE[grad_output.dtype], g.DTYPE_CODE[scale.dtype],
+            g.DTYPE_CODE[out_dtype], g.stream_ptr(gw.device)), "linear_grad_weight")
     return gw
+
+
+def linear_grad_weight_q2(grad_output, packed, scale, min, in_features, out_dtype=None):
+    """The 2-bit fixed-width case of linear_grad_weight (rows in whole groups of four)."""
+    if grad_output.dim() == 2 and grad_output.shape[0] % 4 != 0:
+        raise RuntimeError("linear_grad_weight_q2 needs M % 4 == 0")
+    return linear_grad_weight(grad_output, packed, 2, scale, min, in_features, out_dtype)
 
 
 # ------------------------------------------------------------------------------------------

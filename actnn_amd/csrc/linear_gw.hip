@@ -3,32 +3,41 @@
 //
 //     grad_w[O, I] = grad_out[M, O]^T @ dequant(x)[M, I]
 //
-// x stays in the 2-bit fixed-width stream (byte ((m/4) * I/256 + g) * 256 + d holds rows
-// 4*(m/4) .. +3 of feature g*256 + d, two bits each) with scale/min[M, I/256].  The full
-// precision input is never written to memory: every k-step the 2-bit tile is unpacked,
-// dequantised (code * (1/scale) + min) and narrowed to 16 bits straight into the LDS tile that feeds
-// v_mfma_f32_32x32x16_bf16 (bf16 gradients) or v_mfma_f32_32x32x16_f16 (fp16 gradients), with
-// fp32 accumulation.
+// x stays in the stream the pack kernels wrote - the fixed-width stream (byte
+// ((m / w) * I/256 + g) * 256 + d holds the w = 8/bits rows m of feature g*256 + d) or the
+// mixed-width stream (per-sample widths, 32-lane ballot words) - with scale/min[M, I/256].  The
+// full precision input is never written to memory: every k-step the tile is unpacked, dequantised
+// and narrowed to the 16-bit format of grad_out straight into the LDS tile that feeds
+// v_mfma_f32_32x32x16_bf16 / _f16, fp32 accumulation.
 //
 // Tiling: the reduction runs over the samples m (K of the GEMM).  A 512-thread block (one per CU)
 // owns a 256 (O) x 256 (I) output tile - one whole quantisation group, so a block needs one
-// scale/min per sample - as 8 waves of 64 x 128, each 2 x 4 MFMA tiles of 32 x 32.  The large tile
-// is what keeps the L2 -> CU traffic (grad_out is re-read once per column tile) below what the
-// vector caches deliver.  Per k-step of 64 samples (LDS tiles double-buffered, one barrier a step):
-//   * grad_out lies o-contiguous in memory but MFMA fragments want 8 consecutive k per row, so a
-//     thread loads 4 consecutive k-rows x 8 o's (16-byte vectors, a wave covers whole rows of the
-//     tile), transposes them in registers with 16 byte-permutes and writes 8 rows of 4 k's;
-//   * the packed bytes already hold 4 consecutive k per feature: a thread unpacks 2 x (4 features
-//     x 4 samples) from two 32-bit loads and writes them k-contiguous.  A wave works on 8
-//     consecutive samples: 16 lanes fetch their 8 scales and 8 minima with one load and v_readlane
-//     hands them out (scalar loads of one value per cache line were 40% of the kernel's time).
-//   Both LDS tiles are [row][k] with a 144-byte pitch, every MFMA fragment is one 16-byte LDS read.
-//   Rows are stored permuted - tile row o at LDS row (o % 8) * 32 + o / 8, tile column i at LDS row
-//   (i % 4) * 64 + i / 4 - which makes lane pairs of a staging write fill 16 contiguous bytes of
-//   consecutive LDS rows (no bank conflicts) and lets the epilogue store 4 consecutive columns
-//   per lane.
-// Global loads run two steps ahead of the MFMAs (two register sets), LDS writes one step ahead.
-#include "device_utils.h"
+// scale/min per sample - as 8 waves of 64 (O) x 128 (I).  Per k-step of 64 samples, LDS tiles
+// double-buffered, one barrier a step:
+//   * Both operand tiles lie in LDS the way they lie in memory: [sample][column], 512 bytes a row.
+//     MFMA fragments want 8 consecutive samples of one column per lane; the transposing LDS read
+//     (ds_read_b64_tr_b16: a 16-lane block that points at four rows of four 8-byte units gets back,
+//     lane by lane, four consecutive samples of 16 consecutive columns) delivers exactly that, two
+//     reads per fragment and no register transposes.  The 16-byte chunks of a row are stored at
+//     chunk ^ ((sample & 7) << 2): the four rows that 32 lanes of such a read touch (64 bytes each)
+//     then fall into the four quarters of the 64 banks, and the two reads of a fragment into
+//     different halves of the row (measured: 1.4 times the rate of a swizzle that only separates
+//     the rows within 16 lanes, 2.7 times no swizzle).
+//   * grad_out tiles go from global memory straight into LDS (global_load_lds, 16 bytes per lane,
+//     the swizzle applied to the source address): no registers, no VALU work.
+//   * the 2-bit fixed-width stream: a thread takes one 32-bit load = 4 features x 4 samples.  The
+//     four possible values of a sample, code / scale + min exactly as unpack_single rounds them,
+//     are a table of eight bytes per sample (computed once per wave and step); v_perm_b32 with the
+//     2-bit codes as byte selectors picks the low and the high bytes of four values at a time: 1.5
+//     VALU instructions per value instead of extract + convert + multiply-add + narrow.
+//   * any other stream (mixed widths; fixed 1, 4, 8 bits) takes a general loader: a lane unpacks
+//     8 consecutive features of one sample (bit transpose as in unpack_mixed, or byte fields),
+//     dequantises them with the unpack kernels' arithmetic and writes 16 bytes of the row.
+//   The roles of the operands are chosen so that an accumulator register quad holds four
+//   consecutive columns of grad_w: the epilogue stores 16 bytes (fp32) per lane and register quad.
+// Loads of packed data and scale/min run one step ahead of the staging code (widths and stream
+// offsets of the mixed stream two steps ahead).
+#include "quant_math.h"
 
 namespace actnn {
 namespace {
@@ -36,22 +45,32 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 512;
-constexpr int BM = 256;            // output rows (O) per block
-constexpr int BN = 256;            // output columns (I) per block: one quantisation group
-constexpr int BK = 64;             // samples per k-step
-constexpr int kPitch = BK + 8;     // 16-bit elements per row of either LDS tile (144 bytes)
-constexpr int kTile = 256 * kPitch;                 // elements of one operand tile
-constexpr int kLdsBytes = 2 * 2 * kTile * 2;        // two operands, two buffers
+constexpr int kWaves = kThreads / 64;
+constexpr int BM = 256;             // output rows (O) per block
+constexpr int BN = 256;             // output columns (I) per block: one quantisation group
+constexpr int BK = 64;              // samples per k-step
+constexpr int kRowBytes = 512;      // one sample of either tile: 256 16-bit values
+constexpr int kTileBytes = BK * kRowBytes;
+constexpr int kTabBytes = kWaves * 2 * 64;          // per wave and buffer: 8 samples x 8 bytes
 
-// The MFMA runs in the 16-bit format of grad_out, so its rows go to LDS exactly as loaded:
-// bf16 gradients (bf16 autocast) use v_mfma_f32_32x32x16_bf16 and the dequantised activations are
-// rounded to bf16 (nearest even); fp16 gradients use v_mfma_f32_32x32x16_f16 and the activations
-// are narrowed to fp16 with v_cvt_pkrtz (truncation: 2^-11 relative, far below a 2-bit step).
+template <int N> struct Slot { static constexpr int value = N; };
+template <int N, typename F> ACTNN_DEV void for_each_slot(F&& f) {
+  if constexpr (N > 0) {
+    for_each_slot<N - 1>(f);
+    f(Slot<N - 1>{});
+  }
+}
+
+// byte offset of 16-byte chunk `ch` of row `k` inside a tile (the swizzle described above)
+ACTNN_DEV int chunk_offset(int k, int ch) { return k * kRowBytes + ((ch ^ ((k & 7) << 2)) << 4); }
+
 template <typename TG> struct Mma;
 template <> struct Mma<bf16_t> {
   static ACTNN_DEV uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
+  static ACTNN_DEV uint32_t bits16(float v) { return float_to_bf16_bits(v); }
   static ACTNN_DEV f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
@@ -59,26 +78,13 @@ template <> struct Mma<bf16_t> {
 };
 template <> struct Mma<__half> {
   static ACTNN_DEV uint32_t pack2(float lo, float hi) {
-    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
+    return float_to_half_bits(lo) | (float_to_half_bits(hi) << 16);
   }
+  static ACTNN_DEV uint32_t bits16(float v) { return float_to_half_bits(v); }
   static ACTNN_DEV f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
                                                   __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   }
-};
-
-template <typename T> struct RawScalar;          // a scale/min value exactly as loaded
-template <> struct RawScalar<float> {
-  static ACTNN_DEV uint32_t load(const float* p, int64_t i) { return as_uint(p[i]); }
-  static ACTNN_DEV float widen(uint32_t v) { return as_float(v); }
-};
-template <> struct RawScalar<__half> {
-  static ACTNN_DEV uint32_t load(const __half* p, int64_t i) { return reinterpret_cast<const uint16_t*>(p)[i]; }
-  static ACTNN_DEV float widen(uint32_t v) { return half_bits_to_float(v); }
-};
-template <> struct RawScalar<bf16_t> {
-  static ACTNN_DEV uint32_t load(const bf16_t* p, int64_t i) { return p[i].bits; }
-  static ACTNN_DEV float widen(uint32_t v) { return bf16_bits_to_float(v); }
 };
 
 template <typename TO> ACTNN_DEV void store_out4(TO* p, float a, float b, float c, float d);
@@ -93,18 +99,244 @@ template <> ACTNN_DEV void store_out4<bf16_t>(bf16_t* p, float a, float b, float
   *reinterpret_cast<u32x2*>(p) = (u32x2){pack_bf16x2(a, b), pack_bf16x2(c, d)};
 }
 
-template <typename TG, typename TS, typename TO>
-__global__ __launch_bounds__(kThreads, 1) void linear_gw_q2_kernel(
-    const TG* __restrict__ gout, const uint8_t* __restrict__ packed, const TS* __restrict__ scale,
-    const TS* __restrict__ mn, TO* __restrict__ gw, int M, int O, int I) {
-  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-  auto tileA = [&](int buf) { return smem + buf * 2 * kTile; };
-  auto tileB = [&](int buf) { return smem + buf * 2 * kTile + kTile; };
+// A scale / min value exactly as loaded: nothing may consume a load where it is issued (the wave would
+// wait out the memory latency there), so prefetched values stay raw until the staging code runs.
+template <typename T> struct RawScalar;
+template <> struct RawScalar<float> {
+  static ACTNN_DEV uint32_t load(const float* p, int64_t i) { return as_uint(p[i]); }
+  static ACTNN_DEV float widen(uint32_t v) { return as_float(v); }
+};
+template <> struct RawScalar<__half> {
+  static ACTNN_DEV uint32_t load(const __half* p, int64_t i) { return reinterpret_cast<const uint16_t*>(p)[i]; }
+  static ACTNN_DEV float widen(uint32_t v) { return half_bits_to_float(v); }
+};
+template <> struct RawScalar<bf16_t> {
+  static ACTNN_DEV uint32_t load(const bf16_t* p, int64_t i) { return p[i].bits; }
+  static ACTNN_DEV float widen(uint32_t v) { return bf16_bits_to_float(v); }
+};
+
+// four consecutive samples of this lane's column (see the file comment for the lane pattern)
+ACTNN_DEV u32x2 read_transposed(const uint8_t* p) {
+  const i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) i16x4*)(p));
+  return __builtin_bit_cast(u32x2, v);
+}
+
+// 16 bytes per lane from global memory straight into LDS: lane l's data lands at lds_base + 16 * l
+// (lds_base uniform in the wave).  Written as an instruction sequence of its own: the load is
+// asynchronous and the code that issues it waits for it explicitly (vmcnt) before the barrier that
+// publishes the tile; issued through the compiler's builtin, every LDS read that follows - also of
+// the other buffer - would first wait for all loads in flight.
+ACTNN_DEV void load_to_lds16(const void* src, const uint8_t* lds_base) {
+  const uint32_t base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)lds_base;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(base)), "v"(src)
+               : "memory");
+}
+
+// What describes the packed input.  bits == nullptr: the fixed-width stream at `fixed_bits`.
+struct Stream {
+  const uint8_t* packed;
+  const int32_t* bits;
+  const int32_t* prefix;
+  int fixed_bits;
+};
+
+// ------------------------------------------------------------------------------------------
+// Loader of the 2-bit fixed-width stream (table + byte permutes)
+// ------------------------------------------------------------------------------------------
+template <typename TG, typename TS> struct TableLoader {
+  uint32_t rb[2];          // this lane's 32-bit loads of the wave's two sample quads
+  uint32_t rsc, rmn;       // scale / min (raw) of sample (lane / 4) % 8 of the wave's eight
+  u32x2 tt[8];             // the wave's eight table entries, read back from LDS
+  const uint8_t* pb0;      // this lane's bytes of quad 0
+  const TS* psc0;          // scale / min of sample 0 in the block's group
+  const TS* pmn0;
+  int next;                // first sample of the step the next prefetch loads
+  int M, G, quad_rows;     // quad_rows: bytes from one sample quad to the next in the stream
+
+  ACTNN_DEV void init(const Stream& st, const TS* scale, const TS* mn, int M_, int G_, int g, int wave, int lane) {
+    M = M_;
+    G = G_;
+    next = 0;
+    quad_rows = G * 256;
+    pb0 = st.packed + (int64_t)g * 256 + lane * 4;
+    psc0 = scale + g;
+    pmn0 = mn + g;
+  }
+  // (no branches: out-of-range quads and samples read the last valid one and are ignored later -
+  // the table gives samples past M the value 0 for every code - so that the loop body stays one
+  // basic block and the compiler's wait counts for LDS stay exact)
+  ACTNN_DEV void prefetch() {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int first = next + wave * 8;
+    const int last_quad = (M - 1) >> 2;
+#pragma unroll
+    for (int qq = 0; qq < 2; ++qq) {
+      int quad = (first >> 2) + qq;
+      quad = quad < last_quad ? quad : last_quad;
+      rb[qq] = *reinterpret_cast<const uint32_t*>(pb0 + (int64_t)quad * quad_rows);
+    }
+    int smp = first + ((lane >> 2) & 7);
+    smp = smp < M - 1 ? smp : M - 1;
+    rsc = RawScalar<TS>::load(psc0, (int64_t)smp * G);
+    rmn = RawScalar<TS>::load(pmn0, (int64_t)smp * G);
+    next += BK;
+  }
+  // The staging work of a step, cut into pieces that the main loop places between its MFMAs (slot
+  // numbers are the loop's).  `tab`: this wave's 64 table bytes; kfirst: first sample of the tile.
+  template <int SLOT> ACTNN_DEV void piece(uint8_t* tile, uint8_t* tab, int kfirst) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if constexpr (SLOT == 4) {
+      // value of code (lane & 3) for sample (lane / 4) % 8, rounded exactly as unpack_single rounds it
+      // (the two half-waves compute and write the same bytes: no branch)
+      const int smp = (lane >> 2) & 7;
+      const bool valid = kfirst + wave * 8 + smp < M;
+      const Dequant<TS> dq(RawScalar<TS>::widen(rsc), RawScalar<TS>::widen(rmn));
+      const uint32_t v = valid ? Mma<TG>::bits16(dq((uint32_t)(lane & 3))) : 0u;
+      uint8_t* t = tab + smp * 8 + (lane & 3);
+      t[0] = (uint8_t)v;            // low bytes of the sample's four values, then their high bytes
+      t[4] = (uint8_t)(v >> 8);
+    } else if constexpr (SLOT == 6) {
+      // same wave writes and reads: LDS operations of a wave complete in order
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int i = 0; i < 8; ++i) tt[i] = *reinterpret_cast<const u32x2*>(tab + i * 8);
+    } else if constexpr (SLOT >= 8 && SLOT < 16) {
+      constexpr int qq = (SLOT - 8) / 4, j = (SLOT - 8) % 4;
+      const int ch = lane >> 1, half = (lane & 1) * 8;
+      const uint32_t sel = (rb[qq] >> (2 * j)) & 0x03030303u;       // codes of 4 features as byte selectors
+      const uint32_t lo = __builtin_amdgcn_perm(0u, tt[qq * 4 + j].x, sel);
+      const uint32_t hi = __builtin_amdgcn_perm(0u, tt[qq * 4 + j].y, sel);
+      const u32x2 out = {__builtin_amdgcn_perm(hi, lo, 0x05010400u), __builtin_amdgcn_perm(hi, lo, 0x07030602u)};
+      const int k = wave * 8 + qq * 4 + j;
+      *reinterpret_cast<u32x2*>(tile + chunk_offset(k, ch) + half) = out;
+    } else if constexpr (SLOT == 20) {
+      prefetch();
+    }
+  }
+};
+
+// ------------------------------------------------------------------------------------------
+// General loader: any fixed width, and the mixed-width stream.  A half-wave takes four samples of
+// a step; lane j unpacks features 8j .. 8j+7 of each.
+// ------------------------------------------------------------------------------------------
+template <typename TG, typename TS> struct GeneralLoader {
+  static constexpr int U = 4;          // samples per half-wave and step
+  uint32_t w0[U], w1[U];               // packed data of the step being loaded
+  uint32_t rsc[U], rmn[U];             // raw scale / min
+  int wb[U];                           // widths that belong to w0/w1 (mixed stream)
+  int nb[U];                           // widths and stream offsets of the step after (mixed stream)
+  int64_t nbase[U];
+  Stream st;
+  const TS* scale;
+  const TS* mn;
+  int M, G, g, next_data, next_bits;
+
+  ACTNN_DEV void init(const Stream& st_, const TS* scale_, const TS* mn_, int M_, int G_, int g_) {
+    st = st_; scale = scale_; mn = mn_; M = M_; G = G_; g = g_;
+    next_data = next_bits = 0;
+#pragma unroll
+    for (int u = 0; u < U; ++u) { nb[u] = 0; nbase[u] = 0; wb[u] = 0; w0[u] = w1[u] = 0u; rsc[u] = rmn[u] = 0u; }
+    if (st.bits) prefetch_bits();
+  }
+  ACTNN_DEV void prefetch_bits() {
+    const int hw = threadIdx.x >> 5;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int m = next_bits + hw * U + u;
+      nb[u] = 0;
+      nbase[u] = 0;
+      if (m < M) {
+        nb[u] = st.bits[m];
+        nbase[u] = ((int64_t)st.prefix[m] * G + (int64_t)nb[u] * g) * 8;      // first word of (m, g)
+      }
+    }
+    next_bits += BK;
+  }
+  ACTNN_DEV void prefetch() {
+    const int hw = threadIdx.x >> 5, j = threadIdx.x & 31;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int m = next_data + hw * U + u;
+      w0[u] = w1[u] = 0u;
+      rsc[u] = rmn[u] = 0u;
+      wb[u] = st.bits ? nb[u] : st.fixed_bits;
+      if (m < M) {
+        if (st.bits) {
+          const int32_t* words = reinterpret_cast<const int32_t*>(st.packed) + nbase[u];
+          const int n_words = 8 * wb[u];
+          if (j < n_words) w0[u] = (uint32_t)words[j];
+          if (32 + j < n_words) w1[u] = (uint32_t)words[32 + j];
+        } else {
+          const int wpt = 8 / st.fixed_bits;
+          const u32x2 v = *reinterpret_cast<const u32x2*>(st.packed + ((int64_t)(m / wpt) * G + g) * 256 + j * 8);
+          w0[u] = v.x;
+          w1[u] = v.y;
+        }
+        rsc[u] = RawScalar<TS>::load(scale, (int64_t)m * G + g);
+        rmn[u] = RawScalar<TS>::load(mn, (int64_t)m * G + g);
+      }
+    }
+    next_data += BK;
+    if (st.bits) prefetch_bits();
+  }
+  template <int SLOT> ACTNN_DEV void piece(uint8_t* tile, uint8_t*, int kfirst) {
+    if constexpr (SLOT == 4) stage(tile, kfirst);
+    else if constexpr (SLOT == 20) prefetch();
+  }
+  ACTNN_DEV void stage(uint8_t* tile, int kfirst) {
+    const int hw = threadIdx.x >> 5, j = threadIdx.x & 31;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = hw * U + u;
+      const int m = kfirst + k;
+      const int b = wb[u];
+      u32x4 out = {0u, 0u, 0u, 0u};
+      // the exchange below involves every lane: no lane may skip it (b is uniform per half-wave)
+      uint64_t codes;
+      int shift, step;
+      if (st.bits) {
+        codes = (uint64_t)transpose32(w0[u], (uint32_t)j) | ((uint64_t)transpose32(w1[u], (uint32_t)j) << 32);
+        shift = 0;
+        step = b;                       // code of feature 8j + e: bits [e*b, e*b + b)
+      } else {
+        codes = (uint64_t)w0[u] | ((uint64_t)w1[u] << 32);
+        shift = (m % (8 / st.fixed_bits)) * b;      // byte e holds feature 8j + e, this sample at `shift`
+        step = 8;
+      }
+      if (m < M && b >= 1 && b <= 8) {
+        const uint32_t mask = (1u << b) - 1u;
+        const Dequant<TS> dq(RawScalar<TS>::widen(rsc[u]), RawScalar<TS>::widen(rmn[u]));
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = dq((uint32_t)(codes >> (e * step + shift)) & mask);
+        out = (u32x4){Mma<TG>::pack2(v[0], v[1]), Mma<TG>::pack2(v[2], v[3]),
+                      Mma<TG>::pack2(v[4], v[5]), Mma<TG>::pack2(v[6], v[7])};
+      }
+      *reinterpret_cast<u32x4*>(tile + chunk_offset(k, j)) = out;
+    }
+  }
+};
+
+template <typename TG, typename TS, typename TO, bool TABLE>
+__global__ __launch_bounds__(kThreads, 1) void linear_gw_kernel(
+    const TG* __restrict__ gout, Stream st, const TS* __restrict__ scale, const TS* __restrict__ mn,
+    TO* __restrict__ gw, int M, int O, int I) {
+  // grad_out tiles first: the direct loads address LDS through M0, keep their targets low
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * kTileBytes + kTabBytes];
+  auto tileG = [&](int buf) { return smem + buf * kTileBytes; };
+  auto tileX = [&](int buf) { return smem + (2 + buf) * kTileBytes; };
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wr = wave & 3, wn = wave >> 2;   // the wave's 64-row group and 128-column half
+  const int wr = wave & 3, wn = wave >> 2;   // the wave's 64 rows (O) and 128 columns (I) of the tile
   const int G = I / 256;
   // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give every XCD whole
   // panels of grad_out rows (all column tiles of tile_m), so that a panel is pulled into one L2
@@ -119,210 +351,186 @@ __global__ __launch_bounds__(kThreads, 1) void linear_gw_q2_kernel(
   const int o0 = (tile / tiles_n) * BM;
   const int g = tile % tiles_n;              // the block's columns are quantisation group g
   const int i0 = g * 256;
+  uint8_t* tab = smem + 4 * kTileBytes + wave * 128;
 
-  // A wave stages the sample quads 2 * wave and 2 * wave + 1 (8 consecutive samples) of a step.
-  // Neighbouring lanes take the two quads of the same row, so that the 32 lanes served by one LDS
-  // cycle write 16 rows x 16 contiguous bytes: no bank conflicts with the 144-byte pitch.
-  // A staging: thread -> k rows 4 * quad .. + 3, o offset ao * 8 (a wave: 2 quads x whole rows)
-  // B staging: thread -> the same quad, features 4 * fl .. + 3 and 128 + 4 * fl .. + 3
-  const int par = lane & 1;
-  const int quad = 2 * wave + par;
-  const int ao = lane >> 1, fl = lane >> 1;
-  const bool ovalid = o0 + ao * 8 < O;       // O % 8 == 0: a vector is inside or outside as a whole
-  // running pointers / indices, advanced by one k-step per prefetch
-  const TG* pa = gout + (int64_t)(quad * 4) * O + o0 + ao * 8;
-  const uint8_t* pb = packed + ((int64_t)quad * G + g) * 256 + fl * 4;
-  int64_t si = (int64_t)(wave * 8) * G + g;  // index of the wave's first sample in scale / min
-  const int64_t a_step = (int64_t)BK * O;
-  const int64_t b_step = (int64_t)(BK / 4) * G * 256;
-  const int64_t s_step = (int64_t)BK * G;
-
-  f32x16 acc[2][4];
-#pragma unroll
-  for (int a = 0; a < 2; ++a)
-#pragma unroll
-    for (int b = 0; b < 4; ++b)
-#pragma unroll
-      for (int c = 0; c < 16; ++c) acc[a][b][c] = 0.0f;
-
-  // The prefetch registers hold the data of the step after the one being multiplied, exactly as
-  // loaded (nothing may consume a load where it is issued, or the wave would wait out the memory
-  // latency there).  They are refilled as soon as the staging code has read them, most of a
-  // k-step before they are needed again.
-  u32x4 ra[4];
-  uint32_t rb[2];
-  uint32_t rsm = 0u;                         // lanes 0..15: scale / min of the wave's 8 samples
-  // lane l < 16 fetches for quad 2 * wave + l / 8: scale (l % 8 < 4) or min of its sample l % 4
-  const int sm_h = (lane >> 3) & 1, sm_j = lane & 3;
-  const TS* sm_base = (lane & 4) ? mn : scale;
-  int ka_next = 0, kb_next = 0;              // first sample of the step the next prefetch loads
-
-  auto prefetch_a = [&]() {
-    const bool avalid = ovalid && ka_next + quad * 4 < M;   // M % 4 == 0: a quad is inside or outside as a whole
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      ra[r] = (u32x4){0u, 0u, 0u, 0u};
-      if (avalid) ra[r] = load16(pa + (int64_t)r * O);
-    }
-    pa += a_step;
-    ka_next += BK;
-  };
-  auto prefetch_b = [&]() {
-    rb[0] = rb[1] = 0u;
-    if (kb_next + quad * 4 < M) {
-      rb[0] = *reinterpret_cast<const uint32_t*>(pb);
-      rb[1] = *reinterpret_cast<const uint32_t*>(pb + 128);
-    }
-    rsm = 0u;
-    if (lane < 16 && kb_next + (2 * wave + sm_h) * 4 < M)
-      rsm = RawScalar<TS>::load(sm_base, si + (int64_t)(4 * sm_h + sm_j) * G);
-    pb += b_step;
-    si += s_step;
-    kb_next += BK;
+  // ---- grad_out tile: straight from global memory into LDS.  One instruction of a wave fills 1 KiB
+  // of LDS (two rows); lane -> row 2*rp + lane/32, LDS chunk lane%32, which holds source chunk
+  // lane%32 ^ swizzle(row).  Rows past M are read from the last row (their activations are staged as
+  // zeros, so any finite value will do), columns past O from the block's first column (they only
+  // reach output rows that are not stored): every lane loads, nothing else writes these tiles.
+  const int g_row = lane >> 5;
+  // rows of one instruction: 2 * rp + g_row with rp = 8 * jj + wave, so (row & 7) only depends on the wave
+  const int g_chunk = (lane & 31) ^ (((2 * (wave & 3) + g_row) & 7) << 2);
+  const int g_col = o0 + g_chunk * 8 < O ? o0 + g_chunk * 8 : o0;
+  auto load_g_piece = [&](uint8_t* tile_g, int kfirst, int jj) {
+    const int rp = jj * 8 + wave;                         // row pair of the tile, uniform in the wave
+    int m = kfirst + 2 * rp + g_row;
+    m = m < M ? m : M - 1;
+    load_to_lds16(gout + (int64_t)m * O + g_col, tile_g + rp * 2 * kRowBytes);
   };
 
-  // 4 (k) x 8 (o) -> 8 (o) x 4 (k): word p of ra[r] holds o = 2p (low half) and 2p + 1 (high half)
-  auto stage_a = [&](int buf) {
-    uint16_t* sA = tileA(buf);
-#pragma unroll
-    for (int p2 = 0; p2 < 4; ++p2) {
-      const uint32_t w0 = ra[0][p2], w1 = ra[1][p2], w2 = ra[2][p2], w3 = ra[3][p2];
-      const u32x2 even = {__builtin_amdgcn_perm(w1, w0, 0x05040100u), __builtin_amdgcn_perm(w3, w2, 0x05040100u)};
-      const u32x2 odd = {__builtin_amdgcn_perm(w1, w0, 0x07060302u), __builtin_amdgcn_perm(w3, w2, 0x07060302u)};
-      *reinterpret_cast<u32x2*>(&sA[((2 * p2) * 32 + ao) * kPitch + quad * 4]) = even;
-      *reinterpret_cast<u32x2*>(&sA[((2 * p2 + 1) * 32 + ao) * kPitch + quad * 4]) = odd;
-    }
+  // ---- fragments: lane -> column n0 + lane%32, samples 16*kb + 8*(lane/32) + 0..7
+  const int blk = lane >> 4, r = lane & 15;
+  const int f_row = 8 * (blk >> 1) + (r >> 2);
+  // chunk of column block n0 = 32*q: 4*q + 2*(blk&1) + ((r&3)>>1); bytes inside the chunk: (r&1)*8
+  auto frag_offset = [&](int n0) {
+    const int ch = n0 / 8 + 2 * (blk & 1) + ((r & 3) >> 1);
+    return chunk_offset(f_row, ch) + (r & 1) * 8;
   };
-  // the step whose first sample is kfirst (rows past M dequantise to 0; their grad_out rows were
-  // loaded as 0)
-  auto stage_b = [&](int buf, int kfirst) {
-    uint16_t* sB = tileB(buf);
-    const bool bvalid = kfirst + quad * 4 < M;
-    float inv[4], m4[4];
+  int offx[4], offg[2];          // first read of a fragment; the second (4 rows on) lies at (offset ^ 256) + 4 rows
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint32_t sc0 = (uint32_t)__builtin_amdgcn_readlane((int)rsm, j);
-      const uint32_t mn0 = (uint32_t)__builtin_amdgcn_readlane((int)rsm, 4 + j);
-      const uint32_t sc1 = (uint32_t)__builtin_amdgcn_readlane((int)rsm, 8 + j);
-      const uint32_t mn1 = (uint32_t)__builtin_amdgcn_readlane((int)rsm, 12 + j);
-      inv[j] = bvalid ? __builtin_amdgcn_rcpf(RawScalar<TS>::widen(par ? sc1 : sc0)) : 0.0f;
-      m4[j] = bvalid ? RawScalar<TS>::widen(par ? mn1 : mn0) : 0.0f;
-    }
+  for (int e = 0; e < 4; ++e) offx[e] = frag_offset(wn * 128 + 32 * e);
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+  for (int a = 0; a < 2; ++a) offg[a] = frag_offset(wr * 64 + 32 * a);
+
+  f32x16 acc[4][2];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const uint32_t by = rb[h] >> (8 * e);
-        const float x0 = fmaf((float)(by & 3u), inv[0], m4[0]);
-        const float x1 = fmaf((float)((by >> 2) & 3u), inv[1], m4[1]);
-        const float x2 = fmaf((float)((by >> 4) & 3u), inv[2], m4[2]);
-        const float x3 = fmaf((float)((by >> 6) & 3u), inv[3], m4[3]);
-        *reinterpret_cast<u32x2*>(&sB[(e * 64 + 32 * h + fl) * kPitch + quad * 4]) =
-            (u32x2){Mma<TG>::pack2(x0, x1), Mma<TG>::pack2(x2, x3)};
-      }
-    }
+  for (int e = 0; e < 4; ++e)
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int c = 0; c < 16; ++c) acc[e][a][c] = 0.0f;
+
+  // fragment f of k-block kb: f = 0..3 activations (MFMA rows), 4..5 grad_out (MFMA columns);
+  // double-buffered in registers by the parity of kb
+  u32x4 fx[2][4], fg[2][2];
+  auto read_fragment = [&](const uint8_t* tile_g, const uint8_t* tile_x, auto KB, auto F) {
+    constexpr int kb = decltype(KB)::value, f = decltype(F)::value;
+    const int off = f < 4 ? offx[f < 4 ? f : 0] : offg[f < 4 ? 0 : f - 4];
+    const uint8_t* tile = (f < 4 ? tile_x : tile_g) + kb * 16 * kRowBytes;
+    const u32x2 lo = read_transposed(tile + off);
+    const u32x2 hi = read_transposed(tile + (off ^ 256) + 4 * kRowBytes);
+    const u32x4 v = {lo.x, lo.y, hi.x, hi.y};
+    if constexpr (f < 4) fx[kb & 1][f] = v; else fg[kb & 1][f - 4] = v;
   };
 
-  // Fragments are double-buffered in registers: those of k-block kb+1 are requested before the
-  // MFMAs of k-block kb are issued, so the matrix pipe does not wait for LDS inside a step.
-  u32x4 fa[2][2], fb[2][4];
-  auto fragments = [&](int buf, int kb) {
-    const uint16_t* sA = tileA(buf) + ((2 * wr) * 32 + (lane & 31)) * kPitch + (lane >> 5) * 8;
-    const uint16_t* sB = tileB(buf) + (wn * 32 + (lane & 31)) * kPitch + (lane >> 5) * 8;
-#pragma unroll
-    for (int a = 0; a < 2; ++a) fa[kb & 1][a] = *reinterpret_cast<const u32x4*>(sA + a * 32 * kPitch + kb * 16);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) fb[kb & 1][e] = *reinterpret_cast<const u32x4*>(sB + e * 64 * kPitch + kb * 16);
-  };
-  auto mfmas = [&](int kb) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e)
-#pragma unroll
-      for (int a = 0; a < 2; ++a) acc[a][e] = Mma<TG>::mfma(fa[kb & 1][a], fb[kb & 1][e], acc[a][e]);
-  };
-  auto multiply_step = [&](int buf) {
-    fragments(buf, 0);
-#pragma unroll
-    for (int kb = 0; kb < BK / 16; ++kb) {
-      // keep the compiler from sinking the reads of kb+1 below the MFMAs of kb
-      __builtin_amdgcn_sched_barrier(0);
-      if (kb + 1 < BK / 16) fragments(buf, kb + 1);
-      __builtin_amdgcn_sched_barrier(0);
-      mfmas(kb);
-    }
-  };
-  auto stage_step = [&](int j) {             // write tile j, then get the loads of tile j+1 in flight
-    stage_a(j & 1);
-    stage_b(j & 1, j * BK);
-    prefetch_a();
-    prefetch_b();
-  };
-
-  // Step t is multiplied out of LDS buffer t % 2 while the tile of step t+1 is written into the
-  // other buffer (its last readers passed the barrier at the end of step t-1) and the loads of
-  // step t+2 are issued: one barrier per step.
   const int steps = (M + BK - 1) / BK;
-  prefetch_a();
-  prefetch_b();
-  if (steps > 0) stage_step(0);
-  __syncthreads();
-  for (int t = 0; t < steps; ++t) {
-    if (t + 1 < steps) stage_step(t + 1);
-    multiply_step(t & 1);
+  // The schedule.  Step t is multiplied out of LDS buffer t % 2; the tiles of step t+1 go into the
+  // other buffer, whose last readers finished before the barrier that ended step t-1.  Between two
+  // barriers a wave issues 32 MFMAs - the last k-block of the step before (its fragments were read
+  // before the barrier) and the first three of this step - and everything else is cut into pieces
+  // placed between them, so that the matrix pipe always has work queued while the wave computes
+  // addresses, permutes bytes and waits for LDS:
+  //   MFMA slot  0.. 7: k-block 3 of step t-1 | direct loads of G(t+1), table of X(t+1), reads (t, 0)
+  //   MFMA slot  8..15: k-block 0 of step t   | the eight staging pieces of X(t+1), reads (t, 1)
+  //   MFMA slot 16..23: k-block 1             | loads for X(t+2), reads (t, 2)
+  //   MFMA slot 24..31: k-block 2             | reads (t, 3)
+  //   wait for the direct loads; barrier
+  // Fragment reads are issued eight MFMAs ahead of their use, into the register set the MFMAs of
+  // the same slots do not read.
+  // The body between two barriers has no branches (first / last step are separate copies): with
+  // branches around the pieces the compiler's LDS wait counts lose one position per join and every
+  // MFMA ends up waiting for reads issued a moment before it.
+  auto step = [&](auto& ld, auto FIRST, auto MORE, int t) {
+    constexpr bool first = decltype(FIRST)::value != 0, more = decltype(MORE)::value != 0;
+    const uint8_t* cur_g = tileG(t & 1);
+    const uint8_t* cur_x = tileX(t & 1);
+    const int nb = (t + 1) & 1;
+    for_each_slot<32>([&](auto S) {
+      constexpr int slot = decltype(S)::value;
+      constexpr int kb_mfma = (slot / 8 + 3) % 4, e = (slot % 8) / 2, a = slot % 2;
+      if constexpr (slot >= 8 || !first)
+        acc[e][a] = Mma<TG>::mfma(fx[kb_mfma & 1][e], fg[kb_mfma & 1][a], acc[e][a]);
+      // the two grad_out fragments first: the first MFMAs of the next group need them
+      if constexpr (slot % 8 < 6) read_fragment(cur_g, cur_x, Slot<slot / 8>{}, Slot<(slot % 8 + 4) % 6>{});
+      if constexpr (more) {
+        if constexpr (slot < 4) load_g_piece(tileG(nb), (t + 1) * BK, slot);
+        ld.template piece<slot>(tileX(nb), tab + nb * 64, (t + 1) * BK);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
+  };
+  auto run = [&](auto& ld) {
+    if (steps > 0) {
+      ld.prefetch();
+      for_each_slot<32>([&](auto S) { ld.template piece<(decltype(S)::value == 20 ? 31 : decltype(S)::value)>(tileX(0), tab, 0); });
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) load_g_piece(tileG(0), 0, jj);
+      ld.prefetch();
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (steps == 1) {
+      step(ld, Slot<1>{}, Slot<0>{}, 0);
+    } else if (steps > 1) {
+      step(ld, Slot<1>{}, Slot<1>{}, 0);
+      for (int t = 1; t + 1 < steps; ++t) step(ld, Slot<0>{}, Slot<1>{}, t);
+      step(ld, Slot<0>{}, Slot<0>{}, steps - 1);
+    }
+    if (steps > 0) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int a = 0; a < 2; ++a) acc[e][a] = Mma<TG>::mfma(fx[1][e], fg[1][a], acc[e][a]);
+    }
+  };
+  if constexpr (TABLE) {
+    TableLoader<TG, TS> ld;
+    ld.init(st, scale, mn, M, G, g, wave, lane);
+    run(ld);
+  } else {
+    GeneralLoader<TG, TS> ld;
+    ld.init(st, scale, mn, M, G, g);
+    run(ld);
   }
 
-  // 32x32 accumulator layout: register c of a lane is fragment row 8*(c/4) + 4*(lane/32) + c%4,
-  // fragment column lane%32.  Fragment row r of A-fragment a is tile row 8*r + 2*wr + a; fragment
-  // column l of B-fragment e is tile column 128*wn + 4*l + e.
+  // 32x32 accumulator layout: register c of a lane is fragment row 8*(c/4) + 4*(lane/32) + c%4 (a
+  // column of grad_w: feature), fragment column lane%32 (a row of grad_w: output unit).
 #pragma unroll
   for (int a = 0; a < 2; ++a) {
+    const int row = o0 + wr * 64 + 32 * a + (lane & 31);
+    if (row < O) {
 #pragma unroll
-    for (int c = 0; c < 16; ++c) {
-      const int r = 8 * (c >> 2) + 4 * (lane >> 5) + (c & 3);
-      const int row = o0 + 8 * r + 2 * wr + a;
-      const int col = i0 + 128 * wn + 4 * (lane & 31);
-      if (row < O)
-        store_out4<TO>(gw + (int64_t)row * I + col, acc[a][0][c], acc[a][1][c], acc[a][2][c], acc[a][3][c]);
+      for (int e = 0; e < 4; ++e) {
+#pragma unroll
+        for (int cq = 0; cq < 4; ++cq) {
+          const int col = i0 + wn * 128 + 32 * e + 8 * cq + 4 * (lane >> 5);
+          store_out4<TO>(gw + (int64_t)row * I + col, acc[e][a][4 * cq], acc[e][a][4 * cq + 1],
+                         acc[e][a][4 * cq + 2], acc[e][a][4 * cq + 3]);
+        }
+      }
     }
   }
 }
 
 template <typename TG, typename TS, typename TO>
-int launch(const void* gout, const int8_t* packed, const void* scale, const void* mn, void* gw,
-           int64_t M, int64_t O, int64_t I, hipStream_t s) {
+int launch(const void* gout, const Stream& st, const void* scale, const void* mn, void* gw, int64_t M,
+           int64_t O, int64_t I, hipStream_t s) {
   const int64_t blocks = ((O + BM - 1) / BM) * (I / BN);
   if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
-  auto kernel = linear_gw_q2_kernel<TG, TS, TO>;
-  // more than the 64 KB a kernel may use without asking
-  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-  if (e != hipSuccess) return (int)e;
-  kernel<<<dim3((unsigned)blocks), dim3(kThreads), kLdsBytes, s>>>(
-      static_cast<const TG*>(gout), reinterpret_cast<const uint8_t*>(packed),
-      static_cast<const TS*>(scale), static_cast<const TS*>(mn), static_cast<TO*>(gw), (int)M, (int)O,
-      (int)I);
+  const bool table = !st.bits && st.fixed_bits == 2;
+  if (table) {
+    linear_gw_kernel<TG, TS, TO, true><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+        static_cast<const TG*>(gout), st, static_cast<const TS*>(scale), static_cast<const TS*>(mn),
+        static_cast<TO*>(gw), (int)M, (int)O, (int)I);
+  } else {
+    linear_gw_kernel<TG, TS, TO, false><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+        static_cast<const TG*>(gout), st, static_cast<const TS*>(scale), static_cast<const TS*>(mn),
+        static_cast<TO*>(gw), (int)M, (int)O, (int)I);
+  }
   ACTNN_RETURN_LAUNCH_STATUS();
 }
 
 template <typename TG, typename TS>
-int launch_out(int out_dtype, const void* gout, const int8_t* packed, const void* scale,
-               const void* mn, void* gw, int64_t M, int64_t O, int64_t I, hipStream_t s) {
+int launch_out(int out_dtype, const void* gout, const Stream& st, const void* scale, const void* mn,
+               void* gw, int64_t M, int64_t O, int64_t I, hipStream_t s) {
   switch (out_dtype) {
-    case ACTNN_F32: return launch<TG, TS, float>(gout, packed, scale, mn, gw, M, O, I, s);
-    case ACTNN_F16: return launch<TG, TS, __half>(gout, packed, scale, mn, gw, M, O, I, s);
-    case ACTNN_BF16: return launch<TG, TS, bf16_t>(gout, packed, scale, mn, gw, M, O, I, s);
+    case ACTNN_F32: return launch<TG, TS, float>(gout, st, scale, mn, gw, M, O, I, s);
+    case ACTNN_F16: return launch<TG, TS, __half>(gout, st, scale, mn, gw, M, O, I, s);
+    case ACTNN_BF16: return launch<TG, TS, bf16_t>(gout, st, scale, mn, gw, M, O, I, s);
     default: return ACTNN_EDTYPE;
   }
 }
 
 template <typename TG>
-int launch_sm(int sm_dtype, int out_dtype, const void* gout, const int8_t* packed, const void* scale,
+int launch_sm(int sm_dtype, int out_dtype, const void* gout, const Stream& st, const void* scale,
               const void* mn, void* gw, int64_t M, int64_t O, int64_t I, hipStream_t s) {
   switch (sm_dtype) {
-    case ACTNN_F32: return launch_out<TG, float>(out_dtype, gout, packed, scale, mn, gw, M, O, I, s);
-    case ACTNN_F16: return launch_out<TG, __half>(out_dtype, gout, packed, scale, mn, gw, M, O, I, s);
-    case ACTNN_BF16: return launch_out<TG, bf16_t>(out_dtype, gout, packed, scale, mn, gw, M, O, I, s);
+    case ACTNN_F32: return launch_out<TG, float>(out_dtype, gout, st, scale, mn, gw, M, O, I, s);
+    case ACTNN_F16: return launch_out<TG, __half>(out_dtype, gout, st, scale, mn, gw, M, O, I, s);
+    case ACTNN_BF16: return launch_out<TG, bf16_t>(out_dtype, gout, st, scale, mn, gw, M, O, I, s);
     default: return ACTNN_EDTYPE;
   }
 }
@@ -330,22 +538,36 @@ int launch_sm(int sm_dtype, int out_dtype, const void* gout, const int8_t* packe
 }  // namespace
 }  // namespace actnn
 
-extern "C" int actnn_linear_grad_weight_q2(const void* grad_out, const int8_t* packed,
-                                           const void* scale, const void* mn, void* grad_w,
-                                           int64_t M, int64_t O, int64_t I, int go_dtype,
-                                           int sm_dtype, int out_dtype, void* stream) {
+extern "C" int actnn_linear_grad_weight(const void* grad_out, const void* packed, const int32_t* bits,
+                                        const int32_t* prefix, int fixed_bits, const void* scale,
+                                        const void* mn, void* grad_w, int64_t M, int64_t O, int64_t I,
+                                        int go_dtype, int sm_dtype, int out_dtype, void* stream) {
   using namespace actnn;
-  if (M < 0 || O < 0 || I < 0 || M % 4 != 0 || I % 256 != 0 || O % 8 != 0) return ACTNN_EINVAL;
-  if (M > 0x7fffffffLL || O > 0x7fffffffLL || I > 0x7fffffffLL) return ACTNN_EINVAL;
+  if (M < 0 || O < 0 || I < 0 || I % 256 != 0 || O % 8 != 0) return ACTNN_EINVAL;
+  if (M > 0x7fffffffLL - BK || O > 0x7fffffffLL - BM || I > 0x7fffffffLL) return ACTNN_EINVAL;
+  if (bits) {
+    if (!prefix) return ACTNN_EINVAL;
+  } else if (fixed_bits != 1 && fixed_bits != 2 && fixed_bits != 4 && fixed_bits != 8) {
+    return ACTNN_EBITS;
+  }
   if (O == 0 || I == 0) return ACTNN_OK;
   if (!grad_w || (M > 0 && (!grad_out || !packed || !scale || !mn))) return ACTNN_EINVAL;
-  if (M > 0 && (!aligned16(grad_out) || !aligned16(grad_w) || reinterpret_cast<uintptr_t>(packed) % 4 != 0 ||
+  if (M > 0 && (!aligned16(grad_out) || !aligned16(grad_w) || reinterpret_cast<uintptr_t>(packed) % 8 != 0 ||
                 reinterpret_cast<uintptr_t>(scale) % 4 != 0 || reinterpret_cast<uintptr_t>(mn) % 4 != 0))
     return ACTNN_EALIGN;
+  const Stream st{static_cast<const uint8_t*>(packed), bits, prefix, bits ? 0 : fixed_bits};
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (go_dtype) {
-    case ACTNN_F16: return launch_sm<__half>(sm_dtype, out_dtype, grad_out, packed, scale, mn, grad_w, M, O, I, s);
-    case ACTNN_BF16: return launch_sm<bf16_t>(sm_dtype, out_dtype, grad_out, packed, scale, mn, grad_w, M, O, I, s);
+    case ACTNN_F16: return launch_sm<__half>(sm_dtype, out_dtype, grad_out, st, scale, mn, grad_w, M, O, I, s);
+    case ACTNN_BF16: return launch_sm<bf16_t>(sm_dtype, out_dtype, grad_out, st, scale, mn, grad_w, M, O, I, s);
     default: return ACTNN_EDTYPE;
   }
+}
+
+extern "C" int actnn_linear_grad_weight_q2(const void* grad_out, const int8_t* packed, const void* scale,
+                                           const void* mn, void* grad_w, int64_t M, int64_t O, int64_t I,
+                                           int go_dtype, int sm_dtype, int out_dtype, void* stream) {
+  if (M % 4 != 0) return ACTNN_EINVAL;
+  return actnn_linear_grad_weight(grad_out, packed, nullptr, nullptr, 2, scale, mn, grad_w, M, O, I, go_dtype,
+                                  sm_dtype, out_dtype, stream);
 }

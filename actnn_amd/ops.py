@@ -329,17 +329,20 @@ class conv_transpose3d(Function):
 # linear (ops.py:386-433)
 # ------------------------------------------------------------------------------------------
 def _fused_grad_weight_ok(quantized, shape, go):
-    """The fused kernel applies to a 2-D input saved with the 2-bit fixed-width stream whose rows
-    are whole groups, with 16-bit gradients and native (not bf16-compacted) scale/min."""
-    if not config.compress_activation or config.simulate or config.swap:
+    """The fused kernel takes a 2-D input saved in whole groups of 256 per row - as the fixed-width
+    stream (levels L1 / L2, or any int width) or the per-sample stream of the schemes (L3 and up) -
+    with 16-bit gradients (autocast, or a 16-bit model)."""
+    if not config.compress_activation or config.simulate or config.swap or not config.fused_linear_grad_weight:
         return False
     q_input, q_bits, q_scale, q_min = quantized
-    return (isinstance(q_bits, int) and q_bits == 2 and len(shape) == 2
-            and shape[-1] % config.group_size == 0 and config.group_size == 256
-            and shape[0] % 4 == 0 and go.shape[1] % 8 == 0
-            and go.dtype in (torch.float16, torch.bfloat16) and q_scale.dtype == go.dtype
-            and q_input.is_cuda)
-
+    if isinstance(q_bits, int):
+        if q_bits not in (1, 2, 4, 8):
+            return False
+    elif not (isinstance(q_bits, torch.Tensor) and q_bits.dtype == torch.int32 and q_bits.is_cuda):
+        return False
+    return (len(shape) == 2 and shape[-1] % config.group_size == 0 and config.group_size == 256
+            and go.shape[1] % 8 == 0 and go.dtype in (torch.float16, torch.bfloat16)
+            and isinstance(q_input, torch.Tensor) and q_input.is_cuda)
 
 
 class linear(Function):
@@ -362,11 +365,13 @@ class linear(Function):
         q_input_shape = ctx.other_args
         go = grad_output.reshape(-1, grad_output.shape[-1])
         if _fused_grad_weight_ok(quantized, q_input_shape, go):
-            # 2-bit fixed-width input: the weight gradient is computed straight from the packed
-            # stream (dequantised tiles only ever exist in LDS), nothing is materialised
-            q_input, _, q_scale, q_min = quantized
-            grad_weight = ext_quantization.linear_grad_weight_q2(
-                go, q_input, q_scale, q_min, q_input_shape[-1], weight.dtype) \
+            # the weight gradient is computed straight from the packed stream (dequantised tiles
+            # only ever exist in LDS), nothing is materialised
+            q_input, q_bits, q_scale, q_min = quantized
+            if q_scale.dtype == torch.bfloat16 and _stored_as_bf16(q_input_shape, quantized):
+                q_scale, q_min = q_scale.to(torch.float32), q_min.to(torch.float32)    # ops.py:129-131
+            grad_weight = ext_quantization.linear_grad_weight(
+                go, q_input, q_bits, q_scale, q_min, q_input_shape[-1], weight.dtype) \
                 if ctx.needs_input_grad[1] else None
         else:
             input = dequantize_activation(quantized, q_input_shape)

@@ -252,6 +252,17 @@ def other_configs(device, reps):
     out["unpack_single_4bit_bf16_512x256x56x56"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
     del xb16, lo16, hi16, bits16, p4, s4
     torch.cuda.empty_cache()
+    out.update(config4(device, reps))
+    return {k_: {kk: round(vv, 4) for kk, vv in v.items()} for k_, v in out.items()}
+
+
+def config4(device, reps):
+    """Benchmark config 4: fixed-width 2-bit pack / unpack of fp16 [8192,4096] and the fused
+    dequantise + weight-gradient GEMM (MFMA roofline), the unfused path beside it."""
+    import torch
+    import actnn_amd.cpp_extension.minimax as ext_minimax
+    import actnn_amd.cpp_extension.quantization as ext_q
+    out = {}
     # config 4: fp16 [8192,4096], Student-t(nu=3) heavy tails with a per-feature scale, through the
     # fixed-width path (2 bits per row group of 256)
     M, I = 8192, 4096
@@ -284,7 +295,7 @@ def other_configs(device, reps):
     t = _event_time_ms(unfused, reps)
     out["linear_grad_weight_unfused_unpack_plus_mm"] = {"ms": t, "TFLOP/s": flops / t / 1e9,
                                                         "frac_mfma_bf16": flops / t / 1e9 / MFMA_BF16_PEAK_TFLOPS}
-    return {k_: {kk: round(vv, 4) for kk, vv in v.items()} for k_, v in out.items()}
+    return out
 
 
 def _width_histogram(bits_host):
@@ -337,7 +348,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the config-2 hot path")
-    ap.add_argument("--only", choices=["other", "resnet50", "resnet50_channels_last", "resnet50_fp32", "resnet50_levels", "batch_norm_shapes"],
+    ap.add_argument("--only", choices=["other", "config4", "resnet50", "resnet50_channels_last", "resnet50_fp32", "resnet50_levels", "batch_norm_shapes"],
                     default=None,
                     help="profiling aid: run just the other single-GPU configs (ReLU, max-pool, "
                          "fixed-width pack, fused GEMM), just the ResNet-50 L3 step, the fp32 "
@@ -359,6 +370,10 @@ def main():
     torch.cuda.set_device(device)
     if args.only == "other":
         print(json.dumps({"other_configs": other_configs(device, max(10, args.steps // 2))}))
+        return
+    if args.only == "config4":
+        print(json.dumps({"config4": {k: {kk: round(vv, 4) for kk, vv in v.items()}
+                                      for k, v in config4(device, max(10, args.steps // 2)).items()}}))
         return
     if args.only == "resnet50":
         import bench_extra

@@ -197,16 +197,24 @@ int actnn_allocate_bits_device(const void* mn, const void* mx, float factor, con
                                int64_t target, int dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------
- * Fused QLinear weight gradient: grad_w[O, I] = grad_out[M, O]^T @ dequant(x)[M, I] where x
- * is held as the pack_single 2-bit stream (4 consecutive rows m per byte) with
- * scale/min[M, I/256, 1].  The 2-bit tile is unpacked and dequantised to the 16-bit format of
- * grad_out inside the LDS loader of an MFMA GEMM (fp32 accumulation); the full-precision input
- * is never written to memory.  Replaces dequantize_activation + grad_output.t().mm(input) in
- * linear.backward, actnn/actnn/ops.py:407-421.
+ * Fused QLinear weight gradient: grad_w[O, I] = grad_out[M, O]^T @ dequant(x)[M, I] where x is
+ * held as a stream of this library with scale/min[M, I/256, 1] (groups of 256 along a row):
+ *   bits == NULL: the fixed-width stream of actnn_pack_single at `fixed_bits` (1, 2, 4 or 8);
+ *   bits != NULL: the mixed-width stream of actnn_pack_mixed with bits[M] and prefix[M + 1]
+ *                 (fixed_bits ignored) - what QScheme hands linear.backward at the default level.
+ * The tile is unpacked and dequantised (code / scale + min, rounded as the unpack kernels round)
+ * to the 16-bit format of grad_out inside the LDS loader of an MFMA GEMM (fp32 accumulation); the
+ * full-precision input is never written to memory.  Replaces dequantize_activation +
+ * grad_output.t().mm(input) in linear.backward, actnn/actnn/ops.py:407-421.
  * grad_out dtype: f16 or bf16; scale/min dtype = sm_dtype; grad_w dtype = out_dtype
- * (f32, f16 or bf16).  M % 4 == 0, I % 256 == 0, O % 8 == 0; grad_out and grad_w 16-byte,
- * packed, scale and min 4-byte aligned.
+ * (f32, f16 or bf16).  I % 256 == 0, O % 8 == 0; grad_out and grad_w 16-byte, packed 8-byte,
+ * scale and min 4-byte aligned.  The 2-bit fixed-width stream takes the fast loader.
+ * actnn_linear_grad_weight_q2 is the 2-bit fixed-width case with M % 4 == 0.
  * ------------------------------------------------------------------------------- */
+int actnn_linear_grad_weight(const void* grad_out, const void* packed, const int32_t* bits,
+                             const int32_t* prefix, int fixed_bits, const void* scale, const void* mn,
+                             void* grad_w, int64_t M, int64_t O, int64_t I, int go_dtype,
+                             int sm_dtype, int out_dtype, void* stream);
 int actnn_linear_grad_weight_q2(const void* grad_out, const int8_t* packed, const void* scale,
                                 const void* mn, void* grad_w, int64_t M, int64_t O, int64_t I,
                                 int go_dtype, int sm_dtype, int out_dtype, void* stream);

@@ -150,6 +150,38 @@ def test_qlinear_fused_weight_gradient_path(dtype):
     assert torch.equal(gp_f[1], gp_u[1])
 
 
+@pytest.mark.parametrize("level", ["L2", "L3"])
+def test_qlinear_takes_the_fused_gemm_at_the_reference_levels(level, monkeypatch):
+    # under bf16 autocast a QLinear's weight gradient comes from the fused kernel at every level that
+    # compresses: the 4-bit fixed-width stream at L1 / L2, the per-sample stream of the scheme at L3;
+    # the result agrees with the unfused path (unpack + mm) on the same packed input
+    from actnn_amd import ops
+    import actnn_amd.cpp_extension.quantization as ext_q
+    set_optimization_level(level)
+    torch.manual_seed(0)
+    q = actnn_amd.QLinear(2048, 1000).to(DEV)
+    x = torch.randn(128, 2048, device=DEV)
+    calls = []
+    fused = ext_q.linear_grad_weight
+    monkeypatch.setattr(ext_q, "linear_grad_weight", lambda *a: calls.append(type(a[2])) or fused(*a))
+
+    def step():
+        q.zero_grad()
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            y = q(x.clone().requires_grad_(True))
+        y.float().square().mean().backward()
+        return q.weight.grad.clone()
+    step()                                          # first step: degenerate widths at L3
+    torch.cuda.manual_seed(5)
+    gw_fused = step()
+    assert len(calls) == 2 and calls[0] is (int if level == "L2" else torch.Tensor)
+    config.fused_linear_grad_weight = False
+    torch.cuda.manual_seed(5)
+    gw_unfused = step()
+    assert len(calls) == 2
+    assert (gw_fused - gw_unfused).norm() / gw_unfused.norm() < 1e-2
+
+
 def test_l3_first_step_uses_the_degenerate_allocation_then_rebalances():
     # gradient scale starts at 0 (qscheme.py:24): the first forward gives 8 bits to the first
     # samples and 1 to the rest; after one backward the scale is positive and bits follow C
