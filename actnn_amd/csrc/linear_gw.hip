@@ -10,10 +10,11 @@
 // and narrowed to the 16-bit format of grad_out straight into the LDS tile that feeds
 // v_mfma_f32_32x32x16_bf16 / _f16, fp32 accumulation.
 //
-// Tiling: the reduction runs over the samples m (K of the GEMM).  A 512-thread block (one per CU)
+// Tiling: the reduction runs over the samples m (K of the GEMM).  A 256-thread block (one per CU)
 // owns a 256 (O) x 256 (I) output tile - one whole quantisation group, so a block needs one
-// scale/min per sample - as 8 waves of 64 (O) x 128 (I).  Per k-step of 64 samples, LDS tiles
-// double-buffered, one barrier a step:
+// scale/min per sample - as 4 waves of 128 (O) x 128 (I), one per SIMD, 256 accumulator registers
+// each: a fragment read from LDS feeds four MFMAs (with 8 waves of 64 x 128 it feeds two or four:
+// a third more LDS traffic).  Per k-step of 64 samples, LDS tiles double-buffered, one barrier a step:
 //   * Both operand tiles lie in LDS the way they lie in memory: [sample][column], 512 bytes a row.
 //     MFMA fragments want 8 consecutive samples of one column per lane; the transposing LDS read
 //     (ds_read_b64_tr_b16: a 16-lane block that points at four rows of four 8-byte units gets back,
@@ -22,7 +23,8 @@
 //     chunk ^ ((sample & 7) << 2): the four rows that 32 lanes of such a read touch (64 bytes each)
 //     then fall into the four quarters of the 64 banks, and the two reads of a fragment into
 //     different halves of the row (measured: 1.4 times the rate of a swizzle that only separates
-//     the rows within 16 lanes, 2.7 times no swizzle).
+//     the rows within 16 lanes, 2.7 times no swizzle; 16-byte reads reach 1.3 times more still,
+//     but need sample-contiguous tiles, i.e. register transposes of grad_out).
 //   * grad_out tiles go from global memory straight into LDS (global_load_lds, 16 bytes per lane,
 //     the swizzle applied to the source address): no registers, no VALU work.
 //   * the 2-bit fixed-width stream: a thread takes one 32-bit load = 4 features x 4 samples.  The
@@ -35,8 +37,18 @@
 //     dequantises them with the unpack kernels' arithmetic and writes 16 bytes of the row.
 //   The roles of the operands are chosen so that an accumulator register quad holds four
 //   consecutive columns of grad_w: the epilogue stores 16 bytes (fp32) per lane and register quad.
-// Loads of packed data and scale/min run one step ahead of the staging code (widths and stream
-// offsets of the mixed stream two steps ahead).
+// All work of a step other than the MFMAs is cut into pieces that sit between the MFMAs (see the
+// schedule in the kernel).  Loads of packed data and scale/min run one step ahead of the staging
+// code (widths and stream offsets of the mixed stream two steps ahead).
+//
+// What bounds it on MI355X: with normally distributed 16-bit operands the matrix pipes are held
+// back by the power limit, not by this kernel's structure - the vendor GEMM (rocBLAS) on the same
+// dequantised operands and three differently organised versions of this kernel (8 waves of 64 x 128
+// with register transposes; the same with transposing reads; this one) all take 0.29 - 0.32 ms for
+// [8192, 4096]^T x [8192, 4096] (0.86 - 0.95 PFLOP/s at about 1.8 GHz), and all of them speed up by
+// a quarter to a third when one operand is all zeros or ones.
+#include <type_traits>
+
 #include "quant_math.h"
 
 namespace actnn {
@@ -47,14 +59,20 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kThreads = 512;
+constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / 64;
+constexpr int NE = 4;               // 32-column fragments of the activation tile per wave (128 columns)
+constexpr int NA = 4;               // 32-row fragments of the grad_out tile per wave (128 rows)
+constexpr int kGroup = NE * NA;     // MFMAs per k-block and wave
+constexpr int kSlots = 4 * kGroup;  // MFMAs per step and wave
+constexpr int kSamplesPerWave = 64 / kWaves;
 constexpr int BM = 256;             // output rows (O) per block
 constexpr int BN = 256;             // output columns (I) per block: one quantisation group
 constexpr int BK = 64;              // samples per k-step
 constexpr int kRowBytes = 512;      // one sample of either tile: 256 16-bit values
 constexpr int kTileBytes = BK * kRowBytes;
-constexpr int kTabBytes = kWaves * 2 * 64;          // per wave and buffer: 8 samples x 8 bytes
+constexpr int kTabWave = kSamplesPerWave * 8;       // table bytes per wave and buffer: 8 per sample
+constexpr int kTabBytes = kWaves * 2 * kTabWave;
 
 template <int N> struct Slot { static constexpr int value = N; };
 template <int N, typename F> ACTNN_DEV void for_each_slot(F&& f) {
@@ -147,16 +165,21 @@ struct Stream {
 // Loader of the 2-bit fixed-width stream (table + byte permutes)
 // ------------------------------------------------------------------------------------------
 template <typename TG, typename TS> struct TableLoader {
-  uint32_t rb[2];          // this lane's 32-bit loads of the wave's two sample quads
-  uint32_t rsc, rmn;       // scale / min (raw) of sample (lane / 4) % 8 of the wave's eight
-  u32x2 tt[8];             // the wave's eight table entries, read back from LDS
+  static constexpr int Q = kSamplesPerWave / 4;      // sample quads per wave and step
+  // where the main loop places this loader's pieces (MFMA slot numbers of a step)
+  static constexpr int kTableSlot = kGroup, kReadbackSlot = kGroup + 4, kStageSlot = kGroup + 8,
+                       kPrefetchSlot = kStageSlot + 4 * Q + 4;
+  uint32_t rb[Q];          // this lane's 32-bit loads of the wave's sample quads
+  uint32_t rsc, rmn;       // scale / min (raw) of sample lane / 4 of the wave's sixteen
+  u32x2 tt[4 * Q];         // the wave's table entries, read back from LDS
   const uint8_t* pb0;      // this lane's bytes of quad 0
   const TS* psc0;          // scale / min of sample 0 in the block's group
   const TS* pmn0;
   int next;                // first sample of the step the next prefetch loads
   int M, G, quad_rows;     // quad_rows: bytes from one sample quad to the next in the stream
 
-  ACTNN_DEV void init(const Stream& st, const TS* scale, const TS* mn, int M_, int G_, int g, int wave, int lane) {
+  ACTNN_DEV void init(const Stream& st, const TS* scale, const TS* mn, int M_, int G_, int g) {
+    const int lane = threadIdx.x & 63;
     M = M_;
     G = G_;
     next = 0;
@@ -171,52 +194,51 @@ template <typename TG, typename TS> struct TableLoader {
   ACTNN_DEV void prefetch() {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int first = next + wave * 8;
+    const int first = next + wave * kSamplesPerWave;
     const int last_quad = (M - 1) >> 2;
 #pragma unroll
-    for (int qq = 0; qq < 2; ++qq) {
+    for (int qq = 0; qq < Q; ++qq) {
       int quad = (first >> 2) + qq;
       quad = quad < last_quad ? quad : last_quad;
       rb[qq] = *reinterpret_cast<const uint32_t*>(pb0 + (int64_t)quad * quad_rows);
     }
-    int smp = first + ((lane >> 2) & 7);
+    int smp = first + (lane >> 2);
     smp = smp < M - 1 ? smp : M - 1;
     rsc = RawScalar<TS>::load(psc0, (int64_t)smp * G);
     rmn = RawScalar<TS>::load(pmn0, (int64_t)smp * G);
     next += BK;
   }
-  // The staging work of a step, cut into pieces that the main loop places between its MFMAs (slot
-  // numbers are the loop's).  `tab`: this wave's 64 table bytes; kfirst: first sample of the tile.
+  // The staging work of a step, cut into pieces that the main loop places between its MFMAs.
+  // `tab`: this wave's table bytes; kfirst: first sample of the tile.
   template <int SLOT> ACTNN_DEV void piece(uint8_t* tile, uint8_t* tab, int kfirst) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if constexpr (SLOT == 4) {
-      // value of code (lane & 3) for sample (lane / 4) % 8, rounded exactly as unpack_single rounds it
-      // (the two half-waves compute and write the same bytes: no branch)
-      const int smp = (lane >> 2) & 7;
-      const bool valid = kfirst + wave * 8 + smp < M;
+    if constexpr (SLOT == kTableSlot) {
+      // value of code (lane & 3) for sample lane / 4, rounded exactly as unpack_single rounds it
+      const int smp = lane >> 2;
+      const bool valid = kfirst + wave * kSamplesPerWave + smp < M;
       const Dequant<TS> dq(RawScalar<TS>::widen(rsc), RawScalar<TS>::widen(rmn));
       const uint32_t v = valid ? Mma<TG>::bits16(dq((uint32_t)(lane & 3))) : 0u;
       uint8_t* t = tab + smp * 8 + (lane & 3);
       t[0] = (uint8_t)v;            // low bytes of the sample's four values, then their high bytes
       t[4] = (uint8_t)(v >> 8);
-    } else if constexpr (SLOT == 6) {
+    } else if constexpr (SLOT == kReadbackSlot) {
       // same wave writes and reads: LDS operations of a wave complete in order
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-      for (int i = 0; i < 8; ++i) tt[i] = *reinterpret_cast<const u32x2*>(tab + i * 8);
-    } else if constexpr (SLOT >= 8 && SLOT < 16) {
-      constexpr int qq = (SLOT - 8) / 4, j = (SLOT - 8) % 4;
+      for (int i = 0; i < 4 * Q; ++i) tt[i] = *reinterpret_cast<const u32x2*>(tab + i * 8);
+    } else if constexpr (SLOT >= kStageSlot && SLOT < kStageSlot + 4 * Q) {
+      constexpr int qq = (SLOT - kStageSlot) / 4, j = (SLOT - kStageSlot) % 4;
       const int ch = lane >> 1, half = (lane & 1) * 8;
       const uint32_t sel = (rb[qq] >> (2 * j)) & 0x03030303u;       // codes of 4 features as byte selectors
       const uint32_t lo = __builtin_amdgcn_perm(0u, tt[qq * 4 + j].x, sel);
       const uint32_t hi = __builtin_amdgcn_perm(0u, tt[qq * 4 + j].y, sel);
       const u32x2 out = {__builtin_amdgcn_perm(hi, lo, 0x05010400u), __builtin_amdgcn_perm(hi, lo, 0x07030602u)};
-      const int k = wave * 8 + qq * 4 + j;
+      const int k = wave * kSamplesPerWave + qq * 4 + j;
       *reinterpret_cast<u32x2*>(tile + chunk_offset(k, ch) + half) = out;
-    } else if constexpr (SLOT == 20) {
+    } else if constexpr (SLOT == kPrefetchSlot) {
       prefetch();
     }
   }
@@ -227,7 +249,8 @@ template <typename TG, typename TS> struct TableLoader {
 // a step; lane j unpacks features 8j .. 8j+7 of each.
 // ------------------------------------------------------------------------------------------
 template <typename TG, typename TS> struct GeneralLoader {
-  static constexpr int U = 4;          // samples per half-wave and step
+  static constexpr int U = BK / (kThreads / 32);      // samples per half-wave and step
+  static constexpr int kStageSlot = kGroup, kPrefetchSlot = 2 * kGroup + 8;
   uint32_t w0[U], w1[U];               // packed data of the step being loaded
   uint32_t rsc[U], rmn[U];             // raw scale / min
   int wb[U];                           // widths that belong to w0/w1 (mixed stream)
@@ -287,8 +310,8 @@ template <typename TG, typename TS> struct GeneralLoader {
     if (st.bits) prefetch_bits();
   }
   template <int SLOT> ACTNN_DEV void piece(uint8_t* tile, uint8_t*, int kfirst) {
-    if constexpr (SLOT == 4) stage(tile, kfirst);
-    else if constexpr (SLOT == 20) prefetch();
+    if constexpr (SLOT == kStageSlot) stage(tile, kfirst);
+    else if constexpr (SLOT == kPrefetchSlot) prefetch();
   }
   ACTNN_DEV void stage(uint8_t* tile, int kfirst) {
     const int hw = threadIdx.x >> 5, j = threadIdx.x & 31;
@@ -336,7 +359,7 @@ __global__ __launch_bounds__(kThreads, 1) void linear_gw_kernel(
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wr = wave & 3, wn = wave >> 2;   // the wave's 64 rows (O) and 128 columns (I) of the tile
+  const int wr = wave & 1, wn = wave >> 1;   // the wave's 128 rows (O) and 128 columns (I) of the tile
   const int G = I / 256;
   // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give every XCD whole
   // panels of grad_out rows (all column tiles of tile_m), so that a panel is pulled into one L2
@@ -351,7 +374,7 @@ __global__ __launch_bounds__(kThreads, 1) void linear_gw_kernel(
   const int o0 = (tile / tiles_n) * BM;
   const int g = tile % tiles_n;              // the block's columns are quantisation group g
   const int i0 = g * 256;
-  uint8_t* tab = smem + 4 * kTileBytes + wave * 128;
+  uint8_t* tab = smem + 4 * kTileBytes + wave * 2 * kTabWave;
 
   // ---- grad_out tile: straight from global memory into LDS.  One instruction of a wave fills 1 KiB
   // of LDS (two rows); lane -> row 2*rp + lane/32, LDS chunk lane%32, which holds source chunk
@@ -359,11 +382,12 @@ __global__ __launch_bounds__(kThreads, 1) void linear_gw_kernel(
   // zeros, so any finite value will do), columns past O from the block's first column (they only
   // reach output rows that are not stored): every lane loads, nothing else writes these tiles.
   const int g_row = lane >> 5;
-  // rows of one instruction: 2 * rp + g_row with rp = 8 * jj + wave, so (row & 7) only depends on the wave
+  // rows of one instruction: 2 * rp + g_row with rp = kWaves * jj + wave, so (row & 7) only depends on the wave
+  static_assert(kWaves % 4 == 0, "the swizzle of a direct load must not depend on jj");
   const int g_chunk = (lane & 31) ^ (((2 * (wave & 3) + g_row) & 7) << 2);
   const int g_col = o0 + g_chunk * 8 < O ? o0 + g_chunk * 8 : o0;
   auto load_g_piece = [&](uint8_t* tile_g, int kfirst, int jj) {
-    const int rp = jj * 8 + wave;                         // row pair of the tile, uniform in the wave
+    const int rp = jj * kWaves + wave;                    // row pair of the tile, uniform in the wave
     int m = kfirst + 2 * rp + g_row;
     m = m < M ? m : M - 1;
     load_to_lds16(gout + (int64_t)m * O + g_col, tile_g + rp * 2 * kRowBytes);
@@ -377,65 +401,66 @@ __global__ __launch_bounds__(kThreads, 1) void linear_gw_kernel(
     const int ch = n0 / 8 + 2 * (blk & 1) + ((r & 3) >> 1);
     return chunk_offset(f_row, ch) + (r & 1) * 8;
   };
-  int offx[4], offg[2];          // first read of a fragment; the second (4 rows on) lies at (offset ^ 256) + 4 rows
+  int offx[NE], offg[NA];        // first read of a fragment; the second (4 rows on) lies at (offset ^ 256) + 4 rows
 #pragma unroll
-  for (int e = 0; e < 4; ++e) offx[e] = frag_offset(wn * 128 + 32 * e);
+  for (int e = 0; e < NE; ++e) offx[e] = frag_offset(wn * 32 * NE + 32 * e);
 #pragma unroll
-  for (int a = 0; a < 2; ++a) offg[a] = frag_offset(wr * 64 + 32 * a);
+  for (int a = 0; a < NA; ++a) offg[a] = frag_offset(wr * 32 * NA + 32 * a);
 
-  f32x16 acc[4][2];
+  f32x16 acc[NE][NA];
 #pragma unroll
-  for (int e = 0; e < 4; ++e)
+  for (int e = 0; e < NE; ++e)
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+    for (int a = 0; a < NA; ++a)
 #pragma unroll
       for (int c = 0; c < 16; ++c) acc[e][a][c] = 0.0f;
 
-  // fragment f of k-block kb: f = 0..3 activations (MFMA rows), 4..5 grad_out (MFMA columns);
-  // double-buffered in registers by the parity of kb
-  u32x4 fx[2][4], fg[2][2];
+  // fragment f of k-block kb: f = 0..NA-1 grad_out (MFMA columns), then NE activations (MFMA
+  // rows); double-buffered in registers by the parity of kb
+  u32x4 fx[2][NE], fg[2][NA];
   auto read_fragment = [&](const uint8_t* tile_g, const uint8_t* tile_x, auto KB, auto F) {
     constexpr int kb = decltype(KB)::value, f = decltype(F)::value;
-    const int off = f < 4 ? offx[f < 4 ? f : 0] : offg[f < 4 ? 0 : f - 4];
-    const uint8_t* tile = (f < 4 ? tile_x : tile_g) + kb * 16 * kRowBytes;
+    constexpr bool is_g = f < NA;
+    const int off = is_g ? offg[is_g ? f : 0] : offx[is_g ? 0 : f - NA];
+    const uint8_t* tile = (is_g ? tile_g : tile_x) + kb * 16 * kRowBytes;
     const u32x2 lo = read_transposed(tile + off);
     const u32x2 hi = read_transposed(tile + (off ^ 256) + 4 * kRowBytes);
     const u32x4 v = {lo.x, lo.y, hi.x, hi.y};
-    if constexpr (f < 4) fx[kb & 1][f] = v; else fg[kb & 1][f - 4] = v;
+    if constexpr (is_g) fg[kb & 1][f] = v; else fx[kb & 1][f - NA] = v;
   };
 
   const int steps = (M + BK - 1) / BK;
   // The schedule.  Step t is multiplied out of LDS buffer t % 2; the tiles of step t+1 go into the
   // other buffer, whose last readers finished before the barrier that ended step t-1.  Between two
-  // barriers a wave issues 32 MFMAs - the last k-block of the step before (its fragments were read
-  // before the barrier) and the first three of this step - and everything else is cut into pieces
-  // placed between them, so that the matrix pipe always has work queued while the wave computes
-  // addresses, permutes bytes and waits for LDS:
-  //   MFMA slot  0.. 7: k-block 3 of step t-1 | direct loads of G(t+1), table of X(t+1), reads (t, 0)
-  //   MFMA slot  8..15: k-block 0 of step t   | the eight staging pieces of X(t+1), reads (t, 1)
-  //   MFMA slot 16..23: k-block 1             | loads for X(t+2), reads (t, 2)
-  //   MFMA slot 24..31: k-block 2             | reads (t, 3)
+  // barriers a wave issues its 64 MFMAs of a step - the last k-block of the step before (its
+  // fragments were read before the barrier) and the first three of this step - and everything else
+  // is cut into pieces placed between them, so that the matrix pipe always has work queued while
+  // the wave computes addresses, permutes bytes and waits for LDS:
+  //   MFMA slot  0..15: k-block 3 of step t-1 | reads (t, 0), direct loads of G(t+1)
+  //   MFMA slot 16..31: k-block 0 of step t   | reads (t, 1), table of X(t+1), first staging pieces
+  //   MFMA slot 32..47: k-block 1             | reads (t, 2), staging pieces, loads for X(t+2)
+  //   MFMA slot 48..63: k-block 2             | reads (t, 3)
   //   wait for the direct loads; barrier
-  // Fragment reads are issued eight MFMAs ahead of their use, into the register set the MFMAs of
-  // the same slots do not read.
+  // The eight fragments of a k-block are read in the first eight slots of the group before the one
+  // that multiplies them, into the register set the MFMAs of those slots do not read.
   // The body between two barriers has no branches (first / last step are separate copies): with
   // branches around the pieces the compiler's LDS wait counts lose one position per join and every
   // MFMA ends up waiting for reads issued a moment before it.
+  constexpr int kDirectLoads = kTileBytes / (kThreads * 16);
   auto step = [&](auto& ld, auto FIRST, auto MORE, int t) {
     constexpr bool first = decltype(FIRST)::value != 0, more = decltype(MORE)::value != 0;
     const uint8_t* cur_g = tileG(t & 1);
     const uint8_t* cur_x = tileX(t & 1);
     const int nb = (t + 1) & 1;
-    for_each_slot<32>([&](auto S) {
+    for_each_slot<kSlots>([&](auto S) {
       constexpr int slot = decltype(S)::value;
-      constexpr int kb_mfma = (slot / 8 + 3) % 4, e = (slot % 8) / 2, a = slot % 2;
-      if constexpr (slot >= 8 || !first)
+      constexpr int kb_mfma = (slot / kGroup + 3) % 4, e = (slot % kGroup) / NA, a = slot % NA;
+      if constexpr (slot >= kGroup || !first)
         acc[e][a] = Mma<TG>::mfma(fx[kb_mfma & 1][e], fg[kb_mfma & 1][a], acc[e][a]);
-      // the two grad_out fragments first: the first MFMAs of the next group need them
-      if constexpr (slot % 8 < 6) read_fragment(cur_g, cur_x, Slot<slot / 8>{}, Slot<(slot % 8 + 4) % 6>{});
+      if constexpr (slot % kGroup < NE + NA) read_fragment(cur_g, cur_x, Slot<slot / kGroup>{}, Slot<slot % kGroup>{});
       if constexpr (more) {
-        if constexpr (slot < 4) load_g_piece(tileG(nb), (t + 1) * BK, slot);
-        ld.template piece<slot>(tileX(nb), tab + nb * 64, (t + 1) * BK);
+        if constexpr (slot < kDirectLoads) load_g_piece(tileG(nb), (t + 1) * BK, slot);
+        ld.template piece<slot>(tileX(nb), tab + nb * kTabWave, (t + 1) * BK);
       }
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -443,11 +468,16 @@ __global__ __launch_bounds__(kThreads, 1) void linear_gw_kernel(
     __syncthreads();
   };
   auto run = [&](auto& ld) {
+    using Loader = std::remove_reference_t<decltype(ld)>;
     if (steps > 0) {
       ld.prefetch();
-      for_each_slot<32>([&](auto S) { ld.template piece<(decltype(S)::value == 20 ? 31 : decltype(S)::value)>(tileX(0), tab, 0); });
+      // the whole staging of tile 0 (every piece but the prefetch, which follows)
+      for_each_slot<kSlots>([&](auto S) {
+        constexpr int slot = decltype(S)::value;
+        if constexpr (slot != Loader::kPrefetchSlot) ld.template piece<slot>(tileX(0), tab, 0);
+      });
 #pragma unroll
-      for (int jj = 0; jj < 4; ++jj) load_g_piece(tileG(0), 0, jj);
+      for (int jj = 0; jj < kDirectLoads; ++jj) load_g_piece(tileG(0), 0, jj);
       ld.prefetch();
     }
     __builtin_amdgcn_s_waitcnt(0);
@@ -461,14 +491,14 @@ __global__ __launch_bounds__(kThreads, 1) void linear_gw_kernel(
     }
     if (steps > 0) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
+      for (int e = 0; e < NE; ++e)
 #pragma unroll
-        for (int a = 0; a < 2; ++a) acc[e][a] = Mma<TG>::mfma(fx[1][e], fg[1][a], acc[e][a]);
+        for (int a = 0; a < NA; ++a) acc[e][a] = Mma<TG>::mfma(fx[1][e], fg[1][a], acc[e][a]);
     }
   };
   if constexpr (TABLE) {
     TableLoader<TG, TS> ld;
-    ld.init(st, scale, mn, M, G, g, wave, lane);
+    ld.init(st, scale, mn, M, G, g);
     run(ld);
   } else {
     GeneralLoader<TG, TS> ld;
@@ -479,14 +509,14 @@ __global__ __launch_bounds__(kThreads, 1) void linear_gw_kernel(
   // 32x32 accumulator layout: register c of a lane is fragment row 8*(c/4) + 4*(lane/32) + c%4 (a
   // column of grad_w: feature), fragment column lane%32 (a row of grad_w: output unit).
 #pragma unroll
-  for (int a = 0; a < 2; ++a) {
-    const int row = o0 + wr * 64 + 32 * a + (lane & 31);
+  for (int a = 0; a < NA; ++a) {
+    const int row = o0 + wr * 32 * NA + 32 * a + (lane & 31);
     if (row < O) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
+      for (int e = 0; e < NE; ++e) {
 #pragma unroll
         for (int cq = 0; cq < 4; ++cq) {
-          const int col = i0 + wn * 128 + 32 * e + 8 * cq + 4 * (lane >> 5);
+          const int col = i0 + wn * 32 * NE + 32 * e + 8 * cq + 4 * (lane >> 5);
           store_out4<TO>(gw + (int64_t)row * I + col, acc[e][a][4 * cq], acc[e][a][4 * cq + 1],
                          acc[e][a][4 * cq + 2], acc[e][a][4 * cq + 3]);
         }
