@@ -36,7 +36,7 @@ def test_deterministic_mode_bit_exact(bits, N, dtype):
 
 
 @pytest.mark.parametrize("bits", [1, 2, 4, 8])
-@pytest.mark.parametrize("gs", [256, 64])
+@pytest.mark.parametrize("gs", [256, 64, 24, 8])
 def test_rng_mode_matches_kernel_model(bits, gs):
     N, G = 6, 5
     x, _ = make_groups(N, G, gs, torch.float32, bits, "chan")
