@@ -272,13 +272,14 @@ ACTNN_DEV void leave_wave_sum(float* table, float v) {
     table[((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * kWaves + (threadIdx.x >> 6)] = v;
 }
 
-template <int BITS>
-ACTNN_DEV void pack_chunk_bits(const float (&v)[8], const uint32_t (&r16)[8], float mul, float sub,
+template <typename T, int BITS>
+ACTNN_DEV void pack_chunk_bits(const float (&v)[8], const uint32_t (&rw)[Noise<T>::kWords], float mul, float sub,
                                uint32_t lane32, int32_t* __restrict__ dst) {
-  constexpr float kBfix = (float)((1 << BITS) - 1) * 65536.0f;
-  uint64_t acc = 0;
+  constexpr float kUnit = (float)(1u << (32 - BITS - Noise<T>::kBits));
+  CodeShifter<BITS, (BITS > 4)> sh;
 #pragma unroll
-  for (int k = 0; k < 8; ++k) acc |= (uint64_t)rng_code(v[k], r16[k], mul, sub, kBfix) << (k * BITS);
+  for (int k = 7; k >= 0; --k) sh.push(RngFixed<T>::word(v[k], Noise<T>::at(rw, k), mul, sub, kUnit));
+  const uint64_t acc = ((uint64_t)sh.hi << 32) | sh.lo;
   const uint32_t lo = transpose32((uint32_t)acc, lane32);
   if ((int)lane32 < 8 * BITS) __builtin_nontemporal_store((int32_t)lo, dst + lane32);
   if (BITS > 4) {
@@ -303,18 +304,18 @@ ACTNN_DEV void pack_chunk(const PackSink& ps, const u32x4& ux, int64_t n, int64_
   float v[8];
 #pragma unroll
   for (int k = 0; k < 4; ++k) Chunk<T>::widen(w[k], v + k * PD);
-  uint32_t r16[8];
-  philox_octet((uint64_t)octet, ps.seed, ps.offset, r16);
+  uint32_t rw[Noise<T>::kWords];
+  Noise<T>::octet((uint64_t)octet, ps.seed, ps.offset, rw);
   int32_t* dst = ps.packed + first_word + grp * b * 8;
   switch (b) {                           // uniform over the half-wave: one sample, one width
-    case 1: pack_chunk_bits<1>(v, r16, mul, sub, lane32, dst); break;
-    case 2: pack_chunk_bits<2>(v, r16, mul, sub, lane32, dst); break;
-    case 3: pack_chunk_bits<3>(v, r16, mul, sub, lane32, dst); break;
-    case 4: pack_chunk_bits<4>(v, r16, mul, sub, lane32, dst); break;
-    case 5: pack_chunk_bits<5>(v, r16, mul, sub, lane32, dst); break;
-    case 6: pack_chunk_bits<6>(v, r16, mul, sub, lane32, dst); break;
-    case 7: pack_chunk_bits<7>(v, r16, mul, sub, lane32, dst); break;
-    case 8: pack_chunk_bits<8>(v, r16, mul, sub, lane32, dst); break;
+    case 1: pack_chunk_bits<T, 1>(v, rw, mul, sub, lane32, dst); break;
+    case 2: pack_chunk_bits<T, 2>(v, rw, mul, sub, lane32, dst); break;
+    case 3: pack_chunk_bits<T, 3>(v, rw, mul, sub, lane32, dst); break;
+    case 4: pack_chunk_bits<T, 4>(v, rw, mul, sub, lane32, dst); break;
+    case 5: pack_chunk_bits<T, 5>(v, rw, mul, sub, lane32, dst); break;
+    case 6: pack_chunk_bits<T, 6>(v, rw, mul, sub, lane32, dst); break;
+    case 7: pack_chunk_bits<T, 7>(v, rw, mul, sub, lane32, dst); break;
+    case 8: pack_chunk_bits<T, 8>(v, rw, mul, sub, lane32, dst); break;
     default: break;
   }
 }

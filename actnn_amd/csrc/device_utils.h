@@ -99,6 +99,35 @@ ACTNN_DEV void load8(const bf16_t* p, float (&v)[8]) {
     v[2 * i + 1] = as_float(w[i] & 0xffff0000u);
   }
 }
+// The same 8 elements kept as loaded (4 registers for 16-bit types instead of 8 floats) until
+// they are needed: raw8_load_nt / raw8_widen.
+template <typename T> struct Raw8 { u32x4 a; };
+template <> struct Raw8<float> { u32x4 a, b; };
+ACTNN_DEV void raw8_load_nt(const float* p, Raw8<float>& r) { r.a = load16(p); r.b = load16(p + 4); }
+ACTNN_DEV void raw8_load_nt(const __half* p, Raw8<__half>& r) { r.a = load16_nt(p); }
+ACTNN_DEV void raw8_load_nt(const bf16_t* p, Raw8<bf16_t>& r) { r.a = load16_nt(p); }
+template <typename T> ACTNN_DEV void raw8_zero(Raw8<T>& r) {
+  r.a = (u32x4){0, 0, 0, 0};
+  if constexpr (sizeof(T) == 4) r.b = (u32x4){0, 0, 0, 0};
+}
+ACTNN_DEV void raw8_widen(const Raw8<float>& r, float (&v)[8]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { v[i] = as_float(r.a[i]); v[4 + i] = as_float(r.b[i]); }
+}
+ACTNN_DEV void raw8_widen(const Raw8<__half>& r, float (&v)[8]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = half_bits_to_float(r.a[i] & 0xffffu);
+    v[2 * i + 1] = half_bits_to_float(r.a[i] >> 16);
+  }
+}
+ACTNN_DEV void raw8_widen(const Raw8<bf16_t>& r, float (&v)[8]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = as_float(r.a[i] << 16);
+    v[2 * i + 1] = as_float(r.a[i] & 0xffff0000u);
+  }
+}
 // Non-temporal variants for streams that are touched once and whose cache lines are covered whole
 // by one instruction of the wave (16 bytes per lane, lanes contiguous).
 ACTNN_DEV void load8_nt(const float* p, float (&v)[8]) { load8(p, v); }   // fp32: 32 bytes per lane, plain
@@ -285,16 +314,73 @@ ACTNN_DEV Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t 
   return Philox4{c0, c1, c2, c3};
 }
 
-// The eight 16-bit noises of the octet of elements [8*o, 8*o + 8): element k uses the
-// (k & 1)-th half (low first) of output word k >> 1.
+// ------------------------------------------------------------------ rounding noise
+// The stochastic rounding draws one uniform integer per element; elements are numbered as they lie
+// in memory and taken in octets (8 consecutive elements).  How many bits an element gets follows
+// the resolution of the data: 16 for fp32 tensors, 8 for fp16 / bf16 tensors (whose own spacing
+// near the top of a group's range is 2^-11 / 2^-8 of the value; an 8-bit draw rounds up with a
+// probability within 2^-9 of the fractional part, centred).
+//  * 16 bits: one Philox call per octet, counter = the octet's index; element k takes the
+//    (k & 1)-th half (low first) of output word k >> 1.
+//  * 8 bits: one Philox call per two consecutive octets, counter = octet index >> 1; octet h = index
+//    & 1 takes output words 2h and 2h + 1, element k byte k & 3 of word 2h + (k >> 2).
+// Dropout always uses the 16-bit form.
+ACTNN_DEV Philox4 philox_at(uint64_t counter, uint64_t seed, uint64_t offset) {
+  return philox4x32_10((uint32_t)counter, (uint32_t)(counter >> 32), (uint32_t)offset,
+                       (uint32_t)(offset >> 32), (uint32_t)seed, (uint32_t)(seed >> 32));
+}
+
 ACTNN_DEV void philox_octet(uint64_t octet, uint64_t seed, uint64_t offset, uint32_t (&r16)[8]) {
-  const Philox4 r = philox4x32_10((uint32_t)octet, (uint32_t)(octet >> 32), (uint32_t)offset,
-                                  (uint32_t)(offset >> 32), (uint32_t)seed, (uint32_t)(seed >> 32));
+  const Philox4 r = philox_at(octet, seed, offset);
   r16[0] = r.x & 0xffffu; r16[1] = r.x >> 16;
   r16[2] = r.y & 0xffffu; r16[3] = r.y >> 16;
   r16[4] = r.z & 0xffffu; r16[5] = r.z >> 16;
   r16[6] = r.w & 0xffffu; r16[7] = r.w >> 16;
 }
+
+template <typename T> struct Noise {
+  static constexpr int kBits = sizeof(T) == 2 ? 8 : 16;
+  static constexpr int kWords = 8 * kBits / 32;                 // words of noise per octet
+  // the draw of element k of an octet whose words are w
+  static ACTNN_DEV uint32_t at(const uint32_t (&w)[kWords], int k) {
+    constexpr int per = 32 / kBits;
+    return (w[k / per] >> (kBits * (k % per))) & ((1u << kBits) - 1u);
+  }
+  // Noise words of one octet, whatever the lanes around hold.
+  static ACTNN_DEV void octet(uint64_t o, uint64_t seed, uint64_t offset, uint32_t (&w)[kWords]) {
+    if constexpr (kBits == 16) {
+      const Philox4 r = philox_at(o, seed, offset);
+      w[0] = r.x; w[1] = r.y; w[2] = r.z; w[3] = r.w;
+    } else {
+      const Philox4 r = philox_at(o >> 1, seed, offset);
+      const bool h = o & 1;
+      w[0] = h ? r.z : r.x;
+      w[1] = h ? r.w : r.y;
+    }
+  }
+  // Noise words of two octets oa, ob of this lane when lane ^ 1 holds oa ^ 1 and ob ^ 1 and is
+  // active, and the parity of the lane is the parity of both octets.  With 8-bit noise the two
+  // lanes then need two Philox calls between them instead of four: the even lane evaluates the
+  // pair of oa, the odd lane the pair of ob, and they hand each other the half they do not use.
+  static ACTNN_DEV void octets(uint64_t oa, uint64_t ob, uint64_t seed, uint64_t offset,
+                               uint32_t (&wa)[kWords], uint32_t (&wb)[kWords]) {
+    if constexpr (kBits == 16) {
+      octet(oa, seed, offset, wa);
+      octet(ob, seed, offset, wb);
+    } else {
+      const bool odd = oa & 1;
+      const Philox4 r = philox_at((odd ? ob : oa) >> 1, seed, offset);
+      // even lane: r = pair(oa): (x, y) are mine for oa, (z, w) the neighbour's for oa ^ 1
+      // odd lane:  r = pair(ob): (z, w) are mine for ob, (x, y) the neighbour's for ob ^ 1
+      const uint32_t nx = lane_xor<1>(r.x), ny = lane_xor<1>(r.y);
+      const uint32_t nz = lane_xor<1>(r.z), nw = lane_xor<1>(r.w);
+      wa[0] = odd ? nz : r.x;
+      wa[1] = odd ? nw : r.y;
+      wb[0] = odd ? r.z : nx;
+      wb[1] = odd ? r.w : ny;
+    }
+  }
+};
 
 // ------------------------------------------------------------------ host-side helpers
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -86,9 +86,11 @@ template <> struct IsF32<float> { static constexpr bool value = true; };
 
 // ---------------------------------------------------------------------------- pack (gs = 256)
 // Issue the loads of this lane's elements (and noise in deterministic mode) for its GPH groups.
+// The elements stay as loaded until their group is packed (16-bit types: 4 registers per group
+// rather than 8), which keeps the kernel within the registers of 8 waves per SIMD.
 template <typename T, bool DET, int GPH>
 ACTNN_DEV void load_groups(const T* __restrict__ data, const T* __restrict__ noise, int64_t elem_base,
-                           int groups_valid, float (&v)[GPH][8], float (&nz)[DET ? GPH : 1][8]) {
+                           int groups_valid, Raw8<T> (&v)[GPH], Raw8<T> (&nz)[DET ? GPH : 1]) {
   using TL = Tile<1, GPH>;
   const uint32_t lane = threadIdx.x & 31;
   const int hw = threadIdx.x >> 5;
@@ -97,17 +99,17 @@ ACTNN_DEV void load_groups(const T* __restrict__ data, const T* __restrict__ noi
     const int gl = TL::group_of(hw, q);
     if (gl < groups_valid) {
       const int64_t e = elem_base + (int64_t)gl * kGs + lane * 8;
-      load8_nt(data + e, v[q]);      // non-temporal for 16-bit types only (one instruction per line)
-      if (DET) load8(noise + e, nz[DET ? q : 0]);
+      raw8_load_nt(data + e, v[q]);      // non-temporal for 16-bit types only (one instruction per line)
+      if (DET) raw8_load_nt(noise + e, nz[DET ? q : 0]);
     } else {
-#pragma unroll
-      for (int k = 0; k < 8; ++k) { v[q][k] = 0.0f; if (DET) nz[DET ? q : 0][k] = 0.0f; }
+      raw8_zero(v[q]);
+      if (DET) raw8_zero(nz[DET ? q : 0]);
     }
   }
 }
 
 template <typename T, int BITS, bool DET>
-ACTNN_DEV void pack_groups(const float (&v)[Gph<T>::kPack][8], const float (&nz)[DET ? Gph<T>::kPack : 1][8],
+ACTNN_DEV void pack_groups(const Raw8<T> (&raw)[Gph<T>::kPack], const Raw8<T> (&nzraw)[DET ? Gph<T>::kPack : 1],
                            int32_t* __restrict__ packed, int64_t elem_base, int64_t word_base,
                            int groups_valid, const float* s_mul, const float* s_sub,
                            uint64_t seed, uint64_t offset) {
@@ -118,25 +120,40 @@ ACTNN_DEV void pack_groups(const float (&v)[Gph<T>::kPack][8], const float (&nz)
   constexpr float Bf = (float)((1 << BITS) - 1);
   const uint32_t lane = threadIdx.x & 31;
   const int hw = threadIdx.x >> 5;
+  static_assert(kGroupsPerHalf % 2 == 0, "the noise of the groups is drawn in pairs");
+  constexpr int NB = R > 2 ? R : 2;                    // groups whose noise is drawn together
+  constexpr float kUnit = (float)(1u << (32 - BITS - Noise<T>::kBits));
+  uint32_t rw[NB][Noise<T>::kWords];
 
 #pragma unroll
   for (int q0 = 0; q0 < kGroupsPerHalf; q0 += R) {
-    uint64_t acc = 0;
+    uint64_t acc = 0;                                  // DET
+    CodeShifter<BITS, TL::kTwoRegs> sh;                // RNG
+    if (!DET && q0 % NB == 0) {
+      // noise of NB groups, two at a time: the octets of lane ^ 1 in the same two groups are
+      // their neighbours (elem_base is a multiple of 256, so octet and lane parity agree)
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
+      for (int p = 0; p < NB; p += 2) {
+        const uint64_t o = (uint64_t)(elem_base >> 3) + (uint64_t)TL::group_of(hw, q0 + p) * 32 + lane;
+        Noise<T>::octets(o, o + 32, seed, offset, rw[p], rw[p + 1]);
+      }
+    }
+#pragma unroll
+    for (int r = R - 1; r >= 0; --r) {                 // last group first: see CodeShifter
       const int q = q0 + r;
       const int gl = TL::group_of(hw, q);
       const float mul = s_mul[gl];
       const float sub = s_sub[gl];
-      uint32_t r16[8];
-      if (!DET) philox_octet((uint64_t)(elem_base >> 3) + (uint64_t)gl * 32 + lane, seed, offset, r16);
+      float v[8], nz[8];
+      raw8_widen(raw[q], v);
+      if (DET) raw8_widen(nzraw[DET ? q : 0], nz);
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const uint32_t c = DET ? det_code<T>(v[q][k], nz[DET ? q : 0][k], mul, sub, Bf)
-                               : rng_code(v[q][k], r16[k], mul, sub, Bf * 65536.0f);
-        acc |= (uint64_t)c << (r * WPG + k * BITS);
+      for (int k = 7; k >= 0; --k) {
+        if (DET) acc |= (uint64_t)det_code<T>(v[k], nz[k], mul, sub, Bf) << (r * WPG + k * BITS);
+        else sh.push(RngFixed<T>::word(v[k], Noise<T>::at(rw[q % NB], k), mul, sub, kUnit));
       }
     }
+    if (!DET) acc = ((uint64_t)sh.hi << 32) | sh.lo;
     const int glt = TL::group_of(hw, q0);            // first group of this register tile
     const int64_t tile_words = word_base + (int64_t)glt * WPG;
     const uint32_t lo = transpose32((uint32_t)acc, lane);
@@ -157,7 +174,7 @@ ACTNN_DEV void pack_groups(const float (&v)[Gph<T>::kPack][8], const float (&nz)
 }
 
 template <typename T, bool DET>
-__global__ __launch_bounds__(kThreads) void pack_mixed_kernel(
+__global__ __launch_bounds__(kThreads, DET ? 1 : 8) void pack_mixed_kernel(
     const T* __restrict__ data, const T* __restrict__ mn, const T* __restrict__ mx,
     const int32_t* __restrict__ bits, const int32_t* __restrict__ prefix, T* __restrict__ scale,
     int32_t* __restrict__ packed, const T* __restrict__ noise, uint64_t seed, uint64_t offset,
@@ -173,8 +190,8 @@ __global__ __launch_bounds__(kThreads) void pack_mixed_kernel(
 
   // The element loads do not depend on the bit width or the scales: get them in flight first,
   // then compute the block's scales while they travel.
-  float v[GPH][8];
-  float nz[DET ? GPH : 1][8];
+  Raw8<T> v[GPH];
+  Raw8<T> nz[DET ? GPH : 1];
   load_groups<T, DET, GPH>(data, noise, elem_base, groups_valid, v, nz);
 
   const int b = bits[n];
@@ -337,12 +354,12 @@ __global__ __launch_bounds__(kThreads) void pack_mixed_generic_kernel(
     if (DET) {
       c = det_code<T>(x, Conv<T>::load(noise, e), mul, sub, Bf);
     } else {
-      uint32_t r16[8];
-      philox_octet((uint64_t)e >> 3, seed, offset, r16);
-      uint32_t r = r16[0];
+      uint32_t w[Noise<T>::kWords];
+      Noise<T>::octet((uint64_t)e >> 3, seed, offset, w);
+      uint32_t r = Noise<T>::at(w, 0);
 #pragma unroll
-      for (int k = 1; k < 8; ++k) r = ((int)(e & 7) == k) ? r16[k] : r;
-      c = rng_code(x, r, mul, sub, Bf * 65536.0f);
+      for (int k = 1; k < 8; ++k) r = ((int)(e & 7) == k) ? Noise<T>::at(w, k) : r;
+      c = RngFixed<T>::word(x, r, mul, sub, RngFixed<T>::unit(b)) >> (32 - b);
     }
     s_code[d] = (uint8_t)c;
   }

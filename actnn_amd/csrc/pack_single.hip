@@ -64,26 +64,56 @@ __global__ __launch_bounds__(kThreads) void pack_single_kernel(
         mul[ni] = sc;
         sub[ni] = Conv<T>::round(m - Conv<T>::round(1e-6f));    // shifted minimum, ops.py:31
       } else {
-        mul[ni] = sc * 65536.0f;
-        sub[ni] = m;
+        RngFixed<T>::params(sc, m, BITS, mul[ni], sub[ni]);
       }
+    } else {                            // samples past the end of the batch: code 0
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[ni][k] = 0.0f;
+      mul[ni] = 0.0f;
+      sub[ni] = 0.0f;
     }
   }
   uint32_t lo = 0, hi = 0;   // bytes 0..3 and 4..7
+  if constexpr (DET) {
 #pragma unroll
-  for (int ni = 0; ni < WPT; ++ni) {
-    const int64_t n = no * WPT + ni;
-    if (n < N) {
-      uint32_t r16[8];
-      if (!DET) philox_octet((uint64_t)(((n * G + g) * gs + d0) >> 3), seed, offset, r16);
+    for (int ni = 0; ni < WPT; ++ni) {
+      const int64_t n = no * WPT + ni;
+      if (n < N) {
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const uint32_t c = DET ? det_code<T>(v[ni][k], nz[DET ? ni : 0][k], mul[ni], sub[ni], Bf)
-                               : rng_code(v[ni][k], r16[k], mul[ni], sub[ni], Bf * 65536.0f);
-        if (k < 4) lo |= c << (8 * k + ni * BITS);
-        else hi |= c << (8 * (k - 4) + ni * BITS);
+        for (int k = 0; k < 8; ++k) {
+          const uint32_t c = det_code<T>(v[ni][k], nz[ni][k], mul[ni], sub[ni], Bf);
+          if (k < 4) lo |= c << (8 * k + ni * BITS);
+          else hi |= c << (8 * (k - 4) + ni * BITS);
+        }
       }
     }
+  } else {
+    // Noise of the lane's octet in each sample.  Lane ^ 1 holds the neighbouring octet of the same
+    // samples when a group has an even number of octets (units is then even too, so the two lanes
+    // are here together), and the two share their Philox calls.
+    uint32_t rw[WPT][Noise<T>::kWords];
+    const uint64_t o0 = (uint64_t)(((no * WPT * G + g) * gs + d0) >> 3);    // sample no * WPT
+    const uint64_t per_sample = (uint64_t)(G * gs) >> 3;
+    if (WPT >= 2 && (chunks & 1) == 0) {
+#pragma unroll
+      for (int ni = 0; ni + 1 < WPT; ni += 2)
+        Noise<T>::octets(o0 + ni * per_sample, o0 + (ni + 1) * per_sample, seed, offset, rw[ni], rw[ni + 1]);
+    } else {
+#pragma unroll
+      for (int ni = 0; ni < WPT; ++ni) Noise<T>::octet(o0 + ni * per_sample, seed, offset, rw[ni]);
+    }
+    constexpr float kUnit = (float)(1u << (32 - BITS - Noise<T>::kBits));
+    CodeShifter<BITS, false> slo, shi;     // last byte first, last sample first within a byte
+#pragma unroll
+    for (int k = 3; k >= 0; --k) {
+#pragma unroll
+      for (int ni = WPT - 1; ni >= 0; --ni) {
+        slo.push(RngFixed<T>::word(v[ni][k], Noise<T>::at(rw[ni], k), mul[ni], sub[ni], kUnit));
+        shi.push(RngFixed<T>::word(v[ni][k + 4], Noise<T>::at(rw[ni], k + 4), mul[ni], sub[ni], kUnit));
+      }
+    }
+    lo = slo.lo;
+    hi = shi.lo;
   }
   *reinterpret_cast<uint2*>(packed + og * gs + d0) = make_uint2(lo, hi);
 }

@@ -7,8 +7,11 @@
 //    rounding per tensor op in the tensor dtype, clamp to [0, B], round half to even.
 //  * RNG (in-kernel Philox): the reference's CUDA kernel, quantization_cuda_kernel.cu:32,:65
 //    - scale = B / (max - min + 2e-6) evaluated in double, code = stochastic rounding of
-//    (x - min) * scale.  The rounding is done as floor(t + u) in 16.16 fixed point with a
-//    16-bit uniform u, which rounds up with probability frac(t) like rint(t + u - 0.5).
+//    (x - min) * scale.  The rounding is done as floor(t + u) with a uniform integer draw of
+//    K = Noise<T>::kBits bits (16 for fp32 tensors, 8 for 16-bit tensors), which rounds up with
+//    probability frac(t) like rint(t + u - 0.5).  It is evaluated in a 32-bit fixed point whose
+//    top `bits` bits are the code (see RngFixed below), so that the conversion to an integer is
+//    also the clamp and the code can be shifted into the output word with one instruction.
 //
 // This file must be compiled with -ffp-contract=off: every operation below is meant to
 // round on its own unless it is written as an explicit fmaf.
@@ -18,10 +21,47 @@
 
 namespace actnn {
 
+// RNG mode arithmetic.  One code level is 2^(32 - bits) and one step of the K-bit draw r is
+// U = 2^(32 - bits - K):
+//   t = fma(x - min, scale * 2^(32 - bits), U / 2)                        fp32 tensors
+//   t = fma(x, scale * 2^(32 - bits), U / 2 - min * scale * 2^(32 - bits)) 16-bit tensors
+//   word = sat_u32(fma(r, U, t));  code = word >> (32 - bits)
+// The conversion saturates (below 0 and NaN give 0, 2^32 and above give 2^32 - 1), which is the
+// clamp to [0, B].  16-bit tensors fold the subtraction of the minimum into the constant: their
+// values cannot resolve a group range below 2^-11 (2^-8 for bf16) of |min|, so the rounding of the
+// constant moves t by at most 2^-13 * B / 2^bits of a level (bf16: 2^-16); for fp32 tensors
+// |min| / range is unbounded and x - min (exact for nearby values) is kept.
+template <typename T> struct RngFixed {
+  static constexpr bool kFold = sizeof(T) == 2;
+  static ACTNN_DEV float unit(int bits) { return ldexpf(1.0f, 32 - bits - Noise<T>::kBits); }
+  // (mul, sub) for `word` from the stored scale (a value of T) and the group minimum
+  static ACTNN_DEV void params(float sc, float mn, int bits, float& mul, float& sub) {
+    mul = sc * ldexpf(1.0f, 32 - bits);
+    sub = kFold ? fmaf(-mn, mul, 0.5f * unit(bits)) : mn;
+  }
+  static ACTNN_DEV uint32_t word(float x, uint32_t r, float mul, float sub, float u) {
+    const float t = kFold ? fmaf(x, mul, sub) : fmaf(x - sub, mul, 0.5f * u);
+    const float w = fmaf((float)r, u, t);
+    uint32_t out;
+    asm("v_cvt_u32_f32_e32 %0, %1" : "=v"(out) : "v"(w));     // the instruction saturates
+    return out;
+  }
+};
+
+// Shift register that collects codes from the top of RngFixed words: push() moves the register up
+// by BITS and takes the code of `word` in at the bottom, so elements are pushed last-first.
+template <int BITS, bool TWO> struct CodeShifter {
+  uint32_t lo = 0, hi = 0;
+  ACTNN_DEV void push(uint32_t word) {
+    if (TWO) hi = __builtin_amdgcn_alignbit(hi, lo, 32 - BITS);
+    lo = __builtin_amdgcn_alignbit(lo, word, 32 - BITS);
+  }
+};
+
 template <typename T, bool DET> struct GroupQuant {
   // Returns the scale to store (already rounded to T, as float) and sets the two values
-  // the per-element code needs: `mul` (scale, times 2^16 in RNG mode) and `sub` (the
-  // minimum to subtract: shifted in DET mode, original in RNG mode).
+  // the per-element code needs.  DET mode: `mul` = scale, `sub` = the shifted minimum.
+  // RNG mode: the (mul, sub) of RngFixed<T>::params.
   static ACTNN_DEV float prepare(float mn, float mx, int bits, float& mul, float& sub) {
     const float Bf = (float)((1 << bits) - 1);
     if (DET) {
@@ -37,8 +77,7 @@ template <typename T, bool DET> struct GroupQuant {
       const float range = Conv<T>::round(mx - mn);              // max - min in scalar_t
       const double q = (double)Bf / ((double)range + 2e-6);     // .cu:32 (double literal)
       const float sc = Conv<T>::round((float)q);
-      mul = sc * 65536.0f;
-      sub = mn;
+      RngFixed<T>::params(sc, mn, bits, mul, sub);
       return sc;
     }
   }
@@ -86,12 +125,5 @@ template <typename T> struct Dequant {
     return Conv<T>::round(Conv<T>::round(q) + m);
   }
 };
-
-// RNG code: fix = trunc(clamp(fma(x - min, scale * 2^16, 0.5), 0, B * 2^16)); (fix + r16) >> 16.
-ACTNN_DEV uint32_t rng_code(float x, uint32_t r16, float mul, float sub, float Bfix) {
-  const float d = x - sub;
-  const float f = __builtin_amdgcn_fmed3f(fmaf(d, mul, 0.5f), 0.0f, Bfix);
-  return ((uint32_t)f + r16) >> 16;
-}
 
 }  // namespace actnn

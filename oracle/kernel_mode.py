@@ -7,9 +7,10 @@ Reference arithmetic (quantization_cuda_kernel.cu):
   code   = rint(max((x - min) * scale + u - 0.5, 0)), u ~ U(0,1]   :65, :253
   dequant= (scalar_t)code / scale + min                      :171, :359
 
-The HIP kernels draw ``u`` as a 16-bit Philox value and evaluate the equivalent
-stochastic floor ``floor(t + u)`` in 16.16 fixed point (``rng_codes`` below).  Rounding up
-with probability frac(t) is the same distribution as the reference's ``rint(t + u - 0.5)``;
+The HIP kernels draw ``u`` as a K-bit Philox value (K = 16 for fp32 tensors, 8 for fp16 / bf16
+tensors) and evaluate the equivalent stochastic floor ``floor(t + u)`` in a 32-bit fixed point
+whose top b bits are the code (``rng_codes`` below).  Rounding up with probability frac(t) (to
+within 2^-(K+1), centred) is the same distribution as the reference's ``rint(t + u - 0.5)``;
 the stream values themselves are not comparable with cuRAND's (parity unpinned) - the
 distribution is pinned by ``expected_code`` / ``code_variance`` (exact closed forms).
 """
@@ -50,41 +51,106 @@ def kernel_dequant(codes, scale, mn):
     return (q / scale + mn).to(dtype)
 
 
-def rng_fixed_point(data, mn, scale, bits):
-    """16.16 fixed-point image of t = (x - min) * scale as the HIP kernels compute it:
-    d = fl32(x - mn); f = fl32(fma(d, scale * 2^16, 0.5)); f = min(f, B * 2^16);
-    fix = trunc(max(f, 0)).  Returns uint32 [N,G,gs]."""
+def fma32(a, b, c):
+    """Correctly rounded float32 fma(a, b, c) of float32 arrays.  The product is exact in float64;
+    the float64 sum is turned into round-to-odd with the error term of the addition, after which
+    the narrowing to float32 rounds once (Boldo & Melquiond, "Emulation of FMA and correctly
+    rounded sums", 2008).  Pinned in tests/test_oracle_kernel_mode.py against exact rational
+    arithmetic."""
+    a = np.asarray(a, dtype=np.float32).astype(np.float64)
+    b = np.asarray(b, dtype=np.float32).astype(np.float64)
+    c = np.asarray(c, dtype=np.float32).astype(np.float64)
+    a, b, c = np.broadcast_arrays(a, b, c)
+    with np.errstate(invalid="ignore", over="ignore"):
+        p = a * b
+        s = p + c
+        bb = s - p
+        err = (p - (s - bb)) + (c - bb)                      # TwoSum: p + c = s + err exactly
+        inexact = np.isfinite(s) & np.isfinite(err) & (err != 0)
+        bits = s.view(np.int64) if s.flags["C_CONTIGUOUS"] else np.ascontiguousarray(s).view(np.int64)
+        even = (bits & 1) == 0
+        # an inexact sum with an even last bit moves one step towards the true value (then odd)
+        toward = np.where((err > 0) == (s > 0), 1, -1)       # the magnitude grows when err has the sign of s
+        toward = np.where(s == 0, 0, toward)
+        adj = np.where(inexact & even, toward, 0).astype(np.int64)
+        s = (bits + adj).view(np.float64)
+        return s.astype(np.float32)
+
+
+def noise_bits(dtype):
+    """Bits of the uniform draw per element: 16 for fp32 tensors, 8 for fp16 / bf16 tensors."""
+    return 16 if dtype == torch.float32 else 8
+
+
+def _rng_t(data, mn, scale, bits):
+    """The noise-free part t of the HIP kernels' fixed point (one level = 2^(32 - b), one noise
+    step U = 2^(32 - b - K)) and U.  fp32 tensors: t = fma(x - mn, scale * 2^(32-b), U/2);
+    16-bit tensors: t = fma(x, scale * 2^(32-b), fma(-mn, scale * 2^(32-b), U/2))."""
     N = data.shape[0]
+    K = noise_bits(data.dtype)
     b = np.broadcast_to(np.asarray(bits, dtype=np.int64), (N,)).reshape(N, 1, 1)
-    B = ((1 << b) - 1).astype(np.float64)
     x = data.detach().to(torch.float32).numpy()
     m = mn.detach().to(torch.float32).numpy()
-    d = (x - m).astype(np.float32)
-    S = (scale.detach().to(torch.float32).numpy() * np.float32(65536.0)).astype(np.float32)
-    f = (d.astype(np.float64) * S.astype(np.float64) + 0.5).astype(np.float32)   # exact fma
-    f = np.minimum(f, (B * 65536.0).astype(np.float32))
-    f = np.maximum(np.nan_to_num(f, nan=0.0), np.float32(0))
-    return np.trunc(f).astype(np.uint32)
+    with np.errstate(over="ignore", invalid="ignore"):
+        S = (scale.detach().to(torch.float32).numpy() * np.exp2(32 - b).astype(np.float32)).astype(np.float32)
+        U = np.exp2(32 - b - K).astype(np.float32)
+        if K == 16:
+            t = fma32((x - m).astype(np.float32), S, np.float32(0.5) * U)
+        else:
+            t = fma32(x, S, fma32(-m, S, np.float32(0.5) * U))
+    return t, U, b
+
+
+def _sat_u32(w):
+    """v_cvt_u32_f32: truncation, saturating at 0 and 2^32 - 1, NaN -> 0."""
+    w = np.nan_to_num(np.asarray(w, dtype=np.float64), nan=0.0, posinf=2.0 ** 32, neginf=0.0)
+    return np.clip(np.trunc(w), 0, 2.0 ** 32 - 1).astype(np.uint64)
+
+
+def _codes_for(t, U, b, r):
+    with np.errstate(over="ignore", invalid="ignore"):
+        w = fma32(np.asarray(r, dtype=np.float32), U, t)
+    return (_sat_u32(w) >> (32 - b).astype(np.uint64)).astype(np.int32)
 
 
 def rng_codes(data, mn, scale, bits, seed, offset):
-    """Codes the HIP RNG-mode kernels must produce (given their Philox stream)."""
-    fix = rng_fixed_point(data, mn, scale, bits)
-    e = np.arange(fix.size, dtype=np.uint64).reshape(fix.shape)
-    r = philox.noise16(e, seed, offset)
-    return ((fix.astype(np.uint64) + r.astype(np.uint64)) >> np.uint64(16)).astype(np.int32)
+    """Codes the HIP RNG-mode kernels must produce (given their Philox stream):
+    word = sat_u32(fma(r, U, t)), code = word >> (32 - b)."""
+    t, U, b = _rng_t(data, mn, scale, bits)
+    e = np.arange(t.size, dtype=np.uint64).reshape(t.shape)
+    r = philox.noise16(e, seed, offset) if noise_bits(data.dtype) == 16 else philox.noise8(e, seed, offset)
+    return _codes_for(t, U, b, r)
+
+
+def _round_up_count(data, mn, scale, bits):
+    """(code at draw 0, number of draws r in [0, 2^K) that give the next code, K).  The code is
+    non-decreasing in r and the draws span less than one level, so the count is found by bisection."""
+    t, U, b = _rng_t(data, mn, scale, bits)
+    K = noise_bits(data.dtype)
+    c0 = _codes_for(t, U, b, np.zeros(t.shape, np.float32))
+    lo = np.zeros(t.shape, np.int64)            # invariant: code(lo - 1) == c0 (or lo == 0)
+    hi = np.full(t.shape, 1 << K, np.int64)     # invariant: code(hi) > c0 (or hi == 2^K)
+    for _ in range(K + 1):
+        mid = (lo + hi) // 2
+        up = _codes_for(t, U, b, np.minimum(mid, (1 << K) - 1).astype(np.float32)) > c0
+        up &= mid < (1 << K)
+        hi = np.where(up, mid, hi)
+        lo = np.where(up, lo, np.minimum(mid + 1, hi))
+    return c0, (1 << K) - hi, K
 
 
 def expected_code(data, mn, scale, bits):
-    """E[code] under the 16-bit stochastic floor = fix / 2^16 (exact)."""
-    return rng_fixed_point(data, mn, scale, bits).astype(np.float64) / 65536.0
+    """E[code] under the K-bit uniform draw (exact: code(0) + P(next code))."""
+    c0, ups, K = _round_up_count(data, mn, scale, bits)
+    return c0.astype(np.float64) + ups.astype(np.float64) / (1 << K)
 
 
 def code_variance(data, mn, scale, bits):
-    """Var[code] = f (1 - f), f = fractional part of fix / 2^16 (exact closed form;
-    ActNN's bound R^2/(4 B^2) per element is its maximum, qscheme.py:84)."""
-    f = (rng_fixed_point(data, mn, scale, bits) & np.uint32(0xFFFF)).astype(np.float64) / 65536.0
-    return f * (1.0 - f)
+    """Var[code] = p (1 - p), p = P(next code) (exact; ActNN's bound R^2/(4 B^2) per element is its
+    maximum, qscheme.py:84)."""
+    _, ups, K = _round_up_count(data, mn, scale, bits)
+    p = ups.astype(np.float64) / (1 << K)
+    return p * (1.0 - p)
 
 
 def range_sqr(mn, mx, factor=1.0, mult=None):

@@ -46,3 +46,19 @@ def noise16(elem_index, seed, offset):
     k = (e & np.uint64(7)).astype(np.int64)
     w = np.take_along_axis(r, (k >> 1)[..., None], axis=-1)[..., 0]
     return ((w >> ((k & 1) * 16).astype(np.uint32)) & np.uint32(0xFFFF)).astype(np.uint32)
+
+
+def noise8(elem_index, seed, offset):
+    """8-bit noise of flat element index ``e`` as the HIP kernels define it for fp16 / bf16 tensors:
+    one Philox call per 16 consecutive elements, counter = (lo(e>>4), hi(e>>4), lo(offset),
+    hi(offset)), key = (lo(seed), hi(seed)); element ``e & 15`` takes byte ``e & 3`` (low first) of
+    output word ``(e & 15) >> 2``."""
+    e = np.asarray(elem_index, dtype=np.uint64)
+    o = e >> np.uint64(4)
+    ctr = np.stack([(o & MASK32).astype(np.uint32), (o >> np.uint64(32)).astype(np.uint32),
+                    np.full(o.shape, offset & 0xFFFFFFFF, np.uint32),
+                    np.full(o.shape, (offset >> 32) & 0xFFFFFFFF, np.uint32)], axis=-1)
+    r = philox4x32_10(ctr, (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF))
+    k = (e & np.uint64(15)).astype(np.int64)
+    w = np.take_along_axis(r, (k >> 2)[..., None], axis=-1)[..., 0]
+    return ((w >> ((k & 3) * 8).astype(np.uint32)) & np.uint32(0xFF)).astype(np.uint32)

@@ -141,6 +141,25 @@ def test_rng_mode_unbiased_with_closed_form_variance(bits):
     assert (out64.var(axis=0) <= (rng_ ** 2) / (4 * B * B) * 1.1 + 1e-12).all()
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+def test_rng_mode_mean_code_of_16bit_tensors(dtype, bits):
+    # 16-bit tensors round with an 8-bit draw: over 4096 independent roundings the mean code of every
+    # element is the model's expectation (within 5 sigma of its exact variance), and that
+    # expectation is the exact (x - min) * scale to within 2^-9 of a level
+    trials, G = 4096, 2
+    base, _ = make_groups(1, G, 256, dtype, 78, "chan")
+    x = base.expand(trials, G, 256).contiguous()
+    xd, mn, mx, bits_dev, bits_host, packed, scale, seed, offset = _rng_pack(x, [bits] * trials, 17)
+    codes = layouts.unpack_mixed(packed.cpu().numpy(), bits_host.numpy(), trials, G, 256)
+    mean = codes.astype(np.float64).mean(axis=0)
+    expect = kernel_mode.expected_code(base, mn[:1].cpu(), scale[:1].cpu(), bits)[0]
+    sigma = np.sqrt(kernel_mode.code_variance(base, mn[:1].cpu(), scale[:1].cpu(), bits)[0] / trials)
+    assert (np.abs(mean - expect) <= 5 * sigma + 1e-9).all()
+    exact = (base.double() - mn[:1].double().cpu()).numpy()[0] * scale[0].double().cpu().numpy()
+    assert (np.abs(expect - np.minimum(exact, 2 ** bits - 1)) <= 2.0 ** -9 + 2.0 ** -12).all()
+
+
 def test_streams_of_different_calls_differ():
     x, _ = make_groups(4, 8, 256, torch.float32, 1)
     a = _rng_pack(x, [2] * 4, 5)[5]

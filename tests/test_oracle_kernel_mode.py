@@ -151,3 +151,51 @@ def test_dequant_rounds_once_per_operation(dtype, fmt):
                 fused_differs += float(rn(c / s + m, fmt)) != float(want)
     if fmt != "f32":
         assert fused_differs > 0        # the test would notice a single-rounding implementation
+
+
+def test_fma32_rounds_once():
+    # against exact rational arithmetic, with cancelling addends (where a product rounded first, or a
+    # float64 sum rounded a second time, gives another answer)
+    rng = np.random.default_rng(0)
+    n = 3000
+    a = (rng.standard_normal(n) * 10.0 ** rng.integers(-3, 6, n)).astype(np.float32)
+    b = (rng.standard_normal(n) * 10.0 ** rng.integers(-3, 6, n)).astype(np.float32)
+    c = (rng.standard_normal(n) * 10.0 ** rng.integers(-3, 9, n)).astype(np.float32)
+    c[: n // 3] = (-a[: n // 3].astype(np.float64) * b[: n // 3]).astype(np.float32)
+    got = km.fma32(a, b, c)
+    product_first_differs = 0
+    for i in range(n):
+        exact = Fraction(float(a[i])) * Fraction(float(b[i])) + Fraction(float(c[i]))
+        assert float(got[i]) == float(rn(exact, "f32")), i
+        product_first_differs += float(np.float32(a[i] * b[i]) + c[i]) != float(got[i])
+    assert product_first_differs > 0
+    # ties of the float64 sum that a second rounding would resolve the wrong way
+    one, eps = np.float32(1.0), np.float32(2.0 ** -24)
+    assert float(km.fma32(one, one + np.float32(2.0 ** -23), -one)) == 2.0 ** -23
+    assert float(km.fma32(np.float32(1 + 2.0 ** -23), np.float32(1 + 2.0 ** -23), eps * eps)) == \
+        float(rn(Fraction(1 + 2.0 ** -23) ** 2 + Fraction(2.0 ** -48), "f32"))
+
+
+@pytest.mark.parametrize("dtype,K", [(torch.float32, 16), (torch.float16, 8), (torch.bfloat16, 8)])
+def test_rng_model_rounds_up_with_probability_of_the_fraction(dtype, K):
+    # brute force over every draw on a small case: the mean code is the exact t to within half a
+    # step of the draw (plus, for 16-bit tensors, the rounding of the folded constant), for each width
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(8, 2, 256, generator=g) * 3 + 1).to(dtype)
+    mn, mx = x.min(2, keepdim=True)[0], x.max(2, keepdim=True)[0]
+    bits = torch.arange(1, 9, dtype=torch.int32)
+    scale = km.kernel_scale(mn, mx, bits)
+    t, U, b = km._rng_t(x, mn, scale, bits)
+    draws = np.arange(1 << K, dtype=np.float32) if K == 8 else np.arange(0, 1 << K, 97, dtype=np.float32)
+    mean = np.mean([km._codes_for(t, U, b, np.full(t.shape, r, np.float32)) for r in draws], axis=0)
+    exact = (x.double() - mn.double()).numpy() * scale.double().numpy()
+    # a scale rounded up in the tensor dtype can put the group maximum above B: the kernels clamp
+    exact = np.minimum(exact, (2.0 ** bits.numpy() - 1).reshape(-1, 1, 1))
+    tol = 2.0 ** -(K + 1) + (97 / 2.0 ** K if K == 16 else 0) + 2.0 ** -12
+    assert np.abs(mean - exact).max() <= tol
+    if K == 8:
+        assert np.allclose(km.expected_code(x, mn, scale, bits), mean, atol=1e-12)
+        p = mean - np.floor(mean + 1e-12)
+        assert np.allclose(km.code_variance(x, mn, scale, bits), p * (1 - p), atol=1e-9)
+    assert km._codes_for(t, U, b, np.full(t.shape, (1 << K) - 1, np.float32)).max() == 255
+    assert (km._codes_for(t, U, b, np.zeros(t.shape, np.float32)).reshape(8, -1).max(1) <= 2 ** np.arange(1, 9) - 1).all()

@@ -38,3 +38,22 @@ def test_noise16_uniform():
     r = philox.noise16(np.arange(1 << 18, dtype=np.uint64), 7, 0).astype(np.float64)
     assert abs(r.mean() - 32767.5) < 120
     assert abs(r.var() - (65536.0 ** 2 - 1) / 12) / (65536.0 ** 2 / 12) < 0.01
+
+
+def test_noise8_mapping():
+    # element e uses byte (e & 3) of word (e & 15) >> 2 of the call with counter e >> 4
+    seed, off = 0x1234567890ABCDEF, 0x55AA000012345678
+    e = np.arange(96, dtype=np.uint64)
+    got = philox.noise8(e, seed, off)
+    for o in range(6):
+        r = philox.philox4x32_10(np.array([[o, 0, off & 0xFFFFFFFF, off >> 32]], dtype=np.uint32),
+                                 (seed & 0xFFFFFFFF, seed >> 32))[0]
+        for k in range(16):
+            assert int(got[16 * o + k]) == (int(r[k >> 2]) >> (8 * (k & 3))) & 0xFF
+
+
+def test_noise8_uniform():
+    r = philox.noise8(np.arange(1 << 18, dtype=np.uint64), 7, 0).astype(np.float64)
+    assert abs(r.mean() - 127.5) < 0.5
+    assert abs(r.var() - (256.0 ** 2 - 1) / 12) / (256.0 ** 2 / 12) < 0.01
+    assert np.bincount(r.astype(np.int64), minlength=256).min() > 0.8 * (1 << 18) / 256
