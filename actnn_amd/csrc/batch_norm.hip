@@ -288,24 +288,56 @@ ACTNN_DEV void pack_chunk_bits(const float (&v)[8], const uint32_t (&rw)[Noise<T
   }
 }
 
-// b = bits[n], first_word = prefix[n] * G * 8: looked up by the caller, who knows how often n changes
+// Quantisation parameters of the next 32 chunks a half-wave will pack (its 32 lanes own one group in
+// every chunk): lane j works out the scale of chunk j - one evaluation of the double-precision
+// quotient per group instead of one per lane and group - stores it, and hands (mul, sub) to the
+// other lanes when chunk j's turn comes.
+template <typename T> struct ParamQueue {
+  float mul = 0.0f, sub = 0.0f;
+  // lane j: gi = index of the group of chunk j (n * G + group within the sample), b = its width;
+  // live = chunk j exists
+  ACTNN_DEV void fill(const PackSink& ps, int64_t gi, int b, bool live) {
+    mul = 0.0f;
+    sub = 0.0f;
+    if (live) {
+      const float sc = GroupQuant<T, false>::prepare(Conv<T>::load(static_cast<const T*>(ps.mn), gi),
+                                                     Conv<T>::load(static_cast<const T*>(ps.mx), gi), b, mul, sub);
+      Conv<T>::store(static_cast<T*>(ps.scale), gi, sc);
+    }
+  }
+  ACTNN_DEV void get(int j, float& m, float& sb) const {
+    m = __shfl(mul, j, 32);
+    sb = __shfl(sub, j, 32);
+  }
+};
+
+// Noise words of two octets of this lane whose neighbours (index ^ 1) lane ^ 1 holds: the two lanes
+// share their Philox calls when octet and lane parity agree (they do wherever a block starts on an
+// even octet; the test is the same for every lane of a block).
 template <typename T>
-ACTNN_DEV void pack_chunk(const PackSink& ps, const u32x4& ux, int64_t n, int64_t grp, int64_t octet, int b,
-                          int64_t first_word) {
+ACTNN_DEV void noise_pair(const PackSink& ps, uint64_t oa, uint64_t ob, uint32_t (&wa)[Noise<T>::kWords],
+                          uint32_t (&wb)[Noise<T>::kWords], bool together) {
+  // together: lane ^ 1 is known to make this call in the same step
+  if (together && (((uint32_t)oa ^ threadIdx.x) & 1u) == 0 && (((uint32_t)ob ^ threadIdx.x) & 1u) == 0) {
+    Noise<T>::octets(oa, ob, ps.seed, ps.offset, wa, wb);
+  } else {
+    Noise<T>::octet(oa, ps.seed, ps.offset, wa);
+    Noise<T>::octet(ob, ps.seed, ps.offset, wb);
+  }
+}
+
+// b = bits[n], first_word = prefix[n] * G * 8: looked up by the caller, who knows how often n changes;
+// (mul, sub): the group's parameters from the queue; rw: the noise words of the chunk's octet
+template <typename T>
+ACTNN_DEV void pack_chunk(const PackSink& ps, const u32x4& ux, const uint32_t (&rw)[Noise<T>::kWords],
+                          float mul, float sub, int64_t grp, int b, int64_t first_word) {
   constexpr int PD = Chunk<T>::kPerDword;
   static_assert(Chunk<T>::kElems == 8, "16-bit types only");
   const uint32_t lane32 = threadIdx.x & 31;
-  const int64_t gi = n * ps.G + grp;
-  float mul, sub;
-  const float sc = GroupQuant<T, false>::prepare(Conv<T>::load(static_cast<const T*>(ps.mn), gi),
-                                                 Conv<T>::load(static_cast<const T*>(ps.mx), gi), b, mul, sub);
-  if (lane32 == 0) Conv<T>::store(static_cast<T*>(ps.scale), gi, sc);
   const uint32_t w[4] = {ux.x, ux.y, ux.z, ux.w};
   float v[8];
 #pragma unroll
   for (int k = 0; k < 4; ++k) Chunk<T>::widen(w[k], v + k * PD);
-  uint32_t rw[Noise<T>::kWords];
-  Noise<T>::octet((uint64_t)octet, ps.seed, ps.offset, rw);
   int32_t* dst = ps.packed + first_word + grp * b * 8;
   switch (b) {                           // uniform over the half-wave: one sample, one width
     case 1: pack_chunk_bits<T, 1>(v, rw, mul, sub, lane32, dst); break;
@@ -499,7 +531,8 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
   constexpr int E = Chunk<T>::kElems;
   constexpr int PD = Chunk<T>::kPerDword;
   constexpr int NC = BWD ? 3 : 2;
-  constexpr int kUnroll = PACK ? 2 : XS::kInFlight;      // measured: 2 beats 1 and 4 with the pack
+  constexpr int kUnroll = XS::kInFlight;
+  static_assert(!(PACK && BWD), "the packed copy is made by the forward pass");
   const Place p = place_of<E>(F, HW);
   float sumsq = 0.0f;
   if (!BWD && !p.active) return;       // whole quantisation groups (32 lanes) leave together
@@ -544,6 +577,49 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
 
   const T* pd = BWD ? dy + p.elem : nullptr;
   T* po = out + p.elem;
+  if constexpr (PACK) {
+    // 32 samples at a time: lane j prepares the group's parameters for sample nb + j, then the
+    // half-wave packs the samples two by two (the two chunks of a lane and those of lane ^ 1 are
+    // neighbouring octets of the same two groups, and whole groups are present or absent together)
+    const int lane32 = threadIdx.x & 31;
+    const int64_t grp = p.elem >> 8;
+    ParamQueue<T> queue;
+    for (int64_t nb = n0; nb < n1; nb += 32) {
+      const int64_t ne = nb + 32 < n1 ? nb + 32 : n1;
+      {
+        const int64_t nj = nb + lane32;
+        const bool live = nj < ne;
+        queue.fill(ps, nj * ps.G + grp, live ? ps.bits[nj] : 1, live);
+      }
+      int64_t n = nb;
+      for (; n + 2 <= ne; n += 2) {
+        typename XS::Raw rx[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) rx[u] = xs.fetch(n + u);
+        uint32_t rw[2][Noise<T>::kWords];
+        const uint64_t o = (uint64_t)((n * F + p.elem) >> 3);
+        noise_pair<T>(ps, o, o + (uint64_t)(F >> 3), rw[0], rw[1], true);
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const u32x4 ux = xs.decode(rx[u]);
+          store_out(po + (n + u) * F, apply(ux, ux));
+          float mul, sub;
+          queue.get((int)(n + u - nb), mul, sub);
+          pack_chunk<T>(ps, ux, rw[u], mul, sub, grp, ps.bits[n + u], (int64_t)ps.prefix[n + u] * ps.G * 8);
+        }
+      }
+      for (; n < ne; ++n) {
+        const typename XS::Raw rx = xs.fetch(n);
+        const u32x4 ux = xs.decode(rx);
+        store_out(po + n * F, apply(ux, ux));
+        uint32_t rw[Noise<T>::kWords];
+        Noise<T>::octet((uint64_t)((n * F + p.elem) >> 3), ps.seed, ps.offset, rw);
+        float mul, sub;
+        queue.get((int)(n - nb), mul, sub);
+        pack_chunk<T>(ps, ux, rw, mul, sub, grp, ps.bits[n], (int64_t)ps.prefix[n] * ps.G * 8);
+      }
+    }
+  } else {
   int64_t n = n0;
   for (; n + kUnroll <= n1; n += kUnroll) {
     typename XS::Raw rx[kUnroll];
@@ -557,17 +633,13 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
     for (int u = 0; u < kUnroll; ++u) {
       const u32x4 ux = xs.decode(rx[u]);
       store_out(po + (n + u) * F, apply(ux, BWD ? ud[u] : ux));
-      if constexpr (PACK)
-        pack_chunk<T>(ps, ux, n + u, p.elem >> 8, ((n + u) * F + p.elem) >> 3, ps.bits[n + u],
-                      (int64_t)ps.prefix[n + u] * ps.G * 8);
     }
   }
   for (; n < n1; ++n) {
     const typename XS::Raw rx = xs.fetch(n);
     const u32x4 ux = xs.decode(rx);
     store_out(po + n * F, apply(ux, BWD ? load_last(pd + n * F) : ux));
-    if constexpr (PACK)
-      pack_chunk<T>(ps, ux, n, p.elem >> 8, (n * F + p.elem) >> 3, ps.bits[n], (int64_t)ps.prefix[n] * ps.G * 8);
+  }
   }
   }
   if (BWD && ps.sumsq) leave_wave_sum(ps.sumsq, sumsq);
@@ -733,20 +805,17 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
   constexpr int E = Chunk<T>::kElems;
   constexpr int PD = Chunk<T>::kPerDword;
   constexpr int NC = BWD ? 3 : 2;
-  constexpr int U = PACK ? 1 : XS::kInFlight;            // measured: 1 beats 2 and 4 with the pack here
+  constexpr int U = XS::kInFlight;
+  static_assert(!(PACK && BWD), "the packed copy is made by the forward pass");
   uint32_t cur_n = 0;                    // the sample whose width and first word are held below
   int cur_b = 1;
   int64_t cur_first = 0, cur_row0 = -(int64_t)HW - 1;
-  auto pack_row = [&](const u32x4& ux, int64_t row, int64_t col) {
-    if constexpr (PACK) {
-      if ((uint64_t)(row - cur_row0) >= HW) {              // left the sample (or the first row)
-        cur_n = (uint32_t)row / HW;                        // rows < 2^31 (checked by the launcher)
-        cur_row0 = (int64_t)cur_n * HW;
-        cur_b = ps.bits[cur_n];
-        cur_first = (int64_t)ps.prefix[cur_n] * ps.G * 8;
-      }
-      const int64_t flat = row * C + col;
-      pack_chunk<T>(ps, ux, cur_n, (flat >> 8) - (int64_t)cur_n * ps.G, flat >> 3, cur_b, cur_first);
+  auto locate = [&](int64_t row) {       // width and first word of the sample that holds `row`
+    if ((uint64_t)(row - cur_row0) >= HW) {                // left the sample (or the first row)
+      cur_n = (uint32_t)row / HW;                          // rows < 2^31 (checked by the launcher)
+      cur_row0 = (int64_t)cur_n * HW;
+      cur_b = ps.bits[cur_n];
+      cur_first = (int64_t)ps.prefix[cur_n] * ps.G * 8;
     }
   };
   const RowTile t = row_tile<E>(C, tpr, R);
@@ -786,6 +855,49 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
 
   const T* pd = BWD ? dy + t.col : nullptr;
   T* po = out + t.col;
+  if constexpr (PACK) {
+    // 32 steps (rows r0, r0 + R, ...) at a time: lane j prepares the parameters of the group the
+    // half-wave meets in step j, then the rows are packed two by two so that lane pairs can share
+    // their noise
+    const int lane32 = threadIdx.x & 31;
+    ParamQueue<T> queue;
+    auto pack_one = [&](const u32x4& ux, const uint32_t (&rw)[Noise<T>::kWords], int64_t row, int j) {
+      locate(row);
+      float mul, sub;
+      queue.get(j, mul, sub);
+      pack_chunk<T>(ps, ux, rw, mul, sub, ((row * C + t.col) >> 8) - (int64_t)cur_n * ps.G, cur_b, cur_first);
+    };
+    for (int64_t rb = p0 + t.r; rb < p1; rb += (int64_t)32 * R) {
+      {
+        const int64_t rj = rb + (int64_t)lane32 * R;
+        const bool live = rj < p1;
+        const uint32_t nj = live ? (uint32_t)rj / HW : 0;
+        queue.fill(ps, (rj * C + t.col) >> 8, live ? ps.bits[nj] : 1, live);
+      }
+      int j = 0;
+      for (; j + 2 <= 32 && rb + (int64_t)(j + 1) * R < p1; j += 2) {
+        const int64_t r0 = rb + (int64_t)j * R, r1 = r0 + R;
+        const typename XS::Raw rx0 = xs.fetch(r0), rx1 = xs.fetch(r1);
+        uint32_t rw[2][Noise<T>::kWords];
+        noise_pair<T>(ps, (uint64_t)((r0 * C + t.col) >> 3), (uint64_t)((r1 * C + t.col) >> 3), rw[0], rw[1],
+                      (tpr & 1) == 0);      // lane ^ 1 is in the same row, hence in the same steps
+        const u32x4 ux0 = xs.decode(rx0);
+        store_out(po + r0 * C, apply(ux0, ux0));
+        pack_one(ux0, rw[0], r0, j);
+        const u32x4 ux1 = xs.decode(rx1);
+        store_out(po + r1 * C, apply(ux1, ux1));
+        pack_one(ux1, rw[1], r1, j + 1);
+      }
+      for (; j < 32 && rb + (int64_t)j * R < p1; ++j) {
+        const int64_t r0 = rb + (int64_t)j * R;
+        const u32x4 ux = xs.decode(xs.fetch(r0));
+        store_out(po + r0 * C, apply(ux, ux));
+        uint32_t rw[Noise<T>::kWords];
+        Noise<T>::octet((uint64_t)((r0 * C + t.col) >> 3), ps.seed, ps.offset, rw);
+        pack_one(ux, rw, r0, j);
+      }
+    }
+  } else {
   int64_t row = p0 + t.r;
   for (; row + (int64_t)(U - 1) * R < p1; row += (int64_t)U * R) {
     typename XS::Raw rx[U];
@@ -799,14 +911,13 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
     for (int u = 0; u < U; ++u) {
       const u32x4 ux = xs.decode(rx[u]);
       store_out(po + (row + (int64_t)u * R) * C, apply(ux, BWD ? ud[u] : ux));
-      pack_row(ux, row + (int64_t)u * R, t.col);
     }
   }
   for (; row < p1; row += R) {
     const typename XS::Raw rx = xs.fetch(row);
     const u32x4 ux = xs.decode(rx);
     store_out(po + row * C, apply(ux, BWD ? load_last(pd + row * C) : ux));
-    pack_row(ux, row, t.col);
+  }
   }
   }
   if (BWD && ps.sumsq) leave_wave_sum(ps.sumsq, sumsq);
