@@ -253,7 +253,14 @@ def other_configs(device, reps):
     del xb16, lo16, hi16, bits16, p4, s4
     torch.cuda.empty_cache()
     out.update(config4(device, reps))
-    return {k_: {kk: round(vv, 4) for kk, vv in v.items()} for k_, v in out.items()}
+    return _rounded(out)
+
+
+def _rounded(v):
+    """Floats of a nested dict rounded to 4 decimals."""
+    if isinstance(v, dict):
+        return {k: _rounded(x) for k, x in v.items()}
+    return round(v, 4) if isinstance(v, float) else v
 
 
 def config4(device, reps):
@@ -295,6 +302,15 @@ def config4(device, reps):
     t = _event_time_ms(unfused, reps)
     out["linear_grad_weight_unfused_unpack_plus_mm"] = {"ms": t, "TFLOP/s": flops / t / 1e9,
                                                         "frac_mfma_bf16": flops / t / 1e9 / MFMA_BF16_PEAK_TFLOPS}
+    # How much of the GEMM's time is the operands' data (the matrix pipes run against the power
+    # limit): the same two launches - the fused kernel, and rocBLAS alone on the dequantised
+    # input - with grad_out drawn from N(0,1), all zeros, and all ones.
+    xd = ext_q.unpack_single_precision(packed, 2, scale, mn, M, I // 256, 256).view(M, I)
+    dep = {}
+    for name, g in (("normal", go), ("zeros", torch.zeros_like(go)), ("ones", torch.ones_like(go))):
+        dep[name] = {"fused_ms": _event_time_ms(lambda: ext_q.linear_grad_weight_q2(g, packed, scale, mn, I), reps),
+                     "rocblas_mm_ms": _event_time_ms(lambda: g.t().mm(xd), reps)}
+    out["linear_grad_weight_time_by_grad_out_data"] = dep
     return out
 
 
@@ -372,8 +388,7 @@ def main():
         print(json.dumps({"other_configs": other_configs(device, max(10, args.steps // 2))}))
         return
     if args.only == "config4":
-        print(json.dumps({"config4": {k: {kk: round(vv, 4) for kk, vv in v.items()}
-                                      for k, v in config4(device, max(10, args.steps // 2)).items()}}))
+        print(json.dumps({"config4": _rounded(config4(device, max(10, args.steps // 2)))}))
         return
     if args.only == "resnet50":
         import bench_extra
@@ -469,14 +484,14 @@ def main():
     }
     del xg, mn, mx, bits
     torch.cuda.empty_cache()
-    xs, mns, mxs, bits_s, bits_s_host = make_config2(device, sample_spread=0.7)
-    avg_s = float(bits_s_host.float().mean())
-    ks, pair_s = config2_kernel_times(xs, mns, mxs, bits_s, algorithmic_bytes(n, 4, avg_s), reps)
-    result["kernels_mixed_spread"] = {"widths": _width_histogram(bits_s_host), "avg_bits": round(avg_s, 3),
-                                      "kernels": ks, "minimax_plus_pack": pair_s}
-    del xs, mns, mxs, bits_s
-    torch.cuda.empty_cache()
     if not args.skip_extra:
+        xs, mns, mxs, bits_s, bits_s_host = make_config2(device, sample_spread=0.7)
+        avg_s = float(bits_s_host.float().mean())
+        ks, pair_s = config2_kernel_times(xs, mns, mxs, bits_s, algorithmic_bytes(n, 4, avg_s), reps)
+        result["kernels_mixed_spread"] = {"widths": _width_histogram(bits_s_host), "avg_bits": round(avg_s, 3),
+                                          "kernels": ks, "minimax_plus_pack": pair_s}
+        del xs, mns, mxs, bits_s
+        torch.cuda.empty_cache()
         try:
             result["other_configs"] = other_configs(device, max(10, args.steps // 2))
         except Exception as e:                       # keep the headline line even if an extra fails
