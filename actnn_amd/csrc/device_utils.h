@@ -70,6 +70,26 @@ ACTNN_DEV u32x4 load16(const void* p) { return *reinterpret_cast<const u32x4*>(p
 ACTNN_DEV void store16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
 ACTNN_DEV void store16_nt(void* p, u32x4 v) { __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p)); }
 
+// 16 bytes per lane from global memory straight into LDS: lane l's data lands at lds_base + 16 * l
+// (lds_base uniform in the wave).  Written as an instruction sequence of its own: the load is
+// asynchronous and the code that issues it waits for it explicitly (vmcnt) before the data is read; issued through the compiler's builtin, every LDS read that follows - also of
+// another buffer - would first wait for all loads in flight.
+ACTNN_DEV void load_to_lds16(const void* src, const uint8_t* lds_base) {
+  const uint32_t base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)lds_base;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(base)), "v"(src)
+               : "memory");
+}
+// The same with the non-temporal hint, for data that is read once.
+ACTNN_DEV void load_to_lds16_nt(const void* src, const uint8_t* lds_base) {
+  const uint32_t base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)lds_base;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(base)), "v"(src)
+               : "memory");
+}
+
 // ------------------------------------------------------------------ 8 / 16 contiguous elements
 // load8: 8 consecutive elements starting at p (32-byte aligned for f32, 16 for 16-bit types).
 ACTNN_DEV void load8(const float* p, float (&v)[8]) {

@@ -140,19 +140,6 @@ ACTNN_DEV u32x2 read_transposed(const uint8_t* p) {
   return __builtin_bit_cast(u32x2, v);
 }
 
-// 16 bytes per lane from global memory straight into LDS: lane l's data lands at lds_base + 16 * l
-// (lds_base uniform in the wave).  Written as an instruction sequence of its own: the load is
-// asynchronous and the code that issues it waits for it explicitly (vmcnt) before the barrier that
-// publishes the tile; issued through the compiler's builtin, every LDS read that follows - also of
-// the other buffer - would first wait for all loads in flight.
-ACTNN_DEV void load_to_lds16(const void* src, const uint8_t* lds_base) {
-  const uint32_t base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)lds_base;
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-               :
-               : "s"(__builtin_amdgcn_readfirstlane(base)), "v"(src)
-               : "memory");
-}
-
 // What describes the packed input.  bits == nullptr: the fixed-width stream at `fixed_bits`.
 struct Stream {
   const uint8_t* packed;

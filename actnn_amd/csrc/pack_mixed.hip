@@ -192,7 +192,24 @@ __global__ __launch_bounds__(kThreads, DET ? 1 : 8) void pack_mixed_kernel(
   // then compute the block's scales while they travel.
   Raw8<T> v[GPH];
   Raw8<T> nz[DET ? GPH : 1];
-  load_groups<T, DET, GPH>(data, noise, elem_base, groups_valid, v, nz);
+  // fp32 in RNG mode: a lane's 8 elements are 32 bytes, so a direct load would touch every cache
+  // line with two instructions of the wave.  The wave's groups (4 KiB, contiguous) instead travel
+  // straight into LDS, one whole 1 KiB group per instruction and no registers, and each lane then
+  // picks its 32 bytes out of LDS.
+  constexpr bool kViaLds = sizeof(T) == 4 && !DET;
+  __shared__ __align__(16) uint8_t s_stage[kViaLds ? kGroupsPerBlock * kGs * 4 : 16];
+  if constexpr (kViaLds) {
+    const int wave = threadIdx.x >> 6;
+    const uint32_t wl = threadIdx.x & 63;
+#pragma unroll
+    for (int i = 0; i < 2 * GPH; ++i) {
+      const int gl = wave * 2 * GPH + i;                       // the wave's two half-waves own these groups
+      if (gl < groups_valid)
+        load_to_lds16_nt(data + elem_base + (int64_t)gl * kGs + wl * 4, s_stage + gl * (kGs * 4));
+    }
+  } else {
+    load_groups<T, DET, GPH>(data, noise, elem_base, groups_valid, v, nz);
+  }
 
   const int b = bits[n];
   if (threadIdx.x < kGroupsPerBlock) {
@@ -206,6 +223,21 @@ __global__ __launch_bounds__(kThreads, DET ? 1 : 8) void pack_mixed_kernel(
     s_sub[threadIdx.x] = sub;
   }
   __syncthreads();
+  if constexpr (kViaLds) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");             // this wave's own groups have landed
+    const uint32_t lane = threadIdx.x & 31;
+    const int hw = threadIdx.x >> 5;
+#pragma unroll
+    for (int q = 0; q < GPH; ++q) {
+      const int gl = Tile<1, GPH>::group_of(hw, q);
+      raw8_zero(v[q]);
+      if (gl < groups_valid) {
+        const u32x4* src = reinterpret_cast<const u32x4*>(s_stage + gl * (kGs * 4) + lane * 32);
+        v[q].a = src[0];
+        v[q].b = src[1];
+      }
+    }
+  }
 
   const int64_t word_base = (int64_t)prefix[n] * G * 8 + gb * 8 * b;
   switch (b) {

@@ -1,6 +1,7 @@
 """Extra benchmark legs used by bench.py: the ResNet-50 training step under QModule at L3
 (benchmark config 5) with the reference's speed and memory protocols
 (mem_speed_benchmark/train.py:363-397 memory, :422-438 speed)."""
+import sys
 import time
 
 import torch
@@ -49,6 +50,11 @@ def resnet50_step(device, level="L3", batch=512, warmup=3, steps=10, autocast=Tr
         torch.cuda.synchronize()
         if it >= warmup:
             times.append(time.perf_counter() - t0)
+        # progress on stderr: the first steps of a fresh process spend minutes in the convolution
+        # library's solver search, and a silent process looks hung to whoever supervises it
+        print(f"[bench] resnet50 {level} {'channels_last' if channels_last else 'contiguous'} "
+              f"autocast={autocast} step {it + 1}/{warmup + steps}: {time.perf_counter() - t0:.3f} s",
+              file=sys.stderr, flush=True)
     peak = torch.cuda.max_memory_allocated()
     times.sort()
     med = times[len(times) // 2]

@@ -25,8 +25,12 @@ Pinning status (what fixes each function besides its own formula):
   tests/test_oracle_kernel_mode.py: known answers where evaluating the scale in float instead
   of double, or narrowing double -> half directly, would store another value; an exact
   rational-arithmetic model of the rounding chain; constant groups (+inf in fp16) and B = 255.
-* ``kernel_mode.rng_codes`` and the rest of the in-kernel-RNG model - values are only pinned
-  statistically (unbiasedness, closed-form variance) because the reference's RNG stream
-  (cuRAND) is not reproducible here: the *stream values* are parity unpinned, the
-  distribution is pinned.
+* ``kernel_mode.fma32`` (correctly rounded float32 fma, used by the RNG model) - exact
+  rational arithmetic on random and cancelling operands (tests/test_oracle_kernel_mode.py).
+* ``kernel_mode.rng_codes`` and the rest of the in-kernel-RNG model - the arithmetic is pinned
+  against the exact (x - min) * scale by brute force over every draw (8-bit noise) or a
+  sweep (16-bit noise), and ``philox.noise8`` / ``noise16`` against the generator's words;
+  the *stream values* of the reference's generator (cuRAND) are not reproducible here:
+  parity unpinned for the values, the distribution (unbiasedness, closed-form variance) is
+  pinned.
 """
