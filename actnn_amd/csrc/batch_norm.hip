@@ -362,7 +362,7 @@ template <typename T> ACTNN_DEV void bind_input(PackedInput<T>& xs, const Place&
 // Pass 1 of either direction.  Forward: per-channel sum(x) and sum(x*x) (+ per-group min/max of
 // x when MINMAX).  Backward: per-channel sum(dy) and sum(x*dy).
 template <typename T, bool SPLIT, bool BWD, bool MINMAX, typename XS>
-__global__ __launch_bounds__(kThreads) void bn_reduce_kernel(
+__global__ __launch_bounds__(kThreads, 6) void bn_reduce_kernel(
     XS xs, const T* __restrict__ dy, float* __restrict__ part,
     T* __restrict__ mn, T* __restrict__ mx, int64_t N, int64_t F, int64_t HW, int per_block, int slots) {
   constexpr int E = Chunk<T>::kElems;
@@ -712,7 +712,7 @@ template <int E> ACTNN_DEV RowTile row_tile(int64_t C, int tpr, int R) {
 }
 
 template <typename T, bool BWD, bool MINMAX, typename XS>
-__global__ __launch_bounds__(kThreads) void bn_cl_reduce_kernel(
+__global__ __launch_bounds__(kThreads, 5) void bn_cl_reduce_kernel(
     XS xs, const T* __restrict__ dy, float* __restrict__ part, T* __restrict__ mn, T* __restrict__ mx,
     int64_t P, int64_t C, int tpr, int R, int64_t ppb) {
   constexpr int E = Chunk<T>::kElems;
