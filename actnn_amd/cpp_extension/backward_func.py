@@ -173,7 +173,7 @@ def hip_batch_norm_forward_apply(input, workspace, bits=None, mn=None, mx=None):
 
 def hip_batch_norm_pack_applies(input, weight, bias, running_mean, running_var):
     """True when the forward pass can also write the packed copy of its input."""
-    if input.dtype not in (torch.float16, torch.bfloat16):
+    if input.dtype not in (torch.float16, torch.bfloat16, torch.float32):
         return False
     if not hip_batch_norm_minmax_applies(input, weight, bias, running_mean, running_var):
         return False
@@ -207,17 +207,20 @@ def hip_batch_norm_backward(input, grad_output, weight, save_mean, save_invstd, 
 
 def hip_batch_norm_backward_packed_applies(shape, quantized, grad_output, weight, save_mean, save_invstd):
     """True when the batch-norm backward kernels can read the saved input straight from its
-    mixed-precision stream: 16-bit activation with scale/min in its own dtype, whole groups of
-    256, and a gradient laid out like the activation was when it was compressed."""
+    mixed-precision stream: activation with scale/min in its own dtype (or, for an fp32
+    activation, in their compact bf16 storage, ops.py:115-116), whole groups of 256, and a
+    gradient laid out like the activation was when it was compressed."""
     q_input, q_bits, q_scale, q_min = quantized
     dtype = grad_output.dtype
     memory_format = getattr(quantized, "memory_format", None)
     channels_last = memory_format is not None
     geo = _shape_geometry(shape, dtype, channels_last)
-    return (geo is not None and dtype in (torch.float16, torch.bfloat16)
+    compact = (dtype == torch.float32 and q_scale.dtype == torch.bfloat16
+               and not getattr(quantized, "native_bf16", False))
+    return (geo is not None and dtype in (torch.float16, torch.bfloat16, torch.float32)
             and _groups_align(geo[1], geo[2], channels_last) and isinstance(q_bits, torch.Tensor)
             and isinstance(q_input, torch.Tensor) and q_input.is_cuda and q_input.dtype == torch.int32
-            and q_scale.dtype == dtype and q_min.dtype == dtype
+            and (q_scale.dtype == dtype or compact) and q_min.dtype == q_scale.dtype
             and q_scale.is_contiguous() and q_min.is_contiguous()
             and tuple(grad_output.shape) == tuple(shape)
             and grad_output.is_contiguous(memory_format=memory_format or torch.contiguous_format)
@@ -238,6 +241,9 @@ def hip_batch_norm_backward_packed(shape, quantized, grad_output, weight, save_m
     total, prefix = _bits_info(q_bits)
     if q_input.numel() < total * (C * HW // 256) * 8:
         raise RuntimeError("batch_norm_backward_packed: packed stream is too short")
+    if q_scale.dtype != grad_output.dtype:              # fp32 activation, bf16 storage: widened as
+        q_scale = q_scale.to(grad_output.dtype)         # dequantize_activation widens it (ops.py:129-131)
+        q_min = q_min.to(grad_output.dtype)
     ws_bytes = _workspace_bytes(N, C, HW, code, int(channels_last))
     dev = grad_output.device
     entries = _sumsq_entries(N, C, HW, code, int(channels_last)) if sumsq else 0

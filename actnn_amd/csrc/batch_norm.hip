@@ -169,9 +169,14 @@ template <typename T> struct PlainInput {
 // code of element 8j + k is bit j of word k * bits + i).  The 32 lanes that own a group here are
 // the 32 lanes of that layout - lane j holds elements 8j .. 8j+7 - so a half-wave loads the group's
 // words, transposes them (32x32 bits) and every lane finds its 8 codes in its own register.
-// Values are rebuilt exactly as actnn_unpack_mixed rebuilds them.  16-bit types only.
+// Values are rebuilt exactly as actnn_unpack_mixed rebuilds them.
+// fp32: a lane's 16-byte chunk is 4 elements, so the 64 lanes of a wave own a group and lanes 2j and
+// 2j+1 share stream lane j.  Lane l loads word l (up to 64 words at 8 bits), each half of the wave
+// transposes its 32 words, and lane l collects the two 32-bit halves of stream lane l >> 1 from
+// lanes l >> 1 and 32 + (l >> 1) (ds_bpermute) before it takes its four codes out of them.
 template <typename T> struct PackedInput {
   static constexpr bool kRows = false;
+  static constexpr int kLanes = 256 / Chunk<T>::kElems;     // lanes that own a group: 32, or 64 for fp32
   static constexpr int kInFlight = 2;      // the decode needs registers: 2 measured faster than 1 and 4
   const int32_t* words;
   const int32_t* bits;
@@ -179,7 +184,7 @@ template <typename T> struct PackedInput {
   const T* scale;
   const T* mn;
   int64_t G, g;          // groups per sample, this thread's group
-  uint32_t lane32;
+  uint32_t lane32;       // lane within the group's kLanes lanes
   bool active;
   struct Raw { uint32_t lo, hi; float sc, m; int b; };
   // group `grp` of sample n, whose width b and first word (prefix[n] * G * 8) the caller knows
@@ -188,7 +193,7 @@ template <typename T> struct PackedInput {
     if (active) {
       const int32_t* w = words + first_word + grp * b * 8;
       if ((int)lane32 < 8 * b) r.lo = (uint32_t)w[lane32];
-      if ((int)lane32 + 32 < 8 * b) r.hi = (uint32_t)w[lane32 + 32];
+      if (kLanes == 32 && (int)lane32 + 32 < 8 * b) r.hi = (uint32_t)w[lane32 + 32];
       r.sc = Conv<T>::load(scale, n * G + grp);
       r.m = Conv<T>::load(mn, n * G + grp);
     }
@@ -231,16 +236,34 @@ template <typename T> struct PackedInput {
     for (int k = 0; k < 8; ++k) v[k] = dq((uint32_t)(acc >> (k * BITS)) & ((1u << BITS) - 1u));
     return u32x4{Chunk<T>::narrow(v), Chunk<T>::narrow(v + 2), Chunk<T>::narrow(v + 4), Chunk<T>::narrow(v + 6)};
   }
+  ACTNN_DEV u32x4 decode_f32(const Raw& r) const {
+    const uint32_t t = transpose32(r.lo, lane32 & 31u);       // lanes 0..31: words 0..31, lanes 32..63: words 32..63
+    const int j = (int)(lane32 >> 1);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute(j << 2, (int)t);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute((32 + j) << 2, (int)t);
+    const uint64_t acc = (uint64_t)lo | ((uint64_t)hi << 32);  // the 8 codes of stream lane j
+    const uint32_t mine = (uint32_t)(acc >> (4 * r.b * (int)(lane32 & 1u)));   // elements 4 (l & 1) .. + 3
+    const uint32_t mask = (1u << r.b) - 1u;
+    const Dequant<T> dq(r.sc, r.m);
+    u32x4 out;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) out[m] = as_uint(dq((mine >> (m * r.b)) & mask));
+    return out;
+  }
   ACTNN_DEV u32x4 decode(const Raw& r) const {
-    switch (r.b) {                       // uniform over the block: one sample, one width
-      case 1: return decode_bits<1>(r);
-      case 2: return decode_bits<2>(r);
-      case 3: return decode_bits<3>(r);
-      case 4: return decode_bits<4>(r);
-      case 5: return decode_bits<5>(r);
-      case 6: return decode_bits<6>(r);
-      case 7: return decode_bits<7>(r);
-      default: return decode_bits<8>(r);
+    if constexpr (sizeof(T) == 4) {
+      return decode_f32(r);
+    } else {
+      switch (r.b) {                     // uniform over the block: one sample, one width
+        case 1: return decode_bits<1>(r);
+        case 2: return decode_bits<2>(r);
+        case 3: return decode_bits<3>(r);
+        case 4: return decode_bits<4>(r);
+        case 5: return decode_bits<5>(r);
+        case 6: return decode_bits<6>(r);
+        case 7: return decode_bits<7>(r);
+        default: return decode_bits<8>(r);
+      }
     }
   }
 };
@@ -305,11 +328,63 @@ template <typename T> struct ParamQueue {
       Conv<T>::store(static_cast<T*>(ps.scale), gi, sc);
     }
   }
+  // (the lanes that own a group: a half-wave, or the whole wave for fp32)
   ACTNN_DEV void get(int j, float& m, float& sb) const {
-    m = __shfl(mul, j, 32);
-    sb = __shfl(sub, j, 32);
+    constexpr int kLanes = 256 / Chunk<T>::kElems;
+    m = __shfl(mul, j, kLanes);
+    sb = __shfl(sub, j, kLanes);
   }
 };
+
+// fp32: one group spans the wave - lane l holds elements 4l .. 4l+3, i.e. lanes 2j and 2j+1 share
+// stream lane j and octet j.  Two chunks A and B of a lane (two samples, or two rows) are packed
+// together: the even lane evaluates A's Philox call and the odd lane B's (each hands the other the
+// two words it does not use), both quantise their four elements of A and of B, then the even lane
+// collects A's eight codes and the odd lane B's (one exchange), and two interleaved 32x32 bit
+// transposes leave word p of A in lane 2p and of B in lane 2p+1.  The widths of A and B may differ
+// (different samples): everything here takes the width at run time.  Same arithmetic, counters
+// and layout as actnn_pack_mixed, hence the same bits.
+struct ChunkParams {
+  float mul, sub;
+  int b;
+  int32_t* dst;            // first word of the chunk's group in the stream
+  uint64_t octet;          // index of the lane pair's octet
+};
+ACTNN_DEV void pack_chunk_pair_f32(const PackSink& ps, const u32x4& xa, const ChunkParams& A, const u32x4& xb,
+                                   const ChunkParams& B, bool has_b) {
+  const uint32_t l = threadIdx.x & 63u;
+  const bool odd = l & 1u;
+  const uint32_t j = l >> 1;
+  const Philox4 r = philox_at(odd ? B.octet : A.octet, ps.seed, ps.offset);
+  const uint32_t nx = lane_xor<1>(r.x), ny = lane_xor<1>(r.y), nz = lane_xor<1>(r.z), nw = lane_xor<1>(r.w);
+  // even lane: elements 0..3 of both octets (words 0, 1); odd lane: elements 4..7 (words 2, 3)
+  const uint32_t na[2] = {odd ? nz : r.x, odd ? nw : r.y};
+  const uint32_t nb[2] = {odd ? r.z : nx, odd ? r.w : ny};
+  auto codes = [](const u32x4& x, const uint32_t (&n)[2], const ChunkParams& q) -> uint32_t {
+    const float unit = as_float((uint32_t)(127 + 16 - q.b) << 23);          // 2^(32 - b - 16)
+    uint32_t c = 0;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const uint32_t r16 = (n[m >> 1] >> (16 * (m & 1))) & 0xffffu;
+      c |= (RngFixed<float>::word(as_float(x[m]), r16, q.mul, q.sub, unit) >> (32 - q.b)) << (m * q.b);
+    }
+    return c;
+  };
+  const uint32_t ca = codes(xa, na, A), cb = codes(xb, nb, B);
+  // the even lane keeps A and takes the odd lane's A codes (elements 4..7); the odd lane keeps B
+  // and takes the even lane's B codes (elements 0..3)
+  const uint32_t got = lane_xor<1>(odd ? ca : cb);
+  const int b = odd ? B.b : A.b;
+  const uint64_t acc = (uint64_t)(odd ? got : ca) | ((uint64_t)(odd ? cb : got) << (4 * b));
+  int32_t* dst = odd ? B.dst : A.dst;
+  const bool live = !odd || has_b;
+  const uint32_t lo = transpose32_x2((uint32_t)acc, l);
+  if (live && (int)j < 8 * b) __builtin_nontemporal_store((int32_t)lo, dst + j);
+  if (A.b > 4 || B.b > 4) {                                                  // uniform over the wave
+    const uint32_t hi = transpose32_x2((uint32_t)(acc >> 32), l);
+    if (live && (int)j + 32 < 8 * b) __builtin_nontemporal_store((int32_t)hi, dst + 32 + j);
+  }
+}
 
 // Noise words of two octets of this lane whose neighbours (index ^ 1) lane ^ 1 holds: the two lanes
 // share their Philox calls when octet and lane parity agree (they do wherever a block starts on an
@@ -355,7 +430,7 @@ ACTNN_DEV void pack_chunk(const PackSink& ps, const u32x4& ux, const uint32_t (&
 template <typename T> ACTNN_DEV void bind_input(PlainInput<T>& xs, const Place& p) { xs.p += p.elem; }
 template <typename T> ACTNN_DEV void bind_input(PackedInput<T>& xs, const Place& p) {
   xs.g = p.elem >> 8;
-  xs.lane32 = threadIdx.x & 31;
+  xs.lane32 = threadIdx.x & (PackedInput<T>::kLanes - 1);
   xs.active = p.active;
 }
 
@@ -577,7 +652,42 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
 
   const T* pd = BWD ? dy + p.elem : nullptr;
   T* po = out + p.elem;
-  if constexpr (PACK) {
+  if constexpr (PACK && sizeof(T) == 4) {
+    // fp32: 64 samples at a time (the wave's 64 lanes own the group), packed two by two
+    const int lane = threadIdx.x & 63;
+    const int64_t grp = p.elem >> 8;
+    ParamQueue<T> queue;
+    auto params = [&](int64_t n, int jq) {
+      ChunkParams q;
+      queue.get(jq, q.mul, q.sub);
+      q.b = ps.bits[n];
+      q.dst = ps.packed + (int64_t)ps.prefix[n] * ps.G * 8 + grp * q.b * 8;
+      q.octet = (uint64_t)((n * F + p.elem) >> 3);
+      return q;
+    };
+    for (int64_t nb = n0; nb < n1; nb += 64) {
+      const int64_t ne = nb + 64 < n1 ? nb + 64 : n1;
+      {
+        const int64_t nj = nb + lane;
+        const bool live = nj < ne;
+        queue.fill(ps, nj * ps.G + grp, live ? ps.bits[nj] : 1, live);
+      }
+      int64_t n = nb;
+      for (; n + 2 <= ne; n += 2) {
+        const typename XS::Raw rx0 = xs.fetch(n), rx1 = xs.fetch(n + 1);
+        const u32x4 ux0 = xs.decode(rx0), ux1 = xs.decode(rx1);
+        store_out(po + n * F, apply(ux0, ux0));
+        store_out(po + (n + 1) * F, apply(ux1, ux1));
+        pack_chunk_pair_f32(ps, ux0, params(n, (int)(n - nb)), ux1, params(n + 1, (int)(n + 1 - nb)), true);
+      }
+      if (n < ne) {
+        const u32x4 ux = xs.decode(xs.fetch(n));
+        store_out(po + n * F, apply(ux, ux));
+        const ChunkParams q = params(n, (int)(n - nb));
+        pack_chunk_pair_f32(ps, ux, q, ux, q, false);
+      }
+    }
+  } else if constexpr (PACK) {
     // 32 samples at a time: lane j prepares the group's parameters for sample nb + j, then the
     // half-wave packs the samples two by two (the two chunks of a lane and those of lane ^ 1 are
     // neighbouring octets of the same two groups, and whole groups are present or absent together)
@@ -673,7 +783,7 @@ template <typename T> struct PackedRows {
   using Raw = typename PackedInput<T>::Raw;
   ACTNN_DEV void bind(int64_t column, int64_t) {
     col = column;
-    in.lane32 = threadIdx.x & 31;
+    in.lane32 = threadIdx.x & (PackedInput<T>::kLanes - 1);
     in.active = true;
     cur_row0 = -(int64_t)HW - 1;                           // no row is inside: the first fetch looks up
   }
@@ -855,7 +965,47 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
 
   const T* pd = BWD ? dy + t.col : nullptr;
   T* po = out + t.col;
-  if constexpr (PACK) {
+  if constexpr (PACK && sizeof(T) == 4) {
+    // fp32: 64 steps at a time (the wave's 64 lanes own the group), rows packed two by two
+    const int lane = threadIdx.x & 63;
+    ParamQueue<T> queue;
+    auto params = [&](int64_t row, int jq) {
+      locate(row);
+      ChunkParams q;
+      queue.get(jq, q.mul, q.sub);
+      q.b = cur_b;
+      const int64_t flat = row * C + t.col;
+      q.dst = ps.packed + cur_first + ((flat >> 8) - (int64_t)cur_n * ps.G) * q.b * 8;
+      q.octet = (uint64_t)(flat >> 3);
+      return q;
+    };
+    for (int64_t rb = p0 + t.r; rb < p1; rb += (int64_t)64 * R) {
+      {
+        const int64_t rj = rb + (int64_t)lane * R;
+        const bool live = rj < p1;
+        const uint32_t nj = live ? (uint32_t)rj / HW : 0;
+        queue.fill(ps, (rj * C + t.col) >> 8, live ? ps.bits[nj] : 1, live);
+      }
+      int j = 0;
+      for (; j + 2 <= 64 && rb + (int64_t)(j + 1) * R < p1; j += 2) {
+        const int64_t r0 = rb + (int64_t)j * R, r1 = r0 + R;
+        const typename XS::Raw rx0 = xs.fetch(r0), rx1 = xs.fetch(r1);
+        const u32x4 ux0 = xs.decode(rx0), ux1 = xs.decode(rx1);
+        store_out(po + r0 * C, apply(ux0, ux0));
+        store_out(po + r1 * C, apply(ux1, ux1));
+        const ChunkParams qa = params(r0, j);
+        const ChunkParams qb = params(r1, j + 1);
+        pack_chunk_pair_f32(ps, ux0, qa, ux1, qb, true);
+      }
+      if (j < 64 && rb + (int64_t)j * R < p1) {
+        const int64_t r0 = rb + (int64_t)j * R;
+        const u32x4 ux = xs.decode(xs.fetch(r0));
+        store_out(po + r0 * C, apply(ux, ux));
+        const ChunkParams q = params(r0, j);
+        pack_chunk_pair_f32(ps, ux, q, ux, q, false);
+      }
+    }
+  } else if constexpr (PACK) {
     // 32 steps (rows r0, r0 + R, ...) at a time: lane j prepares the parameters of the group the
     // half-wave meets in step j, then the rows are packed two by two so that lane pairs can share
     // their noise
@@ -1076,15 +1226,11 @@ int forward_apply_t(const Plan& pl, const void* x, void* y, const float* ws, con
   const PackSink none{};
   if (pl.channels_last) {
     const PlainRows<T> xs{static_cast<const T*>(x), C};
-    if constexpr (sizeof(T) == 2) {
-      if (sink) { launch_cl_apply<T, false, true>(pl, xs, nullptr, coef, y, C, *sink, s); ACTNN_RETURN_LAUNCH_STATUS(); }
-    }
+    if (sink) { launch_cl_apply<T, false, true>(pl, xs, nullptr, coef, y, C, *sink, s); ACTNN_RETURN_LAUNCH_STATUS(); }
     launch_cl_apply<T, false, false>(pl, xs, nullptr, coef, y, C, none, s);
   } else {
     const PlainInput<T> xs{static_cast<const T*>(x), pl.F};
-    if constexpr (sizeof(T) == 2) {
-      if (sink) { launch_apply<T, false, true>(pl, xs, nullptr, coef, y, N, HW, *sink, s); ACTNN_RETURN_LAUNCH_STATUS(); }
-    }
+    if (sink) { launch_apply<T, false, true>(pl, xs, nullptr, coef, y, N, HW, *sink, s); ACTNN_RETURN_LAUNCH_STATUS(); }
     launch_apply<T, false, false>(pl, xs, nullptr, coef, y, N, HW, none, s);
   }
   ACTNN_RETURN_LAUNCH_STATUS();
@@ -1191,13 +1337,13 @@ extern "C" int actnn_batch_norm_forward_apply(const void* x, void* y, const void
   PackSink sink{bits, prefix, mn, mx, scale, packed, seed, offset, pl.F / 256};
   const bool pack = bits != nullptr;
   if (pack) {
-    if (dtype == ACTNN_F32 || !pl.groups_align || !prefix || !mn || !mx || !scale || !packed) return ACTNN_EINVAL;
+    if (!pl.groups_align || !prefix || !mn || !mx || !scale || !packed) return ACTNN_EINVAL;
     if (channels_last && pl.P > 0x7fffffffLL) return ACTNN_EINVAL;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const float* ws = static_cast<const float*>(workspace);
   switch (dtype) {
-    case ACTNN_F32: return forward_apply_t<float>(pl, x, y, ws, nullptr, N, C, HW, s);
+    case ACTNN_F32: return forward_apply_t<float>(pl, x, y, ws, pack ? &sink : nullptr, N, C, HW, s);
     case ACTNN_F16: return forward_apply_t<__half>(pl, x, y, ws, pack ? &sink : nullptr, N, C, HW, s);
     default: return forward_apply_t<bf16_t>(pl, x, y, ws, pack ? &sink : nullptr, N, C, HW, s);
   }
@@ -1309,7 +1455,7 @@ extern "C" int actnn_batch_norm_backward_packed(const int32_t* packed, const int
                                                 int64_t HW, int dtype, int channels_last,
                                                 void* stream) {
   using namespace actnn;
-  if (dtype != ACTNN_F16 && dtype != ACTNN_BF16) return ACTNN_EDTYPE;
+  if (dtype != ACTNN_F16 && dtype != ACTNN_BF16 && dtype != ACTNN_F32) return ACTNN_EDTYPE;
   Plan pl;
   if (!make_plan(N, C, HW, dtype, channels_last, pl) || !pl.groups_align) return ACTNN_EINVAL;
   if (channels_last && pl.P > 0x7fffffffLL) return ACTNN_EINVAL;
@@ -1321,5 +1467,7 @@ extern "C" int actnn_batch_norm_backward_packed(const int32_t* packed, const int
   float* ws = static_cast<float*>(workspace);
   if (dtype == ACTNN_F16)
     return backward_packed<__half>(pl, packed, bits, prefix, scale, mn, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
+  if (dtype == ACTNN_F32)
+    return backward_packed<float>(pl, packed, bits, prefix, scale, mn, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
   return backward_packed<bf16_t>(pl, packed, bits, prefix, scale, mn, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
 }

@@ -440,6 +440,9 @@ class batch_norm(Function):
                 q_min, q_max = mn.view(N, -1, 1), mx.view(N, -1, 1)
             output, q_input, q_scale = ext_backward_func.hip_batch_norm_forward_apply(
                 input, ws, q_bits, q_min, q_max)
+            if input.dtype == torch.float32:
+                # compact storage of an fp32 activation's scale and minimum (ops.py:115-116)
+                q_scale, q_min = q_scale.to(torch.bfloat16), q_min.to(torch.bfloat16)
             if config.swap:
                 q_input = swap_to_cpu(q_input)
             reserve = None

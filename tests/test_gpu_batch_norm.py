@@ -123,7 +123,7 @@ def test_no_affine_no_running_stats_and_fallback_shapes():
         assert np.allclose(ys.cpu().numpy(), ref, rtol=1e-4, atol=1e-4)
 
 
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("N,C,spatial", [(8, 64, (56, 56)), (16, 256, (7, 7)), (37, 64, (14, 14)),
                                          (9, 32, (4, 2)), (12, 128, (28, 28))])
 def test_backward_from_the_packed_stream_equals_unpack_then_backward(N, C, spatial, dtype):
@@ -149,6 +149,30 @@ def test_backward_from_the_packed_stream_equals_unpack_then_backward(N, C, spati
         assert torch.equal(a, r)
     _check_sumsq(lambda: ext_bf.hip_batch_norm_backward_packed(x.shape, quantized, dy, w, mean, invstd, sumsq=True),
                  lambda: ext_bf.hip_batch_norm_backward(xq, dy, w, mean, invstd, sumsq=True), ref)
+
+
+def test_backward_from_the_packed_stream_fp32_with_compact_scale_storage():
+    """An fp32 activation keeps its scale and minimum as bf16 (ops.py:115-116); the packed backward
+    widens them exactly as dequantize_activation does (ops.py:129-131)."""
+    import actnn_amd.cpp_extension.quantization as ext_q
+    from _util import bits_tensor
+    N, C, spatial = 10, 64, (28, 28)
+    x, w, b, rm, rv, dy = _inputs(N, C, spatial, torch.float32, 23)
+    G = x[0].numel() // 256
+    groups = x.view(N, G, 256)
+    mn, mx = ext_minimax.minimax(groups.view(-1, 256))
+    mn, mx = mn.view(N, G, 1), mx.view(N, G, 1)
+    bits_dev, _ = bits_tensor([1 + (5 * i) % 8 for i in range(N)])
+    packed, scale = ext_q.pack_mixed_precision(groups, mn, mx, bits_dev, True)
+    scale16, mn16 = scale.bfloat16(), mn.bfloat16()
+    _, mean, invstd, _, _ = ext_bf.hip_batch_norm_forward(x, w, b, None, None, 0.1, 1e-5)
+    xq = ext_q.unpack_mixed_precision(packed, bits_dev, scale16.float(), mn16.float(), N, G, 256).view_as(x)
+    ref = ext_bf.hip_batch_norm_backward(xq, dy, w, mean, invstd)
+    quantized = (packed, bits_dev, scale16, mn16)
+    assert ext_bf.hip_batch_norm_backward_packed_applies(x.shape, quantized, dy, w, mean, invstd)
+    got = ext_bf.hip_batch_norm_backward_packed(x.shape, quantized, dy, w, mean, invstd)
+    for a, r in zip(got, ref):
+        assert torch.equal(a, r)
 
 
 def _check_sumsq(*args):
@@ -222,7 +246,7 @@ def test_channels_last_group_min_max(N, C, spatial, dtype):
     assert torch.equal(y, y0) and torch.equal(m, m0) and torch.equal(i, i0)
 
 
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("N,C,spatial", [(8, 64, (56, 56)), (16, 256, (7, 7)), (37, 128, (14, 14)),
                                          (9, 32, (4, 2)), (5, 1024, (6, 6))])
 def test_channels_last_backward_from_the_packed_stream(N, C, spatial, dtype):
@@ -255,9 +279,9 @@ def test_channels_last_backward_from_the_packed_stream(N, C, spatial, dtype):
 
 
 @pytest.mark.parametrize("channels_last", [False, True])
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("N,C,spatial", [(8, 64, (56, 56)), (16, 256, (7, 7)), (37, 128, (14, 14)),
-                                         (9, 32, (4, 2)), (5, 1024, (6, 6))])
+                                         (9, 32, (4, 2)), (5, 1024, (6, 6)), (70, 64, (8, 8))])
 def test_forward_with_packed_copy_equals_forward_then_pack(N, C, spatial, dtype, channels_last):
     """The normalising pass that also packs its input: output equal to the plain forward pass,
     stream and scales equal to pack_mixed_precision with the same generator state (every width)."""
