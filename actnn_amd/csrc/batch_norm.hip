@@ -1218,7 +1218,7 @@ int forward_stats_t(const Plan& pl, const void* x, const float* weight, const fl
 }
 
 // y = a*x + b from the coefficients the statistics step left in the workspace; with a sink the
-// same pass also writes the packed copy of x (16-bit types).
+// same pass also writes the packed copy of x.
 template <typename T>
 int forward_apply_t(const Plan& pl, const void* x, void* y, const float* ws, const PackSink* sink, int64_t N,
                     int64_t C, int64_t HW, hipStream_t s) {

@@ -280,7 +280,7 @@ int actnn_batch_norm_forward_static(const void* x, const float* weight, const fl
  * of x: _stats runs the statistics pass (save_mean/save_invstd, running estimates, optional group
  * min/max) and leaves the per-channel coefficients in `workspace`; the caller may then derive the
  * per-sample bit widths from mn/mx; _apply writes y from x and the same workspace and, when `bits`
- * is given (16-bit dtypes, the alignment conditions of mn/mx), also scale[N*G] and the packed
+ * is given (any dtype, the alignment conditions of mn/mx), also scale[N*G] and the packed
  * stream - bit for bit what actnn_pack_mixed(x, mn, mx, bits, prefix, ..., seed, offset) writes in
  * its in-kernel Philox mode.  actnn_batch_norm_forward is _stats followed by _apply without bits. */
 int actnn_batch_norm_forward_stats(const void* x, const float* weight, const float* bias,
@@ -296,7 +296,8 @@ int actnn_batch_norm_forward_apply(const void* x, void* y, const void* workspace
                                    int64_t C, int64_t HW, int dtype, int channels_last, void* stream);
 
 /* The same backward pass with x held as the mixed-precision stream of actnn_pack_mixed (group
- * size 256 over the sample in memory order, the conditions of mn/mx above, 16-bit dtype; bits / prefix / scale / mn as for actnn_unpack_mixed):
+ * size 256 over the sample in memory order, the conditions of mn/mx above, any dtype with scale / mn
+ * in that dtype; bits / prefix / scale / mn as for actnn_unpack_mixed):
  * both passes rebuild x in registers, bit for bit what actnn_unpack_mixed would write, so the
  * full-precision copy of x that ops.py:478 (dequantize_activation before
  * cudnn_batch_norm_backward) materialises never exists. */
