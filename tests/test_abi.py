@@ -42,7 +42,7 @@ def test_argument_errors_need_no_gpu(lib):
     assert lib.actnn_batch_norm_forward(None, None, None, None, None, None, None, None, None, None, None, 0,
                                         8, 64, 3136, 0.1, 1e-5, 2, 0, None) == -1   # null pointers
     assert lib.actnn_batch_norm_backward_packed(None, None, None, None, None, None, None, None, None, None, None,
-                                                None, None, 0, None, 0, 8, 64, 3136, 0, 0, None) == -2   # f32 not supported
+                                                None, None, 0, None, 0, 8, 64, 3136, 7, 0, None) == -2   # unknown dtype code
     assert lib.actnn_batch_norm_backward_sumsq_entries(8, 64, 3136, 2, 0) > 0
     assert lib.actnn_batch_norm_backward_sumsq_entries(4, 3, 49, 2, 0) == -1
     assert lib.actnn_sample_sqnorm(None, None, 4, 30, 1, 2, None) == -1           # F % 8 != 0
