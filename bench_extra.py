@@ -100,13 +100,16 @@ def batch_norm_shapes(device, channels_last=True, batch=512, reps=10):
         for _ in range(3):
             fn()
         torch.cuda.synchronize(device)
-        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
-        for _ in range(reps):
+        # every repetition is timed on its own and the median taken: a one-off stall of a few
+        # milliseconds (the caching allocator growing, a clock change) would otherwise end up in
+        # the figure of whichever shape it happened to hit
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+        marks[0].record()
+        for i in range(reps):
             fn()
-        stop.record()
+            marks[i + 1].record()
         torch.cuda.synchronize(device)
-        return start.elapsed_time(stop) / reps
+        return sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(reps))[reps // 2]
 
     rows, totals = [], [0.0, 0.0, 0.0]
     for C, H, count in RESNET50_BN_SHAPES:
