@@ -83,6 +83,8 @@ ACTNN_DEV void stage_out_f32(float* __restrict__ out, int64_t elem_base, int gro
 
 template <typename T> struct IsF32 { static constexpr bool value = false; };
 template <> struct IsF32<float> { static constexpr bool value = true; };
+template <typename T> struct IsBf16 { static constexpr bool value = false; };
+template <> struct IsBf16<bf16_t> { static constexpr bool value = true; };
 
 // ---------------------------------------------------------------------------- pack (gs = 256)
 // Issue the loads of this lane's elements (and noise in deterministic mode) for its GPH groups.
@@ -302,6 +304,31 @@ ACTNN_DEV void unpack_groups(const int32_t* __restrict__ packed, T* __restrict__
       const int gl = TL::group_of(hw, q0 + r);
       if (gl < groups_valid) {
         const Dequant<T> dq(s_scale[gl], s_min[gl]);
+        if constexpr (sizeof(T) == 2 && BITS <= 2) {
+          // A group at 1 or 2 bits has at most four distinct values.  Lane l evaluates level l & 3
+          // (once instead of once per element), the four lanes of a quad exchange them (DPP
+          // quad_perm broadcasts) into an 8-byte table, and every pair of elements is one byte
+          // permute of that table.  Same arithmetic per level, hence the same bits.
+          const float mine = dq(lane & 3u);
+          const int h = (int)(sizeof(T) == 2 && IsBf16<T>::value ? float_to_bf16_bits(mine) : float_to_half_bits(mine));
+          const uint32_t l0 = (uint32_t)__builtin_amdgcn_update_dpp(0, h, 0x00, 0xF, 0xF, true);   // quad_perm [0,0,0,0]
+          const uint32_t l1 = (uint32_t)__builtin_amdgcn_update_dpp(0, h, 0x55, 0xF, 0xF, true);   // [1,1,1,1]
+          const uint32_t l2 = (uint32_t)__builtin_amdgcn_update_dpp(0, h, 0xAA, 0xF, 0xF, true);   // [2,2,2,2]
+          const uint32_t l3 = (uint32_t)__builtin_amdgcn_update_dpp(0, h, 0xFF, 0xF, 0xF, true);   // [3,3,3,3]
+          const uint32_t lut_lo = l0 | (l1 << 16), lut_hi = l2 | (l3 << 16);
+          const uint32_t a = (uint32_t)(acc >> (r * WPG));
+          u32x4 outw;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const uint32_t c0 = (a >> (2 * j * BITS)) & kMask;
+            const uint32_t c1 = (a >> ((2 * j + 1) * BITS)) & kMask;
+            // bytes 2c, 2c+1 of the table for each of the two elements
+            const uint32_t sel = (c0 * 0x0202u + 0x0100u) | ((c1 * 0x0202u + 0x0100u) << 16);
+            outw[j] = __builtin_amdgcn_perm(lut_hi, lut_lo, sel);
+          }
+          store16_nt(out + elem_base + (int64_t)gl * kGs + lane * 8, outw);
+          continue;
+        }
         float v[8];
 #pragma unroll
         for (int k = 0; k < 8; ++k) v[k] = dq((uint32_t)(acc >> (r * WPG + k * BITS)) & kMask);
