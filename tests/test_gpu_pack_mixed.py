@@ -157,7 +157,13 @@ def test_rng_mode_mean_code_of_16bit_tensors(dtype, bits):
     sigma = np.sqrt(kernel_mode.code_variance(base, mn[:1].cpu(), scale[:1].cpu(), bits)[0] / trials)
     assert (np.abs(mean - expect) <= 5 * sigma + 1e-9).all()
     exact = (base.double() - mn[:1].double().cpu()).numpy()[0] * scale[0].double().cpu().numpy()
-    assert (np.abs(expect - np.minimum(exact, 2 ** bits - 1)) <= 2.0 ** -9 + 2.0 ** -12).all()
+    exact = np.minimum(exact, 2 ** bits - 1)
+    assert (np.abs(expect - exact) <= 2.0 ** -9 + 2.0 ** -12).all()
+    # the criterion of the RNG mode - mean error below 1e-3 of the range - per group, measured and
+    # in expectation (one level is 1 / (2^bits - 1) of the range)
+    B = 2 ** bits - 1
+    assert (np.abs((mean - exact).mean(axis=1)) / B < 1e-3).all()
+    assert (np.abs((expect - exact).mean(axis=1)) / B < 2e-4).all()
 
 
 def test_streams_of_different_calls_differ():
