@@ -9,14 +9,7 @@
 // (delta, index, earlier step first).  Every block builds the keys of all candidates with the
 // reference's arithmetic (delta evaluated in double, narrowed to float) - each thread a 256th of
 // them, in registers - and ranks the steps of a few items by counting the keys above each of
-// them, so the whole allocation is one launch of independent blocks: no sort.
-//
-// When the caller also wants the prefix sum of the widths (where each sample's words start in the
-// stream), the block that finishes last computes it: every block publishes its widths (fence), then
-// takes a ticket from a counter in device memory; the block that draws the last ticket knows all
-// widths are written, scans them, and puts the counter back to zero for the next launch.  Nobody
-// waits for anybody.  The counter is one word per GPU inside this library: launches that overlap in
-// time on one GPU (different streams) would share it, launches on one stream are ordered.
+// them, so the whole allocation is one launch of independent blocks: no sort, no atomics.
 #include "device_utils.h"
 
 namespace actnn {
@@ -40,50 +33,8 @@ __global__ __launch_bounds__(kThreads) void fill_kernel(int32_t* __restrict__ ou
   if (i < n) out[i] = value;
 }
 
-__device__ unsigned int g_ticket = 0;
-
-// prefix[0] = 0, prefix[i + 1] = bits[0] + ... + bits[i], by one block; the widths were written by
-// other blocks, so they are read past this CU's cache.
-ACTNN_DEV void block_prefix(const int32_t* bits, int32_t* __restrict__ prefix, int N) {
-  __shared__ int32_t s_part[kThreads];
-  const int per = (N + kThreads - 1) / kThreads;
-  const int lo = (int)threadIdx.x * per;
-  const int hi = lo + per < N ? lo + per : N;
-  int32_t sum = 0;
-  for (int i = lo; i < hi; ++i) sum += __hip_atomic_load(bits + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  s_part[threadIdx.x] = sum;
-  __syncthreads();
-  for (int off = 1; off < kThreads; off <<= 1) {         // inclusive Hillis-Steele scan
-    const int32_t add = (int)threadIdx.x >= off ? s_part[threadIdx.x - off] : 0;
-    __syncthreads();
-    s_part[threadIdx.x] += add;
-    __syncthreads();
-  }
-  int32_t run = threadIdx.x == 0 ? 0 : s_part[threadIdx.x - 1];
-  if (threadIdx.x == 0) prefix[0] = 0;
-  for (int i = lo; i < hi; ++i) {
-    run += __hip_atomic_load(bits + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    prefix[i + 1] = run;
-  }
-}
-
-// Called by every thread of every block after the block's widths are stored: the last block to
-// arrive computes the prefix sum.
-ACTNN_DEV void finish_with_prefix(const int32_t* bits, int32_t* __restrict__ prefix, int N) {
-  __shared__ bool s_last;
-  __threadfence();                                       // this block's widths are visible device-wide
-  __syncthreads();
-  if (threadIdx.x == 0) s_last = atomicAdd(&g_ticket, 1u) == gridDim.x - 1;
-  __syncthreads();
-  if (!s_last) return;
-  __threadfence();
-  block_prefix(bits, prefix, N);
-  if (threadIdx.x == 0) atomicExch(&g_ticket, 0u);
-}
-
-template <bool PREFIX>
 __global__ __launch_bounds__(kThreads) void calc_precision_device_kernel(
-    const float* __restrict__ C, int32_t* bits, int32_t* __restrict__ prefix, int N, int initial, int64_t K) {
+    const float* __restrict__ C, int32_t* __restrict__ bits, int N, int initial, int64_t K) {
   constexpr int kWaves = kThreads / 64;
   __shared__ double factors[8];
   __shared__ float C_s[kMaxCand];                      // N <= kMaxCand / L
@@ -98,7 +49,6 @@ __global__ __launch_bounds__(kThreads) void calc_precision_device_kernel(
   if (K <= 0 || K >= total) {                          // nothing to take, or everything
     if ((int)threadIdx.x < items_per_block && item0 + (int)threadIdx.x < N)
       bits[item0 + threadIdx.x] = K <= 0 ? initial : 1;
-    if constexpr (PREFIX) finish_with_prefix(bits, prefix, N);
     return;
   }
   for (int n = threadIdx.x; n < N; n += kThreads) C_s[n] = C[n];      // one trip to memory for all keys
@@ -161,41 +111,28 @@ __global__ __launch_bounds__(kThreads) void calc_precision_device_kernel(
     for (int k = 0; k < L; ++k) t += taken[threadIdx.x * L + k];
     bits[item0 + threadIdx.x] = initial - t;
   }
-  if constexpr (PREFIX) finish_with_prefix(bits, prefix, N);
 }
 
 }  // namespace
+}  // namespace actnn
 
-// bits as actnn_calc_precision_device; with `prefix` (N + 1 entries) the same launch also leaves
-// the exclusive prefix sum of the widths.  -> ACTNN_OK, an error code, or 1 when the widths are
-// written but the prefix is left to the caller (the one-bit case, which launches no ranking kernel).
-int calc_precision_device_launch(const float* C, int32_t* bits, int32_t* prefix, int64_t N, int initial_bits,
-                                 int64_t target, hipStream_t s) {
+extern "C" int actnn_calc_precision_device(const float* C, int32_t* bits, int64_t N, int initial_bits,
+                                           int64_t target, void* stream) {
+  using namespace actnn;
   if (N < 0) return ACTNN_EINVAL;
-  if (N == 0) return prefix ? 1 : ACTNN_OK;
+  if (N == 0) return ACTNN_OK;
   if (!C || !bits) return ACTNN_EINVAL;
   if (initial_bits < 1 || initial_bits > 8) return ACTNN_EBITS;
   const int64_t total = N * (initial_bits - 1);
   if (total > kMaxCand) return ACTNN_EINVAL;           // larger batches take the host routine
   const int64_t K = N * initial_bits - target;         // widths to take away
+  hipStream_t s = static_cast<hipStream_t>(stream);
   if (initial_bits == 1) {                             // no steps to take: every item keeps its one bit
     fill_kernel<<<dim3((unsigned)((N + kThreads - 1) / kThreads)), dim3(kThreads), 0, s>>>(bits, (int)N, 1);
-    hipError_t e = hipGetLastError();
-    return e == hipSuccess ? (prefix ? 1 : ACTNN_OK) : (int)e;
+    ACTNN_RETURN_LAUNCH_STATUS();
   }
   const int items_per_block = kSlots / (initial_bits - 1);
   const int64_t blocks = (N + items_per_block - 1) / items_per_block;
-  if (prefix)
-    calc_precision_device_kernel<true><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(C, bits, prefix, (int)N, initial_bits, K);
-  else
-    calc_precision_device_kernel<false><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(C, bits, nullptr, (int)N, initial_bits, K);
+  calc_precision_device_kernel<<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(C, bits, (int)N, initial_bits, K);
   ACTNN_RETURN_LAUNCH_STATUS();
-}
-
-}  // namespace actnn
-
-extern "C" int actnn_calc_precision_device(const float* C, int32_t* bits, int64_t N, int initial_bits,
-                                           int64_t target, void* stream) {
-  return actnn::calc_precision_device_launch(C, bits, nullptr, N, initial_bits, target,
-                                             static_cast<hipStream_t>(stream));
 }

@@ -42,10 +42,6 @@ extern "C" int actnn_range_sqr(const void* mn, const void* mx, float* out, int64
 extern "C" int actnn_calc_precision_device(const float* C, int32_t* bits, int64_t N, int initial_bits,
                                            int64_t target, void* stream);
 extern "C" int actnn_bits_prefix(const int32_t* bits, int32_t* prefix, int64_t N, void* stream);
-namespace actnn {
-int calc_precision_device_launch(const float* C, int32_t* bits, int32_t* prefix, int64_t N, int initial_bits,
-                                 int64_t target, hipStream_t s);
-}
 
 extern "C" int actnn_allocate_bits_device(const void* mn, const void* mx, float factor, const float* mult,
                                           int mult_per_sample, float* sensitivity, int32_t* bits,
@@ -53,10 +49,8 @@ extern "C" int actnn_allocate_bits_device(const void* mn, const void* mx, float 
                                           int64_t target, int dtype, void* stream) {
   int rc = actnn_range_sqr(mn, mx, sensitivity, N, G, factor, mult, mult_per_sample, dtype, stream);
   if (rc != ACTNN_OK) return rc;
-  // the ranking kernel's last block also writes the prefix sum (1: left to a launch of its own)
-  rc = actnn::calc_precision_device_launch(sensitivity, bits, prefix, N, initial_bits, target,
-                                           static_cast<hipStream_t>(stream));
-  if (rc != 1) return rc;
+  rc = actnn_calc_precision_device(sensitivity, bits, N, initial_bits, target, stream);
+  if (rc != ACTNN_OK) return rc;
   return actnn_bits_prefix(bits, prefix, N, stream);
 }
 
