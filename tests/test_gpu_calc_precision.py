@@ -77,3 +77,9 @@ def test_allocation_in_one_call_equals_the_three_calls(N, G, dtype):
         assert torch.equal(sens, sens_ref) and torch.equal(bits, bits_ref)
         assert torch.equal(prefix, _bits_info(bits_ref)[1])
         assert int(prefix[-1]) == int(bits.sum()) == 2 * N
+    # also where the ranking takes nothing (every width stays 8), everything (every width 1), or
+    # does not run at all (start width 1)
+    for initial, target in ((8, 8 * N), (8, N), (1, N), (4, 3 * N)):
+        sens, bits, prefix = ext_cp.allocate_bits_device(mn, mx, N, 0.37, None, initial, target)
+        assert int(bits.sum()) == target and int(bits.min()) >= 1 and int(bits.max()) <= initial
+        assert torch.equal(prefix[1:], torch.cumsum(bits, 0).to(torch.int32)) and int(prefix[0]) == 0
