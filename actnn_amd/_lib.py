@@ -52,6 +52,14 @@ SIGNATURES = {
                                     c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
     "actnn_max_pool2d_backward_cl": [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
                                      c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
+    "actnn_max_pool2d_forward_nibble": [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
+                                        c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
+    "actnn_max_pool2d_backward_nibble": [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
+                                         c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
+    "actnn_max_pool2d_forward_cl_nibble": [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
+                                           c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
+    "actnn_max_pool2d_backward_cl_nibble": [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
+                                            c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
     "actnn_calc_precision": [c_vp, c_vp, c_vp, c_i64, ctypes.c_double],
     "actnn_linear_grad_weight": [c_vp, c_vp, c_vp, c_vp, c_i32, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64,
                                  c_i32, c_i32, c_i32, c_vp],

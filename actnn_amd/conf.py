@@ -33,6 +33,7 @@ class QuantizationConfig:
         self.share_grad_sqnorm = True                  # batch-norm backward leaves sum(dx^2) for the conv's set_scale
         self.fused_bn_pack = True                      # batch-norm forward writes the packed copy of its input
         self.fused_linear_grad_weight = True           # QLinear's weight gradient straight from the packed input
+        self.pool_index_nibbles = True                 # max-pool keeps its arg-max indices two per byte
         # memory management (conf.py:54-58)
         self.empty_cache_threshold = None
         self.pipeline_threshold = None

@@ -400,8 +400,10 @@ def pool_takes_channels_last(x):
             and x.data_ptr() % 16 == 0)
 
 
-def max_pool2d_forward(x, kernel_size, stride, padding, dilation):
-    """-> (y, idx) in the memory format of x (default or channels-last)."""
+def max_pool2d_forward(x, kernel_size, stride, padding, dilation, nibble_indices=False):
+    """-> (y, idx) in the memory format of x (default or channels-last).  idx: int8 of y's shape as in
+    the reference, or with nibble_indices a flat uint8 tensor holding two indices per byte
+    ((y.numel() + 1) // 2 bytes, in the order of y's memory)."""
     N, C, H, W = x.shape
     KH, KW = kernel_size
     Ho = (H + 2 * padding[0] - dilation[0] * (KH - 1) - 1) // stride[0] + 1       # .cu:679
@@ -411,8 +413,12 @@ def max_pool2d_forward(x, kernel_size, stride, padding, dilation):
     if not channels_last:
         x = x.contiguous()
     y = torch.empty((N, C, Ho, Wo), dtype=x.dtype, device=x.device, memory_format=fmt)
-    idx = torch.empty((N, C, Ho, Wo), dtype=torch.int8, device=x.device, memory_format=fmt)
-    fn = g.lib().actnn_max_pool2d_forward_cl if channels_last else g.lib().actnn_max_pool2d_forward
+    if nibble_indices:
+        idx = torch.empty(((N * C * Ho * Wo + 1) // 2,), dtype=torch.uint8, device=x.device)
+        fn = g.lib().actnn_max_pool2d_forward_cl_nibble if channels_last else g.lib().actnn_max_pool2d_forward_nibble
+    else:
+        idx = torch.empty((N, C, Ho, Wo), dtype=torch.int8, device=x.device, memory_format=fmt)
+        fn = g.lib().actnn_max_pool2d_forward_cl if channels_last else g.lib().actnn_max_pool2d_forward
     with g.on_device(x.device):
         check(fn(
             x.data_ptr(), y.data_ptr(), idx.data_ptr(), N, C, H, W, Ho, Wo, KH, KW, stride[0],
@@ -421,15 +427,27 @@ def max_pool2d_forward(x, kernel_size, stride, padding, dilation):
     return y, idx
 
 
-def max_pool2d_backward(grad_output, idx, input_shape, kernel_size, stride, padding):
-    """The gradient comes back in the memory format of `idx` (the format of the forward input)."""
-    channels_last = channels_last_format(idx) is not None
+def max_pool2d_backward(grad_output, idx, input_shape, kernel_size, stride, padding, channels_last=None):
+    """The gradient comes back in the memory format of `idx` (the format of the forward input).
+    A uint8 `idx` is the two-per-byte format, which carries no layout of its own: `channels_last`
+    says which kernels wrote it (default: whatever layout grad_output has)."""
+    nibble_indices = idx.dtype == torch.uint8
+    if nibble_indices:
+        if channels_last is None:
+            channels_last = pool_takes_channels_last(grad_output)
+    else:
+        channels_last = channels_last_format(idx) is not None
     fmt = torch.channels_last if channels_last else torch.contiguous_format
     grad_output = grad_output.contiguous(memory_format=fmt)
     N, C, H, W = input_shape
     Ho, Wo = grad_output.shape[2], grad_output.shape[3]
     gin = torch.empty((N, C, H, W), dtype=grad_output.dtype, device=grad_output.device, memory_format=fmt)
-    fn = g.lib().actnn_max_pool2d_backward_cl if channels_last else g.lib().actnn_max_pool2d_backward
+    if nibble_indices:
+        if idx.numel() != (grad_output.numel() + 1) // 2:
+            raise RuntimeError("max_pool2d_backward: the index tensor does not match grad_output")
+        fn = g.lib().actnn_max_pool2d_backward_cl_nibble if channels_last else g.lib().actnn_max_pool2d_backward_nibble
+    else:
+        fn = g.lib().actnn_max_pool2d_backward_cl if channels_last else g.lib().actnn_max_pool2d_backward
     with g.on_device(gin.device):
         check(fn(
             grad_output.data_ptr(), idx.data_ptr(), gin.data_ptr(), N, C, H, W, Ho, Wo,
@@ -442,7 +460,8 @@ class ActQuantizedMaxPool2d(Function):
     """quantization.cc:152-191."""
 
     @staticmethod
-    def forward(ctx, input, kernel_size, stride, padding, dilation, ceil_mode, return_indices):
+    def forward(ctx, input, kernel_size, stride, padding, dilation, ceil_mode, return_indices,
+                nibble_indices=False):
         kernel_size = _pair_check(kernel_size, "kernel_size")
         stride = _pair_check(stride, "stride")
         padding = _pair_check(padding, "padding")
@@ -455,21 +474,24 @@ class ActQuantizedMaxPool2d(Function):
             raise RuntimeError("kernel_size[0] * kernel_size[1] must be < 16")    # quantization.cc:162
         if input.dim() != 4:
             raise RuntimeError("The dimension of input is not correct!")
-        output, idx = max_pool2d_forward(input, kernel_size, stride, padding, dilation)
+        output, idx = max_pool2d_forward(input, kernel_size, stride, padding, dilation, nibble_indices)
         ctx.save_for_backward(idx)
-        ctx.geom = (tuple(input.shape), kernel_size, stride, padding)
+        ctx.geom = (tuple(input.shape), kernel_size, stride, padding, pool_takes_channels_last(input))
         return output
 
     @staticmethod
     def backward(ctx, grad_output):
         (idx,) = ctx.saved_tensors
-        shape, kernel_size, stride, padding = ctx.geom
-        gin = max_pool2d_backward(grad_output, idx, shape, kernel_size, stride, padding)
-        return gin, None, None, None, None, None, None
+        shape, kernel_size, stride, padding, channels_last = ctx.geom
+        gin = max_pool2d_backward(grad_output, idx, shape, kernel_size, stride, padding, channels_last)
+        return gin, None, None, None, None, None, None, None
 
 
-def act_quantized_max_pool2d(input, kernel_size, stride, padding, dilation, ceil_mode, return_indices):
+def act_quantized_max_pool2d(input, kernel_size, stride, padding, dilation, ceil_mode, return_indices,
+                             nibble_indices=False):
+    """The reference's operator (quantization.cc:193-196); nibble_indices keeps the saved indices two
+    per byte instead of one int8 each."""
     if not (isinstance(input, torch.Tensor) and input.is_cuda and input.dim() == 4 and pool_takes_channels_last(input)):
         g.check_float(input, "input")                                              # quantization.cc:194
     return ActQuantizedMaxPool2d.apply(input, kernel_size, stride, padding, dilation, ceil_mode,
-                                       return_indices)
+                                       return_indices, nibble_indices)

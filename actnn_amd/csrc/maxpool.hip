@@ -1,5 +1,9 @@
 // MaxPool2d with int8 arg-max-in-window indices (replaces quantization_cuda_kernel.cu:630-754).
 //
+// Index storage: one int8 per output element as in the reference, or (template parameter NIB of
+// every kernel, the *_nibble entry points) two outputs per byte - an index is below 16 - with
+// output o of the flat output order in bits 4 * (o & 1) .. of byte o >> 1.
+//
 // Forward: every output element scans its clipped window in row-major order and keeps the first
 // strict maximum (index relative to the unclipped window origin).
 // Backward: a gather - every input element sums, in a fixed order, the grad_output of the
@@ -26,37 +30,75 @@ struct PoolGeom {
   int H, W, Ho, Wo, KH, KW, SH, SW, PH, PW;
 };
 
-template <typename T>
+// index of output o
+template <bool NIB> ACTNN_DEV int read_index(const int8_t* __restrict__ idx, int64_t o) {
+  if (NIB) return ((int)(uint8_t)idx[o >> 1] >> (4 * (int)(o & 1))) & 15;
+  return (int)idx[o];
+}
+// the same from a staged copy: i counts outputs from the first staged one, whose byte is s[0]
+// and whose parity is folded into i by the caller
+template <bool NIB> ACTNN_DEV int staged_index(const int8_t* s, int i) {
+  if (NIB) return ((int)(uint8_t)s[i >> 1] >> (4 * (i & 1))) & 15;
+  return (int)s[i];
+}
+// E (4 or 8) indices of outputs o .. o + E - 1 (o a multiple of E) as fields of kBits bits of one
+// integer, field e = output o + e: what the kernels that own several adjacent outputs store and load
+template <bool NIB> struct IndexFields {
+  static constexpr int kBits = NIB ? 4 : 8;
+  static constexpr uint32_t kMask = NIB ? 0xfu : 0xffu;
+  static ACTNN_DEV int get(uint64_t fields, int e) { return (int)((uint32_t)(fields >> (kBits * e)) & kMask); }
+  template <int E, typename P> static ACTNN_DEV void store(P* idx, int64_t o, uint64_t fields) {
+    P* at = idx + (NIB ? o >> 1 : o);
+    if constexpr (E * kBits == 16) *reinterpret_cast<uint16_t*>(at) = (uint16_t)fields;
+    else if constexpr (E * kBits == 32) *reinterpret_cast<uint32_t*>(at) = (uint32_t)fields;
+    else *reinterpret_cast<uint64_t*>(at) = fields;
+  }
+  template <int E, typename P> static ACTNN_DEV uint64_t load(const P* idx, int64_t o) {
+    const P* at = idx + (NIB ? o >> 1 : o);
+    if constexpr (E * kBits == 16) return *reinterpret_cast<const uint16_t*>(at);
+    else if constexpr (E * kBits == 32) return *reinterpret_cast<const uint32_t*>(at);
+    else return *reinterpret_cast<const uint64_t*>(at);
+  }
+};
+
+template <typename T, bool NIB>
 __global__ __launch_bounds__(kThreads) void max_pool2d_forward_kernel(const T* __restrict__ x,
                                                                       T* __restrict__ y,
                                                                       int8_t* __restrict__ idx,
                                                                       int64_t total, PoolGeom g) {
   const int64_t id = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-  if (id >= total) return;
-  const int w = (int)(id % g.Wo);
-  const int h = (int)((id / g.Wo) % g.Ho);
-  const int64_t nc = id / ((int64_t)g.Wo * g.Ho);
-  const int h_base = h * g.SH - g.PH, w_base = w * g.SW - g.PW;
-  const int h_start = h_base > 0 ? h_base : 0, h_end = h_base + g.KH < g.H ? h_base + g.KH : g.H;
-  const int w_start = w_base > 0 ? w_base : 0, w_end = w_base + g.KW < g.W ? w_base + g.KW : g.W;
-  // the reference starts from -1e10 narrowed to the element type (-inf for f16), .cu:656
-  float v = Conv<T>::round(-1e10f);
+  const bool live = id < total;
   int index = 0;
-  const T* plane = x + nc * (int64_t)g.H * g.W;
-  for (int i = h_start; i < h_end; ++i) {
-    for (int j = w_start; j < w_end; ++j) {
-      const float c = Conv<T>::load(plane, (int64_t)i * g.W + j);
-      if (c > v) {
-        v = c;
-        index = (i - h_base) * g.KW + (j - w_base);
+  if (live) {
+    const int w = (int)(id % g.Wo);
+    const int h = (int)((id / g.Wo) % g.Ho);
+    const int64_t nc = id / ((int64_t)g.Wo * g.Ho);
+    const int h_base = h * g.SH - g.PH, w_base = w * g.SW - g.PW;
+    const int h_start = h_base > 0 ? h_base : 0, h_end = h_base + g.KH < g.H ? h_base + g.KH : g.H;
+    const int w_start = w_base > 0 ? w_base : 0, w_end = w_base + g.KW < g.W ? w_base + g.KW : g.W;
+    // the reference starts from -1e10 narrowed to the element type (-inf for f16), .cu:656
+    float v = Conv<T>::round(-1e10f);
+    const T* plane = x + nc * (int64_t)g.H * g.W;
+    for (int i = h_start; i < h_end; ++i) {
+      for (int j = w_start; j < w_end; ++j) {
+        const float c = Conv<T>::load(plane, (int64_t)i * g.W + j);
+        if (c > v) {
+          v = c;
+          index = (i - h_base) * g.KW + (j - w_base);
+        }
       }
     }
+    Conv<T>::store(y, id, v);
+    if (!NIB) idx[id] = (int8_t)index;
   }
-  Conv<T>::store(y, id, v);
-  idx[id] = (int8_t)index;
+  if (NIB) {
+    // the even thread writes the byte of outputs id and id + 1 (0 for an output past the end)
+    const int next = lane_xor<1>(index);
+    if (live && !(id & 1)) idx[id >> 1] = (int8_t)(index | (next << 4));
+  }
 }
 
-template <typename T>
+template <typename T, bool NIB>
 __global__ __launch_bounds__(kThreads) void max_pool2d_backward_kernel(const T* __restrict__ gout,
                                                                        const int8_t* __restrict__ idx,
                                                                        T* __restrict__ gin,
@@ -82,7 +124,7 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_backward_kernel(const T* 
     for (int wo = wo_lo; wo <= wo_hi; ++wo) {
       const int kw = w - (wo * g.SW - g.PW);
       const int64_t o = obase + (int64_t)ho * g.Wo + wo;
-      if ((int)idx[o] == kh * g.KW + kw) acc += Conv<T>::load(gout, o);
+      if (read_index<NIB>(idx, o) == kh * g.KW + kw) acc += Conv<T>::load(gout, o);
     }
   }
   Conv<T>::store(gin, id, acc);
@@ -156,7 +198,7 @@ inline int preset_of(const PoolGeom& g) {
   return 0;
 }
 
-template <typename T, int PRESET>
+template <typename T, int PRESET, bool NIB>      // NIB: Wo even, so the two outputs of a byte sit in one row
 __global__ __launch_bounds__(kThreads) void max_pool2d_forward_lds_kernel(
     const T* __restrict__ x, T* __restrict__ y, int8_t* __restrict__ idx, int64_t total_in,
     PoolGeom g, int rows_per_band, int bands) {
@@ -198,12 +240,17 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_forward_lds_kernel(
         }
       }
       Conv<T>::store(y, orow + wo, v);
-      idx[orow + wo] = (int8_t)index;
+      if (NIB) {
+        const int next = lane_xor<1>(index);           // lane and wo have the same parity
+        if (!(wo & 1)) idx[(orow + wo) >> 1] = (int8_t)(index | (next << 4));
+      } else {
+        idx[orow + wo] = (int8_t)index;
+      }
     }
   }
 }
 
-template <typename T, int PRESET>
+template <typename T, int PRESET, bool NIB>
 __global__ __launch_bounds__(kThreads) void max_pool2d_backward_lds_kernel(
     const T* __restrict__ gout, const int8_t* __restrict__ idx, T* __restrict__ gin,
     int64_t total_out, PoolGeom g, int rows_per_band, int bands, int max_out_rows) {
@@ -225,7 +272,12 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_backward_lds_kernel(
     const int64_t first = (nc * g.Ho + ho_lo) * (int64_t)g.Wo;
     const int count = (ho_hi - ho_lo + 1) * g.Wo;
     shift_g = stage_span(gout, first, count, total_out, s_g);
-    shift_i = stage_span(idx, first, count, total_out, s_i);
+    if (NIB) {
+      const int64_t b0 = first >> 1, b1 = (first + count + 1) >> 1;
+      shift_i = 2 * stage_span(idx, b0, (int)(b1 - b0), (total_out + 1) >> 1, s_i) + (int)(first & 1);
+    } else {
+      shift_i = stage_span(idx, first, count, total_out, s_i);
+    }
   }
   __syncthreads();
   const int lane = threadIdx.x & 63;
@@ -247,7 +299,7 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_backward_lds_kernel(
         const int rr = (ho - ho_lo) * g.Wo;
         for (int wo = b_lo; wo <= b_hi; ++wo) {
           const int kw = w - (wo * k.SW - k.PW);
-          if ((int)s_i[shift_i + rr + wo] == kh * k.KW + kw) acc += lds_value<T>(s_g, shift_g + rr + wo);
+          if (staged_index<NIB>(s_i, shift_i + rr + wo) == kh * k.KW + kw) acc += lds_value<T>(s_g, shift_g + rr + wo);
         }
       }
       Conv<T>::store(gin, irow + w, acc);
@@ -292,7 +344,7 @@ ACTNN_DEV void load4(const bf16_t* p, float (&v)[4]) {
   v[2] = as_float(hi << 16), v[3] = as_float(hi & 0xffff0000u);
 }
 
-template <typename T, int K, int P>
+template <typename T, int K, int P, bool NIB>
 __global__ __launch_bounds__(kFwdS2Threads) void max_pool2d_forward_s2_kernel(
     const T* __restrict__ x, T* __restrict__ y, int8_t* __restrict__ idx, PoolGeom g, int rows_per_band,
     int bands) {
@@ -327,7 +379,7 @@ __global__ __launch_bounds__(kFwdS2Threads) void max_pool2d_forward_s2_kernel(
       cc[a][0] = P == 1 && q > 0 ? left : init;
     }
     float out[4];
-    uint32_t packed_idx = 0;
+    uint64_t packed_idx = 0;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       float v = init;
@@ -343,15 +395,15 @@ __global__ __launch_bounds__(kFwdS2Threads) void max_pool2d_forward_s2_kernel(
           }
         }
       out[u] = v;
-      packed_idx |= index << (8 * u);
+      packed_idx |= (uint64_t)index << (IndexFields<NIB>::kBits * u);
     }
     const int64_t o = (nc * g.Ho + ho0 + r) * (int64_t)g.Wo + 4 * q;
     store4<T>(y + o, out);
-    *reinterpret_cast<uint32_t*>(idx + o) = packed_idx;
+    IndexFields<NIB>::template store<4>(idx, o, packed_idx);
   }
 }
 
-template <typename T, int K, int P>
+template <typename T, int K, int P, bool NIB>
 __global__ __launch_bounds__(kBwdS2Threads) void max_pool2d_backward_s2_kernel(
     const T* __restrict__ gout, const int8_t* __restrict__ idx, T* __restrict__ gin, int64_t total_out,
     PoolGeom g, int pairs_per_band, int bands, int max_out_rows) {
@@ -367,7 +419,9 @@ __global__ __launch_bounds__(kBwdS2Threads) void max_pool2d_backward_s2_kernel(
   const int64_t first = (nc * g.Ho + s0) * (int64_t)g.Wo;
   const int count = (ho_hi - s0 + 1) * g.Wo;
   const int shift_g = stage_span<T, kBwdS2Threads, false>(gout, first, count, total_out, s_g);
-  const int shift_i = stage_span<int8_t, kBwdS2Threads, false>(idx, first, count, total_out, s_i);
+  // (first and count are multiples of 4: whole bytes in the two-per-byte format)
+  const int shift_i = NIB ? 2 * stage_span<int8_t, kBwdS2Threads, false>(idx, first >> 1, count >> 1, total_out >> 1, s_i)
+                          : stage_span<int8_t, kBwdS2Threads, false>(idx, first, count, total_out, s_i);
   __syncthreads();
   const int cpr = g.W >> 3;
   const int items = pairs * cpr;
@@ -381,12 +435,12 @@ __global__ __launch_bounds__(kBwdS2Threads) void max_pool2d_backward_s2_kernel(
       const bool row_ok = s0 + r + j < g.Ho;
       // Wo % 4 == 0 makes both positions 4-element aligned
       load4(s_g + shift_g + at, reinterpret_cast<float(&)[4]>(gv[j][0]));
-      const uint32_t i4 = *reinterpret_cast<const uint32_t*>(s_i + shift_i + at);
+      const uint64_t i4 = IndexFields<NIB>::template load<4>(s_i, (int64_t)(shift_i + at));
 #pragma unroll
-      for (int t = 0; t < 4; ++t) iv[j][t] = row_ok ? (int)((i4 >> (8 * t)) & 0xffu) : -1;
+      for (int t = 0; t < 4; ++t) iv[j][t] = row_ok ? IndexFields<NIB>::get(i4, t) : -1;
       if (EXTRA) {
         gv[j][NW - 1] = lds_value<T>(s_g, shift_g + at + 4);
-        iv[j][NW - 1] = row_ok && q < cpr - 1 ? (int)s_i[shift_i + at + 4] : -1;
+        iv[j][NW - 1] = row_ok && q < cpr - 1 ? staged_index<NIB>(s_i, shift_i + at + 4) : -1;
       }
     }
 #pragma unroll
@@ -453,7 +507,7 @@ template <typename F> int pick_band(int units, int per_unit, int threads, int ma
   return best;
 }
 
-template <typename T>
+template <typename T, bool NIB>
 int launch_fwd(const void* x, void* y, int8_t* idx, int64_t total, const PoolGeom& g, hipStream_t s) {
   const int64_t planes = total / ((int64_t)g.Ho * g.Wo);
   auto need = [&](int rows) { return ((size_t)((rows - 1) * g.SH + g.KH) * g.W + 16) * sizeof(T); };
@@ -464,13 +518,13 @@ int launch_fwd(const void* x, void* y, int8_t* idx, int64_t total, const PoolGeo
       const dim3 grid((unsigned)(planes * bands)), blk(kFwdS2Threads);
       const T* xi = static_cast<const T*>(x);
       T* yo = static_cast<T*>(y);
-      if (k == 3) max_pool2d_forward_s2_kernel<T, 3, 1><<<grid, blk, need(rb), s>>>(xi, yo, idx, g, rb, bands);
-      else max_pool2d_forward_s2_kernel<T, 2, 0><<<grid, blk, need(rb), s>>>(xi, yo, idx, g, rb, bands);
+      if (k == 3) max_pool2d_forward_s2_kernel<T, 3, 1, NIB><<<grid, blk, need(rb), s>>>(xi, yo, idx, g, rb, bands);
+      else max_pool2d_forward_s2_kernel<T, 2, 0, NIB><<<grid, blk, need(rb), s>>>(xi, yo, idx, g, rb, bands);
       ACTNN_RETURN_LAUNCH_STATUS();
     }
   }
   const int rb = pick_rows(g.Ho, g.Wo, 1024, need);
-  if (rb > 0 && aligned16(x)) {
+  if (rb > 0 && aligned16(x) && (!NIB || g.Wo % 2 == 0)) {
     const int bands = (g.Ho + rb - 1) / rb;
     if (planes * bands <= 0x7fffffffLL) {
       const dim3 grid((unsigned)(planes * bands)), blk(kThreads);
@@ -478,22 +532,22 @@ int launch_fwd(const void* x, void* y, int8_t* idx, int64_t total, const PoolGeo
       T* yo = static_cast<T*>(y);
       const int64_t tin = planes * g.H * g.W;
       switch (preset_of(g)) {
-        case 1: max_pool2d_forward_lds_kernel<T, 1><<<grid, blk, need(rb), s>>>(xi, yo, idx, tin, g, rb, bands); break;
-        case 2: max_pool2d_forward_lds_kernel<T, 2><<<grid, blk, need(rb), s>>>(xi, yo, idx, tin, g, rb, bands); break;
-        case 3: max_pool2d_forward_lds_kernel<T, 3><<<grid, blk, need(rb), s>>>(xi, yo, idx, tin, g, rb, bands); break;
-        default: max_pool2d_forward_lds_kernel<T, 0><<<grid, blk, need(rb), s>>>(xi, yo, idx, tin, g, rb, bands); break;
+        case 1: max_pool2d_forward_lds_kernel<T, 1, NIB><<<grid, blk, need(rb), s>>>(xi, yo, idx, tin, g, rb, bands); break;
+        case 2: max_pool2d_forward_lds_kernel<T, 2, NIB><<<grid, blk, need(rb), s>>>(xi, yo, idx, tin, g, rb, bands); break;
+        case 3: max_pool2d_forward_lds_kernel<T, 3, NIB><<<grid, blk, need(rb), s>>>(xi, yo, idx, tin, g, rb, bands); break;
+        default: max_pool2d_forward_lds_kernel<T, 0, NIB><<<grid, blk, need(rb), s>>>(xi, yo, idx, tin, g, rb, bands); break;
       }
       ACTNN_RETURN_LAUNCH_STATUS();
     }
   }
   const int64_t blocks = (total + kThreads - 1) / kThreads;
   if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
-  max_pool2d_forward_kernel<T><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+  max_pool2d_forward_kernel<T, NIB><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
       static_cast<const T*>(x), static_cast<T*>(y), idx, total, g);
   ACTNN_RETURN_LAUNCH_STATUS();
 }
 
-template <typename T>
+template <typename T, bool NIB>
 int launch_bwd(const void* gout, const int8_t* idx, void* gin, int64_t total, const PoolGeom& g,
                hipStream_t s) {
   const int64_t planes = total / ((int64_t)g.H * g.W);
@@ -516,8 +570,8 @@ int launch_bwd(const void* gout, const int8_t* idx, void* gin, int64_t total, co
       const T* go = static_cast<const T*>(gout);
       T* gi = static_cast<T*>(gin);
       const int64_t tout = planes * g.Ho * g.Wo;
-      if (k == 3) max_pool2d_backward_s2_kernel<T, 3, 1><<<grid, blk, need2(pb), s>>>(go, idx, gi, tout, g, pb, bands, pb + 2);
-      else max_pool2d_backward_s2_kernel<T, 2, 0><<<grid, blk, need2(pb), s>>>(go, idx, gi, tout, g, pb, bands, pb + 2);
+      if (k == 3) max_pool2d_backward_s2_kernel<T, 3, 1, NIB><<<grid, blk, need2(pb), s>>>(go, idx, gi, tout, g, pb, bands, pb + 2);
+      else max_pool2d_backward_s2_kernel<T, 2, 0, NIB><<<grid, blk, need2(pb), s>>>(go, idx, gi, tout, g, pb, bands, pb + 2);
       ACTNN_RETURN_LAUNCH_STATUS();
     }
   }
@@ -531,17 +585,17 @@ int launch_bwd(const void* gout, const int8_t* idx, void* gin, int64_t total, co
       const int64_t tout = planes * g.Ho * g.Wo;
       const int orows = out_rows(rb);
       switch (preset_of(g)) {
-        case 1: max_pool2d_backward_lds_kernel<T, 1><<<grid, blk, need(rb), s>>>(go, idx, gi, tout, g, rb, bands, orows); break;
-        case 2: max_pool2d_backward_lds_kernel<T, 2><<<grid, blk, need(rb), s>>>(go, idx, gi, tout, g, rb, bands, orows); break;
-        case 3: max_pool2d_backward_lds_kernel<T, 3><<<grid, blk, need(rb), s>>>(go, idx, gi, tout, g, rb, bands, orows); break;
-        default: max_pool2d_backward_lds_kernel<T, 0><<<grid, blk, need(rb), s>>>(go, idx, gi, tout, g, rb, bands, orows); break;
+        case 1: max_pool2d_backward_lds_kernel<T, 1, NIB><<<grid, blk, need(rb), s>>>(go, idx, gi, tout, g, rb, bands, orows); break;
+        case 2: max_pool2d_backward_lds_kernel<T, 2, NIB><<<grid, blk, need(rb), s>>>(go, idx, gi, tout, g, rb, bands, orows); break;
+        case 3: max_pool2d_backward_lds_kernel<T, 3, NIB><<<grid, blk, need(rb), s>>>(go, idx, gi, tout, g, rb, bands, orows); break;
+        default: max_pool2d_backward_lds_kernel<T, 0, NIB><<<grid, blk, need(rb), s>>>(go, idx, gi, tout, g, rb, bands, orows); break;
       }
       ACTNN_RETURN_LAUNCH_STATUS();
     }
   }
   const int64_t blocks = (total + kThreads - 1) / kThreads;
   if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
-  max_pool2d_backward_kernel<T><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+  max_pool2d_backward_kernel<T, NIB><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
       static_cast<const T*>(gout), idx, static_cast<T*>(gin), total, g);
   ACTNN_RETURN_LAUNCH_STATUS();
 }
@@ -569,7 +623,7 @@ template <typename T, int E> ACTNN_DEV void narrow_chunk(T* p, const float (&v)[
   else store8(p, v);
 }
 
-template <typename T>
+template <typename T, bool NIB>
 __global__ __launch_bounds__(kThreads) void max_pool2d_forward_cl_kernel(
     const T* __restrict__ x, T* __restrict__ y, int8_t* __restrict__ idx, int64_t chunks, int cpp /* chunks per pixel */,
     int64_t C, PoolGeom g) {
@@ -601,19 +655,15 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_forward_cl_kernel(
     }
   }
   narrow_chunk<T, E>(y + pix * C + c, best);
-  uint32_t packed[E / 4];
+  uint64_t fields = 0;
 #pragma unroll
-  for (int q = 0; q < E / 4; ++q)
-    packed[q] = (uint32_t)where[4 * q] | ((uint32_t)where[4 * q + 1] << 8) | ((uint32_t)where[4 * q + 2] << 16) |
-                ((uint32_t)where[4 * q + 3] << 24);
-  uint32_t* out = reinterpret_cast<uint32_t*>(idx + pix * C + c);
-#pragma unroll
-  for (int q = 0; q < E / 4; ++q) out[q] = packed[q];
+  for (int e = 0; e < E; ++e) fields |= (uint64_t)where[e] << (IndexFields<NIB>::kBits * e);
+  IndexFields<NIB>::template store<E>(idx, pix * C + c, fields);
 }
 
 // Gather form of the backward pass: every input position sums the gradients of the windows that
 // chose it, in a fixed order (no atomics, no zero fill).
-template <typename T>
+template <typename T, bool NIB>
 __global__ __launch_bounds__(kThreads) void max_pool2d_backward_cl_kernel(
     const T* __restrict__ gout, const int8_t* __restrict__ idx, T* __restrict__ gin, int64_t chunks, int cpp,
     int64_t C, PoolGeom g) {
@@ -644,25 +694,21 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_backward_cl_kernel(
       const int64_t o = (obase + (int64_t)ho * g.Wo + wo) * C + c;
       float v[E];
       widen_chunk<T, E>(gout + o, v);
-      const uint32_t* pi = reinterpret_cast<const uint32_t*>(idx + o);
+      const uint64_t fields = IndexFields<NIB>::template load<E>(idx, o);
 #pragma unroll
-      for (int q = 0; q < E / 4; ++q) {
-        const uint32_t word = pi[q];
-#pragma unroll
-        for (int b = 0; b < 4; ++b)
-          if ((int)((word >> (8 * b)) & 0xffu) == k) acc[4 * q + b] += v[4 * q + b];
-      }
+      for (int e = 0; e < E; ++e)
+        if (IndexFields<NIB>::get(fields, e) == k) acc[e] += v[e];
     }
   }
   narrow_chunk<T, E>(gin + pix * C + c, acc);
 }
 
-template <typename T>
+template <typename T, bool NIB>
 int launch_cl(bool forward, const void* a, const int8_t* idx_in, int8_t* idx_out, void* out, int64_t N, int64_t C,
               const PoolGeom& g, hipStream_t s) {
   constexpr int E = PoolChunk<T>::kElems;
   if (C % E != 0 || C / E > 0x7fffffffLL) return ACTNN_EINVAL;
-  if (!aligned16(a) || !aligned16(out)) return ACTNN_EALIGN;
+  if (!aligned16(a) || !aligned16(out) || !aligned16(forward ? idx_out : idx_in)) return ACTNN_EALIGN;
   const int cpp = (int)(C / E);
   const int64_t pixels = forward ? N * g.Ho * g.Wo : N * (int64_t)g.H * g.W;
   const int64_t chunks = pixels * cpp;
@@ -670,10 +716,10 @@ int launch_cl(bool forward, const void* a, const int8_t* idx_in, int8_t* idx_out
   if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
   if (blocks == 0) return ACTNN_OK;
   if (forward)
-    max_pool2d_forward_cl_kernel<T><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+    max_pool2d_forward_cl_kernel<T, NIB><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
         static_cast<const T*>(a), static_cast<T*>(out), idx_out, chunks, cpp, C, g);
   else
-    max_pool2d_backward_cl_kernel<T><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+    max_pool2d_backward_cl_kernel<T, NIB><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
         static_cast<const T*>(a), idx_in, static_cast<T*>(out), chunks, cpp, C, g);
   ACTNN_RETURN_LAUNCH_STATUS();
 }
@@ -693,10 +739,12 @@ int check_geom(int64_t N, int64_t C, int64_t H, int64_t W, int64_t Ho, int64_t W
 }  // namespace
 }  // namespace actnn
 
-extern "C" int actnn_max_pool2d_forward(const void* x, void* y, int8_t* idx, int64_t N, int64_t C,
-                                        int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH, int KW,
-                                        int SH, int SW, int PH, int PW, int dtype, void* stream) {
-  using namespace actnn;
+// The four operators (forward / backward, default / channels-last layout) with either index format.
+namespace actnn {
+namespace {
+template <bool NIB>
+int pool_forward(bool cl, const void* x, void* y, int8_t* idx, int64_t N, int64_t C, int64_t H, int64_t W,
+                 int64_t Ho, int64_t Wo, int KH, int KW, int SH, int SW, int PH, int PW, int dtype, void* stream) {
   const int rc = check_geom(N, C, H, W, Ho, Wo, KH, KW, SH, SW, PH, PW);
   if (rc != ACTNN_OK) return rc;
   const int64_t total = N * C * Ho * Wo;
@@ -705,18 +753,16 @@ extern "C" int actnn_max_pool2d_forward(const void* x, void* y, int8_t* idx, int
   const PoolGeom g{(int)H, (int)W, (int)Ho, (int)Wo, KH, KW, SH, SW, PH, PW};
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (dtype) {
-    case ACTNN_F32: return launch_fwd<float>(x, y, idx, total, g, s);
-    case ACTNN_F16: return launch_fwd<__half>(x, y, idx, total, g, s);
-    case ACTNN_BF16: return launch_fwd<bf16_t>(x, y, idx, total, g, s);
+    case ACTNN_F32: return cl ? launch_cl<float, NIB>(true, x, nullptr, idx, y, N, C, g, s) : launch_fwd<float, NIB>(x, y, idx, total, g, s);
+    case ACTNN_F16: return cl ? launch_cl<__half, NIB>(true, x, nullptr, idx, y, N, C, g, s) : launch_fwd<__half, NIB>(x, y, idx, total, g, s);
+    case ACTNN_BF16: return cl ? launch_cl<bf16_t, NIB>(true, x, nullptr, idx, y, N, C, g, s) : launch_fwd<bf16_t, NIB>(x, y, idx, total, g, s);
     default: return ACTNN_EDTYPE;
   }
 }
-
-extern "C" int actnn_max_pool2d_backward(const void* grad_out, const int8_t* idx, void* grad_in,
-                                         int64_t N, int64_t C, int64_t H, int64_t W, int64_t Ho,
-                                         int64_t Wo, int KH, int KW, int SH, int SW, int PH, int PW,
-                                         int dtype, void* stream) {
-  using namespace actnn;
+template <bool NIB>
+int pool_backward(bool cl, const void* grad_out, const int8_t* idx, void* grad_in, int64_t N, int64_t C, int64_t H,
+                  int64_t W, int64_t Ho, int64_t Wo, int KH, int KW, int SH, int SW, int PH, int PW, int dtype,
+                  void* stream) {
   const int rc = check_geom(N, C, H, W, Ho, Wo, KH, KW, SH, SW, PH, PW);
   if (rc != ACTNN_OK) return rc;
   const int64_t total = N * C * H * W;
@@ -725,46 +771,40 @@ extern "C" int actnn_max_pool2d_backward(const void* grad_out, const int8_t* idx
   const PoolGeom g{(int)H, (int)W, (int)Ho, (int)Wo, KH, KW, SH, SW, PH, PW};
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (dtype) {
-    case ACTNN_F32: return launch_bwd<float>(grad_out, idx, grad_in, total, g, s);
-    case ACTNN_F16: return launch_bwd<__half>(grad_out, idx, grad_in, total, g, s);
-    case ACTNN_BF16: return launch_bwd<bf16_t>(grad_out, idx, grad_in, total, g, s);
+    case ACTNN_F32: return cl ? launch_cl<float, NIB>(false, grad_out, idx, nullptr, grad_in, N, C, g, s) : launch_bwd<float, NIB>(grad_out, idx, grad_in, total, g, s);
+    case ACTNN_F16: return cl ? launch_cl<__half, NIB>(false, grad_out, idx, nullptr, grad_in, N, C, g, s) : launch_bwd<__half, NIB>(grad_out, idx, grad_in, total, g, s);
+    case ACTNN_BF16: return cl ? launch_cl<bf16_t, NIB>(false, grad_out, idx, nullptr, grad_in, N, C, g, s) : launch_bwd<bf16_t, NIB>(grad_out, idx, grad_in, total, g, s);
     default: return ACTNN_EDTYPE;
   }
 }
+}  // namespace
+}  // namespace actnn
 
-extern "C" int actnn_max_pool2d_forward_cl(const void* x, void* y, int8_t* idx, int64_t N, int64_t C,
-                                           int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH, int KW,
-                                           int SH, int SW, int PH, int PW, int dtype, void* stream) {
-  using namespace actnn;
-  const int rc = check_geom(N, C, H, W, Ho, Wo, KH, KW, SH, SW, PH, PW);
-  if (rc != ACTNN_OK) return rc;
-  if (N * C * Ho * Wo == 0) return ACTNN_OK;
-  if (!x || !y || !idx) return ACTNN_EINVAL;
-  const PoolGeom g{(int)H, (int)W, (int)Ho, (int)Wo, KH, KW, SH, SW, PH, PW};
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  switch (dtype) {
-    case ACTNN_F32: return launch_cl<float>(true, x, nullptr, idx, y, N, C, g, s);
-    case ACTNN_F16: return launch_cl<__half>(true, x, nullptr, idx, y, N, C, g, s);
-    case ACTNN_BF16: return launch_cl<bf16_t>(true, x, nullptr, idx, y, N, C, g, s);
-    default: return ACTNN_EDTYPE;
-  }
+#define ACTNN_POOL_GEOM_PARAMS int64_t N, int64_t C, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH, int KW, \
+                               int SH, int SW, int PH, int PW, int dtype, void* stream
+#define ACTNN_POOL_GEOM_ARGS N, C, H, W, Ho, Wo, KH, KW, SH, SW, PH, PW, dtype, stream
+
+extern "C" int actnn_max_pool2d_forward(const void* x, void* y, int8_t* idx, ACTNN_POOL_GEOM_PARAMS) {
+  return actnn::pool_forward<false>(false, x, y, idx, ACTNN_POOL_GEOM_ARGS);
 }
-
-extern "C" int actnn_max_pool2d_backward_cl(const void* grad_out, const int8_t* idx, void* grad_in,
-                                            int64_t N, int64_t C, int64_t H, int64_t W, int64_t Ho,
-                                            int64_t Wo, int KH, int KW, int SH, int SW, int PH, int PW,
-                                            int dtype, void* stream) {
-  using namespace actnn;
-  const int rc = check_geom(N, C, H, W, Ho, Wo, KH, KW, SH, SW, PH, PW);
-  if (rc != ACTNN_OK) return rc;
-  if (N * C * H * W == 0) return ACTNN_OK;
-  if (!grad_out || !grad_in || !idx) return ACTNN_EINVAL;
-  const PoolGeom g{(int)H, (int)W, (int)Ho, (int)Wo, KH, KW, SH, SW, PH, PW};
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  switch (dtype) {
-    case ACTNN_F32: return launch_cl<float>(false, grad_out, idx, nullptr, grad_in, N, C, g, s);
-    case ACTNN_F16: return launch_cl<__half>(false, grad_out, idx, nullptr, grad_in, N, C, g, s);
-    case ACTNN_BF16: return launch_cl<bf16_t>(false, grad_out, idx, nullptr, grad_in, N, C, g, s);
-    default: return ACTNN_EDTYPE;
-  }
+extern "C" int actnn_max_pool2d_backward(const void* grad_out, const int8_t* idx, void* grad_in, ACTNN_POOL_GEOM_PARAMS) {
+  return actnn::pool_backward<false>(false, grad_out, idx, grad_in, ACTNN_POOL_GEOM_ARGS);
+}
+extern "C" int actnn_max_pool2d_forward_cl(const void* x, void* y, int8_t* idx, ACTNN_POOL_GEOM_PARAMS) {
+  return actnn::pool_forward<false>(true, x, y, idx, ACTNN_POOL_GEOM_ARGS);
+}
+extern "C" int actnn_max_pool2d_backward_cl(const void* grad_out, const int8_t* idx, void* grad_in, ACTNN_POOL_GEOM_PARAMS) {
+  return actnn::pool_backward<false>(true, grad_out, idx, grad_in, ACTNN_POOL_GEOM_ARGS);
+}
+extern "C" int actnn_max_pool2d_forward_nibble(const void* x, void* y, uint8_t* idx, ACTNN_POOL_GEOM_PARAMS) {
+  return actnn::pool_forward<true>(false, x, y, reinterpret_cast<int8_t*>(idx), ACTNN_POOL_GEOM_ARGS);
+}
+extern "C" int actnn_max_pool2d_backward_nibble(const void* grad_out, const uint8_t* idx, void* grad_in, ACTNN_POOL_GEOM_PARAMS) {
+  return actnn::pool_backward<true>(false, grad_out, reinterpret_cast<const int8_t*>(idx), grad_in, ACTNN_POOL_GEOM_ARGS);
+}
+extern "C" int actnn_max_pool2d_forward_cl_nibble(const void* x, void* y, uint8_t* idx, ACTNN_POOL_GEOM_PARAMS) {
+  return actnn::pool_forward<true>(true, x, y, reinterpret_cast<int8_t*>(idx), ACTNN_POOL_GEOM_ARGS);
+}
+extern "C" int actnn_max_pool2d_backward_cl_nibble(const void* grad_out, const uint8_t* idx, void* grad_in, ACTNN_POOL_GEOM_PARAMS) {
+  return actnn::pool_backward<true>(true, grad_out, reinterpret_cast<const int8_t*>(idx), grad_in, ACTNN_POOL_GEOM_ARGS);
 }

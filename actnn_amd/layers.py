@@ -302,10 +302,11 @@ class QMaxPool2d(_MaxPoolNd):
             # the model stays channels-last
             out = ext_quantization.act_quantized_max_pool2d(
                 input.contiguous(), self.kernel_size, self.stride, self.padding, self.dilation,
-                self.ceil_mode, self.return_indices)
+                self.ceil_mode, self.return_indices, config.pool_index_nibbles)
             return out.contiguous(memory_format=torch.channels_last)
         return ext_quantization.act_quantized_max_pool2d(input, self.kernel_size, self.stride, self.padding,
-                                                         self.dilation, self.ceil_mode, self.return_indices)
+                                                         self.dilation, self.ceil_mode, self.return_indices,
+                                                         config.pool_index_nibbles)
 
 
 class QAvgPool2d(_AvgPoolNd):
@@ -325,4 +326,4 @@ class QAvgPool2d(_AvgPoolNd):
     def forward(self, input):
         warnings.warn("avg_pool2d is replaced by max_pool2d: no memory-saving average-pool kernel exists.")
         return ext_quantization.act_quantized_max_pool2d(input, self.kernel_size, self.stride, self.padding,
-                                                         (1, 1), self.ceil_mode, False)
+                                                         (1, 1), self.ceil_mode, False, config.pool_index_nibbles)

@@ -196,6 +196,17 @@ def other_configs(device, reps):
     out["max_pool2d_forward_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
     t = _event_time_ms(lambda: ext_q.max_pool2d_backward(gp, idx, x.shape, k, s, p), reps)
     out["max_pool2d_backward_f16"] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
+    # the same with the indices kept two per byte (what QMaxPool2d saves by default), in both layouts
+    b = 2 * n + 2 * n / 4 + n / 8
+    for tag, xin, gin in (("", x, gp), ("_channels_last", x.contiguous(memory_format=torch.channels_last),
+                                        gp.contiguous(memory_format=torch.channels_last))):
+        cl = tag != ""
+        _, idx4 = ext_q.max_pool2d_forward(xin, k, s, p, (1, 1), nibble_indices=True)
+        t = _event_time_ms(lambda: ext_q.max_pool2d_forward(xin, k, s, p, (1, 1), nibble_indices=True), reps)
+        out["max_pool2d_forward_nibble_indices%s_f16" % tag] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
+        t = _event_time_ms(lambda: ext_q.max_pool2d_backward(gin, idx4, x.shape, k, s, p, channels_last=cl), reps)
+        out["max_pool2d_backward_nibble_indices%s_f16" % tag] = {"ms": t, "GB/s": b / t / 1e6, "frac": b / t / 1e6 / HBM_PEAK_GBS}
+        del idx4, xin, gin
     del y, mask, yp, idx, gp
     # training-mode batch norm on the same tensor, in both layouts: forward (statistics + normalise;
     # with the quantiser's group min/max from the statistics pass; with the 2-bit pack in the

@@ -157,6 +157,24 @@ int actnn_max_pool2d_forward_cl(const void* x, void* y, int8_t* idx, int64_t N, 
 int actnn_max_pool2d_backward_cl(const void* grad_out, const int8_t* idx, void* grad_in, int64_t N,
                                  int64_t C, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH,
                                  int KW, int SH, int SW, int PH, int PW, int dtype, void* stream);
+/* The same four operators with the indices kept two per byte.  No counterpart in the reference,
+ * which keeps one int8 per output although it already requires KH * KW < 16
+ * (quantization.cc:162): output o of the flat order of y (default layout: [N, C, Ho, Wo];
+ * channels-last: [N, Ho, Wo, C]) is stored in bits 4 * (o & 1) .. 4 * (o & 1) + 3 of byte
+ * o / 2; idx holds (N * C * Ho * Wo + 1) / 2 bytes and the unused half of the last byte of an
+ * odd count is written as 0.  Values, indices and gradients equal those of the int8 operators. */
+int actnn_max_pool2d_forward_nibble(const void* x, void* y, uint8_t* idx, int64_t N, int64_t C,
+                                    int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH, int KW,
+                                    int SH, int SW, int PH, int PW, int dtype, void* stream);
+int actnn_max_pool2d_backward_nibble(const void* grad_out, const uint8_t* idx, void* grad_in, int64_t N,
+                                     int64_t C, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH,
+                                     int KW, int SH, int SW, int PH, int PW, int dtype, void* stream);
+int actnn_max_pool2d_forward_cl_nibble(const void* x, void* y, uint8_t* idx, int64_t N, int64_t C,
+                                       int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH, int KW,
+                                       int SH, int SW, int PH, int PW, int dtype, void* stream);
+int actnn_max_pool2d_backward_cl_nibble(const void* grad_out, const uint8_t* idx, void* grad_in, int64_t N,
+                                        int64_t C, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH,
+                                        int KW, int SH, int SW, int PH, int PW, int dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------
  * calc_precision (HOST pointers): greedy bit allocation, mutates b in place.

@@ -92,3 +92,22 @@ def max_pool2d_backward(gout, idx, in_shape, kernel, stride, padding):
     for r in range(N * C):
         np.add.at(gin[r], lin[r], g[r])
     return gin.reshape(N, C, H, W)
+
+
+def pack_index_nibbles(idx):
+    """Two indices per byte, the format of the *_nibble operators of the library (the reference has
+    none: it keeps one int8 per output, quantization_cuda_kernel.cu:683): element o of `idx` in memory order
+    -> bits 4 * (o & 1) .. of byte o // 2; the spare half of the last byte of an odd count is 0."""
+    flat = np.asarray(idx).reshape(-1).astype(np.uint8)
+    assert flat.size == 0 or flat.max() < 16
+    if flat.size & 1:
+        flat = np.concatenate([flat, np.zeros(1, np.uint8)])
+    return (flat[0::2] | (flat[1::2] << 4)).astype(np.uint8)
+
+
+def unpack_index_nibbles(packed, count):
+    packed = np.asarray(packed, dtype=np.uint8)
+    out = np.empty(packed.size * 2, np.int8)
+    out[0::2] = packed & 15
+    out[1::2] = packed >> 4
+    return out[:count]

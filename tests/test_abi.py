@@ -47,6 +47,10 @@ def test_argument_errors_need_no_gpu(lib):
     assert lib.actnn_batch_norm_backward_sumsq_entries(4, 3, 49, 2, 0) == -1
     assert lib.actnn_sample_sqnorm(None, None, 4, 30, 1, 2, None) == -1           # F % 8 != 0
     assert lib.actnn_max_pool2d_forward_cl(None, None, None, 1, 8, 8, 8, 4, 4, 4, 4, 2, 2, 1, 1, 0, None) == -1
+    for name in ("actnn_max_pool2d_forward_nibble", "actnn_max_pool2d_forward_cl_nibble",
+                 "actnn_max_pool2d_backward_nibble", "actnn_max_pool2d_backward_cl_nibble"):
+        assert getattr(lib, name)(None, None, None, 1, 8, 8, 8, 4, 4, 4, 4, 2, 2, 1, 1, 0, None) == -1    # KH*KW >= 16
+        assert getattr(lib, name)(None, None, None, 1, 8, 8, 8, 4, 4, 3, 3, 2, 2, 1, 1, 0, None) == -1    # null pointers
     # the entry point with the built-in scratch array refuses what the array cannot hold
     assert lib.actnn_batch_norm_workspace_bytes(64, 1 << 20, 8, 2, 1) > lib.actnn_batch_norm_forward_static_limit()
     assert lib.actnn_batch_norm_forward_static(None, None, None, None, None, None, None, None, None, None,

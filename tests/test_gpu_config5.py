@@ -45,7 +45,7 @@ def _elems(shapes):
 
 
 QUANTISED_ELEMS = _elems(CONV_INPUTS) + _elems(BN_INPUTS) + FC_INPUT      # per sample
-MASK_AND_INDEX_BYTES = _elems(RELU_OUTPUTS) // 8 + POOL_OUTPUT[0] * POOL_OUTPUT[1] ** 2
+MASK_AND_INDEX_BYTES = _elems(RELU_OUTPUTS) // 8 + POOL_OUTPUT[0] * POOL_OUTPUT[1] ** 2 // 2
 assert QUANTISED_ELEMS == 21_778_432 and QUANTISED_ELEMS % 256 == 0 and _elems(RELU_OUTPUTS) == 9_608_704
 
 
@@ -57,7 +57,7 @@ def compressed_bytes_per_sample(avg_bits=2):
 
 def closed_form_bytes_per_sample(avg_bits=2):
     """Bytes the L3 model keeps per sample for the backward pass: the compressed inputs, 1-bit ReLU
-    masks, int8 max-pool indices."""
+    masks, max-pool indices at two per byte."""
     return compressed_bytes_per_sample(avg_bits) + MASK_AND_INDEX_BYTES
 
 
@@ -121,7 +121,7 @@ def test_resnet50_l3_batch512_bf16_step(channels_last):
                 avg = sum(b * d for b, d in zip(budgets, dims)) / sum(dims)
                 assert 1.9 < avg <= 2.0 + 1e-6, avg
             # The reference's protocol (train.py:363-397).  Besides the compressed inputs the layers'
-            # contexts hold the 1-bit ReLU masks, the int8 pool indices and the bf16 copies of the
+            # contexts hold the 1-bit ReLU masks, the 4-bit pool indices and the bf16 copies of the
             # weights that autocast makes (25.6 M parameters).
             weights_bf16 = sum(p.numel() for p in model.parameters() if p.dim() > 1) * 2
             if step == 0:

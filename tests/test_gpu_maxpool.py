@@ -122,3 +122,72 @@ def test_channels_last_special_values():
     out_o, idx_o = pool.max_pool2d_forward_literal(x, (3, 3), (2, 2), (1, 1))
     assert np.array_equal(idx.cpu().numpy(), idx_o)
     assert np.array_equal(y.cpu().numpy(), out_o, equal_nan=True)
+
+
+def _memory_order(t):
+    """the elements of a 4-d tensor in the order of its memory (default or channels-last)"""
+    if t.is_contiguous():
+        return t.reshape(-1)
+    return t.permute(0, 2, 3, 1).reshape(-1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("k,s,p", GEOMS)
+@pytest.mark.parametrize("shape", [(4, 8, 28, 28), (2, 3, 13, 17), (1, 1, 5, 5), (3, 5, 32, 24), (2, 3, 16, 8),
+                                   (1, 2, 224, 224), (3, 1, 7, 9), (1, 16, 31, 30)])
+def test_two_indices_per_byte_equal_the_int8_operators(dtype, k, s, p, shape):
+    """The *_nibble operators: same values; the packed indices are the int8 indices (checked against
+    the oracle above) packed two per byte in memory order, spare half byte 0; the gradient is
+    bit-identical to the int8 operators' gradient.  The shapes reach the stride-2 kernels, the
+    LDS-tiled ones (even output width), the one-thread-per-output ones (odd width, odd count) and,
+    with 8 or 16 channels, the channels-last ones."""
+    torch.manual_seed(sum(shape) + 5)
+    x = torch.randn(*shape).to(dtype).to(DEV)
+    layouts = [x]
+    if shape[1] % 8 == 0:
+        layouts.append(x.contiguous(memory_format=torch.channels_last))
+    for xin in layouts:
+        cl = xin is not x
+        assert ext_q.pool_takes_channels_last(xin) == cl
+        y, idx = ext_q.max_pool2d_forward(xin, k, s, p, (1, 1))
+        y4, idx4 = ext_q.max_pool2d_forward(xin, k, s, p, (1, 1), nibble_indices=True)
+        assert torch.equal(y4, y) and y4.stride() == y.stride()
+        assert idx4.dtype == torch.uint8 and idx4.shape == ((y.numel() + 1) // 2,)
+        want = pool.pack_index_nibbles(_memory_order(idx).cpu().numpy())
+        assert np.array_equal(idx4.cpu().numpy(), want)
+        g = torch.randn_like(y)
+        gin = ext_q.max_pool2d_backward(g, idx, x.shape, k, s, p)
+        gin4 = ext_q.max_pool2d_backward(g, idx4, x.shape, k, s, p, channels_last=cl)
+        assert torch.equal(gin4, gin) and gin4.stride() == gin.stride()
+
+
+@pytest.mark.parametrize("channels_last", [False, True])
+def test_layer_keeps_half_a_byte_per_output(channels_last):
+    """QMaxPool2d under config.pool_index_nibbles saves (numel + 1) // 2 bytes and gives torch's gradient."""
+    from actnn_amd.conf import config
+    from actnn_amd.layers import QMaxPool2d
+    x = torch.randn(4, 16, 28, 28, device=DEV, dtype=torch.float16)
+    if channels_last:
+        x = x.contiguous(memory_format=torch.channels_last)
+    saved = {}
+    g = torch.randn(4, 16, 14, 14, device=DEV, dtype=torch.float16)
+    if channels_last:
+        g = g.contiguous(memory_format=torch.channels_last)
+    for flag in (True, False):
+        config.pool_index_nibbles = flag
+        try:
+            xa = x.clone(memory_format=torch.preserve_format).requires_grad_(True)
+            sizes = []
+            with torch.autograd.graph.saved_tensors_hooks(lambda t: (sizes.append(t.numel() * t.element_size()), t)[1],
+                                                          lambda t: t):
+                y = QMaxPool2d(3, 2, 1)(xa)
+            y.backward(g)
+            saved[flag] = (sizes, xa.grad.clone())
+        finally:
+            config.pool_index_nibbles = True
+    n_out = 4 * 16 * 14 * 14
+    assert saved[True][0] == [n_out // 2] and saved[False][0] == [n_out]
+    assert torch.equal(saved[True][1], saved[False][1])
+    xr = x.clone().requires_grad_(True)
+    F.max_pool2d(xr, 3, 2, 1).backward(g)
+    assert torch.allclose(saved[True][1].float(), xr.grad.float(), atol=2e-2, rtol=2e-2)

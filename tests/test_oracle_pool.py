@@ -37,3 +37,16 @@ def test_literal_agrees_and_ties_take_first(k, s, p):
             i = h * s[0] - p[0] + idx[0, 0, h, w] // k[1]
             j = w * s[1] - p[1] + idx[0, 0, h, w] % k[1]
             assert x[0, 0, i, j] == out[0, 0, h, w]
+
+
+def test_index_nibbles_known_bytes_and_round_trip():
+    idx = np.array([1, 8, 0, 14, 3], np.int8)
+    packed = pool.pack_index_nibbles(idx)
+    assert packed.dtype == np.uint8 and packed.tolist() == [0x81, 0xE0, 0x03]
+    assert np.array_equal(pool.unpack_index_nibbles(packed, 5), idx)
+    rng = np.random.default_rng(0)
+    for n in (0, 1, 2, 17, 256):
+        idx = rng.integers(0, 15, n).astype(np.int8)
+        p = pool.pack_index_nibbles(idx)
+        assert p.size == (n + 1) // 2
+        assert np.array_equal(pool.unpack_index_nibbles(p, n), idx)
