@@ -45,21 +45,35 @@ def measured_traffic(kernel_name, path=TRAFFIC_SUMMARY):
     return None, None
 
 
+WARM_MS = 25.0      # the first ~20 ms of work after an idle spell run up to 7 % slower than the steady state
+
+
 def _event_time_ms(fn, reps, warmup=3):
-    """Average duration of fn() over `reps` launches, HIP events on the current stream (the
-    stream every kernel of this library is launched on)."""
+    """Average duration of fn() over back-to-back launches (about `reps` in all), HIP events on the
+    current stream (the stream every kernel of this library is launched on), after at least
+    `warmup` launches and WARM_MS of untimed work."""
     import torch
-    for _ in range(warmup):
-        fn()
     start = torch.cuda.Event(enable_timing=True)
     stop = torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    start.record()
-    for _ in range(reps):
+    for _ in range(warmup):
         fn()
+    start.record()
+    fn()
     stop.record()
     torch.cuda.synchronize()
-    return start.elapsed_time(stop) / reps
+    for _ in range(min(500, int(WARM_MS / max(start.elapsed_time(stop), 1e-3)))):
+        fn()
+    # five back-to-back chunks, the median chunk: a one-off stall (a few ms, now and then) spoils one
+    chunk = max(1, reps // 5)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(6)]
+    torch.cuda.synchronize()
+    marks[0].record()
+    for i in range(5):
+        for _ in range(chunk):
+            fn()
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    return sorted(marks[i].elapsed_time(marks[i + 1]) / chunk for i in range(5))[2]
 
 
 def make_config2(device, N=256, C=256, H=56, W=56, seed=0, sample_spread=0.0, dtype=None):
@@ -381,8 +395,8 @@ def main():
     _heartbeat()
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the config-2 hot path")
     ap.add_argument("--only", choices=["other", "config4", "resnet50", "resnet50_channels_last", "resnet50_fp32", "resnet50_levels", "batch_norm_shapes"],
