@@ -703,6 +703,63 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_backward_cl_kernel(
   narrow_chunk<T, E>(gin + pix * C + c, acc);
 }
 
+// Backward for the stride-2 windows of the stem / VGG-style layers (3x3 pad 1 and 2x2 pad 0, H and W
+// even): a thread owns the 2x2 block of input pixels (2a.., 2b..) of one chunk of channels.  The windows
+// that reach the block are (a..a+1) x (b..b+1) (3x3) or (a, b) alone (2x2): one (gradient, index) load
+// per input pixel where the general kernel needs 2.25 (3x3).  Every pixel adds its windows in the
+// general kernel's order (rows, then columns), hence the same bits.
+template <typename T, int K, int P, bool NIB>
+__global__ __launch_bounds__(kThreads) void max_pool2d_backward_cl_s2_kernel(
+    const T* __restrict__ gout, const int8_t* __restrict__ idx, T* __restrict__ gin, int64_t items, int cpp,
+    int64_t C, PoolGeom g) {
+  constexpr int E = PoolChunk<T>::kElems;
+  constexpr int NWIN = K == 3 ? 2 : 1;
+  const int64_t id = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (id >= items) return;
+  const int c = (int)(id % cpp) * E;
+  const int64_t blk = id / cpp;
+  const int b = (int)(blk % g.Wo);
+  const int a = (int)((blk / g.Wo) % g.Ho);
+  const int64_t n = blk / ((int64_t)g.Wo * g.Ho);
+  float acc[2][2][E];
+#pragma unroll
+  for (int rr = 0; rr < 2; ++rr)
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+      for (int e = 0; e < E; ++e) acc[rr][cc][e] = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NWIN; ++j) {
+#pragma unroll
+    for (int t = 0; t < NWIN; ++t) {
+      if (a + j >= g.Ho || b + t >= g.Wo) continue;
+      const int64_t o = ((n * g.Ho + a + j) * (int64_t)g.Wo + b + t) * C + c;
+      float v[E];
+      widen_chunk<T, E>(gout + o, v);
+      const uint64_t fields = IndexFields<NIB>::template load<E>(idx, o);
+      // input row 2a + rr sits at window row kh = rr + P - 2j of window row a + j; columns alike
+#pragma unroll
+      for (int rr = 0; rr < 2; ++rr) {
+        const int kh = rr + P - 2 * j;
+        if (kh < 0 || kh >= K) continue;
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+          const int kw = cc + P - 2 * t;
+          if (kw < 0 || kw >= K) continue;
+#pragma unroll
+          for (int e = 0; e < E; ++e)
+            if (IndexFields<NIB>::get(fields, e) == kh * K + kw) acc[rr][cc][e] += v[e];
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int rr = 0; rr < 2; ++rr)
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc)
+      narrow_chunk<T, E>(gin + ((n * g.H + 2 * a + rr) * (int64_t)g.W + 2 * b + cc) * C + c, acc[rr][cc]);
+}
+
 template <typename T, bool NIB>
 int launch_cl(bool forward, const void* a, const int8_t* idx_in, int8_t* idx_out, void* out, int64_t N, int64_t C,
               const PoolGeom& g, hipStream_t s) {
@@ -715,12 +772,22 @@ int launch_cl(bool forward, const void* a, const int8_t* idx_in, int8_t* idx_out
   const int64_t blocks = (chunks + kThreads - 1) / kThreads;
   if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
   if (blocks == 0) return ACTNN_OK;
-  if (forward)
+  if (forward) {
     max_pool2d_forward_cl_kernel<T, NIB><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
         static_cast<const T*>(a), static_cast<T*>(out), idx_out, chunks, cpp, C, g);
-  else
+  } else if (const int p = preset_of(g); (p == 1 || p == 2) && g.H == 2 * g.Ho && g.W == 2 * g.Wo) {
+    const int64_t items = N * g.Ho * g.Wo * cpp;
+    const dim3 grid((unsigned)((items + kThreads - 1) / kThreads)), blk(kThreads);
+    if (p == 1)
+      max_pool2d_backward_cl_s2_kernel<T, 3, 1, NIB><<<grid, blk, 0, s>>>(
+          static_cast<const T*>(a), idx_in, static_cast<T*>(out), items, cpp, C, g);
+    else
+      max_pool2d_backward_cl_s2_kernel<T, 2, 0, NIB><<<grid, blk, 0, s>>>(
+          static_cast<const T*>(a), idx_in, static_cast<T*>(out), items, cpp, C, g);
+  } else {
     max_pool2d_backward_cl_kernel<T, NIB><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
         static_cast<const T*>(a), idx_in, static_cast<T*>(out), chunks, cpp, C, g);
+  }
   ACTNN_RETURN_LAUNCH_STATUS();
 }
 

@@ -191,3 +191,27 @@ def test_layer_keeps_half_a_byte_per_output(channels_last):
     xr = x.clone().requires_grad_(True)
     F.max_pool2d(xr, 3, 2, 1).backward(g)
     assert torch.allclose(saved[True][1].float(), xr.grad.float(), atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("k,s,p", [((3, 3), (2, 2), (1, 1)), ((2, 2), (2, 2), (0, 0))])
+@pytest.mark.parametrize("shape", [(2, 8, 8, 8), (3, 16, 14, 18), (1, 64, 112, 112), (2, 8, 4, 4), (2, 24, 6, 4)])
+def test_channels_last_stride2_backward_adds_in_the_order_of_the_default_layout(dtype, k, s, p, shape):
+    """Even H and W with a stride-2 window take the channels-last kernel that owns 2x2 input blocks;
+    it adds the windows of a pixel in the same order as the default-layout kernels, so the gradient is
+    the same bit for bit (heavily tied inputs make several windows point at one pixel)."""
+    torch.manual_seed(sum(shape) + 11)
+    x = torch.randint(-2, 3, shape).to(dtype).to(DEV)          # many ties
+    x_cl = x.contiguous(memory_format=torch.channels_last)
+    y, idx = ext_q.max_pool2d_forward(x, k, s, p, (1, 1))
+    _, idx_cl = ext_q.max_pool2d_forward(x_cl, k, s, p, (1, 1))
+    g = torch.randn_like(y)
+    gin = ext_q.max_pool2d_backward(g, idx, x.shape, k, s, p)
+    gin_cl = ext_q.max_pool2d_backward(g.contiguous(memory_format=torch.channels_last), idx_cl, x.shape, k, s, p)
+    assert gin_cl.is_contiguous(memory_format=torch.channels_last)
+    assert torch.equal(gin_cl, gin)
+    xr = x.clone().requires_grad_(True)
+    F.max_pool2d(xr, k, s, p).backward(g)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    # torch picks the first maximum too, so the sums hold the same terms
+    assert torch.allclose(gin_cl.float(), xr.grad.float(), atol=tol, rtol=tol)
