@@ -209,6 +209,16 @@ ACTNN_DEV void store8_nt(bf16_t* p, const float (&v)[8]) {
 // ------------------------------------------------------------------ cross-lane exchange
 // Value held by lane (lane ^ D), D in {1, 2, 4, 8, 16}.  1/2/8 are DPP moves, 4/16 go
 // through ds_swizzle (LDS crossbar, no memory), so they do not take a VALU slot.
+// Workgroups are dealt to the 8 XCDs round-robin by their index, and every XCD has its own L2.  A
+// kernel whose neighbouring blocks read the same lines (overlapping windows) renumbers its blocks so
+// that a run of consecutive logical blocks stays on one XCD: launch xcd_grid(n) blocks, work on block
+// xcd_block(); logical blocks >= n have nothing to do.
+constexpr int kXcds = 8;
+inline unsigned xcd_grid(int64_t n) { return (unsigned)((n + kXcds - 1) / kXcds * kXcds); }
+ACTNN_DEV int64_t xcd_block() {
+  return (int64_t)(blockIdx.x % kXcds) * (gridDim.x / kXcds) + blockIdx.x / kXcds;
+}
+
 template <int D> ACTNN_DEV uint32_t lane_xor(uint32_t x);
 template <> ACTNN_DEV uint32_t lane_xor<1>(uint32_t x) {
   return (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]

@@ -618,17 +618,32 @@ template <typename T, int E> ACTNN_DEV void widen_chunk(const T* p, float (&v)[E
     load8(p, v);
   }
 }
+// a dword filled with the value v of type T
+template <typename T> ACTNN_DEV uint32_t dword_of(float v);
+template <> ACTNN_DEV uint32_t dword_of<float>(float v) { return as_uint(v); }
+template <> ACTNN_DEV uint32_t dword_of<__half>(float v) { return float_to_half_bits(v) * 0x10001u; }
+template <> ACTNN_DEV uint32_t dword_of<bf16_t>(float v) { return float_to_bf16_bits(v) * 0x10001u; }
+template <typename T, int E> ACTNN_DEV void raw_widen_chunk(const u32x4& u, float (&v)[E]) {
+  if constexpr (E == 4) {
+    v[0] = as_float(u.x); v[1] = as_float(u.y); v[2] = as_float(u.z); v[3] = as_float(u.w);
+  } else {
+    Raw8<T> r;
+    r.a = u;
+    raw8_widen(r, v);
+  }
+}
 template <typename T, int E> ACTNN_DEV void narrow_chunk(T* p, const float (&v)[E]) {
   if constexpr (E == 4) store16(p, u32x4{as_uint(v[0]), as_uint(v[1]), as_uint(v[2]), as_uint(v[3])});
   else store8(p, v);
 }
 
-template <typename T, bool NIB>
+template <typename T, int PRESET, bool NIB>
 __global__ __launch_bounds__(kThreads) void max_pool2d_forward_cl_kernel(
     const T* __restrict__ x, T* __restrict__ y, int8_t* __restrict__ idx, int64_t chunks, int cpp /* chunks per pixel */,
     int64_t C, PoolGeom g) {
   constexpr int E = PoolChunk<T>::kElems;
-  const int64_t id = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  // (neighbouring output rows share input rows: their blocks stay on one XCD)
+  const int64_t id = xcd_block() * kThreads + threadIdx.x;
   if (id >= chunks) return;
   const int c = (int)(id % cpp) * E;
   const int64_t pix = id / cpp;
@@ -644,14 +659,40 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_forward_cl_kernel(
 #pragma unroll
   for (int e = 0; e < E; ++e) { best[e] = init; where[e] = 0; }
   const T* img = x + n * (int64_t)g.H * g.W * C + c;
-  for (int i = h_start; i < h_end; ++i) {
-    for (int j = w_start; j < w_end; ++j) {
+  if constexpr (PRESET != 0) {
+    // window known at compile time: all its loads are issued before the first comparison (taken one
+    // at a time, as the loop below does, their latencies add up); positions outside the image get the
+    // start value, which never wins the strict compare
+    const Win<PRESET> k(g);
+    constexpr int KH = PRESET == 2 ? 2 : 3, KW = KH;
+    u32x4 raw[KH * KW];
+    const uint32_t fill = dword_of<T>(init);
+#pragma unroll
+    for (int a = 0; a < KH; ++a)
+#pragma unroll
+      for (int b = 0; b < KW; ++b) {
+        const int i = h * k.SH - k.PH + a, j = w * k.SW - k.PW + b;
+        raw[a * KW + b] = (i >= 0 && i < g.H && j >= 0 && j < g.W) ? load16(img + ((int64_t)i * g.W + j) * C)
+                                                                 : u32x4{fill, fill, fill, fill};
+      }
+#pragma unroll
+    for (int q = 0; q < KH * KW; ++q) {
       float v[E];
-      widen_chunk<T, E>(img + ((int64_t)i * g.W + j) * C, v);
-      const int k = (i - h_base) * g.KW + (j - w_base);
+      raw_widen_chunk<T, E>(raw[q], v);
 #pragma unroll
       for (int e = 0; e < E; ++e)
-        if (v[e] > best[e]) { best[e] = v[e]; where[e] = k; }
+        if (v[e] > best[e]) { best[e] = v[e]; where[e] = q; }
+    }
+  } else {
+    for (int i = h_start; i < h_end; ++i) {
+      for (int j = w_start; j < w_end; ++j) {
+        float v[E];
+        widen_chunk<T, E>(img + ((int64_t)i * g.W + j) * C, v);
+        const int k = (i - h_base) * g.KW + (j - w_base);
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+          if (v[e] > best[e]) { best[e] = v[e]; where[e] = k; }
+      }
     }
   }
   narrow_chunk<T, E>(y + pix * C + c, best);
@@ -668,7 +709,7 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_backward_cl_kernel(
     const T* __restrict__ gout, const int8_t* __restrict__ idx, T* __restrict__ gin, int64_t chunks, int cpp,
     int64_t C, PoolGeom g) {
   constexpr int E = PoolChunk<T>::kElems;
-  const int64_t id = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const int64_t id = xcd_block() * kThreads + threadIdx.x;
   if (id >= chunks) return;
   const int c = (int)(id % cpp) * E;
   const int64_t pix = id / cpp;
@@ -714,7 +755,7 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_backward_cl_s2_kernel(
     int64_t C, PoolGeom g) {
   constexpr int E = PoolChunk<T>::kElems;
   constexpr int NWIN = K == 3 ? 2 : 1;
-  const int64_t id = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const int64_t id = xcd_block() * kThreads + threadIdx.x;       // neighbouring block rows share windows
   if (id >= items) return;
   const int c = (int)(id % cpp) * E;
   const int64_t blk = id / cpp;
@@ -770,14 +811,21 @@ int launch_cl(bool forward, const void* a, const int8_t* idx_in, int8_t* idx_out
   const int64_t pixels = forward ? N * g.Ho * g.Wo : N * (int64_t)g.H * g.W;
   const int64_t chunks = pixels * cpp;
   const int64_t blocks = (chunks + kThreads - 1) / kThreads;
-  if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
+  if (blocks > 0x7ffffff0LL) return ACTNN_EINVAL;
   if (blocks == 0) return ACTNN_OK;
   if (forward) {
-    max_pool2d_forward_cl_kernel<T, NIB><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
-        static_cast<const T*>(a), static_cast<T*>(out), idx_out, chunks, cpp, C, g);
+    const dim3 grid(xcd_grid(blocks)), blk(kThreads);
+    const T* xi = static_cast<const T*>(a);
+    T* yo = static_cast<T*>(out);
+    switch (preset_of(g)) {
+      case 1: max_pool2d_forward_cl_kernel<T, 1, NIB><<<grid, blk, 0, s>>>(xi, yo, idx_out, chunks, cpp, C, g); break;
+      case 2: max_pool2d_forward_cl_kernel<T, 2, NIB><<<grid, blk, 0, s>>>(xi, yo, idx_out, chunks, cpp, C, g); break;
+      case 3: max_pool2d_forward_cl_kernel<T, 3, NIB><<<grid, blk, 0, s>>>(xi, yo, idx_out, chunks, cpp, C, g); break;
+      default: max_pool2d_forward_cl_kernel<T, 0, NIB><<<grid, blk, 0, s>>>(xi, yo, idx_out, chunks, cpp, C, g); break;
+    }
   } else if (const int p = preset_of(g); (p == 1 || p == 2) && g.H == 2 * g.Ho && g.W == 2 * g.Wo) {
     const int64_t items = N * g.Ho * g.Wo * cpp;
-    const dim3 grid((unsigned)((items + kThreads - 1) / kThreads)), blk(kThreads);
+    const dim3 grid(xcd_grid((items + kThreads - 1) / kThreads)), blk(kThreads);
     if (p == 1)
       max_pool2d_backward_cl_s2_kernel<T, 3, 1, NIB><<<grid, blk, 0, s>>>(
           static_cast<const T*>(a), idx_in, static_cast<T*>(out), items, cpp, C, g);
@@ -785,7 +833,7 @@ int launch_cl(bool forward, const void* a, const int8_t* idx_in, int8_t* idx_out
       max_pool2d_backward_cl_s2_kernel<T, 2, 0, NIB><<<grid, blk, 0, s>>>(
           static_cast<const T*>(a), idx_in, static_cast<T*>(out), items, cpp, C, g);
   } else {
-    max_pool2d_backward_cl_kernel<T, NIB><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+    max_pool2d_backward_cl_kernel<T, NIB><<<dim3(xcd_grid(blocks)), dim3(kThreads), 0, s>>>(
         static_cast<const T*>(a), idx_in, static_cast<T*>(out), chunks, cpp, C, g);
   }
   ACTNN_RETURN_LAUNCH_STATUS();
