@@ -1391,8 +1391,8 @@ constexpr int kMaxDevices = 64;
 float* g_scratch_of_device[kMaxDevices];          // device address of `scratch`, per device
 std::mutex g_scratch_mutex;
 
-// -> ACTNN_OK and *out = this device's copy of the array, or an error code
-int static_scratch(float** out) {
+// -> ACTNN_OK and *out = the copy of the array on the current device, or an error code
+int static_scratch(float** out, int* device) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return (int)e;
@@ -1406,12 +1406,20 @@ int static_scratch(float** out) {
     g_scratch_of_device[dev] = ptr;
   }
   *out = g_scratch_of_device[dev];
+  *device = dev;
   return ACTNN_OK;
 }
 }  // namespace
 }  // namespace actnn
 
-extern "C" int64_t actnn_batch_norm_forward_static_limit(void) { return actnn::kStaticScratchBytes; }
+// Also the set-up call: it looks up the array's address on the current device, so that a later
+// actnn_batch_norm_forward_static on this device (under graph capture, say) finds it resolved.
+extern "C" int64_t actnn_batch_norm_forward_static_limit(void) {
+  float* ws = nullptr;
+  int dev = -1;
+  (void)actnn::static_scratch(&ws, &dev);          // an error here is reported by the forward call
+  return actnn::kStaticScratchBytes;
+}
 
 extern "C" int actnn_batch_norm_forward_static(const void* x, const float* weight, const float* bias,
                                                float* running_mean, float* running_var, void* y,
@@ -1425,8 +1433,15 @@ extern "C" int actnn_batch_norm_forward_static(const void* x, const float* weigh
   const int64_t need = workspace_floats(pl, C) * (int64_t)sizeof(float);
   if (need > kStaticScratchBytes) return ACTNN_ETOOBIG;
   float* ws = nullptr;
-  const int rc = static_scratch(&ws);
+  int dev = -1;
+  const int rc = static_scratch(&ws, &dev);
   if (rc != ACTNN_OK) return rc;
+  // the array was looked up on the current device: a stream of another GPU would hand that GPU's
+  // kernels an address of this one
+  int stream_dev = -1;
+  const hipError_t e = hipStreamGetDevice(static_cast<hipStream_t>(stream), &stream_dev);
+  if (e != hipSuccess) return (int)e;
+  if (stream_dev != dev) return ACTNN_EINVAL;
   // every partial sum and coefficient the second kernel reads is written by the first ones in this
   // call: nothing in the array has to start at zero
   return actnn_batch_norm_forward(x, weight, bias, running_mean, running_var, y, save_mean, save_invstd, mn,

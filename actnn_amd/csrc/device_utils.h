@@ -74,12 +74,17 @@ ACTNN_DEV void store16_nt(void* p, u32x4 v) { __builtin_nontemporal_store(v, rei
 // (lds_base uniform in the wave).  Written as an instruction sequence of its own: the load is
 // asynchronous and the code that issues it waits for it explicitly (vmcnt) before the data is read; issued through the compiler's builtin, every LDS read that follows - also of
 // another buffer - would first wait for all loads in flight.
+// The statements write m0 and say so in their clobber lists, so that the compiler never assumes a
+// value of its own survives them (it keeps m0 to itself - "reserved" - and warns about any clobber
+// of it; the warning is switched off for these two functions only).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 ACTNN_DEV void load_to_lds16(const void* src, const uint8_t* lds_base) {
   const uint32_t base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)lds_base;
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                :
                : "s"(__builtin_amdgcn_readfirstlane(base)), "v"(src)
-               : "memory");
+               : "memory", "m0");
 }
 // The same with the non-temporal hint, for data that is read once.
 ACTNN_DEV void load_to_lds16_nt(const void* src, const uint8_t* lds_base) {
@@ -87,8 +92,9 @@ ACTNN_DEV void load_to_lds16_nt(const void* src, const uint8_t* lds_base) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt"
                :
                : "s"(__builtin_amdgcn_readfirstlane(base)), "v"(src)
-               : "memory");
+               : "memory", "m0");
 }
+#pragma clang diagnostic pop
 
 // ------------------------------------------------------------------ 8 / 16 contiguous elements
 // load8: 8 consecutive elements starting at p (32-byte aligned for f32, 16 for 16-bit types).

@@ -806,7 +806,10 @@ int launch_cl(bool forward, const void* a, const int8_t* idx_in, int8_t* idx_out
               const PoolGeom& g, hipStream_t s) {
   constexpr int E = PoolChunk<T>::kElems;
   if (C % E != 0 || C / E > 0x7fffffffLL) return ACTNN_EINVAL;
-  if (!aligned16(a) || !aligned16(out) || !aligned16(forward ? idx_out : idx_in)) return ACTNN_EALIGN;
+  // a thread stores or loads the E indices of its chunk as one integer of E * (4 or 8) bits
+  constexpr uintptr_t kIdxAlign = E * (NIB ? 4 : 8) / 8;
+  if (!aligned16(a) || !aligned16(out)) return ACTNN_EALIGN;
+  if (reinterpret_cast<uintptr_t>(forward ? idx_out : idx_in) % kIdxAlign != 0) return ACTNN_EALIGN;
   const int cpp = (int)(C / E);
   const int64_t pixels = forward ? N * g.Ho * g.Wo : N * (int64_t)g.H * g.W;
   const int64_t chunks = pixels * cpp;

@@ -26,23 +26,47 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "config2_minimax_pack_unpack_mixed_f32.txt")
+# the sources pack_mixed_kernel is compiled from: the summary above records their hash, and a
+# summary taken from other sources is not quoted as this build's traffic
+TRAFFIC_SOURCES = ["pack_mixed.hip", "quant_math.h", "device_utils.h"]
+
+
+def kernel_source_hash(names=TRAFFIC_SOURCES):
+    """sha256 over the named files of actnn_amd/csrc, in order (first 16 hex digits)."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in names:
+        with open(os.path.join(ROOT, "actnn_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def measured_traffic(kernel_name, path=TRAFFIC_SUMMARY):
     """HBM bytes per launch of `kernel_name` as measured with rocprofv3 --pmc (FETCH_SIZE, then
     WRITE_SIZE, each scaled by what the same counter reads for actnn_stream_copy of a known size):
     read from the table of the committed summary (columns: kernel, FETCH_SIZE, WRITE_SIZE, HBM
-    bytes, algorithmic bytes, ratio).  -> (bytes or None, algorithmic bytes the measurement was
-    taken against or None)."""
+    bytes, algorithmic bytes, ratio).  The summary names the hash of the sources it was measured on
+    (a line `source_hash: ...`); when the sources have changed since, the figure is stale and not
+    reported.  -> (bytes or None, algorithmic bytes the measurement was taken against or None,
+    note or None)."""
+    found, recorded = (None, None), None
     try:
         with open(path) as f:
             for line in f:
                 parts = line.split()
+                if len(parts) == 2 and parts[0] == "source_hash:":
+                    recorded = parts[1]
                 if len(parts) == 6 and parts[0] == kernel_name:
-                    return int(parts[3]), int(parts[4])
+                    found = (int(parts[3]), int(parts[4]))
     except (OSError, ValueError):
         pass
-    return None, None
+    if found[0] is None:
+        return None, None, "no counter summary for this kernel"
+    current = kernel_source_hash()
+    if recorded != current:
+        return None, None, (f"stale: the summary was measured on sources {recorded}, these are {current} "
+                            "- profile again")
+    return found[0], found[1], None
 
 
 WARM_MS = 25.0      # the first ~20 ms of work after an idle spell run up to 7 % slower than the steady state
@@ -378,6 +402,35 @@ def config2_kernel_times(xg, mn, mx, bits, ab, reps):
     return kernels, pair
 
 
+def kernels_in_step(xg, bits, ab, steps):
+    """The three kernels timed where the headline runs them - inside the minimax -> pack -> unpack
+    loop, each launch between two HIP events of its own - beside the back-to-back figures of
+    `kernels`: every kernel then starts on caches and translations the kernel before it left.
+    Median over the steps."""
+    import torch
+    import actnn_amd.cpp_extension.minimax as ext_minimax
+    import actnn_amd.cpp_extension.quantization as ext_q
+    N, G, gs = xg.shape
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
+    for warm in (True, False):
+        for m in marks:
+            m[0].record()
+            lo, hi = ext_minimax.minimax(xg.view(-1, gs))
+            m[1].record()
+            packed, scale = ext_q.pack_mixed_precision(xg, lo.view(N, G, 1), hi.view(N, G, 1), bits, True)
+            m[2].record()
+            ext_q.unpack_mixed_precision(packed, bits, scale, lo.view(N, G, 1), N, G, gs)
+            m[3].record()
+        torch.cuda.synchronize()
+    out = {}
+    for i, name in enumerate(("minimax", "pack_mixed", "unpack_mixed")):
+        t = sorted(m[i].elapsed_time(m[i + 1]) for m in marks)[steps // 2]
+        out[name] = {"ms": round(t, 4), "GB/s": round(ab[name] / t / 1e6, 1),
+                     "frac": round(ab[name] / t / 1e6 / HBM_PEAK_GBS, 4)}
+    out["note"] = "median over %d steps; the interval between two events includes the launch gap" % steps
+    return out
+
+
 def _heartbeat(period=30.0):
     """Progress lines on stderr while the long legs run (MIOpen's solver search during the first
     ResNet-50 step is silent for minutes); stdout stays the single JSON line."""
@@ -495,11 +548,12 @@ def main():
     value = step_bytes / ms_per_step / 1e6
 
     dom = "pack_mixed"
-    traffic, traffic_alg = measured_traffic("pack_mixed_kernel")
+    traffic, traffic_alg, traffic_note = measured_traffic("pack_mixed_kernel")
     roofline = {"bound": "hbm", "kernel": dom, "achieved": kernels[dom]["GB/s"], "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": kernels[dom]["frac"], "traffic": traffic,
                 "traffic_source": "profiles/" + os.path.basename(TRAFFIC_SUMMARY) +
-                                  (f" (measured against {traffic_alg} algorithmic bytes)" if traffic_alg else "")}
+                                  (f" (measured against {traffic_alg} algorithmic bytes)" if traffic_alg
+                                   else f" ({traffic_note})")}
 
     result = {
         "metric": "pack+unpack GB/s & % HBM peak at avg 2-bit; R50 L3 train images/sec",
@@ -518,30 +572,38 @@ def main():
         "kernels": kernels,
         "minimax_plus_pack": pair,
     }
+    result["kernels_in_step"] = kernels_in_step(xg, bits, ab, min(args.steps, 100))
     del xg, mn, mx, bits
     torch.cuda.empty_cache()
-    if not args.skip_extra:
-        xs, mns, mxs, bits_s, bits_s_host = make_config2(device, sample_spread=0.7)
-        avg_s = float(bits_s_host.float().mean())
-        ks, pair_s = config2_kernel_times(xs, mns, mxs, bits_s, algorithmic_bytes(n, 4, avg_s), reps)
-        result["kernels_mixed_spread"] = {"widths": _width_histogram(bits_s_host), "avg_bits": round(avg_s, 3),
-                                          "kernels": ks, "minimax_plus_pack": pair_s}
-        del xs, mns, mxs, bits_s
-        torch.cuda.empty_cache()
-        try:
-            result["other_configs"] = other_configs(device, max(10, args.steps // 2))
-        except Exception as e:                       # keep the headline line even if an extra fails
-            result["other_configs"] = {"error": repr(e)}
-        try:
-            import bench_extra
-            result.update(bench_extra.run(device))
-        except ImportError:
-            pass
-        except Exception as e:
-            result["extra_error"] = repr(e)
     if not args.skip_cpu:
         result["cpu_baseline"] = cpu_baseline(device=device)
-    print(json.dumps(result))
+    if args.skip_extra:
+        print(json.dumps(result), flush=True)
+        return
+    # the headline is complete here: print it now, so that nothing that follows (the first
+    # ResNet-50 steps spend minutes in the convolution library's solver search) can lose it; the
+    # extended line printed at the end repeats it with the other configurations added
+    print(json.dumps(dict(result, partial="headline only; the extended line follows at the end of the run")),
+          flush=True)
+    xs, mns, mxs, bits_s, bits_s_host = make_config2(device, sample_spread=0.7)
+    avg_s = float(bits_s_host.float().mean())
+    ks, pair_s = config2_kernel_times(xs, mns, mxs, bits_s, algorithmic_bytes(n, 4, avg_s), reps)
+    result["kernels_mixed_spread"] = {"widths": _width_histogram(bits_s_host), "avg_bits": round(avg_s, 3),
+                                      "kernels": ks, "minimax_plus_pack": pair_s}
+    del xs, mns, mxs, bits_s
+    torch.cuda.empty_cache()
+    try:
+        result["other_configs"] = other_configs(device, max(10, args.steps // 2))
+    except Exception as e:                       # keep the headline line even if an extra fails
+        result["other_configs"] = {"error": repr(e)}
+    try:
+        import bench_extra
+        result.update(bench_extra.run(device))
+    except ImportError:
+        pass
+    except Exception as e:
+        result["extra_error"] = repr(e)
+    print(json.dumps(result), flush=True)
 
 
 if __name__ == "__main__":

@@ -148,9 +148,11 @@ int actnn_max_pool2d_backward(const void* grad_out, const int8_t* idx, void* gra
                               int64_t C, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH,
                               int KW, int SH, int SW, int PH, int PW, int dtype, void* stream);
 /* The same two operators on channels-last tensors: x, y, idx and the gradients are laid out
- * [N, H, W, C] / [N, Ho, Wo, C] (C a multiple of 4 for f32, 8 for 16-bit types; 16-byte aligned
- * pointers).  Values and indices equal those of the default-layout operators on the transposed
- * tensors. */
+ * [N, H, W, C] / [N, Ho, Wo, C] (C a multiple of 4 for f32, 8 for 16-bit types; x, y and the
+ * gradients 16-byte aligned; idx aligned to the indices of one 16-byte chunk of channels: 4 bytes
+ * for f32, 8 bytes for 16-bit types - half of that for the two-per-byte format below;
+ * ACTNN_EALIGN otherwise).  Values and indices equal those of the default-layout operators on the
+ * transposed tensors. */
 int actnn_max_pool2d_forward_cl(const void* x, void* y, int8_t* idx, int64_t N, int64_t C,
                                 int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH, int KW,
                                 int SH, int SW, int PH, int PW, int dtype, void* stream);
@@ -162,7 +164,9 @@ int actnn_max_pool2d_backward_cl(const void* grad_out, const int8_t* idx, void* 
  * (quantization.cc:162): output o of the flat order of y (default layout: [N, C, Ho, Wo];
  * channels-last: [N, Ho, Wo, C]) is stored in bits 4 * (o & 1) .. 4 * (o & 1) + 3 of byte
  * o / 2; idx holds (N * C * Ho * Wo + 1) / 2 bytes and the unused half of the last byte of an
- * odd count is written as 0.  Values, indices and gradients equal those of the int8 operators. */
+ * odd count is written as 0.  Values, indices and gradients equal those of the int8 operators.
+ * Default layout: idx needs no alignment (16-byte aligned pointers take the faster kernels);
+ * channels-last: 2 bytes for f32, 4 bytes for 16-bit types. */
 int actnn_max_pool2d_forward_nibble(const void* x, void* y, uint8_t* idx, int64_t N, int64_t C,
                                     int64_t H, int64_t W, int64_t Ho, int64_t Wo, int KH, int KW,
                                     int SH, int SW, int PH, int PW, int dtype, void* stream);
@@ -286,7 +290,12 @@ int64_t actnn_batch_norm_backward_sumsq_entries(int64_t N, int64_t C, int64_t HW
  * actnn_batch_norm_workspace_bytes exceeds it is rejected with ACTNN_ETOOBIG.  Calls no hipMalloc,
  * hipFree or other allocating routine.  Results are bit-identical to actnn_batch_norm_forward.
  * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different
- * streams or threads) race; calls on one stream are ordered and safe. */
+ * streams or threads) race; calls on one stream are ordered and safe.  `stream` must belong to the
+ * current device (ACTNN_EINVAL otherwise: the array is looked up on the current device).
+ * actnn_batch_norm_forward_static_limit() doubles as the set-up call: it resolves the array's
+ * address on the current device (hipGetSymbolAddress, once per device); call it once per GPU, with
+ * that GPU current, before the first forward call that runs under graph capture - a forward call on
+ * a device that was not set up resolves the address itself, outside capture only. */
 int64_t actnn_batch_norm_forward_static_limit(void);
 int actnn_batch_norm_forward_static(const void* x, const float* weight, const float* bias,
                                     float* running_mean, float* running_var, void* y,

@@ -11,7 +11,7 @@ import torch
 
 import actnn_amd.cpp_extension.quantization as ext_q
 from oracle import kernel_mode, layouts, simulate
-from _util import DEV, bits_tensor, make_groups, minmax_dev, np_bits, ulp_diff_f32
+from _util import DEV, assert_rng_tier, bits_tensor, make_groups, minmax_dev, np_bits, ulp_diff_f32
 
 pytestmark = pytest.mark.gpu
 
@@ -139,6 +139,21 @@ def test_rng_mode_unbiased_with_closed_form_variance(bits):
     # ActNN's bound: per-element variance <= R^2 / (4 B^2)   (qscheme.py:84)
     B = 2 ** bits - 1
     assert (out64.var(axis=0) <= (rng_ ** 2) / (4 * B * B) * 1.1 + 1e-12).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bits", [1, 2, 3, 4, 5, 6, 7, 8])
+def test_rng_mode_criterion_on_every_dtype_and_width(dtype, bits):
+    # 10^4 roundings of the same 4 groups; the codes are read back with the unpack kernel itself
+    # (scale 1, min 0 in fp32: code / 1 + 0 is the code)
+    trials, G = 10_000, 4
+    base, _ = make_groups(1, G, 256, dtype, 70 + bits, "chan")
+    x = base.expand(trials, G, 256).contiguous()
+    xd, mn, mx, bits_dev, bits_host, packed, scale, seed, offset = _rng_pack(x, [bits] * trials, 31 + bits)
+    ones = torch.ones(trials, G, 1, device=DEV)
+    codes = ext_q.unpack_mixed_precision(packed, bits_dev, ones, torch.zeros_like(ones), trials, G, 256)
+    assert codes.dtype == torch.float32 and float(codes.max()) <= 2 ** bits - 1 and float(codes.min()) >= 0
+    assert_rng_tier(base, bits, codes, mn, scale)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])

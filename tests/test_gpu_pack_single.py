@@ -5,7 +5,7 @@ import torch
 
 import actnn_amd.cpp_extension.quantization as ext_q
 from oracle import kernel_mode, layouts, simulate
-from _util import DEV, make_groups, minmax_dev, np_bits, ulp_diff_f32
+from _util import DEV, assert_rng_tier, make_groups, minmax_dev, np_bits, ulp_diff_f32
 
 pytestmark = pytest.mark.gpu
 
@@ -56,6 +56,21 @@ def test_rng_mode_matches_kernel_model(bits, gs, dtype):
     assert np.array_equal(packed.cpu().numpy()[:live], ref[:live])
     out = ext_q.unpack_single_precision(packed, bits, scale, mn, N, G, gs)
     assert np.array_equal(np_bits(out), np_bits(kernel_mode.kernel_dequant(codes, scale_o, mn.cpu())))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+def test_rng_mode_criterion_on_every_dtype_and_width(dtype, bits):
+    # 10^4 roundings of the same 4 groups, codes read back with the unpack kernel (scale 1, min 0)
+    trials, G = 10_000, 4
+    base, _ = make_groups(1, G, 256, dtype, 40 + bits, "chan")
+    xd = base.expand(trials, G, 256).contiguous().to(DEV)
+    mn, mx = minmax_dev(xd)
+    packed, scale = ext_q.pack_single_precision(xd, mn, mx, bits, True)
+    ones = torch.ones(trials, G, 1, device=DEV)
+    codes = ext_q.unpack_single_precision(packed, bits, ones, torch.zeros_like(ones), trials, G, 256)
+    assert codes.dtype == torch.float32
+    assert_rng_tier(base, bits, codes, mn, scale)
 
 
 def test_rng_mode_unbiased():

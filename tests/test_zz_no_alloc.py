@@ -61,6 +61,31 @@ def test_static_scratch_forward_matches_workspace_forward(dtype, channels_last):
             assert torch.equal(a, e)
 
 
+def test_static_scratch_forward_allocates_nothing():
+    lib = _lib.load()
+    assert lib.actnn_batch_norm_forward_static_limit() > 0         # the set-up call resolves the array
+    N, C, H = 32, 128, 14
+    x = torch.randn(N, C, H, H, device=DEV).to(torch.bfloat16)
+    w, b = torch.rand(C, device=DEV) + 0.5, torch.randn(C, device=DEV)
+    y, mean, invstd = torch.empty_like(x), torch.empty(C, device=DEV), torch.empty(C, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def call():
+        return lib.actnn_batch_norm_forward_static(
+            x.data_ptr(), w.data_ptr(), b.data_ptr(), None, None, y.data_ptr(), mean.data_ptr(),
+            invstd.data_ptr(), None, None, N, C, H * H, 0.1, 1e-5, 2, 0, stream)
+    assert call() == 0
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    torch_alloc0, torch_reserved0 = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    for _ in range(10):
+        assert call() == 0
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0                                           # no device memory taken from the driver
+    assert torch.cuda.memory_allocated() == torch_alloc0 and torch.cuda.memory_reserved() == torch_reserved0
+
+
 def test_static_scratch_rejects_what_does_not_fit():
     lib = _lib.load()
     limit = lib.actnn_batch_norm_forward_static_limit()
