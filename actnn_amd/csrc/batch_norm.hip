@@ -764,14 +764,21 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
 // 512 bytes.  With C % 256 == 0 or 256 % C == 0 a quantisation group (256 consecutive elements)
 // is an aligned run of 256 / E threads, as in the default layout, so the group min/max and the
 // decoding of a packed input carry over unchanged.
-template <typename T> struct PlainRows {
+// A thread's row is `rb + r`: rb is the same for the whole block (a scalar: the loads then take a
+// scalar base and a lane offset that never changes, so no per-load address arithmetic and no address
+// registers), r is the thread's row inside one iteration.
+template <typename T, bool NT = false> struct PlainRows {
   static constexpr bool kRows = true;
   static constexpr int kInFlight = 4;
-  const T* p;            // offset to the thread's columns of row 0 once bound
+  const T* p;
   int64_t C;
+  uint32_t lane_bytes;   // (r * C + col) * sizeof(T) once bound
   struct Raw { u32x4 v; };
-  ACTNN_DEV void bind(int64_t col, int64_t) { p += col; }
-  ACTNN_DEV Raw fetch(int64_t row) const { return Raw{load16(p + row * C)}; }
+  ACTNN_DEV void bind(int64_t col, int r) { lane_bytes = (uint32_t)(((int64_t)r * C + col) * (int64_t)sizeof(T)); }
+  ACTNN_DEV Raw fetch(int64_t rb) const {
+    const char* q = reinterpret_cast<const char*>(p) + rb * C * (int64_t)sizeof(T) + lane_bytes;
+    return Raw{NT ? load16_nt(q) : load16(q)};
+  }
   ACTNN_DEV u32x4 decode(const Raw& r) const { return r.v; }
 };
 template <typename T> struct PackedRows {
@@ -781,8 +788,10 @@ template <typename T> struct PackedRows {
   int64_t C, col;
   uint32_t HW;
   using Raw = typename PackedInput<T>::Raw;
-  ACTNN_DEV void bind(int64_t column, int64_t) {
+  int r;
+  ACTNN_DEV void bind(int64_t column, int row_in_iteration) {
     col = column;
+    r = row_in_iteration;
     in.lane32 = threadIdx.x & (PackedInput<T>::kLanes - 1);
     in.active = true;
     cur_row0 = -(int64_t)HW - 1;                           // no row is inside: the first fetch looks up
@@ -793,7 +802,8 @@ template <typename T> struct PackedRows {
   uint32_t cur_n;        // sample of the last fetch; cur_row0 = cur_n * HW
   int cur_b;
   int64_t cur_first, cur_row0;
-  ACTNN_DEV Raw fetch(int64_t row) {
+  ACTNN_DEV Raw fetch(int64_t rb) {
+    const int64_t row = rb + r;
     if ((uint64_t)(row - cur_row0) >= HW) {                // left the sample (or the first fetch)
       cur_n = (uint32_t)row / HW;                          // rows < 2^31 (checked by the launcher)
       cur_row0 = (int64_t)cur_n * HW;
@@ -821,8 +831,13 @@ template <int E> ACTNN_DEV RowTile row_tile(int64_t C, int tpr, int R) {
   return t;
 }
 
-template <typename T, bool BWD, bool MINMAX, typename XS>
-__global__ __launch_bounds__(kThreads, 5) void bn_cl_reduce_kernel(
+// Waves per SIMD the reduce pass is compiled for: the plain statistics pass fits 8 (64 registers),
+// with the group min/max or the gradient 7, with the decoder of a packed input 5.
+template <bool BWD, bool MINMAX, typename XS> constexpr int cl_reduce_waves() {
+  return XS::kInFlight == 2 ? 5 : (BWD || MINMAX) ? 7 : 8;
+}
+template <typename T, bool BWD, bool MINMAX, bool NT, typename XS>
+__global__ __launch_bounds__(kThreads, (cl_reduce_waves<BWD, MINMAX, XS>())) void bn_cl_reduce_kernel(
     XS xs, const T* __restrict__ dy, float* __restrict__ part, T* __restrict__ mn, T* __restrict__ mx,
     int64_t P, int64_t C, int tpr, int R, int64_t ppb) {
   constexpr int E = Chunk<T>::kElems;
@@ -830,15 +845,21 @@ __global__ __launch_bounds__(kThreads, 5) void bn_cl_reduce_kernel(
   constexpr int U = XS::kInFlight;
   __shared__ float s_part[kThreads * 2 * E];
   const RowTile t = row_tile<E>(C, tpr, R);
-  xs.bind(t.col, C);
-  const T* pd = BWD ? dy + t.col : nullptr;
+  xs.bind(t.col, t.r);
   const int64_t p0 = (int64_t)blockIdx.y * ppb;
   const int64_t p1 = p0 + ppb < P ? p0 + ppb : P;
+  // everything a lane adds to the block's (scalar) position: bytes into dy, groups into mn / mx
+  const uint32_t lane_bytes = (uint32_t)(((int64_t)t.r * C + t.col) * (int64_t)sizeof(T));
+  const uint32_t lane_group = (uint32_t)(((int64_t)t.r * C + t.col) >> 8);
+  auto dy_at = [&](int64_t rb) -> u32x4 {
+    const char* q = reinterpret_cast<const char*>(dy) + rb * C * (int64_t)sizeof(T) + lane_bytes;
+    return NT ? load16_nt(q) : load16(q);
+  };
   float s[E], q[E];
 #pragma unroll
   for (int i = 0; i < E; ++i) { s[i] = 0.0f; q[i] = 0.0f; }
 
-  auto accumulate = [&](const u32x4& ux, const u32x4& ud, int64_t row) {
+  auto accumulate = [&](const u32x4& ux, const u32x4& ud, int64_t rb) {
     const uint32_t w[4] = {ux.x, ux.y, ux.z, ux.w};
     const uint32_t d[4] = {ud.x, ud.y, ud.z, ud.w};
     float v[E], g[E];
@@ -861,33 +882,38 @@ __global__ __launch_bounds__(kThreads, 5) void bn_cl_reduce_kernel(
       lo = rows_min<LPG / 16>(row16_min(lo));
       hi = rows_max<LPG / 16>(row16_max(hi));
       if ((threadIdx.x & (LPG - 1)) == LPG - 1) {
-        const int64_t g_index = (row * C + t.col) >> 8;
-        Conv<T>::store(mn, g_index, lo);
-        Conv<T>::store(mx, g_index, hi);
+        // rb * C is a multiple of 256 (rb a multiple of R, and R * C of 256, wherever groups align)
+        T* lo_at = mn + ((rb * C) >> 8) + lane_group;
+        T* hi_at = mx + ((rb * C) >> 8) + lane_group;
+        Conv<T>::store(lo_at, 0, lo);
+        Conv<T>::store(hi_at, 0, hi);
       }
     }
   };
 
   if (t.active) {
-    int64_t row = p0 + t.r;
-    for (; row + (int64_t)(U - 1) * R < p1; row += (int64_t)U * R) {
+    int64_t rb = p0;
+    // whole iterations: every row rb + u * R + r of the U loads lies below p1
+    for (; rb + (int64_t)U * R <= p1; rb += (int64_t)U * R) {
       typename XS::Raw rx[U];
       u32x4 ud[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        rx[u] = xs.fetch(row + (int64_t)u * R);
-        if (BWD) ud[u] = load16(pd + (row + (int64_t)u * R) * C);
+        rx[u] = xs.fetch(rb + (int64_t)u * R);
+        if (BWD) ud[u] = dy_at(rb + (int64_t)u * R);
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const u32x4 ux = xs.decode(rx[u]);
-        accumulate(ux, BWD ? ud[u] : ux, row + (int64_t)u * R);
+        accumulate(ux, BWD ? ud[u] : ux, rb + (int64_t)u * R);
       }
     }
-    for (; row < p1; row += R) {
-      const typename XS::Raw rx = xs.fetch(row);
-      const u32x4 ux = xs.decode(rx);
-      accumulate(ux, BWD ? load16(pd + row * C) : ux, row);
+    for (; rb < p1; rb += R) {
+      if (rb + t.r < p1) {
+        const typename XS::Raw rx = xs.fetch(rb);
+        const u32x4 ux = xs.decode(rx);
+        accumulate(ux, BWD ? dy_at(rb) : ux, rb);
+      }
     }
   }
   // rows of the tile are folded in a fixed order; table: [channel][sum][block row]
@@ -932,7 +958,7 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
   float sumsq = 0.0f;
   if (!BWD && !t.active) return;       // whole quantisation groups leave together
   if (t.active) {                      // (backward: the lanes meet again for the wave's sum below)
-  xs.bind(t.col, C);
+  xs.bind(t.col, t.r);
   float ka[E], kb[E], kc[E];
 #pragma unroll
   for (int i = 0; i < E; ++i) {
@@ -963,23 +989,34 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
     return u32x4{r[0], r[1], r[2], r[3]};
   };
 
-  const T* pd = BWD ? dy + t.col : nullptr;
-  T* po = out + t.col;
+  // row rb + t.r of dy / out: a scalar base (rb is the same for the whole block) plus the lane's bytes
+  const uint32_t lane_bytes = (uint32_t)(((int64_t)t.r * C + t.col) * (int64_t)sizeof(T));
+  auto dy_at = [&](int64_t rb) -> u32x4 {
+    return load_last(reinterpret_cast<const char*>(dy) + rb * C * (int64_t)sizeof(T) + lane_bytes);
+  };
+  auto out_at = [&](int64_t rb) -> void* {
+    return reinterpret_cast<char*>(out) + rb * C * (int64_t)sizeof(T) + lane_bytes;
+  };
+  // Position of the lane's chunk of row ru + t.r (ru the same for the whole block) in elements:
+  // ru * C + lane_elems.  ru is a multiple of R and R * C of 256 wherever groups align, so the
+  // octet and the group of the chunk are a scalar part plus a part that never changes.
+  const uint32_t lane_elems = (uint32_t)((int64_t)t.r * C + t.col);
   if constexpr (PACK && sizeof(T) == 4) {
     // fp32: 64 steps at a time (the wave's 64 lanes own the group), rows packed two by two
     const int lane = threadIdx.x & 63;
     ParamQueue<T> queue;
-    auto params = [&](int64_t row, int jq) {
-      locate(row);
+    auto params = [&](int64_t ru, int jq) {
+      locate(ru + t.r);
       ChunkParams q;
       queue.get(jq, q.mul, q.sub);
       q.b = cur_b;
-      const int64_t flat = row * C + t.col;
-      q.dst = ps.packed + cur_first + ((flat >> 8) - (int64_t)cur_n * ps.G) * q.b * 8;
-      q.octet = (uint64_t)(flat >> 3);
+      const int64_t grp = ((ru * C) >> 8) + (lane_elems >> 8);
+      q.dst = ps.packed + cur_first + (grp - (int64_t)cur_n * ps.G) * q.b * 8;
+      q.octet = (uint64_t)((ru * C) >> 3) + (lane_elems >> 3);
       return q;
     };
-    for (int64_t rb = p0 + t.r; rb < p1; rb += (int64_t)64 * R) {
+    for (int64_t rb0 = p0; rb0 + t.r < p1; rb0 += (int64_t)64 * R) {
+      const int64_t rb = rb0 + t.r;
       {
         const int64_t rj = rb + (int64_t)lane * R;
         const bool live = rj < p1;
@@ -988,20 +1025,20 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
       }
       int j = 0;
       for (; j + 2 <= 64 && rb + (int64_t)(j + 1) * R < p1; j += 2) {
-        const int64_t r0 = rb + (int64_t)j * R, r1 = r0 + R;
-        const typename XS::Raw rx0 = xs.fetch(r0), rx1 = xs.fetch(r1);
+        const int64_t ru0 = rb0 + (int64_t)j * R, ru1 = ru0 + R;
+        const typename XS::Raw rx0 = xs.fetch(ru0), rx1 = xs.fetch(ru1);
         const u32x4 ux0 = xs.decode(rx0), ux1 = xs.decode(rx1);
-        store_out(po + r0 * C, apply(ux0, ux0));
-        store_out(po + r1 * C, apply(ux1, ux1));
-        const ChunkParams qa = params(r0, j);
-        const ChunkParams qb = params(r1, j + 1);
+        store_out(out_at(ru0), apply(ux0, ux0));
+        store_out(out_at(ru1), apply(ux1, ux1));
+        const ChunkParams qa = params(ru0, j);
+        const ChunkParams qb = params(ru1, j + 1);
         pack_chunk_pair_f32(ps, ux0, qa, ux1, qb, true);
       }
       if (j < 64 && rb + (int64_t)j * R < p1) {
-        const int64_t r0 = rb + (int64_t)j * R;
-        const u32x4 ux = xs.decode(xs.fetch(r0));
-        store_out(po + r0 * C, apply(ux, ux));
-        const ChunkParams q = params(r0, j);
+        const int64_t ru0 = rb0 + (int64_t)j * R;
+        const u32x4 ux = xs.decode(xs.fetch(ru0));
+        store_out(out_at(ru0), apply(ux, ux));
+        const ChunkParams q = params(ru0, j);
         pack_chunk_pair_f32(ps, ux, q, ux, q, false);
       }
     }
@@ -1011,13 +1048,14 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
     // their noise
     const int lane32 = threadIdx.x & 31;
     ParamQueue<T> queue;
-    auto pack_one = [&](const u32x4& ux, const uint32_t (&rw)[Noise<T>::kWords], int64_t row, int j) {
-      locate(row);
+    auto pack_one = [&](const u32x4& ux, const uint32_t (&rw)[Noise<T>::kWords], int64_t ru, int j) {
+      locate(ru + t.r);
       float mul, sub;
       queue.get(j, mul, sub);
-      pack_chunk<T>(ps, ux, rw, mul, sub, ((row * C + t.col) >> 8) - (int64_t)cur_n * ps.G, cur_b, cur_first);
+      pack_chunk<T>(ps, ux, rw, mul, sub, ((ru * C) >> 8) + (lane_elems >> 8) - (int64_t)cur_n * ps.G, cur_b, cur_first);
     };
-    for (int64_t rb = p0 + t.r; rb < p1; rb += (int64_t)32 * R) {
+    for (int64_t rb0 = p0; rb0 + t.r < p1; rb0 += (int64_t)32 * R) {
+      const int64_t rb = rb0 + t.r;
       {
         const int64_t rj = rb + (int64_t)lane32 * R;
         const bool live = rj < p1;
@@ -1026,47 +1064,49 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
       }
       int j = 0;
       for (; j + 2 <= 32 && rb + (int64_t)(j + 1) * R < p1; j += 2) {
-        const int64_t r0 = rb + (int64_t)j * R, r1 = r0 + R;
-        const typename XS::Raw rx0 = xs.fetch(r0), rx1 = xs.fetch(r1);
+        const int64_t ru0 = rb0 + (int64_t)j * R, ru1 = ru0 + R;
+        const typename XS::Raw rx0 = xs.fetch(ru0), rx1 = xs.fetch(ru1);
         uint32_t rw[2][Noise<T>::kWords];
-        noise_pair<T>(ps, (uint64_t)((r0 * C + t.col) >> 3), (uint64_t)((r1 * C + t.col) >> 3), rw[0], rw[1],
-                      (tpr & 1) == 0);      // lane ^ 1 is in the same row, hence in the same steps
+        noise_pair<T>(ps, (uint64_t)((ru0 * C) >> 3) + (lane_elems >> 3), (uint64_t)((ru1 * C) >> 3) + (lane_elems >> 3),
+                      rw[0], rw[1], (tpr & 1) == 0);      // lane ^ 1 is in the same row, hence in the same steps
         const u32x4 ux0 = xs.decode(rx0);
-        store_out(po + r0 * C, apply(ux0, ux0));
-        pack_one(ux0, rw[0], r0, j);
+        store_out(out_at(ru0), apply(ux0, ux0));
+        pack_one(ux0, rw[0], ru0, j);
         const u32x4 ux1 = xs.decode(rx1);
-        store_out(po + r1 * C, apply(ux1, ux1));
-        pack_one(ux1, rw[1], r1, j + 1);
+        store_out(out_at(ru1), apply(ux1, ux1));
+        pack_one(ux1, rw[1], ru1, j + 1);
       }
       for (; j < 32 && rb + (int64_t)j * R < p1; ++j) {
-        const int64_t r0 = rb + (int64_t)j * R;
-        const u32x4 ux = xs.decode(xs.fetch(r0));
-        store_out(po + r0 * C, apply(ux, ux));
+        const int64_t ru0 = rb0 + (int64_t)j * R;
+        const u32x4 ux = xs.decode(xs.fetch(ru0));
+        store_out(out_at(ru0), apply(ux, ux));
         uint32_t rw[Noise<T>::kWords];
-        Noise<T>::octet((uint64_t)((r0 * C + t.col) >> 3), ps.seed, ps.offset, rw);
-        pack_one(ux, rw, r0, j);
+        Noise<T>::octet((uint64_t)((ru0 * C) >> 3) + (lane_elems >> 3), ps.seed, ps.offset, rw);
+        pack_one(ux, rw, ru0, j);
       }
     }
   } else {
-  int64_t row = p0 + t.r;
-  for (; row + (int64_t)(U - 1) * R < p1; row += (int64_t)U * R) {
+  int64_t rb = p0;
+  for (; rb + (int64_t)U * R <= p1; rb += (int64_t)U * R) {
     typename XS::Raw rx[U];
     u32x4 ud[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      rx[u] = xs.fetch(row + (int64_t)u * R);
-      if (BWD) ud[u] = load_last(pd + (row + (int64_t)u * R) * C);
+      rx[u] = xs.fetch(rb + (int64_t)u * R);
+      if (BWD) ud[u] = dy_at(rb + (int64_t)u * R);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const u32x4 ux = xs.decode(rx[u]);
-      store_out(po + (row + (int64_t)u * R) * C, apply(ux, BWD ? ud[u] : ux));
+      store_out(out_at(rb + (int64_t)u * R), apply(ux, BWD ? ud[u] : ux));
     }
   }
-  for (; row < p1; row += R) {
-    const typename XS::Raw rx = xs.fetch(row);
-    const u32x4 ux = xs.decode(rx);
-    store_out(po + row * C, apply(ux, BWD ? load_last(pd + row * C) : ux));
+  for (; rb < p1; rb += R) {
+    if (rb + t.r < p1) {
+      const typename XS::Raw rx = xs.fetch(rb);
+      const u32x4 ux = xs.decode(rx);
+      store_out(out_at(rb), apply(ux, BWD ? dy_at(rb) : ux));
+    }
   }
   }
   }
@@ -1087,7 +1127,12 @@ struct Plan {
   int nsplit_apply;
   int tiles, tpr, R;
   bool groups_align;   // quantisation groups are aligned runs of threads
+  bool big;            // the tensor does not fit the last-level cache: a pass finds nothing of it there
 };
+// The memory-side cache holds 256 MiB.  A tensor above that is gone from it by the time the next pass
+// starts, so the passes that only read may use non-temporal loads (7.0 against 6.1 TB/s on a plain
+// read); a smaller one is found there by the next pass, and non-temporal loads would lose that.
+constexpr int64_t kLastLevelCacheBytes = (int64_t)256 << 20;
 bool make_plan_cl(int64_t N, int64_t C, int64_t HW, int dtype, Plan& pl) {
   if (N <= 0 || C <= 0 || HW <= 0 || dtype < 0 || dtype > 2) return false;
   pl.channels_last = true;
@@ -1098,10 +1143,12 @@ bool make_plan_cl(int64_t N, int64_t C, int64_t HW, int dtype, Plan& pl) {
   pl.tiles = (int)((C + 255) / 256);
   pl.tpr = (int)((C < 256 ? C : 256) / pl.elems);
   pl.R = kThreads / pl.tpr;
-  // One or two rounds of blocks (2048 fit on the chip at once) measured best here: the block's
-  // final reduction over its R rows is dearer than in the default layout.  At least 64 rows per
-  // block keep the table of partial sums below 6 % of the data.
-  constexpr int64_t target = 4096, min_ppb = 64;
+  // About one round of blocks (7 or 8 of them fit a CU): what a block leaves in the table of partial
+  // sums is still in the caches when the kernel ends and is written back then, at a fraction of the
+  // streaming rate (measured on a plain read of 822 MB with such an epilogue: 4 MB of partial sums
+  // cost 7 us, 8 MB 11 us, 16 MB 18 us), so fewer, longer blocks win: 2048 blocks measured 4 % faster
+  // than 4096 over ResNet-50's shapes.  At least 64 rows per block.
+  constexpr int64_t target = 2048, min_ppb = 64;
   const int64_t want = (target + pl.tiles - 1) / pl.tiles;
   int64_t ppb = (pl.P + want - 1) / want;
   if (ppb < min_ppb) ppb = min_ppb;
@@ -1123,6 +1170,7 @@ bool make_plan_cl(int64_t N, int64_t C, int64_t HW, int dtype, Plan& pl) {
   pl.split = false;
   pl.part_floats = C * 2 * pl.nsplit;
   pl.groups_align = pl.F % 256 == 0 && (C % 256 == 0 || 256 % C == 0);
+  pl.big = N * pl.F * (dtype == ACTNN_F32 ? 4 : 2) > kLastLevelCacheBytes;
   pl.L = 0; pl.spans = 0; pl.per_block = 0;
   return true;
 }
@@ -1155,6 +1203,7 @@ bool make_plan(int64_t N, int64_t C, int64_t HW, int dtype, Plan& pl) {
   pl.split = HW % pl.elems != 0;
   pl.part_floats = pl.spans * nsplit * slots * 2;
   pl.groups_align = pl.F % 256 == 0;
+  pl.big = N * pl.F * (dtype == ACTNN_F32 ? 4 : 2) > kLastLevelCacheBytes;
   return true;
 }
 bool make_plan(int64_t N, int64_t C, int64_t HW, int dtype, int channels_last, Plan& pl) {
@@ -1191,11 +1240,11 @@ void launch_apply(const Plan& pl, const XS& xs, const void* dy, const float* coe
     bn_apply_kernel<T, false, BWD, PACK, XS><<<grid, blk, 0, s>>>(xs, pd, coef, po, N, pl.F, HW, pl.per_block, ps);
 }
 
-template <typename T, bool BWD, bool MINMAX, typename XS>
+template <typename T, bool BWD, bool MINMAX, bool NT, typename XS>
 void launch_cl_reduce(const Plan& pl, const XS& xs, const void* dy, float* part, void* mn, void* mx,
                       int64_t C, hipStream_t s) {
   const dim3 grid((unsigned)pl.tiles, (unsigned)pl.nsplit), blk(kThreads);
-  bn_cl_reduce_kernel<T, BWD, MINMAX, XS><<<grid, blk, 0, s>>>(
+  bn_cl_reduce_kernel<T, BWD, MINMAX, NT, XS><<<grid, blk, 0, s>>>(
       xs, static_cast<const T*>(dy), part, static_cast<T*>(mn), static_cast<T*>(mx), pl.P, C, pl.tpr, pl.R, pl.ppb);
 }
 template <typename T, bool BWD, bool PACK, typename XS>
@@ -1214,9 +1263,15 @@ int forward_stats_t(const Plan& pl, const void* x, const float* weight, const fl
   float* part = ws;
   float* coef = ws + pl.part_floats;
   if (pl.channels_last) {
-    const PlainRows<T> xs{static_cast<const T*>(x), C};
-    if (mn) launch_cl_reduce<T, false, true>(pl, xs, nullptr, part, mn, mx, C, s);
-    else launch_cl_reduce<T, false, false>(pl, xs, nullptr, part, nullptr, nullptr, C, s);
+    if (pl.big) {
+      const PlainRows<T, true> xs{static_cast<const T*>(x), C};
+      if (mn) launch_cl_reduce<T, false, true, true>(pl, xs, nullptr, part, mn, mx, C, s);
+      else launch_cl_reduce<T, false, false, true>(pl, xs, nullptr, part, nullptr, nullptr, C, s);
+    } else {
+      const PlainRows<T> xs{static_cast<const T*>(x), C};
+      if (mn) launch_cl_reduce<T, false, true, false>(pl, xs, nullptr, part, mn, mx, C, s);
+      else launch_cl_reduce<T, false, false, false>(pl, xs, nullptr, part, nullptr, nullptr, C, s);
+    }
   } else {
     const PlainInput<T> xs{static_cast<const T*>(x), pl.F};
     if (mn) launch_reduce<T, false, true>(pl, xs, nullptr, part, mn, mx, N, HW, s);
@@ -1253,7 +1308,10 @@ int backward_t(const Plan& pl, const XS& xs, const void* dy, const float* weight
                int64_t C, int64_t HW, float* sumsq, hipStream_t s) {
   float* part = ws;
   float* coef = ws + pl.part_floats;
-  if constexpr (XS::kRows) launch_cl_reduce<T, true, false>(pl, xs, dy, part, nullptr, nullptr, C, s);
+  if constexpr (XS::kRows) {
+    if (pl.big) launch_cl_reduce<T, true, false, true>(pl, xs, dy, part, nullptr, nullptr, C, s);
+    else launch_cl_reduce<T, true, false, false>(pl, xs, dy, part, nullptr, nullptr, C, s);
+  }
   else launch_reduce<T, true, false>(pl, xs, dy, part, nullptr, nullptr, N, HW, s);
   bn_backward_finalize_kernel<<<dim3((unsigned)((C + kWaves - 1) / kWaves)), dim3(kThreads), 0, s>>>(
       part, weight, save_mean, save_invstd, dweight, dbias, coef, N, C, HW, pl.L, pl.nsplit, pl.slots);
@@ -1286,7 +1344,7 @@ int backward_packed(const Plan& pl, const int32_t* packed, const int32_t* bits, 
   const PackedInput<T> in{packed, bits, prefix, static_cast<const T*>(scale), static_cast<const T*>(mn),
                           pl.F / 256, 0, 0u, false};
   if (pl.channels_last) {
-    const PackedRows<T> xs{in, C, 0, (uint32_t)HW, 0u, 1, 0, 0};
+    const PackedRows<T> xs{in, C, 0, (uint32_t)HW, 0, 0u, 1, 0, 0};
     return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
   }
   return backward_t<T>(pl, in, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
