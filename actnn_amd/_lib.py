@@ -63,9 +63,13 @@ SIGNATURES = {
     "actnn_calc_precision": [c_vp, c_vp, c_vp, c_i64, ctypes.c_double],
     "actnn_linear_grad_weight": [c_vp, c_vp, c_vp, c_vp, c_i32, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64,
                                  c_i32, c_i32, c_i32, c_vp],
+    "actnn_linear_grad_weight_workspace_bytes": [c_i64, c_i64, c_i64],
+    "actnn_linear_grad_weight_ws": [c_vp, c_vp, c_vp, c_vp, c_i32, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64,
+                                    c_i32, c_i32, c_i32, c_vp, c_i64, c_vp],
     "actnn_linear_grad_weight_q2": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64,
                                     c_i32, c_i32, c_i32, c_vp],
     "actnn_stream_copy": [c_vp, c_vp, c_i64, c_vp],
+    "actnn_matrix_pipe_probe": [c_vp, c_vp, c_i32, c_i32, c_vp],
     "actnn_batch_norm_workspace_bytes": [c_i64, c_i64, c_i64, c_i32, c_i32],
     "actnn_batch_norm_forward": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,
                                  c_i64, c_i64, c_i64, ctypes.c_double, ctypes.c_double, c_i32, c_i32, c_vp],
@@ -83,6 +87,7 @@ SIGNATURES = {
     "actnn_batch_norm_backward_sumsq_entries": [c_i64, c_i64, c_i64, c_i32, c_i32],
 }
 _RESTYPES = {"actnn_strerror": ctypes.c_char_p, "actnn_version": ctypes.c_char_p,
+             "actnn_linear_grad_weight_workspace_bytes": ctypes.c_int64,
              "actnn_batch_norm_workspace_bytes": ctypes.c_int64,
              "actnn_batch_norm_forward_static_limit": ctypes.c_int64,
              "actnn_batch_norm_backward_sumsq_entries": ctypes.c_int64}

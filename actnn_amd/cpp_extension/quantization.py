@@ -234,11 +234,15 @@ def linear_grad_weight(grad_output, packed, bits, scale, min, in_features, out_d
         bits_ptr = prefix_ptr = None
     out_dtype = out_dtype or grad_output.dtype
     gw = torch.empty(O, I, dtype=out_dtype, device=grad_output.device)
+    # few output tiles and many rows: the sum over the rows is split over blocks (partial tiles in `ws`)
+    ws_bytes = g.lib().actnn_linear_grad_weight_workspace_bytes(M, O, I)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=gw.device) if ws_bytes > 0 else None
     with g.on_device(gw.device):
-        check(g.lib().actnn_linear_grad_weight(
+        check(g.lib().actnn_linear_grad_weight_ws(
             grad_output.data_ptr(), packed.data_ptr(), bits_ptr, prefix_ptr, fixed, scale.data_ptr(),
             min.data_ptr(), gw.data_ptr(), M, O, I, g.DTYPE_CODE[grad_output.dtype], g.DTYPE_CODE[scale.dtype],
-            g.DTYPE_CODE[out_dtype], g.stream_ptr(gw.device)), "linear_grad_weight")
+            g.DTYPE_CODE[out_dtype], ws.data_ptr() if ws is not None else None, ws_bytes,
+            g.stream_ptr(gw.device)), "linear_grad_weight")
     return gw
 
 

@@ -94,6 +94,18 @@ ACTNN_DEV void load_to_lds16_nt(const void* src, const uint8_t* lds_base) {
                : "s"(__builtin_amdgcn_readfirstlane(base)), "v"(src)
                : "memory", "m0");
 }
+// The same with the source given as a base that is the same for the whole wave (it travels in
+// scalar registers) plus a 32-bit byte offset per lane: no 64-bit address arithmetic per lane.
+ACTNN_DEV void load_to_lds16_base(const void* wave_base, uint32_t lane_bytes, const uint8_t* lds_base) {
+  const uint32_t base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)lds_base;
+  const uint64_t b = (uint64_t)(uintptr_t)wave_base;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b), hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+  const uint64_t sb = ((uint64_t)hi << 32) | lo;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(base)), "v"(lane_bytes), "s"(sb)
+               : "memory", "m0");
+}
 #pragma clang diagnostic pop
 
 // ------------------------------------------------------------------ 8 / 16 contiguous elements

@@ -1,5 +1,5 @@
-// Library-level helpers: error strings, version, and the plain streaming copy used to
-// calibrate bandwidth counters.
+// Library-level helpers: error strings, version, the plain streaming copy used to calibrate
+// bandwidth counters, and the matrix-pipe probe the benchmark prices the fused GEMM against.
 #include "device_utils.h"
 
 namespace actnn {
@@ -18,8 +18,58 @@ __global__ __launch_bounds__(256) void stream_copy_kernel(const uint4* __restric
     if (base + i * 256 < nvec) dst[base + i * 256] = v[i];      // this kernel is the calibration yardstick
 }
 
+// What the matrix pipes alone sustain: every wave (one per SIMD, as in the fused weight-gradient
+// GEMM) loads eight 16-byte operand fragments once and then issues nothing but
+// v_mfma_f32_32x32x16_bf16 on them - 16 per k-block into 16 independent accumulators, the operand
+// registers rotated between k-blocks so that every instruction meets a fresh pair.  No loads, no
+// LDS, no other arithmetic in the loop.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+__global__ __launch_bounds__(256, 1) void matrix_pipe_kernel(const u32x4* __restrict__ operands,
+                                                             float* __restrict__ out, int kblocks) {
+  f32x16_t acc[4][4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int c = 0; c < 16; ++c) acc[e][a][c] = 0.0f;
+  u32x4 f[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) f[i] = operands[((size_t)blockIdx.x * 8 + i) * 256 + threadIdx.x];
+  for (int kb = 0; kb < kblocks; ++kb) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+        acc[e][a] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, f[e]),
+                                                            __builtin_bit_cast(bf16x8_t, f[4 + a]), acc[e][a], 0, 0, 0);
+    const u32x4 t = f[0];
+#pragma unroll
+    for (int i = 0; i < 7; ++i) f[i] = f[i + 1];
+    f[7] = t;
+  }
+  float sum = 0.0f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int c = 0; c < 16; ++c) sum += acc[e][a][c];
+  out[(size_t)blockIdx.x * 256 + threadIdx.x] = sum;
+}
+
 }  // namespace
 }  // namespace actnn
+
+extern "C" int actnn_matrix_pipe_probe(const void* operands, float* out, int blocks, int kblocks, void* stream) {
+  using namespace actnn;
+  if (blocks <= 0 || kblocks < 0 || !operands || !out) return ACTNN_EINVAL;
+  if (!aligned16(operands)) return ACTNN_EALIGN;
+  matrix_pipe_kernel<<<dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<const u32x4*>(operands), out, kblocks);
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
 
 extern "C" int actnn_stream_copy(const void* src, void* dst, int64_t bytes, void* stream) {
   using namespace actnn;

@@ -331,14 +331,19 @@ class conv_transpose3d(Function):
 def _fused_grad_weight_ok(quantized, shape, go):
     """The fused kernel takes a 2-D input saved in whole groups of 256 per row - as the fixed-width
     stream (levels L1 / L2, or any int width) or the per-sample stream of the schemes (L3 and up) -
-    with 16-bit gradients (autocast, or a 16-bit model)."""
+    with 16-bit gradients (autocast, or a 16-bit model).  Every block of that kernel decodes the
+    activation tile it multiplies, so a tile is decoded once per 256 output rows: that hides behind
+    the matrix instructions for the 2-bit fixed-width stream (a table and byte permutes, 1.5
+    instructions per value) and not for the others, which cost 2.8 - 3.5 times unpack + mm on
+    [8192,4096]^T x [8192,4096].  By default only the former takes the fused kernel."""
     if not config.compress_activation or config.simulate or config.swap or not config.fused_linear_grad_weight:
         return False
     q_input, q_bits, q_scale, q_min = quantized
+    every_stream = config.fused_linear_grad_weight == "always"
     if isinstance(q_bits, int):
-        if q_bits not in (1, 2, 4, 8):
+        if q_bits not in (1, 2, 4, 8) or (q_bits != 2 and not every_stream):
             return False
-    elif not (isinstance(q_bits, torch.Tensor) and q_bits.dtype == torch.int32 and q_bits.is_cuda):
+    elif not (every_stream and isinstance(q_bits, torch.Tensor) and q_bits.dtype == torch.int32 and q_bits.is_cuda):
         return False
     return (len(shape) == 2 and shape[-1] % config.group_size == 0 and config.group_size == 256
             and go.shape[1] % 8 == 0 and go.dtype in (torch.float16, torch.bfloat16)

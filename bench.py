@@ -315,6 +315,11 @@ def other_configs(device, reps):
     return _rounded(out)
 
 
+def _lib_handle():
+    from actnn_amd import _lib
+    return _lib.load()
+
+
 def _rounded(v):
     """Floats of a nested dict rounded to 4 decimals."""
     if isinstance(v, dict):
@@ -361,6 +366,63 @@ def config4(device, reps):
     t = _event_time_ms(unfused, reps)
     out["linear_grad_weight_unfused_unpack_plus_mm"] = {"ms": t, "TFLOP/s": flops / t / 1e9,
                                                         "frac_mfma_bf16": flops / t / 1e9 / MFMA_BF16_PEAK_TFLOPS}
+    # The other streams linear.backward hands this kernel (the general loader: per-element
+    # dequantisation, no table): 4 bits fixed (levels L1 / L2) and the mixed-width stream with greedy
+    # widths at an average of 2 bits (level L3 and up), each beside its unfused pair
+    import actnn_amd.cpp_extension.calc_precision as ext_cp
+    p4, s4 = ext_q.pack_single_precision(xs, mn, mx, 4, True)
+    t = _event_time_ms(lambda: ext_q.linear_grad_weight(go, p4, 4, s4, mn, I), reps)
+    out["linear_grad_weight_4bit_fused"] = {"ms": t, "TFLOP/s": flops / t / 1e9,
+                                            "frac_mfma_bf16": flops / t / 1e9 / MFMA_BF16_PEAK_TFLOPS}
+    t = _event_time_ms(lambda: go.t().mm(ext_q.unpack_single_precision(p4, 4, s4, mn, M, I // 256, 256).view(M, I)), reps)
+    out["linear_grad_weight_4bit_unfused_unpack_plus_mm"] = {"ms": t, "TFLOP/s": flops / t / 1e9,
+                                                             "frac_mfma_bf16": flops / t / 1e9 / MFMA_BF16_PEAK_TFLOPS}
+    del p4, s4
+    range_sqr = torch.norm((mx - mn).view(M, -1).float(), dim=1).square() * 256.0          # qscheme.py:80, one pixel
+    widths = ext_cp.calc_precision(torch.full((M,), 8, dtype=torch.int32), (range_sqr / 4).cpu(),
+                                   torch.ones(M, dtype=torch.int32), 2 * M)
+    bm = ext_q.attach_bits_host(widths.to(device), widths)
+    pm, sm = ext_q.pack_mixed_precision(xs, mn, mx, bm, True)
+    t = _event_time_ms(lambda: ext_q.linear_grad_weight(go, pm, bm, sm, mn, I), reps)
+    out["linear_grad_weight_mixed_fused"] = {"ms": t, "TFLOP/s": flops / t / 1e9,
+                                             "frac_mfma_bf16": flops / t / 1e9 / MFMA_BF16_PEAK_TFLOPS,
+                                             "widths": _width_histogram(widths)}
+    t = _event_time_ms(lambda: go.t().mm(ext_q.unpack_mixed_precision(pm, bm, sm, mn, M, I // 256, 256).view(M, I)), reps)
+    out["linear_grad_weight_mixed_unfused_unpack_plus_mm"] = {"ms": t, "TFLOP/s": flops / t / 1e9,
+                                                              "frac_mfma_bf16": flops / t / 1e9 / MFMA_BF16_PEAK_TFLOPS}
+    del pm, sm, bm
+    # Shapes with few output tiles: the ResNet-50 classifier at batch 512 ([512,1000]^T x [512,2048],
+    # 32 tiles, too few rows for a split to pay) and a narrow layer with many rows ([32768,256]^T x
+    # [32768,512], 2 tiles: the sum over the rows is split over blocks)
+    for key, (Ms, Os, Is) in (("classifier_512x1000x2048", (512, 1000, 2048)), ("narrow_32768x256x512", (32768, 256, 512))):
+        xq = torch.randn(Ms, Is // 256, 256, generator=gen, device=device).to(torch.bfloat16)
+        lo, hi = ext_minimax.minimax(xq.view(-1, 256))
+        lo, hi = lo.view(Ms, -1, 1), hi.view(Ms, -1, 1)
+        pq, sq = ext_q.pack_single_precision(xq, lo, hi, 2, True)
+        gq = torch.randn(Ms, Os, generator=gen, device=device).to(torch.bfloat16)
+        fl = 2.0 * Ms * Os * Is
+        tf = _event_time_ms(lambda: ext_q.linear_grad_weight(gq, pq, 2, sq, lo, Is), reps)
+        tu = _event_time_ms(lambda: gq.t().mm(ext_q.unpack_single_precision(pq, 2, sq, lo, Ms, Is // 256, 256).view(Ms, Is)), reps)
+        out["linear_grad_weight_" + key] = {
+            "fused_ms": tf, "fused_TFLOP/s": fl / tf / 1e9, "unfused_unpack_plus_mm_ms": tu,
+            "split_workspace_bytes": int(_lib_handle().actnn_linear_grad_weight_workspace_bytes(Ms, Os, Is))}
+        del xq, lo, hi, pq, sq, gq
+    # The ceiling the part itself sets: the matrix pipes alone, as many v_mfma_f32_32x32x16_bf16 per
+    # wave as the config-4 product needs (256 blocks x 4 waves x 8192), on operand registers drawn
+    # from N(0,1), all zeros, all ones
+    lib = _lib_handle()
+    pipe = {}
+    probe_out = torch.empty(256 * 256, device=device)
+    for name, ops in (("normal", torch.randn(256 * 8 * 256 * 8, generator=gen, device=device).to(torch.bfloat16)),
+                      ("zeros", torch.zeros(256 * 8 * 256 * 8, device=device, dtype=torch.bfloat16)),
+                      ("ones", torch.ones(256 * 8 * 256 * 8, device=device, dtype=torch.bfloat16))):
+        def probe():
+            rc = lib.actnn_matrix_pipe_probe(ops.data_ptr(), probe_out.data_ptr(), 256, 512,
+                                             torch.cuda.current_stream().cuda_stream)
+            assert rc == 0
+        t = _event_time_ms(probe, reps)
+        pipe[name] = {"ms": t, "TFLOP/s": flops / t / 1e9, "frac_mfma_bf16": flops / t / 1e9 / MFMA_BF16_PEAK_TFLOPS}
+    out["matrix_pipes_alone_same_mfma_count"] = pipe
     # How much of the GEMM's time is the operands' data (the matrix pipes run against the power
     # limit): the same two launches - the fused kernel, and rocBLAS alone on the dequantised
     # input - with grad_out drawn from N(0,1), all zeros, and all ones.

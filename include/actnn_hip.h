@@ -237,6 +237,19 @@ int actnn_linear_grad_weight(const void* grad_out, const void* packed, const int
                              const int32_t* prefix, int fixed_bits, const void* scale, const void* mn,
                              void* grad_w, int64_t M, int64_t O, int64_t I, int go_dtype,
                              int sm_dtype, int out_dtype, void* stream);
+/* The same with a workspace for shapes whose few output tiles (256 x 256) would leave most of the
+ * chip idle: the sum over the M samples is then split over several blocks per tile, their fp32
+ * partial tiles go to `workspace` and a second kernel adds them in a fixed order (reproducible).
+ * actnn_linear_grad_weight_workspace_bytes says how much such a shape needs (0: the plain kernel
+ * is used and `workspace` may be null); with less than that the call runs unsplit, as
+ * actnn_linear_grad_weight always does.  workspace 16-byte aligned.  The reference's cuBLAS mm
+ * (ops.py:421) picks its own split the same way. */
+int64_t actnn_linear_grad_weight_workspace_bytes(int64_t M, int64_t O, int64_t I);
+int actnn_linear_grad_weight_ws(const void* grad_out, const void* packed, const int32_t* bits,
+                                const int32_t* prefix, int fixed_bits, const void* scale,
+                                const void* mn, void* grad_w, int64_t M, int64_t O, int64_t I,
+                                int go_dtype, int sm_dtype, int out_dtype, void* workspace,
+                                int64_t workspace_bytes, void* stream);
 int actnn_linear_grad_weight_q2(const void* grad_out, const int8_t* packed, const void* scale,
                                 const void* mn, void* grad_w, int64_t M, int64_t O, int64_t I,
                                 int go_dtype, int sm_dtype, int out_dtype, void* stream);
@@ -339,6 +352,14 @@ int actnn_batch_norm_backward_packed(const int32_t* packed, const int32_t* bits,
 /* Plain device-to-device streaming copy of `bytes` bytes (16-byte aligned pointers and
  * size); used by the benchmark to calibrate bandwidth counters.  No reference counterpart. */
 int actnn_stream_copy(const void* src, void* dst, int64_t bytes, void* stream);
+
+/* What the matrix pipes alone sustain on given operand data; used by the benchmark to price the
+ * fused weight-gradient GEMM against the rate the part reaches with the same operand statistics.
+ * `blocks` blocks of 256 threads (one wave per SIMD) each load 8 fragments of 16 bytes per thread
+ * from operands[blocks][8][256] (16 bytes each, bf16 values) and issue 16 * kblocks
+ * v_mfma_f32_32x32x16_bf16 per wave on them (2 * 32 * 32 * 16 flop each); out[blocks * 256]
+ * receives a checksum.  No reference counterpart. */
+int actnn_matrix_pipe_probe(const void* operands, float* out, int blocks, int kblocks, void* stream);
 
 #ifdef __cplusplus
 }

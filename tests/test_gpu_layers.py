@@ -150,14 +150,17 @@ def test_qlinear_fused_weight_gradient_path(dtype):
     assert torch.equal(gp_f[1], gp_u[1])
 
 
-@pytest.mark.parametrize("level", ["L2", "L3"])
-def test_qlinear_takes_the_fused_gemm_at_the_reference_levels(level, monkeypatch):
-    # under bf16 autocast a QLinear's weight gradient comes from the fused kernel at every level that
-    # compresses: the 4-bit fixed-width stream at L1 / L2, the per-sample stream of the scheme at L3;
-    # the result agrees with the unfused path (unpack + mm) on the same packed input
-    from actnn_amd import ops
+@pytest.mark.parametrize("level,bits,mode,stream", [("L2", 2, True, int), ("L2", 4, True, None), ("L3", 2, True, None),
+                                                     ("L2", 4, "always", int), ("L3", 2, "always", torch.Tensor)])
+def test_qlinear_takes_the_fused_gemm_where_it_is_the_faster_path(level, bits, mode, stream, monkeypatch):
+    # under bf16 autocast a QLinear's weight gradient comes from the fused kernel when its input was
+    # saved as the 2-bit fixed-width stream; the 4-bit stream of L1 / L2 and the per-sample stream
+    # of L3 take unpack + mm unless config.fused_linear_grad_weight == "always".  Where the fused
+    # kernel runs, its result agrees with the unfused path on the same packed input
     import actnn_amd.cpp_extension.quantization as ext_q
     set_optimization_level(level)
+    config.activation_compression_bits = [bits] + config.activation_compression_bits[1:]
+    config.fused_linear_grad_weight = mode
     torch.manual_seed(0)
     q = actnn_amd.QLinear(2048, 1000).to(DEV)
     x = torch.randn(128, 2048, device=DEV)
@@ -174,7 +177,10 @@ def test_qlinear_takes_the_fused_gemm_at_the_reference_levels(level, monkeypatch
     step()                                          # first step: degenerate widths at L3
     torch.cuda.manual_seed(5)
     gw_fused = step()
-    assert len(calls) == 2 and calls[0] is (int if level == "L2" else torch.Tensor)
+    if stream is None:
+        assert calls == []
+        return
+    assert len(calls) == 2 and calls[0] is stream
     config.fused_linear_grad_weight = False
     torch.cuda.manual_seed(5)
     gw_unfused = step()

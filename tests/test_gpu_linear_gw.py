@@ -96,6 +96,42 @@ def test_mixed_width_stream(dtype):
     _check(gw, ref, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_few_tiles_and_many_rows_split_the_sum_over_blocks(dtype):
+    # one to four output tiles and thousands of rows: the library asks for a workspace and splits
+    # the sum over the rows (rows that do not fill the last split or the last 64-row step included)
+    from actnn_amd import _lib
+    lib = _lib.load()
+    torch.manual_seed(1)
+    for M, O, I, bits in ((8192, 256, 256, 2), (4096 + 37, 264, 512, 2), (6000, 128, 256, 4),
+                          (5000, 256, 512, None), (3000, 72, 256, 1)):
+        assert lib.actnn_linear_grad_weight_workspace_bytes(M, O, I) >= 2 * O * I * 4, (M, O, I)
+        widths = bits if bits is not None else torch.randint(1, 9, (M,)).tolist()
+        print(f"[linear_gw] split M={M} O={O} I={I} bits={bits} {dtype}", flush=True)
+        gw, ref = _case(M, O, I, dtype, dtype, seed=M, bits=widths)
+        _check(gw, ref, dtype)
+    # shapes that fill the chip, or have too few rows to gain, stay unsplit
+    assert lib.actnn_linear_grad_weight_workspace_bytes(8192, 4096, 4096) == 0
+    assert lib.actnn_linear_grad_weight_workspace_bytes(512, 1000, 2048) == 0
+    assert lib.actnn_linear_grad_weight_workspace_bytes(64, 256, 256) == 0
+
+
+def test_split_sum_multiplies_the_same_values():
+    # one-hot gradients over 4096 rows (split over blocks): every row of the dequantised input comes
+    # out of the sum exactly, whichever block multiplied it
+    from actnn_amd import _lib
+    M, I = 4096, 256
+    assert _lib.load().actnn_linear_grad_weight_workspace_bytes(M, 256, I) > 0
+    xg, _, mn, mx = _inputs(M, 64, I, torch.bfloat16, seed=5)
+    packed, scale = ext_q.pack_single_precision(xg, mn, mx, 2, True)
+    deq = ext_q.unpack_single_precision(packed, 2, scale, mn, M, 1, 256).view(M, I)
+    for first in (0, 1000, M - 256):
+        go = torch.zeros(M, 256, device=DEV, dtype=torch.bfloat16)
+        go[first:first + 256] = torch.eye(256, device=DEV, dtype=torch.bfloat16)
+        gw = ext_q.linear_grad_weight(go, packed, 2, scale, mn, I, torch.float32)
+        assert torch.equal(gw, deq[first:first + 256].float()), first
+
+
 def test_fp32_output_and_config4_shape():
     gw, ref = _case(8192, 4096, 4096, torch.float16, torch.float32)
     assert gw.dtype == torch.float32
