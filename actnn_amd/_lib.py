@@ -85,6 +85,11 @@ SIGNATURES = {
     "actnn_batch_norm_backward": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_vp, c_i64,
                                   c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
     "actnn_batch_norm_backward_sumsq_entries": [c_i64, c_i64, c_i64, c_i32, c_i32],
+    "actnn_batch_norm_groups_align": [c_i64, c_i64, c_i64, c_i32, c_i32],
+    "actnn_batch_norm_forward_eval": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64,
+                                      c_i64, ctypes.c_double, c_i32, c_i32, c_vp],
+    "actnn_batch_norm_backward_eval": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64,
+                                       c_i64, c_i32, c_i32, c_vp],
 }
 _RESTYPES = {"actnn_strerror": ctypes.c_char_p, "actnn_version": ctypes.c_char_p,
              "actnn_linear_grad_weight_workspace_bytes": ctypes.c_int64,

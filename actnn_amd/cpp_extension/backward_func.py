@@ -1,8 +1,9 @@
 """Backward ATen entry points the reference re-exports (cpp_extension/backward_func.cc:81-91),
 under the reference's names and argument order.  The convolutions map onto the ATen ops that
-exist on PyTorch-ROCm (MIOpen behind them); training-mode batch norm runs this library's own
-kernels (actnn_batch_norm_forward / _backward) whenever the shape qualifies and falls back to
-ATen's miopen_batch_norm otherwise.
+exist on PyTorch-ROCm (MIOpen behind them); batch norm - training and evaluation mode, any dense
+shape in the default or the channels-last layout, [N, C] inputs included - runs this library's
+own kernels (actnn_batch_norm_*) and falls back to ATen only for tensors that are not dense or
+whose affine parameters are not fp32.
 
 The three layer-norm exports of the reference have no Python caller and are not provided.
 """
@@ -79,17 +80,19 @@ def hip_batch_norm_applies(input, weight, bias, running_mean, running_var):
             and all(_f32_or_none(t) for t in (weight, bias, running_mean, running_var)))
 
 
-def _groups_align(C, HW, channels_last):
-    """Groups of 256 elements (in memory order) coincide with runs of threads of the kernels."""
-    return (C * HW) % 256 == 0 and (not channels_last or C % 256 == 0 or 256 % C == 0)
+@functools.lru_cache(maxsize=4096)
+def _groups_align(N, C, HW, code, channels_last):
+    """Groups of 256 elements (in memory order) coincide with runs of threads of the streaming
+    kernels: the group min/max, the packed copy and the packed backward exist for the shape."""
+    return bool(_glue.lib().actnn_batch_norm_groups_align(N, C, HW, code, int(channels_last)))
 
 
 def hip_batch_norm_minmax_applies(input, weight, bias, running_mean, running_var):
     """True when the forward pass can also return the quantiser's per-group min/max."""
     if not hip_batch_norm_applies(input, weight, bias, running_mean, running_var):
         return False
-    _, C, HW, channels_last = _bn_geometry(input)
-    return _groups_align(C, HW, channels_last)
+    N, C, HW, channels_last = _bn_geometry(input)
+    return _groups_align(N, C, HW, _glue.DTYPE_CODE[input.dtype], channels_last)
 
 
 def _ptr(t):
@@ -218,7 +221,8 @@ def hip_batch_norm_backward_packed_applies(shape, quantized, grad_output, weight
     compact = (dtype == torch.float32 and q_scale.dtype == torch.bfloat16
                and not getattr(quantized, "native_bf16", False))
     return (geo is not None and dtype in (torch.float16, torch.bfloat16, torch.float32)
-            and _groups_align(geo[1], geo[2], channels_last) and isinstance(q_bits, torch.Tensor)
+            and _groups_align(geo[0], geo[1], geo[2], _glue.DTYPE_CODE[dtype], channels_last)
+            and isinstance(q_bits, torch.Tensor)
             and isinstance(q_input, torch.Tensor) and q_input.is_cuda and q_input.dtype == torch.int32
             and (q_scale.dtype == dtype or compact) and q_min.dtype == q_scale.dtype
             and q_scale.is_contiguous() and q_min.is_contiguous()
@@ -322,14 +326,67 @@ def cudnn_batch_norm_backward(input, grad_output, weight, running_mean, running_
                                             save_mean, save_var, epsilon)
 
 
+def hip_batch_norm_forward_eval(input, weight, bias, running_mean, running_var, eps):
+    """-> (output, mean, invstd): evaluation-mode batch norm with this library's kernels; mean and
+    invstd are the running mean and 1 / sqrt(running_var + eps), kept for the backward pass."""
+    N, C, HW, channels_last = _bn_geometry(input)
+    lib = _glue.lib()
+    code = _glue.DTYPE_CODE[input.dtype]
+    ws_bytes = _workspace_bytes(N, C, HW, code, int(channels_last))
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=input.device)
+    out = torch.empty_like(input)
+    mean = torch.empty(C, dtype=torch.float32, device=input.device)
+    invstd = torch.empty(C, dtype=torch.float32, device=input.device)
+    with _glue.on_device(input.device):
+        _glue._lib.check(lib.actnn_batch_norm_forward_eval(
+            input.data_ptr(), _ptr(weight), _ptr(bias), running_mean.data_ptr(), running_var.data_ptr(),
+            out.data_ptr(), mean.data_ptr(), invstd.data_ptr(), ws.data_ptr(), ws_bytes, N, C, HW, float(eps),
+            code, int(channels_last), _glue.stream_ptr(input.device)), "batch_norm_forward_eval")
+    return out, mean, invstd
+
+
+def hip_batch_norm_backward_eval(input, grad_output, weight, mean, invstd):
+    """-> (grad_input, grad_weight, grad_bias) of evaluation-mode batch norm."""
+    N, C, HW, channels_last = _bn_geometry(input)
+    lib = _glue.lib()
+    code = _glue.DTYPE_CODE[input.dtype]
+    ws_bytes = _workspace_bytes(N, C, HW, code, int(channels_last))
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=input.device)
+    grad_input = torch.empty_like(input)
+    grad_weight = torch.empty(C, dtype=torch.float32, device=input.device)
+    grad_bias = torch.empty(C, dtype=torch.float32, device=input.device)
+    with _glue.on_device(input.device):
+        _glue._lib.check(lib.actnn_batch_norm_backward_eval(
+            input.data_ptr(), grad_output.data_ptr(), _ptr(weight), mean.data_ptr(), invstd.data_ptr(),
+            grad_input.data_ptr(), grad_weight.data_ptr(), grad_bias.data_ptr(), ws.data_ptr(), ws_bytes,
+            N, C, HW, code, int(channels_last), _glue.stream_ptr(input.device)), "batch_norm_backward_eval")
+    return grad_input, grad_weight, grad_bias
+
+
 def native_batch_norm(input, weight, bias, running_mean, running_var, training, momentum, eps):
-    """at::native_batch_norm (backward_func.cc:89)."""
+    """at::native_batch_norm (backward_func.cc:89).  In evaluation mode with running estimates - the
+    case the reference's batch_norm Function calls it for (ops.py:458-461) - this library's kernels
+    run whenever the tensors qualify; save_mean / save_invstd then hold the running mean and
+    1 / sqrt(running_var + eps) where ATen returns empty tensors."""
+    if (not training and running_mean is not None and running_var is not None
+            and hip_batch_norm_applies(input, weight, bias, running_mean, running_var)):
+        return hip_batch_norm_forward_eval(input, weight, bias, running_mean, running_var, eps)
     return _aten.native_batch_norm(input, weight, bias, running_mean, running_var, training, momentum, eps)
 
 
 def native_batch_norm_backward(grad_out, input, weight, running_mean, running_var, save_mean,
                                save_invstd, train, eps, output_mask):
-    """at::native_batch_norm_backward (backward_func.cc:90)."""
+    """at::native_batch_norm_backward (backward_func.cc:90); evaluation mode as above."""
+    if (not train and running_mean is not None and running_var is not None
+            and hip_batch_norm_applies(input, weight, None, running_mean, running_var)
+            and grad_out.dtype == input.dtype and grad_out.shape == input.shape
+            and grad_out.stride() == input.stride() and grad_out.data_ptr() % 16 == 0):
+        C = input.shape[1]
+        if save_mean is None or save_mean.numel() != C or save_invstd is None or save_invstd.numel() != C:
+            save_mean, save_invstd = running_mean, torch.rsqrt(running_var + eps)
+        gi, gw, gb = hip_batch_norm_backward_eval(input, grad_out, weight, save_mean, save_invstd)
+        mask = list(output_mask)
+        return (gi if mask[0] else None, gw if mask[1] else None, gb if mask[2] else None)
     return _aten.native_batch_norm_backward(grad_out, input, weight, running_mean, running_var,
                                             save_mean, save_invstd, train, eps, list(output_mask))
 

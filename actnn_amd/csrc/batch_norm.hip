@@ -579,7 +579,7 @@ __global__ __launch_bounds__(kThreads) void bn_forward_finalize_kernel(
 __global__ __launch_bounds__(kThreads) void bn_backward_finalize_kernel(
     const float* __restrict__ part, const float* __restrict__ weight, const float* __restrict__ save_mean,
     const float* __restrict__ save_invstd, float* __restrict__ dweight, float* __restrict__ dbias,
-    float* __restrict__ coef, int64_t N, int64_t C, int64_t HW, int64_t L, int nsplit, int slots) {
+    float* __restrict__ coef, int64_t N, int64_t C, int64_t HW, int64_t L, int nsplit, int slots, bool eval) {
   const int64_t c = (int64_t)blockIdx.x * kWaves + (threadIdx.x >> 6);     // one wave per channel
   if (c >= C) return;
   double S, Q;                                   // sum(dy), sum(x*dy)
@@ -591,12 +591,88 @@ __global__ __launch_bounds__(kThreads) void bn_backward_finalize_kernel(
   const double dot = (Q - mean * S) * r;         // sum(dy * xhat)
   if (dweight) dweight[c] = (float)dot;
   if (dbias) dbias[c] = (float)S;
+  // evaluation mode: mean and r are constants (the running estimates), so dx = w * r * dy
   const double A = w * r;
-  const double B = -w * r * r * (dot / M);
+  const double B = eval ? 0.0 : -w * r * r * (dot / M);
   coef[3 * c] = (float)A;
   coef[3 * c + 1] = (float)B;
-  coef[3 * c + 2] = (float)(-A * (S / M) - B * mean);
+  coef[3 * c + 2] = eval ? 0.0f : (float)(-A * (S / M) - B * mean);
 }
+
+// Evaluation mode: mean and variance are the running estimates; leaves them (as mean and inverse
+// standard deviation) for the backward pass and the coefficients of y = a*x + b for the apply pass.
+__global__ __launch_bounds__(kThreads) void bn_eval_coefficients_kernel(
+    const float* __restrict__ weight, const float* __restrict__ bias, const float* __restrict__ running_mean,
+    const float* __restrict__ running_var, float* __restrict__ save_mean, float* __restrict__ save_invstd,
+    float* __restrict__ coef, int64_t C, double eps) {
+  const int64_t c = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (c >= C) return;
+  const double mean = running_mean[c];
+  const double invstd = 1.0 / sqrt((double)running_var[c] + eps);
+  if (save_mean) save_mean[c] = (float)mean;
+  if (save_invstd) save_invstd[c] = (float)invstd;
+  const double a = (weight ? (double)weight[c] : 1.0) * invstd;
+  coef[2 * c] = (float)a;
+  coef[2 * c + 1] = (float)((bias ? (double)bias[c] : 0.0) - mean * a);
+}
+
+// ------------------------------------------------------------------ any shape
+// Shapes the chunked kernels do not take - a row of C*HW elements that is not a whole number of
+// 16-byte chunks, planes shorter than a chunk, channels-last tensors whose C is not a multiple of
+// the chunk - go element by element: a block per channel and slice of the batch for the sums (table
+// layout of the channels-last passes: [channel][sum][slice]), a thread per element for the second
+// pass.  Same arithmetic (fp32 sums folded in double, y = fma(x, a, b)), a fraction of the speed;
+// such shapes are rare.
+template <typename T, bool BWD, bool CL>
+__global__ __launch_bounds__(kThreads) void bn_any_reduce_kernel(
+    const T* __restrict__ x, const T* __restrict__ dy, float* __restrict__ part, int64_t N, int64_t C,
+    int64_t HW, int64_t per_block) {
+  __shared__ float s_wave[2 * kWaves];
+  const int64_t c = blockIdx.x;
+  const int64_t n0 = (int64_t)blockIdx.y * per_block;
+  const int64_t n1 = n0 + per_block < N ? n0 + per_block : N;
+  float s = 0.0f, q = 0.0f;
+  for (int64_t n = n0; n < n1; ++n) {
+    for (int64_t hw = threadIdx.x; hw < HW; hw += kThreads) {
+      const int64_t at = CL ? (n * HW + hw) * C + c : (n * C + c) * HW + hw;
+      const float xv = Conv<T>::load(x, at);
+      const float a = BWD ? Conv<T>::load(dy, at) : xv;
+      s += a;
+      q = fmaf(xv, a, q);
+    }
+  }
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) {
+    s += __shfl_xor(s, d);
+    q += __shfl_xor(q, d);
+  }
+  if ((threadIdx.x & 63) == 0) {
+    s_wave[2 * (threadIdx.x >> 6)] = s;
+    s_wave[2 * (threadIdx.x >> 6) + 1] = q;
+  }
+  __syncthreads();
+  if (threadIdx.x < 2) {
+    float v = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) v += s_wave[2 * w + threadIdx.x];
+    part[(c * 2 + threadIdx.x) * gridDim.y + blockIdx.y] = v;
+  }
+}
+
+template <typename T, bool BWD, bool CL>
+__global__ __launch_bounds__(kThreads) void bn_any_apply_kernel(
+    const T* __restrict__ x, const T* __restrict__ dy, const float* __restrict__ coef, T* __restrict__ out,
+    int64_t total, int64_t C, int64_t HW) {
+  constexpr int NC = BWD ? 3 : 2;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kThreads) {
+    const int64_t c = CL ? i % C : (i / HW) % C;
+    const float xv = Conv<T>::load(x, i);
+    const float v = BWD ? fmaf(Conv<T>::load(dy, i), coef[NC * c], fmaf(xv, coef[NC * c + 1], coef[NC * c + 2]))
+                        : fmaf(xv, coef[NC * c], coef[NC * c + 1]);
+    Conv<T>::store(out, i, v);
+  }
+}
+
 
 // Pass 2 of either direction.  Forward: y = a*x + b.  Backward: dx = A*dy + B*x + K.
 template <typename T, bool SPLIT, bool BWD, bool PACK, typename XS>
@@ -1128,6 +1204,8 @@ struct Plan {
   int tiles, tpr, R;
   bool groups_align;   // quantisation groups are aligned runs of threads
   bool big;            // the tensor does not fit the last-level cache: a pass finds nothing of it there
+  bool any_shape;      // not a whole number of chunks per row / per pixel: the element-by-element kernels
+  int64_t any_per_block;   // samples per block of their reduce pass
 };
 // The memory-side cache holds 256 MiB.  A tensor above that is gone from it by the time the next pass
 // starts, so the passes that only read may use non-temporal loads (7.0 against 6.1 TB/s on a plain
@@ -1206,11 +1284,42 @@ bool make_plan(int64_t N, int64_t C, int64_t HW, int dtype, Plan& pl) {
   pl.big = N * pl.F * (dtype == ACTNN_F32 ? 4 : 2) > kLastLevelCacheBytes;
   return true;
 }
+// The plan of the element-by-element kernels: grid (C, nsplit) for the sums.
+bool make_plan_any(int64_t N, int64_t C, int64_t HW, int dtype, bool channels_last, Plan& pl) {
+  if (N <= 0 || C <= 0 || HW <= 0 || dtype < 0 || dtype > 2) return false;
+  if (C > 0x7fffffffLL || HW > 0x7fffffffLL || C > ((int64_t)1 << 40) / HW || N > ((int64_t)1 << 62) / (C * HW)) return false;
+  pl = Plan{};
+  pl.any_shape = true;
+  pl.channels_last = channels_last;
+  pl.elems = dtype == ACTNN_F32 ? 4 : 8;
+  pl.F = C * HW;
+  pl.P = N * HW;
+  // about 4096 blocks in all, each at least one sample
+  int64_t want = (4096 + C - 1) / C;
+  if (want > 65535) want = 65535;
+  int64_t per_block = (N + want - 1) / want;
+  if (per_block < 1) per_block = 1;
+  pl.any_per_block = per_block;
+  pl.nsplit = (int)((N + per_block - 1) / per_block);
+  pl.slots = 0;                                  // the table layout of the channels-last passes
+  pl.part_floats = C * 2 * pl.nsplit;
+  pl.groups_align = false;
+  pl.big = false;
+  return true;
+}
 bool make_plan(int64_t N, int64_t C, int64_t HW, int dtype, int channels_last, Plan& pl) {
-  return channels_last ? make_plan_cl(N, C, HW, dtype, pl) : make_plan(N, C, HW, dtype, pl);
+  if (N <= 0 || C <= 0 || HW <= 0 || dtype < 0 || dtype > 2) return false;
+  const int elems = dtype == ACTNN_F32 ? 4 : 8;
+  // [N, C] (one position per channel) is the channels-last layout with a single pixel per sample
+  const bool cl = channels_last || HW == 1;
+  pl.any_shape = false;
+  pl.any_per_block = 0;
+  if (cl ? C % elems != 0 : (HW < elems || (C * HW) % elems != 0)) return make_plan_any(N, C, HW, dtype, cl, pl);
+  return cl ? make_plan_cl(N, C, HW, dtype, pl) : make_plan(N, C, HW, dtype, pl);
 }
 int64_t workspace_floats(const Plan& pl, int64_t C) { return pl.part_floats + 3 * C; }
 int64_t apply_waves(const Plan& pl) {      // entries of the sum-of-squares table of the backward apply pass
+  if (pl.any_shape) return 0;              // (the element-by-element kernels leave none)
   return (pl.channels_last ? (int64_t)pl.tiles * pl.nsplit_apply : pl.spans * pl.nsplit) * kWaves;
 }
 
@@ -1262,7 +1371,13 @@ int forward_stats_t(const Plan& pl, const void* x, const float* weight, const fl
                     int64_t N, int64_t C, int64_t HW, double momentum, double eps, hipStream_t s) {
   float* part = ws;
   float* coef = ws + pl.part_floats;
-  if (pl.channels_last) {
+  if (pl.any_shape) {
+    const dim3 grid((unsigned)C, (unsigned)pl.nsplit), blk(kThreads);
+    if (pl.channels_last)
+      bn_any_reduce_kernel<T, false, true><<<grid, blk, 0, s>>>(static_cast<const T*>(x), nullptr, part, N, C, HW, pl.any_per_block);
+    else
+      bn_any_reduce_kernel<T, false, false><<<grid, blk, 0, s>>>(static_cast<const T*>(x), nullptr, part, N, C, HW, pl.any_per_block);
+  } else if (pl.channels_last) {
     if (pl.big) {
       const PlainRows<T, true> xs{static_cast<const T*>(x), C};
       if (mn) launch_cl_reduce<T, false, true, true>(pl, xs, nullptr, part, mn, mx, C, s);
@@ -1290,6 +1405,18 @@ int forward_apply_t(const Plan& pl, const void* x, void* y, const float* ws, con
                     int64_t C, int64_t HW, hipStream_t s) {
   const float* coef = ws + pl.part_floats;
   const PackSink none{};
+  if (pl.any_shape) {
+    const int64_t total = N * C * HW;
+    int64_t blocks = (total + kThreads - 1) / kThreads;
+    if (blocks > 65536) blocks = 65536;
+    if (pl.channels_last)
+      bn_any_apply_kernel<T, false, true><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+          static_cast<const T*>(x), nullptr, coef, static_cast<T*>(y), total, C, HW);
+    else
+      bn_any_apply_kernel<T, false, false><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+          static_cast<const T*>(x), nullptr, coef, static_cast<T*>(y), total, C, HW);
+    ACTNN_RETURN_LAUNCH_STATUS();
+  }
   if (pl.channels_last) {
     const PlainRows<T> xs{static_cast<const T*>(x), C};
     if (sink) { launch_cl_apply<T, false, true>(pl, xs, nullptr, coef, y, C, *sink, s); ACTNN_RETURN_LAUNCH_STATUS(); }
@@ -1305,7 +1432,7 @@ int forward_apply_t(const Plan& pl, const void* x, void* y, const float* ws, con
 template <typename T, typename XS>
 int backward_t(const Plan& pl, const XS& xs, const void* dy, const float* weight, const float* save_mean,
                const float* save_invstd, void* dx, float* dweight, float* dbias, float* ws, int64_t N,
-               int64_t C, int64_t HW, float* sumsq, hipStream_t s) {
+               int64_t C, int64_t HW, float* sumsq, hipStream_t s, bool eval = false) {
   float* part = ws;
   float* coef = ws + pl.part_floats;
   if constexpr (XS::kRows) {
@@ -1314,7 +1441,7 @@ int backward_t(const Plan& pl, const XS& xs, const void* dy, const float* weight
   }
   else launch_reduce<T, true, false>(pl, xs, dy, part, nullptr, nullptr, N, HW, s);
   bn_backward_finalize_kernel<<<dim3((unsigned)((C + kWaves - 1) / kWaves)), dim3(kThreads), 0, s>>>(
-      part, weight, save_mean, save_invstd, dweight, dbias, coef, N, C, HW, pl.L, pl.nsplit, pl.slots);
+      part, weight, save_mean, save_invstd, dweight, dbias, coef, N, C, HW, pl.L, pl.nsplit, pl.slots, eval);
   if (dx) {
     PackSink extra{};
     extra.sumsq = sumsq;
@@ -1324,16 +1451,42 @@ int backward_t(const Plan& pl, const XS& xs, const void* dy, const float* weight
   ACTNN_RETURN_LAUNCH_STATUS();
 }
 
+template <typename T, bool CL>
+int backward_any(const Plan& pl, const void* x, const void* dy, const float* weight, const float* save_mean,
+                 const float* save_invstd, void* dx, float* dweight, float* dbias, float* ws, int64_t N,
+                 int64_t C, int64_t HW, hipStream_t s, bool eval) {
+  float* part = ws;
+  float* coef = ws + pl.part_floats;
+  const T* px = static_cast<const T*>(x);
+  const T* pd = static_cast<const T*>(dy);
+  bn_any_reduce_kernel<T, true, CL><<<dim3((unsigned)C, (unsigned)pl.nsplit), dim3(kThreads), 0, s>>>(
+      px, pd, part, N, C, HW, pl.any_per_block);
+  bn_backward_finalize_kernel<<<dim3((unsigned)((C + kWaves - 1) / kWaves)), dim3(kThreads), 0, s>>>(
+      part, weight, save_mean, save_invstd, dweight, dbias, coef, N, C, HW, pl.L, pl.nsplit, pl.slots, eval);
+  if (dx) {
+    const int64_t total = N * C * HW;
+    int64_t blocks = (total + kThreads - 1) / kThreads;
+    if (blocks > 65536) blocks = 65536;
+    bn_any_apply_kernel<T, true, CL><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
+        px, pd, coef, static_cast<T*>(dx), total, C, HW);
+  }
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
+
 template <typename T>
 int backward_plain(const Plan& pl, const void* x, const void* dy, const float* weight, const float* save_mean,
                    const float* save_invstd, void* dx, float* dweight, float* dbias, float* ws, int64_t N,
-                   int64_t C, int64_t HW, float* sumsq, hipStream_t s) {
+                   int64_t C, int64_t HW, float* sumsq, hipStream_t s, bool eval = false) {
+  if (pl.any_shape) {
+    if (pl.channels_last) return backward_any<T, true>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s, eval);
+    return backward_any<T, false>(pl, x, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, s, eval);
+  }
   if (pl.channels_last) {
     const PlainRows<T> xs{static_cast<const T*>(x), C};
-    return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
+    return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s, eval);
   }
   const PlainInput<T> xs{static_cast<const T*>(x), pl.F};
-  return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
+  return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s, eval);
 }
 
 template <typename T>
@@ -1367,6 +1520,12 @@ extern "C" int64_t actnn_batch_norm_backward_sumsq_entries(int64_t N, int64_t C,
   return actnn::apply_waves(pl);
 }
 
+extern "C" int actnn_batch_norm_groups_align(int64_t N, int64_t C, int64_t HW, int dtype, int channels_last) {
+  actnn::Plan pl;
+  if (!actnn::make_plan(N, C, HW, dtype, channels_last, pl)) return 0;
+  return pl.groups_align && !pl.any_shape ? 1 : 0;
+}
+
 extern "C" int actnn_batch_norm_forward_stats(const void* x, const float* weight, const float* bias,
                                               float* running_mean, float* running_var, float* save_mean,
                                               float* save_invstd, void* mn, void* mx, void* workspace,
@@ -1380,7 +1539,7 @@ extern "C" int actnn_batch_norm_forward_stats(const void* x, const float* weight
   if (!x || !save_mean || !save_invstd || !workspace || (mn == nullptr) != (mx == nullptr)) return ACTNN_EINVAL;
   if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
   if (mn && !pl.groups_align) return ACTNN_EINVAL;
-  if (!aligned16(x) || !aligned16(workspace)) return ACTNN_EALIGN;
+  if ((!pl.any_shape && !aligned16(x)) || !aligned16(workspace)) return ACTNN_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   float* ws = static_cast<float*>(workspace);
   switch (dtype) {
@@ -1402,7 +1561,7 @@ extern "C" int actnn_batch_norm_forward_apply(const void* x, void* y, const void
   if (!make_plan(N, C, HW, dtype, channels_last, pl)) return ACTNN_EINVAL;
   if (!x || !y || !workspace) return ACTNN_EINVAL;
   if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
-  if (!aligned16(x) || !aligned16(y) || !aligned16(workspace)) return ACTNN_EALIGN;
+  if ((!pl.any_shape && (!aligned16(x) || !aligned16(y))) || !aligned16(workspace)) return ACTNN_EALIGN;
   PackSink sink{bits, prefix, mn, mx, scale, packed, seed, offset, pl.F / 256};
   const bool pack = bits != nullptr;
   if (pack) {
@@ -1431,6 +1590,51 @@ extern "C" int actnn_batch_norm_forward(const void* x, const float* weight, cons
   if (rc != ACTNN_OK) return rc;
   return actnn_batch_norm_forward_apply(x, y, workspace, workspace_bytes, nullptr, nullptr, nullptr, nullptr,
                                         nullptr, nullptr, 0, 0, N, C, HW, dtype, channels_last, stream);
+}
+
+// Evaluation mode: the running estimates take the place of the batch statistics.
+extern "C" int actnn_batch_norm_forward_eval(const void* x, const float* weight, const float* bias,
+                                             const float* running_mean, const float* running_var, void* y,
+                                             float* save_mean, float* save_invstd, void* workspace,
+                                             int64_t workspace_bytes, int64_t N, int64_t C, int64_t HW, double eps,
+                                             int dtype, int channels_last, void* stream) {
+  using namespace actnn;
+  if (dtype < 0 || dtype > 2) return ACTNN_EDTYPE;
+  Plan pl;
+  if (!make_plan(N, C, HW, dtype, channels_last, pl)) return ACTNN_EINVAL;
+  if (!x || !y || !running_mean || !running_var || !workspace) return ACTNN_EINVAL;
+  if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
+  if ((!pl.any_shape && (!aligned16(x) || !aligned16(y))) || !aligned16(workspace)) return ACTNN_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float* ws = static_cast<float*>(workspace);
+  bn_eval_coefficients_kernel<<<dim3((unsigned)((C + kThreads - 1) / kThreads)), dim3(kThreads), 0, s>>>(
+      weight, bias, running_mean, running_var, save_mean, save_invstd, ws + pl.part_floats, C, eps);
+  switch (dtype) {
+    case ACTNN_F32: return forward_apply_t<float>(pl, x, y, ws, nullptr, N, C, HW, s);
+    case ACTNN_F16: return forward_apply_t<__half>(pl, x, y, ws, nullptr, N, C, HW, s);
+    default: return forward_apply_t<bf16_t>(pl, x, y, ws, nullptr, N, C, HW, s);
+  }
+}
+
+extern "C" int actnn_batch_norm_backward_eval(const void* x, const void* dy, const float* weight,
+                                              const float* mean, const float* invstd, void* dx,
+                                              float* dweight, float* dbias, void* workspace,
+                                              int64_t workspace_bytes, int64_t N, int64_t C, int64_t HW,
+                                              int dtype, int channels_last, void* stream) {
+  using namespace actnn;
+  if (dtype < 0 || dtype > 2) return ACTNN_EDTYPE;
+  Plan pl;
+  if (!make_plan(N, C, HW, dtype, channels_last, pl)) return ACTNN_EINVAL;
+  if (!x || !dy || !mean || !invstd || !workspace) return ACTNN_EINVAL;
+  if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
+  if ((!pl.any_shape && (!aligned16(x) || !aligned16(dy) || (dx && !aligned16(dx)))) || !aligned16(workspace)) return ACTNN_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float* ws = static_cast<float*>(workspace);
+  switch (dtype) {
+    case ACTNN_F32: return backward_plain<float>(pl, x, dy, weight, mean, invstd, dx, dweight, dbias, ws, N, C, HW, nullptr, s, true);
+    case ACTNN_F16: return backward_plain<__half>(pl, x, dy, weight, mean, invstd, dx, dweight, dbias, ws, N, C, HW, nullptr, s, true);
+    default: return backward_plain<bf16_t>(pl, x, dy, weight, mean, invstd, dx, dweight, dbias, ws, N, C, HW, nullptr, s, true);
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1519,7 +1723,7 @@ extern "C" int actnn_batch_norm_backward(const void* x, const void* dy, const fl
   if (!x || !dy || !save_mean || !save_invstd || !workspace) return ACTNN_EINVAL;
   if (sumsq && (!dx || sumsq_entries < apply_waves(pl))) return ACTNN_EINVAL;
   if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
-  if (!aligned16(x) || !aligned16(dy) || (dx && !aligned16(dx)) || !aligned16(workspace)) return ACTNN_EALIGN;
+  if ((!pl.any_shape && (!aligned16(x) || !aligned16(dy) || (dx && !aligned16(dx)))) || !aligned16(workspace)) return ACTNN_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   float* ws = static_cast<float*>(workspace);
   switch (dtype) {

@@ -256,9 +256,8 @@ int actnn_linear_grad_weight_q2(const void* grad_out, const int8_t* packed, cons
 
 /* ---------------------------------------------------------------------------------
  * Training-mode batch normalisation over a dense tensor of N samples, C channels and HW
- * positions, laid out [N, C, HW] (channels_last = 0; HW >= 4 for f32, >= 8 for 16-bit types and
- * C*HW a multiple of that - [N, C] inputs with HW = 1 are not covered) or [N, HW, C]
- * (channels_last = 1, the layout of this GPU's convolution kernels; C a multiple of 4 / 8).
+ * positions, laid out [N, C, HW] (channels_last = 0) or [N, HW, C] (channels_last = 1, the
+ * layout of this GPU's convolution kernels).
  * Replaces the two cuDNN calls the reference re-exports, at::cudnn_batch_norm and
  * at::cudnn_batch_norm_backward (cpp_extension/backward_func.cc:87-88; callers ops.py:448-449
  * and ops.py:479-481).  weight/bias (may be null = 1/0), running_* (may be null), save_* and
@@ -272,9 +271,33 @@ int actnn_linear_grad_weight_q2(const void* grad_out, const int8_t* packed, cons
  * backward: dx, dweight, dbias from x, dy and the saved statistics (dx may be null).
  * `workspace`: device scratch of actnn_batch_norm_workspace_bytes(...) bytes (16-byte aligned;
  * -1 = shape not supported), contents undefined before and after.
+ * Shapes: every dense [N, C, HW] / [N, HW, C] tensor is taken.  Rows of whole 16-byte chunks
+ * (C*HW a multiple of 4 for f32, 8 for 16-bit types, HW at least that; channels_last: C such a
+ * multiple) take the streaming kernels; [N, C] inputs (HW = 1) are the channels-last layout
+ * with one pixel per sample and take its kernels whatever `channels_last` says; anything else
+ * goes element by element (correct, a fraction of the speed, no group min/max, no sumsq).
+ * actnn_batch_norm_groups_align: 1 when the quantiser's groups of 256 coincide with runs of
+ * threads of the streaming kernels, i.e. when mn/mx, the packed copy of _forward_apply and
+ * _backward_packed are available for the shape.
  * ------------------------------------------------------------------------------- */
 int64_t actnn_batch_norm_workspace_bytes(int64_t N, int64_t C, int64_t HW, int dtype,
                                          int channels_last);
+int actnn_batch_norm_groups_align(int64_t N, int64_t C, int64_t HW, int dtype, int channels_last);
+/* Evaluation mode (training = false in the reference's batch_norm Function, ops.py:458-461 and
+ * :495-499, which calls at::native_batch_norm / _backward there, backward_func.cc:89-90): the
+ * running estimates are the statistics.  forward_eval: y = (x - running_mean) / sqrt(running_var +
+ * eps) * weight + bias; save_mean / save_invstd (may be null) receive running_mean and
+ * 1 / sqrt(running_var + eps) for the backward call.  backward_eval: dx = dy * weight * invstd
+ * (dx may be null), dweight = sum(dy * (x - mean) * invstd), dbias = sum(dy). */
+int actnn_batch_norm_forward_eval(const void* x, const float* weight, const float* bias,
+                                  const float* running_mean, const float* running_var, void* y,
+                                  float* save_mean, float* save_invstd, void* workspace,
+                                  int64_t workspace_bytes, int64_t N, int64_t C, int64_t HW, double eps,
+                                  int dtype, int channels_last, void* stream);
+int actnn_batch_norm_backward_eval(const void* x, const void* dy, const float* weight,
+                                   const float* mean, const float* invstd, void* dx, float* dweight,
+                                   float* dbias, void* workspace, int64_t workspace_bytes, int64_t N,
+                                   int64_t C, int64_t HW, int dtype, int channels_last, void* stream);
 int actnn_batch_norm_forward(const void* x, const float* weight, const float* bias,
                              float* running_mean, float* running_var, void* y, float* save_mean,
                              float* save_invstd, void* mn, void* mx, void* workspace,

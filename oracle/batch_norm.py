@@ -56,3 +56,29 @@ def backward(x, grad_out, weight, eps):
     grad_input = (w * invstd).reshape(shape) * (
         dy - (grad_bias / count).reshape(shape) - xhat * (grad_weight / count).reshape(shape))
     return grad_input, grad_weight, grad_bias
+
+
+def forward_eval(x, weight, bias, running_mean, running_var, eps):
+    """Evaluation mode -> (y, mean, invstd): the running estimates are the statistics
+    (ops.py:458-461 hands this case to at::native_batch_norm with training = false)."""
+    x = np.asarray(x, np.float64)
+    shape = (1, -1) + (1,) * (x.ndim - 2)
+    mean = np.asarray(running_mean, np.float64)
+    invstd = 1.0 / np.sqrt(np.asarray(running_var, np.float64) + eps)
+    w = np.ones_like(mean) if weight is None else np.asarray(weight, np.float64)
+    b = np.zeros_like(mean) if bias is None else np.asarray(bias, np.float64)
+    return (x - mean.reshape(shape)) * (invstd * w).reshape(shape) + b.reshape(shape), mean, invstd
+
+
+def backward_eval(x, grad_out, weight, running_mean, running_var, eps):
+    """Evaluation mode -> (grad_input, grad_weight, grad_bias): the statistics are constants, so
+    grad_input = dy * weight * invstd, grad_weight = sum(dy * xhat), grad_bias = sum(dy)."""
+    x = np.asarray(x, np.float64)
+    dy = np.asarray(grad_out, np.float64)
+    axes = (0,) + tuple(range(2, x.ndim))
+    shape = (1, -1) + (1,) * (x.ndim - 2)
+    mean = np.asarray(running_mean, np.float64)
+    invstd = 1.0 / np.sqrt(np.asarray(running_var, np.float64) + eps)
+    w = np.ones_like(mean) if weight is None else np.asarray(weight, np.float64)
+    xhat = (x - mean.reshape(shape)) * invstd.reshape(shape)
+    return dy * (w * invstd).reshape(shape), (dy * xhat).sum(axes), dy.sum(axes)

@@ -33,18 +33,25 @@ def test_argument_errors_need_no_gpu(lib):
     assert lib.actnn_relu_forward(None, None, None, -1, 0, None) == -1
     assert lib.actnn_relu_forward(None, None, None, 0, 7, None) == 0
     assert lib.actnn_max_pool2d_forward(None, None, None, 1, 1, 8, 8, 4, 4, 4, 4, 2, 2, 1, 1, 0, None) == -1
-    # batch norm: shapes outside the kernels' reach are reported through the workspace query
+    # batch norm takes every dense shape; the quantiser's outputs only where its groups align
     assert lib.actnn_batch_norm_workspace_bytes(8, 64, 56 * 56, 2, 0) > 0
     assert lib.actnn_batch_norm_workspace_bytes(8, 64, 56 * 56, 2, 1) > 0
-    assert lib.actnn_batch_norm_workspace_bytes(32, 10, 1, 0, 0) == -1            # [N, C] rows, default layout
-    assert lib.actnn_batch_norm_workspace_bytes(4, 3, 49, 2, 0) == -1             # C*HW not in whole 16-byte chunks
-    assert lib.actnn_batch_norm_workspace_bytes(4, 12, 49, 2, 1) == -1            # channels-last: C % 8 != 0
+    assert lib.actnn_batch_norm_workspace_bytes(32, 10, 1, 0, 0) > 0              # [N, C] rows, C % 4 != 0: element by element
+    assert lib.actnn_batch_norm_workspace_bytes(32, 512, 1, 2, 0) > 0             # [N, C] rows: the channels-last kernels
+    assert lib.actnn_batch_norm_workspace_bytes(4, 3, 49, 2, 0) > 0               # C*HW not in whole 16-byte chunks
+    assert lib.actnn_batch_norm_workspace_bytes(4, 12, 49, 2, 1) > 0              # channels-last: C % 8 != 0
+    assert lib.actnn_batch_norm_workspace_bytes(0, 12, 49, 2, 1) == -1
+    assert lib.actnn_batch_norm_groups_align(8, 64, 56 * 56, 2, 0) == 1
+    assert lib.actnn_batch_norm_groups_align(32, 512, 1, 2, 0) == 1               # [N, 512]: two groups per row
+    assert lib.actnn_batch_norm_groups_align(32, 100, 1, 2, 0) == 0
+    assert lib.actnn_batch_norm_groups_align(4, 3, 49, 2, 0) == 0
+    assert lib.actnn_batch_norm_groups_align(8, 192, 64, 2, 1) == 0               # channels-last: 256 % C and C % 256 != 0
     assert lib.actnn_batch_norm_forward(None, None, None, None, None, None, None, None, None, None, None, 0,
                                         8, 64, 3136, 0.1, 1e-5, 2, 0, None) == -1   # null pointers
     assert lib.actnn_batch_norm_backward_packed(None, None, None, None, None, None, None, None, None, None, None,
                                                 None, None, 0, None, 0, 8, 64, 3136, 7, 0, None) == -2   # unknown dtype code
     assert lib.actnn_batch_norm_backward_sumsq_entries(8, 64, 3136, 2, 0) > 0
-    assert lib.actnn_batch_norm_backward_sumsq_entries(4, 3, 49, 2, 0) == -1
+    assert lib.actnn_batch_norm_backward_sumsq_entries(4, 3, 49, 2, 0) == 0       # element-by-element kernels leave none
     assert lib.actnn_sample_sqnorm(None, None, 4, 30, 1, 2, None) == -1           # F % 8 != 0
     assert lib.actnn_max_pool2d_forward_cl(None, None, None, 1, 8, 8, 8, 4, 4, 4, 4, 2, 2, 1, 1, 0, None) == -1
     for name in ("actnn_max_pool2d_forward_nibble", "actnn_max_pool2d_forward_cl_nibble",

@@ -18,7 +18,11 @@ pytestmark = pytest.mark.gpu
 # (49, 196, 12, 10), several spans per channel, one span over many channels, ragged batch splits
 SHAPES = [(8, 64, (112, 112)), (8, 16, (56, 56)), (5, 32, (28, 28)), (37, 24, (14, 14)),
           (16, 256, (7, 7)), (3, 6, (4, 3)), (9, 4, (10,)), (2, 8, (3, 4, 5)), (70, 8, (8, 8)),
-          (4, 2048, (7, 7)), (1, 8, (16, 16))]
+          (4, 2048, (7, 7)), (1, 8, (16, 16)),
+          # [N, C] inputs (the channels-last kernels with one pixel per sample), and shapes that are
+          # not whole 16-byte chunks per row or per plane (element by element)
+          (32, 512, ()), (64, 104, ()), (300, 8, ()), (33, 10, ()), (4, 3, (7, 7)), (6, 5, (3,)), (5, 4, (1, 1)),
+          (70000, 3, (1,))]
 RND = {torch.float32: 2.0 ** -19, torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}
 
 
@@ -80,7 +84,8 @@ def test_against_torch_batch_norm_and_autograd(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("N,C,spatial", [(8, 64, (56, 56)), (5, 256, (7, 7)), (9, 64, (14, 14)), (3, 8, (8, 4))])
+@pytest.mark.parametrize("N,C,spatial", [(8, 64, (56, 56)), (5, 256, (7, 7)), (9, 64, (14, 14)), (3, 8, (8, 4)),
+                                         (40, 512, ()), (7, 256, ())])
 def test_group_min_max_from_the_statistics_pass(N, C, spatial, dtype):
     x, w, b, rm, rv, _ = _inputs(N, C, spatial, dtype, 11)
     y0, m0, i0, _, _ = ext_bf.hip_batch_norm_forward(x, w, b, rm.clone(), rv.clone(), 0.1, 1e-5)
@@ -111,21 +116,61 @@ def test_no_affine_no_running_stats_and_fallback_shapes():
     gi, gw, gb = ext_bf.cudnn_batch_norm_backward(x, dy, None, None, None, mean, invstd, 1e-5, None)
     gi_o, _, gb_o = o_bn.backward(x.double().cpu().numpy(), dy.double().cpu().numpy(), None, 1e-5)
     assert np.allclose(gi.cpu().numpy(), gi_o, rtol=1e-4, atol=1e-5)
-    # shapes the kernels do not take ([N, C] rows, C*HW not a multiple of the chunk) go to ATen
+    # every dense shape runs the library's kernels; tensors that are not dense go to ATen
     for shape in ((32, 10), (4, 3, 7, 7)):
         xs = torch.randn(*shape, device=DEV)
-        assert not ext_bf.hip_batch_norm_applies(xs, None, None, None, None)
-        w = torch.ones(shape[1], device=DEV)
-        b = torch.zeros(shape[1], device=DEV)
-        rm, rv = torch.zeros(shape[1], device=DEV), torch.ones(shape[1], device=DEV)
-        ys = ext_bf.cudnn_batch_norm(xs, w, b, rm, rv, True, 0.1, 1e-5)[0]
-        ref = o_bn.forward(xs.double().cpu().numpy(), None, None, None, None, 0.1, 1e-5)[0]
-        assert np.allclose(ys.cpu().numpy(), ref, rtol=1e-4, atol=1e-4)
+        assert ext_bf.hip_batch_norm_applies(xs, None, None, None, None)
+    xs = torch.randn(8, 6, 5, 5, device=DEV)[:, ::2]
+    assert not ext_bf.hip_batch_norm_applies(xs, None, None, None, None)
+    # affine parameters that are not fp32: ATen's native kernels
+    xh = torch.randn(8, 16, 4, 4, device=DEV, dtype=torch.float16)
+    wh, bh = torch.ones(16, device=DEV, dtype=torch.float16), torch.zeros(16, device=DEV, dtype=torch.float16)
+    assert not ext_bf.hip_batch_norm_applies(xh, wh, bh, None, None)
+    ys = ext_bf.cudnn_batch_norm(xh, wh, bh, None, None, True, 0.1, 1e-5)[0]
+    ref = o_bn.forward(xh.double().cpu().numpy(), None, None, None, None, 0.1, 1e-5)[0]
+    assert np.allclose(ys.double().cpu().numpy(), ref, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,C,spatial,channels_last", [
+    (8, 64, (28, 28), False), (8, 64, (28, 28), True), (5, 24, (7, 7), False), (5, 24, (7, 7), True),
+    (4, 3, (7, 7), False), (4, 3, (7, 7), True), (32, 512, (), False), (33, 10, (), False)])
+def test_evaluation_mode_against_float64_and_torch(N, C, spatial, dtype, channels_last):
+    # training = False in the reference's batch_norm Function (ops.py:458-461, :495-499)
+    x, w, b, rm, rv, dy = _inputs(N, C, spatial, dtype, 77 + C)
+    if channels_last:
+        x, dy = _cl(x), _cl(dy)
+    rm0, rv0 = rm.clone(), rv.clone()
+    y, mean, invstd = ext_bf.native_batch_norm(x, w, b, rm, rv, False, 0.1, 1e-5)
+    assert torch.equal(rm, rm0) and torch.equal(rv, rv0)             # the running estimates are only read
+    assert y.dtype == dtype and y.stride() == x.stride()
+    yo, mean_o, invstd_o = o_bn.forward_eval(x.double().cpu().numpy(), w.cpu().numpy(), b.cpu().numpy(),
+                                             rm.cpu().numpy(), rv.cpu().numpy(), 1e-5)
+    assert np.allclose(mean.cpu().numpy(), mean_o, rtol=1e-6) and np.allclose(invstd.cpu().numpy(), invstd_o, rtol=1e-6)
+    err = np.abs(y.double().cpu().numpy() - yo)
+    assert (err <= RND[dtype] * (np.abs(yo) + 4.0)).all(), float(err.max())
+    gi, gw, gb = ext_bf.native_batch_norm_backward(dy, x, w, rm, rv, mean, invstd, False, 1e-5, [True, True, True])
+    gi_o, gw_o, gb_o = o_bn.backward_eval(x.double().cpu().numpy(), dy.double().cpu().numpy(), w.cpu().numpy(),
+                                          rm.cpu().numpy(), rv.cpu().numpy(), 1e-5)
+    scale = np.sqrt(x.numel() / C)
+    assert np.allclose(gb.cpu().numpy(), gb_o, rtol=1e-5, atol=2e-5 * scale)
+    assert np.allclose(gw.cpu().numpy(), gw_o, rtol=1e-5, atol=8e-5 * scale)
+    err = np.abs(gi.double().cpu().numpy() - gi_o)
+    assert (err <= RND[dtype] * (np.abs(gi_o) + 4.0)).all(), float(err.max())
+    # the same through autograd against torch's own evaluation-mode batch norm; empty saved
+    # statistics (what ATen's forward returns in this mode) are rebuilt from the running estimates
+    gi2, gw2, gb2 = ext_bf.native_batch_norm_backward(dy, x, w, rm, rv, x.new_empty(0), x.new_empty(0), False, 1e-5,
+                                                      [True, False, True])
+    assert gw2 is None and torch.equal(gb2, gb)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    xt = x.detach().clone().requires_grad_(True)
+    F.batch_norm(xt, rm, rv, w, b, False, 0.1, 1e-5).backward(dy)
+    assert torch.allclose(gi2.float(), xt.grad.float(), rtol=tol, atol=tol)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("N,C,spatial", [(8, 64, (56, 56)), (16, 256, (7, 7)), (37, 64, (14, 14)),
-                                         (9, 32, (4, 2)), (12, 128, (28, 28))])
+                                         (9, 32, (4, 2)), (12, 128, (28, 28)), (70, 512, ()), (9, 256, ())])
 def test_backward_from_the_packed_stream_equals_unpack_then_backward(N, C, spatial, dtype):
     """The fused pass rebuilds x exactly as unpack_mixed_precision does, so every output is
     bit-identical to the two-step path, for every width 1..8 in one batch."""
@@ -201,7 +246,8 @@ def _cl(t):
 
 
 CL_SHAPES = [(8, 64, (56, 56)), (16, 256, (7, 7)), (5, 32, (28, 28)), (37, 24, (14, 14)),
-             (4, 2048, (7, 7)), (3, 320, (5, 5)), (2, 16, (3, 4, 5)), (70, 8, (8, 8)), (2, 512, (28, 28))]
+             (4, 2048, (7, 7)), (3, 320, (5, 5)), (2, 16, (3, 4, 5)), (70, 8, (8, 8)), (2, 512, (28, 28)),
+             (4, 12, (7, 7)), (3, 20, (4, 4)), (2, 3, (9, 5))]          # C not a whole chunk: element by element
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
@@ -278,10 +324,11 @@ def test_channels_last_backward_from_the_packed_stream(N, C, spatial, dtype):
                  lambda: ext_bf.hip_batch_norm_backward(xq, dy, w, mean, invstd, sumsq=True), ref)
 
 
-@pytest.mark.parametrize("channels_last", [False, True])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("N,C,spatial", [(8, 64, (56, 56)), (16, 256, (7, 7)), (37, 128, (14, 14)),
-                                         (9, 32, (4, 2)), (5, 1024, (6, 6)), (70, 64, (8, 8))])
+@pytest.mark.parametrize("N,C,spatial,channels_last",
+                         [(n, c, sp, cl) for (n, c, sp) in [(8, 64, (56, 56)), (16, 256, (7, 7)), (37, 128, (14, 14)),
+                                                            (9, 32, (4, 2)), (5, 1024, (6, 6)), (70, 64, (8, 8))]
+                          for cl in (False, True)] + [(70, 512, (), False), (9, 256, (), False)])
 def test_forward_with_packed_copy_equals_forward_then_pack(N, C, spatial, dtype, channels_last):
     """The normalising pass that also packs its input: output equal to the plain forward pass,
     stream and scales equal to pack_mixed_precision with the same generator state (every width)."""

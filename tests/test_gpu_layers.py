@@ -417,6 +417,43 @@ def test_batch_norm_fused_and_unfused_paths_save_the_same_stream(channels_last):
         assert torch.allclose(gw, ref[3], rtol=2e-2, atol=2e-1)
 
 
+def test_batch_norm_1d_on_rows_takes_the_fused_passes():
+    """QBatchNorm1d on [N, C] inputs (layers.py:270-310 serves them through the same Function): the
+    fused sequence - statistics + group min/max, allocation, normalise + pack, backward from the
+    stream - runs on the library's kernels and saves the same tuple as the reference's sequence;
+    a width that is not a whole number of groups takes minimax + pack and the plain kernels."""
+    import actnn_amd.cpp_extension.backward_func as ext_bf
+
+    def run(fused, C):
+        config.reset(); QScheme.reset(); QBNScheme.reset()
+        config.fused_bn_pack = config.fused_bn_backward = fused
+        config.perlayer = False
+        torch.manual_seed(0)
+        lin = actnn_amd.QLinear(64, C).to(DEV)
+        bn = actnn_amd.QBatchNorm1d(C).to(DEV)
+        x = torch.randn(96, 64, device=DEV)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            h = lin(x)
+            torch.cuda.manual_seed(11)
+            y = bn(h)
+        saved = y.grad_fn.saved[0]
+        g = torch.randn_like(y)
+        gh, gw = torch.autograd.grad(y, [h, bn.weight], g)
+        return y, saved, gh, gw, h
+    for C in (512, 104):
+        ref = run(False, C)
+        y, saved, gh, gw, h = run(True, C)
+        assert ext_bf.hip_batch_norm_applies(h, None, None, None, None)
+        assert ext_bf.hip_batch_norm_minmax_applies(h, None, None, None, None) == (C % 256 == 0)
+        assert torch.equal(saved[1].cpu(), ref[1][1].cpu())
+        assert torch.equal(saved[0], ref[1][0]) and torch.equal(saved[2], ref[1][2]) and torch.equal(saved[3], ref[1][3])
+        assert torch.allclose(y.float(), ref[0].float(), atol=2e-2, rtol=2e-2)
+        assert torch.allclose(gh.float(), ref[2].float(), atol=3e-2, rtol=3e-2)
+        assert torch.allclose(gw, ref[3], rtol=2e-2, atol=2e-1)
+        exact = torch.nn.functional.batch_norm(h.float(), None, None, None, None, True, 0.1, 1e-5)
+        assert torch.allclose(y.float(), exact * 1.0, atol=3e-2, rtol=3e-2)
+
+
 @pytest.mark.parametrize("channels_last", [False, True])
 @pytest.mark.parametrize("level", ["L0", "L1", "L2", "L3", "L3.1", "L4", "swap"])
 def test_every_optimization_level_trains_a_step(level, channels_last):
