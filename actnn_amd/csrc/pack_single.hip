@@ -32,20 +32,42 @@ __global__ __launch_bounds__(kThreads) void scale_single_kernel(const T* __restr
   }
 }
 
+
+// Where a thread works: the grid's x dimension runs over the G * chunks positions of one row of the
+// stream (chunks = lanes per group), y over the rows (groups of 8/bits samples), so that the group
+// and the offset inside it come out of one 32-bit shift or division and the sample from blockIdx -
+// no 64-bit divisions per thread (they cost more instructions than the quantisation of the thread's
+// elements: 4-bit pack of bf16 [512,256,56,56] 0.198 -> 0.180 ms, unpack 0.173 -> 0.155 ms).
+struct SingleGeom {
+  int64_t N, G;
+  int gs, chunks, chunk_shift;     // chunk_shift < 0: chunks is not a power of two
+  int64_t rows;                    // ceil(N / (8 / bits))
+  uint32_t per_row;                // G * chunks
+};
+struct SingleAt { uint32_t g; int d0; bool live; };
+template <int ELEMS> ACTNN_DEV SingleAt single_at(const SingleGeom& q) {
+  const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+  SingleAt a;
+  a.live = i < q.per_row;
+  a.g = q.chunk_shift >= 0 ? i >> q.chunk_shift : i / (uint32_t)q.chunks;
+  a.d0 = (int)(q.chunk_shift >= 0 ? i & (uint32_t)(q.chunks - 1) : i % (uint32_t)q.chunks) * ELEMS;
+  return a;
+}
+
 template <typename T, int BITS, bool DET>
 __global__ __launch_bounds__(kThreads) void pack_single_kernel(
     const T* __restrict__ data, const T* __restrict__ mn, const T* __restrict__ scale,
     int8_t* __restrict__ packed, const T* __restrict__ noise, uint64_t seed, uint64_t offset,
-    int64_t N, int64_t G, int gs, int64_t units) {
+    SingleGeom q) {
   constexpr int WPT = 8 / BITS;
   constexpr float Bf = (float)((1 << BITS) - 1);
-  const int64_t u = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-  if (u >= units) return;
-  const int chunks = gs / 8;
-  const int64_t og = u / chunks;            // no * G + g
-  const int d0 = (int)(u % chunks) * 8;
-  const int64_t no = og / G;
-  const int64_t g = og % G;
+  const SingleAt at = single_at<8>(q);
+  if (!at.live) return;
+  const int64_t N = q.N, G = q.G;
+  const int gs = q.gs, chunks = q.chunks, d0 = at.d0;
+  const int64_t g = at.g;
+  for (int64_t no = blockIdx.y; no < q.rows; no += gridDim.y) {
+  const int64_t og = no * G + g;
 
   float v[WPT][8];
   float nz[DET ? WPT : 1][8];
@@ -116,35 +138,36 @@ __global__ __launch_bounds__(kThreads) void pack_single_kernel(
     hi = shi.lo;
   }
   *reinterpret_cast<uint2*>(packed + og * gs + d0) = make_uint2(lo, hi);
+  }
 }
 
 template <typename T, int BITS>
 __global__ __launch_bounds__(kThreads) void unpack_single_kernel(
     const int8_t* __restrict__ packed, const T* __restrict__ scale, const T* __restrict__ mn,
-    T* __restrict__ out, int64_t N, int64_t G, int gs, int64_t units) {
+    T* __restrict__ out, SingleGeom q) {
   constexpr int WPT = 8 / BITS;
   constexpr uint32_t kMask = (1u << BITS) - 1u;
-  const int64_t u = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-  if (u >= units) return;
-  const int chunks = gs / 8;
-  const int64_t og = u / chunks;
-  const int d0 = (int)(u % chunks) * 8;
-  const int64_t no = og / G;
-  const int64_t g = og % G;
-  const uint2 w = *reinterpret_cast<const uint2*>(packed + og * gs + d0);
+  const SingleAt at = single_at<8>(q);
+  if (!at.live) return;
+  const int64_t N = q.N, G = q.G, g = at.g;
+  const int gs = q.gs, d0 = at.d0;
+  for (int64_t no = blockIdx.y; no < q.rows; no += gridDim.y) {
+    const int64_t og = no * G + g;
+    const uint2 w = *reinterpret_cast<const uint2*>(packed + og * gs + d0);
 #pragma unroll
-  for (int ni = 0; ni < WPT; ++ni) {
-    const int64_t n = no * WPT + ni;
-    if (n < N) {
-      const int64_t gi = n * G + g;
-      const Dequant<T> dq(Conv<T>::load(scale, gi), Conv<T>::load(mn, gi));
-      float v[8];
+    for (int ni = 0; ni < WPT; ++ni) {
+      const int64_t n = no * WPT + ni;
+      if (n < N) {
+        const int64_t gi = n * G + g;
+        const Dequant<T> dq(Conv<T>::load(scale, gi), Conv<T>::load(mn, gi));
+        float v[8];
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const uint32_t word = k < 4 ? w.x : w.y;
-        v[k] = dq((word >> (8 * (k & 3) + ni * BITS)) & kMask);
+        for (int k = 0; k < 8; ++k) {
+          const uint32_t word = k < 4 ? w.x : w.y;
+          v[k] = dq((word >> (8 * (k & 3) + ni * BITS)) & kMask);
+        }
+        store8_nt(out + gi * gs + d0, v);
       }
-      store8_nt(out + gi * gs + d0, v);
     }
   }
 }
@@ -153,45 +176,64 @@ __global__ __launch_bounds__(kThreads) void unpack_single_kernel(
 template <int BITS>
 __global__ __launch_bounds__(kThreads) void unpack_single_f32_kernel(
     const int8_t* __restrict__ packed, const float* __restrict__ scale, const float* __restrict__ mn,
-    float* __restrict__ out, int64_t N, int64_t G, int gs, int64_t units) {
+    float* __restrict__ out, SingleGeom q) {
   constexpr int WPT = 8 / BITS;
   constexpr uint32_t kMask = (1u << BITS) - 1u;
-  const int64_t u = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-  if (u >= units) return;
-  const int chunks = gs / 4;
-  const int64_t og = u / chunks;
-  const int d0 = (int)(u % chunks) * 4;
-  const int64_t no = og / G;
-  const int64_t g = og % G;
-  const uint32_t w = *reinterpret_cast<const uint32_t*>(packed + og * gs + d0);
+  const SingleAt at = single_at<4>(q);
+  if (!at.live) return;
+  const int64_t N = q.N, G = q.G, g = at.g;
+  const int gs = q.gs, d0 = at.d0;
+  for (int64_t no = blockIdx.y; no < q.rows; no += gridDim.y) {
+    const int64_t og = no * G + g;
+    const uint32_t w = *reinterpret_cast<const uint32_t*>(packed + og * gs + d0);
 #pragma unroll
-  for (int ni = 0; ni < WPT; ++ni) {
-    const int64_t n = no * WPT + ni;
-    if (n < N) {
-      const int64_t gi = n * G + g;
-      const Dequant<float> dq(scale[gi], mn[gi]);
-      u32x4 v;
+    for (int ni = 0; ni < WPT; ++ni) {
+      const int64_t n = no * WPT + ni;
+      if (n < N) {
+        const int64_t gi = n * G + g;
+        const Dequant<float> dq(scale[gi], mn[gi]);
+        u32x4 v;
 #pragma unroll
-      for (int k = 0; k < 4; ++k) v[k] = as_uint(dq((w >> (8 * k + ni * BITS)) & kMask));
-      store16_nt(out + gi * gs + d0, v);
+        for (int k = 0; k < 4; ++k) v[k] = as_uint(dq((w >> (8 * k + ni * BITS)) & kMask));
+        store16_nt(out + gi * gs + d0, v);
+      }
     }
   }
+}
+
+// grid: x over the G * (gs / elems) lane positions of a stream row, y over the rows (capped; the
+// kernels stride over the rest)
+bool single_geometry(int64_t N, int64_t G, int64_t gs, int bits, int elems, SingleGeom& q, dim3& grid) {
+  const int wpt = 8 / bits;
+  q.N = N;
+  q.G = G;
+  q.gs = (int)gs;
+  q.chunks = (int)(gs / elems);
+  q.chunk_shift = -1;
+  for (int sh = 0; sh < 31; ++sh)
+    if ((1 << sh) == q.chunks) q.chunk_shift = sh;
+  q.rows = (N + wpt - 1) / wpt;
+  const int64_t per_row = G * q.chunks;
+  if (per_row > 0x7fffffffLL || gs > 0x7fffffffLL) return false;
+  q.per_row = (uint32_t)per_row;
+  const int64_t bx = (per_row + kThreads - 1) / kThreads;
+  grid = dim3((unsigned)bx, (unsigned)(q.rows < 65535 ? q.rows : 65535));
+  return true;
 }
 
 template <typename T, bool DET>
 int launch_pack_bits(int bits, const T* data, const T* mn, const T* scale, int8_t* packed,
                      const T* noise, uint64_t seed, uint64_t offset, int64_t N, int64_t G, int gs,
                      hipStream_t s) {
-  const int wpt = 8 / bits;
-  const int64_t units = ((N + wpt - 1) / wpt) * G * (gs / 8);
-  const int64_t blocks = (units + kThreads - 1) / kThreads;
-  if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
-  const dim3 grid((unsigned)blocks), blk(kThreads);
+  SingleGeom q;
+  dim3 grid;
+  if (!single_geometry(N, G, gs, bits, 8, q, grid)) return ACTNN_EINVAL;
+  const dim3 blk(kThreads);
   switch (bits) {
-    case 1: pack_single_kernel<T, 1, DET><<<grid, blk, 0, s>>>(data, mn, scale, packed, noise, seed, offset, N, G, gs, units); break;
-    case 2: pack_single_kernel<T, 2, DET><<<grid, blk, 0, s>>>(data, mn, scale, packed, noise, seed, offset, N, G, gs, units); break;
-    case 4: pack_single_kernel<T, 4, DET><<<grid, blk, 0, s>>>(data, mn, scale, packed, noise, seed, offset, N, G, gs, units); break;
-    case 8: pack_single_kernel<T, 8, DET><<<grid, blk, 0, s>>>(data, mn, scale, packed, noise, seed, offset, N, G, gs, units); break;
+    case 1: pack_single_kernel<T, 1, DET><<<grid, blk, 0, s>>>(data, mn, scale, packed, noise, seed, offset, q); break;
+    case 2: pack_single_kernel<T, 2, DET><<<grid, blk, 0, s>>>(data, mn, scale, packed, noise, seed, offset, q); break;
+    case 4: pack_single_kernel<T, 4, DET><<<grid, blk, 0, s>>>(data, mn, scale, packed, noise, seed, offset, q); break;
+    case 8: pack_single_kernel<T, 8, DET><<<grid, blk, 0, s>>>(data, mn, scale, packed, noise, seed, offset, q); break;
     default: return ACTNN_EBITS;
   }
   ACTNN_RETURN_LAUNCH_STATUS();
@@ -221,36 +263,32 @@ int launch_pack(const void* data, const void* mn, const void* mx, int bits, void
 template <typename T>
 int launch_unpack(const int8_t* packed, int bits, const void* scale, const void* mn, void* out,
                   int64_t N, int64_t G, int64_t gs, hipStream_t s) {
-  const int wpt = 8 / bits;
+  SingleGeom q;
+  dim3 grid;
+  const dim3 blk(kThreads);
   if constexpr (sizeof(T) == 4) {
-    const int64_t units4 = ((N + wpt - 1) / wpt) * G * (gs / 4);
-    const int64_t blocks4 = (units4 + kThreads - 1) / kThreads;
-    if (blocks4 > 0x7fffffffLL) return ACTNN_EINVAL;
-    const dim3 grid4((unsigned)blocks4), blk4(kThreads);
+    if (gs % 4 != 0 || !single_geometry(N, G, gs, bits, 4, q, grid)) return ACTNN_EINVAL;
     const float* sc4 = static_cast<const float*>(scale);
     const float* lo4 = static_cast<const float*>(mn);
     float* o4 = static_cast<float*>(out);
     switch (bits) {
-      case 1: unpack_single_f32_kernel<1><<<grid4, blk4, 0, s>>>(packed, sc4, lo4, o4, N, G, (int)gs, units4); break;
-      case 2: unpack_single_f32_kernel<2><<<grid4, blk4, 0, s>>>(packed, sc4, lo4, o4, N, G, (int)gs, units4); break;
-      case 4: unpack_single_f32_kernel<4><<<grid4, blk4, 0, s>>>(packed, sc4, lo4, o4, N, G, (int)gs, units4); break;
-      case 8: unpack_single_f32_kernel<8><<<grid4, blk4, 0, s>>>(packed, sc4, lo4, o4, N, G, (int)gs, units4); break;
+      case 1: unpack_single_f32_kernel<1><<<grid, blk, 0, s>>>(packed, sc4, lo4, o4, q); break;
+      case 2: unpack_single_f32_kernel<2><<<grid, blk, 0, s>>>(packed, sc4, lo4, o4, q); break;
+      case 4: unpack_single_f32_kernel<4><<<grid, blk, 0, s>>>(packed, sc4, lo4, o4, q); break;
+      case 8: unpack_single_f32_kernel<8><<<grid, blk, 0, s>>>(packed, sc4, lo4, o4, q); break;
       default: return ACTNN_EBITS;
     }
     ACTNN_RETURN_LAUNCH_STATUS();
   }
-  const int64_t units = ((N + wpt - 1) / wpt) * G * (gs / 8);
-  const int64_t blocks = (units + kThreads - 1) / kThreads;
-  if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
-  const dim3 grid((unsigned)blocks), blk(kThreads);
+  if (!single_geometry(N, G, gs, bits, 8, q, grid)) return ACTNN_EINVAL;
   const T* sc = static_cast<const T*>(scale);
   const T* lo = static_cast<const T*>(mn);
   T* o = static_cast<T*>(out);
   switch (bits) {
-    case 1: unpack_single_kernel<T, 1><<<grid, blk, 0, s>>>(packed, sc, lo, o, N, G, (int)gs, units); break;
-    case 2: unpack_single_kernel<T, 2><<<grid, blk, 0, s>>>(packed, sc, lo, o, N, G, (int)gs, units); break;
-    case 4: unpack_single_kernel<T, 4><<<grid, blk, 0, s>>>(packed, sc, lo, o, N, G, (int)gs, units); break;
-    case 8: unpack_single_kernel<T, 8><<<grid, blk, 0, s>>>(packed, sc, lo, o, N, G, (int)gs, units); break;
+    case 1: unpack_single_kernel<T, 1><<<grid, blk, 0, s>>>(packed, sc, lo, o, q); break;
+    case 2: unpack_single_kernel<T, 2><<<grid, blk, 0, s>>>(packed, sc, lo, o, q); break;
+    case 4: unpack_single_kernel<T, 4><<<grid, blk, 0, s>>>(packed, sc, lo, o, q); break;
+    case 8: unpack_single_kernel<T, 8><<<grid, blk, 0, s>>>(packed, sc, lo, o, q); break;
     default: return ACTNN_EBITS;
   }
   ACTNN_RETURN_LAUNCH_STATUS();
