@@ -237,6 +237,26 @@ ACTNN_DEV int64_t xcd_block() {
   return (int64_t)(blockIdx.x % kXcds) * (gridDim.x / kXcds) + blockIdx.x / kXcds;
 }
 
+// Division of a 32-bit unsigned number by a divisor that is fixed at launch: one multiply-high, two
+// shifts and two additions (Granlund & Montgomery, "Division by invariant integers using
+// multiplication", 1994, figure 4.1), exact for every numerator.  Built on the host, passed by value.
+struct FastDiv {
+  uint32_t d, m;
+  int s1, s2;
+  FastDiv() = default;
+  explicit FastDiv(uint32_t divisor) : d(divisor) {
+    int l = 0;
+    while ((uint64_t(1) << l) < divisor) ++l;
+    m = (uint32_t)(((uint64_t(1) << 32) * ((uint64_t(1) << l) - divisor)) / divisor + 1);
+    s1 = l < 1 ? l : 1;
+    s2 = l > 0 ? l - 1 : 0;
+  }
+  ACTNN_DEV uint32_t div(uint32_t n) const {
+    const uint32_t t = __umulhi(n, m);
+    return (t + ((n - t) >> s1)) >> s2;
+  }
+};
+
 template <int D> ACTNN_DEV uint32_t lane_xor(uint32_t x);
 template <> ACTNN_DEV uint32_t lane_xor<1>(uint32_t x) {
   return (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]

@@ -22,7 +22,11 @@ namespace {
 constexpr int kThreads = 256;             // general kernels
 // Stride-2 kernels (measured on 256x64x112x112 f16): the forward likes tall bands and streamed
 // (non-temporal) staging loads; the backward, whose bands share their edge rows and whose cache
-// lines are split between neighbouring blocks, likes short bands and cached loads.
+// lines are split between neighbouring blocks, likes short bands and cached loads (256 threads:
+// 0.114 ms, two passes per block: 0.138 ms, against 0.105 ms).  The backward issues as many vector
+// instructions as fit its run time (counters: one per 4 cycles and SIMD), so what it saves in
+// staging and index arithmetic shows directly: staging both spans in one round and dividing by
+// multiply-high took it from 0.117 to 0.105 ms on the same machine.
 constexpr int kFwdS2Threads = 256, kFwdS2Passes = 4;
 constexpr int kBwdS2Threads = 128, kBwdS2Passes = 1;
 
@@ -47,6 +51,9 @@ template <bool NIB> struct IndexFields {
   static constexpr int kBits = NIB ? 4 : 8;
   static constexpr uint32_t kMask = NIB ? 0xfu : 0xffu;
   static ACTNN_DEV int get(uint64_t fields, int e) { return (int)((uint32_t)(fields >> (kBits * e)) & kMask); }
+  // bytes from the start of idx to the field of output o (o even)
+  static ACTNN_DEV uint32_t byte_of(uint32_t o) { return NIB ? o >> 1 : o; }
+  static ACTNN_DEV int64_t byte_of(int64_t o) { return NIB ? o >> 1 : o; }
   template <int E, typename P> static ACTNN_DEV void store(P* idx, int64_t o, uint64_t fields) {
     P* at = idx + (NIB ? o >> 1 : o);
     if constexpr (E * kBits == 16) *reinterpret_cast<uint16_t*>(at) = (uint16_t)fields;
@@ -170,6 +177,45 @@ ACTNN_DEV int stage_span(const T* __restrict__ src, int64_t first, int count, in
       if (e + i < total) dst[(nvec - 1) * V + i] = src[e + i];
   }
   return shift;
+}
+
+// Two spans staged together: the loads of both are issued before the first LDS write, so a short
+// band pays one round trip to memory, not two.
+template <typename T> struct Span {
+  const T* base;          // aligned start
+  int whole;              // 16-byte vectors that lie inside the tensor
+  int tail;               // elements of the ragged last vector (0: none)
+  int shift;              // position of the span's first element in the staged copy
+};
+template <typename T> ACTNN_DEV Span<T> span_of(const T* __restrict__ src, int64_t first, int count, int64_t total) {
+  constexpr int V = 16 / (int)sizeof(T);
+  Span<T> sp;
+  sp.shift = (int)(first & (V - 1));
+  const int64_t base = first - sp.shift;
+  const int nvec = (sp.shift + count + V - 1) / V;
+  const bool ragged = base + (int64_t)nvec * V > total;          // only the last vector can reach past the end
+  sp.base = src + base;
+  sp.whole = ragged ? nvec - 1 : nvec;
+  sp.tail = ragged ? (int)(total - base - (int64_t)(nvec - 1) * V) : 0;
+  return sp;
+}
+template <int THREADS, typename A, typename B>
+ACTNN_DEV void stage_two(const Span<A>& a, A* da, const Span<B>& b, B* db) {
+  constexpr int VA = 16 / (int)sizeof(A), VB = 16 / (int)sizeof(B);
+  const int most = a.whole > b.whole ? a.whole : b.whole;
+#pragma unroll 1
+  for (int v = threadIdx.x; v < most; v += THREADS) {
+    u32x4 x, y;
+    const bool in_a = v < a.whole, in_b = v < b.whole;
+    if (in_a) x = load16(a.base + v * VA);
+    if (in_b) y = load16(b.base + v * VB);
+    if (in_a) reinterpret_cast<u32x4*>(da)[v] = x;
+    if (in_b) reinterpret_cast<u32x4*>(db)[v] = y;
+  }
+#pragma unroll 1
+  for (int i = threadIdx.x; i < a.tail; i += THREADS) da[a.whole * VA + i] = a.base[a.whole * VA + i];
+#pragma unroll 1
+  for (int i = threadIdx.x; i < b.tail; i += THREADS) db[b.whole * VB + i] = b.base[b.whole * VB + i];
 }
 
 template <typename T> ACTNN_DEV float lds_value(const T* p, int i);
@@ -406,7 +452,7 @@ __global__ __launch_bounds__(kFwdS2Threads) void max_pool2d_forward_s2_kernel(
 template <typename T, int K, int P, bool NIB>
 __global__ __launch_bounds__(kBwdS2Threads) void max_pool2d_backward_s2_kernel(
     const T* __restrict__ gout, const int8_t* __restrict__ idx, T* __restrict__ gin, int64_t total_out,
-    PoolGeom g, int pairs_per_band, int bands, int max_out_rows) {
+    PoolGeom g, int pairs_per_band, int bands, int max_out_rows, FastDiv by_cpr) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   constexpr int EXTRA = K == 3 ? 1 : 0;                 // windows of the next output row reach odd input rows
   constexpr int NW = 4 + EXTRA;                         // output columns that touch 8 input columns
@@ -418,15 +464,16 @@ __global__ __launch_bounds__(kBwdS2Threads) void max_pool2d_backward_s2_kernel(
   const int ho_hi = s0 + pairs - 1 + EXTRA < g.Ho - 1 ? s0 + pairs - 1 + EXTRA : g.Ho - 1;
   const int64_t first = (nc * g.Ho + s0) * (int64_t)g.Wo;
   const int count = (ho_hi - s0 + 1) * g.Wo;
-  const int shift_g = stage_span<T, kBwdS2Threads, false>(gout, first, count, total_out, s_g);
   // (first and count are multiples of 4: whole bytes in the two-per-byte format)
-  const int shift_i = NIB ? 2 * stage_span<int8_t, kBwdS2Threads, false>(idx, first >> 1, count >> 1, total_out >> 1, s_i)
-                          : stage_span<int8_t, kBwdS2Threads, false>(idx, first, count, total_out, s_i);
+  const Span<T> span_g = span_of(gout, first, count, total_out);
+  const Span<int8_t> span_i = NIB ? span_of(idx, first >> 1, count >> 1, total_out >> 1) : span_of(idx, first, count, total_out);
+  stage_two<kBwdS2Threads>(span_g, s_g, span_i, s_i);
+  const int shift_g = span_g.shift, shift_i = NIB ? 2 * span_i.shift : span_i.shift;
   __syncthreads();
   const int cpr = g.W >> 3;
   const int items = pairs * cpr;
   for (int item = threadIdx.x; item < items; item += kBwdS2Threads) {
-    const int r = item / cpr, q = item - r * cpr;
+    const int r = (int)by_cpr.div((uint32_t)item), q = item - r * cpr;
     float gv[1 + EXTRA][NW];
     int iv[1 + EXTRA][NW];
 #pragma unroll
@@ -570,8 +617,8 @@ int launch_bwd(const void* gout, const int8_t* idx, void* gin, int64_t total, co
       const T* go = static_cast<const T*>(gout);
       T* gi = static_cast<T*>(gin);
       const int64_t tout = planes * g.Ho * g.Wo;
-      if (k == 3) max_pool2d_backward_s2_kernel<T, 3, 1, NIB><<<grid, blk, need2(pb), s>>>(go, idx, gi, tout, g, pb, bands, pb + 2);
-      else max_pool2d_backward_s2_kernel<T, 2, 0, NIB><<<grid, blk, need2(pb), s>>>(go, idx, gi, tout, g, pb, bands, pb + 2);
+      if (k == 3) max_pool2d_backward_s2_kernel<T, 3, 1, NIB><<<grid, blk, need2(pb), s>>>(go, idx, gi, tout, g, pb, bands, pb + 2, FastDiv((uint32_t)(g.W / 8)));
+      else max_pool2d_backward_s2_kernel<T, 2, 0, NIB><<<grid, blk, need2(pb), s>>>(go, idx, gi, tout, g, pb, bands, pb + 2, FastDiv((uint32_t)(g.W / 8)));
       ACTNN_RETURN_LAUNCH_STATUS();
     }
   }
@@ -636,8 +683,13 @@ template <typename T, int E> ACTNN_DEV void narrow_chunk(T* p, const float (&v)[
   if constexpr (E == 4) store16(p, u32x4{as_uint(v[0]), as_uint(v[1]), as_uint(v[2]), as_uint(v[3])});
   else store8(p, v);
 }
+// the same as a streamed store: for tensors that are written once and not read by the kernel
+template <typename T, int E> ACTNN_DEV void narrow_chunk_nt(T* p, const float (&v)[E]) {
+  if constexpr (E == 4) store16_nt(p, u32x4{as_uint(v[0]), as_uint(v[1]), as_uint(v[2]), as_uint(v[3])});
+  else store8_nt(p, v);
+}
 
-template <typename T, int PRESET, bool NIB>
+template <typename T, bool NIB>
 __global__ __launch_bounds__(kThreads) void max_pool2d_forward_cl_kernel(
     const T* __restrict__ x, T* __restrict__ y, int8_t* __restrict__ idx, int64_t chunks, int cpp /* chunks per pixel */,
     int64_t C, PoolGeom g) {
@@ -659,40 +711,14 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_forward_cl_kernel(
 #pragma unroll
   for (int e = 0; e < E; ++e) { best[e] = init; where[e] = 0; }
   const T* img = x + n * (int64_t)g.H * g.W * C + c;
-  if constexpr (PRESET != 0) {
-    // window known at compile time: all its loads are issued before the first comparison (taken one
-    // at a time, as the loop below does, their latencies add up); positions outside the image get the
-    // start value, which never wins the strict compare
-    const Win<PRESET> k(g);
-    constexpr int KH = PRESET == 2 ? 2 : 3, KW = KH;
-    u32x4 raw[KH * KW];
-    const uint32_t fill = dword_of<T>(init);
-#pragma unroll
-    for (int a = 0; a < KH; ++a)
-#pragma unroll
-      for (int b = 0; b < KW; ++b) {
-        const int i = h * k.SH - k.PH + a, j = w * k.SW - k.PW + b;
-        raw[a * KW + b] = (i >= 0 && i < g.H && j >= 0 && j < g.W) ? load16(img + ((int64_t)i * g.W + j) * C)
-                                                                 : u32x4{fill, fill, fill, fill};
-      }
-#pragma unroll
-    for (int q = 0; q < KH * KW; ++q) {
+  for (int i = h_start; i < h_end; ++i) {
+    for (int j = w_start; j < w_end; ++j) {
       float v[E];
-      raw_widen_chunk<T, E>(raw[q], v);
+      widen_chunk<T, E>(img + ((int64_t)i * g.W + j) * C, v);
+      const int k = (i - h_base) * g.KW + (j - w_base);
 #pragma unroll
       for (int e = 0; e < E; ++e)
-        if (v[e] > best[e]) { best[e] = v[e]; where[e] = q; }
-    }
-  } else {
-    for (int i = h_start; i < h_end; ++i) {
-      for (int j = w_start; j < w_end; ++j) {
-        float v[E];
-        widen_chunk<T, E>(img + ((int64_t)i * g.W + j) * C, v);
-        const int k = (i - h_base) * g.KW + (j - w_base);
-#pragma unroll
-        for (int e = 0; e < E; ++e)
-          if (v[e] > best[e]) { best[e] = v[e]; where[e] = k; }
-      }
+        if (v[e] > best[e]) { best[e] = v[e]; where[e] = k; }
     }
   }
   narrow_chunk<T, E>(y + pix * C + c, best);
@@ -700,6 +726,87 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_forward_cl_kernel(
 #pragma unroll
   for (int e = 0; e < E; ++e) fields |= (uint64_t)where[e] << (IndexFields<NIB>::kBits * e);
   IndexFields<NIB>::template store<E>(idx, pix * C + c, fields);
+}
+
+// Where a thread of the window kernels below works, without 64-bit arithmetic (which costs more
+// instructions than the window itself: these kernels are bound by the vector ALUs, not by memory).
+// Blocks are numbered image by image; a thread's number inside its image (below 2^31) splits into
+// pixel row, column and chunk of channels by multiply-high divisions, and every address is a
+// uniform base (image, window position) plus one 32-bit lane offset.
+struct ClGeom {
+  uint32_t cpp, cols;                     // chunks per pixel; pixels per row of the thread grid
+  uint32_t per_image;                     // threads per image: rows * cols * cpp
+  uint32_t blocks_per_image, blocks;
+  FastDiv by_cpp, by_cols, by_blocks_per_image;
+};
+struct ClAt {
+  uint32_t n, i, row, col, chunk;
+  bool live;
+};
+ACTNN_DEV ClAt cl_at(const ClGeom& q) {
+  ClAt a;
+  // (neighbouring rows share input rows or windows: their blocks stay on one XCD)
+  const uint32_t block = (blockIdx.x % kXcds) * (gridDim.x / kXcds) + blockIdx.x / kXcds;
+  a.n = q.by_blocks_per_image.div(block);
+  a.i = (block - a.n * q.blocks_per_image) * kThreads + threadIdx.x;
+  a.live = block < q.blocks && a.i < q.per_image;
+  const uint32_t pixel = q.by_cpp.div(a.i);
+  a.chunk = a.i - pixel * q.cpp;
+  a.row = q.by_cols.div(pixel);
+  a.col = pixel - a.row * q.cols;
+  return a;
+}
+
+// Forward for the windows known at compile time (the presets): all loads of the window are issued
+// before the first comparison (taken one at a time their latencies add up); positions outside the
+// image get the start value, which never wins the strict compare.  Same scan order as above.
+template <typename T, int PRESET, bool NIB>
+__global__ __launch_bounds__(kThreads) void max_pool2d_forward_cl_window_kernel(
+    const T* __restrict__ x, T* __restrict__ y, int8_t* __restrict__ idx, ClGeom q, PoolGeom g) {
+  constexpr int E = PoolChunk<T>::kElems;
+  constexpr int KH = PRESET == 2 ? 2 : 3, KW = KH;
+  const Win<PRESET> k(g);
+  const ClAt at = cl_at(q);
+  if (!at.live) return;
+  const uint32_t C = q.cpp * E;
+  const int i0 = (int)at.row * k.SH - k.PH, j0 = (int)at.col * k.SW - k.PW;
+  // the lane's offset counts from the window origin moved by the padding, so it is never negative;
+  // the uniform bases take the padding back
+  const uint32_t lane = ((at.row * k.SH) * (uint32_t)g.W + at.col * k.SW) * C + at.chunk * E;
+  const T* img = x + (int64_t)at.n * g.H * g.W * C;
+  const float init = Conv<T>::round(-1e10f);      // .cu:656, narrowed to the element type
+  const uint32_t fill = dword_of<T>(init);
+  u32x4 raw[KH * KW];
+#pragma unroll
+  for (int a = 0; a < KH; ++a)
+#pragma unroll
+    for (int b = 0; b < KW; ++b) {
+      const bool inside = (uint32_t)(i0 + a) < (uint32_t)g.H && (uint32_t)(j0 + b) < (uint32_t)g.W;
+      const T* base = img + ((int64_t)(a - k.PH) * g.W + (b - k.PW)) * (int64_t)C;
+      // pixels that no other window reads (every pixel of a 2x2 stride-2 window, the centre of a 3x3
+      // stride-2 one) are streamed; the others are read again by the neighbours and stay cached
+      const bool once = PRESET == 2 || (PRESET == 1 && a == 1 && b == 1);   // (constant after unrolling)
+      raw[a * KW + b] = inside ? (once ? load16_nt(base + lane) : load16(base + lane)) : u32x4{fill, fill, fill, fill};
+    }
+  float best[E];
+  int where[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) { best[e] = init; where[e] = 0; }
+#pragma unroll
+  for (int p = 0; p < KH * KW; ++p) {
+    float v[E];
+    raw_widen_chunk<T, E>(raw[p], v);
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+      if (v[e] > best[e]) { best[e] = v[e]; where[e] = p; }
+  }
+  const int64_t image_o = (int64_t)at.n * q.per_image * E;     // outputs before this image
+  const uint32_t lane_o = at.i * E;
+  narrow_chunk_nt<T, E>(y + image_o + lane_o, best);
+  uint64_t fields = 0;
+#pragma unroll
+  for (int e = 0; e < E; ++e) fields |= (uint64_t)where[e] << (IndexFields<NIB>::kBits * e);
+  IndexFields<NIB>::template store<E>(idx + IndexFields<NIB>::byte_of(image_o), (int64_t)lane_o, fields);
 }
 
 // Gather form of the backward pass: every input position sums the gradients of the windows that
@@ -748,20 +855,32 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_backward_cl_kernel(
 // even): a thread owns the 2x2 block of input pixels (2a.., 2b..) of one chunk of channels.  The windows
 // that reach the block are (a..a+1) x (b..b+1) (3x3) or (a, b) alone (2x2): one (gradient, index) load
 // per input pixel where the general kernel needs 2.25 (3x3).  Every pixel adds its windows in the
-// general kernel's order (rows, then columns), hence the same bits.
+// general kernel's order (rows, then columns), hence the same bits.  grad_in is written once and
+// not read: streamed stores (measured 0.104 -> 0.079 ms on f16 [256,64,112,112]).
 template <typename T, int K, int P, bool NIB>
 __global__ __launch_bounds__(kThreads) void max_pool2d_backward_cl_s2_kernel(
-    const T* __restrict__ gout, const int8_t* __restrict__ idx, T* __restrict__ gin, int64_t items, int cpp,
-    int64_t C, PoolGeom g) {
+    const T* __restrict__ gout, const int8_t* __restrict__ idx, T* __restrict__ gin, ClGeom q, PoolGeom g) {
   constexpr int E = PoolChunk<T>::kElems;
   constexpr int NWIN = K == 3 ? 2 : 1;
-  const int64_t id = xcd_block() * kThreads + threadIdx.x;       // neighbouring block rows share windows
-  if (id >= items) return;
-  const int c = (int)(id % cpp) * E;
-  const int64_t blk = id / cpp;
-  const int b = (int)(blk % g.Wo);
-  const int a = (int)((blk / g.Wo) % g.Ho);
-  const int64_t n = blk / ((int64_t)g.Wo * g.Ho);
+  constexpr uint64_t kNone = ~uint64_t(0);             // fields that match no window position (K * K < 15)
+  const ClAt at = cl_at(q);                            // rows and columns of windows
+  if (!at.live) return;
+  const uint32_t C = q.cpp * E;
+  const int64_t image_o = (int64_t)at.n * q.per_image * E;
+  const uint32_t lane_o = at.i * E;                    // window (row, col) of this chunk inside the image
+  const T* gimg = gout + image_o;
+  const int8_t* iimg = idx + IndexFields<NIB>::byte_of(image_o);
+  u32x4 raw[NWIN][NWIN];
+  uint64_t fields[NWIN][NWIN];
+#pragma unroll
+  for (int j = 0; j < NWIN; ++j)
+#pragma unroll
+    for (int t = 0; t < NWIN; ++t) {
+      const bool inside = at.row + j < (uint32_t)g.Ho && at.col + t < (uint32_t)g.Wo;
+      const int64_t step = ((int64_t)j * g.Wo + t) * C;              // uniform
+      raw[j][t] = inside ? load16(gimg + step + lane_o) : u32x4{0, 0, 0, 0};
+      fields[j][t] = inside ? IndexFields<NIB>::template load<E>(iimg + IndexFields<NIB>::byte_of(step), (int64_t)lane_o) : kNone;
+    }
   float acc[2][2][E];
 #pragma unroll
   for (int rr = 0; rr < 2; ++rr)
@@ -773,11 +892,8 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_backward_cl_s2_kernel(
   for (int j = 0; j < NWIN; ++j) {
 #pragma unroll
     for (int t = 0; t < NWIN; ++t) {
-      if (a + j >= g.Ho || b + t >= g.Wo) continue;
-      const int64_t o = ((n * g.Ho + a + j) * (int64_t)g.Wo + b + t) * C + c;
       float v[E];
-      widen_chunk<T, E>(gout + o, v);
-      const uint64_t fields = IndexFields<NIB>::template load<E>(idx, o);
+      raw_widen_chunk<T, E>(raw[j][t], v);
       // input row 2a + rr sits at window row kh = rr + P - 2j of window row a + j; columns alike
 #pragma unroll
       for (int rr = 0; rr < 2; ++rr) {
@@ -789,16 +905,35 @@ __global__ __launch_bounds__(kThreads) void max_pool2d_backward_cl_s2_kernel(
           if (kw < 0 || kw >= K) continue;
 #pragma unroll
           for (int e = 0; e < E; ++e)
-            if (IndexFields<NIB>::get(fields, e) == kh * K + kw) acc[rr][cc][e] += v[e];
+            if (IndexFields<NIB>::get(fields[j][t], e) == kh * K + kw) acc[rr][cc][e] += v[e];
         }
       }
     }
   }
+  T* out = gin + (int64_t)at.n * g.H * g.W * C;
+  const uint32_t lane_in = (2 * at.row * (uint32_t)g.W + 2 * at.col) * C + at.chunk * E;
 #pragma unroll
   for (int rr = 0; rr < 2; ++rr)
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc)
-      narrow_chunk<T, E>(gin + ((n * g.H + 2 * a + rr) * (int64_t)g.W + 2 * b + cc) * C + c, acc[rr][cc]);
+      narrow_chunk_nt<T, E>(out + ((int64_t)rr * g.W + cc) * C + lane_in, acc[rr][cc]);
+}
+
+// thread positions for rows x cols pixels per image; false when an image is too large for 32-bit offsets
+inline bool cl_geometry(int64_t N, int64_t rows, int64_t cols, int64_t cpp, int64_t image_elems, ClGeom& q) {
+  const int64_t per_image = rows * cols * cpp;
+  if (image_elems >= 0x7fffffffLL || per_image >= 0x7fffffffLL || per_image == 0) return false;
+  const int64_t bpi = (per_image + kThreads - 1) / kThreads;
+  if (N * bpi > 0x7ffffff0LL) return false;
+  q.cpp = (uint32_t)cpp;
+  q.cols = (uint32_t)cols;
+  q.per_image = (uint32_t)per_image;
+  q.blocks_per_image = (uint32_t)bpi;
+  q.blocks = (uint32_t)(N * bpi);
+  q.by_cpp = FastDiv((uint32_t)cpp);
+  q.by_cols = FastDiv((uint32_t)cols);
+  q.by_blocks_per_image = FastDiv((uint32_t)bpi);
+  return true;
 }
 
 template <typename T, bool NIB>
@@ -816,25 +951,31 @@ int launch_cl(bool forward, const void* a, const int8_t* idx_in, int8_t* idx_out
   const int64_t blocks = (chunks + kThreads - 1) / kThreads;
   if (blocks > 0x7ffffff0LL) return ACTNN_EINVAL;
   if (blocks == 0) return ACTNN_OK;
+  ClGeom q;
+  // the padded input image must fit 32-bit element offsets for the window kernels
+  const int64_t image_elems = ((int64_t)g.H + 2) * ((int64_t)g.W + 2) * C;
+  const int p = preset_of(g);
   if (forward) {
-    const dim3 grid(xcd_grid(blocks)), blk(kThreads);
     const T* xi = static_cast<const T*>(a);
     T* yo = static_cast<T*>(out);
-    switch (preset_of(g)) {
-      case 1: max_pool2d_forward_cl_kernel<T, 1, NIB><<<grid, blk, 0, s>>>(xi, yo, idx_out, chunks, cpp, C, g); break;
-      case 2: max_pool2d_forward_cl_kernel<T, 2, NIB><<<grid, blk, 0, s>>>(xi, yo, idx_out, chunks, cpp, C, g); break;
-      case 3: max_pool2d_forward_cl_kernel<T, 3, NIB><<<grid, blk, 0, s>>>(xi, yo, idx_out, chunks, cpp, C, g); break;
-      default: max_pool2d_forward_cl_kernel<T, 0, NIB><<<grid, blk, 0, s>>>(xi, yo, idx_out, chunks, cpp, C, g); break;
+    if (p != 0 && cl_geometry(N, g.Ho, g.Wo, cpp, image_elems, q)) {
+      const dim3 grid(xcd_grid(q.blocks)), blk(kThreads);
+      switch (p) {
+        case 1: max_pool2d_forward_cl_window_kernel<T, 1, NIB><<<grid, blk, 0, s>>>(xi, yo, idx_out, q, g); break;
+        case 2: max_pool2d_forward_cl_window_kernel<T, 2, NIB><<<grid, blk, 0, s>>>(xi, yo, idx_out, q, g); break;
+        default: max_pool2d_forward_cl_window_kernel<T, 3, NIB><<<grid, blk, 0, s>>>(xi, yo, idx_out, q, g); break;
+      }
+    } else {
+      max_pool2d_forward_cl_kernel<T, NIB><<<dim3(xcd_grid(blocks)), dim3(kThreads), 0, s>>>(xi, yo, idx_out, chunks, cpp, C, g);
     }
-  } else if (const int p = preset_of(g); (p == 1 || p == 2) && g.H == 2 * g.Ho && g.W == 2 * g.Wo) {
-    const int64_t items = N * g.Ho * g.Wo * cpp;
-    const dim3 grid(xcd_grid((items + kThreads - 1) / kThreads)), blk(kThreads);
+  } else if ((p == 1 || p == 2) && g.H == 2 * g.Ho && g.W == 2 * g.Wo && cl_geometry(N, g.Ho, g.Wo, cpp, image_elems, q)) {
+    const dim3 grid(xcd_grid(q.blocks)), blk(kThreads);
     if (p == 1)
       max_pool2d_backward_cl_s2_kernel<T, 3, 1, NIB><<<grid, blk, 0, s>>>(
-          static_cast<const T*>(a), idx_in, static_cast<T*>(out), items, cpp, C, g);
+          static_cast<const T*>(a), idx_in, static_cast<T*>(out), q, g);
     else
       max_pool2d_backward_cl_s2_kernel<T, 2, 0, NIB><<<grid, blk, 0, s>>>(
-          static_cast<const T*>(a), idx_in, static_cast<T*>(out), items, cpp, C, g);
+          static_cast<const T*>(a), idx_in, static_cast<T*>(out), q, g);
   } else {
     max_pool2d_backward_cl_kernel<T, NIB><<<dim3(xcd_grid(blocks)), dim3(kThreads), 0, s>>>(
         static_cast<const T*>(a), idx_in, static_cast<T*>(out), chunks, cpp, C, g);
