@@ -219,14 +219,16 @@ template <typename T> struct PackedInput {
       const uint32_t l2 = (uint32_t)__builtin_amdgcn_update_dpp(0, h, 0xAA, 0xF, 0xF, true);   // [2,2,2,2]
       const uint32_t l3 = (uint32_t)__builtin_amdgcn_update_dpp(0, h, 0xFF, 0xF, 0xF, true);   // [3,3,3,3]
       const uint32_t lut_lo = l0 | (l1 << 16), lut_hi = l2 | (l3 << 16);
-      const uint32_t a = (uint32_t)acc;
+      // a copy of the codes moved up by 16 - BITS puts the second code of every pair 16 bits above the
+      // first: one shift and one mask then give both (c0 | c1 << 16), and a multiply-add turns them into
+      // the byte selectors 2c, 2c + 1 of the two elements
+      constexpr uint32_t kPair = ((1u << BITS) - 1u) * 0x00010001u;
+      const uint32_t a = (uint32_t)acc & 0xffffu;
+      const uint32_t both = a | (a << (16 - BITS));
       uint32_t out[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const uint32_t c0 = (a >> (2 * j * BITS)) & ((1u << BITS) - 1u);
-        const uint32_t c1 = (a >> ((2 * j + 1) * BITS)) & ((1u << BITS) - 1u);
-        // bytes 2c, 2c+1 of the table for each of the two elements
-        const uint32_t sel = (c0 * 0x0202u + 0x0100u) | ((c1 * 0x0202u + 0x0100u) << 16);
+        const uint32_t sel = __umul24((both >> (2 * j * BITS)) & kPair, 0x0202u) + 0x01000100u;
         out[j] = __builtin_amdgcn_perm(lut_hi, lut_lo, sel);
       }
       return u32x4{out[0], out[1], out[2], out[3]};
@@ -471,11 +473,9 @@ __global__ __launch_bounds__(kThreads, 6) void bn_reduce_kernel(
       float v[E];
 #pragma unroll
       for (int j = 0; j < 4; ++j) Chunk<T>::widen(w[j], v + j * PD);
-      float lo = v[0], hi = v[0];
-#pragma unroll
-      for (int i = 1; i < E; ++i) { lo = fminf(lo, v[i]); hi = fmaxf(hi, v[i]); }
-      lo = rows_min<LPG / 16>(row16_min(lo));
-      hi = rows_max<LPG / 16>(row16_max(hi));
+      float lo, hi;
+      minmax_of<E>(v, lo, hi);
+      lanes_minmax<LPG / 16>(lo, hi);
       if ((threadIdx.x & (LPG - 1)) == LPG - 1 && p.active) {
         const int64_t g = n * (F >> 8) + (p.elem >> 8);
         Conv<T>::store(mn, g, lo);
@@ -861,35 +861,61 @@ template <typename T> struct PackedRows {
   static constexpr bool kRows = true;
   static constexpr int kInFlight = 2;
   PackedInput<T> in;     // G = groups per sample
-  int64_t C, col;
+  int64_t C;
   uint32_t HW;
+  FastDiv by_hw;
   using Raw = typename PackedInput<T>::Raw;
-  int r;
+  // Per lane, fixed at bind(): its row inside one iteration and what it adds to the block's (scalar)
+  // group position.  A thread stays inside one sample for many rows: the sample's width, its first
+  // word and its first group are kept in registers and looked up again only when the row moves on to
+  // the next sample, and everything else is 32-bit arithmetic on top of them (rows, groups and the
+  // words of one sample stay below 2^31, which the launcher checks) - the fetch is a handful of
+  // instructions where 64-bit index arithmetic per row took forty.
+  uint32_t r, lane_group;
+  uint32_t cur_row0, cur_group0;     // first row / first group of the sample of the last fetch
+  int cur_b;
+  const int32_t* cur_words;          // the sample's first word
   ACTNN_DEV void bind(int64_t column, int row_in_iteration) {
-    col = column;
-    r = row_in_iteration;
+    r = (uint32_t)row_in_iteration;
+    lane_group = (uint32_t)(((int64_t)row_in_iteration * C + column) >> 8);
     in.lane32 = threadIdx.x & (PackedInput<T>::kLanes - 1);
     in.active = true;
-    cur_row0 = -(int64_t)HW - 1;                           // no row is inside: the first fetch looks up
+    cur_row0 = 0x80000000u;          // no row is inside: the first fetch looks up (rows < 2^31)
+    cur_group0 = 0;
+    cur_b = 1;
+    cur_words = in.words;
   }
-  // A thread stays inside one sample for many rows: the sample's width and first word are kept
-  // in registers and reloaded only when the row moves on to the next sample, which takes two
-  // dependent loads off the path of every fetch.
-  uint32_t cur_n;        // sample of the last fetch; cur_row0 = cur_n * HW
-  int cur_b;
-  int64_t cur_first, cur_row0;
   ACTNN_DEV Raw fetch(int64_t rb) {
-    const int64_t row = rb + r;
-    if ((uint64_t)(row - cur_row0) >= HW) {                // left the sample (or the first fetch)
-      cur_n = (uint32_t)row / HW;                          // rows < 2^31 (checked by the launcher)
-      cur_row0 = (int64_t)cur_n * HW;
-      cur_b = in.bits[cur_n];
-      cur_first = (int64_t)in.prefix[cur_n] * in.G * 8;
+    const uint32_t row = (uint32_t)rb + r;
+    if (row - cur_row0 >= HW) {                            // left the sample (or the first fetch)
+      const uint32_t n = by_hw.div(row);
+      cur_row0 = n * HW;
+      cur_group0 = n * (uint32_t)in.G;
+      cur_b = in.bits[n];
+      cur_words = in.words + (int64_t)in.prefix[n] * in.G * 8;
     }
-    const int64_t grp = ((row * C + col) >> 8) - (int64_t)cur_n * in.G;
-    return in.fetch_known(cur_n, grp, cur_b, cur_first);
+    // rb * C is a multiple of 256 (rb a multiple of R, and R * C of 256, wherever groups align)
+    const int64_t block_group = (rb * C) >> 8;             // the same for the whole block
+    const uint32_t group = (uint32_t)block_group + lane_group;
+    const uint32_t at = __umul24(group - cur_group0, (uint32_t)(8 * cur_b)) + in.lane32;
+    Raw raw{0u, 0u, 1.0f, 0.0f, cur_b};
+    if ((int)in.lane32 < 8 * cur_b) raw.lo = (uint32_t)cur_words[at];
+    if (PackedInput<T>::kLanes == 32 && (int)in.lane32 + 32 < 8 * cur_b) raw.hi = (uint32_t)cur_words[at + 32];
+    raw.sc = Conv<T>::load(in.scale + block_group, lane_group);
+    raw.m = Conv<T>::load(in.mn + block_group, lane_group);
+    return raw;
   }
-  ACTNN_DEV u32x4 decode(const Raw& r) const { return in.decode(r); }
+  ACTNN_DEV u32x4 decode(const Raw& r) const {
+    // a wave holds a few consecutive rows, nearly always of one sample: then the width is one number
+    // and the choice of the decoder a scalar branch, not a walk through eight masked ones
+    const int b0 = __builtin_amdgcn_readfirstlane(r.b);
+    if (__builtin_amdgcn_ballot_w64(r.b != b0) == 0) {
+      Raw u = r;
+      u.b = b0;
+      return in.decode(u);
+    }
+    return in.decode(r);
+  }
 };
 
 struct RowTile {
@@ -952,11 +978,9 @@ __global__ __launch_bounds__(kThreads, (cl_reduce_waves<BWD, MINMAX, XS>())) voi
     }
     if (MINMAX) {
       constexpr int LPG = 256 / E;
-      float lo = v[0], hi = v[0];
-#pragma unroll
-      for (int i = 1; i < E; ++i) { lo = fminf(lo, v[i]); hi = fmaxf(hi, v[i]); }
-      lo = rows_min<LPG / 16>(row16_min(lo));
-      hi = rows_max<LPG / 16>(row16_max(hi));
+      float lo, hi;
+      minmax_of<E>(v, lo, hi);
+      lanes_minmax<LPG / 16>(lo, hi);
       if ((threadIdx.x & (LPG - 1)) == LPG - 1) {
         // rb * C is a multiple of 256 (rb a multiple of R, and R * C of 256, wherever groups align)
         T* lo_at = mn + ((rb * C) >> 8) + lane_group;
@@ -1497,7 +1521,9 @@ int backward_packed(const Plan& pl, const int32_t* packed, const int32_t* bits, 
   const PackedInput<T> in{packed, bits, prefix, static_cast<const T*>(scale), static_cast<const T*>(mn),
                           pl.F / 256, 0, 0u, false};
   if (pl.channels_last) {
-    const PackedRows<T> xs{in, C, 0, (uint32_t)HW, 0, 0u, 1, 0, 0};
+    // (32-bit positions inside a sample and over the tensor's groups)
+    if (C * HW >= ((int64_t)1 << 32) || N * (pl.F / 256) >= 0x7fffffffLL) return ACTNN_EINVAL;
+    const PackedRows<T> xs{in, C, (uint32_t)HW, FastDiv((uint32_t)HW), 0u, 0u, 0u, 0u, 1, packed};
     return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
   }
   return backward_t<T>(pl, in, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);

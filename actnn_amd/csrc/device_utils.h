@@ -318,6 +318,82 @@ ACTNN_DEV uint32_t transpose32_x2(uint32_t x, uint32_t lane) {
   return x;
 }
 
+// Minimum / maximum as single instructions.  fminf / fmaxf compile to the same instruction plus one
+// more per operand that quiets signalling NaNs (the loops that use these are bound by
+// instruction issue, and the extra instructions were a quarter of them); here a quiet NaN operand is
+// ignored as in fminf / fmaxf, a signalling NaN is returned quieted.
+ACTNN_DEV float min_f32(float a, float b) {
+  float r;
+  asm("v_min_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+ACTNN_DEV float max_f32(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+ACTNN_DEV float min3_f32(float a, float b, float c) {
+  float r;
+  asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+ACTNN_DEV float max3_f32(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+// minimum and maximum of N values (N = 4 or 8) in N / 2 instructions each
+template <int N> ACTNN_DEV void minmax_of(const float (&v)[N], float& lo, float& hi) {
+  lo = min3_f32(v[0], v[1], v[2]);
+  hi = max3_f32(v[0], v[1], v[2]);
+  if constexpr (N == 8) {
+    lo = min3_f32(lo, v[3], v[4]);
+    hi = max3_f32(hi, v[3], v[4]);
+    lo = min3_f32(lo, v[5], v[6]);
+    hi = max3_f32(hi, v[5], v[6]);
+    lo = min_f32(lo, v[7]);
+    hi = max_f32(hi, v[7]);
+  } else {
+    static_assert(N == 4, "4 or 8 values");
+    lo = min_f32(lo, v[3]);
+    hi = max_f32(hi, v[3]);
+  }
+}
+
+// Minimum of lo and maximum of hi over groups of 16 * ROWS consecutive lanes (ROWS = 1, 2 or 4), both
+// at once, with the lane exchange inside the arithmetic instruction (one instruction per step and
+// value; through the exchange builtins it took three).  ROWS == 1: every lane ends with the result
+// of its row of 16; ROWS == 2: the last row of each 32-lane half holds the half's result; ROWS == 4:
+// the last row of the wave holds the wave's result.  All lanes of the groups must be active.  The
+// s_nop's are the wait states the hardware asks for between a vector write and a cross-lane read
+// of the same register (2) and after a vector write of EXEC (5); the compiler does not see into the
+// block.
+template <int ROWS> ACTNN_DEV void lanes_minmax(float& lo, float& hi) {
+  asm("s_nop 4\n\t"
+      "v_min_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 0\n\t"
+      "v_min_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 0\n\t"
+      "v_min_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 0\n\t"
+      "v_min_f32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf\n\t"
+      "v_max_f32_dpp %1, %1, %1 row_mirror row_mask:0xf bank_mask:0xf"
+      : "+v"(lo), "+v"(hi));
+  if constexpr (ROWS >= 2)     // the last lane of rows 0 and 2 into rows 1 and 3
+    asm("s_nop 1\n\t"
+        "v_min_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+        "v_max_f32_dpp %1, %1, %1 row_bcast:15 row_mask:0xa bank_mask:0xf"
+        : "+v"(lo), "+v"(hi));
+  if constexpr (ROWS >= 4)     // the last lane of row 1 into rows 2 and 3
+    asm("s_nop 1\n\t"
+        "v_min_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+        "v_max_f32_dpp %1, %1, %1 row_bcast:31 row_mask:0xc bank_mask:0xf"
+        : "+v"(lo), "+v"(hi));
+}
+
 // Reductions over a DPP row (16 consecutive lanes); every lane ends with the result.
 ACTNN_DEV float row16_max(float v) {
   v = fmaxf(v, __builtin_bit_cast(float, lane_xor<1>(__builtin_bit_cast(uint32_t, v))));
