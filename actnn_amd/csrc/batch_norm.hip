@@ -403,20 +403,15 @@ ACTNN_DEV void noise_pair(const PackSink& ps, uint64_t oa, uint64_t ob, uint32_t
   }
 }
 
-// b = bits[n], first_word = prefix[n] * G * 8: looked up by the caller, who knows how often n changes;
-// (mul, sub): the group's parameters from the queue; rw: the noise words of the chunk's octet
+// b: the sample's width, dst: first word of the chunk's group in the stream (both looked up by the
+// caller, who knows how often the sample changes); (mul, sub): the group's parameters from the queue;
+// rw: the noise words of the chunk's octet.  SCALAR_B: b is known to be one number for the wave (the
+// sample comes from the block's index); otherwise the wave checks, and takes one scalar branch when
+// its lanes agree - as they do except where a wave spans two samples of different widths.
 template <typename T>
-ACTNN_DEV void pack_chunk(const PackSink& ps, const u32x4& ux, const uint32_t (&rw)[Noise<T>::kWords],
-                          float mul, float sub, int64_t grp, int b, int64_t first_word) {
-  constexpr int PD = Chunk<T>::kPerDword;
-  static_assert(Chunk<T>::kElems == 8, "16-bit types only");
-  const uint32_t lane32 = threadIdx.x & 31;
-  const uint32_t w[4] = {ux.x, ux.y, ux.z, ux.w};
-  float v[8];
-#pragma unroll
-  for (int k = 0; k < 4; ++k) Chunk<T>::widen(w[k], v + k * PD);
-  int32_t* dst = ps.packed + first_word + grp * b * 8;
-  switch (b) {                           // uniform over the half-wave: one sample, one width
+ACTNN_DEV void pack_chunk_width(const float (&v)[8], const uint32_t (&rw)[Noise<T>::kWords], float mul, float sub,
+                                uint32_t lane32, int32_t* __restrict__ dst, int b) {
+  switch (b) {
     case 1: pack_chunk_bits<T, 1>(v, rw, mul, sub, lane32, dst); break;
     case 2: pack_chunk_bits<T, 2>(v, rw, mul, sub, lane32, dst); break;
     case 3: pack_chunk_bits<T, 3>(v, rw, mul, sub, lane32, dst); break;
@@ -426,6 +421,24 @@ ACTNN_DEV void pack_chunk(const PackSink& ps, const u32x4& ux, const uint32_t (&
     case 7: pack_chunk_bits<T, 7>(v, rw, mul, sub, lane32, dst); break;
     case 8: pack_chunk_bits<T, 8>(v, rw, mul, sub, lane32, dst); break;
     default: break;
+  }
+}
+template <typename T, bool SCALAR_B>
+ACTNN_DEV void pack_chunk(const u32x4& ux, const uint32_t (&rw)[Noise<T>::kWords], float mul, float sub,
+                          int32_t* __restrict__ dst, int b) {
+  constexpr int PD = Chunk<T>::kPerDword;
+  static_assert(Chunk<T>::kElems == 8, "16-bit types only");
+  const uint32_t lane32 = threadIdx.x & 31;
+  const uint32_t w[4] = {ux.x, ux.y, ux.z, ux.w};
+  float v[8];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) Chunk<T>::widen(w[k], v + k * PD);
+  if constexpr (SCALAR_B) {
+    pack_chunk_width<T>(v, rw, mul, sub, lane32, dst, b);
+  } else {
+    const int b0 = __builtin_amdgcn_readfirstlane(b);
+    if (__builtin_amdgcn_ballot_w64(b != b0) == 0) pack_chunk_width<T>(v, rw, mul, sub, lane32, dst, b0);
+    else pack_chunk_width<T>(v, rw, mul, sub, lane32, dst, b);
   }
 }
 
@@ -791,7 +804,8 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
           store_out(po + (n + u) * F, apply(ux, ux));
           float mul, sub;
           queue.get((int)(n + u - nb), mul, sub);
-          pack_chunk<T>(ps, ux, rw[u], mul, sub, grp, ps.bits[n + u], (int64_t)ps.prefix[n + u] * ps.G * 8);
+          const int b = ps.bits[n + u];
+          pack_chunk<T, true>(ux, rw[u], mul, sub, ps.packed + (int64_t)ps.prefix[n + u] * ps.G * 8 + grp * b * 8, b);
         }
       }
       for (; n < ne; ++n) {
@@ -802,7 +816,8 @@ __global__ __launch_bounds__(kThreads) void bn_apply_kernel(
         Noise<T>::octet((uint64_t)((n * F + p.elem) >> 3), ps.seed, ps.offset, rw);
         float mul, sub;
         queue.get((int)(n - nb), mul, sub);
-        pack_chunk<T>(ps, ux, rw, mul, sub, grp, ps.bits[n], (int64_t)ps.prefix[n] * ps.G * 8);
+        const int b = ps.bits[n];
+        pack_chunk<T, true>(ux, rw, mul, sub, ps.packed + (int64_t)ps.prefix[n] * ps.G * 8 + grp * b * 8, b);
       }
     }
   } else {
@@ -1037,23 +1052,31 @@ __global__ __launch_bounds__(kThreads, (cl_reduce_waves<BWD, MINMAX, XS>())) voi
 template <typename T, bool BWD, bool PACK, typename XS>
 __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
     XS xs, const T* __restrict__ dy, const float* __restrict__ coef, T* __restrict__ out,
-    int64_t P, int64_t C, int tpr, int R, int64_t ppb, PackSink ps, uint32_t HW) {
+    int64_t P, int64_t C, int tpr, int R, int64_t ppb, PackSink ps, FastDiv by_hw) {
   constexpr int E = Chunk<T>::kElems;
   constexpr int PD = Chunk<T>::kPerDword;
   constexpr int NC = BWD ? 3 : 2;
   constexpr int U = XS::kInFlight;
   static_assert(!(PACK && BWD), "the packed copy is made by the forward pass");
-  uint32_t cur_n = 0;                    // the sample whose width and first word are held below
+  // The sample that holds the row of the last pack: its width, its first word in the stream and its
+  // first row / group.  A thread stays inside one sample for many rows, so these are looked up only
+  // when a row leaves it, and a chunk's place in the stream is 32-bit arithmetic on top of them (rows,
+  // groups and the words of one sample stay below 2^31, which the launcher checks).
+  const uint32_t HW = by_hw.d;
+  uint32_t cur_row0 = 0x80000000u, cur_group0 = 0;       // no row is inside: the first pack looks up
   int cur_b = 1;
-  int64_t cur_first = 0, cur_row0 = -(int64_t)HW - 1;
-  auto locate = [&](int64_t row) {       // width and first word of the sample that holds `row`
-    if ((uint64_t)(row - cur_row0) >= HW) {                // left the sample (or the first row)
-      cur_n = (uint32_t)row / HW;                          // rows < 2^31 (checked by the launcher)
-      cur_row0 = (int64_t)cur_n * HW;
-      cur_b = ps.bits[cur_n];
-      cur_first = (int64_t)ps.prefix[cur_n] * ps.G * 8;
+  int32_t* cur_words = ps.packed;
+  auto locate = [&](uint32_t row) {
+    if (row - cur_row0 >= HW) {
+      const uint32_t n = by_hw.div(row);
+      cur_row0 = n * HW;
+      cur_group0 = n * (uint32_t)ps.G;
+      cur_b = ps.bits[n];
+      cur_words = ps.packed + (int64_t)ps.prefix[n] * ps.G * 8;
     }
   };
+  // first word of group `group` (counted over the tensor) of the located sample
+  auto group_words = [&](uint32_t group) -> int32_t* { return cur_words + __umul24(group - cur_group0, (uint32_t)(8 * cur_b)); };
   const RowTile t = row_tile<E>(C, tpr, R);
   float sumsq = 0.0f;
   if (!BWD && !t.active) return;       // whole quantisation groups leave together
@@ -1106,12 +1129,11 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
     const int lane = threadIdx.x & 63;
     ParamQueue<T> queue;
     auto params = [&](int64_t ru, int jq) {
-      locate(ru + t.r);
+      locate((uint32_t)ru + (uint32_t)t.r);
       ChunkParams q;
       queue.get(jq, q.mul, q.sub);
       q.b = cur_b;
-      const int64_t grp = ((ru * C) >> 8) + (lane_elems >> 8);
-      q.dst = ps.packed + cur_first + (grp - (int64_t)cur_n * ps.G) * q.b * 8;
+      q.dst = group_words((uint32_t)((ru * C) >> 8) + (lane_elems >> 8));
       q.octet = (uint64_t)((ru * C) >> 3) + (lane_elems >> 3);
       return q;
     };
@@ -1120,7 +1142,7 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
       {
         const int64_t rj = rb + (int64_t)lane * R;
         const bool live = rj < p1;
-        const uint32_t nj = live ? (uint32_t)rj / HW : 0;
+        const uint32_t nj = live ? by_hw.div((uint32_t)rj) : 0;
         queue.fill(ps, (rj * C + t.col) >> 8, live ? ps.bits[nj] : 1, live);
       }
       int j = 0;
@@ -1149,17 +1171,17 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
     const int lane32 = threadIdx.x & 31;
     ParamQueue<T> queue;
     auto pack_one = [&](const u32x4& ux, const uint32_t (&rw)[Noise<T>::kWords], int64_t ru, int j) {
-      locate(ru + t.r);
+      locate((uint32_t)ru + (uint32_t)t.r);
       float mul, sub;
       queue.get(j, mul, sub);
-      pack_chunk<T>(ps, ux, rw, mul, sub, ((ru * C) >> 8) + (lane_elems >> 8) - (int64_t)cur_n * ps.G, cur_b, cur_first);
+      pack_chunk<T, false>(ux, rw, mul, sub, group_words((uint32_t)((ru * C) >> 8) + (lane_elems >> 8)), cur_b);
     };
     for (int64_t rb0 = p0; rb0 + t.r < p1; rb0 += (int64_t)32 * R) {
       const int64_t rb = rb0 + t.r;
       {
         const int64_t rj = rb + (int64_t)lane32 * R;
         const bool live = rj < p1;
-        const uint32_t nj = live ? (uint32_t)rj / HW : 0;
+        const uint32_t nj = live ? by_hw.div((uint32_t)rj) : 0;
         queue.fill(ps, (rj * C + t.col) >> 8, live ? ps.bits[nj] : 1, live);
       }
       int j = 0;
@@ -1386,7 +1408,7 @@ void launch_cl_apply(const Plan& pl, const XS& xs, const void* dy, const float* 
   const dim3 grid((unsigned)pl.tiles, (unsigned)pl.nsplit_apply), blk(kThreads);
   bn_cl_apply_kernel<T, BWD, PACK, XS><<<grid, blk, 0, s>>>(
       xs, static_cast<const T*>(dy), coef, static_cast<T*>(out), pl.P, C, pl.tpr, pl.R, pl.ppb_apply, ps,
-      (uint32_t)(pl.F / C));
+      FastDiv((uint32_t)(pl.F / C)));
 }
 
 template <typename T>
@@ -1592,7 +1614,9 @@ extern "C" int actnn_batch_norm_forward_apply(const void* x, void* y, const void
   const bool pack = bits != nullptr;
   if (pack) {
     if (!pl.groups_align || !prefix || !mn || !mx || !scale || !packed) return ACTNN_EINVAL;
-    if (channels_last && pl.P > 0x7fffffffLL) return ACTNN_EINVAL;
+    // channels-last: 32-bit rows, groups and positions inside a sample
+    if (channels_last && (pl.P > 0x7fffffffLL || C * HW >= ((int64_t)1 << 32) || N * (pl.F / 256) >= 0x7fffffffLL))
+      return ACTNN_EINVAL;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const float* ws = static_cast<const float*>(workspace);
