@@ -68,12 +68,18 @@ def calc_precision_device(C, initial_bits, target):
     return bits
 
 
-def allocate_bits_device(mn, mx, N, factor, mult, initial_bits, target):
+def allocate_bits_device(mn, mx, N, factor, mult, initial_bits, target, sens_out=None):
     """-> (sensitivity fp32 [N], bits int32 [N], prefix int32 [N + 1]) on the device of mn:
-    ``range_sqr`` -> ``calc_precision_device`` -> exclusive prefix of the widths, in one call."""
+    ``range_sqr`` -> ``calc_precision_device`` -> exclusive prefix of the widths, in one call.
+    `sens_out`: where to write the sensitivities (fp32 [N], contiguous, same device)."""
     G = mn.numel() // N
     dev = mn.device
-    sens = torch.empty(N, dtype=torch.float32, device=dev)
+    if sens_out is None:
+        sens = torch.empty(N, dtype=torch.float32, device=dev)
+    else:
+        if sens_out.dtype != torch.float32 or sens_out.device != dev or sens_out.numel() != N or not sens_out.is_contiguous():
+            raise RuntimeError("allocate_bits_device: sens_out must be contiguous fp32 [N] on the same device")
+        sens = sens_out
     bits = torch.empty(N, dtype=torch.int32, device=dev)
     prefix = torch.empty(N + 1, dtype=torch.int32, device=dev)
     mult_ptr, per_sample = None, 0

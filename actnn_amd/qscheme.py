@@ -73,6 +73,49 @@ class PendingBits:
         return self.host
 
 
+class SensitivityPool:
+    """One device buffer and one pinned host buffer for the sensitivities of every layer of a step.
+
+    With the widths made on the device, the host needs the sensitivities only at the end of the step
+    (per-layer re-balancing).  A copy per layer put a device->host transfer and an event between the
+    kernels of every layer; here every layer's allocation kernel writes its row of one [layers, N]
+    buffer, and the whole buffer goes to the host in a single transfer, queued when the first
+    backward of the step starts (behind the forward's kernels, ahead of the backward's, so that it
+    has long arrived when the last backward asks for it)."""
+
+    def __init__(self, rows, N, device):
+        self.dev = torch.empty((rows, N), dtype=torch.float32, device=device)
+        self.host = torch.empty((rows, N), dtype=torch.float32, pin_memory=True)
+        self.event = torch.cuda.Event()
+        self.dirty = False           # rows written since the last transfer
+        self.rows = [self.dev[i] for i in range(rows)]
+
+    def fits(self, rows, N, device):
+        return self.dev.shape[0] >= rows and self.dev.shape[1] == N and self.dev.device == device
+
+    def flush(self):
+        """Queue the transfer if any row has been written since the last one."""
+        if self.dirty:
+            self.host.copy_(self.dev, non_blocking=True)
+            self.event.record()
+            self.dirty = False
+
+    def row_on_host(self, index):
+        self.flush()
+        self.event.synchronize()
+        return self.host[index].clone()
+
+
+class _PooledRow:
+    """What a layer keeps of its row of the pool: `wait()` as PendingBits has it."""
+
+    def __init__(self, pool, index):
+        self.pool, self.index = pool, index
+
+    def wait(self):
+        return self.pool.row_on_host(self.index)
+
+
 def greedy_bits(C_host, N, initial_bits, avg_bits, device):
     """Per-sample widths: calc_precision(b = initial_bits, C, w = 1, target = int(avg_bits * N)),
     returned on the device with the host copy attached (qscheme.py:86-94)."""
@@ -92,13 +135,13 @@ def greedy_bits_device(C_dev, N, initial_bits, avg_bits):
     return attach_bits_total(bits, N * initial - taken)
 
 
-def allocate_bits_on_device(mn, mx, N, num_pixels, factor, mult, initial_bits, avg_bits):
+def allocate_bits_on_device(mn, mx, N, num_pixels, factor, mult, initial_bits, avg_bits, sens_out=None):
     """Sensitivities, widths and the prefix of the widths in one call -> (C on the device, bits
-    with their sum and prefix attached)."""
+    with their sum and prefix attached).  `sens_out`: fp32 [N] on the device to write C into."""
     initial = int(initial_bits)
     target = int(avg_bits * N)
     C_dev, bits, prefix = ext_calc_precision.allocate_bits_device(
-        mn, mx, N, factor * config.group_size / num_pixels, mult, initial, target)
+        mn, mx, N, factor * config.group_size / num_pixels, mult, initial, target, sens_out)
     taken = min(max(N * initial - target, 0), N * (initial - 1))
     return C_dev, attach_bits_total(bits, N * initial - taken, prefix)
 
@@ -141,6 +184,20 @@ class QScheme(_LazyHost):
     update_scale = True
     layers = []
     prev_layer = None
+    sensitivity_pool = None
+
+    @staticmethod
+    def pool_row(index, N, device):
+        """Row `index` of the step's sensitivity pool (made, or made anew, when the number of layers,
+        the batch size or the device changes)."""
+        pool = QScheme.sensitivity_pool
+        if pool is None or not pool.fits(len(QScheme.layers), N, device):
+            if pool is not None:
+                pool.flush()
+                pool.event.synchronize()         # rows handed out earlier keep their host values
+            pool = QScheme.sensitivity_pool = SensitivityPool(len(QScheme.layers), N, device)
+        pool.dirty = True
+        return pool, pool.rows[index]
 
     def __init__(self, layer, group=0, num_locations=1, depthwise_groups=1):
         self.initial_bits = config.initial_bits
@@ -150,6 +207,7 @@ class QScheme(_LazyHost):
             self.scales = torch.zeros(QScheme.num_samples)
         else:
             self.scales = torch.tensor([0.0])
+        self.index = len(QScheme.layers)            # row of the sensitivity pool
         QScheme.layers.append(self)
         self.C = None
         self.b = None
@@ -188,6 +246,8 @@ class QScheme(_LazyHost):
 
     def set_scale(self, grad):
         """Squared gradient norm per sample, kept as a running value (qscheme.py:47-55)."""
+        if QScheme.sensitivity_pool is not None:
+            QScheme.sensitivity_pool.flush()        # (called from every backward: the first one queues the transfer)
         if not QScheme.update_scale:
             return
         if not config.use_gradient and config.share_grad_sqnorm:
@@ -224,12 +284,14 @@ class QScheme(_LazyHost):
         bits_dev = None
         if allocate_on_device(N, self.initial_bits) and mn.is_contiguous() and mx.is_contiguous():
             grad_sum = self.get_scale(mn.device).to(device=mn.device, dtype=torch.float32)
-            C_dev, bits_dev = allocate_bits_on_device(
+            pool, row = QScheme.pool_row(self.index, N, mn.device)
+            _, bits_dev = allocate_bits_on_device(
                 mn, mx, N, num_pixels, self.num_locations / 4 / self.depthwise_groups, grad_sum,
-                self.initial_bits, self.bits)
+                self.initial_bits, self.bits, row)
+            pending = _PooledRow(pool, self.index)
         else:
             C_dev = self.sensitivity(mn, mx, N, num_pixels)
-        pending = self._last_pending = PendingBits(C_dev, getattr(self, "_last_pending", None))
+            pending = self._last_pending = PendingBits(C_dev, getattr(self, "_last_pending", None))
         return groups, mn, mx, pending, input.numel() // N, bits_dev
 
     def finish_quantization_bits(self, started):
@@ -295,3 +357,4 @@ class QScheme(_LazyHost):
         QScheme.prev_layer = None
         QScheme.batch = None
         QScheme._batch_index_cache = None
+        QScheme.sensitivity_pool = None

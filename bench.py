@@ -13,6 +13,8 @@ L3 step when the host layer is importable) and the CPU baseline (the oracle's re
 the reference's config.simulate quantiser on this box's host cores).
 """
 import argparse
+import contextlib
+import gc
 import json
 import os
 import sys
@@ -69,6 +71,23 @@ def measured_traffic(kernel_name, path=TRAFFIC_SUMMARY):
     return found[0], found[1], None
 
 
+@contextlib.contextmanager
+def gc_paused():
+    """Timed loops collect garbage first and keep CPython's collector off meanwhile.  A full collection
+    takes about 40 ms in a process that has torch loaded (170 k tracked objects) and starts whenever the
+    allocation counters say so - between two launches of a timed loop as readily as anywhere: a trace
+    of such a loop showed a 38-48 ms gap between two dispatches with no HIP call inside, and
+    gc.callbacks timed the collection at 40 ms."""
+    gc.collect()
+    was_on = gc.isenabled()
+    gc.disable()
+    try:
+        yield
+    finally:
+        if was_on:
+            gc.enable()
+
+
 WARM_MS = 25.0      # the first ~20 ms of work after an idle spell run up to 7 % slower than the steady state
 
 
@@ -87,16 +106,18 @@ def _event_time_ms(fn, reps, warmup=3):
     torch.cuda.synchronize()
     for _ in range(min(500, int(WARM_MS / max(start.elapsed_time(stop), 1e-3)))):
         fn()
-    # five back-to-back chunks, the median chunk: a one-off stall (a few ms, now and then) spoils one
+    # five back-to-back chunks, the median chunk (the stalls once seen here were the garbage collector,
+    # which is now kept off; the median stays as a guard against whatever else the host may do)
     chunk = max(1, reps // 5)
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(6)]
-    torch.cuda.synchronize()
-    marks[0].record()
-    for i in range(5):
-        for _ in range(chunk):
-            fn()
-        marks[i + 1].record()
-    torch.cuda.synchronize()
+    with gc_paused():
+        torch.cuda.synchronize()
+        marks[0].record()
+        for i in range(5):
+            for _ in range(chunk):
+                fn()
+            marks[i + 1].record()
+        torch.cuda.synchronize()
     return sorted(marks[i].elapsed_time(marks[i + 1]) / chunk for i in range(5))[2]
 
 
@@ -600,12 +621,13 @@ def main():
 
     for _ in range(args.warmup):
         step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    with gc_paused():
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     step_bytes = ab["minimax"] + ab["pack_mixed"] + ab["unpack_mixed"]
     value = step_bytes / ms_per_step / 1e6
 

@@ -2,6 +2,7 @@
 (benchmark config 5) with the reference's speed and memory protocols
 (mem_speed_benchmark/train.py:363-397 memory, :422-438 speed)."""
 import sys
+import gc
 import time
 
 import torch
@@ -96,20 +97,31 @@ def batch_norm_shapes(device, channels_last=True, batch=512, reps=10):
     from actnn_amd.cpp_extension.quantization import attach_bits_total
     from actnn_amd.ops import _Quantized
 
+    worst = []      # slowest repetition over the median, per timed call
+
     def timed(fn):
         for _ in range(3):
             fn()
         torch.cuda.synchronize(device)
-        # every repetition is timed on its own and the median taken: a one-off stall of a few
-        # milliseconds (the caching allocator growing, a clock change) would otherwise end up in
-        # the figure of whichever shape it happened to hit
+        # Every repetition is timed on its own, the median taken and the slowest reported.  The
+        # stalls of tens of milliseconds once seen here were CPython's full garbage collection
+        # (40 ms with torch loaded, timed through gc.callbacks; in a kernel trace a gap between two
+        # dispatches with no HIP call inside), which started wherever the allocation counters said
+        # so: the timed loop collects first and keeps the collector off.
         marks = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
-        marks[0].record()
-        for i in range(reps):
-            fn()
-            marks[i + 1].record()
-        torch.cuda.synchronize(device)
-        return sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(reps))[reps // 2]
+        gc.collect()
+        gc.disable()
+        try:
+            marks[0].record()
+            for i in range(reps):
+                fn()
+                marks[i + 1].record()
+            torch.cuda.synchronize(device)
+        finally:
+            gc.enable()
+        each = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(reps))
+        worst.append((each[-1] / each[reps // 2], each[-1]))
+        return each[reps // 2]
 
     rows, totals = [], [0.0, 0.0, 0.0]
     for C, H, count in RESNET50_BN_SHAPES:
@@ -136,4 +148,8 @@ def batch_norm_shapes(device, channels_last=True, batch=512, reps=10):
             totals[k] += count * t[k]
     return {"steps": ["statistics+minmax", "normalise+pack", "backward_from_2bit_stream"], "batch": batch,
             "memory_format": "channels_last" if channels_last else "contiguous", "shapes": rows,
-            "ms_per_training_step": [round(v, 3) for v in totals]}
+            "ms_per_training_step": [round(v, 3) for v in totals],
+            # (three timed calls per shape, in the order of `steps`)
+            "slowest_repetition": {"over_median": round(max(worst)[0], 2), "ms": round(max(worst)[1], 3),
+                                   "shape": RESNET50_BN_SHAPES[worst.index(max(worst)) // 3][:2],
+                                   "step": worst.index(max(worst)) % 3}}
