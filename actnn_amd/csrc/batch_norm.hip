@@ -938,11 +938,11 @@ struct RowTile {
   int r;                 // row of the thread inside one iteration
   bool active;
 };
-template <int E> ACTNN_DEV RowTile row_tile(int64_t C, int tpr, int R) {
+template <int E> ACTNN_DEV RowTile row_tile(int64_t C, int tpr, int R, int tile) {
   RowTile t;
   const int j = threadIdx.x % tpr;
   t.r = threadIdx.x / tpr;
-  t.col = (int64_t)blockIdx.x * 256 + (int64_t)j * E;
+  t.col = (int64_t)tile * 256 + (int64_t)j * E;
   t.active = t.r < R && t.col < C && j * E < 256;
   if (!t.active) t.col = 0;
   return t;
@@ -956,14 +956,21 @@ template <bool BWD, bool MINMAX, typename XS> constexpr int cl_reduce_waves() {
 template <typename T, bool BWD, bool MINMAX, bool NT, typename XS>
 __global__ __launch_bounds__(kThreads, (cl_reduce_waves<BWD, MINMAX, XS>())) void bn_cl_reduce_kernel(
     XS xs, const T* __restrict__ dy, float* __restrict__ part, T* __restrict__ mn, T* __restrict__ mx,
-    int64_t P, int64_t C, int tpr, int R, int64_t ppb) {
+    int64_t P, int64_t C, int tpr, int R, int64_t ppb, int tiles, int nsplit) {
   constexpr int E = Chunk<T>::kElems;
   constexpr int PD = Chunk<T>::kPerDword;
   constexpr int U = XS::kInFlight;
   __shared__ float s_part[kThreads * 2 * E];
-  const RowTile t = row_tile<E>(C, tpr, R);
+  // Blocks are numbered so that consecutive block rows of a column tile run on one XCD.  A line of the
+  // table of partial sums holds the values of 16 consecutive block rows; dealt round-robin, those rows
+  // sat on different XCDs, each L2 sent its 4 bytes of the line to memory on its own, and the write
+  // counter read eight times the table's size (26 MB on a pass that reads a 51 MB tensor).
+  const int64_t block = xcd_block();
+  if (block >= (int64_t)tiles * nsplit) return;
+  const int tile = (int)(block % tiles), brow = (int)(block / tiles);
+  const RowTile t = row_tile<E>(C, tpr, R, tile);
   xs.bind(t.col, t.r);
-  const int64_t p0 = (int64_t)blockIdx.y * ppb;
+  const int64_t p0 = (int64_t)brow * ppb;
   const int64_t p1 = p0 + ppb < P ? p0 + ppb : P;
   // everything a lane adds to the block's (scalar) position: bytes into dy, groups into mn / mx
   const uint32_t lane_bytes = (uint32_t)(((int64_t)t.r * C + t.col) * (int64_t)sizeof(T));
@@ -1040,11 +1047,11 @@ __global__ __launch_bounds__(kThreads, (cl_reduce_waves<BWD, MINMAX, XS>())) voi
   __syncthreads();
   for (int i = threadIdx.x; i < tpr * 2 * E; i += kThreads) {
     const int j = i / (2 * E), k = i % (2 * E);
-    const int64_t channel = (int64_t)blockIdx.x * 256 + j * E + k % E;
+    const int64_t channel = (int64_t)tile * 256 + j * E + k % E;
     if (j * E < 256 && channel < C) {
       float v = 0.0f;
       for (int rr = 0; rr < R; ++rr) v += s_part[(rr * tpr + j) * 2 * E + k];
-      part[(channel * 2 + k / E) * gridDim.y + blockIdx.y] = v;
+      part[(channel * 2 + k / E) * nsplit + brow] = v;
     }
   }
 }
@@ -1077,7 +1084,7 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
   };
   // first word of group `group` (counted over the tensor) of the located sample
   auto group_words = [&](uint32_t group) -> int32_t* { return cur_words + __umul24(group - cur_group0, (uint32_t)(8 * cur_b)); };
-  const RowTile t = row_tile<E>(C, tpr, R);
+  const RowTile t = row_tile<E>(C, tpr, R, blockIdx.x);
   float sumsq = 0.0f;
   if (!BWD && !t.active) return;       // whole quantisation groups leave together
   if (t.active) {                      // (backward: the lanes meet again for the wave's sum below)
@@ -1398,9 +1405,10 @@ void launch_apply(const Plan& pl, const XS& xs, const void* dy, const float* coe
 template <typename T, bool BWD, bool MINMAX, bool NT, typename XS>
 void launch_cl_reduce(const Plan& pl, const XS& xs, const void* dy, float* part, void* mn, void* mx,
                       int64_t C, hipStream_t s) {
-  const dim3 grid((unsigned)pl.tiles, (unsigned)pl.nsplit), blk(kThreads);
+  const dim3 grid(xcd_grid((int64_t)pl.tiles * pl.nsplit)), blk(kThreads);
   bn_cl_reduce_kernel<T, BWD, MINMAX, NT, XS><<<grid, blk, 0, s>>>(
-      xs, static_cast<const T*>(dy), part, static_cast<T*>(mn), static_cast<T*>(mx), pl.P, C, pl.tpr, pl.R, pl.ppb);
+      xs, static_cast<const T*>(dy), part, static_cast<T*>(mn), static_cast<T*>(mx), pl.P, C, pl.tpr, pl.R, pl.ppb,
+      pl.tiles, pl.nsplit);
 }
 template <typename T, bool BWD, bool PACK, typename XS>
 void launch_cl_apply(const Plan& pl, const XS& xs, const void* dy, const float* coef, void* out, int64_t C,

@@ -394,48 +394,6 @@ template <int ROWS> ACTNN_DEV void lanes_minmax(float& lo, float& hi) {
         : "+v"(lo), "+v"(hi));
 }
 
-// Reductions over a DPP row (16 consecutive lanes); every lane ends with the result.
-ACTNN_DEV float row16_max(float v) {
-  v = fmaxf(v, __builtin_bit_cast(float, lane_xor<1>(__builtin_bit_cast(uint32_t, v))));
-  v = fmaxf(v, __builtin_bit_cast(float, lane_xor<2>(__builtin_bit_cast(uint32_t, v))));
-  v = fmaxf(v, __builtin_bit_cast(float, (uint32_t)__builtin_amdgcn_update_dpp(
-                   0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false)));   // row_half_mirror
-  v = fmaxf(v, __builtin_bit_cast(float, (uint32_t)__builtin_amdgcn_update_dpp(
-                   0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false)));   // row_mirror
-  return v;
-}
-ACTNN_DEV float row16_min(float v) {
-  v = fminf(v, __builtin_bit_cast(float, lane_xor<1>(__builtin_bit_cast(uint32_t, v))));
-  v = fminf(v, __builtin_bit_cast(float, lane_xor<2>(__builtin_bit_cast(uint32_t, v))));
-  v = fminf(v, __builtin_bit_cast(float, (uint32_t)__builtin_amdgcn_update_dpp(
-                   0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false)));
-  v = fminf(v, __builtin_bit_cast(float, (uint32_t)__builtin_amdgcn_update_dpp(
-                   0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false)));
-  return v;
-}
-
-// Combine the per-row results of row16_min/max across the rows of the wave.  After the call
-// with ROWS == 2 the last row of each 32-lane half holds the half's result; with ROWS == 4
-// the last row of the wave (lanes 48..63) holds the wave's result.
-template <int ROWS> ACTNN_DEV float rows_min(float v) {
-  if (ROWS >= 2)   // row_bcast15 into rows 1 and 3
-    v = fminf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
-                     __builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false)));
-  if (ROWS >= 4)   // row_bcast31 into rows 2 and 3
-    v = fminf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
-                     __builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false)));
-  return v;
-}
-template <int ROWS> ACTNN_DEV float rows_max(float v) {
-  if (ROWS >= 2)
-    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
-                     __builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false)));
-  if (ROWS >= 4)
-    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
-                     __builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false)));
-  return v;
-}
-
 // ------------------------------------------------------------------ Philox4x32-10
 struct Philox4 { uint32_t x, y, z, w; };
 

@@ -183,11 +183,9 @@ __global__ __launch_bounds__(kThreads) void mask_forward16_kernel(const T* __res
   if (MINMAX) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      float lo = v[i][0], hi = v[i][0];
-#pragma unroll
-      for (int k = 1; k < 8; ++k) { lo = fminf(lo, v[i][k]); hi = fmaxf(hi, v[i][k]); }
-      lo = rows_min<2>(row16_min(lo));
-      hi = rows_max<2>(row16_max(hi));
+      float lo, hi;
+      minmax_of<8>(v[i], lo, hi);
+      lanes_minmax<2>(lo, hi);
       if ((lane & 31u) == 31u) {
         const int64_t g = tile * (kTileElems / 256) + i * (kMaskBlock / 256) + (lane >> 5);
         Conv<T>::store(mn, g, lo);

@@ -22,8 +22,8 @@ template <> struct Vec16<float> {
   static ACTNN_DEV void minmax(const float* p, float& lo, float& hi) {
     const u32x4 u = load16_nt(p);
     const float a = as_float(u.x), b = as_float(u.y), c = as_float(u.z), d = as_float(u.w);
-    lo = fminf(fminf(lo, a), fminf(b, fminf(c, d)));
-    hi = fmaxf(fmaxf(hi, a), fmaxf(b, fmaxf(c, d)));
+    lo = min3_f32(min3_f32(lo, a, b), c, d);
+    hi = max3_f32(max3_f32(hi, a, b), c, d);
   }
 };
 template <> struct Vec16<__half> {
@@ -37,8 +37,10 @@ template <> struct Vec16<__half> {
       v[2 * i] = half_bits_to_float(w[i] & 0xffffu);
       v[2 * i + 1] = half_bits_to_float(w[i] >> 16);
     }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) { lo = fminf(lo, v[i]); hi = fmaxf(hi, v[i]); }
+    float l8, h8;
+    minmax_of<8>(v, l8, h8);
+    lo = min_f32(lo, l8);
+    hi = max_f32(hi, h8);
   }
 };
 template <> struct Vec16<bf16_t> {
@@ -52,8 +54,10 @@ template <> struct Vec16<bf16_t> {
       v[2 * i] = as_float(w[i] << 16);
       v[2 * i + 1] = as_float(w[i] & 0xffff0000u);
     }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) { lo = fminf(lo, v[i]); hi = fmaxf(hi, v[i]); }
+    float l8, h8;
+    minmax_of<8>(v, l8, h8);
+    lo = min_f32(lo, l8);
+    hi = max_f32(hi, h8);
   }
 };
 
@@ -90,8 +94,8 @@ __global__ __launch_bounds__(kThreads) void minimax_vec_kernel(const T* __restri
   }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const float l = rows_min<LPR / 16>(row16_min(lo[r]));
-    const float h = rows_max<LPR / 16>(row16_max(hi[r]));
+    float l = lo[r], h = hi[r];
+    lanes_minmax<LPR / 16>(l, h);
     const int64_t row = row0 + r * kSlots;
     if (sub == LPR - 1 && row < M) {      // the last lane of the group holds the combined result
       Conv<T>::store(mn, row, l);
@@ -113,12 +117,11 @@ __global__ __launch_bounds__(kThreads) void minimax_generic_kernel(const T* __re
     const T* p = data + row * D;
     for (int64_t i = sub; i < D; i += 16) {
       const float v = Conv<T>::load(p, i);
-      lo = fminf(lo, v);
-      hi = fmaxf(hi, v);
+      lo = min_f32(lo, v);
+      hi = max_f32(hi, v);
     }
   }
-  lo = row16_min(lo);
-  hi = row16_max(hi);
+  lanes_minmax<1>(lo, hi);
   if (sub == 0 && row < M) {
     Conv<T>::store(mn, row, lo);
     Conv<T>::store(mx, row, hi);

@@ -3,8 +3,8 @@ quantise / dequantise glue around the kernels (behaviour of the reference's
 actnn/actnn/ops.py:22-629; sync_batch_norm across ranks is not part of this build).
 """
 import functools
+import math
 
-import numpy as np
 import torch
 import torch.nn.functional as F
 from torch.autograd.function import Function
@@ -53,7 +53,7 @@ def dequantize_and_unpack(data, shape, bits, scale, mn):
         data = swap_to_device(data)
     N = shape[0]
     gs = config.group_size
-    features = int(np.prod(shape[1:]))
+    features = math.prod(shape[1:])
     features = features + (gs - features % gs) % gs
     unpack = ext_quantization.unpack_single_precision if isinstance(bits, int) \
         else ext_quantization.unpack_mixed_precision
@@ -113,7 +113,7 @@ def dequantize_activation(quantized, q_input_shape):
         q_min = q_min.to(torch.float32)
     out = dequantize_and_unpack(q_input, q_input_shape, q_bits, q_scale, q_min)
     N = q_input_shape[0]
-    features = int(np.prod(q_input_shape[1:]))
+    features = math.prod(q_input_shape[1:])
     out = out.view(N, -1)[:, :features]
     memory_format = getattr(quantized, "memory_format", None)
     if memory_format is not None:

@@ -143,7 +143,7 @@ def compute_tensor_bytes(tensors):
     total = 0
     for t in tensors:
         if isinstance(t, torch.Tensor):
-            total += int(np.prod(t.size())) * _BYTES.get(t.dtype, 0)
+            total += t.numel() * _BYTES.get(t.dtype, 0)
     return total
 
 

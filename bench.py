@@ -535,6 +535,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the config-2 hot path")
+    ap.add_argument("--bn-shapes", default="", help="with --only batch_norm_shapes: CxH,... to keep (e.g. 256x14,512x7)")
     ap.add_argument("--only", choices=["other", "config4", "resnet50", "resnet50_channels_last", "resnet50_fp32", "resnet50_levels", "batch_norm_shapes"],
                     default=None,
                     help="profiling aid: run just the other single-GPU configs (ReLU, max-pool, "
@@ -593,7 +594,8 @@ def main():
         return
     if args.only == "batch_norm_shapes":
         import bench_extra
-        print(json.dumps({"batch_norm_shapes": [bench_extra.batch_norm_shapes(device, channels_last=cl)
+        keep = [tuple(int(v) for v in item.split("x")) for item in args.bn_shapes.split(",") if item]
+        print(json.dumps({"batch_norm_shapes": [bench_extra.batch_norm_shapes(device, channels_last=cl, keep=keep)
                                                 for cl in (True, False)]}))
         return
     xg, mn, mx, bits, bits_host = make_config2(device)

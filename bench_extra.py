@@ -88,11 +88,12 @@ RESNET50_BN_SHAPES = [(64, 112, 1), (64, 56, 6), (256, 56, 4), (128, 56, 1), (12
                       (256, 28, 1), (256, 14, 11), (1024, 14, 7), (512, 14, 1), (512, 7, 5), (2048, 7, 4)]
 
 
-def batch_norm_shapes(device, channels_last=True, batch=512, reps=10):
+def batch_norm_shapes(device, channels_last=True, batch=512, reps=10, keep=()):
     """The three fused batch-norm steps of an L3 training step (statistics + group min/max;
     normalise + 2-bit pack; backward from the packed input with the gradient norm), timed with
     events on every batch-norm shape of ResNet-50 in bf16: ms and GB/s of algorithmic bytes per
-    shape, and the totals weighted by the number of layers."""
+    shape, and the totals weighted by the number of layers.  `keep`: (C, H) pairs to restrict the run
+    to (for counter runs on single shapes)."""
     import actnn_amd.cpp_extension.backward_func as bf
     from actnn_amd.cpp_extension.quantization import attach_bits_total
     from actnn_amd.ops import _Quantized
@@ -124,7 +125,8 @@ def batch_norm_shapes(device, channels_last=True, batch=512, reps=10):
         return each[reps // 2]
 
     rows, totals = [], [0.0, 0.0, 0.0]
-    for C, H, count in RESNET50_BN_SHAPES:
+    shapes = [sh for sh in RESNET50_BN_SHAPES if not keep or sh[:2] in keep]
+    for C, H, count in shapes:
         x = torch.randn(batch, C, H, H, device=device, dtype=torch.bfloat16)
         dy = torch.randn_like(x)
         if channels_last:
@@ -151,5 +153,5 @@ def batch_norm_shapes(device, channels_last=True, batch=512, reps=10):
             "ms_per_training_step": [round(v, 3) for v in totals],
             # (three timed calls per shape, in the order of `steps`)
             "slowest_repetition": {"over_median": round(max(worst)[0], 2), "ms": round(max(worst)[1], 3),
-                                   "shape": RESNET50_BN_SHAPES[worst.index(max(worst)) // 3][:2],
+                                   "shape": shapes[worst.index(max(worst)) // 3][:2],
                                    "step": worst.index(max(worst)) % 3}}
