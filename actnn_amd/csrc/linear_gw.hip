@@ -41,12 +41,20 @@
 // schedule in the kernel).  Loads of packed data and scale/min run one step ahead of the staging
 // code (widths and stream offsets of the mixed stream two steps ahead).
 //
-// What bounds it on MI355X: with normally distributed 16-bit operands the matrix pipes are held
-// back by the power limit, not by this kernel's structure - the vendor GEMM (rocBLAS) on the same
-// dequantised operands and three differently organised versions of this kernel (8 waves of 64 x 128
-// with register transposes; the same with transposing reads; this one) all take 0.29 - 0.32 ms for
-// [8192, 4096]^T x [8192, 4096] (0.86 - 0.95 PFLOP/s at about 1.8 GHz), and all of them speed up by
-// a quarter to a third when one operand is all zeros or ones.
+// Shapes with few output tiles and many samples (fewer than half the CUs busy) split the sum over the
+// samples across blocks: every block writes its fp32 tile into a workspace and a second kernel adds
+// the tiles in a fixed order (bit-reproducible, no atomics).
+//
+// What bounds it on MI355X: the matrix pipes themselves.  A kernel that issues the same 8.4 M
+// v_mfma_f32_32x32x16 from registers and nothing else (actnn_matrix_pipe_probe) takes 0.167 ms with
+// normally distributed operands against 0.127 ms with zeros: in both cases the pipes are busy 79 % of
+// the cycles, but the part lowers its clock from 2.49 to 2.01 GHz when the operands switch many bits.
+// 1650 TFLOP/s (66 % of the published 2.5 PFLOP/s) is therefore the ceiling of a 16-bit GEMM on
+// N(0,1) data; this kernel reaches 0.25 ms = 1090 TFLOP/s on [8192, 4096]^T x [8192, 4096] with the
+// 2-bit stream, level with rocBLAS on the dequantised copy (0.24 ms) and ahead of unpack + rocBLAS.
+// The general loader decodes every element with shifts and a multiply-add (six times the vector
+// instructions of the table loader) and loses to unpack + rocBLAS by 3-4x: the layers route only the
+// 2-bit fixed-width stream here by default.
 #include <type_traits>
 
 #include "quant_math.h"

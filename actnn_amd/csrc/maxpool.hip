@@ -464,11 +464,20 @@ __global__ __launch_bounds__(kBwdS2Threads) void max_pool2d_backward_s2_kernel(
   const int ho_hi = s0 + pairs - 1 + EXTRA < g.Ho - 1 ? s0 + pairs - 1 + EXTRA : g.Ho - 1;
   const int64_t first = (nc * g.Ho + s0) * (int64_t)g.Wo;
   const int count = (ho_hi - s0 + 1) * g.Wo;
-  // (first and count are multiples of 4: whole bytes in the two-per-byte format)
-  const Span<T> span_g = span_of(gout, first, count, total_out);
-  const Span<int8_t> span_i = NIB ? span_of(idx, first >> 1, count >> 1, total_out >> 1) : span_of(idx, first, count, total_out);
-  stage_two<kBwdS2Threads>(span_g, s_g, span_i, s_i);
-  const int shift_g = span_g.shift, shift_i = NIB ? 2 * span_i.shift : span_i.shift;
+  int shift_g, shift_i;
+  if constexpr (NIB) {
+    // (first and count are multiples of 4: whole bytes in the two-per-byte format)
+    const Span<T> span_g = span_of(gout, first, count, total_out);
+    const Span<int8_t> span_i = span_of(idx, first >> 1, count >> 1, total_out >> 1);
+    stage_two<kBwdS2Threads>(span_g, s_g, span_i, s_i);
+    shift_g = span_g.shift;
+    shift_i = 2 * span_i.shift;
+  } else {
+    // (one index per byte: staged one span after the other; in one round it measured 10 % faster on
+    // one machine and 19 % slower on another)
+    shift_g = stage_span<T, kBwdS2Threads, false>(gout, first, count, total_out, s_g);
+    shift_i = stage_span<int8_t, kBwdS2Threads, false>(idx, first, count, total_out, s_i);
+  }
   __syncthreads();
   const int cpr = g.W >> 3;
   const int items = pairs * cpr;
