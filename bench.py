@@ -535,6 +535,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the config-2 hot path")
+    ap.add_argument("--batch", type=int, default=512, help="with --only resnet50_levels: images per step")
     ap.add_argument("--bn-shapes", default="", help="with --only batch_norm_shapes: CxH,... to keep (e.g. 256x14,512x7)")
     ap.add_argument("--only", choices=["other", "config4", "resnet50", "resnet50_channels_last", "resnet50_fp32", "resnet50_levels", "batch_norm_shapes"],
                     default=None,
@@ -588,7 +589,8 @@ def main():
         for level in ("exact", "L0", "L1", "L2", "L3", "L3.1", "L4", "swap"):
             torch.cuda.empty_cache()
             torch.cuda.reset_peak_memory_stats()
-            out["resnet50_" + level] = bench_extra.resnet50_step(device, level, warmup=2, steps=5, channels_last=True)
+            out["resnet50_" + level] = bench_extra.resnet50_step(device, level, batch=args.batch, warmup=2, steps=5,
+                                                                 channels_last=True)
             print("[bench] %s done" % level, file=sys.stderr, flush=True)
         print(json.dumps(out))
         return
