@@ -36,8 +36,25 @@ def _config2(dtype=torch.float32):
 
 def test_config2_full_size_deterministic_mode():
     x, mn, mx, bits = _config2()
+    assert len(set(bits)) > 2
+    _check_config2(x, mn, mx, bits)
+
+
+def test_config2_full_size_on_the_benchmarks_own_tensor():
+    """The tensor and widths `bench.py` measures (BASELINE's distribution: identically distributed
+    samples, so the greedy allocation gives nearly every sample 2 bits), through the same checks."""
+    import os
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench
+    x, mn, mx, _, b = bench.make_config2(DEV)
+    _check_config2(x, mn, mx, [int(v) for v in b])
+
+
+def _check_config2(x, mn, mx, bits):
     N, G, gs = x.shape
-    assert min(bits) >= 1 and max(bits) <= 8 and abs(np.mean(bits) - 2.0) < 0.02 and len(set(bits)) > 2
+    assert (N, G, gs) == (256, 3136, 256)
+    assert min(bits) >= 1 and max(bits) <= 8 and abs(np.mean(bits) - 2.0) < 0.02
     bits_dev, bits_host = bits_tensor(bits)
     noise = torch.rand(x.shape, generator=torch.Generator(device=DEV).manual_seed(3), device=DEV) - 0.5
     packed, scale = ext_q.pack_mixed_precision(x, mn, mx, bits_dev, True, noise=noise)

@@ -205,6 +205,38 @@ def test_l3_first_step_uses_the_degenerate_allocation_then_rebalances():
     assert int(s0.b.sum()) <= int(budgets[0] * 16) and int(s0.b.min()) >= 1
 
 
+def test_sensitivities_reach_the_host_in_one_transfer_per_step():
+    """The widths are made on the device; the sensitivities of all layers travel in one pool.  What
+    the host reads per layer equals what the layer's own kernel computes from its input's ranges,
+    one step after another, and a change of the batch size makes a new pool."""
+    from actnn_amd import qscheme
+    torch.manual_seed(0)
+    model = QModule(nn.Sequential(nn.Conv2d(8, 8, 3, padding=1), nn.ReLU(), nn.Conv2d(8, 8, 3, padding=1),
+                                  nn.ReLU(), nn.Conv2d(8, 4, 1))).to(DEV)
+    seen = []
+    start = QScheme.start_quantization_bits
+
+    def spy(self, input, known_minmax=None):
+        groups, mn, mx, num_pixels = qscheme.group_min_max(input, known_minmax)
+        seen.append((self, self.sensitivity(mn, mx, input.shape[0], num_pixels).clone()))
+        return start(self, input, known_minmax)
+
+    QScheme.start_quantization_bits = spy
+    try:
+        for step, n in enumerate((16, 16, 8)):
+            seen.clear()
+            x = torch.randn(n, 8, 16, 16, device=DEV)
+            model(x).square().mean().backward()
+            pool = QScheme.sensitivity_pool
+            assert pool is not None and pool.dev.shape == (3, n) and not pool.dirty
+            assert len(seen) == 3
+            for scheme, expected in seen:
+                assert scheme.C.shape == (n,)
+                assert torch.equal(scheme.C, expected.cpu()), (step, scheme.name)
+    finally:
+        QScheme.start_quantization_bits = start
+
+
 @pytest.mark.parametrize("channels_last", [False, True])
 def test_small_model_trains_at_l3(channels_last):
     # the same toy problem with stock layers and with 2-bit compressed activations: the loss
