@@ -41,6 +41,7 @@ SIGNATURES = {
     "actnn_unpack_single": [c_vp, c_i32, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i32, c_vp],
     "actnn_relu_forward": [c_vp, c_vp, c_vp, c_i64, c_i32, c_vp],
     "actnn_relu_forward_minmax": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i32, c_vp],
+    "actnn_relu_add_forward": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i32, c_vp],
     "actnn_relu_backward": [c_vp, c_vp, c_vp, c_i64, c_i32, c_vp],
     "actnn_dropout_forward": [c_vp, c_vp, c_vp, c_i64, ctypes.c_float, c_u64, c_u64, c_i32, c_vp],
     "actnn_dropout_backward": [c_vp, c_vp, c_vp, c_i64, ctypes.c_float, c_i32, c_vp],

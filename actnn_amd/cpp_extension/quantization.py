@@ -339,6 +339,69 @@ class ActQuantizedReLUMinMax(Function):
         return relu_backward(grad_output, mask)
 
 
+def relu_add_forward(x, residual, minmax=False):
+    """-> (y, mask[, mn, mx]) of relu(x + residual) in one pass; the sum is rounded to the tensors'
+    dtype as the tensor addition rounds it."""
+    n = x.numel()
+    y = torch.empty_like(x)
+    mask = torch.empty(mask_words(n), dtype=torch.int32, device=x.device)
+    mn = mx = None
+    if minmax:
+        mn = torch.empty(n // 256, dtype=x.dtype, device=x.device)
+        mx = torch.empty(n // 256, dtype=x.dtype, device=x.device)
+    with g.on_device(x.device):
+        check(g.lib().actnn_relu_add_forward(
+            x.data_ptr(), residual.data_ptr(), y.data_ptr(), mask.data_ptr(),
+            mn.data_ptr() if minmax else None, mx.data_ptr() if minmax else None, n,
+            g.DTYPE_CODE[x.dtype], g.stream_ptr(x.device)), "relu_add_forward")
+    return (y, mask, mn, mx) if minmax else (y, mask)
+
+
+class ActQuantizedAddReLU(Function):
+    """relu(input + residual) that saves only the 1-bit mask; both operands receive the masked
+    gradient."""
+
+    @staticmethod
+    def forward(ctx, input, residual):
+        output, mask = relu_add_forward(input, residual)
+        ctx.save_for_backward(mask)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (mask,) = ctx.saved_tensors
+        grad = relu_backward(grad_output, mask)
+        return grad, grad
+
+
+class ActQuantizedAddReLUMinMax(Function):
+    """The same, additionally returning the group min / max of the output (not differentiable)."""
+
+    @staticmethod
+    def forward(ctx, input, residual):
+        output, mask, mn, mx = relu_add_forward(input, residual, minmax=True)
+        ctx.save_for_backward(mask)
+        ctx.mark_non_differentiable(mn, mx)
+        ctx.set_materialize_grads(False)
+        return output, mn, mx
+
+    @staticmethod
+    def backward(ctx, grad_output, _grad_mn, _grad_mx):
+        if grad_output is None:
+            return None, None
+        (mask,) = ctx.saved_tensors
+        grad = relu_backward(grad_output, mask)
+        return grad, grad
+
+
+def add_relu_applies(x, residual):
+    """Same shape, dtype, device and dense memory order, 16-byte aligned."""
+    return (x.is_cuda and residual.is_cuda and x.device == residual.device and x.dtype == residual.dtype
+            and x.dtype in g.DTYPE_CODE and x.shape == residual.shape and x.is_contiguous()
+            and residual.is_contiguous() and x.numel() > 0
+            and x.data_ptr() % 16 == 0 and residual.data_ptr() % 16 == 0)
+
+
 def act_quantized_relu(input):
     g.check_float(input, "input")                                                  # quantization.cc:122
     return ActQuantizedReLU.apply(input)

@@ -1402,13 +1402,30 @@ void launch_apply(const Plan& pl, const XS& xs, const void* dy, const float* coe
     bn_apply_kernel<T, false, BWD, PACK, XS><<<grid, blk, 0, s>>>(xs, pd, coef, po, N, pl.F, HW, pl.per_block, ps);
 }
 
+// Rows per block and block rows of a channels-last reduce pass whose kernel holds `waves` waves per
+// SIMD: as many blocks as the chip holds at once (a block is one wave on each SIMD of its CU), so that
+// the pass is one round of blocks that end together.  With the plan's 8 blocks per CU a kernel that
+// holds 7 or 5 ran the rest as a second round on a chip that was mostly idle.  Never more block rows
+// than the plan's, which sizes the table.
+struct ClRows { int64_t ppb; int nsplit; };
+ClRows cl_reduce_rows(const Plan& pl, int waves) {
+  int64_t want = (int64_t)kCUs * waves / pl.tiles;
+  if (want < 1) want = 1;
+  int64_t ppb = (pl.P + want - 1) / want;
+  if (ppb < pl.ppb) ppb = pl.ppb;
+  ppb = (ppb + pl.R - 1) / pl.R * pl.R;
+  return ClRows{ppb, (int)((pl.P + ppb - 1) / ppb)};
+}
+// -> the block rows of the table it leaves
 template <typename T, bool BWD, bool MINMAX, bool NT, typename XS>
-void launch_cl_reduce(const Plan& pl, const XS& xs, const void* dy, float* part, void* mn, void* mx,
-                      int64_t C, hipStream_t s) {
-  const dim3 grid(xcd_grid((int64_t)pl.tiles * pl.nsplit)), blk(kThreads);
+int launch_cl_reduce(const Plan& pl, const XS& xs, const void* dy, float* part, void* mn, void* mx,
+                     int64_t C, hipStream_t s) {
+  const ClRows rows = cl_reduce_rows(pl, cl_reduce_waves<BWD, MINMAX, XS>());
+  const dim3 grid(xcd_grid((int64_t)pl.tiles * rows.nsplit)), blk(kThreads);
   bn_cl_reduce_kernel<T, BWD, MINMAX, NT, XS><<<grid, blk, 0, s>>>(
-      xs, static_cast<const T*>(dy), part, static_cast<T*>(mn), static_cast<T*>(mx), pl.P, C, pl.tpr, pl.R, pl.ppb,
-      pl.tiles, pl.nsplit);
+      xs, static_cast<const T*>(dy), part, static_cast<T*>(mn), static_cast<T*>(mx), pl.P, C, pl.tpr, pl.R, rows.ppb,
+      pl.tiles, rows.nsplit);
+  return rows.nsplit;
 }
 template <typename T, bool BWD, bool PACK, typename XS>
 void launch_cl_apply(const Plan& pl, const XS& xs, const void* dy, const float* coef, void* out, int64_t C,
@@ -1425,6 +1442,7 @@ int forward_stats_t(const Plan& pl, const void* x, const float* weight, const fl
                     int64_t N, int64_t C, int64_t HW, double momentum, double eps, hipStream_t s) {
   float* part = ws;
   float* coef = ws + pl.part_floats;
+  int nsplit = pl.nsplit;
   if (pl.any_shape) {
     const dim3 grid((unsigned)C, (unsigned)pl.nsplit), blk(kThreads);
     if (pl.channels_last)
@@ -1434,12 +1452,12 @@ int forward_stats_t(const Plan& pl, const void* x, const float* weight, const fl
   } else if (pl.channels_last) {
     if (pl.big) {
       const PlainRows<T, true> xs{static_cast<const T*>(x), C};
-      if (mn) launch_cl_reduce<T, false, true, true>(pl, xs, nullptr, part, mn, mx, C, s);
-      else launch_cl_reduce<T, false, false, true>(pl, xs, nullptr, part, nullptr, nullptr, C, s);
+      if (mn) nsplit = launch_cl_reduce<T, false, true, true>(pl, xs, nullptr, part, mn, mx, C, s);
+      else nsplit = launch_cl_reduce<T, false, false, true>(pl, xs, nullptr, part, nullptr, nullptr, C, s);
     } else {
       const PlainRows<T> xs{static_cast<const T*>(x), C};
-      if (mn) launch_cl_reduce<T, false, true, false>(pl, xs, nullptr, part, mn, mx, C, s);
-      else launch_cl_reduce<T, false, false, false>(pl, xs, nullptr, part, nullptr, nullptr, C, s);
+      if (mn) nsplit = launch_cl_reduce<T, false, true, false>(pl, xs, nullptr, part, mn, mx, C, s);
+      else nsplit = launch_cl_reduce<T, false, false, false>(pl, xs, nullptr, part, nullptr, nullptr, C, s);
     }
   } else {
     const PlainInput<T> xs{static_cast<const T*>(x), pl.F};
@@ -1447,7 +1465,7 @@ int forward_stats_t(const Plan& pl, const void* x, const float* weight, const fl
     else launch_reduce<T, false, false>(pl, xs, nullptr, part, nullptr, nullptr, N, HW, s);
   }
   bn_forward_finalize_kernel<<<dim3((unsigned)((C + kWaves - 1) / kWaves)), dim3(kThreads), 0, s>>>(
-      part, weight, bias, running_mean, running_var, save_mean, save_invstd, coef, N, C, HW, pl.L, pl.nsplit,
+      part, weight, bias, running_mean, running_var, save_mean, save_invstd, coef, N, C, HW, pl.L, nsplit,
       pl.slots, momentum, eps);
   ACTNN_RETURN_LAUNCH_STATUS();
 }
@@ -1489,13 +1507,14 @@ int backward_t(const Plan& pl, const XS& xs, const void* dy, const float* weight
                int64_t C, int64_t HW, float* sumsq, hipStream_t s, bool eval = false) {
   float* part = ws;
   float* coef = ws + pl.part_floats;
+  int nsplit = pl.nsplit;
   if constexpr (XS::kRows) {
-    if (pl.big) launch_cl_reduce<T, true, false, true>(pl, xs, dy, part, nullptr, nullptr, C, s);
-    else launch_cl_reduce<T, true, false, false>(pl, xs, dy, part, nullptr, nullptr, C, s);
+    if (pl.big) nsplit = launch_cl_reduce<T, true, false, true>(pl, xs, dy, part, nullptr, nullptr, C, s);
+    else nsplit = launch_cl_reduce<T, true, false, false>(pl, xs, dy, part, nullptr, nullptr, C, s);
   }
   else launch_reduce<T, true, false>(pl, xs, dy, part, nullptr, nullptr, N, HW, s);
   bn_backward_finalize_kernel<<<dim3((unsigned)((C + kWaves - 1) / kWaves)), dim3(kThreads), 0, s>>>(
-      part, weight, save_mean, save_invstd, dweight, dbias, coef, N, C, HW, pl.L, pl.nsplit, pl.slots, eval);
+      part, weight, save_mean, save_invstd, dweight, dbias, coef, N, C, HW, pl.L, nsplit, pl.slots, eval);
   if (dx) {
     PackSink extra{};
     extra.sumsq = sumsq;

@@ -55,6 +55,18 @@ template <> struct Conv<bf16_t> {
   static ACTNN_DEV float round(float v) { return bf16_bits_to_float(float_to_bf16_bits(v)); }
 };
 
+// Two values rounded to T and back (what storing and reloading them would give): one packed
+// conversion for bf16.
+template <typename T> ACTNN_DEV void round_pair(float& a, float& b) {
+  a = Conv<T>::round(a);
+  b = Conv<T>::round(b);
+}
+template <> ACTNN_DEV void round_pair<bf16_t>(float& a, float& b) {
+  const uint32_t w = pack_bf16x2(a, b);
+  a = as_float(w << 16);
+  b = as_float(w & 0xffff0000u);
+}
+
 // ------------------------------------------------------------------ 16-byte vector access
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -232,6 +244,7 @@ ACTNN_DEV void store8_nt(bf16_t* p, const float (&v)[8]) {
 // that a run of consecutive logical blocks stays on one XCD: launch xcd_grid(n) blocks, work on block
 // xcd_block(); logical blocks >= n have nothing to do.
 constexpr int kXcds = 8;
+constexpr int kCUs = 256;          // compute units of the chip, 32 per XCD
 inline unsigned xcd_grid(int64_t n) { return (unsigned)((n + kXcds - 1) / kXcds * kXcds); }
 ACTNN_DEV int64_t xcd_block() {
   return (int64_t)(blockIdx.x % kXcds) * (gridDim.x / kXcds) + blockIdx.x / kXcds;

@@ -24,7 +24,8 @@ __global__ __launch_bounds__(kThreads) void mask_forward_kernel(const T* __restr
                                                                 int32_t* __restrict__ mask, int64_t n,
                                                                 int64_t n_mask_blocks, uint32_t thr,
                                                                 float keep_div, uint64_t seed,
-                                                                uint64_t offset, int64_t elem_offset) {
+                                                                uint64_t offset, int64_t elem_offset,
+                                                                const T* __restrict__ add = nullptr) {
   const uint32_t lane = threadIdx.x & 31;
   const int64_t mb0 = (int64_t)blockIdx.x * kMaskBlocksPerBlock + (threadIdx.x >> 5) * 2;
   uint32_t acc = 0;
@@ -40,6 +41,18 @@ __global__ __launch_bounds__(kThreads) void mask_forward_kernel(const T* __restr
     } else {
 #pragma unroll
       for (int k = 0; k < 16; ++k) v[k] = e0 + k < n ? Conv<T>::load(x, e0 + k) : 0.0f;
+    }
+    if (add) {                                       // the sum as a tensor addition rounds it, then the rule
+      float a[16];
+      if (full) {
+        load8(add + e0, reinterpret_cast<float(&)[8]>(a[0]));
+        load8(add + e0 + 8, reinterpret_cast<float(&)[8]>(a[8]));
+      } else {
+#pragma unroll
+        for (int k = 0; k < 16; ++k) a[k] = e0 + k < n ? Conv<T>::load(add, e0 + k) : 0.0f;
+      }
+#pragma unroll
+      for (int k = 0; k < 16; ++k) v[k] = Conv<T>::round(v[k] + a[k]);
     }
     uint32_t bitsr = 0;
     if (OP == Op::kRelu) {
@@ -151,13 +164,16 @@ ACTNN_DEV void word_to_rows(uint32_t w, uint32_t lane, uint32_t (&m)[4]) {
 // MINMAX: also write the minimum and maximum of every group of 256 consecutive outputs (the lower
 // and upper 32 lanes of each load own one group each) - what actnn_minimax returns for the output
 // viewed as rows of 256, for a consumer that quantises it next.
-template <typename T, Op OP, bool MINMAX = false>
+// ADD: the rule is applied to x + add, rounded to T as the tensor addition it replaces rounds it
+// (the closing `relu(out + identity)` of a residual block in one pass over the two operands).
+template <typename T, Op OP, bool MINMAX = false, bool ADD = false>
 __global__ __launch_bounds__(kThreads) void mask_forward16_kernel(const T* __restrict__ x, T* __restrict__ y,
                                                                   int32_t* __restrict__ mask, int64_t tiles,
                                                                   uint32_t thr, float keep_div,
                                                                   uint64_t seed, uint64_t offset,
                                                                   T* __restrict__ mn = nullptr,
-                                                                  T* __restrict__ mx = nullptr) {
+                                                                  T* __restrict__ mx = nullptr,
+                                                                  const T* __restrict__ add = nullptr) {
   const uint32_t lane = threadIdx.x & 63;
   const int64_t tile = (int64_t)blockIdx.x * kTilesPerBlock + (threadIdx.x >> 6);
   if (tile >= tiles) return;                       // whole waves leave together
@@ -165,6 +181,19 @@ __global__ __launch_bounds__(kThreads) void mask_forward16_kernel(const T* __res
   float v[4][8];
 #pragma unroll
   for (int i = 0; i < 4; ++i) load8_nt(x + e0 + i * kMaskBlock, v[i]);
+  if (ADD) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float a[8];
+      load8_nt(add + e0 + i * kMaskBlock, a);
+#pragma unroll
+      for (int k = 0; k < 8; k += 2) {
+        v[i][k] += a[k];
+        v[i][k + 1] += a[k + 1];
+        round_pair<T>(v[i][k], v[i][k + 1]);
+      }
+    }
+  }
   uint32_t m[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -225,17 +254,23 @@ __global__ __launch_bounds__(kThreads) void mask_backward16_kernel(const T* __re
 
 template <typename T, Op OP>
 int launch_forward(const void* x, void* y, int32_t* mask, int64_t n, uint32_t thr, float keep_div,
-                   uint64_t seed, uint64_t offset, hipStream_t s) {
+                   uint64_t seed, uint64_t offset, hipStream_t s, const void* add = nullptr) {
   const T* xi = static_cast<const T*>(x);
+  const T* ai = static_cast<const T*>(add);
   T* yo = static_cast<T*>(y);
   int64_t done = 0;                               // elements handled by the whole-line kernel
   if (sizeof(T) == 2) {
     const int64_t tiles = n / kTileElems;
     const int64_t tblocks = (tiles + kTilesPerBlock - 1) / kTilesPerBlock;
     if (tblocks > 0x7fffffffLL) return ACTNN_EINVAL;
-    if (tiles > 0)
-      mask_forward16_kernel<T, OP><<<dim3((unsigned)tblocks), dim3(kThreads), 0, s>>>(
-          xi, yo, mask, tiles, thr, keep_div, seed, offset);
+    if (tiles > 0) {
+      if (ai)
+        mask_forward16_kernel<T, OP, false, true><<<dim3((unsigned)tblocks), dim3(kThreads), 0, s>>>(
+            xi, yo, mask, tiles, thr, keep_div, seed, offset, nullptr, nullptr, ai);
+      else
+        mask_forward16_kernel<T, OP><<<dim3((unsigned)tblocks), dim3(kThreads), 0, s>>>(
+            xi, yo, mask, tiles, thr, keep_div, seed, offset);
+    }
     done = tiles * kTileElems;
   }
   const int64_t rest = n - done;
@@ -244,7 +279,8 @@ int launch_forward(const void* x, void* y, int32_t* mask, int64_t n, uint32_t th
     const int64_t blocks = (nmb + kMaskBlocksPerBlock - 1) / kMaskBlocksPerBlock;
     if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
     mask_forward_kernel<T, OP><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
-        xi + done, yo + done, mask + done / 32, rest, nmb, thr, keep_div, seed, offset, done);
+        xi + done, yo + done, mask + done / 32, rest, nmb, thr, keep_div, seed, offset, done,
+        ai ? ai + done : nullptr);
   }
   ACTNN_RETURN_LAUNCH_STATUS();
 }
@@ -277,16 +313,16 @@ int launch_backward(const void* gout, const int32_t* mask, void* gin, int64_t n,
 
 template <Op OP>
 int dispatch_forward(const void* x, void* y, int32_t* mask, int64_t n, uint32_t thr, float keep_div,
-                     uint64_t seed, uint64_t offset, int dtype, void* stream) {
+                     uint64_t seed, uint64_t offset, int dtype, void* stream, const void* add = nullptr) {
   if (n < 0) return ACTNN_EINVAL;
   if (n == 0) return ACTNN_OK;
   if (!x || !y || !mask) return ACTNN_EINVAL;
-  if (!aligned16(x) || !aligned16(y)) return ACTNN_EALIGN;
+  if (!aligned16(x) || !aligned16(y) || !aligned16(add)) return ACTNN_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (dtype) {
-    case ACTNN_F32: return launch_forward<float, OP>(x, y, mask, n, thr, keep_div, seed, offset, s);
-    case ACTNN_F16: return launch_forward<__half, OP>(x, y, mask, n, thr, keep_div, seed, offset, s);
-    case ACTNN_BF16: return launch_forward<bf16_t, OP>(x, y, mask, n, thr, keep_div, seed, offset, s);
+    case ACTNN_F32: return launch_forward<float, OP>(x, y, mask, n, thr, keep_div, seed, offset, s, add);
+    case ACTNN_F16: return launch_forward<__half, OP>(x, y, mask, n, thr, keep_div, seed, offset, s, add);
+    case ACTNN_BF16: return launch_forward<bf16_t, OP>(x, y, mask, n, thr, keep_div, seed, offset, s, add);
     default: return ACTNN_EDTYPE;
   }
 }
@@ -342,6 +378,33 @@ extern "C" int actnn_relu_forward_minmax(const void* x, void* y, int32_t* mask, 
     mask_forward16_kernel<bf16_t, Op::kRelu, true><<<grid, blk, 0, s>>>(
         static_cast<const bf16_t*>(x), static_cast<bf16_t*>(y), mask, tiles, 0u, 1.0f, 0, 0,
         static_cast<bf16_t*>(mn), static_cast<bf16_t*>(mx));
+  ACTNN_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int actnn_relu_add_forward(const void* x, const void* residual, void* y, int32_t* mask, void* mn,
+                                      void* mx, int64_t n, int dtype, void* stream) {
+  using namespace actnn;
+  if ((mn == nullptr) != (mx == nullptr)) return ACTNN_EINVAL;
+  if (n > 0 && !residual) return ACTNN_EINVAL;
+  if (!mn) return dispatch_forward<Op::kRelu>(x, y, mask, n, 0u, 1.0f, 0, 0, dtype, stream, residual);
+  if (n < 0 || n % kTileElems != 0) return ACTNN_EINVAL;       // whole tiles of 2048 elements only
+  if (dtype != ACTNN_F16 && dtype != ACTNN_BF16) return ACTNN_EDTYPE;
+  if (n == 0) return ACTNN_OK;
+  if (!x || !y || !mask) return ACTNN_EINVAL;
+  if (!aligned16(x) || !aligned16(residual) || !aligned16(y)) return ACTNN_EALIGN;
+  const int64_t tiles = n / kTileElems;
+  const int64_t blocks = (tiles + kTilesPerBlock - 1) / kTilesPerBlock;
+  if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)blocks), blk(kThreads);
+  if (dtype == ACTNN_F16)
+    mask_forward16_kernel<__half, Op::kRelu, true, true><<<grid, blk, 0, s>>>(
+        static_cast<const __half*>(x), static_cast<__half*>(y), mask, tiles, 0u, 1.0f, 0, 0,
+        static_cast<__half*>(mn), static_cast<__half*>(mx), static_cast<const __half*>(residual));
+  else
+    mask_forward16_kernel<bf16_t, Op::kRelu, true, true><<<grid, blk, 0, s>>>(
+        static_cast<const bf16_t*>(x), static_cast<bf16_t*>(y), mask, tiles, 0u, 1.0f, 0, 0,
+        static_cast<bf16_t*>(mn), static_cast<bf16_t*>(mx), static_cast<const bf16_t*>(residual));
   ACTNN_RETURN_LAUNCH_STATUS();
 }
 

@@ -275,6 +275,37 @@ class QReLU(nn.Module):
         return logical_order(out, fmt) if fmt is not None else out
 
 
+class AddReLU(nn.Module):
+    """relu(a + b): the closing step of a residual block as a module of its own, so that QModule can
+    swap it for the fused layer below (plain torch here; the sum is a tensor of its own)."""
+
+    def forward(self, a, b):
+        return F.relu(a + b, inplace=True)
+
+
+class QAddReLU(nn.Module):
+    """relu(a + b) in one pass over the two operands, saving the 1-bit mask: the values and the mask
+    of the addition followed by QReLU, without writing and re-reading the sum."""
+
+    def __init__(self):
+        super().__init__()
+        self.relu = QReLU()
+
+    def forward(self, a, b):
+        fmt = channels_last_format(a)
+        if fmt == channels_last_format(b):
+            x, r = (memory_order(a), memory_order(b)) if fmt is not None else (a, b)
+            if ext_quantization.add_relu_applies(x, r):
+                if _relu_shares_min_max(x):
+                    out, mn, mx = ext_quantization.ActQuantizedAddReLUMinMax.apply(x, r)
+                    out = logical_order(out, fmt) if fmt is not None else out
+                    out._actnn_group_minmax = (mn, mx, out._version)
+                    return out
+                out = ext_quantization.ActQuantizedAddReLU.apply(x, r)
+                return logical_order(out, fmt) if fmt is not None else out
+        return self.relu(a + b)
+
+
 class QDropout(nn.Dropout):
     def __init__(self, p=0.5):
         super().__init__(p=p)

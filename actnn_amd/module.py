@@ -6,12 +6,12 @@ import torch
 import torch.nn as nn
 
 from .conf import config
-from .layers import (QAvgPool2d, QBatchNorm1d, QBatchNorm2d, QBatchNorm3d, QConv1d, QConv2d, QConv3d,
+from .layers import (AddReLU, QAddReLU, QAvgPool2d, QBatchNorm1d, QBatchNorm2d, QBatchNorm3d, QConv1d, QConv2d, QConv3d,
                      QConvTranspose1d, QConvTranspose2d, QConvTranspose3d, QDropout, QLinear, QMaxPool2d,
                      QReLU, QSyncBatchNorm)
 
 _Q_TYPES = (QConv1d, QConv2d, QConv3d, QConvTranspose1d, QConvTranspose2d, QConvTranspose3d, QBatchNorm1d,
-            QBatchNorm2d, QBatchNorm3d, QSyncBatchNorm, QReLU, QDropout, QLinear, QMaxPool2d, QAvgPool2d)
+            QBatchNorm2d, QBatchNorm3d, QSyncBatchNorm, QReLU, QAddReLU, QDropout, QLinear, QMaxPool2d, QAvgPool2d)
 
 
 def _convert(child):
@@ -38,6 +38,8 @@ def _convert(child):
         return QLinear(child.in_features, child.out_features, child.bias is not None)
     if isinstance(child, nn.ReLU):
         return QReLU()
+    if isinstance(child, AddReLU):
+        return QAddReLU()
     if isinstance(child, nn.Dropout):
         return QDropout(child.p)
     if isinstance(child, nn.MaxPool2d):

@@ -1,9 +1,12 @@
 """ResNet-50 (v1.5: stride on the 3x3 convolution) in the standard public layout, built from
-plain torch.nn layers so that QModule can convert it.  torchvision is not available in this
+plain torch.nn layers (and AddReLU for the closing relu(out + identity) of a block) so that QModule
+can convert it.  torchvision is not available in this
 environment; the reference benchmarks torchvision's resnet50
 (mem_speed_benchmark/train.py:170,203-206)."""
 import torch
 import torch.nn as nn
+
+from .layers import AddReLU
 
 
 class Bottleneck(nn.Module):
@@ -20,7 +23,7 @@ class Bottleneck(nn.Module):
         # three separate modules: a converted ReLU keeps one mask per call site
         self.relu1 = nn.ReLU(inplace=True)
         self.relu2 = nn.ReLU(inplace=True)
-        self.relu3 = nn.ReLU(inplace=True)
+        self.relu3 = AddReLU()          # relu(out + identity), fused into one pass when converted
         self.downsample = downsample
 
     def forward(self, x):
@@ -30,7 +33,7 @@ class Bottleneck(nn.Module):
         out = self.bn3(self.conv3(out))
         if self.downsample is not None:
             identity = self.downsample(x)
-        return self.relu3(out + identity)
+        return self.relu3(out, identity)
 
 
 class ResNet(nn.Module):

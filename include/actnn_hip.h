@@ -119,6 +119,15 @@ int actnn_relu_forward(const void* x, void* y, int32_t* mask, int64_t n, int dty
  * n a multiple of 2048. */
 int actnn_relu_forward_minmax(const void* x, void* y, int32_t* mask, void* mn, void* mx, int64_t n,
                               int dtype, void* stream);
+/* y = relu(x + residual) in one pass over the two operands, with the same mask: the sum is
+ * rounded to `dtype` as the tensor addition rounds it, so y and mask equal those of the addition
+ * followed by actnn_relu_forward.  For the closing `out += identity; out = relu(out)` of a residual
+ * block of the model the reference benchmarks (torchvision's resnet50,
+ * mem_speed_benchmark/train.py:203-206; the ReLU is quantization.cc:106-124).  mn / mx: both
+ * null, or as in actnn_relu_forward_minmax (16-bit dtypes, n a multiple of 2048).  The gradient of
+ * both operands is actnn_relu_backward's. */
+int actnn_relu_add_forward(const void* x, const void* residual, void* y, int32_t* mask, void* mn,
+                           void* mx, int64_t n, int dtype, void* stream);
 int actnn_relu_backward(const void* grad_out, const int32_t* mask, void* grad_in, int64_t n,
                         int dtype, void* stream);
 

@@ -276,6 +276,56 @@ def test_small_model_trains_at_l3(channels_last):
     assert abs(lq[-1] - le[-1]) < 0.05 and max(abs(a - b) for a, b in zip(le, lq)) < 0.1
 
 
+@pytest.mark.parametrize("channels_last", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_converted_add_relu_is_the_addition_followed_by_relu(channels_last, dtype):
+    """QModule swaps AddReLU for the fused layer: output and both gradients are those of the
+    unfused modules, in either memory layout; a 16-bit output of whole 2048-element tiles carries the
+    group min / max for the convolution that compresses it next."""
+    from actnn_amd import AddReLU, QAddReLU
+    from actnn_amd.layers import known_group_minmax
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.close = AddReLU()
+
+        def forward(self, a, b):
+            return self.close(a, b)
+
+    torch.manual_seed(5)
+    a = torch.randn(8, 32, 8, 8, device=DEV).to(dtype)
+    b = torch.randn(8, 32, 8, 8, device=DEV).to(dtype)
+    b[:, ::2] = -a[:, ::2]
+    if channels_last:
+        a, b = (t.contiguous(memory_format=torch.channels_last) for t in (a, b))
+    g = torch.randn_like(a)
+    plain, fused = Block(), QModule(Block())
+    assert isinstance(fused.model.close, QAddReLU)
+    outs = []
+    for model in (plain, fused):
+        a1, b1 = a.clone().requires_grad_(True), b.clone().requires_grad_(True)
+        out = model(a1, b1)
+        out.backward(g)
+        outs.append((out.detach(), a1.grad, b1.grad, out))
+    for u, v in zip(outs[0][:3], outs[1][:3]):
+        assert torch.equal(u, v)
+    assert outs[1][0].is_contiguous(memory_format=torch.channels_last if channels_last else torch.contiguous_format)
+    known = known_group_minmax(outs[1][3])
+    if dtype == torch.bfloat16:
+        from actnn_amd.utils import memory_order
+        groups = memory_order(outs[1][0]).reshape(-1, 256)
+        assert known is not None
+        assert torch.equal(known[0], groups.min(1).values) and torch.equal(known[1], groups.max(1).values)
+    else:
+        assert known is None
+    # operands that do not share a layout take the unfused path, with the same result
+    if channels_last:
+        a1 = a.contiguous().requires_grad_(True)
+        out = fused(a1, b)
+        assert torch.equal(out, outs[0][0])
+
+
 @pytest.mark.parametrize("autocast", [False, True])
 def test_resnet50_step_runs(autocast):
     torch.manual_seed(0)

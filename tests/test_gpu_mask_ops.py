@@ -96,3 +96,65 @@ def test_relu_forward_with_group_min_max(dtype, n):
     mn_ref, mx_ref = ext_minimax.minimax(y.view(-1, 256))
     assert torch.equal(mn, mn_ref) and torch.equal(mx, mx_ref)
     assert not ext_q.relu_minmax_applies(x[:1024]) and not ext_q.relu_minmax_applies(x.float())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", SHAPES + [(4, 64, 16, 16)])
+def test_relu_of_a_sum_equals_the_addition_followed_by_relu(dtype, shape):
+    """Values, mask words and both gradients of the fused pass are those of torch's addition (which
+    rounds the sum to the tensors' dtype) followed by the ReLU above.  The operands are drawn so that
+    sums cancel exactly, round to zero-adjacent values and differ widely in magnitude."""
+    torch.manual_seed(len(shape) + 7)
+    a = torch.randn(*shape).to(dtype)
+    b = torch.randn(*shape).to(dtype)
+    flat_a, flat_b = a.view(-1), b.view(-1)
+    flat_b[::5] = -flat_a[::5]                              # exact cancellation
+    flat_b[1::7] = flat_b[1::7] * 2.0 ** -12                # one operand far below the other's ulp
+    flat_a[2::11] = flat_a[2::11] * 2.0 ** -14
+    flat_b[2::11] = flat_b[2::11] * 2.0 ** -14              # tiny sums of either sign
+    ad, bd = a.to(DEV).requires_grad_(True), b.to(DEV).requires_grad_(True)
+    y = ext_q.ActQuantizedAddReLU.apply(ad, bd)
+    total = a.to(DEV) + b.to(DEV)
+    assert torch.equal(y, F.relu(total))
+    y2, mask = ext_q.relu_add_forward(a.to(DEV), b.to(DEV))
+    _, ref_mask = ext_q.relu_forward(total)
+    assert torch.equal(y2, y.detach()) and torch.equal(mask, ref_mask)
+    assert np.array_equal(mask.cpu().numpy(), layouts.mask_words((total.view(-1) > 0).cpu().numpy()))
+    g = torch.randn(*shape).to(dtype).to(DEV)
+    y.backward(g)
+    expected = torch.where(total > 0, g, torch.zeros_like(g))
+    assert torch.equal(ad.grad, expected) and torch.equal(bd.grad, expected)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_relu_of_a_sum_with_group_min_max(dtype):
+    torch.manual_seed(3)
+    a = torch.randn(6, 2048 * 3).to(dtype).to(DEV)
+    b = torch.randn(6, 2048 * 3).to(dtype).to(DEV)
+    b[:, ::3] = -a[:, ::3]
+    y, mask, mn, mx = ext_q.relu_add_forward(a, b, minmax=True)
+    ref = F.relu(a + b)
+    y1, mask1, mn1, mx1 = ext_q.relu_forward_minmax(a + b)
+    assert torch.equal(y, ref) and torch.equal(mask, mask1)
+    assert torch.equal(mn, mn1) and torch.equal(mx, mx1)
+    groups = ref.view(-1, 256)
+    assert torch.equal(mn, groups.min(1).values) and torch.equal(mx, groups.max(1).values)
+
+
+def test_relu_of_a_sum_rejects_bad_arguments():
+    from actnn_amd import _lib
+    lib = _lib.load()
+    x = torch.zeros(4096, dtype=torch.bfloat16, device=DEV)
+    y = torch.empty_like(x)
+    mask = torch.empty(ext_q.mask_words(4096), dtype=torch.int32, device=DEV)
+    mn = torch.empty(16, dtype=torch.bfloat16, device=DEV)
+    args = lambda **k: (k.get("x", x.data_ptr()), k.get("r", x.data_ptr()), y.data_ptr(), mask.data_ptr(),
+                        k.get("mn", None), k.get("mx", None), k.get("n", 4096), k.get("dtype", 2), None)
+    assert lib.actnn_relu_add_forward(*args()) == 0
+    assert lib.actnn_relu_add_forward(*args(r=None)) != 0                       # no second operand
+    assert lib.actnn_relu_add_forward(*args(mn=mn.data_ptr())) != 0             # one statistic without the other
+    assert lib.actnn_relu_add_forward(*args(r=x.data_ptr() + 2)) != 0           # misaligned
+    assert lib.actnn_relu_add_forward(*args(mn=mn.data_ptr(), mx=mn.data_ptr(), n=4096 - 512)) != 0
+    assert lib.actnn_relu_add_forward(*args(mn=mn.data_ptr(), mx=mn.data_ptr(), dtype=0)) != 0
+    assert lib.actnn_relu_add_forward(*args(n=0)) == 0
+    torch.cuda.synchronize()
