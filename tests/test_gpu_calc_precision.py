@@ -83,3 +83,30 @@ def test_allocation_in_one_call_equals_the_three_calls(N, G, dtype):
         sens, bits, prefix = ext_cp.allocate_bits_device(mn, mx, N, 0.37, None, initial, target)
         assert int(bits.sum()) == target and int(bits.min()) >= 1 and int(bits.max()) <= initial
         assert torch.equal(prefix[1:], torch.cumsum(bits, 0).to(torch.int32)) and int(prefix[0]) == 0
+
+
+@pytest.mark.parametrize("N", [1, 2, 3, 100, 512, 1170])
+def test_prefix_written_by_the_last_block_from_a_dirty_buffer(N):
+    """The prefix comes from whichever block of the greedy kernel finishes last, counted in
+    prefix[0]: the buffer may hold anything on entry, and every repetition gives the same widths and
+    the prefix of exactly those widths."""
+    from actnn_amd import _lib
+    lib = _lib.load()
+    g = torch.Generator(device=DEV).manual_seed(N)
+    G = 7
+    mn = -torch.rand(N * G, generator=g, device=DEV)
+    mx = torch.rand(N * G, generator=g, device=DEV) * torch.exp(torch.randn(N, 1, generator=g, device=DEV)).expand(N, G).reshape(-1)
+    first = None
+    for rep in range(20):
+        sens = torch.empty(N, device=DEV)
+        bits = torch.full((N,), -7, dtype=torch.int32, device=DEV)
+        prefix = torch.full((N + 1,), 0x7fffffff - rep, dtype=torch.int32, device=DEV)
+        rc = lib.actnn_allocate_bits_device(mn.data_ptr(), mx.data_ptr(), 0.5, None, 0, sens.data_ptr(),
+                                            bits.data_ptr(), prefix.data_ptr(), N, G, 8, 2 * N, 0, None)
+        assert rc == 0
+        assert int(prefix[0]) == 0
+        assert torch.equal(prefix[1:], torch.cumsum(bits, 0).to(torch.int32))
+        assert int(prefix[-1]) == 2 * N
+        if first is None:
+            first = bits.clone()
+        assert torch.equal(bits, first)
