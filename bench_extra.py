@@ -91,38 +91,50 @@ RESNET50_BN_SHAPES = [(64, 112, 1), (64, 56, 6), (256, 56, 4), (128, 56, 1), (12
 def batch_norm_shapes(device, channels_last=True, batch=512, reps=10, keep=()):
     """The three fused batch-norm steps of an L3 training step (statistics + group min/max;
     normalise + 2-bit pack; backward from the packed input with the gradient norm), timed with
-    events on every batch-norm shape of ResNet-50 in bf16: ms and GB/s of algorithmic bytes per
+    events - the calls queued behind other work, so that the device sets the pace - on every
+    batch-norm shape of ResNet-50 in bf16: ms and GB/s of algorithmic bytes per
     shape, and the totals weighted by the number of layers.  `keep`: (C, H) pairs to restrict the run
     to (for counter runs on single shapes)."""
     import actnn_amd.cpp_extension.backward_func as bf
     from actnn_amd.cpp_extension.quantization import attach_bits_total
     from actnn_amd.ops import _Quantized
 
-    worst = []      # slowest repetition over the median, per timed call
+    worst = []      # slowest run over the median run, per timed call
+    # Work that keeps the device busy (about 2 ms) while the timed calls are queued behind it: the
+    # passes of the small planes run 10-40 us, less than a call takes to issue from Python, and timed
+    # one by one on an idle device they would show the caller's pace.  In the training step the host is
+    # ahead of the device (28 ms of host time in a 67 ms step at this batch size) and the passes run
+    # back to back, which is what the queue reproduces.
+    blocker = torch.zeros(256 << 20, dtype=torch.uint8, device=device)
 
-    def timed(fn):
+    def timed(fn, batches=5):
         for _ in range(3):
             fn()
         torch.cuda.synchronize(device)
-        # Every repetition is timed on its own, the median taken and the slowest reported.  The
-        # stalls of tens of milliseconds once seen here were CPython's full garbage collection
-        # (40 ms with torch loaded, timed through gc.callbacks; in a kernel trace a gap between two
-        # dispatches with no HIP call inside), which started wherever the allocation counters said
-        # so: the timed loop collects first and keeps the collector off.
-        marks = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+        # `batches` runs of `reps` calls, each run between two events (an event between every two
+        # calls is a barrier packet of its own, several microseconds on passes that last ten); the
+        # median run counts and the slowest is reported.  The stalls of tens of milliseconds once seen
+        # here were CPython's full garbage collection (40 ms with torch loaded, timed through
+        # gc.callbacks; in a kernel trace a gap between two dispatches with no HIP call inside), which
+        # started wherever the allocation counters said so: the timed loop collects first and keeps
+        # the collector off.
+        marks = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(batches)]
         gc.collect()
         gc.disable()
         try:
-            marks[0].record()
-            for i in range(reps):
-                fn()
-                marks[i + 1].record()
+            for start, stop in marks:
+                for _ in range(24):
+                    blocker.add_(1)
+                start.record()
+                for _ in range(reps):
+                    fn()
+                stop.record()
             torch.cuda.synchronize(device)
         finally:
             gc.enable()
-        each = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(reps))
-        worst.append((each[-1] / each[reps // 2], each[-1]))
-        return each[reps // 2]
+        each = sorted(start.elapsed_time(stop) / reps for start, stop in marks)
+        worst.append((each[-1] / each[batches // 2], each[-1]))
+        return each[batches // 2]
 
     rows, totals = [], [0.0, 0.0, 0.0]
     shapes = [sh for sh in RESNET50_BN_SHAPES if not keep or sh[:2] in keep]
@@ -152,6 +164,6 @@ def batch_norm_shapes(device, channels_last=True, batch=512, reps=10, keep=()):
             "memory_format": "channels_last" if channels_last else "contiguous", "shapes": rows,
             "ms_per_training_step": [round(v, 3) for v in totals],
             # (three timed calls per shape, in the order of `steps`)
-            "slowest_repetition": {"over_median": round(max(worst)[0], 2), "ms": round(max(worst)[1], 3),
+            "slowest_run": {"over_median": round(max(worst)[0], 2), "ms": round(max(worst)[1], 3),
                                    "shape": shapes[worst.index(max(worst)) // 3][:2],
                                    "step": worst.index(max(worst)) % 3}}
