@@ -33,51 +33,8 @@ __global__ __launch_bounds__(kThreads) void fill_kernel(int32_t* __restrict__ ou
   if (i < n) out[i] = value;
 }
 
-// The exclusive prefix of the widths by the block of the launch that finishes last.  Every block
-// calls it (all threads) after its last write to `bits`: the block makes its widths visible to the
-// device, takes a ticket from the counter in prefix[0] (zero when the launch starts), and the holder
-// of the last ticket - every other block's widths are visible to it by then - scans all N widths and
-// leaves prefix[0] = 0, which is both its value and the counter's state for the next launch.
-// Nobody waits for anybody: a block that is not the last leaves at once.
-ACTNN_DEV void prefix_by_last_block(const int32_t* bits, int32_t* prefix, int N) {
-  __shared__ int s_last;
-  __shared__ int32_t s_scan[kThreads];
-  __syncthreads();                                     // the block's widths are written
-  if (threadIdx.x == 0) {
-    __threadfence();
-    const unsigned ticket = atomicAdd(reinterpret_cast<unsigned*>(prefix), 1u);
-    s_last = ticket == gridDim.x - 1 ? 1 : 0;
-  }
-  __syncthreads();
-  if (!s_last) return;
-  __threadfence();
-  // thread t owns the contiguous chunk [t * per, (t + 1) * per); the loads go to the device's
-  // coherent level, not to a line this CU may hold from before the other blocks wrote
-  const int per = (N + kThreads - 1) / kThreads;
-  const int lo = (int)threadIdx.x * per;
-  const int hi = lo + per < N ? lo + per : N;
-  int32_t sum = 0;
-  for (int i = lo; i < hi; ++i) sum += __hip_atomic_load(bits + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  s_scan[threadIdx.x] = sum;
-  __syncthreads();
-  for (int off = 1; off < kThreads; off <<= 1) {       // inclusive Hillis-Steele scan
-    const int32_t add = (int)threadIdx.x >= off ? s_scan[threadIdx.x - off] : 0;
-    __syncthreads();
-    s_scan[threadIdx.x] += add;
-    __syncthreads();
-  }
-  int32_t run = threadIdx.x == 0 ? 0 : s_scan[threadIdx.x - 1];
-  for (int i = lo; i < hi; ++i) {
-    run += __hip_atomic_load(bits + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    prefix[i + 1] = run;
-  }
-  if (threadIdx.x == 0) prefix[0] = 0;
-}
-
-template <bool PREFIX>
 __global__ __launch_bounds__(kThreads) void calc_precision_device_kernel(
-    const float* __restrict__ C, int32_t* __restrict__ bits, int32_t* __restrict__ prefix, int N, int initial,
-    int64_t K) {
+    const float* __restrict__ C, int32_t* __restrict__ bits, int N, int initial, int64_t K) {
   constexpr int kWaves = kThreads / 64;
   __shared__ double factors[8];
   __shared__ float C_s[kMaxCand];                      // N <= kMaxCand / L
@@ -92,7 +49,6 @@ __global__ __launch_bounds__(kThreads) void calc_precision_device_kernel(
   if (K <= 0 || K >= total) {                          // nothing to take, or everything
     if ((int)threadIdx.x < items_per_block && item0 + (int)threadIdx.x < N)
       bits[item0 + threadIdx.x] = K <= 0 ? initial : 1;
-    if (PREFIX) prefix_by_last_block(bits, prefix, N);
     return;
   }
   for (int n = threadIdx.x; n < N; n += kThreads) C_s[n] = C[n];      // one trip to memory for all keys
@@ -155,53 +111,28 @@ __global__ __launch_bounds__(kThreads) void calc_precision_device_kernel(
     for (int k = 0; k < L; ++k) t += taken[threadIdx.x * L + k];
     bits[item0 + threadIdx.x] = initial - t;
   }
-  if (PREFIX) prefix_by_last_block(bits, prefix, N);
 }
 
 }  // namespace
 }  // namespace actnn
 
-namespace actnn {
-namespace {
-// prefix: null, or where the launch also leaves the exclusive prefix of the widths (prefix[0] zero
-// on entry); -> ACTNN_OK, an error, or kNoPrefix when the widths are written but the prefix is not
-constexpr int kNoPrefix = -1000;
-int launch_calc_precision(const float* C, int32_t* bits, int32_t* prefix, int64_t N, int initial_bits,
-                          int64_t target, hipStream_t s) {
+extern "C" int actnn_calc_precision_device(const float* C, int32_t* bits, int64_t N, int initial_bits,
+                                           int64_t target, void* stream) {
+  using namespace actnn;
   if (N < 0) return ACTNN_EINVAL;
-  if (N == 0) return prefix ? kNoPrefix : ACTNN_OK;
+  if (N == 0) return ACTNN_OK;
   if (!C || !bits) return ACTNN_EINVAL;
   if (initial_bits < 1 || initial_bits > 8) return ACTNN_EBITS;
   const int64_t total = N * (initial_bits - 1);
   if (total > kMaxCand) return ACTNN_EINVAL;           // larger batches take the host routine
   const int64_t K = N * initial_bits - target;         // widths to take away
+  hipStream_t s = static_cast<hipStream_t>(stream);
   if (initial_bits == 1) {                             // no steps to take: every item keeps its one bit
     fill_kernel<<<dim3((unsigned)((N + kThreads - 1) / kThreads)), dim3(kThreads), 0, s>>>(bits, (int)N, 1);
-    const hipError_t e = hipGetLastError();
-    return e != hipSuccess ? (int)e : prefix ? kNoPrefix : ACTNN_OK;
+    ACTNN_RETURN_LAUNCH_STATUS();
   }
   const int items_per_block = kSlots / (initial_bits - 1);
   const int64_t blocks = (N + items_per_block - 1) / items_per_block;
-  if (prefix)
-    calc_precision_device_kernel<true><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(C, bits, prefix, (int)N,
-                                                                                         initial_bits, K);
-  else
-    calc_precision_device_kernel<false><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(C, bits, nullptr, (int)N,
-                                                                                          initial_bits, K);
+  calc_precision_device_kernel<<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(C, bits, (int)N, initial_bits, K);
   ACTNN_RETURN_LAUNCH_STATUS();
-}
-}  // namespace
-
-int allocate_widths_launch(const float* C, int32_t* bits, int32_t* prefix, int64_t N, int initial_bits,
-                           int64_t target, hipStream_t s) {
-  if (!prefix) return ACTNN_EINVAL;
-  const int rc = launch_calc_precision(C, bits, prefix, N, initial_bits, target, s);
-  if (rc != kNoPrefix) return rc;
-  return actnn_bits_prefix(bits, prefix, N, s);        // the cases without the greedy kernel
-}
-}  // namespace actnn
-
-extern "C" int actnn_calc_precision_device(const float* C, int32_t* bits, int64_t N, int initial_bits,
-                                           int64_t target, void* stream) {
-  return actnn::launch_calc_precision(C, bits, nullptr, N, initial_bits, target, static_cast<hipStream_t>(stream));
 }

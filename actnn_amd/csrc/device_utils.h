@@ -498,15 +498,6 @@ template <typename T> struct Noise {
 };
 
 // ------------------------------------------------------------------ host-side helpers
-// Launchers one translation unit offers to another (the exported entry points are thin wrappers).
-// range_sqr_launch: actnn_range_sqr that also clears one word for the kernel after it.
-// allocate_widths_launch: greedy widths and their exclusive prefix in one launch; prefix[0] must be
-// zero when the kernel starts (it serves as the launch's arrival counter and ends as zero).
-int range_sqr_launch(const void* mn, const void* mx, float* out, int64_t N, int64_t G, float factor,
-                     const float* mult, int mult_per_sample, int dtype, int32_t* clear, hipStream_t s);
-int allocate_widths_launch(const float* C, int32_t* bits, int32_t* prefix, int64_t N, int initial_bits,
-                           int64_t target, hipStream_t s);
-
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 #define ACTNN_RETURN_LAUNCH_STATUS()                       \

@@ -166,11 +166,9 @@ __global__ __launch_bounds__(kThreads) void range_sqr_kernel(const T* __restrict
                                                              const T* __restrict__ mx,
                                                              float* __restrict__ out, int64_t G,
                                                              float factor, const float* __restrict__ mult,
-                                                             int mult_stride, int32_t* __restrict__ clear) {
+                                                             int mult_stride) {
   __shared__ float s_part[kThreads];
   const int64_t n = blockIdx.x;
-  // a counter of the kernel that follows in the stream starts at zero (nobody reads it before then)
-  if (clear && blockIdx.x == 0 && threadIdx.x == 0) *clear = 0;
   float acc = 0.0f;
   for (int64_t g = threadIdx.x; g < G; g += kThreads) {
     const float d = Conv<T>::round(Conv<T>::load(mx, n * G + g) - Conv<T>::load(mn, n * G + g));
@@ -250,29 +248,25 @@ __global__ __launch_bounds__(kThreads) void sample_sqnorm_kernel(const T* __rest
 extern "C" int actnn_range_sqr(const void* mn, const void* mx, float* out, int64_t N, int64_t G,
                                float factor, const float* mult, int mult_per_sample, int dtype,
                                void* stream) {
-  return actnn::range_sqr_launch(mn, mx, out, N, G, factor, mult, mult_per_sample, dtype, nullptr,
-                                 static_cast<hipStream_t>(stream));
-}
-
-int actnn::range_sqr_launch(const void* mn, const void* mx, float* out, int64_t N, int64_t G, float factor,
-                            const float* mult, int mult_per_sample, int dtype, int32_t* clear, hipStream_t s) {
+  using namespace actnn;
   if (N < 0 || G < 0 || N > 0x7fffffffLL) return ACTNN_EINVAL;
   if (N == 0) return ACTNN_OK;
   if (!out || (G > 0 && (!mn || !mx))) return ACTNN_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)N), blk(kThreads);
   const int stride = mult_per_sample ? 1 : 0;
   switch (dtype) {
     case ACTNN_F32:
       range_sqr_kernel<float><<<grid, blk, 0, s>>>(static_cast<const float*>(mn), static_cast<const float*>(mx),
-                                                   out, G, factor, mult, stride, clear);
+                                                   out, G, factor, mult, stride);
       break;
     case ACTNN_F16:
       range_sqr_kernel<__half><<<grid, blk, 0, s>>>(static_cast<const __half*>(mn), static_cast<const __half*>(mx),
-                                                    out, G, factor, mult, stride, clear);
+                                                    out, G, factor, mult, stride);
       break;
     case ACTNN_BF16:
       range_sqr_kernel<bf16_t><<<grid, blk, 0, s>>>(static_cast<const bf16_t*>(mn), static_cast<const bf16_t*>(mx),
-                                                    out, G, factor, mult, stride, clear);
+                                                    out, G, factor, mult, stride);
       break;
     default: return ACTNN_EDTYPE;
   }

@@ -86,7 +86,7 @@ extern "C" int actnn_stream_copy(const void* src, void* dst, int64_t bytes, void
 }
 
 // The three allocation steps of a layer in one call (one crossing of the language boundary instead
-// of three) and two launches: sensitivities, greedy widths on the device, exclusive prefix of the widths.
+// of three): sensitivities, greedy widths on the device, exclusive prefix of the widths.
 extern "C" int actnn_range_sqr(const void* mn, const void* mx, float* out, int64_t N, int64_t G, float factor,
                                const float* mult, int mult_per_sample, int dtype, void* stream);
 extern "C" int actnn_calc_precision_device(const float* C, int32_t* bits, int64_t N, int initial_bits,
@@ -97,13 +97,11 @@ extern "C" int actnn_allocate_bits_device(const void* mn, const void* mx, float 
                                           int mult_per_sample, float* sensitivity, int32_t* bits,
                                           int32_t* prefix, int64_t N, int64_t G, int initial_bits,
                                           int64_t target, int dtype, void* stream) {
-  // two launches: the sensitivities (whose kernel also zeroes prefix[0], the arrival counter of the
-  // next one), then the greedy widths, whose last block to finish writes their prefix
-  if (N > 0 && !prefix) return ACTNN_EINVAL;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const int rc = actnn::range_sqr_launch(mn, mx, sensitivity, N, G, factor, mult, mult_per_sample, dtype, prefix, s);
+  int rc = actnn_range_sqr(mn, mx, sensitivity, N, G, factor, mult, mult_per_sample, dtype, stream);
   if (rc != ACTNN_OK) return rc;
-  return actnn::allocate_widths_launch(sensitivity, bits, prefix, N, initial_bits, target, s);
+  rc = actnn_calc_precision_device(sensitivity, bits, N, initial_bits, target, stream);
+  if (rc != ACTNN_OK) return rc;
+  return actnn_bits_prefix(bits, prefix, N, stream);
 }
 
 extern "C" const char* actnn_strerror(int code) {

@@ -219,11 +219,9 @@ int actnn_sample_sqnorm(const void* x, float* part, int64_t N, int64_t F, int sl
 int actnn_calc_precision_device(const float* C, int32_t* bits, int64_t N, int initial_bits,
                                 int64_t target, void* stream);
 
-/* What actnn_range_sqr, actnn_calc_precision_device and actnn_bits_prefix leave when called back
- * to back on `stream`, for the per-layer allocation of qscheme.py:76-94 in one call and two
- * launches: sensitivity[N] (fp32), bits[N], prefix[N + 1].  Arguments and limits as for the three
- * calls.  While the call's kernels run, prefix[0] is their scratch (a counter of finished blocks);
- * it holds its value, 0, when they are done. */
+/* actnn_range_sqr, actnn_calc_precision_device and actnn_bits_prefix back to back on `stream`, for
+ * the per-layer allocation of qscheme.py:76-94 in one call: sensitivity[N] (fp32), bits[N],
+ * prefix[N + 1].  Arguments and limits as for the three calls. */
 int actnn_allocate_bits_device(const void* mn, const void* mx, float factor, const float* mult,
                                int mult_per_sample, float* sensitivity, int32_t* bits,
                                int32_t* prefix, int64_t N, int64_t G, int initial_bits,

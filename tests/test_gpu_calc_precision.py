@@ -86,9 +86,8 @@ def test_allocation_in_one_call_equals_the_three_calls(N, G, dtype):
 
 
 @pytest.mark.parametrize("N", [1, 2, 3, 100, 512, 1170])
-def test_prefix_written_by_the_last_block_from_a_dirty_buffer(N):
-    """The prefix comes from whichever block of the greedy kernel finishes last, counted in
-    prefix[0]: the buffer may hold anything on entry, and every repetition gives the same widths and
+def test_allocation_in_one_call_from_dirty_buffers(N):
+    """The output buffers may hold anything on entry, and every repetition gives the same widths and
     the prefix of exactly those widths."""
     from actnn_amd import _lib
     lib = _lib.load()
