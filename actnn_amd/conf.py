@@ -32,6 +32,9 @@ class QuantizationConfig:
         self.share_relu_min_max = True                 # ReLU leaves its output's group min/max for the next layer
         self.share_grad_sqnorm = True                  # batch-norm backward leaves sum(dx^2) for the conv's set_scale
         self.fused_bn_pack = True                      # batch-norm forward writes the packed copy of its input
+        # a layer's forward-side sequence (min/max or statistics -> widths -> pack) behind one library
+        # call where the widths are made on the device: same kernels, less host time per layer
+        self.fused_quantize = True
         # QLinear's weight gradient straight from the packed input (the dequantised input is never
         # written): True - where the fused kernel is the faster path, i.e. for the 2-bit fixed-width
         # stream; "always" - for every stream it takes (saves the full-precision copy at 0.7-0.9 ms

@@ -174,6 +174,73 @@ def hip_batch_norm_forward_apply(input, workspace, bits=None, mn=None, mx=None):
     return out, packed, scale
 
 
+def hip_batch_norm_quantize_geometry(input, weight, bias, running_mean, running_var):
+    """(N, C, HW, channels_last) when statistics, group min/max and the packed copy can all come from
+    the fused passes (what hip_batch_norm_minmax_applies and hip_batch_norm_pack_applies ask, looked
+    up once), else None."""
+    geo = _bn_geometry(input)
+    if geo is None or input.data_ptr() % 16 != 0:
+        return None
+    if not (_f32_or_none(weight) and _f32_or_none(bias) and _f32_or_none(running_mean) and _f32_or_none(running_var)):
+        return None
+    N, C, HW, channels_last = geo
+    if not _groups_align(N, C, HW, _glue.DTYPE_CODE[input.dtype], channels_last):
+        return None
+    if channels_last and N * HW >= 2 ** 31:
+        return None
+    return geo
+
+
+def hip_batch_norm_forward_quantize(input, geo, weight, bias, running_mean, running_var, momentum, eps, alloc):
+    """Statistics + group min/max -> widths on the device -> normalise + pack, in one call:
+    -> (output, save_mean, save_invstd, mn, mx, bits, packed, scale), what
+    hip_batch_norm_forward_stats, allocate_bits_device and hip_batch_norm_forward_apply return one
+    after the other.  `geo` from hip_batch_norm_quantize_geometry, `alloc` the scheme's
+    AllocationArgs (factor, mult, initial, target, total, sens_out)."""
+    from .quantization import attach_bits_total
+    N, C, HW, channels_last = geo
+    dev, dtype = input.device, input.dtype
+    code = _glue.DTYPE_CODE[dtype]
+    ws_bytes = _workspace_bytes(N, C, HW, code, int(channels_last))
+    G = C * HW // 256
+    f32, i32 = torch.float32, torch.int32
+    ws = torch.empty(ws_bytes // 4, dtype=f32, device=dev)
+    save_mean = torch.empty(C, dtype=f32, device=dev)
+    save_invstd = torch.empty(C, dtype=f32, device=dev)
+    mn = torch.empty(N * G, dtype=dtype, device=dev)
+    mx = torch.empty(N * G, dtype=dtype, device=dev)
+    out = torch.empty_like(input)
+    sens = alloc.sens_out if alloc.sens_out is not None else torch.empty(N, dtype=f32, device=dev)
+    bits = torch.empty(N, dtype=i32, device=dev)
+    prefix = torch.empty(N + 1, dtype=i32, device=dev)
+    packed = torch.empty(alloc.total * G * 8, dtype=i32, device=dev)
+    scale = torch.empty(N, G, 1, dtype=dtype, device=dev)
+    mult, mult_ptr, per_sample = _mult_args(alloc.mult, N, dev)          # (`mult` held until the launch)
+    seed, offset = _glue.philox_args(dev)
+    with _glue.on_device(dev):
+        _glue._lib.check(_glue.lib().actnn_batch_norm_forward_quantize(
+            input.data_ptr(), _ptr(weight), _ptr(bias), _ptr(running_mean), _ptr(running_var), out.data_ptr(),
+            save_mean.data_ptr(), save_invstd.data_ptr(), mn.data_ptr(), mx.data_ptr(), ws.data_ptr(), ws_bytes,
+            alloc.factor, mult_ptr, per_sample, sens.data_ptr(), bits.data_ptr(), prefix.data_ptr(),
+            alloc.initial, alloc.target, scale.data_ptr(), packed.data_ptr(), seed, offset, N, C, HW,
+            float(momentum), float(eps), code, int(channels_last), _glue.stream_ptr(dev)),
+            "batch_norm_forward_quantize")
+    attach_bits_total(bits, alloc.total, prefix)
+    return out, save_mean, save_invstd, mn, mx, bits, packed, scale
+
+
+def _mult_args(mult, N, dev):
+    """(tensor, pointer, per-sample flag) of the sensitivity's multiplier: nothing, one device scalar
+    or one value per sample (fp32 on `dev`), as allocate_bits_device takes it."""
+    if mult is None:
+        return None, None, 0
+    if mult.dtype != torch.float32 or mult.device != dev or mult.numel() not in (1, N):
+        raise RuntimeError("the sensitivity's multiplier must be fp32 on the same device with 1 or N values")
+    if not mult.is_contiguous():
+        mult = mult.contiguous()
+    return mult, mult.data_ptr(), int(mult.numel() == N and N != 1)
+
+
 def hip_batch_norm_pack_applies(input, weight, bias, running_mean, running_var):
     """True when the forward pass can also write the packed copy of its input."""
     if input.dtype not in (torch.float16, torch.bfloat16, torch.float32):

@@ -103,6 +103,38 @@ def pack_mixed_precision(data, min, max, bits, stochastic, *, noise=None):
     return packed, scale
 
 
+def quantize_activation_device(rows, N, known_minmax, alloc):
+    """[min/max of every group] -> widths on the device -> pack, in one call: what minimax,
+    allocate_bits_device and pack_mixed_precision do one after the other for `rows` (contiguous
+    [N * G, 256] view of the activation).  `known_minmax`: (mn, mx) [N * G] in the rows' dtype when
+    another kernel has produced them, else None.  `alloc`: the scheme's AllocationArgs.
+    -> (packed, bits with sum and prefix attached, scale [N, G, 1], mn [N * G])."""
+    from .backward_func import _mult_args
+    dev, dtype = rows.device, rows.dtype
+    G = rows.shape[0] // N
+    rows = g.aligned(rows)
+    if known_minmax is None:
+        mn = torch.empty(N * G, dtype=dtype, device=dev)
+        mx = torch.empty(N * G, dtype=dtype, device=dev)
+    else:
+        mn, mx = known_minmax
+    sens = alloc.sens_out if alloc.sens_out is not None else torch.empty(N, dtype=torch.float32, device=dev)
+    bits = torch.empty(N, dtype=torch.int32, device=dev)
+    prefix = torch.empty(N + 1, dtype=torch.int32, device=dev)
+    packed = torch.empty(alloc.total * G * 8, dtype=torch.int32, device=dev)
+    scale = torch.empty(N, G, 1, dtype=dtype, device=dev)
+    mult, mult_ptr, per_sample = _mult_args(alloc.mult, N, dev)           # (`mult` held until the launch)
+    seed, offset = g.philox_args(dev)
+    with g.on_device(dev):
+        check(g.lib().actnn_quantize_activation(
+            rows.data_ptr(), mn.data_ptr(), mx.data_ptr(), int(known_minmax is not None), alloc.factor, mult_ptr,
+            per_sample, sens.data_ptr(), bits.data_ptr(), prefix.data_ptr(), alloc.initial, alloc.target,
+            scale.data_ptr(), packed.data_ptr(), seed, offset, N, G, g.DTYPE_CODE[dtype], g.stream_ptr(dev)),
+            "quantize_activation")
+    attach_bits_total(bits, alloc.total, prefix)
+    return packed, bits, scale, mn
+
+
 def unpack_mixed_precision(data, bits, scale, min, N, num_groups, group_size):
     g.check_typed(data, "data", torch.int32, 1)
     g.check_typed(bits, "bits", torch.int32, 1)

@@ -104,6 +104,65 @@ extern "C" int actnn_allocate_bits_device(const void* mn, const void* mx, float 
   return actnn_bits_prefix(bits, prefix, N, stream);
 }
 
+// One crossing of the language boundary for a layer's whole forward-side sequence: the calls below
+// on one stream, arguments as theirs.  Nothing is launched unless the arguments of the first step
+// pass; a later step that refuses its arguments leaves the earlier ones launched (their outputs are
+// then simply unused).
+extern "C" int actnn_batch_norm_forward_stats(const void* x, const float* weight, const float* bias,
+                                              float* running_mean, float* running_var, float* save_mean,
+                                              float* save_invstd, void* mn, void* mx, void* workspace,
+                                              int64_t workspace_bytes, int64_t N, int64_t C, int64_t HW,
+                                              double momentum, double eps, int dtype, int channels_last,
+                                              void* stream);
+extern "C" int actnn_batch_norm_forward_apply(const void* x, void* y, const void* workspace,
+                                              int64_t workspace_bytes, const int32_t* bits,
+                                              const int32_t* prefix, const void* mn, const void* mx, void* scale,
+                                              int32_t* packed, uint64_t seed, uint64_t offset, int64_t N,
+                                              int64_t C, int64_t HW, int dtype, int channels_last, void* stream);
+extern "C" int actnn_minimax(const void* data, void* mn, void* mx, int64_t M, int64_t D, int dtype, void* stream);
+extern "C" int actnn_pack_mixed(const void* data, const void* mn, const void* mx, const int32_t* bits,
+                                const int32_t* prefix, void* scale, int32_t* packed, const void* noise,
+                                uint64_t seed, uint64_t offset, int64_t N, int64_t G, int64_t gs, int dtype,
+                                void* stream);
+
+extern "C" int actnn_batch_norm_forward_quantize(
+    const void* x, const float* weight, const float* bias, float* running_mean, float* running_var, void* y,
+    float* save_mean, float* save_invstd, void* mn, void* mx, void* workspace, int64_t workspace_bytes,
+    float factor, const float* mult, int mult_per_sample, float* sensitivity, int32_t* bits, int32_t* prefix,
+    int initial_bits, int64_t target, void* scale, int32_t* packed, uint64_t seed, uint64_t offset, int64_t N,
+    int64_t C, int64_t HW, double momentum, double eps, int dtype, int channels_last, void* stream) {
+  if (!mn || !mx || !bits || !prefix || !scale || !packed || !sensitivity || !y) return ACTNN_EINVAL;
+  if (N <= 0 || C <= 0 || HW <= 0 || (C * HW) % 256 != 0) return ACTNN_EINVAL;
+  int rc = actnn_batch_norm_forward_stats(x, weight, bias, running_mean, running_var, save_mean, save_invstd, mn,
+                                          mx, workspace, workspace_bytes, N, C, HW, momentum, eps, dtype,
+                                          channels_last, stream);
+  if (rc != ACTNN_OK) return rc;
+  rc = actnn_allocate_bits_device(mn, mx, factor, mult, mult_per_sample, sensitivity, bits, prefix, N,
+                                  C * HW / 256, initial_bits, target, dtype, stream);
+  if (rc != ACTNN_OK) return rc;
+  return actnn_batch_norm_forward_apply(x, y, workspace, workspace_bytes, bits, prefix, mn, mx, scale, packed,
+                                        seed, offset, N, C, HW, dtype, channels_last, stream);
+}
+
+extern "C" int actnn_quantize_activation(const void* data, void* mn, void* mx, int minmax_known, float factor,
+                                         const float* mult, int mult_per_sample, float* sensitivity,
+                                         int32_t* bits, int32_t* prefix, int initial_bits, int64_t target,
+                                         void* scale, int32_t* packed, uint64_t seed, uint64_t offset, int64_t N,
+                                         int64_t G, int dtype, void* stream) {
+  if (!data || !mn || !mx || !bits || !prefix || !scale || !packed || !sensitivity) return ACTNN_EINVAL;
+  if (N <= 0 || G <= 0) return ACTNN_EINVAL;
+  int rc = ACTNN_OK;
+  if (!minmax_known) {
+    rc = actnn_minimax(data, mn, mx, N * G, 256, dtype, stream);
+    if (rc != ACTNN_OK) return rc;
+  }
+  rc = actnn_allocate_bits_device(mn, mx, factor, mult, mult_per_sample, sensitivity, bits, prefix, N, G,
+                                  initial_bits, target, dtype, stream);
+  if (rc != ACTNN_OK) return rc;
+  return actnn_pack_mixed(data, mn, mx, bits, prefix, scale, packed, nullptr, seed, offset, N, G, 256, dtype,
+                          stream);
+}
+
 extern "C" const char* actnn_strerror(int code) {
   switch (code) {
     case ACTNN_OK: return "success";

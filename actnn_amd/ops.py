@@ -141,6 +141,40 @@ def quantize_saved(input, scheme):
     return finish_saved(start_quantize(input, scheme), input)
 
 
+def quantize_on_device(input, scheme, known_minmax=None):
+    """start_quantize + finish_saved behind one library call, for the case the layers meet at every
+    step: a scheme whose widths are made on the device, whole groups of 256, per-group ranges,
+    in-kernel stochastic rounding, nothing swapped.  -> the saved tuple, or None when the case is
+    another one (the caller then takes the two halves; nothing has been launched).  Same kernels on
+    the same generator state: the result is the two halves' bit for bit."""
+    if not (scheme and config.fused_quantize and config.compress_activation and config.pergroup
+            and config.stochastic and not config.simulate and not config.swap and config.group_size == 256):
+        return None
+    if not (input.is_cuda and input.dtype in ext_quantization.g.DTYPE_CODE and input.dim() >= 2):
+        return None
+    N = input.shape[0]
+    fmt = channels_last_format(input)
+    flat = (input.permute(0, *range(2, input.dim()), 1) if fmt is not None else input).reshape(N, -1)
+    features = flat.shape[1]
+    if N == 0 or features == 0 or features % 256 != 0 or not flat.is_contiguous():
+        return None
+    if known_minmax is not None:
+        mn, mx = known_minmax
+        if not (mn.dtype == input.dtype and mx.dtype == input.dtype and mn.numel() * 256 == input.numel()
+                and mx.numel() == mn.numel() and mn.is_contiguous() and mx.is_contiguous()):
+            known_minmax = None
+    alloc = scheme.allocation_arguments(N, features // input.shape[1], input.device)
+    if alloc is None:
+        return None
+    q_input, q_bits, q_scale, mn = ext_quantization.quantize_activation_device(
+        flat.view(-1, 256), N, known_minmax, alloc)
+    scheme.adopt_device_bits(q_bits, features, alloc)
+    q_min = mn.view(N, -1, 1)
+    if input.dtype == torch.float32:
+        q_scale, q_min = q_scale.to(torch.bfloat16), q_min.to(torch.bfloat16)
+    return _mark_saved(_Quantized((q_input, q_bits, q_scale, q_min)), input)
+
+
 def _mark_saved(q, input):
     q.native_bf16 = input.dtype == torch.bfloat16
     q.memory_format = channels_last_format(input)
@@ -166,9 +200,13 @@ def _conv_forward(ctx, forward_op, input, weight, bias, stride, padding, dilatio
     if known_minmax is not None and (known_minmax[0].dtype != input.dtype
                                      or known_minmax[0].numel() * config.group_size != input.numel()):
         known_minmax = None                  # e.g. the input was cast on its way here
-    started = start_quantize(input, scheme, known_minmax)
-    output = forward_op(input, weight, bias, stride, padding, dilation, groups)
-    quantized = finish_saved(started, input)
+    quantized = quantize_on_device(input, scheme, known_minmax)
+    if quantized is not None:
+        output = forward_op(input, weight, bias, stride, padding, dilation, groups)
+    else:
+        started = start_quantize(input, scheme, known_minmax)
+        output = forward_op(input, weight, bias, stride, padding, dilation, groups)
+        quantized = finish_saved(started, input)
     ctx.scheme = scheme
     ctx.saved = quantized, weight, bias
     ctx.other_args = (input.shape, stride, padding, dilation, groups)
@@ -196,7 +234,7 @@ def _conv_backward(ctx, grad_output, bias_reduce_dims, aug):
     grad_output = grad_output.contiguous(memory_format=memory_format)
     need = [ctx.needs_input_grad[0], ctx.needs_input_grad[1]]
 
-    ws_mem = compute_tensor_bytes([grad_output, input, input])
+    ws_mem = compute_tensor_bytes([grad_output, input, input]) if config.pipeline_threshold else 0
     if config.pipeline_threshold and ws_mem > config.pipeline_threshold and all(need):
         # micro-batched backward: grad_input overwrites the dequantised input chunk by chunk so
         # the transient working set stays bounded (ops.py:202-220)
@@ -427,7 +465,27 @@ class batch_norm(Function):
                        and 1 <= config.activation_compression_bits[0] <= 8)
         # (the pass rounds stochastically, like pack_*; with config.stochastic off the unfused
         # sequence below is taken and pack_* refuses, as in the reference)
-        if ((scheme or fixed_width) and config.fused_bn_pack and config.stochastic
+        fused = None
+        if (scheme and config.fused_quantize and config.fused_bn_pack and config.stochastic and training
+                and config.compress_activation and config.pergroup and not config.simulate and not config.swap
+                and config.group_size == 256):
+            # statistics -> widths -> normalise + pack behind one library call (the branch below, for
+            # a scheme whose widths are made on the device; same kernels, same generator state)
+            geo = ext_backward_func.hip_batch_norm_quantize_geometry(input, weight, bias, running_mean, running_var)
+            alloc = scheme.allocation_arguments(geo[0], geo[2], input.device) if geo is not None else None
+            if alloc is not None:
+                fused = ext_backward_func.hip_batch_norm_forward_quantize(
+                    input, geo, weight, bias, running_mean, running_var, exponential_average_factor, eps, alloc)
+        if fused is not None:
+            output, save_mean, save_var, mn, mx, q_bits, q_input, q_scale = fused
+            N = geo[0]
+            scheme.adopt_device_bits(q_bits, input.numel() // N, alloc)
+            q_min = mn.view(N, -1, 1)
+            if input.dtype == torch.float32:
+                q_scale, q_min = q_scale.to(torch.bfloat16), q_min.to(torch.bfloat16)
+            reserve = None
+            started = ("done", _mark_saved(_Quantized((q_input, q_bits, q_scale, q_min)), input))
+        elif ((scheme or fixed_width) and config.fused_bn_pack and config.stochastic
                 and _bn_shares_min_max(input, weight, bias, running_mean, running_var, training)
                 and ext_backward_func.hip_batch_norm_pack_applies(input, weight, bias, running_mean, running_var)):
             # two reads of the input in total: the statistics pass also yields the quantiser's

@@ -1,8 +1,8 @@
 """Bit allocation for batch-norm inputs (behaviour of actnn/actnn/qbnscheme.py:9-60): the
 sensitivity is the range term alone and the per-layer budget follows the preceding conv/linear."""
 from .conf import config
-from .qscheme import (PendingBits, QScheme, allocate_bits_on_device, allocate_on_device, greedy_bits,
-                      group_min_max, range_sqr)
+from .qscheme import (AllocationArgs, PendingBits, QScheme, allocate_bits_on_device, allocate_on_device,
+                      greedy_bits, group_min_max, range_sqr)
 
 
 class QBNScheme(QScheme):
@@ -23,6 +23,15 @@ class QBNScheme(QScheme):
             return groups, mn, mx, None, input.numel() // N, bits_dev
         C_dev = range_sqr(mn, mx, N, num_pixels)                           # qbnscheme.py:44-47
         return groups, mn, mx, PendingBits(C_dev), input.numel() // N, None
+
+    def allocation_arguments(self, N, num_pixels, device):
+        self.prev_linear = QScheme.prev_layer
+        if not allocate_on_device(N, self.initial_bits):
+            return None
+        return AllocationArgs(N, config.group_size / num_pixels, None, self.initial_bits, self.bits)
+
+    def adopt_device_bits(self, bits_dev, dim, args):
+        pass
 
     def finish_quantization_bits(self, started):
         groups, mn, mx, pending, _, bits_dev = started

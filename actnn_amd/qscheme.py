@@ -138,16 +138,33 @@ def greedy_bits_device(C_dev, N, initial_bits, avg_bits):
 def allocate_bits_on_device(mn, mx, N, num_pixels, factor, mult, initial_bits, avg_bits, sens_out=None):
     """Sensitivities, widths and the prefix of the widths in one call -> (C on the device, bits
     with their sum and prefix attached).  `sens_out`: fp32 [N] on the device to write C into."""
-    initial = int(initial_bits)
-    target = int(avg_bits * N)
+    args = AllocationArgs(N, factor * config.group_size / num_pixels, mult, initial_bits, avg_bits, sens_out)
     C_dev, bits, prefix = ext_calc_precision.allocate_bits_device(
-        mn, mx, N, factor * config.group_size / num_pixels, mult, initial, target, sens_out)
-    taken = min(max(N * initial - target, 0), N * (initial - 1))
-    return C_dev, attach_bits_total(bits, N * initial - taken, prefix)
+        mn, mx, N, args.factor, mult, args.initial, args.target, sens_out)
+    return C_dev, attach_bits_total(bits, args.total, prefix)
 
 
 def allocate_on_device(N, initial_bits):
     return config.device_allocation and ext_calc_precision.device_allocation_fits(N, initial_bits)
+
+
+class AllocationArgs:
+    """What the allocation kernels need for one layer's input (allocate_bits_on_device's arguments,
+    resolved): `factor` and `mult` of the sensitivity, start width and target sum of the widths,
+    the sum the widths will have (fixed by the budget, so the stream can be sized without a look
+    at them), where the sensitivities go (a row of the step's pool, or None) and what the scheme
+    keeps to read them back."""
+    __slots__ = ("factor", "mult", "initial", "target", "total", "sens_out", "pending")
+
+    def __init__(self, N, factor, mult, initial_bits, avg_bits, sens_out=None, pending=None):
+        self.factor = float(factor)
+        self.mult = mult
+        self.initial = int(initial_bits)
+        self.target = int(avg_bits * N)
+        taken = min(max(N * self.initial - self.target, 0), N * (self.initial - 1))
+        self.total = N * self.initial - taken
+        self.sens_out = sens_out
+        self.pending = pending
 
 
 class _LazyHost:
@@ -275,6 +292,24 @@ class QScheme(_LazyHost):
     def compute_quantization_bits(self, input):
         """-> (groups [N,G,gs], bits on device, mn [N,G,1], mx [N,G,1])  (qscheme.py:57-94)."""
         return self.finish_quantization_bits(self.start_quantization_bits(input))
+
+    def allocation_arguments(self, N, num_pixels, device):
+        """The layer's AllocationArgs when its widths are made on the device, else None; with the
+        bookkeeping of start_quantization_bits (this layer becomes the one a batch norm follows, its
+        row of the sensitivity pool is claimed)."""
+        QScheme.prev_layer = self
+        if not allocate_on_device(N, self.initial_bits):
+            return None
+        grad_sum = self.get_scale(device).to(device=device, dtype=torch.float32)
+        pool, row = QScheme.pool_row(self.index, N, device)
+        return AllocationArgs(N, self.num_locations / 4 / self.depthwise_groups * config.group_size / num_pixels,
+                              grad_sum, self.initial_bits, self.bits, row, _PooledRow(pool, self.index))
+
+    def adopt_device_bits(self, bits_dev, dim, args):
+        """What finish_quantization_bits records when the widths were made on the device."""
+        self.dim = dim
+        self._pending_C = args.pending
+        self.b = bits_dev
 
     def start_quantization_bits(self, input, known_minmax=None):
         """First half: min/max kernel, sensitivities, asynchronous copy to the host."""

@@ -227,6 +227,26 @@ int actnn_allocate_bits_device(const void* mn, const void* mx, float factor, con
                                int32_t* prefix, int64_t N, int64_t G, int initial_bits,
                                int64_t target, int dtype, void* stream);
 
+/* A layer's forward-side sequence in one call (the host layer's glue between the steps - Python
+ * here, the Function bodies of actnn/actnn/ops.py:99-118 and :436-470 in the reference - costs more
+ * than the kernels at small batch sizes).  Same kernels, same results, arguments as in the calls
+ * they stand for:
+ *   actnn_batch_norm_forward_quantize = actnn_batch_norm_forward_stats (with mn / mx)
+ *       -> actnn_allocate_bits_device (G = C * HW / 256) -> actnn_batch_norm_forward_apply (with bits);
+ *   actnn_quantize_activation = [actnn_minimax of data as rows of 256 unless minmax_known]
+ *       -> actnn_allocate_bits_device -> actnn_pack_mixed (gs = 256, in-kernel Philox mode).
+ * Every output pointer is required. */
+int actnn_batch_norm_forward_quantize(
+    const void* x, const float* weight, const float* bias, float* running_mean, float* running_var, void* y,
+    float* save_mean, float* save_invstd, void* mn, void* mx, void* workspace, int64_t workspace_bytes,
+    float factor, const float* mult, int mult_per_sample, float* sensitivity, int32_t* bits, int32_t* prefix,
+    int initial_bits, int64_t target, void* scale, int32_t* packed, uint64_t seed, uint64_t offset, int64_t N,
+    int64_t C, int64_t HW, double momentum, double eps, int dtype, int channels_last, void* stream);
+int actnn_quantize_activation(const void* data, void* mn, void* mx, int minmax_known, float factor,
+                              const float* mult, int mult_per_sample, float* sensitivity, int32_t* bits,
+                              int32_t* prefix, int initial_bits, int64_t target, void* scale, int32_t* packed,
+                              uint64_t seed, uint64_t offset, int64_t N, int64_t G, int dtype, void* stream);
+
 /* ---------------------------------------------------------------------------------
  * Fused QLinear weight gradient: grad_w[O, I] = grad_out[M, O]^T @ dequant(x)[M, I] where x is
  * held as a stream of this library with scale/min[M, I/256, 1] (groups of 256 along a row):

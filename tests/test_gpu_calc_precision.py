@@ -109,3 +109,74 @@ def test_allocation_in_one_call_from_dirty_buffers(N):
         if first is None:
             first = bits.clone()
         assert torch.equal(bits, first)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("known", [False, True])
+def test_quantise_an_activation_in_one_call_equals_the_three_calls(dtype, known):
+    """actnn_quantize_activation is [minimax] -> allocation -> pack_mixed on one stream: stream, scale,
+    min, widths, prefix and sensitivities are those of the separate calls on the same generator state."""
+    import actnn_amd.cpp_extension.minimax as ext_minimax
+    import actnn_amd.cpp_extension.quantization as ext_q
+    from actnn_amd.qscheme import AllocationArgs
+    N, G = 24, 13
+    g = torch.Generator(device=DEV).manual_seed(5)
+    rows = (torch.randn(N * G, 256, generator=g, device=DEV)
+            * torch.exp(torch.randn(N, 1, 1, generator=g, device=DEV)).expand(N, G, 256).reshape(N * G, 256)).to(dtype)
+    per_sample = torch.rand(N, generator=g, device=DEV) + 0.5
+    for mult in (None, per_sample[:1].reshape(()), per_sample):
+        sens_row = torch.empty(N, device=DEV)
+        alloc = AllocationArgs(N, 0.37, mult, 8, 2.25, sens_row)
+        mn, mx = ext_minimax.minimax(rows)
+        torch.cuda.manual_seed(11)
+        packed, bits, scale, mn_out = ext_q.quantize_activation_device(rows, N, (mn, mx) if known else None, alloc)
+        torch.cuda.manual_seed(11)
+        sens_ref, bits_ref, prefix_ref = ext_cp.allocate_bits_device(mn, mx, N, 0.37, mult, 8, int(2.25 * N))
+        ext_q.attach_bits_total(bits_ref, alloc.total, prefix_ref)
+        packed_ref, scale_ref = ext_q.pack_mixed_precision(rows.view(N, G, 256), mn.view(N, G, 1), mx.view(N, G, 1),
+                                                           bits_ref, True)
+        assert torch.equal(bits, bits_ref) and int(bits.sum()) == alloc.total == int(2.25 * N)
+        assert torch.equal(ext_q._bits_info(bits)[1], prefix_ref)
+        assert torch.equal(sens_row, sens_ref) and torch.equal(mn_out, mn)
+        assert torch.equal(packed, packed_ref) and torch.equal(scale, scale_ref)
+
+
+def test_one_call_entry_points_reject_what_their_steps_reject():
+    from actnn_amd import _lib
+    lib = _lib.load()
+    N, G = 4, 2
+    rows = torch.randn(N * G, 256, device=DEV)
+    mn, mx = torch.empty(N * G, device=DEV), torch.empty(N * G, device=DEV)
+    sens, bits, prefix = torch.empty(N, device=DEV), torch.empty(N, dtype=torch.int32, device=DEV), torch.empty(N + 1, dtype=torch.int32, device=DEV)
+    scale, packed = torch.empty(N * G, device=DEV), torch.empty(8 * N * G * 8, dtype=torch.int32, device=DEV)
+
+    def call(**k):
+        a = dict(data=rows.data_ptr(), mn=mn.data_ptr(), mx=mx.data_ptr(), known=0, sens=sens.data_ptr(),
+                 bits=bits.data_ptr(), prefix=prefix.data_ptr(), initial=8, target=2 * N, scale=scale.data_ptr(),
+                 packed=packed.data_ptr(), N=N, G=G, dtype=0)
+        a.update(k)
+        return lib.actnn_quantize_activation(a["data"], a["mn"], a["mx"], a["known"], 1.0, None, 0, a["sens"], a["bits"],
+                                             a["prefix"], a["initial"], a["target"], a["scale"], a["packed"], 1, 0,
+                                             a["N"], a["G"], a["dtype"], None)
+    assert call() == 0
+    for bad in (dict(data=None), dict(mn=None), dict(prefix=None), dict(packed=None), dict(N=0), dict(G=0),
+                dict(initial=9), dict(dtype=7), dict(data=rows.data_ptr() + 4)):
+        assert call(**bad) != 0, bad
+    # batch norm: every output is required, whole groups of 256 only
+    x = torch.randn(4, 8, 8, 8, device=DEV)
+    y = torch.empty_like(x)
+    ws_bytes = lib.actnn_batch_norm_workspace_bytes(4, 8, 64, 0, 0)
+    ws = torch.empty(ws_bytes // 4, device=DEV)
+    sm, si = torch.empty(8, device=DEV), torch.empty(8, device=DEV)
+
+    def bn(**k):
+        a = dict(y=y.data_ptr(), mn=mn.data_ptr(), packed=packed.data_ptr(), HW=64)
+        a.update(k)
+        return lib.actnn_batch_norm_forward_quantize(
+            x.data_ptr(), None, None, None, None, a["y"], sm.data_ptr(), si.data_ptr(), a["mn"], mx.data_ptr(),
+            ws.data_ptr(), ws_bytes, 1.0, None, 0, sens.data_ptr(), bits.data_ptr(), prefix.data_ptr(), 8, 2 * N,
+            scale.data_ptr(), a["packed"], 1, 0, 4, 8, a["HW"], 0.1, 1e-5, 0, 0, None)
+    assert bn() == 0
+    for bad in (dict(y=None), dict(mn=None), dict(packed=None), dict(HW=63)):
+        assert bn(**bad) != 0, bad
+    torch.cuda.synchronize()

@@ -205,23 +205,32 @@ def test_l3_first_step_uses_the_degenerate_allocation_then_rebalances():
     assert int(s0.b.sum()) <= int(budgets[0] * 16) and int(s0.b.min()) >= 1
 
 
-def test_sensitivities_reach_the_host_in_one_transfer_per_step():
+@pytest.mark.parametrize("one_call", [False, True])
+def test_sensitivities_reach_the_host_in_one_transfer_per_step(one_call):
     """The widths are made on the device; the sensitivities of all layers travel in one pool.  What
     the host reads per layer equals what the layer's own kernel computes from its input's ranges,
-    one step after another, and a change of the batch size makes a new pool."""
+    one step after another, and a change of the batch size makes a new pool - whether the layer's
+    sequence goes through one library call or step by step."""
     from actnn_amd import qscheme
+    from actnn_amd.cpp_extension import minimax as ext_minimax, quantization as ext_q
+    config.fused_quantize = one_call
     torch.manual_seed(0)
     model = QModule(nn.Sequential(nn.Conv2d(8, 8, 3, padding=1), nn.ReLU(), nn.Conv2d(8, 8, 3, padding=1),
                                   nn.ReLU(), nn.Conv2d(8, 4, 1))).to(DEV)
     seen = []
-    start = QScheme.start_quantization_bits
+    start, call = QScheme.start_quantization_bits, ext_q.quantize_activation_device
 
-    def spy(self, input, known_minmax=None):
+    def spy_start(self, input, known_minmax=None):
         groups, mn, mx, num_pixels = qscheme.group_min_max(input, known_minmax)
         seen.append((self, self.sensitivity(mn, mx, input.shape[0], num_pixels).clone()))
         return start(self, input, known_minmax)
 
-    QScheme.start_quantization_bits = spy
+    def spy_call(rows, N, known_minmax, alloc):
+        mn, mx = ext_minimax.minimax(rows)
+        seen.append((QScheme.layers[alloc.pending.index], ext_minimax.range_sqr(mn, mx, N, alloc.factor, alloc.mult)))
+        return call(rows, N, known_minmax, alloc)
+
+    QScheme.start_quantization_bits, ext_q.quantize_activation_device = spy_start, spy_call
     try:
         for step, n in enumerate((16, 16, 8)):
             seen.clear()
@@ -234,7 +243,84 @@ def test_sensitivities_reach_the_host_in_one_transfer_per_step():
                 assert scheme.C.shape == (n,)
                 assert torch.equal(scheme.C, expected.cpu()), (step, scheme.name)
     finally:
-        QScheme.start_quantization_bits = start
+        QScheme.start_quantization_bits, ext_q.quantize_activation_device = start, call
+
+
+@pytest.mark.parametrize("channels_last", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_one_library_call_per_layer_equals_the_step_by_step_sequence(channels_last, dtype):
+    """config.fused_quantize puts min/max (or the batch-norm statistics), the widths and the pack of a
+    layer behind one library call.  Same kernels on the same generator state: outputs, gradients,
+    widths and sensitivities of three training steps (per-layer re-balancing included) are those
+    of the step-by-step sequence bit for bit."""
+    from actnn_amd.cpp_extension import backward_func as bf, quantization as q
+
+    from actnn_amd import ops
+    plain_tuple = ops._Quantized
+
+    def run(fused):
+        config.reset(); QScheme.reset(); QBNScheme.reset()
+        set_optimization_level("L3")
+        config.fused_quantize = fused
+        torch.manual_seed(0)
+        model = QModule(nn.Sequential(nn.Conv2d(8, 16, 3, padding=1), nn.BatchNorm2d(16), nn.ReLU(),
+                                      nn.Conv2d(16, 16, 3, padding=1), nn.BatchNorm2d(16), nn.ReLU(),
+                                      nn.Conv2d(16, 8, 1))).to(DEV)
+        if channels_last:
+            model = model.to(memory_format=torch.channels_last)
+        torch.cuda.manual_seed(77)
+        calls = {"bn": 0, "conv": 0}
+        saved = []
+        real_bn, real_conv = bf.hip_batch_norm_forward_quantize, q.quantize_activation_device
+
+        def count_bn(*a, **k):
+            calls["bn"] += 1
+            return real_bn(*a, **k)
+
+        def count_conv(*a, **k):
+            calls["conv"] += 1
+            return real_conv(*a, **k)
+
+        class Recorded(plain_tuple):                      # every tuple a layer saves for its backward
+            def __new__(cls, items):
+                self = plain_tuple.__new__(cls, items)
+                saved.append(self)
+                return self
+
+        bf.hip_batch_norm_forward_quantize, q.quantize_activation_device = count_bn, count_conv
+        ops._Quantized = Recorded
+        out = []
+        try:
+            # (the weights stay as they are: MIOpen's weight-gradient kernels add with atomics, and
+            # what is compared here must not depend on their order)
+            for step in range(3):
+                g = torch.Generator(device=DEV).manual_seed(step)
+                x = torch.randn(16, 8, 16, 16, device=DEV, generator=g)
+                if channels_last:
+                    x = x.contiguous(memory_format=torch.channels_last)
+                model.zero_grad()
+                del saved[:]
+                with torch.autocast("cuda", dtype=torch.bfloat16, enabled=dtype == torch.bfloat16):
+                    y = model(x)
+                assert len(saved) == 5
+                kept = [t.clone() for tup in saved for t in tup] + \
+                       [torch.as_tensor([tup.native_bf16, tup.memory_format is not None]) for tup in saved]
+                y.float().square().mean().backward()
+                out.append([y.detach().clone()] + kept + [p.grad.clone() for p in model.parameters() if p.dim() == 1]
+                           + [l.b.clone() for l in QScheme.layers] + [l.C.clone() for l in QScheme.layers]
+                           + [torch.as_tensor(float(l.bits)) for l in QScheme.layers + QBNScheme.layers])
+        finally:
+            bf.hip_batch_norm_forward_quantize, q.quantize_activation_device = real_bn, real_conv
+            ops._Quantized = plain_tuple
+        return out, calls
+
+    (slow, slow_calls), (fast, fast_calls) = run(False), run(True)
+    assert slow_calls == {"bn": 0, "conv": 0}
+    assert fast_calls == {"bn": 6, "conv": 9}            # every batch norm and every convolution, every step
+    for step, (a, b) in enumerate(zip(slow, fast)):
+        assert len(a) == len(b)
+        for i, (u, v) in enumerate(zip(a, b)):
+            assert torch.equal(u.cpu(), v.cpu()), (step, i)
 
 
 @pytest.mark.parametrize("channels_last", [False, True])
