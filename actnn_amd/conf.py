@@ -35,6 +35,9 @@ class QuantizationConfig:
         # a layer's forward-side sequence (min/max or statistics -> widths -> pack) behind one library
         # call where the widths are made on the device: same kernels, less host time per layer
         self.fused_quantize = True
+        # relu(bn(x)) in the batch norm's normalise + pack pass where a model hands the pair over
+        # together (layers.bn_relu) and the shape allows it: bn(x) is never written
+        self.fused_bn_relu = True
         # QLinear's weight gradient straight from the packed input (the dequantised input is never
         # written): True - where the fused kernel is the faster path, i.e. for the 2-bit fixed-width
         # stream; "always" - for every stream it takes (saves the full-precision copy at 0.7-0.9 ms

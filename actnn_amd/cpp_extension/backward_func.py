@@ -191,13 +191,24 @@ def hip_batch_norm_quantize_geometry(input, weight, bias, running_mean, running_
     return geo
 
 
-def hip_batch_norm_forward_quantize(input, geo, weight, bias, running_mean, running_var, momentum, eps, alloc):
+def hip_batch_norm_relu_applies(geo, dtype):
+    """True when the normalise + pack pass can also apply the ReLU that follows the batch norm:
+    channels-last 16-bit tensors whose waves own whole 512-element blocks of the mask."""
+    N, C, HW, channels_last = geo
+    return (channels_last and dtype in (torch.float16, torch.bfloat16) and C <= 256 and 256 % C == 0
+            and (N * C * HW) % 2048 == 0)
+
+
+def hip_batch_norm_forward_quantize(input, geo, weight, bias, running_mean, running_var, momentum, eps, alloc,
+                                    relu=False):
     """Statistics + group min/max -> widths on the device -> normalise + pack, in one call:
     -> (output, save_mean, save_invstd, mn, mx, bits, packed, scale), what
     hip_batch_norm_forward_stats, allocate_bits_device and hip_batch_norm_forward_apply return one
     after the other.  `geo` from hip_batch_norm_quantize_geometry, `alloc` the scheme's
-    AllocationArgs (factor, mult, initial, target, total, sens_out)."""
-    from .quantization import attach_bits_total
+    AllocationArgs (factor, mult, initial, target, total, sens_out).  With `relu`
+    (hip_batch_norm_relu_applies) the output is relu(bn(input)) and the tuple ends with the ReLU's
+    mask and the group min / max of the output."""
+    from .quantization import attach_bits_total, mask_words
     N, C, HW, channels_last = geo
     dev, dtype = input.device, input.dtype
     code = _glue.DTYPE_CODE[dtype]
@@ -215,6 +226,11 @@ def hip_batch_norm_forward_quantize(input, geo, weight, bias, running_mean, runn
     prefix = torch.empty(N + 1, dtype=i32, device=dev)
     packed = torch.empty(alloc.total * G * 8, dtype=i32, device=dev)
     scale = torch.empty(N, G, 1, dtype=dtype, device=dev)
+    mask = zmn = zmx = None
+    if relu:
+        mask = torch.empty(mask_words(N * C * HW), dtype=i32, device=dev)
+        zmn = torch.empty(N * G, dtype=dtype, device=dev)
+        zmx = torch.empty(N * G, dtype=dtype, device=dev)
     mult, mult_ptr, per_sample = _mult_args(alloc.mult, N, dev)          # (`mult` held until the launch)
     seed, offset = _glue.philox_args(dev)
     with _glue.on_device(dev):
@@ -222,10 +238,12 @@ def hip_batch_norm_forward_quantize(input, geo, weight, bias, running_mean, runn
             input.data_ptr(), _ptr(weight), _ptr(bias), _ptr(running_mean), _ptr(running_var), out.data_ptr(),
             save_mean.data_ptr(), save_invstd.data_ptr(), mn.data_ptr(), mx.data_ptr(), ws.data_ptr(), ws_bytes,
             alloc.factor, mult_ptr, per_sample, sens.data_ptr(), bits.data_ptr(), prefix.data_ptr(),
-            alloc.initial, alloc.target, scale.data_ptr(), packed.data_ptr(), seed, offset, N, C, HW,
-            float(momentum), float(eps), code, int(channels_last), _glue.stream_ptr(dev)),
+            alloc.initial, alloc.target, scale.data_ptr(), packed.data_ptr(), seed, offset, _ptr(mask), _ptr(zmn),
+            _ptr(zmx), N, C, HW, float(momentum), float(eps), code, int(channels_last), _glue.stream_ptr(dev)),
             "batch_norm_forward_quantize")
     attach_bits_total(bits, alloc.total, prefix)
+    if relu:
+        return out, save_mean, save_invstd, mn, mx, bits, packed, scale, mask, zmn, zmx
     return out, save_mean, save_invstd, mn, mx, bits, packed, scale
 
 

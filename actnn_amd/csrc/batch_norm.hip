@@ -288,7 +288,35 @@ struct PackSink {
   // it wrote (as stored, i.e. rounded to T) in sumsq[(blockIdx.y * gridDim.x + blockIdx.x) * kWaves +
   // wave] - the gradient-norm statistic of the layer that receives this gradient, for free
   float* sumsq;
+  // forward apply with the ReLU folded in: the 1-bit mask (layout of the ReLU operator: 16 words per
+  // block of 512 elements) and the min / max of every group of 256 outputs
+  int32_t* relu_mask;
+  void* relu_mn;
+  void* relu_mx;
 };
+
+// ReLU on a word of two 16-bit values (already rounded to T, so the rule sees what a separate pass
+// over the stored tensor would see): -> the word with the non-positive halves zeroed; their keep
+// flags in bits 0 and 1 of `keep`; the two results as floats.
+template <typename T> ACTNN_DEV uint32_t relu_word(uint32_t w, uint32_t& keep, float& z0, float& z1) {
+  float v[2];
+  Chunk<T>::widen(w, v);
+  const bool k0 = v[0] > 0.0f, k1 = v[1] > 0.0f;
+  z0 = k0 ? v[0] : 0.0f;
+  z1 = k1 ? v[1] : 0.0f;
+  keep = (k0 ? 1u : 0u) | (k1 ? 2u : 0u);
+  return (k0 ? w & 0x0000ffffu : 0u) | (k1 ? w & 0xffff0000u : 0u);
+}
+// Keep bits of four 512-element blocks (per lane: 8 bits for each block, the lane's 8 elements) ->
+// this lane's mask word: lane 2p + h holds word p % 16 of block 2h + p / 16.
+ACTNN_DEV uint32_t mask_word_of_rows(const uint32_t (&m)[4], uint32_t lane) {
+  const bool odd = lane & 1u;
+  const uint32_t ab = m[0] | (m[1] << 16), cd = m[2] | (m[3] << 16);
+  const uint32_t recv = lane_xor<1>(odd ? ab : cd);
+  const uint32_t mine = odd ? cd : ab;
+  const uint32_t row = odd ? (recv | (mine << 8)) : (mine | (recv << 8));
+  return transpose32_x2(row, lane);
+}
 
 ACTNN_DEV void leave_wave_sum(float* table, float v) {
 #pragma unroll
@@ -1056,7 +1084,7 @@ __global__ __launch_bounds__(kThreads, (cl_reduce_waves<BWD, MINMAX, XS>())) voi
   }
 }
 
-template <typename T, bool BWD, bool PACK, typename XS>
+template <typename T, bool BWD, bool PACK, typename XS, bool RELU = false>
 __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
     XS xs, const T* __restrict__ dy, const float* __restrict__ coef, T* __restrict__ out,
     int64_t P, int64_t C, int tpr, int R, int64_t ppb, PackSink ps, FastDiv by_hw) {
@@ -1065,6 +1093,7 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
   constexpr int NC = BWD ? 3 : 2;
   constexpr int U = XS::kInFlight;
   static_assert(!(PACK && BWD), "the packed copy is made by the forward pass");
+  static_assert(!RELU || (PACK && sizeof(T) == 2), "the ReLU is folded into the packing pass of 16-bit tensors");
   // The sample that holds the row of the last pack: its width, its first word in the stream and its
   // first row / group.  A thread stays inside one sample for many rows, so these are looked up only
   // when a row leaves it, and a chunk's place in the stream is 32-bit arithmetic on top of them (rows,
@@ -1177,11 +1206,68 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
     // their noise
     const int lane32 = threadIdx.x & 31;
     ParamQueue<T> queue;
-    auto pack_one = [&](const u32x4& ux, const uint32_t (&rw)[Noise<T>::kWords], int64_t ru, int j) {
+    auto pack_one = [&](const u32x4& ux, const uint32_t (&rw)[Noise<T>::kWords], int64_t ru, int j) __attribute__((always_inline)) {
       locate((uint32_t)ru + (uint32_t)t.r);
       float mul, sub;
       queue.get(j, mul, sub);
       pack_chunk<T, false>(ux, rw, mul, sub, group_words((uint32_t)((ru * C) >> 8) + (lane_elems >> 8)), cur_b);
+    };
+    // RELU: the wave's 64 chunks of a step are 512 consecutive elements - one block of the mask - and
+    // a half-wave's 32 chunks one group of 256 outputs (the launcher takes this path only when that
+    // holds and every step of a block is whole).  emit() applies the rule to the normalised chunk,
+    // stores it, leaves the group's min / max and the lane's 8 keep bits in `row`; four steps' rows
+    // make the wave's 64 mask words (blocks 4 apart: a step of the block is 2048 elements).
+    const uint32_t lane = threadIdx.x & 63u;
+    auto emit = [&](int64_t ru, const u32x4& y, uint32_t& row) __attribute__((always_inline)) {
+      if constexpr (RELU) {
+        uint32_t w[4] = {y.x, y.y, y.z, y.w};
+        float z[8];
+        row = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          uint32_t keep;
+          w[k] = relu_word<T>(w[k], keep, z[2 * k], z[2 * k + 1]);
+          row |= keep << (2 * k);
+        }
+        store_out(out_at(ru), u32x4{w[0], w[1], w[2], w[3]});
+        float lo, hi;
+        minmax_of<8>(z, lo, hi);
+        lanes_minmax<2>(lo, hi);
+        if ((lane & 31u) == 31u) {
+          const uint32_t g = (uint32_t)((ru * C) >> 8) + (lane_elems >> 8);
+          Conv<T>::store(static_cast<T*>(ps.relu_mn), g, lo);
+          Conv<T>::store(static_cast<T*>(ps.relu_mx), g, hi);
+        }
+      } else {
+        store_out(out_at(ru), y);
+      }
+    };
+    auto leave_mask = [&](int64_t ru_first, const uint32_t (&rows)[4], int count) __attribute__((always_inline)) {
+      const uint32_t word = mask_word_of_rows(rows, lane);
+      const int slot = 2 * (int)(lane & 1u) + (int)(lane >> 5);
+      const int64_t block = ((ru_first * C) >> 9) + (threadIdx.x >> 6) + 4 * slot;
+      if (slot < count) ps.relu_mask[block * 16 + ((lane >> 1) & 15u)] = (int32_t)word;
+    };
+    auto pair = [&](int64_t rb0, int j, uint32_t& row0, uint32_t& row1) __attribute__((always_inline)) {
+      const int64_t ru0 = rb0 + (int64_t)j * R, ru1 = ru0 + R;
+      const typename XS::Raw rx0 = xs.fetch(ru0), rx1 = xs.fetch(ru1);
+      uint32_t rw[2][Noise<T>::kWords];
+      noise_pair<T>(ps, (uint64_t)((ru0 * C) >> 3) + (lane_elems >> 3), (uint64_t)((ru1 * C) >> 3) + (lane_elems >> 3),
+                    rw[0], rw[1], (tpr & 1) == 0);      // lane ^ 1 is in the same row, hence in the same steps
+      const u32x4 ux0 = xs.decode(rx0);
+      emit(ru0, apply(ux0, ux0), row0);
+      pack_one(ux0, rw[0], ru0, j);
+      const u32x4 ux1 = xs.decode(rx1);
+      emit(ru1, apply(ux1, ux1), row1);
+      pack_one(ux1, rw[1], ru1, j + 1);
+    };
+    auto single = [&](int64_t rb0, int j, uint32_t& row) __attribute__((always_inline)) {
+      const int64_t ru0 = rb0 + (int64_t)j * R;
+      const u32x4 ux = xs.decode(xs.fetch(ru0));
+      emit(ru0, apply(ux, ux), row);
+      uint32_t rw[Noise<T>::kWords];
+      Noise<T>::octet((uint64_t)((ru0 * C) >> 3) + (lane_elems >> 3), ps.seed, ps.offset, rw);
+      pack_one(ux, rw, ru0, j);
     };
     for (int64_t rb0 = p0; rb0 + t.r < p1; rb0 += (int64_t)32 * R) {
       const int64_t rb = rb0 + t.r;
@@ -1192,26 +1278,42 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
         queue.fill(ps, (rj * C + t.col) >> 8, live ? ps.bits[nj] : 1, live);
       }
       int j = 0;
-      for (; j + 2 <= 32 && rb + (int64_t)(j + 1) * R < p1; j += 2) {
-        const int64_t ru0 = rb0 + (int64_t)j * R, ru1 = ru0 + R;
-        const typename XS::Raw rx0 = xs.fetch(ru0), rx1 = xs.fetch(ru1);
-        uint32_t rw[2][Noise<T>::kWords];
-        noise_pair<T>(ps, (uint64_t)((ru0 * C) >> 3) + (lane_elems >> 3), (uint64_t)((ru1 * C) >> 3) + (lane_elems >> 3),
-                      rw[0], rw[1], (tpr & 1) == 0);      // lane ^ 1 is in the same row, hence in the same steps
-        const u32x4 ux0 = xs.decode(rx0);
-        store_out(out_at(ru0), apply(ux0, ux0));
-        pack_one(ux0, rw[0], ru0, j);
-        const u32x4 ux1 = xs.decode(rx1);
-        store_out(out_at(ru1), apply(ux1, ux1));
-        pack_one(ux1, rw[1], ru1, j + 1);
-      }
-      for (; j < 32 && rb + (int64_t)j * R < p1; ++j) {
-        const int64_t ru0 = rb0 + (int64_t)j * R;
-        const u32x4 ux = xs.decode(xs.fetch(ru0));
-        store_out(out_at(ru0), apply(ux, ux));
-        uint32_t rw[Noise<T>::kWords];
-        Noise<T>::octet((uint64_t)((ru0 * C) >> 3) + (lane_elems >> 3), ps.seed, ps.offset, rw);
-        pack_one(ux, rw, ru0, j);
+      if constexpr (RELU) {
+        uint32_t rows[4] = {0u, 0u, 0u, 0u};
+        for (; j + 4 <= 32 && rb + (int64_t)(j + 3) * R < p1; j += 4) {
+          pair(rb0, j, rows[0], rows[1]);
+          pair(rb0, j + 2, rows[2], rows[3]);
+          leave_mask(rb0 + (int64_t)j * R, rows, 4);
+        }
+        // what is left of the block's rows: up to three steps
+        const int64_t ru_first = rb0 + (int64_t)j * R;
+        int left = 0;
+        if (j < 32 && rb + (int64_t)j * R < p1) { single(rb0, j, rows[0]); ++j; ++left; }
+        if (j < 32 && rb + (int64_t)j * R < p1) { single(rb0, j, rows[1]); ++j; ++left; }
+        if (j < 32 && rb + (int64_t)j * R < p1) { single(rb0, j, rows[2]); ++j; ++left; }
+        if (left) leave_mask(ru_first, rows, left);
+      } else {
+        for (; j + 2 <= 32 && rb + (int64_t)(j + 1) * R < p1; j += 2) {
+          const int64_t ru0 = rb0 + (int64_t)j * R, ru1 = ru0 + R;
+          const typename XS::Raw rx0 = xs.fetch(ru0), rx1 = xs.fetch(ru1);
+          uint32_t rw[2][Noise<T>::kWords];
+          noise_pair<T>(ps, (uint64_t)((ru0 * C) >> 3) + (lane_elems >> 3), (uint64_t)((ru1 * C) >> 3) + (lane_elems >> 3),
+                        rw[0], rw[1], (tpr & 1) == 0);      // lane ^ 1 is in the same row, hence in the same steps
+          const u32x4 ux0 = xs.decode(rx0);
+          store_out(out_at(ru0), apply(ux0, ux0));
+          pack_one(ux0, rw[0], ru0, j);
+          const u32x4 ux1 = xs.decode(rx1);
+          store_out(out_at(ru1), apply(ux1, ux1));
+          pack_one(ux1, rw[1], ru1, j + 1);
+        }
+        for (; j < 32 && rb + (int64_t)j * R < p1; ++j) {
+          const int64_t ru0 = rb0 + (int64_t)j * R;
+          const u32x4 ux = xs.decode(xs.fetch(ru0));
+          store_out(out_at(ru0), apply(ux, ux));
+          uint32_t rw[Noise<T>::kWords];
+          Noise<T>::octet((uint64_t)((ru0 * C) >> 3) + (lane_elems >> 3), ps.seed, ps.offset, rw);
+          pack_one(ux, rw, ru0, j);
+        }
       }
     }
   } else {
@@ -1427,11 +1529,11 @@ int launch_cl_reduce(const Plan& pl, const XS& xs, const void* dy, float* part, 
       pl.tiles, rows.nsplit);
   return rows.nsplit;
 }
-template <typename T, bool BWD, bool PACK, typename XS>
+template <typename T, bool BWD, bool PACK, typename XS, bool RELU = false>
 void launch_cl_apply(const Plan& pl, const XS& xs, const void* dy, const float* coef, void* out, int64_t C,
                      const PackSink& ps, hipStream_t s) {
   const dim3 grid((unsigned)pl.tiles, (unsigned)pl.nsplit_apply), blk(kThreads);
-  bn_cl_apply_kernel<T, BWD, PACK, XS><<<grid, blk, 0, s>>>(
+  bn_cl_apply_kernel<T, BWD, PACK, XS, RELU><<<grid, blk, 0, s>>>(
       xs, static_cast<const T*>(dy), coef, static_cast<T*>(out), pl.P, C, pl.tpr, pl.R, pl.ppb_apply, ps,
       FastDiv((uint32_t)(pl.F / C)));
 }
@@ -1491,6 +1593,12 @@ int forward_apply_t(const Plan& pl, const void* x, void* y, const float* ws, con
   }
   if (pl.channels_last) {
     const PlainRows<T> xs{static_cast<const T*>(x), C};
+    if constexpr (sizeof(T) == 2) {
+      if (sink && sink->relu_mask) {
+        launch_cl_apply<T, false, true, PlainRows<T>, true>(pl, xs, nullptr, coef, y, C, *sink, s);
+        ACTNN_RETURN_LAUNCH_STATUS();
+      }
+    }
     if (sink) { launch_cl_apply<T, false, true>(pl, xs, nullptr, coef, y, C, *sink, s); ACTNN_RETURN_LAUNCH_STATUS(); }
     launch_cl_apply<T, false, false>(pl, xs, nullptr, coef, y, C, none, s);
   } else {
@@ -1652,6 +1760,34 @@ extern "C" int actnn_batch_norm_forward_apply(const void* x, void* y, const void
     case ACTNN_F16: return forward_apply_t<__half>(pl, x, y, ws, pack ? &sink : nullptr, N, C, HW, s);
     default: return forward_apply_t<bf16_t>(pl, x, y, ws, pack ? &sink : nullptr, N, C, HW, s);
   }
+}
+
+// _apply with the ReLU that follows the batch norm folded in: y = relu(bn(x)) as the ReLU operator
+// would make it from the stored bn(x), with its 1-bit mask and the min / max of every group of 256
+// outputs; packed copy of x as in _apply.
+extern "C" int actnn_batch_norm_forward_apply_relu(const void* x, void* y, const void* workspace,
+                                                   int64_t workspace_bytes, const int32_t* bits,
+                                                   const int32_t* prefix, const void* mn, const void* mx,
+                                                   void* scale, int32_t* packed, uint64_t seed, uint64_t offset,
+                                                   int32_t* relu_mask, void* relu_mn, void* relu_mx, int64_t N,
+                                                   int64_t C, int64_t HW, int dtype, int channels_last,
+                                                   void* stream) {
+  using namespace actnn;
+  if (dtype != ACTNN_F16 && dtype != ACTNN_BF16) return ACTNN_EDTYPE;
+  Plan pl;
+  if (!channels_last || !make_plan(N, C, HW, dtype, channels_last, pl) || pl.any_shape) return ACTNN_EINVAL;
+  if (!x || !y || !workspace || !bits || !prefix || !mn || !mx || !scale || !packed || !relu_mask || !relu_mn || !relu_mx)
+    return ACTNN_EINVAL;
+  if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
+  if (!aligned16(x) || !aligned16(y) || !aligned16(workspace)) return ACTNN_EALIGN;
+  // a wave's step is one 512-element block of the mask, every step of every block is whole
+  if (!pl.groups_align || C > 256 || 256 % C != 0 || (N * pl.F) % 2048 != 0) return ACTNN_EINVAL;
+  if (pl.P > 0x7fffffffLL || C * HW >= ((int64_t)1 << 32) || N * (pl.F / 256) >= 0x7fffffffLL) return ACTNN_EINVAL;
+  PackSink sink{bits, prefix, mn, mx, scale, packed, seed, offset, pl.F / 256, nullptr, relu_mask, relu_mn, relu_mx};
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const float* ws = static_cast<const float*>(workspace);
+  if (dtype == ACTNN_F16) return forward_apply_t<__half>(pl, x, y, ws, &sink, N, C, HW, s);
+  return forward_apply_t<bf16_t>(pl, x, y, ws, &sink, N, C, HW, s);
 }
 
 extern "C" int actnn_batch_norm_forward(const void* x, const float* weight, const float* bias,

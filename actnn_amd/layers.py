@@ -15,7 +15,7 @@ from torch.nn.modules.utils import _pair, _single, _triple
 
 from .conf import config
 from .cpp_extension import quantization as ext_quantization
-from .ops import (batch_norm, conv1d, conv2d, conv3d, conv_transpose1d, conv_transpose2d, conv_transpose3d,
+from .ops import (batch_norm, batch_norm_relu, batch_norm_relu_geometry, conv1d, conv2d, conv3d, conv_transpose1d, conv_transpose2d, conv_transpose3d,
                   linear)
 from .qbnscheme import QBNScheme
 from .qscheme import QScheme
@@ -195,9 +195,12 @@ class _QBatchNormMixin:
     def _init_scheme(self, group):
         self.scheme = QBNScheme(group=group) if config.adaptive_bn_scheme else None
 
-    def forward(self, input):
+    def forward(self, input, relu=None):
+        """`relu`: the QReLU that follows this layer, when the caller hands the pair over together
+        (bn_relu): where the shape allows, the ReLU is folded into the normalise + pack pass."""
         if not config.training:
-            return super().forward(input)
+            out = super().forward(input)
+            return out if relu is None else relu(out)
         self._check_input_dim(input)
         factor = 0.0 if self.momentum is None else self.momentum
         if self.training and self.track_running_stats and self.num_batches_tracked is not None:
@@ -207,9 +210,20 @@ class _QBatchNormMixin:
         bn_training = True if self.training else (self.running_mean is None and self.running_var is None)
         keep_buffers = (not self.training) or self.track_running_stats
         # statistics and affine parameters stay fp32 under autocast (mixed-precision batch norm)
-        return batch_norm.apply(input, self.running_mean if keep_buffers else None,
-                                self.running_var if keep_buffers else None, self.weight, self.bias,
-                                bn_training, factor, self.eps, self.scheme)
+        running_mean = self.running_mean if keep_buffers else None
+        running_var = self.running_var if keep_buffers else None
+        if relu is not None:
+            geo = batch_norm_relu_geometry(input, running_mean, running_var, self.weight, self.bias, bn_training,
+                                           self.scheme)
+            if geo is not None:
+                out, mn, mx = batch_norm_relu.apply(input, running_mean, running_var, self.weight, self.bias,
+                                                    bn_training, factor, self.eps, self.scheme, geo)
+                if _relu_shares_min_max(memory_order(out)):
+                    out._actnn_group_minmax = (mn, mx, out._version)
+                return out
+        out = batch_norm.apply(input, running_mean, running_var, self.weight, self.bias, bn_training, factor,
+                               self.eps, self.scheme)
+        return out if relu is None else relu(out)
 
 
 class QBatchNorm1d(_QBatchNormMixin, nn.BatchNorm1d):
@@ -273,6 +287,15 @@ class QReLU(nn.Module):
             return out
         out = ext_quantization.act_quantized_relu(x)
         return logical_order(out, fmt) if fmt is not None else out
+
+
+def bn_relu(bn, relu, input):
+    """relu(bn(input)) for a model that knows the two layers follow each other: converted layers get
+    the pair in one pass where the shape allows (the normalised tensor is then never written),
+    everything else is the two calls."""
+    if isinstance(bn, _QBatchNormMixin) and not isinstance(bn, QSyncBatchNorm) and type(relu) is QReLU:
+        return bn(input, relu)
+    return relu(bn(input))
 
 
 class AddReLU(nn.Module):

@@ -14,7 +14,7 @@ from .conf import config
 from .cpp_extension import backward_func as ext_backward_func
 from .cpp_extension import quantization as ext_quantization
 from .utils import (channels_last_format, compute_tensor_bytes, empty_cache, get_memory_usage,
-                    logical_order, swap_to_cpu, swap_to_device)
+                    logical_order, memory_order, swap_to_cpu, swap_to_device)
 
 
 # ------------------------------------------------------------------------------------------
@@ -456,6 +456,28 @@ def _uniform_bits(N, bits, device):
     return q_bits
 
 
+def _bn_quantize_geometry(input, running_mean, running_var, weight, bias, training, scheme):
+    """(N, C, HW, channels_last) when statistics -> widths -> normalise + pack can go through one
+    library call for this input, else None."""
+    if not (scheme and config.fused_quantize and config.fused_bn_pack and config.stochastic and training
+            and config.compress_activation and config.pergroup and not config.simulate and not config.swap
+            and config.group_size == 256):
+        return None
+    return ext_backward_func.hip_batch_norm_quantize_geometry(input, weight, bias, running_mean, running_var)
+
+
+def batch_norm_relu_geometry(input, running_mean, running_var, weight, bias, training, scheme):
+    """The geometry to hand to batch_norm_relu when the ReLU that follows the batch norm can be
+    folded into its normalise + pack pass, else None (the caller then applies the two layers)."""
+    from .qscheme import allocate_on_device
+    if not config.fused_bn_relu:
+        return None
+    geo = _bn_quantize_geometry(input, running_mean, running_var, weight, bias, training, scheme)
+    if geo is None or not ext_backward_func.hip_batch_norm_relu_applies(geo, input.dtype):
+        return None
+    return geo if allocate_on_device(geo[0], scheme.initial_bits) else None
+
+
 class batch_norm(Function):
     @staticmethod
     def forward(ctx, input, running_mean, running_var, weight, bias, training,
@@ -466,16 +488,13 @@ class batch_norm(Function):
         # (the pass rounds stochastically, like pack_*; with config.stochastic off the unfused
         # sequence below is taken and pack_* refuses, as in the reference)
         fused = None
-        if (scheme and config.fused_quantize and config.fused_bn_pack and config.stochastic and training
-                and config.compress_activation and config.pergroup and not config.simulate and not config.swap
-                and config.group_size == 256):
-            # statistics -> widths -> normalise + pack behind one library call (the branch below, for
-            # a scheme whose widths are made on the device; same kernels, same generator state)
-            geo = ext_backward_func.hip_batch_norm_quantize_geometry(input, weight, bias, running_mean, running_var)
-            alloc = scheme.allocation_arguments(geo[0], geo[2], input.device) if geo is not None else None
-            if alloc is not None:
-                fused = ext_backward_func.hip_batch_norm_forward_quantize(
-                    input, geo, weight, bias, running_mean, running_var, exponential_average_factor, eps, alloc)
+        # statistics -> widths -> normalise + pack behind one library call (the second branch below,
+        # for a scheme whose widths are made on the device; same kernels, same generator state)
+        geo = _bn_quantize_geometry(input, running_mean, running_var, weight, bias, training, scheme)
+        alloc = scheme.allocation_arguments(geo[0], geo[2], input.device) if geo is not None else None
+        if alloc is not None:
+            fused = ext_backward_func.hip_batch_norm_forward_quantize(
+                input, geo, weight, bias, running_mean, running_var, exponential_average_factor, eps, alloc)
         if fused is not None:
             output, save_mean, save_var, mn, mx, q_bits, q_input, q_scale = fused
             N = geo[0]
@@ -542,41 +561,80 @@ class batch_norm(Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        quantized, weight, running_mean, running_var, save_mean, save_var, training, eps, reserve = ctx.saved
-        if (training and config.compress_activation and not config.simulate
-                and config.group_size == 256 and config.fused_bn_backward):
-            if config.swap and isinstance(quantized[0], torch.Tensor) and not quantized[0].is_cuda:
-                back = _Quantized((swap_to_device(quantized[0]),) + tuple(quantized[1:]))
-                back.native_bf16, back.memory_format = quantized.native_bf16, quantized.memory_format
-                quantized = back
-            grad_output = grad_output.contiguous(
-                memory_format=getattr(quantized, "memory_format", None) or torch.contiguous_format)
-            if ext_backward_func.hip_batch_norm_backward_packed_applies(
-                    ctx.other_args, quantized, grad_output, weight, save_mean, save_var):
-                # the kernels decode the saved input from its bit stream: no full-precision copy
-                grads = ext_backward_func.hip_batch_norm_backward_packed(
-                    ctx.other_args, quantized, grad_output, weight, save_mean, save_var,
-                    sumsq=_leaves_grad_sqnorm())
-                del quantized, ctx.saved
-                if ctx.scheme:
-                    ctx.scheme.if_allocate_perlayer()
-                return grads[0], None, None, grads[1], grads[2], None, None, None, None
-        input = dequantize_activation(quantized, ctx.other_args)
-        memory_format = getattr(quantized, "memory_format", None) or torch.contiguous_format
-        del quantized, ctx.saved
+        return _batch_norm_backward(ctx, grad_output)
+
+
+def _batch_norm_backward(ctx, grad_output):
+    quantized, weight, running_mean, running_var, save_mean, save_var, training, eps, reserve = ctx.saved
+    if (training and config.compress_activation and not config.simulate
+            and config.group_size == 256 and config.fused_bn_backward):
+        if config.swap and isinstance(quantized[0], torch.Tensor) and not quantized[0].is_cuda:
+            back = _Quantized((swap_to_device(quantized[0]),) + tuple(quantized[1:]))
+            back.native_bf16, back.memory_format = quantized.native_bf16, quantized.memory_format
+            quantized = back
+        grad_output = grad_output.contiguous(
+            memory_format=getattr(quantized, "memory_format", None) or torch.contiguous_format)
+        if ext_backward_func.hip_batch_norm_backward_packed_applies(
+                ctx.other_args, quantized, grad_output, weight, save_mean, save_var):
+            # the kernels decode the saved input from its bit stream: no full-precision copy
+            grads = ext_backward_func.hip_batch_norm_backward_packed(
+                ctx.other_args, quantized, grad_output, weight, save_mean, save_var,
+                sumsq=_leaves_grad_sqnorm())
+            del quantized, ctx.saved
+            if ctx.scheme:
+                ctx.scheme.if_allocate_perlayer()
+            return grads[0], None, None, grads[1], grads[2], None, None, None, None
+    input = dequantize_activation(quantized, ctx.other_args)
+    memory_format = getattr(quantized, "memory_format", None) or torch.contiguous_format
+    del quantized, ctx.saved
+    empty_cache(config.empty_cache_threshold)
+    if training:
+        grad_input, grad_weight, grad_bias = ext_backward_func.cudnn_batch_norm_backward(
+            input.contiguous(memory_format=memory_format),
+            grad_output.contiguous(memory_format=memory_format), weight, running_mean, running_var,
+            save_mean, save_var, eps, reserve, sumsq=_leaves_grad_sqnorm())
+    else:
+        grad_input, grad_weight, grad_bias = ext_backward_func.native_batch_norm_backward(
+            grad_output, input, weight, running_mean, running_var, save_mean, save_var, training, eps,
+            [ctx.needs_input_grad[0], ctx.needs_input_grad[3], ctx.needs_input_grad[4]])
+    if ctx.scheme:
+        ctx.scheme.if_allocate_perlayer()
+    return grad_input, None, None, grad_weight, grad_bias, None, None, None, None
+
+
+class batch_norm_relu(Function):
+    """relu(batch_norm(input)) with the ReLU folded into the pass that normalises and packs: the
+    normalised tensor is never written.  Saves what the two layers save - the compressed input and
+    the ReLU's 1-bit mask - and returns the group min / max of the output beside it (not
+    differentiable), as QReLU does.  Only for inputs batch_norm_relu_geometry accepts (`geo`)."""
+
+    @staticmethod
+    def forward(ctx, input, running_mean, running_var, weight, bias, training,
+                exponential_average_factor, eps, scheme, geo):
+        alloc = scheme.allocation_arguments(geo[0], geo[2], input.device)
+        (output, save_mean, save_var, mn, _mx, q_bits, q_input, q_scale, mask, out_mn,
+         out_mx) = ext_backward_func.hip_batch_norm_forward_quantize(
+            input, geo, weight, bias, running_mean, running_var, exponential_average_factor, eps, alloc, relu=True)
+        N = geo[0]
+        scheme.adopt_device_bits(q_bits, input.numel() // N, alloc)
+        quantized = _mark_saved(_Quantized((q_input, q_bits, q_scale, mn.view(N, -1, 1))), input)
         empty_cache(config.empty_cache_threshold)
-        if training:
-            grad_input, grad_weight, grad_bias = ext_backward_func.cudnn_batch_norm_backward(
-                input.contiguous(memory_format=memory_format),
-                grad_output.contiguous(memory_format=memory_format), weight, running_mean, running_var,
-                save_mean, save_var, eps, reserve, sumsq=_leaves_grad_sqnorm())
-        else:
-            grad_input, grad_weight, grad_bias = ext_backward_func.native_batch_norm_backward(
-                grad_output, input, weight, running_mean, running_var, save_mean, save_var, training, eps,
-                [ctx.needs_input_grad[0], ctx.needs_input_grad[3], ctx.needs_input_grad[4]])
-        if ctx.scheme:
-            ctx.scheme.if_allocate_perlayer()
-        return grad_input, None, None, grad_weight, grad_bias, None, None, None, None
+        ctx.scheme = scheme
+        ctx.other_args = input.shape
+        ctx.saved = (quantized, weight, running_mean, running_var, save_mean, save_var, training, eps, None)
+        ctx.relu_mask = mask
+        ctx.mark_non_differentiable(out_mn, out_mx)
+        ctx.set_materialize_grads(False)
+        return output, out_mn, out_mx
+
+    @staticmethod
+    def backward(ctx, grad_output, _grad_mn, _grad_mx):
+        if grad_output is None:
+            return (None,) * 10
+        fmt = ctx.saved[0].memory_format
+        grad = ext_quantization.relu_backward(memory_order(grad_output.contiguous(memory_format=fmt)), ctx.relu_mask)
+        ctx.relu_mask = None
+        return _batch_norm_backward(ctx, logical_order(grad, fmt)) + (None,)
 
 
 class adaptive_avg_pool2d(Function):

@@ -1,12 +1,13 @@
 """ResNet-50 (v1.5: stride on the 3x3 convolution) in the standard public layout, built from
 plain torch.nn layers (and AddReLU for the closing relu(out + identity) of a block) so that QModule
-can convert it.  torchvision is not available in this
+can convert it; relu(bn(x)) pairs are handed to layers.bn_relu, which is the two calls for plain
+layers.  torchvision is not available in this
 environment; the reference benchmarks torchvision's resnet50
 (mem_speed_benchmark/train.py:170,203-206)."""
 import torch
 import torch.nn as nn
 
-from .layers import AddReLU
+from .layers import AddReLU, bn_relu
 
 
 class Bottleneck(nn.Module):
@@ -28,8 +29,8 @@ class Bottleneck(nn.Module):
 
     def forward(self, x):
         identity = x
-        out = self.relu1(self.bn1(self.conv1(x)))
-        out = self.relu2(self.bn2(self.conv2(out)))
+        out = bn_relu(self.bn1, self.relu1, self.conv1(x))
+        out = bn_relu(self.bn2, self.relu2, self.conv2(out))
         out = self.bn3(self.conv3(out))
         if self.downsample is not None:
             identity = self.downsample(x)
@@ -66,7 +67,7 @@ class ResNet(nn.Module):
         return nn.Sequential(*layers)
 
     def forward(self, x):
-        x = self.maxpool(self.relu(self.bn1(self.conv1(x))))
+        x = self.maxpool(bn_relu(self.bn1, self.relu, self.conv1(x)))
         x = self.layer4(self.layer3(self.layer2(self.layer1(x))))
         return self.fc(torch.flatten(self.avgpool(x), 1))
 

@@ -227,12 +227,29 @@ int actnn_allocate_bits_device(const void* mn, const void* mx, float factor, con
                                int32_t* prefix, int64_t N, int64_t G, int initial_bits,
                                int64_t target, int dtype, void* stream);
 
+/* actnn_batch_norm_forward_apply (with bits) with the ReLU that follows the batch norm folded into
+ * the pass: y = relu(bn(x)), relu_mask and relu_mn / relu_mx[N * C * HW / 256] are what
+ * actnn_relu_forward_minmax makes of the stored bn(x) (the normalised value is rounded to `dtype`
+ * before the rule is applied), bn(x) itself is never written; scale and the packed copy of x as in
+ * _apply.  One pass over x instead of a pass over x and a pass over bn(x) (torchvision's
+ * `relu(bn(conv(x)))`, mem_speed_benchmark/train.py:203-206; ops.py:436-470 and
+ * quantization.cc:106-124 in the reference).  Channels-last 16-bit tensors with C a divisor of 256
+ * and N * C * HW a multiple of 2048 (a wave's 64 chunks are then one 512-element block of the
+ * mask); everything else is ACTNN_EINVAL / ACTNN_EDTYPE. */
+int actnn_batch_norm_forward_apply_relu(const void* x, void* y, const void* workspace,
+                                        int64_t workspace_bytes, const int32_t* bits,
+                                        const int32_t* prefix, const void* mn, const void* mx, void* scale,
+                                        int32_t* packed, uint64_t seed, uint64_t offset, int32_t* relu_mask,
+                                        void* relu_mn, void* relu_mx, int64_t N, int64_t C, int64_t HW,
+                                        int dtype, int channels_last, void* stream);
+
 /* A layer's forward-side sequence in one call (the host layer's glue between the steps - Python
  * here, the Function bodies of actnn/actnn/ops.py:99-118 and :436-470 in the reference - costs more
  * than the kernels at small batch sizes).  Same kernels, same results, arguments as in the calls
  * they stand for:
  *   actnn_batch_norm_forward_quantize = actnn_batch_norm_forward_stats (with mn / mx)
- *       -> actnn_allocate_bits_device (G = C * HW / 256) -> actnn_batch_norm_forward_apply (with bits);
+ *       -> actnn_allocate_bits_device (G = C * HW / 256) -> actnn_batch_norm_forward_apply (with bits),
+ *       or, with relu_mask / relu_mn / relu_mx given (all three), -> actnn_batch_norm_forward_apply_relu;
  *   actnn_quantize_activation = [actnn_minimax of data as rows of 256 unless minmax_known]
  *       -> actnn_allocate_bits_device -> actnn_pack_mixed (gs = 256, in-kernel Philox mode).
  * Every output pointer is required. */
@@ -240,8 +257,9 @@ int actnn_batch_norm_forward_quantize(
     const void* x, const float* weight, const float* bias, float* running_mean, float* running_var, void* y,
     float* save_mean, float* save_invstd, void* mn, void* mx, void* workspace, int64_t workspace_bytes,
     float factor, const float* mult, int mult_per_sample, float* sensitivity, int32_t* bits, int32_t* prefix,
-    int initial_bits, int64_t target, void* scale, int32_t* packed, uint64_t seed, uint64_t offset, int64_t N,
-    int64_t C, int64_t HW, double momentum, double eps, int dtype, int channels_last, void* stream);
+    int initial_bits, int64_t target, void* scale, int32_t* packed, uint64_t seed, uint64_t offset,
+    int32_t* relu_mask, void* relu_mn, void* relu_mx, int64_t N, int64_t C, int64_t HW, double momentum,
+    double eps, int dtype, int channels_last, void* stream);
 int actnn_quantize_activation(const void* data, void* mn, void* mx, int minmax_known, float factor,
                               const float* mult, int mult_per_sample, float* sensitivity, int32_t* bits,
                               int32_t* prefix, int initial_bits, int64_t target, void* scale, int32_t* packed,

@@ -356,3 +356,50 @@ def test_forward_with_packed_copy_equals_forward_then_pack(N, C, spatial, dtype,
     assert torch.equal(packed, packed_ref)
     y2, none1, none2 = ext_bf.hip_batch_norm_forward_apply(x, ws)
     assert torch.equal(y2, y_ref) and none1 is None and none2 is None
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("N,C,H", [(8, 64, 8), (4, 256, 4), (32, 16, 4), (6, 128, 8)])
+def test_apply_with_the_relu_folded_in_equals_apply_then_relu(dtype, N, C, H):
+    """actnn_batch_norm_forward_apply_relu against actnn_batch_norm_forward_apply followed by
+    actnn_relu_forward_minmax on the stored result: output, mask words, group min / max, scale and
+    the packed stream bit for bit, over several widths and a sample boundary inside a block."""
+    from actnn_amd import _lib
+    import actnn_amd.cpp_extension.backward_func as bf
+    import actnn_amd.cpp_extension.quantization as ext_q
+    lib = _lib.load()
+    g = torch.Generator(device=DEV).manual_seed(N * C + H)
+    x = (torch.randn(N, C, H, H, device=DEV, generator=g) * 1.5).to(dtype).contiguous(memory_format=torch.channels_last)
+    w = torch.rand(C, device=DEV, generator=g) * 2 - 0.5
+    b = torch.randn(C, device=DEV, generator=g)
+    ws, mean, invstd, mn, mx = bf.hip_batch_norm_forward_stats(x, w, b, None, None, 0.1, 1e-5)
+    widths = torch.randint(1, 9, (N,), generator=torch.Generator().manual_seed(1), dtype=torch.int32)
+    bits = ext_q.attach_bits_host(widths.to(DEV), widths)
+    torch.cuda.manual_seed(5)
+    y, packed, scale = bf.hip_batch_norm_forward_apply(x, ws, bits, mn, mx)
+    from actnn_amd.utils import memory_order
+    z_ref, mask_ref, zmn_ref, zmx_ref = ext_q.relu_forward_minmax(memory_order(y).contiguous())
+    total, prefix = ext_q._bits_info(bits)
+    HW, n = H * H, x.numel()
+    out = torch.empty_like(x)
+    packed2, scale2 = torch.empty_like(packed), torch.empty_like(scale)
+    mask = torch.empty(ext_q.mask_words(n), dtype=torch.int32, device=DEV)
+    zmn, zmx = torch.empty(n // 256, dtype=dtype, device=DEV), torch.empty(n // 256, dtype=dtype, device=DEV)
+    torch.cuda.manual_seed(5)
+    seed, offset = ext_q.g.philox_args(x.device)
+    rc = lib.actnn_batch_norm_forward_apply_relu(
+        x.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel() * 4, bits.data_ptr(), prefix.data_ptr(), mn.data_ptr(),
+        mx.data_ptr(), scale2.data_ptr(), packed2.data_ptr(), seed, offset, mask.data_ptr(), zmn.data_ptr(),
+        zmx.data_ptr(), N, C, HW, ext_q.g.DTYPE_CODE[dtype], 1, None)
+    assert rc == 0
+    assert torch.equal(memory_order(out), z_ref) and torch.equal(mask, mask_ref)
+    assert torch.equal(zmn, zmn_ref) and torch.equal(zmx, zmx_ref)
+    assert torch.equal(packed2, packed) and torch.equal(scale2, scale)
+    # refused: default layout, fp32, C that does not divide 256, elements not a multiple of 2048
+    args = lambda **k: (x.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel() * 4, bits.data_ptr(), prefix.data_ptr(),
+                        mn.data_ptr(), mx.data_ptr(), scale2.data_ptr(), packed2.data_ptr(), seed, offset,
+                        k.get("mask", mask.data_ptr()), zmn.data_ptr(), zmx.data_ptr(), k.get("N", N), k.get("C", C), HW,
+                        k.get("dtype", ext_q.g.DTYPE_CODE[dtype]), k.get("cl", 1), None)
+    for bad in (dict(cl=0), dict(dtype=0), dict(mask=None), dict(C=C * 3), dict(N=N + 1) if (C * HW) % 2048 else dict(mask=None)):
+        assert lib.actnn_batch_norm_forward_apply_relu(*args(**bad)) != 0, bad
+    torch.cuda.synchronize()

@@ -922,3 +922,53 @@ def test_fixed_width_batch_norm_takes_the_fused_passes(channels_last):
     xr = x.detach().float().requires_grad_(True)
     (gx,) = torch.autograd.grad(ref(xr), xr, g.float())
     assert (grads1[0].float() - gx).abs().max() <= 0.05 * gx.abs().max() + 0.05
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("channels,size,folded", [(64, 8, True), (128, 4, True), (256, 8, True), (32, 8, True),
+                                                  (512, 4, False), (96, 8, False)])
+def test_relu_folded_into_the_batch_norm_pass_equals_the_two_layers(dtype, channels, size, folded):
+    """layers.bn_relu hands a converted batch norm and the ReLU after it over together: where the
+    shape allows (channels-last, 16-bit, C a divisor of 256) the ReLU runs inside the normalise +
+    pack pass.  Output, group min / max left for the next layer, running statistics, the compressed
+    input and every gradient are those of the two layers, bit for bit; other shapes take the two
+    layers."""
+    from actnn_amd import ops
+    from actnn_amd.layers import QBatchNorm2d, QReLU, bn_relu, known_group_minmax
+    calls = []
+    real = ops.batch_norm_relu.forward
+
+    def run(fold):
+        config.reset(); QScheme.reset(); QBNScheme.reset()
+        set_optimization_level("L3")
+        config.fused_bn_relu = fold
+        torch.manual_seed(3)
+        bn, relu = QBatchNorm2d(channels).to(DEV).train(), QReLU()
+        with torch.no_grad():
+            bn.weight.uniform_(-1.0, 1.5)
+            bn.bias.normal_()
+        g = torch.Generator(device=DEV).manual_seed(9)
+        x = (torch.randn(16, channels, size, size, device=DEV, generator=g) * 2 + 0.3).to(dtype)
+        x = x.contiguous(memory_format=torch.channels_last).requires_grad_(True)
+        go = torch.randn(16, channels, size, size, device=DEV, generator=g).to(dtype).contiguous(memory_format=torch.channels_last)
+        torch.cuda.manual_seed(21)
+        out = bn_relu(bn, relu, x)
+        known = known_group_minmax(out)
+        out.backward(go)
+        return [out.detach(), x.grad, bn.weight.grad, bn.bias.grad, bn.running_mean.clone(), bn.running_var.clone()] + \
+               (list(known) if known is not None else [])
+
+    def spy(*a, **k):
+        calls.append(1)
+        return real(*a, **k)
+
+    ops.batch_norm_relu.forward = staticmethod(spy)
+    try:
+        two, one = run(False), run(True)
+    finally:
+        ops.batch_norm_relu.forward = staticmethod(real)
+    assert len(calls) == (1 if folded else 0)
+    assert len(two) == len(one)
+    for i, (u, v) in enumerate(zip(two, one)):
+        assert torch.equal(u, v), i
+    assert one[0].is_contiguous(memory_format=torch.channels_last) and float(one[0].min()) == 0.0
