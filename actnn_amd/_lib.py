@@ -93,6 +93,8 @@ SIGNATURES = {
                                        c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
     "actnn_batch_norm_backward_packed": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp,
                                          c_vp, c_vp, c_i64, c_vp, c_i64, c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
+    "actnn_batch_norm_backward_packed_relu": [c_vp] * 14 + [c_i64, c_vp, c_i64, c_i64, c_i64, c_i64, c_i32, c_i32,
+                                              c_vp],
     "actnn_batch_norm_backward": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_vp, c_i64,
                                   c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
     "actnn_batch_norm_backward_sumsq_entries": [c_i64, c_i64, c_i64, c_i32, c_i32],

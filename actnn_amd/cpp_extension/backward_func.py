@@ -318,9 +318,12 @@ def hip_batch_norm_backward_packed_applies(shape, quantized, grad_output, weight
             and all(_f32_or_none(t) for t in (weight, save_mean, save_invstd)))
 
 
-def hip_batch_norm_backward_packed(shape, quantized, grad_output, weight, save_mean, save_invstd, sumsq=False):
+def hip_batch_norm_backward_packed(shape, quantized, grad_output, weight, save_mean, save_invstd, sumsq=False,
+                                   relu_mask=None):
     """-> (grad_input, grad_weight, grad_bias); the saved input is decoded inside the kernels.
-    `sumsq` as in hip_batch_norm_backward."""
+    `sumsq` as in hip_batch_norm_backward.  `relu_mask`: `grad_output` is the gradient of a ReLU the
+    batch norm's output went through, and the passes apply that ReLU's mask as they read it
+    (shapes of hip_batch_norm_relu_applies)."""
     from .quantization import _bits_info
     q_input, q_bits, q_scale, q_min = quantized
     channels_last = getattr(quantized, "memory_format", None) is not None
@@ -341,12 +344,20 @@ def hip_batch_norm_backward_packed(shape, quantized, grad_output, weight, save_m
     grad_weight = torch.empty(C, dtype=torch.float32, device=dev)
     grad_bias = torch.empty(C, dtype=torch.float32, device=dev)
     with _glue.on_device(dev):
-        _glue._lib.check(lib.actnn_batch_norm_backward_packed(
-            q_input.data_ptr(), q_bits.data_ptr(), prefix.data_ptr(), q_scale.data_ptr(), q_min.data_ptr(),
-            grad_output.data_ptr(), _ptr(weight), save_mean.data_ptr(), save_invstd.data_ptr(),
-            grad_input.data_ptr(), grad_weight.data_ptr(), grad_bias.data_ptr(), ws.data_ptr(), ws_bytes,
-            ws.data_ptr() + ws_bytes if entries else None, entries,
-            N, C, HW, code, int(channels_last), _glue.stream_ptr(dev)), "batch_norm_backward_packed")
+        if relu_mask is not None:
+            _glue._lib.check(lib.actnn_batch_norm_backward_packed_relu(
+                q_input.data_ptr(), q_bits.data_ptr(), prefix.data_ptr(), q_scale.data_ptr(), q_min.data_ptr(),
+                grad_output.data_ptr(), relu_mask.data_ptr(), _ptr(weight), save_mean.data_ptr(),
+                save_invstd.data_ptr(), grad_input.data_ptr(), grad_weight.data_ptr(), grad_bias.data_ptr(),
+                ws.data_ptr(), ws_bytes, ws.data_ptr() + ws_bytes if entries else None, entries,
+                N, C, HW, code, int(channels_last), _glue.stream_ptr(dev)), "batch_norm_backward_packed_relu")
+        else:
+            _glue._lib.check(lib.actnn_batch_norm_backward_packed(
+                q_input.data_ptr(), q_bits.data_ptr(), prefix.data_ptr(), q_scale.data_ptr(), q_min.data_ptr(),
+                grad_output.data_ptr(), _ptr(weight), save_mean.data_ptr(), save_invstd.data_ptr(),
+                grad_input.data_ptr(), grad_weight.data_ptr(), grad_bias.data_ptr(), ws.data_ptr(), ws_bytes,
+                ws.data_ptr() + ws_bytes if entries else None, entries,
+                N, C, HW, code, int(channels_last), _glue.stream_ptr(dev)), "batch_norm_backward_packed")
     if entries:
         _leave_sumsq(grad_input, ws[ws_bytes // 4:])
     return grad_input, grad_weight, grad_bias

@@ -307,15 +307,30 @@ template <typename T> ACTNN_DEV uint32_t relu_word(uint32_t w, uint32_t& keep, f
   keep = (k0 ? 1u : 0u) | (k1 ? 2u : 0u);
   return (k0 ? w & 0x0000ffffu : 0u) | (k1 ? w & 0xffff0000u : 0u);
 }
-// Keep bits of four 512-element blocks (per lane: 8 bits for each block, the lane's 8 elements) ->
-// this lane's mask word: lane 2p + h holds word p % 16 of block 2h + p / 16.
-ACTNN_DEV uint32_t mask_word_of_rows(const uint32_t (&m)[4], uint32_t lane) {
-  const bool odd = lane & 1u;
-  const uint32_t ab = m[0] | (m[1] << 16), cd = m[2] | (m[3] << 16);
-  const uint32_t recv = lane_xor<1>(odd ? ab : cd);
-  const uint32_t mine = odd ? cd : ab;
-  const uint32_t row = odd ? (recv | (mine << 8)) : (mine | (recv << 8));
-  return transpose32_x2(row, lane);
+// The other direction: a backward pass whose incoming gradient is that of a ReLU's output takes the
+// ReLU's mask along and zeroes what the ReLU's own backward pass would have zeroed, instead of reading
+// a masked copy.  Keep bits of the wave's next four steps (a step of a block is 2048 elements: the
+// wave's blocks are 4 apart), one word per lane and two bit transposes for the four.
+struct ReluRows {
+  const int32_t* words;
+  int64_t blocks;          // 512-element blocks of the tensor
+  ACTNN_DEV void load(int64_t rb, int64_t C, uint32_t (&m)[4]) const {
+    const uint32_t lane = threadIdx.x & 63u;
+    const int slot = 2 * (int)(lane & 1u) + (int)(lane >> 5);
+    const int64_t block = ((rb * C) >> 9) + (threadIdx.x >> 6) + 4 * slot;
+    const uint32_t w = block < blocks ? (uint32_t)words[block * 16 + ((lane >> 1) & 15u)] : 0u;
+    word_to_rows(w, lane, m);
+  }
+};
+// the chunk's eight 16-bit values with those zeroed whose keep bit (bit i of `row` for value i) is 0
+ACTNN_DEV u32x4 keep_chunk(const u32x4& d, uint32_t row) {
+  uint32_t w[4] = {d.x, d.y, d.z, d.w};
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const uint32_t a = 0u - ((row >> (2 * q)) & 1u), b = 0u - ((row >> (2 * q + 1)) & 1u);
+    w[q] &= (a & 0x0000ffffu) | (b << 16);
+  }
+  return u32x4{w[0], w[1], w[2], w[3]};
 }
 
 ACTNN_DEV void leave_wave_sum(float* table, float v) {
@@ -978,16 +993,17 @@ template <int E> ACTNN_DEV RowTile row_tile(int64_t C, int tpr, int R, int tile)
 
 // Waves per SIMD the reduce pass is compiled for: the plain statistics pass fits 8 (64 registers),
 // with the group min/max or the gradient 7, with the decoder of a packed input 5.
-template <bool BWD, bool MINMAX, typename XS> constexpr int cl_reduce_waves() {
-  return XS::kInFlight == 2 ? 5 : (BWD || MINMAX) ? 7 : 8;
+template <bool BWD, bool MINMAX, typename XS, bool MASKED = false> constexpr int cl_reduce_waves() {
+  return MASKED ? 4 : XS::kInFlight == 2 ? 5 : (BWD || MINMAX) ? 7 : 8;     // (with the ReLU's mask rows: 4)
 }
-template <typename T, bool BWD, bool MINMAX, bool NT, typename XS>
-__global__ __launch_bounds__(kThreads, (cl_reduce_waves<BWD, MINMAX, XS>())) void bn_cl_reduce_kernel(
+template <typename T, bool BWD, bool MINMAX, bool NT, typename XS, bool MASKED = false>
+__global__ __launch_bounds__(kThreads, (cl_reduce_waves<BWD, MINMAX, XS, MASKED>())) void bn_cl_reduce_kernel(
     XS xs, const T* __restrict__ dy, float* __restrict__ part, T* __restrict__ mn, T* __restrict__ mx,
-    int64_t P, int64_t C, int tpr, int R, int64_t ppb, int tiles, int nsplit) {
+    int64_t P, int64_t C, int tpr, int R, int64_t ppb, int tiles, int nsplit, ReluRows relu = ReluRows{}) {
   constexpr int E = Chunk<T>::kElems;
   constexpr int PD = Chunk<T>::kPerDword;
   constexpr int U = XS::kInFlight;
+  static_assert(!MASKED || (BWD && U == 2 && sizeof(T) == 2), "the ReLU mask goes with a 16-bit gradient, two loads in flight");
   __shared__ float s_part[kThreads * 2 * E];
   // Blocks are numbered so that consecutive block rows of a column tile run on one XCD.  A line of the
   // table of partial sums holds the values of 16 consecutive block rows; dealt round-robin, those rows
@@ -1041,7 +1057,32 @@ __global__ __launch_bounds__(kThreads, (cl_reduce_waves<BWD, MINMAX, XS>())) voi
     }
   };
 
-  if (t.active) {
+  if constexpr (MASKED) {
+    // (every step of a block is whole here - the launcher sees to it - and all lanes are active)
+    auto two = [&](int64_t rb, uint32_t row0, uint32_t row1) __attribute__((always_inline)) {
+      const typename XS::Raw rx0 = xs.fetch(rb), rx1 = xs.fetch(rb + R);
+      const u32x4 ud0 = dy_at(rb), ud1 = dy_at(rb + R);
+      accumulate(xs.decode(rx0), keep_chunk(ud0, row0), rb);
+      accumulate(xs.decode(rx1), keep_chunk(ud1, row1), rb + R);
+    };
+    auto one = [&](int64_t rb, uint32_t row) __attribute__((always_inline)) {
+      const typename XS::Raw rx = xs.fetch(rb);
+      accumulate(xs.decode(rx), keep_chunk(dy_at(rb), row), rb);
+    };
+    int64_t rb = p0;
+    uint32_t m[4];
+    for (; rb + (int64_t)4 * R <= p1; rb += (int64_t)4 * R) {
+      relu.load(rb, C, m);
+      two(rb, m[0], m[1]);
+      two(rb + (int64_t)2 * R, m[2], m[3]);
+    }
+    if (rb < p1) {
+      relu.load(rb, C, m);
+      one(rb, m[0]);
+      if (rb + R < p1) one(rb + R, m[1]);
+      if (rb + (int64_t)2 * R < p1) one(rb + (int64_t)2 * R, m[2]);
+    }
+  } else if (t.active) {
     int64_t rb = p0;
     // whole iterations: every row rb + u * R + r of the U loads lies below p1
     for (; rb + (int64_t)U * R <= p1; rb += (int64_t)U * R) {
@@ -1087,13 +1128,15 @@ __global__ __launch_bounds__(kThreads, (cl_reduce_waves<BWD, MINMAX, XS>())) voi
 template <typename T, bool BWD, bool PACK, typename XS, bool RELU = false>
 __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
     XS xs, const T* __restrict__ dy, const float* __restrict__ coef, T* __restrict__ out,
-    int64_t P, int64_t C, int tpr, int R, int64_t ppb, PackSink ps, FastDiv by_hw) {
+    int64_t P, int64_t C, int tpr, int R, int64_t ppb, PackSink ps, FastDiv by_hw, ReluRows relu = ReluRows{}) {
+  // (RELU with BWD: the gradient that comes in is masked by `relu` as it is read)
+  static_assert(!(RELU && BWD) || (XS::kInFlight == 2 && sizeof(T) == 2), "the ReLU mask goes with a 16-bit gradient, two loads in flight");
   constexpr int E = Chunk<T>::kElems;
   constexpr int PD = Chunk<T>::kPerDword;
   constexpr int NC = BWD ? 3 : 2;
   constexpr int U = XS::kInFlight;
   static_assert(!(PACK && BWD), "the packed copy is made by the forward pass");
-  static_assert(!RELU || (PACK && sizeof(T) == 2), "the ReLU is folded into the packing pass of 16-bit tensors");
+  static_assert(!RELU || BWD || (PACK && sizeof(T) == 2), "the ReLU is folded into the packing pass of 16-bit tensors");
   // The sample that holds the row of the last pack: its width, its first word in the stream and its
   // first row / group.  A thread stays inside one sample for many rows, so these are looked up only
   // when a row leaves it, and a chunk's place in the stream is 32-bit arithmetic on top of them (rows,
@@ -1243,7 +1286,7 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
       }
     };
     auto leave_mask = [&](int64_t ru_first, const uint32_t (&rows)[4], int count) __attribute__((always_inline)) {
-      const uint32_t word = mask_word_of_rows(rows, lane);
+      const uint32_t word = rows_to_word(rows, lane);
       const int slot = 2 * (int)(lane & 1u) + (int)(lane >> 5);
       const int64_t block = ((ru_first * C) >> 9) + (threadIdx.x >> 6) + 4 * slot;
       if (slot < count) ps.relu_mask[block * 16 + ((lane >> 1) & 15u)] = (int32_t)word;
@@ -1315,6 +1358,30 @@ __global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
           pack_one(ux, rw, ru0, j);
         }
       }
+    }
+  } else if constexpr (RELU && BWD) {
+    auto two = [&](int64_t rb, uint32_t row0, uint32_t row1) __attribute__((always_inline)) {
+      const typename XS::Raw rx0 = xs.fetch(rb), rx1 = xs.fetch(rb + R);
+      const u32x4 ud0 = dy_at(rb), ud1 = dy_at(rb + R);
+      store_out(out_at(rb), apply(xs.decode(rx0), keep_chunk(ud0, row0)));
+      store_out(out_at(rb + R), apply(xs.decode(rx1), keep_chunk(ud1, row1)));
+    };
+    auto one = [&](int64_t rb, uint32_t row) __attribute__((always_inline)) {
+      const typename XS::Raw rx = xs.fetch(rb);
+      store_out(out_at(rb), apply(xs.decode(rx), keep_chunk(dy_at(rb), row)));
+    };
+    int64_t rb = p0;
+    uint32_t m[4];
+    for (; rb + (int64_t)4 * R <= p1; rb += (int64_t)4 * R) {
+      relu.load(rb, C, m);
+      two(rb, m[0], m[1]);
+      two(rb + (int64_t)2 * R, m[2], m[3]);
+    }
+    if (rb < p1) {
+      relu.load(rb, C, m);
+      one(rb, m[0]);
+      if (rb + R < p1) one(rb + R, m[1]);
+      if (rb + (int64_t)2 * R < p1) one(rb + (int64_t)2 * R, m[2]);
     }
   } else {
   int64_t rb = p0;
@@ -1519,23 +1586,23 @@ ClRows cl_reduce_rows(const Plan& pl, int waves) {
   return ClRows{ppb, (int)((pl.P + ppb - 1) / ppb)};
 }
 // -> the block rows of the table it leaves
-template <typename T, bool BWD, bool MINMAX, bool NT, typename XS>
+template <typename T, bool BWD, bool MINMAX, bool NT, typename XS, bool MASKED = false>
 int launch_cl_reduce(const Plan& pl, const XS& xs, const void* dy, float* part, void* mn, void* mx,
-                     int64_t C, hipStream_t s) {
-  const ClRows rows = cl_reduce_rows(pl, cl_reduce_waves<BWD, MINMAX, XS>());
+                     int64_t C, hipStream_t s, const ReluRows& relu = ReluRows{}) {
+  const ClRows rows = cl_reduce_rows(pl, cl_reduce_waves<BWD, MINMAX, XS, MASKED>());
   const dim3 grid(xcd_grid((int64_t)pl.tiles * rows.nsplit)), blk(kThreads);
-  bn_cl_reduce_kernel<T, BWD, MINMAX, NT, XS><<<grid, blk, 0, s>>>(
+  bn_cl_reduce_kernel<T, BWD, MINMAX, NT, XS, MASKED><<<grid, blk, 0, s>>>(
       xs, static_cast<const T*>(dy), part, static_cast<T*>(mn), static_cast<T*>(mx), pl.P, C, pl.tpr, pl.R, rows.ppb,
-      pl.tiles, rows.nsplit);
+      pl.tiles, rows.nsplit, relu);
   return rows.nsplit;
 }
 template <typename T, bool BWD, bool PACK, typename XS, bool RELU = false>
 void launch_cl_apply(const Plan& pl, const XS& xs, const void* dy, const float* coef, void* out, int64_t C,
-                     const PackSink& ps, hipStream_t s) {
+                     const PackSink& ps, hipStream_t s, const ReluRows& relu = ReluRows{}) {
   const dim3 grid((unsigned)pl.tiles, (unsigned)pl.nsplit_apply), blk(kThreads);
   bn_cl_apply_kernel<T, BWD, PACK, XS, RELU><<<grid, blk, 0, s>>>(
       xs, static_cast<const T*>(dy), coef, static_cast<T*>(out), pl.P, C, pl.tpr, pl.R, pl.ppb_apply, ps,
-      FastDiv((uint32_t)(pl.F / C)));
+      FastDiv((uint32_t)(pl.F / C)), relu);
 }
 
 template <typename T>
@@ -1612,10 +1679,25 @@ int forward_apply_t(const Plan& pl, const void* x, void* y, const float* ws, con
 template <typename T, typename XS>
 int backward_t(const Plan& pl, const XS& xs, const void* dy, const float* weight, const float* save_mean,
                const float* save_invstd, void* dx, float* dweight, float* dbias, float* ws, int64_t N,
-               int64_t C, int64_t HW, float* sumsq, hipStream_t s, bool eval = false) {
+               int64_t C, int64_t HW, float* sumsq, hipStream_t s, bool eval = false,
+               const ReluRows* relu = nullptr) {
   float* part = ws;
   float* coef = ws + pl.part_floats;
   int nsplit = pl.nsplit;
+  if constexpr (XS::kRows && XS::kInFlight == 2 && sizeof(T) == 2) {
+    if (relu) {        // dy is the gradient of a ReLU's output: masked as it is read, in both passes
+      if (pl.big) nsplit = launch_cl_reduce<T, true, false, true, XS, true>(pl, xs, dy, part, nullptr, nullptr, C, s, *relu);
+      else nsplit = launch_cl_reduce<T, true, false, false, XS, true>(pl, xs, dy, part, nullptr, nullptr, C, s, *relu);
+      bn_backward_finalize_kernel<<<dim3((unsigned)((C + kWaves - 1) / kWaves)), dim3(kThreads), 0, s>>>(
+          part, weight, save_mean, save_invstd, dweight, dbias, coef, N, C, HW, pl.L, nsplit, pl.slots, eval);
+      if (dx) {
+        PackSink extra{};
+        extra.sumsq = sumsq;
+        launch_cl_apply<T, true, false, XS, true>(pl, xs, dy, coef, dx, C, extra, s, *relu);
+      }
+      ACTNN_RETURN_LAUNCH_STATUS();
+    }
+  }
   if constexpr (XS::kRows) {
     if (pl.big) nsplit = launch_cl_reduce<T, true, false, true>(pl, xs, dy, part, nullptr, nullptr, C, s);
     else nsplit = launch_cl_reduce<T, true, false, false>(pl, xs, dy, part, nullptr, nullptr, C, s);
@@ -1674,15 +1756,19 @@ template <typename T>
 int backward_packed(const Plan& pl, const int32_t* packed, const int32_t* bits, const int32_t* prefix,
                     const void* scale, const void* mn, const void* dy, const float* weight,
                     const float* save_mean, const float* save_invstd, void* dx, float* dweight,
-                    float* dbias, float* ws, int64_t N, int64_t C, int64_t HW, float* sumsq, hipStream_t s) {
+                    float* dbias, float* ws, int64_t N, int64_t C, int64_t HW, float* sumsq, hipStream_t s,
+                    const int32_t* relu_mask = nullptr) {
   const PackedInput<T> in{packed, bits, prefix, static_cast<const T*>(scale), static_cast<const T*>(mn),
                           pl.F / 256, 0, 0u, false};
   if (pl.channels_last) {
     // (32-bit positions inside a sample and over the tensor's groups)
     if (C * HW >= ((int64_t)1 << 32) || N * (pl.F / 256) >= 0x7fffffffLL) return ACTNN_EINVAL;
     const PackedRows<T> xs{in, C, (uint32_t)HW, FastDiv((uint32_t)HW), 0u, 0u, 0u, 0u, 1, packed};
-    return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
+    const ReluRows relu{relu_mask, (N * pl.F) >> 9};
+    return backward_t<T>(pl, xs, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s,
+                         false, relu_mask ? &relu : nullptr);
   }
+  if (relu_mask) return ACTNN_EINVAL;
   return backward_t<T>(pl, in, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
 }
 
@@ -1971,4 +2057,33 @@ extern "C" int actnn_batch_norm_backward_packed(const int32_t* packed, const int
   if (dtype == ACTNN_F32)
     return backward_packed<float>(pl, packed, bits, prefix, scale, mn, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
   return backward_packed<bf16_t>(pl, packed, bits, prefix, scale, mn, dy, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s);
+}
+
+// The same for a batch norm whose output went through a ReLU: `grad_out` is the gradient of the
+// ReLU's output and `relu_mask` the ReLU's mask; both passes zero what actnn_relu_backward would
+// have zeroed as they read, so the masked gradient is never written.  Shapes as
+// actnn_batch_norm_forward_apply_relu takes them.
+extern "C" int actnn_batch_norm_backward_packed_relu(const int32_t* packed, const int32_t* bits,
+                                                     const int32_t* prefix, const void* scale, const void* mn,
+                                                     const void* grad_out, const int32_t* relu_mask,
+                                                     const float* weight, const float* save_mean,
+                                                     const float* save_invstd, void* dx, float* dweight,
+                                                     float* dbias, void* workspace, int64_t workspace_bytes,
+                                                     float* sumsq, int64_t sumsq_entries, int64_t N, int64_t C,
+                                                     int64_t HW, int dtype, int channels_last, void* stream) {
+  using namespace actnn;
+  if (dtype != ACTNN_F16 && dtype != ACTNN_BF16) return ACTNN_EDTYPE;
+  Plan pl;
+  if (!channels_last || !make_plan(N, C, HW, dtype, channels_last, pl) || pl.any_shape || !pl.groups_align) return ACTNN_EINVAL;
+  if (C > 256 || 256 % C != 0 || (N * pl.F) % 2048 != 0 || pl.P > 0x7fffffffLL) return ACTNN_EINVAL;
+  if (sumsq && (!dx || sumsq_entries < apply_waves(pl))) return ACTNN_EINVAL;
+  if (!packed || !bits || !prefix || !scale || !mn || !grad_out || !relu_mask || !save_mean || !save_invstd || !workspace)
+    return ACTNN_EINVAL;
+  if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
+  if (!aligned16(grad_out) || (dx && !aligned16(dx)) || !aligned16(workspace)) return ACTNN_EALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float* ws = static_cast<float*>(workspace);
+  if (dtype == ACTNN_F16)
+    return backward_packed<__half>(pl, packed, bits, prefix, scale, mn, grad_out, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s, relu_mask);
+  return backward_packed<bf16_t>(pl, packed, bits, prefix, scale, mn, grad_out, weight, save_mean, save_invstd, dx, dweight, dbias, ws, N, C, HW, sumsq, s, relu_mask);
 }

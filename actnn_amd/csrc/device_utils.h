@@ -429,6 +429,35 @@ ACTNN_DEV Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t 
   return Philox4{c0, c1, c2, c3};
 }
 
+// ------------------------------------------------------------------ 1-bit masks of 16-bit tensors
+// A wave that holds four 512-element blocks of a tensor, lane l elements 8l..8l+7 of each, and the
+// blocks' 64 mask words (element 16j + k of a block is bit j of its word k), lane 2p + h the word
+// p % 16 of block 2h + p / 16: lane pairs swap their 8-bit halves (one DPP move) so that the even
+// lanes hold the rows of blocks A|B and the odd lanes those of C|D, and two interleaved 32x32 bit
+// transposes turn rows into words or back.
+// rows (per lane: 8 keep bits for each of the 4 blocks) -> this lane's mask word
+ACTNN_DEV uint32_t rows_to_word(const uint32_t (&m)[4], uint32_t lane) {
+  const bool odd = lane & 1u;
+  const uint32_t ab = m[0] | (m[1] << 16), cd = m[2] | (m[3] << 16);
+  const uint32_t recv = lane_xor<1>(odd ? ab : cd);           // the half-row the partner computed for me
+  const uint32_t mine = odd ? cd : ab;
+  const uint32_t row = odd ? (recv | (mine << 8)) : (mine | (recv << 8));
+  return transpose32_x2(row, lane);
+}
+// inverse: this lane's mask word -> 8 keep bits for each of the 4 blocks
+ACTNN_DEV void word_to_rows(uint32_t w, uint32_t lane, uint32_t (&m)[4]) {
+  const bool odd = lane & 1u;
+  const uint32_t row = transpose32_x2(w, lane);                // even: row of A|B, odd: row of C|D
+  const uint32_t other = lane_xor<1>(row);
+  const uint32_t ab = odd ? other : row, cd = odd ? row : other;
+  const int sh = odd ? 8 : 0;
+  m[0] = (ab >> sh) & 0xffu;
+  m[1] = (ab >> (16 + sh)) & 0xffu;
+  m[2] = (cd >> sh) & 0xffu;
+  m[3] = (cd >> (16 + sh)) & 0xffu;
+}
+
+
 // ------------------------------------------------------------------ rounding noise
 // The stochastic rounding draws one uniform integer per element; elements are numbered as they lie
 // in memory and taken in octets (8 consecutive elements).  How many bits an element gets follows

@@ -139,28 +139,6 @@ __global__ __launch_bounds__(kThreads) void mask_backward_kernel(const T* __rest
 constexpr int kTileElems = 4 * kMaskBlock;        // elements per wave and iteration
 constexpr int kTilesPerBlock = kThreads / 64;
 
-// rows (per lane: 8 keep bits for each of the 4 blocks) -> this lane's transposed mask word
-ACTNN_DEV uint32_t rows_to_word(const uint32_t (&m)[4], uint32_t lane) {
-  const bool odd = lane & 1u;
-  const uint32_t ab = m[0] | (m[1] << 16), cd = m[2] | (m[3] << 16);
-  const uint32_t recv = lane_xor<1>(odd ? ab : cd);           // the half-row the partner computed for me
-  const uint32_t mine = odd ? cd : ab;
-  const uint32_t row = odd ? (recv | (mine << 8)) : (mine | (recv << 8));
-  return transpose32_x2(row, lane);
-}
-// inverse: this lane's mask word -> 8 keep bits for each of the 4 blocks
-ACTNN_DEV void word_to_rows(uint32_t w, uint32_t lane, uint32_t (&m)[4]) {
-  const bool odd = lane & 1u;
-  const uint32_t row = transpose32_x2(w, lane);                // even: row of A|B, odd: row of C|D
-  const uint32_t other = lane_xor<1>(row);
-  const uint32_t ab = odd ? other : row, cd = odd ? row : other;
-  const int sh = odd ? 8 : 0;
-  m[0] = (ab >> sh) & 0xffu;
-  m[1] = (ab >> (16 + sh)) & 0xffu;
-  m[2] = (cd >> sh) & 0xffu;
-  m[3] = (cd >> (16 + sh)) & 0xffu;
-}
-
 // MINMAX: also write the minimum and maximum of every group of 256 consecutive outputs (the lower
 // and upper 32 lanes of each load own one group each) - what actnn_minimax returns for the output
 // viewed as rows of 256, for a consumer that quantises it next.

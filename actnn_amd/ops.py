@@ -564,8 +564,17 @@ class batch_norm(Function):
         return _batch_norm_backward(ctx, grad_output)
 
 
-def _batch_norm_backward(ctx, grad_output):
+def _batch_norm_backward(ctx, grad_output, relu_mask=None):
+    """`relu_mask`: the mask of a ReLU the batch norm's output went through (batch_norm_relu);
+    `grad_output` is then the gradient of the ReLU's output, masked by the batch-norm passes as they
+    read it where they can, else by the ReLU's own backward pass first."""
     quantized, weight, running_mean, running_var, save_mean, save_var, training, eps, reserve = ctx.saved
+
+    def relu_backward_first(grad):
+        fmt = getattr(quantized, "memory_format", None)
+        grad = ext_quantization.relu_backward(memory_order(grad.contiguous(memory_format=fmt)), relu_mask)
+        return logical_order(grad, fmt)
+
     if (training and config.compress_activation and not config.simulate
             and config.group_size == 256 and config.fused_bn_backward):
         if config.swap and isinstance(quantized[0], torch.Tensor) and not quantized[0].is_cuda:
@@ -577,13 +586,18 @@ def _batch_norm_backward(ctx, grad_output):
         if ext_backward_func.hip_batch_norm_backward_packed_applies(
                 ctx.other_args, quantized, grad_output, weight, save_mean, save_var):
             # the kernels decode the saved input from its bit stream: no full-precision copy
+            # (batch_norm_relu exists only for shapes whose passes take the mask)
+            if relu_mask is not None and not config.fused_bn_relu_backward:
+                grad_output, relu_mask = relu_backward_first(grad_output), None
             grads = ext_backward_func.hip_batch_norm_backward_packed(
                 ctx.other_args, quantized, grad_output, weight, save_mean, save_var,
-                sumsq=_leaves_grad_sqnorm())
+                sumsq=_leaves_grad_sqnorm(), relu_mask=relu_mask)
             del quantized, ctx.saved
             if ctx.scheme:
                 ctx.scheme.if_allocate_perlayer()
             return grads[0], None, None, grads[1], grads[2], None, None, None, None
+    if relu_mask is not None:
+        grad_output = relu_backward_first(grad_output)
     input = dequantize_activation(quantized, ctx.other_args)
     memory_format = getattr(quantized, "memory_format", None) or torch.contiguous_format
     del quantized, ctx.saved
@@ -631,10 +645,8 @@ class batch_norm_relu(Function):
     def backward(ctx, grad_output, _grad_mn, _grad_mx):
         if grad_output is None:
             return (None,) * 10
-        fmt = ctx.saved[0].memory_format
-        grad = ext_quantization.relu_backward(memory_order(grad_output.contiguous(memory_format=fmt)), ctx.relu_mask)
-        ctx.relu_mask = None
-        return _batch_norm_backward(ctx, logical_order(grad, fmt)) + (None,)
+        mask, ctx.relu_mask = ctx.relu_mask, None
+        return _batch_norm_backward(ctx, grad_output, mask) + (None,)
 
 
 class adaptive_avg_pool2d(Function):

@@ -418,6 +418,20 @@ int actnn_batch_norm_backward_packed(const int32_t* packed, const int32_t* bits,
                                      float* dbias, void* workspace, int64_t workspace_bytes,
                                      float* sumsq, int64_t sumsq_entries, int64_t N, int64_t C,
                                      int64_t HW, int dtype, int channels_last, void* stream);
+/* The same for a batch norm whose output went through a ReLU (actnn_batch_norm_forward_apply_relu):
+ * grad_out is the gradient of the ReLU's output and relu_mask the ReLU's mask; both passes zero what
+ * actnn_relu_backward would have zeroed as they read, so the masked gradient is never written and
+ * the results equal actnn_relu_backward followed by actnn_batch_norm_backward_packed bit for bit.
+ * Shapes as actnn_batch_norm_forward_apply_relu takes them (replaces the same reference lines as
+ * the two calls: quantization.cc:106-124, ops.py:472-502). */
+int actnn_batch_norm_backward_packed_relu(const int32_t* packed, const int32_t* bits, const int32_t* prefix,
+                                          const void* scale, const void* mn, const void* grad_out,
+                                          const int32_t* relu_mask, const float* weight,
+                                          const float* save_mean, const float* save_invstd, void* dx,
+                                          float* dweight, float* dbias, void* workspace,
+                                          int64_t workspace_bytes, float* sumsq, int64_t sumsq_entries,
+                                          int64_t N, int64_t C, int64_t HW, int dtype, int channels_last,
+                                          void* stream);
 
 /* Plain device-to-device streaming copy of `bytes` bytes (16-byte aligned pointers and
  * size); used by the benchmark to calibrate bandwidth counters.  No reference counterpart. */

@@ -403,3 +403,35 @@ def test_apply_with_the_relu_folded_in_equals_apply_then_relu(dtype, N, C, H):
     for bad in (dict(cl=0), dict(dtype=0), dict(mask=None), dict(C=C * 3), dict(N=N + 1) if (C * HW) % 2048 else dict(mask=None)):
         assert lib.actnn_batch_norm_forward_apply_relu(*args(**bad)) != 0, bad
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("N,C,H", [(8, 64, 8), (4, 256, 4), (32, 16, 4), (6, 128, 8), (40, 64, 4)])
+def test_backward_with_the_relu_mask_equals_relu_backward_then_backward(dtype, N, C, H):
+    """actnn_batch_norm_backward_packed_relu against actnn_relu_backward followed by
+    actnn_batch_norm_backward_packed: gradients and the table of squared sums bit for bit (several
+    widths, blocks of one to many steps, sample boundaries inside a block of the mask)."""
+    import actnn_amd.cpp_extension.backward_func as bf
+    import actnn_amd.cpp_extension.quantization as ext_q
+    from actnn_amd.ops import _Quantized
+    from actnn_amd.utils import memory_order
+    g = torch.Generator(device=DEV).manual_seed(N + C + H)
+    x = (torch.randn(N, C, H, H, device=DEV, generator=g) * 1.5).to(dtype).contiguous(memory_format=torch.channels_last)
+    go = torch.randn(N, C, H, H, device=DEV, generator=g).to(dtype).contiguous(memory_format=torch.channels_last)
+    keep = torch.rand(N, H, H, C, device=DEV, generator=g) > 0.4
+    _, mask = ext_q.relu_forward(torch.where(keep, 1.0, -1.0).to(dtype))
+    w = torch.rand(C, device=DEV, generator=g) * 2 - 0.5
+    b = torch.randn(C, device=DEV, generator=g)
+    ws, mean, invstd, mn, mx = bf.hip_batch_norm_forward_stats(x, w, b, None, None, 0.1, 1e-5)
+    widths = torch.randint(1, 9, (N,), generator=torch.Generator().manual_seed(2), dtype=torch.int32)
+    bits = ext_q.attach_bits_host(widths.to(DEV), widths)
+    _, packed, scale = bf.hip_batch_norm_forward_apply(x, ws, bits, mn, mx)
+    q = _Quantized((packed, bits, scale, mn.view(N, -1, 1)))
+    q.native_bf16, q.memory_format = dtype == torch.bfloat16, torch.channels_last
+    masked = ext_q.relu_backward(memory_order(go), mask).permute(0, 3, 1, 2)
+    assert torch.equal(memory_order(masked), torch.where(keep, memory_order(go), torch.zeros_like(memory_order(go))))
+    ref = bf.hip_batch_norm_backward_packed(x.shape, q, masked, w, mean, invstd, sumsq=True)
+    got = bf.hip_batch_norm_backward_packed(x.shape, q, go, w, mean, invstd, sumsq=True, relu_mask=mask)
+    for u, v in zip(ref, got):
+        assert torch.equal(u, v)
+    assert torch.equal(bf.known_sumsq(ref[0]), bf.known_sumsq(got[0]))

@@ -930,18 +930,20 @@ def test_fixed_width_batch_norm_takes_the_fused_passes(channels_last):
 def test_relu_folded_into_the_batch_norm_pass_equals_the_two_layers(dtype, channels, size, folded):
     """layers.bn_relu hands a converted batch norm and the ReLU after it over together: where the
     shape allows (channels-last, 16-bit, C a divisor of 256) the ReLU runs inside the normalise +
-    pack pass.  Output, group min / max left for the next layer, running statistics, the compressed
-    input and every gradient are those of the two layers, bit for bit; other shapes take the two
-    layers."""
+    pack pass, and the backward passes apply the ReLU's mask to the gradient as they read it.
+    Output, group min / max left for the next layer, running statistics, the compressed input and
+    every gradient are those of the two layers, bit for bit - also with only the forward folded;
+    other shapes take the two layers."""
     from actnn_amd import ops
     from actnn_amd.layers import QBatchNorm2d, QReLU, bn_relu, known_group_minmax
     calls = []
     real = ops.batch_norm_relu.forward
 
-    def run(fold):
+    def run(fold, fold_backward=True):
         config.reset(); QScheme.reset(); QBNScheme.reset()
         set_optimization_level("L3")
         config.fused_bn_relu = fold
+        config.fused_bn_relu_backward = fold_backward
         torch.manual_seed(3)
         bn, relu = QBatchNorm2d(channels).to(DEV).train(), QReLU()
         with torch.no_grad():
@@ -964,11 +966,11 @@ def test_relu_folded_into_the_batch_norm_pass_equals_the_two_layers(dtype, chann
 
     ops.batch_norm_relu.forward = staticmethod(spy)
     try:
-        two, one = run(False), run(True)
+        two, one, half = run(False), run(True), run(True, False)
     finally:
         ops.batch_norm_relu.forward = staticmethod(real)
-    assert len(calls) == (1 if folded else 0)
-    assert len(two) == len(one)
-    for i, (u, v) in enumerate(zip(two, one)):
-        assert torch.equal(u, v), i
+    assert len(calls) == (2 if folded else 0)
+    assert len(two) == len(one) == len(half)
+    for i, (u, v, w) in enumerate(zip(two, one, half)):
+        assert torch.equal(u, v) and torch.equal(u, w), i
     assert one[0].is_contiguous(memory_format=torch.channels_last) and float(one[0].min()) == 0.0
