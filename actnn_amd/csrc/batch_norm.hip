@@ -994,7 +994,8 @@ template <int E> ACTNN_DEV RowTile row_tile(int64_t C, int tpr, int R, int tile)
 // Waves per SIMD the reduce pass is compiled for: the plain statistics pass fits 8 (64 registers),
 // with the group min/max or the gradient 7, with the decoder of a packed input 5.
 template <bool BWD, bool MINMAX, typename XS, bool MASKED = false> constexpr int cl_reduce_waves() {
-  return MASKED ? 4 : XS::kInFlight == 2 ? 5 : (BWD || MINMAX) ? 7 : 8;     // (with the ReLU's mask rows: 4)
+  // (with the ReLU's mask rows 4: three measured 5 % slower, five spills and is 35 % slower)
+  return MASKED ? 4 : XS::kInFlight == 2 ? 5 : (BWD || MINMAX) ? 7 : 8;
 }
 template <typename T, bool BWD, bool MINMAX, bool NT, typename XS, bool MASKED = false>
 __global__ __launch_bounds__(kThreads, (cl_reduce_waves<BWD, MINMAX, XS, MASKED>())) void bn_cl_reduce_kernel(
@@ -1125,8 +1126,10 @@ __global__ __launch_bounds__(kThreads, (cl_reduce_waves<BWD, MINMAX, XS, MASKED>
   }
 }
 
+// (the backward pass that also applies a ReLU's mask is held to 128 registers, four waves per SIMD:
+// left alone it takes 140 and runs 9 % slower)
 template <typename T, bool BWD, bool PACK, typename XS, bool RELU = false>
-__global__ __launch_bounds__(kThreads) void bn_cl_apply_kernel(
+__global__ __launch_bounds__(kThreads, (RELU && BWD ? 4 : 1)) void bn_cl_apply_kernel(
     XS xs, const T* __restrict__ dy, const float* __restrict__ coef, T* __restrict__ out,
     int64_t P, int64_t C, int tpr, int R, int64_t ppb, PackSink ps, FastDiv by_hw, ReluRows relu = ReluRows{}) {
   // (RELU with BWD: the gradient that comes in is masked by `relu` as it is read)
