@@ -193,10 +193,11 @@ def hip_batch_norm_quantize_geometry(input, weight, bias, running_mean, running_
 
 def hip_batch_norm_relu_applies(geo, dtype):
     """True when the normalise + pack pass can also apply the ReLU that follows the batch norm:
-    channels-last 16-bit tensors whose waves own whole 512-element blocks of the mask."""
+    channels-last 16-bit tensors whose waves own whole 512-element blocks of the mask (rows of a
+    divisor of 256 channels) or the same half of two (rows of a multiple of 512), in whole steps."""
     N, C, HW, channels_last = geo
-    return (channels_last and dtype in (torch.float16, torch.bfloat16) and C <= 256 and 256 % C == 0
-            and (N * C * HW) % 2048 == 0)
+    return (channels_last and dtype in (torch.float16, torch.bfloat16)
+            and ((C <= 256 and 256 % C == 0) or C % 512 == 0) and (N * HW) % (2048 // min(C, 256)) == 0)
 
 
 def hip_batch_norm_forward_quantize(input, geo, weight, bias, running_mean, running_var, momentum, eps, alloc,

@@ -311,15 +311,48 @@ template <typename T> ACTNN_DEV uint32_t relu_word(uint32_t w, uint32_t& keep, f
 // ReLU's mask along and zeroes what the ReLU's own backward pass would have zeroed, instead of reading
 // a masked copy.  Keep bits of the wave's next four steps (a step of a block is 2048 elements: the
 // wave's blocks are 4 apart), one word per lane and two bit transposes for the four.
+// Where the 64 mask words of a wave's four steps lie.  Rows of up to 256 channels: a step of the wave
+// is one whole 512-element block of the mask, and the blocks of consecutive steps are 4 apart.  Rows of
+// a multiple of 512 channels: the wave's lanes 0-31 and 32-63 hold the same 256 columns of two
+// consecutive rows, i.e. the same half (the column tile's parity) of two blocks C / 512 apart - the
+// 16 low bits of each of the wave's words belong to the first block's words, the 16 high bits to the
+// second's, and they are stored and loaded as halfwords.
+struct MaskPlace {
+  int64_t first, second;   // word index (narrow rows) / halfword indices (wide rows) of the lane's word
+  bool wide;
+};
+ACTNN_DEV MaskPlace mask_place(int64_t ru_first, int64_t C, int R, int tile) {
+  const uint32_t lane = threadIdx.x & 63u;
+  const int slot = 2 * (int)(lane & 1u) + (int)(lane >> 5);       // which of the four steps the lane's word is of
+  const int64_t k = (lane >> 1) & 15u;
+  const int64_t wave = threadIdx.x >> 6;
+  MaskPlace at;
+  at.wide = C > 256;
+  if (!at.wide) {
+    at.first = (((ru_first * C) >> 9) + wave + 4 * slot) * 16 + k;
+    at.second = 0;
+  } else {
+    const int64_t row = ru_first + (int64_t)slot * R + 2 * wave;
+    const int64_t block = row * (C >> 9) + (tile >> 1);
+    at.first = (block * 16 + k) * 2 + (tile & 1);
+    at.second = ((block + (C >> 9)) * 16 + k) * 2 + (tile & 1);
+  }
+  return at;
+}
 struct ReluRows {
   const int32_t* words;
   int64_t blocks;          // 512-element blocks of the tensor
-  ACTNN_DEV void load(int64_t rb, int64_t C, uint32_t (&m)[4]) const {
-    const uint32_t lane = threadIdx.x & 63u;
-    const int slot = 2 * (int)(lane & 1u) + (int)(lane >> 5);
-    const int64_t block = ((rb * C) >> 9) + (threadIdx.x >> 6) + 4 * slot;
-    const uint32_t w = block < blocks ? (uint32_t)words[block * 16 + ((lane >> 1) & 15u)] : 0u;
-    word_to_rows(w, lane, m);
+  ACTNN_DEV void load(int64_t rb, int64_t C, int R, int tile, uint32_t (&m)[4]) const {
+    const MaskPlace at = mask_place(rb, C, R, tile);
+    uint32_t w = 0u;
+    if (!at.wide) {
+      if (at.first < blocks * 16) w = (uint32_t)words[at.first];
+    } else {
+      const uint16_t* half = reinterpret_cast<const uint16_t*>(words);
+      if (at.first < blocks * 32) w = half[at.first];
+      if (at.second < blocks * 32) w |= (uint32_t)half[at.second] << 16;
+    }
+    word_to_rows(w, threadIdx.x & 63u, m);
   }
 };
 // the chunk's eight 16-bit values with those zeroed whose keep bit (bit i of `row` for value i) is 0
@@ -1073,12 +1106,12 @@ __global__ __launch_bounds__(kThreads, (cl_reduce_waves<BWD, MINMAX, XS, MASKED>
     int64_t rb = p0;
     uint32_t m[4];
     for (; rb + (int64_t)4 * R <= p1; rb += (int64_t)4 * R) {
-      relu.load(rb, C, m);
+      relu.load(rb, C, R, tile, m);
       two(rb, m[0], m[1]);
       two(rb + (int64_t)2 * R, m[2], m[3]);
     }
     if (rb < p1) {
-      relu.load(rb, C, m);
+      relu.load(rb, C, R, tile, m);
       one(rb, m[0]);
       if (rb + R < p1) one(rb + R, m[1]);
       if (rb + (int64_t)2 * R < p1) one(rb + (int64_t)2 * R, m[2]);
@@ -1258,9 +1291,10 @@ __global__ __launch_bounds__(kThreads, (RELU && BWD ? 4 : 1)) void bn_cl_apply_k
       queue.get(j, mul, sub);
       pack_chunk<T, false>(ux, rw, mul, sub, group_words((uint32_t)((ru * C) >> 8) + (lane_elems >> 8)), cur_b);
     };
-    // RELU: the wave's 64 chunks of a step are 512 consecutive elements - one block of the mask - and
-    // a half-wave's 32 chunks one group of 256 outputs (the launcher takes this path only when that
-    // holds and every step of a block is whole).  emit() applies the rule to the normalised chunk,
+    // RELU: the wave's 64 chunks of a step are 512 consecutive elements - one block of the mask - or,
+    // in rows of a multiple of 512 channels, the same half of two blocks (mask_place), and a half-wave's
+    // 32 chunks one group of 256 outputs (the launcher takes this path only when that holds and every
+    // step of a block is whole).  emit() applies the rule to the normalised chunk,
     // stores it, leaves the group's min / max and the lane's 8 keep bits in `row`; four steps' rows
     // make the wave's 64 mask words (blocks 4 apart: a step of the block is 2048 elements).
     const uint32_t lane = threadIdx.x & 63u;
@@ -1291,8 +1325,16 @@ __global__ __launch_bounds__(kThreads, (RELU && BWD ? 4 : 1)) void bn_cl_apply_k
     auto leave_mask = [&](int64_t ru_first, const uint32_t (&rows)[4], int count) __attribute__((always_inline)) {
       const uint32_t word = rows_to_word(rows, lane);
       const int slot = 2 * (int)(lane & 1u) + (int)(lane >> 5);
-      const int64_t block = ((ru_first * C) >> 9) + (threadIdx.x >> 6) + 4 * slot;
-      if (slot < count) ps.relu_mask[block * 16 + ((lane >> 1) & 15u)] = (int32_t)word;
+      const MaskPlace at = mask_place(ru_first, C, R, blockIdx.x);
+      if (slot < count) {
+        if (!at.wide) {
+          ps.relu_mask[at.first] = (int32_t)word;
+        } else {
+          uint16_t* half = reinterpret_cast<uint16_t*>(ps.relu_mask);
+          half[at.first] = (uint16_t)word;
+          half[at.second] = (uint16_t)(word >> 16);
+        }
+      }
     };
     auto pair = [&](int64_t rb0, int j, uint32_t& row0, uint32_t& row1) __attribute__((always_inline)) {
       const int64_t ru0 = rb0 + (int64_t)j * R, ru1 = ru0 + R;
@@ -1376,12 +1418,12 @@ __global__ __launch_bounds__(kThreads, (RELU && BWD ? 4 : 1)) void bn_cl_apply_k
     int64_t rb = p0;
     uint32_t m[4];
     for (; rb + (int64_t)4 * R <= p1; rb += (int64_t)4 * R) {
-      relu.load(rb, C, m);
+      relu.load(rb, C, R, (int)blockIdx.x, m);
       two(rb, m[0], m[1]);
       two(rb + (int64_t)2 * R, m[2], m[3]);
     }
     if (rb < p1) {
-      relu.load(rb, C, m);
+      relu.load(rb, C, R, (int)blockIdx.x, m);
       one(rb, m[0]);
       if (rb + R < p1) one(rb + R, m[1]);
       if (rb + (int64_t)2 * R < p1) one(rb + (int64_t)2 * R, m[2]);
@@ -1543,6 +1585,11 @@ bool make_plan(int64_t N, int64_t C, int64_t HW, int dtype, int channels_last, P
   return cl ? make_plan_cl(N, C, HW, dtype, pl) : make_plan(N, C, HW, dtype, pl);
 }
 int64_t workspace_floats(const Plan& pl, int64_t C) { return pl.part_floats + 3 * C; }
+// Shapes whose channels-last passes can make or apply a ReLU's mask (MaskPlace): every thread of a block
+// active, whole steps only.
+bool relu_mask_shape(const Plan& pl, int64_t C) {
+  return pl.channels_last && !pl.any_shape && ((C <= 256 && 256 % C == 0) || C % 512 == 0) && pl.P % pl.R == 0;
+}
 int64_t apply_waves(const Plan& pl) {      // entries of the sum-of-squares table of the backward apply pass
   if (pl.any_shape) return 0;              // (the element-by-element kernels leave none)
   return (pl.channels_last ? (int64_t)pl.tiles * pl.nsplit_apply : pl.spans * pl.nsplit) * kWaves;
@@ -1869,8 +1916,8 @@ extern "C" int actnn_batch_norm_forward_apply_relu(const void* x, void* y, const
     return ACTNN_EINVAL;
   if (workspace_bytes < workspace_floats(pl, C) * (int64_t)sizeof(float)) return ACTNN_EINVAL;
   if (!aligned16(x) || !aligned16(y) || !aligned16(workspace)) return ACTNN_EALIGN;
-  // a wave's step is one 512-element block of the mask, every step of every block is whole
-  if (!pl.groups_align || C > 256 || 256 % C != 0 || (N * pl.F) % 2048 != 0) return ACTNN_EINVAL;
+  // a wave's step is one 512-element block of the mask or the same half of two, every step of every block is whole
+  if (!pl.groups_align || !relu_mask_shape(pl, C)) return ACTNN_EINVAL;
   if (pl.P > 0x7fffffffLL || C * HW >= ((int64_t)1 << 32) || N * (pl.F / 256) >= 0x7fffffffLL) return ACTNN_EINVAL;
   PackSink sink{bits, prefix, mn, mx, scale, packed, seed, offset, pl.F / 256, nullptr, relu_mask, relu_mn, relu_mx};
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -2078,7 +2125,7 @@ extern "C" int actnn_batch_norm_backward_packed_relu(const int32_t* packed, cons
   if (dtype != ACTNN_F16 && dtype != ACTNN_BF16) return ACTNN_EDTYPE;
   Plan pl;
   if (!channels_last || !make_plan(N, C, HW, dtype, channels_last, pl) || pl.any_shape || !pl.groups_align) return ACTNN_EINVAL;
-  if (C > 256 || 256 % C != 0 || (N * pl.F) % 2048 != 0 || pl.P > 0x7fffffffLL) return ACTNN_EINVAL;
+  if (!relu_mask_shape(pl, C) || pl.P > 0x7fffffffLL) return ACTNN_EINVAL;
   if (sumsq && (!dx || sumsq_entries < apply_waves(pl))) return ACTNN_EINVAL;
   if (!packed || !bits || !prefix || !scale || !mn || !grad_out || !relu_mask || !save_mean || !save_invstd || !workspace)
     return ACTNN_EINVAL;

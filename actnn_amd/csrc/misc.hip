@@ -144,8 +144,8 @@ extern "C" int actnn_batch_norm_forward_quantize(
   const bool relu = relu_mask || relu_mn || relu_mx;
   if (relu && (!relu_mask || !relu_mn || !relu_mx)) return ACTNN_EINVAL;
   // (what the last step will ask, before anything is launched)
-  if (relu && (!channels_last || (dtype != ACTNN_F16 && dtype != ACTNN_BF16) || C > 256 || 256 % C != 0 ||
-               (N * C * HW) % 2048 != 0))
+  if (relu && (!channels_last || (dtype != ACTNN_F16 && dtype != ACTNN_BF16) ||
+               !((C <= 256 && 256 % C == 0) || C % 512 == 0) || (N * HW) % (2048 / (C < 256 ? C : 256)) != 0))
     return ACTNN_EINVAL;
   int rc = actnn_batch_norm_forward_stats(x, weight, bias, running_mean, running_var, save_mean, save_invstd, mn,
                                           mx, workspace, workspace_bytes, N, C, HW, momentum, eps, dtype,

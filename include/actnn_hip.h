@@ -234,8 +234,9 @@ int actnn_allocate_bits_device(const void* mn, const void* mx, float factor, con
  * _apply.  One pass over x instead of a pass over x and a pass over bn(x) (torchvision's
  * `relu(bn(conv(x)))`, mem_speed_benchmark/train.py:203-206; ops.py:436-470 and
  * quantization.cc:106-124 in the reference).  Channels-last 16-bit tensors with C a divisor of 256
- * and N * C * HW a multiple of 2048 (a wave's 64 chunks are then one 512-element block of the
- * mask); everything else is ACTNN_EINVAL / ACTNN_EDTYPE. */
+ * or a multiple of 512 and N * HW a multiple of 2048 / min(C, 256) (a wave's 64 chunks are then one
+ * 512-element block of the mask, or the same half of two); everything else is ACTNN_EINVAL /
+ * ACTNN_EDTYPE. */
 int actnn_batch_norm_forward_apply_relu(const void* x, void* y, const void* workspace,
                                         int64_t workspace_bytes, const int32_t* bits,
                                         const int32_t* prefix, const void* mn, const void* mx, void* scale,

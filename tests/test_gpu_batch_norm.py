@@ -359,7 +359,8 @@ def test_forward_with_packed_copy_equals_forward_then_pack(N, C, spatial, dtype,
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("N,C,H", [(8, 64, 8), (4, 256, 4), (32, 16, 4), (6, 128, 8)])
+@pytest.mark.parametrize("N,C,H", [(8, 64, 8), (4, 256, 4), (32, 16, 4), (6, 128, 8), (6, 512, 4), (3, 1024, 4),
+                                   (5, 2048, 4)])
 def test_apply_with_the_relu_folded_in_equals_apply_then_relu(dtype, N, C, H):
     """actnn_batch_norm_forward_apply_relu against actnn_batch_norm_forward_apply followed by
     actnn_relu_forward_minmax on the stored result: output, mask words, group min / max, scale and
@@ -400,13 +401,14 @@ def test_apply_with_the_relu_folded_in_equals_apply_then_relu(dtype, N, C, H):
                         mn.data_ptr(), mx.data_ptr(), scale2.data_ptr(), packed2.data_ptr(), seed, offset,
                         k.get("mask", mask.data_ptr()), zmn.data_ptr(), zmx.data_ptr(), k.get("N", N), k.get("C", C), HW,
                         k.get("dtype", ext_q.g.DTYPE_CODE[dtype]), k.get("cl", 1), None)
-    for bad in (dict(cl=0), dict(dtype=0), dict(mask=None), dict(C=C * 3), dict(N=N + 1) if (C * HW) % 2048 else dict(mask=None)):
+    for bad in (dict(cl=0), dict(dtype=0), dict(mask=None), dict(C=C * 3)):
         assert lib.actnn_batch_norm_forward_apply_relu(*args(**bad)) != 0, bad
     torch.cuda.synchronize()
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("N,C,H", [(8, 64, 8), (4, 256, 4), (32, 16, 4), (6, 128, 8), (40, 64, 4)])
+@pytest.mark.parametrize("N,C,H", [(8, 64, 8), (4, 256, 4), (32, 16, 4), (6, 128, 8), (40, 64, 4), (6, 512, 4),
+                                   (3, 1024, 4), (5, 2048, 4), (9, 512, 8)])
 def test_backward_with_the_relu_mask_equals_relu_backward_then_backward(dtype, N, C, H):
     """actnn_batch_norm_backward_packed_relu against actnn_relu_backward followed by
     actnn_batch_norm_backward_packed: gradients and the table of squared sums bit for bit (several

@@ -926,10 +926,10 @@ def test_fixed_width_batch_norm_takes_the_fused_passes(channels_last):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("channels,size,folded", [(64, 8, True), (128, 4, True), (256, 8, True), (32, 8, True),
-                                                  (512, 4, False), (96, 8, False)])
+                                                  (512, 4, True), (1024, 2, True), (96, 8, False), (768, 4, False)])
 def test_relu_folded_into_the_batch_norm_pass_equals_the_two_layers(dtype, channels, size, folded):
     """layers.bn_relu hands a converted batch norm and the ReLU after it over together: where the
-    shape allows (channels-last, 16-bit, C a divisor of 256) the ReLU runs inside the normalise +
+    shape allows (channels-last, 16-bit, C a divisor of 256 or a multiple of 512) the ReLU runs inside the normalise +
     pack pass, and the backward passes apply the ReLU's mask to the gradient as they read it.
     Output, group min / max left for the next layer, running statistics, the compressed input and
     every gradient are those of the two layers, bit for bit - also with only the forward folded;
