@@ -78,13 +78,13 @@ SIGNATURES = {
     "actnn_batch_norm_forward_static": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64,
                                         c_i64, ctypes.c_double, ctypes.c_double, c_i32, c_i32, c_vp],
     # x weight bias rm rv y save_mean save_invstd mn mx ws | ws_bytes | factor mult per_sample | sens bits prefix |
-    # initial target | scale packed | seed offset | relu_mask relu_mn relu_mx | N C HW | momentum eps |
+    # initial target | scale packed | seed offset | relu_mask relu_mn relu_mx residual | N C HW | momentum eps |
     # dtype channels_last stream
     "actnn_batch_norm_forward_quantize": [c_vp] * 11 + [c_i64, ctypes.c_float, c_vp, c_i32, c_vp, c_vp, c_vp,
-                                          c_i32, c_i64, c_vp, c_vp, c_u64, c_u64, c_vp, c_vp, c_vp, c_i64, c_i64,
+                                          c_i32, c_i64, c_vp, c_vp, c_u64, c_u64, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64,
                                           c_i64, ctypes.c_double, ctypes.c_double, c_i32, c_i32, c_vp],
     "actnn_batch_norm_forward_apply_relu": [c_vp, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_u64,
-                                            c_u64, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
+                                            c_u64, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_vp],
     "actnn_quantize_activation": [c_vp, c_vp, c_vp, c_i32, ctypes.c_float, c_vp, c_i32, c_vp, c_vp, c_vp, c_i32,
                                   c_i64, c_vp, c_vp, c_u64, c_u64, c_i64, c_i64, c_i32, c_vp],
     "actnn_batch_norm_forward_stats": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,

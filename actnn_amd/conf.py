@@ -39,6 +39,7 @@ class QuantizationConfig:
         # together (layers.bn_relu) and the shape allows it: bn(x) is never written
         self.fused_bn_relu = True
         self.fused_bn_relu_backward = True             # ... and its backward passes apply the ReLU's mask as they read
+        self.fused_bn_add_relu = True                  # relu(bn(x) + identity) likewise (layers.bn_add_relu)
         # QLinear's weight gradient straight from the packed input (the dequantised input is never
         # written): True - where the fused kernel is the faster path, i.e. for the 2-bit fixed-width
         # stream; "always" - for every stream it takes (saves the full-precision copy at 0.7-0.9 ms

@@ -201,14 +201,15 @@ def hip_batch_norm_relu_applies(geo, dtype):
 
 
 def hip_batch_norm_forward_quantize(input, geo, weight, bias, running_mean, running_var, momentum, eps, alloc,
-                                    relu=False):
+                                    relu=False, residual=None):
     """Statistics + group min/max -> widths on the device -> normalise + pack, in one call:
     -> (output, save_mean, save_invstd, mn, mx, bits, packed, scale), what
     hip_batch_norm_forward_stats, allocate_bits_device and hip_batch_norm_forward_apply return one
     after the other.  `geo` from hip_batch_norm_quantize_geometry, `alloc` the scheme's
     AllocationArgs (factor, mult, initial, target, total, sens_out).  With `relu`
-    (hip_batch_norm_relu_applies) the output is relu(bn(input)) and the tuple ends with the ReLU's
-    mask and the group min / max of the output."""
+    (hip_batch_norm_relu_applies) the output is relu(bn(input)) - relu(bn(input) + residual) with a
+    `residual` laid out like the input - and the tuple ends with the ReLU's mask and the group
+    min / max of the output."""
     from .quantization import attach_bits_total, mask_words
     N, C, HW, channels_last = geo
     dev, dtype = input.device, input.dtype
@@ -240,7 +241,8 @@ def hip_batch_norm_forward_quantize(input, geo, weight, bias, running_mean, runn
             save_mean.data_ptr(), save_invstd.data_ptr(), mn.data_ptr(), mx.data_ptr(), ws.data_ptr(), ws_bytes,
             alloc.factor, mult_ptr, per_sample, sens.data_ptr(), bits.data_ptr(), prefix.data_ptr(),
             alloc.initial, alloc.target, scale.data_ptr(), packed.data_ptr(), seed, offset, _ptr(mask), _ptr(zmn),
-            _ptr(zmx), N, C, HW, float(momentum), float(eps), code, int(channels_last), _glue.stream_ptr(dev)),
+            _ptr(zmx), _ptr(residual), N, C, HW, float(momentum), float(eps), code, int(channels_last),
+            _glue.stream_ptr(dev)),
             "batch_norm_forward_quantize")
     attach_bits_total(bits, alloc.total, prefix)
     if relu:

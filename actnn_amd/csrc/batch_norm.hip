@@ -293,6 +293,8 @@ struct PackSink {
   int32_t* relu_mask;
   void* relu_mn;
   void* relu_mx;
+  // ... and a residual added before the ReLU: y = relu(bn(x) + residual), laid out like x
+  const void* relu_add;
 };
 
 // ReLU on a word of two 16-bit values (already rounded to T, so the rule sees what a separate pass
@@ -318,24 +320,26 @@ template <typename T> ACTNN_DEV uint32_t relu_word(uint32_t w, uint32_t& keep, f
 // 16 low bits of each of the wave's words belong to the first block's words, the 16 high bits to the
 // second's, and they are stored and loaded as halfwords.
 struct MaskPlace {
-  int64_t first, second;   // word index (narrow rows) / halfword indices (wide rows) of the lane's word
-  bool wide;
+  uint32_t first, second;  // word index (narrow rows) / halfword indices (wide rows) of the lane's word
+  bool wide;               // (32-bit: the launcher takes tensors of up to 2^27 blocks)
 };
 ACTNN_DEV MaskPlace mask_place(int64_t ru_first, int64_t C, int R, int tile) {
   const uint32_t lane = threadIdx.x & 63u;
-  const int slot = 2 * (int)(lane & 1u) + (int)(lane >> 5);       // which of the four steps the lane's word is of
-  const int64_t k = (lane >> 1) & 15u;
-  const int64_t wave = threadIdx.x >> 6;
+  const uint32_t slot = 2u * (lane & 1u) + (lane >> 5);            // which of the four steps the lane's word is of
+  const uint32_t k = (lane >> 1) & 15u;
+  const uint32_t wave = threadIdx.x >> 6;
   MaskPlace at;
   at.wide = C > 256;
   if (!at.wide) {
-    at.first = (((ru_first * C) >> 9) + wave + 4 * slot) * 16 + k;
-    at.second = 0;
+    const uint32_t block0 = (uint32_t)((ru_first * C) >> 9);      // the same for the whole block of threads
+    at.first = (block0 + wave + 4u * slot) * 16u + k;
+    at.second = 0u;
   } else {
-    const int64_t row = ru_first + (int64_t)slot * R + 2 * wave;
-    const int64_t block = row * (C >> 9) + (tile >> 1);
-    at.first = (block * 16 + k) * 2 + (tile & 1);
-    at.second = ((block + (C >> 9)) * 16 + k) * 2 + (tile & 1);
+    const uint32_t per_row = (uint32_t)(C >> 9);
+    const uint32_t block0 = (uint32_t)ru_first * per_row + ((uint32_t)tile >> 1);
+    const uint32_t block = block0 + (slot * (uint32_t)R + 2u * wave) * per_row;
+    at.first = (block * 16u + k) * 2u + ((uint32_t)tile & 1u);
+    at.second = at.first + per_row * 32u;
   }
   return at;
 }
@@ -344,13 +348,14 @@ struct ReluRows {
   int64_t blocks;          // 512-element blocks of the tensor
   ACTNN_DEV void load(int64_t rb, int64_t C, int R, int tile, uint32_t (&m)[4]) const {
     const MaskPlace at = mask_place(rb, C, R, tile);
+    const uint32_t end = (uint32_t)blocks * 16u;
     uint32_t w = 0u;
     if (!at.wide) {
-      if (at.first < blocks * 16) w = (uint32_t)words[at.first];
+      if (at.first < end) w = (uint32_t)words[at.first];
     } else {
       const uint16_t* half = reinterpret_cast<const uint16_t*>(words);
-      if (at.first < blocks * 32) w = half[at.first];
-      if (at.second < blocks * 32) w |= (uint32_t)half[at.second] << 16;
+      if (at.first < 2u * end) w = half[at.first];
+      if (at.second < 2u * end) w |= (uint32_t)half[at.second] << 16;
     }
     word_to_rows(w, threadIdx.x & 63u, m);
   }
@@ -1159,10 +1164,12 @@ __global__ __launch_bounds__(kThreads, (cl_reduce_waves<BWD, MINMAX, XS, MASKED>
   }
 }
 
-// (the backward pass that also applies a ReLU's mask is held to 128 registers, four waves per SIMD:
-// left alone it takes 140 and runs 9 % slower)
-template <typename T, bool BWD, bool PACK, typename XS, bool RELU = false>
-__global__ __launch_bounds__(kThreads, (RELU && BWD ? 4 : 1)) void bn_cl_apply_kernel(
+// RELU: 0 - none; 1 - the ReLU after the batch norm is applied by the pass (forward) / its mask to
+// the incoming gradient (backward); 2 - forward only: relu(bn(x) + residual).
+// (the passes that also apply a ReLU or its mask are held to 128 registers, four waves per SIMD: left
+// alone the backward one takes 140 and runs 9 % slower)
+template <typename T, bool BWD, bool PACK, typename XS, int RELU = 0>
+__global__ __launch_bounds__(kThreads, (RELU ? 4 : 1)) void bn_cl_apply_kernel(
     XS xs, const T* __restrict__ dy, const float* __restrict__ coef, T* __restrict__ out,
     int64_t P, int64_t C, int tpr, int R, int64_t ppb, PackSink ps, FastDiv by_hw, ReluRows relu = ReluRows{}) {
   // (RELU with BWD: the gradient that comes in is masked by `relu` as it is read)
@@ -1173,6 +1180,7 @@ __global__ __launch_bounds__(kThreads, (RELU && BWD ? 4 : 1)) void bn_cl_apply_k
   constexpr int U = XS::kInFlight;
   static_assert(!(PACK && BWD), "the packed copy is made by the forward pass");
   static_assert(!RELU || BWD || (PACK && sizeof(T) == 2), "the ReLU is folded into the packing pass of 16-bit tensors");
+  static_assert(RELU != 2 || !BWD, "the residual is added by the forward pass");
   // The sample that holds the row of the last pack: its width, its first word in the stream and its
   // first row / group.  A thread stays inside one sample for many rows, so these are looked up only
   // when a row leaves it, and a chunk's place in the stream is 32-bit arithmetic on top of them (rows,
@@ -1298,9 +1306,23 @@ __global__ __launch_bounds__(kThreads, (RELU && BWD ? 4 : 1)) void bn_cl_apply_k
     // stores it, leaves the group's min / max and the lane's 8 keep bits in `row`; four steps' rows
     // make the wave's 64 mask words (blocks 4 apart: a step of the block is 2048 elements).
     const uint32_t lane = threadIdx.x & 63u;
-    auto emit = [&](int64_t ru, const u32x4& y, uint32_t& row) __attribute__((always_inline)) {
-      if constexpr (RELU) {
+    auto emit = [&](int64_t ru, const u32x4& y, uint32_t& row, const u32x4& res) __attribute__((always_inline)) {
+      if constexpr (RELU != 0) {
         uint32_t w[4] = {y.x, y.y, y.z, y.w};
+        if constexpr (RELU == 2) {
+          // bn(x), rounded to T as its store would round it, plus the residual, rounded as the tensor
+          // addition rounds it
+          const uint32_t a[4] = {res.x, res.y, res.z, res.w};
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            float u[2], v[2];
+            Chunk<T>::widen(w[k], u);
+            Chunk<T>::widen(a[k], v);
+            u[0] += v[0];
+            u[1] += v[1];
+            w[k] = Chunk<T>::narrow(u);
+          }
+        }
         float z[8];
         row = 0;
 #pragma unroll
@@ -1336,23 +1358,31 @@ __global__ __launch_bounds__(kThreads, (RELU && BWD ? 4 : 1)) void bn_cl_apply_k
         }
       }
     };
+    auto res_at = [&](int64_t rb) __attribute__((always_inline)) -> u32x4 {
+      if constexpr (RELU == 2)
+        return load16_nt(reinterpret_cast<const char*>(ps.relu_add) + rb * C * (int64_t)sizeof(T) + lane_bytes);
+      else
+        return u32x4{0u, 0u, 0u, 0u};
+    };
     auto pair = [&](int64_t rb0, int j, uint32_t& row0, uint32_t& row1) __attribute__((always_inline)) {
       const int64_t ru0 = rb0 + (int64_t)j * R, ru1 = ru0 + R;
       const typename XS::Raw rx0 = xs.fetch(ru0), rx1 = xs.fetch(ru1);
+      const u32x4 res0 = res_at(ru0), res1 = res_at(ru1);
       uint32_t rw[2][Noise<T>::kWords];
       noise_pair<T>(ps, (uint64_t)((ru0 * C) >> 3) + (lane_elems >> 3), (uint64_t)((ru1 * C) >> 3) + (lane_elems >> 3),
                     rw[0], rw[1], (tpr & 1) == 0);      // lane ^ 1 is in the same row, hence in the same steps
       const u32x4 ux0 = xs.decode(rx0);
-      emit(ru0, apply(ux0, ux0), row0);
+      emit(ru0, apply(ux0, ux0), row0, res0);
       pack_one(ux0, rw[0], ru0, j);
       const u32x4 ux1 = xs.decode(rx1);
-      emit(ru1, apply(ux1, ux1), row1);
+      emit(ru1, apply(ux1, ux1), row1, res1);
       pack_one(ux1, rw[1], ru1, j + 1);
     };
     auto single = [&](int64_t rb0, int j, uint32_t& row) __attribute__((always_inline)) {
       const int64_t ru0 = rb0 + (int64_t)j * R;
+      const u32x4 res = res_at(ru0);
       const u32x4 ux = xs.decode(xs.fetch(ru0));
-      emit(ru0, apply(ux, ux), row);
+      emit(ru0, apply(ux, ux), row, res);
       uint32_t rw[Noise<T>::kWords];
       Noise<T>::octet((uint64_t)((ru0 * C) >> 3) + (lane_elems >> 3), ps.seed, ps.offset, rw);
       pack_one(ux, rw, ru0, j);
@@ -1366,7 +1396,7 @@ __global__ __launch_bounds__(kThreads, (RELU && BWD ? 4 : 1)) void bn_cl_apply_k
         queue.fill(ps, (rj * C + t.col) >> 8, live ? ps.bits[nj] : 1, live);
       }
       int j = 0;
-      if constexpr (RELU) {
+      if constexpr (RELU != 0) {
         uint32_t rows[4] = {0u, 0u, 0u, 0u};
         for (; j + 4 <= 32 && rb + (int64_t)(j + 3) * R < p1; j += 4) {
           pair(rb0, j, rows[0], rows[1]);
@@ -1588,7 +1618,8 @@ int64_t workspace_floats(const Plan& pl, int64_t C) { return pl.part_floats + 3 
 // Shapes whose channels-last passes can make or apply a ReLU's mask (MaskPlace): every thread of a block
 // active, whole steps only.
 bool relu_mask_shape(const Plan& pl, int64_t C) {
-  return pl.channels_last && !pl.any_shape && ((C <= 256 && 256 % C == 0) || C % 512 == 0) && pl.P % pl.R == 0;
+  return pl.channels_last && !pl.any_shape && ((C <= 256 && 256 % C == 0) || C % 512 == 0) && pl.P % pl.R == 0 &&
+         ((pl.P * C) >> 9) < ((int64_t)1 << 27);
 }
 int64_t apply_waves(const Plan& pl) {      // entries of the sum-of-squares table of the backward apply pass
   if (pl.any_shape) return 0;              // (the element-by-element kernels leave none)
@@ -1646,7 +1677,7 @@ int launch_cl_reduce(const Plan& pl, const XS& xs, const void* dy, float* part, 
       pl.tiles, rows.nsplit, relu);
   return rows.nsplit;
 }
-template <typename T, bool BWD, bool PACK, typename XS, bool RELU = false>
+template <typename T, bool BWD, bool PACK, typename XS, int RELU = 0>
 void launch_cl_apply(const Plan& pl, const XS& xs, const void* dy, const float* coef, void* out, int64_t C,
                      const PackSink& ps, hipStream_t s, const ReluRows& relu = ReluRows{}) {
   const dim3 grid((unsigned)pl.tiles, (unsigned)pl.nsplit_apply), blk(kThreads);
@@ -1712,7 +1743,8 @@ int forward_apply_t(const Plan& pl, const void* x, void* y, const float* ws, con
     const PlainRows<T> xs{static_cast<const T*>(x), C};
     if constexpr (sizeof(T) == 2) {
       if (sink && sink->relu_mask) {
-        launch_cl_apply<T, false, true, PlainRows<T>, true>(pl, xs, nullptr, coef, y, C, *sink, s);
+        if (sink->relu_add) launch_cl_apply<T, false, true, PlainRows<T>, 2>(pl, xs, nullptr, coef, y, C, *sink, s);
+        else launch_cl_apply<T, false, true, PlainRows<T>, 1>(pl, xs, nullptr, coef, y, C, *sink, s);
         ACTNN_RETURN_LAUNCH_STATUS();
       }
     }
@@ -1743,7 +1775,7 @@ int backward_t(const Plan& pl, const XS& xs, const void* dy, const float* weight
       if (dx) {
         PackSink extra{};
         extra.sumsq = sumsq;
-        launch_cl_apply<T, true, false, XS, true>(pl, xs, dy, coef, dx, C, extra, s, *relu);
+        launch_cl_apply<T, true, false, XS, 1>(pl, xs, dy, coef, dx, C, extra, s, *relu);
       }
       ACTNN_RETURN_LAUNCH_STATUS();
     }
@@ -1905,11 +1937,12 @@ extern "C" int actnn_batch_norm_forward_apply_relu(const void* x, void* y, const
                                                    int64_t workspace_bytes, const int32_t* bits,
                                                    const int32_t* prefix, const void* mn, const void* mx,
                                                    void* scale, int32_t* packed, uint64_t seed, uint64_t offset,
-                                                   int32_t* relu_mask, void* relu_mn, void* relu_mx, int64_t N,
-                                                   int64_t C, int64_t HW, int dtype, int channels_last,
-                                                   void* stream) {
+                                                   int32_t* relu_mask, void* relu_mn, void* relu_mx,
+                                                   const void* residual, int64_t N, int64_t C, int64_t HW,
+                                                   int dtype, int channels_last, void* stream) {
   using namespace actnn;
   if (dtype != ACTNN_F16 && dtype != ACTNN_BF16) return ACTNN_EDTYPE;
+  if (!aligned16(residual)) return ACTNN_EALIGN;
   Plan pl;
   if (!channels_last || !make_plan(N, C, HW, dtype, channels_last, pl) || pl.any_shape) return ACTNN_EINVAL;
   if (!x || !y || !workspace || !bits || !prefix || !mn || !mx || !scale || !packed || !relu_mask || !relu_mn || !relu_mx)
@@ -1919,7 +1952,8 @@ extern "C" int actnn_batch_norm_forward_apply_relu(const void* x, void* y, const
   // a wave's step is one 512-element block of the mask or the same half of two, every step of every block is whole
   if (!pl.groups_align || !relu_mask_shape(pl, C)) return ACTNN_EINVAL;
   if (pl.P > 0x7fffffffLL || C * HW >= ((int64_t)1 << 32) || N * (pl.F / 256) >= 0x7fffffffLL) return ACTNN_EINVAL;
-  PackSink sink{bits, prefix, mn, mx, scale, packed, seed, offset, pl.F / 256, nullptr, relu_mask, relu_mn, relu_mx};
+  PackSink sink{bits, prefix, mn, mx, scale, packed, seed, offset, pl.F / 256, nullptr, relu_mask, relu_mn, relu_mx,
+                residual};
   hipStream_t s = static_cast<hipStream_t>(stream);
   const float* ws = static_cast<const float*>(workspace);
   if (dtype == ACTNN_F16) return forward_apply_t<__half>(pl, x, y, ws, &sink, N, C, HW, s);

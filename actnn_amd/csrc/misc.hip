@@ -123,9 +123,9 @@ extern "C" int actnn_batch_norm_forward_apply_relu(const void* x, void* y, const
                                                    int64_t workspace_bytes, const int32_t* bits,
                                                    const int32_t* prefix, const void* mn, const void* mx,
                                                    void* scale, int32_t* packed, uint64_t seed, uint64_t offset,
-                                                   int32_t* relu_mask, void* relu_mn, void* relu_mx, int64_t N,
-                                                   int64_t C, int64_t HW, int dtype, int channels_last,
-                                                   void* stream);
+                                                   int32_t* relu_mask, void* relu_mn, void* relu_mx,
+                                                   const void* residual, int64_t N, int64_t C, int64_t HW,
+                                                   int dtype, int channels_last, void* stream);
 extern "C" int actnn_minimax(const void* data, void* mn, void* mx, int64_t M, int64_t D, int dtype, void* stream);
 extern "C" int actnn_pack_mixed(const void* data, const void* mn, const void* mx, const int32_t* bits,
                                 const int32_t* prefix, void* scale, int32_t* packed, const void* noise,
@@ -137,12 +137,14 @@ extern "C" int actnn_batch_norm_forward_quantize(
     float* save_mean, float* save_invstd, void* mn, void* mx, void* workspace, int64_t workspace_bytes,
     float factor, const float* mult, int mult_per_sample, float* sensitivity, int32_t* bits, int32_t* prefix,
     int initial_bits, int64_t target, void* scale, int32_t* packed, uint64_t seed, uint64_t offset,
-    int32_t* relu_mask, void* relu_mn, void* relu_mx, int64_t N, int64_t C, int64_t HW, double momentum,
-    double eps, int dtype, int channels_last, void* stream) {
+    int32_t* relu_mask, void* relu_mn, void* relu_mx, const void* residual, int64_t N, int64_t C, int64_t HW,
+    double momentum, double eps, int dtype, int channels_last, void* stream) {
   if (!mn || !mx || !bits || !prefix || !scale || !packed || !sensitivity || !y) return ACTNN_EINVAL;
   if (N <= 0 || C <= 0 || HW <= 0 || (C * HW) % 256 != 0) return ACTNN_EINVAL;
   const bool relu = relu_mask || relu_mn || relu_mx;
   if (relu && (!relu_mask || !relu_mn || !relu_mx)) return ACTNN_EINVAL;
+  if (residual && !relu) return ACTNN_EINVAL;
+  if (!actnn::aligned16(residual)) return ACTNN_EALIGN;
   // (what the last step will ask, before anything is launched)
   if (relu && (!channels_last || (dtype != ACTNN_F16 && dtype != ACTNN_BF16) ||
                !((C <= 256 && 256 % C == 0) || C % 512 == 0) || (N * HW) % (2048 / (C < 256 ? C : 256)) != 0))
@@ -156,8 +158,8 @@ extern "C" int actnn_batch_norm_forward_quantize(
   if (rc != ACTNN_OK) return rc;
   if (relu)
     return actnn_batch_norm_forward_apply_relu(x, y, workspace, workspace_bytes, bits, prefix, mn, mx, scale,
-                                               packed, seed, offset, relu_mask, relu_mn, relu_mx, N, C, HW, dtype,
-                                               channels_last, stream);
+                                               packed, seed, offset, relu_mask, relu_mn, relu_mx, residual, N, C, HW,
+                                               dtype, channels_last, stream);
   return actnn_batch_norm_forward_apply(x, y, workspace, workspace_bytes, bits, prefix, mn, mx, scale, packed,
                                         seed, offset, N, C, HW, dtype, channels_last, stream);
 }

@@ -15,7 +15,7 @@ from torch.nn.modules.utils import _pair, _single, _triple
 
 from .conf import config
 from .cpp_extension import quantization as ext_quantization
-from .ops import (batch_norm, batch_norm_relu, batch_norm_relu_geometry, conv1d, conv2d, conv3d, conv_transpose1d, conv_transpose2d, conv_transpose3d,
+from .ops import (batch_norm, batch_norm_add_relu, batch_norm_relu, batch_norm_relu_geometry, conv1d, conv2d, conv3d, conv_transpose1d, conv_transpose2d, conv_transpose3d,
                   linear)
 from .qbnscheme import QBNScheme
 from .qscheme import QScheme
@@ -195,12 +195,13 @@ class _QBatchNormMixin:
     def _init_scheme(self, group):
         self.scheme = QBNScheme(group=group) if config.adaptive_bn_scheme else None
 
-    def forward(self, input, relu=None):
+    def forward(self, input, relu=None, residual=None):
         """`relu`: the QReLU that follows this layer, when the caller hands the pair over together
-        (bn_relu): where the shape allows, the ReLU is folded into the normalise + pack pass."""
+        (bn_relu): where the shape allows, the ReLU is folded into the normalise + pack pass.
+        `residual` with a QAddReLU as `relu` (bn_add_relu): relu(bn(input) + residual) likewise."""
         if not config.training:
             out = super().forward(input)
-            return out if relu is None else relu(out)
+            return out if relu is None else relu(out) if residual is None else relu(out, residual)
         self._check_input_dim(input)
         factor = 0.0 if self.momentum is None else self.momentum
         if self.training and self.track_running_stats and self.num_batches_tracked is not None:
@@ -215,15 +216,23 @@ class _QBatchNormMixin:
         if relu is not None:
             geo = batch_norm_relu_geometry(input, running_mean, running_var, self.weight, self.bias, bn_training,
                                            self.scheme)
+            if geo is not None and residual is not None and not (
+                    config.fused_bn_add_relu and residual.shape == input.shape and residual.dtype == input.dtype and residual.device == input.device
+                    and residual.is_contiguous(memory_format=torch.channels_last) and residual.data_ptr() % 16 == 0):
+                geo = None
             if geo is not None:
-                out, mn, mx = batch_norm_relu.apply(input, running_mean, running_var, self.weight, self.bias,
-                                                    bn_training, factor, self.eps, self.scheme, geo)
+                if residual is None:
+                    out, mn, mx = batch_norm_relu.apply(input, running_mean, running_var, self.weight, self.bias,
+                                                        bn_training, factor, self.eps, self.scheme, geo)
+                else:
+                    out, mn, mx = batch_norm_add_relu.apply(input, residual, running_mean, running_var, self.weight,
+                                                            self.bias, bn_training, factor, self.eps, self.scheme, geo)
                 if _relu_shares_min_max(memory_order(out)):
                     out._actnn_group_minmax = (mn, mx, out._version)
                 return out
         out = batch_norm.apply(input, running_mean, running_var, self.weight, self.bias, bn_training, factor,
                                self.eps, self.scheme)
-        return out if relu is None else relu(out)
+        return out if relu is None else relu(out) if residual is None else relu(out, residual)
 
 
 class QBatchNorm1d(_QBatchNormMixin, nn.BatchNorm1d):
@@ -296,6 +305,15 @@ def bn_relu(bn, relu, input):
     if isinstance(bn, _QBatchNormMixin) and not isinstance(bn, QSyncBatchNorm) and type(relu) is QReLU:
         return bn(input, relu)
     return relu(bn(input))
+
+
+def bn_add_relu(bn, add_relu, input, residual):
+    """add_relu(bn(input), residual) = relu(bn(input) + residual), the closing step of a residual block,
+    for a model that knows the layers follow each other: converted layers get the three in one pass
+    where the shape allows, everything else is the two calls."""
+    if isinstance(bn, _QBatchNormMixin) and not isinstance(bn, QSyncBatchNorm) and type(add_relu) is QAddReLU:
+        return bn(input, add_relu, residual)
+    return add_relu(bn(input), residual)
 
 
 class AddReLU(nn.Module):

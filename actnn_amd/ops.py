@@ -649,6 +649,45 @@ class batch_norm_relu(Function):
         return _batch_norm_backward(ctx, grad_output, mask) + (None,)
 
 
+class batch_norm_add_relu(Function):
+    """relu(batch_norm(input) + residual) - the closing step of a residual block - in the batch norm's
+    normalise + pack pass: neither the normalised tensor nor the sum is written.  Values, mask and
+    gradients are those of the batch norm, the tensor addition and the ReLU one after the other.
+    `residual` is laid out like `input` (same shape, dtype and memory format)."""
+
+    @staticmethod
+    def forward(ctx, input, residual, running_mean, running_var, weight, bias, training,
+                exponential_average_factor, eps, scheme, geo):
+        alloc = scheme.allocation_arguments(geo[0], geo[2], input.device)
+        (output, save_mean, save_var, mn, _mx, q_bits, q_input, q_scale, mask, out_mn,
+         out_mx) = ext_backward_func.hip_batch_norm_forward_quantize(
+            input, geo, weight, bias, running_mean, running_var, exponential_average_factor, eps, alloc, relu=True,
+            residual=residual)
+        N = geo[0]
+        scheme.adopt_device_bits(q_bits, input.numel() // N, alloc)
+        quantized = _mark_saved(_Quantized((q_input, q_bits, q_scale, mn.view(N, -1, 1))), input)
+        empty_cache(config.empty_cache_threshold)
+        ctx.scheme = scheme
+        ctx.other_args = input.shape
+        ctx.saved = (quantized, weight, running_mean, running_var, save_mean, save_var, training, eps, None)
+        ctx.relu_mask = mask
+        ctx.mark_non_differentiable(out_mn, out_mx)
+        ctx.set_materialize_grads(False)
+        return output, out_mn, out_mx
+
+    @staticmethod
+    def backward(ctx, grad_output, _grad_mn, _grad_mx):
+        if grad_output is None:
+            return (None,) * 11
+        # the masked gradient is the residual's gradient, so it is written once and the batch norm reads it
+        fmt = ctx.saved[0].memory_format
+        mask, ctx.relu_mask = ctx.relu_mask, None
+        grad = logical_order(ext_quantization.relu_backward(
+            memory_order(grad_output.contiguous(memory_format=fmt)), mask), fmt)
+        grads = _batch_norm_backward(ctx, grad)
+        return (grads[0], grad) + grads[1:] + (None,)
+
+
 class adaptive_avg_pool2d(Function):
     """Global average pool that keeps only the input's shape for the backward pass
     (ops.py:617-629); output size (1, 1) only, as there."""

@@ -1,13 +1,13 @@
 """ResNet-50 (v1.5: stride on the 3x3 convolution) in the standard public layout, built from
 plain torch.nn layers (and AddReLU for the closing relu(out + identity) of a block) so that QModule
-can convert it; relu(bn(x)) pairs are handed to layers.bn_relu, which is the two calls for plain
-layers.  torchvision is not available in this
+can convert it; relu(bn(x)) pairs and the closing relu(bn(x) + identity) are handed to layers.bn_relu /
+bn_add_relu, which are the separate calls for plain layers.  torchvision is not available in this
 environment; the reference benchmarks torchvision's resnet50
 (mem_speed_benchmark/train.py:170,203-206)."""
 import torch
 import torch.nn as nn
 
-from .layers import AddReLU, bn_relu
+from .layers import AddReLU, bn_add_relu, bn_relu
 
 
 class Bottleneck(nn.Module):
@@ -31,10 +31,9 @@ class Bottleneck(nn.Module):
         identity = x
         out = bn_relu(self.bn1, self.relu1, self.conv1(x))
         out = bn_relu(self.bn2, self.relu2, self.conv2(out))
-        out = self.bn3(self.conv3(out))
         if self.downsample is not None:
             identity = self.downsample(x)
-        return self.relu3(out, identity)
+        return bn_add_relu(self.bn3, self.relu3, self.conv3(out), identity)
 
 
 class ResNet(nn.Module):

@@ -236,13 +236,16 @@ int actnn_allocate_bits_device(const void* mn, const void* mx, float factor, con
  * quantization.cc:106-124 in the reference).  Channels-last 16-bit tensors with C a divisor of 256
  * or a multiple of 512 and N * HW a multiple of 2048 / min(C, 256) (a wave's 64 chunks are then one
  * 512-element block of the mask, or the same half of two); everything else is ACTNN_EINVAL /
- * ACTNN_EDTYPE. */
+ * ACTNN_EDTYPE.  `residual` (null, or a tensor laid out like x): y = relu(bn(x) + residual), the
+ * closing step of a residual block - bn(x) rounded to `dtype` as its store would round it, the sum
+ * rounded as the tensor addition rounds it, so y and the mask equal those of the three separate
+ * operators. */
 int actnn_batch_norm_forward_apply_relu(const void* x, void* y, const void* workspace,
                                         int64_t workspace_bytes, const int32_t* bits,
                                         const int32_t* prefix, const void* mn, const void* mx, void* scale,
                                         int32_t* packed, uint64_t seed, uint64_t offset, int32_t* relu_mask,
-                                        void* relu_mn, void* relu_mx, int64_t N, int64_t C, int64_t HW,
-                                        int dtype, int channels_last, void* stream);
+                                        void* relu_mn, void* relu_mx, const void* residual, int64_t N,
+                                        int64_t C, int64_t HW, int dtype, int channels_last, void* stream);
 
 /* A layer's forward-side sequence in one call (the host layer's glue between the steps - Python
  * here, the Function bodies of actnn/actnn/ops.py:99-118 and :436-470 in the reference - costs more
@@ -250,7 +253,8 @@ int actnn_batch_norm_forward_apply_relu(const void* x, void* y, const void* work
  * they stand for:
  *   actnn_batch_norm_forward_quantize = actnn_batch_norm_forward_stats (with mn / mx)
  *       -> actnn_allocate_bits_device (G = C * HW / 256) -> actnn_batch_norm_forward_apply (with bits),
- *       or, with relu_mask / relu_mn / relu_mx given (all three), -> actnn_batch_norm_forward_apply_relu;
+ *       or, with relu_mask / relu_mn / relu_mx given (all three; `residual` optional),
+ *       -> actnn_batch_norm_forward_apply_relu;
  *   actnn_quantize_activation = [actnn_minimax of data as rows of 256 unless minmax_known]
  *       -> actnn_allocate_bits_device -> actnn_pack_mixed (gs = 256, in-kernel Philox mode).
  * Every output pointer is required. */
@@ -259,8 +263,8 @@ int actnn_batch_norm_forward_quantize(
     float* save_mean, float* save_invstd, void* mn, void* mx, void* workspace, int64_t workspace_bytes,
     float factor, const float* mult, int mult_per_sample, float* sensitivity, int32_t* bits, int32_t* prefix,
     int initial_bits, int64_t target, void* scale, int32_t* packed, uint64_t seed, uint64_t offset,
-    int32_t* relu_mask, void* relu_mn, void* relu_mx, int64_t N, int64_t C, int64_t HW, double momentum,
-    double eps, int dtype, int channels_last, void* stream);
+    int32_t* relu_mask, void* relu_mn, void* relu_mx, const void* residual, int64_t N, int64_t C, int64_t HW,
+    double momentum, double eps, int dtype, int channels_last, void* stream);
 int actnn_quantize_activation(const void* data, void* mn, void* mx, int minmax_known, float factor,
                               const float* mult, int mult_per_sample, float* sensitivity, int32_t* bits,
                               int32_t* prefix, int initial_bits, int64_t target, void* scale, int32_t* packed,

@@ -391,7 +391,19 @@ def test_apply_with_the_relu_folded_in_equals_apply_then_relu(dtype, N, C, H):
     rc = lib.actnn_batch_norm_forward_apply_relu(
         x.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel() * 4, bits.data_ptr(), prefix.data_ptr(), mn.data_ptr(),
         mx.data_ptr(), scale2.data_ptr(), packed2.data_ptr(), seed, offset, mask.data_ptr(), zmn.data_ptr(),
-        zmx.data_ptr(), N, C, HW, ext_q.g.DTYPE_CODE[dtype], 1, None)
+        zmx.data_ptr(), None, N, C, HW, ext_q.g.DTYPE_CODE[dtype], 1, None)
+    assert rc == 0
+    assert torch.equal(memory_order(out), z_ref) and torch.equal(mask, mask_ref)
+    assert torch.equal(zmn, zmn_ref) and torch.equal(zmx, zmx_ref)
+    assert torch.equal(packed2, packed) and torch.equal(scale2, scale)
+    # with a residual: relu(bn(x) + residual) as the addition of the stored bn(x) and the ReLU make it
+    res = (torch.randn(N, C, H, H, device=DEV, generator=g) * 1.5).to(dtype).contiguous(memory_format=torch.channels_last)
+    memory_order(res).reshape(-1)[::3] = -memory_order(y).reshape(-1)[::3]          # exact cancellation
+    z_ref, mask_ref, zmn_ref, zmx_ref = ext_q.relu_forward_minmax(memory_order(y + res).contiguous())
+    rc = lib.actnn_batch_norm_forward_apply_relu(
+        x.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel() * 4, bits.data_ptr(), prefix.data_ptr(), mn.data_ptr(),
+        mx.data_ptr(), scale2.data_ptr(), packed2.data_ptr(), seed, offset, mask.data_ptr(), zmn.data_ptr(),
+        zmx.data_ptr(), res.data_ptr(), N, C, HW, ext_q.g.DTYPE_CODE[dtype], 1, None)
     assert rc == 0
     assert torch.equal(memory_order(out), z_ref) and torch.equal(mask, mask_ref)
     assert torch.equal(zmn, zmn_ref) and torch.equal(zmx, zmx_ref)
@@ -399,7 +411,7 @@ def test_apply_with_the_relu_folded_in_equals_apply_then_relu(dtype, N, C, H):
     # refused: default layout, fp32, C that does not divide 256, elements not a multiple of 2048
     args = lambda **k: (x.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel() * 4, bits.data_ptr(), prefix.data_ptr(),
                         mn.data_ptr(), mx.data_ptr(), scale2.data_ptr(), packed2.data_ptr(), seed, offset,
-                        k.get("mask", mask.data_ptr()), zmn.data_ptr(), zmx.data_ptr(), k.get("N", N), k.get("C", C), HW,
+                        k.get("mask", mask.data_ptr()), zmn.data_ptr(), zmx.data_ptr(), None, k.get("N", N), k.get("C", C), HW,
                         k.get("dtype", ext_q.g.DTYPE_CODE[dtype]), k.get("cl", 1), None)
     for bad in (dict(cl=0), dict(dtype=0), dict(mask=None), dict(C=C * 3)):
         assert lib.actnn_batch_norm_forward_apply_relu(*args(**bad)) != 0, bad

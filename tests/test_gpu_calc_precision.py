@@ -175,8 +175,9 @@ def test_one_call_entry_points_reject_what_their_steps_reject():
         return lib.actnn_batch_norm_forward_quantize(
             x.data_ptr(), None, None, None, None, a["y"], sm.data_ptr(), si.data_ptr(), a["mn"], mx.data_ptr(),
             ws.data_ptr(), ws_bytes, 1.0, None, 0, sens.data_ptr(), bits.data_ptr(), prefix.data_ptr(), 8, 2 * N,
-            scale.data_ptr(), a["packed"], 1, 0, a.get("mask"), None, None, 4, 8, a["HW"], 0.1, 1e-5, 0, 0, None)
+            scale.data_ptr(), a["packed"], 1, 0, a.get("mask"), None, None, a.get("residual"), 4, 8, a["HW"], 0.1,
+            1e-5, 0, 0, None)
     assert bn() == 0
-    for bad in (dict(y=None), dict(mn=None), dict(packed=None), dict(HW=63), dict(mask=packed.data_ptr())):
+    for bad in (dict(y=None), dict(mn=None), dict(packed=None), dict(HW=63), dict(mask=packed.data_ptr()), dict(residual=x.data_ptr())):
         assert bn(**bad) != 0, bad
     torch.cuda.synchronize()

@@ -974,3 +974,57 @@ def test_relu_folded_into_the_batch_norm_pass_equals_the_two_layers(dtype, chann
     for i, (u, v, w) in enumerate(zip(two, one, half)):
         assert torch.equal(u, v) and torch.equal(u, w), i
     assert one[0].is_contiguous(memory_format=torch.channels_last) and float(one[0].min()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("channels,size,folded", [(256, 8, True), (64, 8, True), (512, 4, True), (2048, 2, True),
+                                                  (96, 8, False)])
+def test_closing_step_of_a_residual_block_in_the_batch_norm_pass(dtype, channels, size, folded):
+    """layers.bn_add_relu: relu(bn(x) + identity) with the addition and the ReLU inside the batch norm's
+    normalise + pack pass.  Output, group min / max, running statistics and the gradients of x, of the
+    identity and of the batch norm's parameters are those of QBatchNorm2d, the tensor addition and
+    QReLU (through QAddReLU) one after the other, bit for bit; a residual in another layout, and
+    shapes the pass does not take, go through the separate layers."""
+    from actnn_amd import ops
+    from actnn_amd.layers import QAddReLU, QBatchNorm2d, bn_add_relu, known_group_minmax
+    calls = []
+    real = ops.batch_norm_add_relu.forward
+
+    def run(fold, residual_layout=torch.channels_last):
+        config.reset(); QScheme.reset(); QBNScheme.reset()
+        set_optimization_level("L3")
+        config.fused_bn_relu = fold
+        torch.manual_seed(4)
+        bn, close = QBatchNorm2d(channels).to(DEV).train(), QAddReLU()
+        with torch.no_grad():
+            bn.weight.uniform_(-1.0, 1.5)
+            bn.bias.normal_()
+        g = torch.Generator(device=DEV).manual_seed(10)
+        x = (torch.randn(8, channels, size, size, device=DEV, generator=g) * 2 + 0.3).to(dtype)
+        x = x.contiguous(memory_format=torch.channels_last).requires_grad_(True)
+        res = torch.randn(8, channels, size, size, device=DEV, generator=g).to(dtype)
+        res = res.contiguous(memory_format=residual_layout).requires_grad_(True)
+        go = torch.randn(8, channels, size, size, device=DEV, generator=g).to(dtype).contiguous(memory_format=torch.channels_last)
+        torch.cuda.manual_seed(22)
+        out = bn_add_relu(bn, close, x, res)
+        known = known_group_minmax(out)
+        out.backward(go)
+        return [out.detach(), x.grad, res.grad, bn.weight.grad, bn.bias.grad, bn.running_mean.clone(),
+                bn.running_var.clone()] + (list(known) if known is not None else [])
+
+    def spy(*a, **k):
+        calls.append(1)
+        return real(*a, **k)
+
+    ops.batch_norm_add_relu.forward = staticmethod(spy)
+    try:
+        two, one = run(False), run(True)
+        other_layout = run(True, torch.contiguous_format)
+    finally:
+        ops.batch_norm_add_relu.forward = staticmethod(real)
+    assert len(calls) == (1 if folded else 0)
+    assert len(two) == len(one)
+    for i, (u, v) in enumerate(zip(two, one)):
+        assert torch.equal(u, v), i
+    for i, (u, v) in enumerate(zip(two[:7], other_layout[:7])):
+        assert torch.equal(u, v), i
