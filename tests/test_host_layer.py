@@ -136,6 +136,22 @@ def test_perlayer_allocation_on_host():
     assert float(b1.bits) == bits[2]              # BN copies the preceding layer's budget
 
 
+@pytest.mark.parametrize("layers,N", [(54, 512), (54, 128), (3, 7), (1, 1), (9, 8192)])
+def test_perlayer_mean_widths_in_one_operation_equal_the_per_layer_expression(layers, N):
+    # allocate_perlayer takes every layer's mean width from one reduction over [layers, N]; the
+    # reference's expression is a mean over each layer's slice (qscheme.py:127-128): same values, bit for bit
+    g = torch.Generator().manual_seed(layers * 1000 + N)
+    b = torch.randint(1, 9, (layers * N,), generator=g, dtype=torch.int32)
+    together = b.view(layers, N).float().mean(1)
+    for i in range(layers):
+        one = b[i * N:(i + 1) * N].float().mean()
+        assert one.dtype == together[i].dtype and one.shape == together[i].shape
+        assert torch.equal(one, together[i])
+    dims = torch.randint(1, 10 ** 6, (layers,), generator=g, dtype=torch.int32)
+    assert torch.equal(dims.repeat_interleave(N),
+                       torch.cat([torch.ones(N, dtype=torch.int32) * int(d) for d in dims], 0))
+
+
 def test_adaptive_avg_pool2d_keeps_only_the_shape():
     import torch.nn.functional as F
     from actnn_amd.ops import adaptive_avg_pool2d
