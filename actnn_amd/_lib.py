@@ -43,6 +43,7 @@ SIGNATURES = {
     "actnn_relu_forward_minmax": [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i32, c_vp],
     "actnn_relu_add_forward": [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i32, c_vp],
     "actnn_relu_backward": [c_vp, c_vp, c_vp, c_i64, c_i32, c_vp],
+    "actnn_relu_backward_add": [c_vp, c_vp, c_vp, c_vp, c_i64, c_i32, c_vp],
     "actnn_dropout_forward": [c_vp, c_vp, c_vp, c_i64, ctypes.c_float, c_u64, c_u64, c_i32, c_vp],
     "actnn_dropout_backward": [c_vp, c_vp, c_vp, c_i64, ctypes.c_float, c_i32, c_vp],
     "actnn_max_pool2d_forward": [c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,

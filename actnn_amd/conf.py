@@ -40,6 +40,9 @@ class QuantizationConfig:
         self.fused_bn_relu = True
         self.fused_bn_relu_backward = True             # ... and its backward passes apply the ReLU's mask as they read
         self.fused_bn_add_relu = True                  # relu(bn(x) + identity) likewise (layers.bn_add_relu)
+        # a residual block's input gradient: the closing ReLU's mask applied to the skip connection's
+        # gradient as it is added to the one from the block's layers (layers.skip_connection)
+        self.fused_skip_gradient = True
         # QLinear's weight gradient straight from the packed input (the dequantised input is never
         # written): True - where the fused kernel is the faster path, i.e. for the 2-bit fixed-width
         # stream; "always" - for every stream it takes (saves the full-precision copy at 0.7-0.9 ms

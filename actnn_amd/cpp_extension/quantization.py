@@ -336,6 +336,17 @@ def relu_backward(grad_output, mask):
     return gin
 
 
+def relu_backward_add(grad_output, mask, other):
+    """other + relu_backward(grad_output, mask) in one pass (rounded as the tensor addition rounds);
+    the three tensors are dense in the same memory order."""
+    gin = torch.empty_like(grad_output)
+    with g.on_device(gin.device):
+        check(g.lib().actnn_relu_backward_add(grad_output.data_ptr(), mask.data_ptr(), other.data_ptr(),
+                                              gin.data_ptr(), gin.numel(), g.DTYPE_CODE[gin.dtype],
+                                              g.stream_ptr(gin.device)), "relu_backward_add")
+    return gin
+
+
 class ActQuantizedReLU(Function):
     """quantization.cc:106-119: saves only the 1-bit mask."""
 

@@ -94,12 +94,12 @@ __global__ __launch_bounds__(kThreads) void mask_backward_kernel(const T* __rest
                                                                  const int32_t* __restrict__ mask,
                                                                  T* __restrict__ gin, int64_t n,
                                                                  int64_t n_mask_blocks, float keep_div,
-                                                                 bool divide) {
+                                                                 bool divide, const T* __restrict__ acc = nullptr) {
   const uint32_t lane = threadIdx.x & 31;
   const int64_t mb0 = (int64_t)blockIdx.x * kMaskBlocksPerBlock + (threadIdx.x >> 5) * 2;
   uint32_t w = 0;
   if (mb0 + (lane >> 4) < n_mask_blocks) w = (uint32_t)mask[mb0 * 16 + lane];
-  const uint32_t acc = transpose32(w, lane);       // bits 16*r + k: keep flag of element 16*lane + k of block r
+  const uint32_t rows = transpose32(w, lane);       // bits 16*r + k: keep flag of element 16*lane + k of block r
 #pragma unroll
   for (int r = 0; r < 2; ++r) {
     const int64_t e0 = (mb0 + r) * kMaskBlock + lane * 16;
@@ -115,8 +115,20 @@ __global__ __launch_bounds__(kThreads) void mask_backward_kernel(const T* __rest
     }
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
-      const bool keep = (acc >> (16 * r + k)) & 1u;
+      const bool keep = (rows >> (16 * r + k)) & 1u;
       v[k] = keep ? (divide ? v[k] / keep_div : v[k]) : 0.0f;
+    }
+    if (acc) {                                       // the masked gradient added to another, as a tensor addition adds them
+      float a[16];
+      if (full) {
+        load8(acc + e0, reinterpret_cast<float(&)[8]>(a[0]));
+        load8(acc + e0 + 8, reinterpret_cast<float(&)[8]>(a[8]));
+      } else {
+#pragma unroll
+        for (int k = 0; k < 16; ++k) a[k] = e0 + k < n ? Conv<T>::load(acc, e0 + k) : 0.0f;
+      }
+#pragma unroll
+      for (int k = 0; k < 16; ++k) v[k] = a[k] + v[k];
     }
     if (full) {
       store8(gin + e0, reinterpret_cast<const float(&)[8]>(v[0]));
@@ -205,11 +217,15 @@ __global__ __launch_bounds__(kThreads) void mask_forward16_kernel(const T* __res
   mask[tile * 64 + (lane & 1u) * 32 + (lane >> 1)] = (int32_t)w;
 }
 
-template <typename T>
+// ACC: gin = acc + masked gradient (rounded to T as the tensor addition of the two rounds it): the
+// gradient that arrives at a residual block's input over the skip connection, masked and added to the
+// one from the block's first convolution in one pass.
+template <typename T, bool ACC = false>
 __global__ __launch_bounds__(kThreads) void mask_backward16_kernel(const T* __restrict__ gout,
                                                                    const int32_t* __restrict__ mask,
                                                                    T* __restrict__ gin, int64_t tiles,
-                                                                   float keep_div, bool divide) {
+                                                                   float keep_div, bool divide,
+                                                                   const T* __restrict__ acc = nullptr) {
   const uint32_t lane = threadIdx.x & 63;
   const int64_t tile = (int64_t)blockIdx.x * kTilesPerBlock + (threadIdx.x >> 6);
   if (tile >= tiles) return;
@@ -225,6 +241,12 @@ __global__ __launch_bounds__(kThreads) void mask_backward16_kernel(const T* __re
     for (int k = 0; k < 8; ++k) {
       const bool keep = (m[i] >> k) & 1u;
       v[i][k] = keep ? (divide ? v[i][k] / keep_div : v[i][k]) : 0.0f;
+    }
+    if (ACC) {
+      float a[8];
+      load8_nt(acc + e0 + i * kMaskBlock, a);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[i][k] = a[k] + v[i][k];
     }
     store8_nt(gin + e0 + i * kMaskBlock, v[i]);
   }
@@ -265,17 +287,23 @@ int launch_forward(const void* x, void* y, int32_t* mask, int64_t n, uint32_t th
 
 template <typename T>
 int launch_backward(const void* gout, const int32_t* mask, void* gin, int64_t n, float keep_div,
-                    bool divide, hipStream_t s) {
+                    bool divide, hipStream_t s, const void* acc = nullptr) {
   const T* go = static_cast<const T*>(gout);
+  const T* ac = static_cast<const T*>(acc);
   T* gi = static_cast<T*>(gin);
   int64_t done = 0;
   if (sizeof(T) == 2) {
     const int64_t tiles = n / kTileElems;
     const int64_t tblocks = (tiles + kTilesPerBlock - 1) / kTilesPerBlock;
     if (tblocks > 0x7fffffffLL) return ACTNN_EINVAL;
-    if (tiles > 0)
-      mask_backward16_kernel<T><<<dim3((unsigned)tblocks), dim3(kThreads), 0, s>>>(go, mask, gi, tiles,
-                                                                                   keep_div, divide);
+    if (tiles > 0) {
+      if (ac)
+        mask_backward16_kernel<T, true><<<dim3((unsigned)tblocks), dim3(kThreads), 0, s>>>(go, mask, gi, tiles,
+                                                                                           keep_div, divide, ac);
+      else
+        mask_backward16_kernel<T><<<dim3((unsigned)tblocks), dim3(kThreads), 0, s>>>(go, mask, gi, tiles,
+                                                                                     keep_div, divide);
+    }
     done = tiles * kTileElems;
   }
   const int64_t rest = n - done;
@@ -284,7 +312,7 @@ int launch_backward(const void* gout, const int32_t* mask, void* gin, int64_t n,
     const int64_t blocks = (nmb + kMaskBlocksPerBlock - 1) / kMaskBlocksPerBlock;
     if (blocks > 0x7fffffffLL) return ACTNN_EINVAL;
     mask_backward_kernel<T><<<dim3((unsigned)blocks), dim3(kThreads), 0, s>>>(
-        go + done, mask + done / 32, gi + done, rest, nmb, keep_div, divide);
+        go + done, mask + done / 32, gi + done, rest, nmb, keep_div, divide, ac ? ac + done : nullptr);
   }
   ACTNN_RETURN_LAUNCH_STATUS();
 }
@@ -306,16 +334,16 @@ int dispatch_forward(const void* x, void* y, int32_t* mask, int64_t n, uint32_t 
 }
 
 int dispatch_backward(const void* gout, const int32_t* mask, void* gin, int64_t n, float keep_div,
-                      bool divide, int dtype, void* stream) {
+                      bool divide, int dtype, void* stream, const void* acc = nullptr) {
   if (n < 0) return ACTNN_EINVAL;
   if (n == 0) return ACTNN_OK;
   if (!gout || !gin || !mask) return ACTNN_EINVAL;
-  if (!aligned16(gout) || !aligned16(gin)) return ACTNN_EALIGN;
+  if (!aligned16(gout) || !aligned16(gin) || !aligned16(acc)) return ACTNN_EALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (dtype) {
-    case ACTNN_F32: return launch_backward<float>(gout, mask, gin, n, keep_div, divide, s);
-    case ACTNN_F16: return launch_backward<__half>(gout, mask, gin, n, keep_div, divide, s);
-    case ACTNN_BF16: return launch_backward<bf16_t>(gout, mask, gin, n, keep_div, divide, s);
+    case ACTNN_F32: return launch_backward<float>(gout, mask, gin, n, keep_div, divide, s, acc);
+    case ACTNN_F16: return launch_backward<__half>(gout, mask, gin, n, keep_div, divide, s, acc);
+    case ACTNN_BF16: return launch_backward<bf16_t>(gout, mask, gin, n, keep_div, divide, s, acc);
     default: return ACTNN_EDTYPE;
   }
 }
@@ -389,6 +417,12 @@ extern "C" int actnn_relu_add_forward(const void* x, const void* residual, void*
 extern "C" int actnn_relu_backward(const void* grad_out, const int32_t* mask, void* grad_in,
                                    int64_t n, int dtype, void* stream) {
   return actnn::dispatch_backward(grad_out, mask, grad_in, n, 1.0f, false, dtype, stream);
+}
+
+extern "C" int actnn_relu_backward_add(const void* grad_out, const int32_t* mask, const void* other,
+                                       void* grad_in, int64_t n, int dtype, void* stream) {
+  if (n > 0 && !other) return ACTNN_EINVAL;
+  return actnn::dispatch_backward(grad_out, mask, grad_in, n, 1.0f, false, dtype, stream, other);
 }
 
 extern "C" int actnn_dropout_forward(const void* x, void* y, int32_t* mask, int64_t n, float p,

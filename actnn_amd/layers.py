@@ -15,8 +15,9 @@ from torch.nn.modules.utils import _pair, _single, _triple
 
 from .conf import config
 from .cpp_extension import quantization as ext_quantization
-from .ops import (batch_norm, batch_norm_add_relu, batch_norm_relu, batch_norm_relu_geometry, conv1d, conv2d, conv3d, conv_transpose1d, conv_transpose2d, conv_transpose3d,
-                  linear)
+from .ops import (SkipGradient, batch_norm, batch_norm_add_relu, batch_norm_relu, batch_norm_relu_geometry, conv1d,
+                  conv2d, conv3d, conv_transpose1d, conv_transpose2d, conv_transpose3d, linear)
+from .ops import skip_connection as ops_skip_connection
 from .qbnscheme import QBNScheme
 from .qscheme import QScheme
 from .utils import channels_last_format, logical_order, memory_order
@@ -199,6 +200,7 @@ class _QBatchNormMixin:
         """`relu`: the QReLU that follows this layer, when the caller hands the pair over together
         (bn_relu): where the shape allows, the ReLU is folded into the normalise + pack pass.
         `residual` with a QAddReLU as `relu` (bn_add_relu): relu(bn(input) + residual) likewise."""
+        skip = getattr(residual, "_actnn_skip", None)
         if not config.training:
             out = super().forward(input)
             return out if relu is None else relu(out) if residual is None else relu(out, residual)
@@ -226,7 +228,8 @@ class _QBatchNormMixin:
                                                         bn_training, factor, self.eps, self.scheme, geo)
                 else:
                     out, mn, mx = batch_norm_add_relu.apply(input, residual, running_mean, running_var, self.weight,
-                                                            self.bias, bn_training, factor, self.eps, self.scheme, geo)
+                                                            self.bias, bn_training, factor, self.eps, self.scheme, geo,
+                                                            skip)
                 if _relu_shares_min_max(memory_order(out)):
                     out._actnn_group_minmax = (mn, mx, out._version)
                 return out
@@ -314,6 +317,23 @@ def bn_add_relu(bn, add_relu, input, residual):
     if isinstance(bn, _QBatchNormMixin) and not isinstance(bn, QSyncBatchNorm) and type(add_relu) is QAddReLU:
         return bn(input, add_relu, residual)
     return add_relu(bn(input), residual)
+
+
+def skip_connection(add_relu, input):
+    """(input for the block's layers, input for the skip connection) of a residual block that ends in
+    bn_add_relu(bn, add_relu, ..., the second one).  With converted layers the two are tied so that the
+    closing ReLU's backward and the addition of the two gradients of `input` become one pass; anything
+    else gets `input` twice."""
+    if (type(add_relu) is QAddReLU and config.training and config.fused_skip_gradient and input.is_cuda
+            and input.requires_grad and torch.is_grad_enabled()):
+        skip = SkipGradient()
+        main, identity = ops_skip_connection.apply(input, skip)
+        shared = getattr(input, "_actnn_group_minmax", None)
+        if shared is not None and shared[2] == input._version:
+            main._actnn_group_minmax = (shared[0], shared[1], main._version)
+        identity._actnn_skip = skip
+        return main, identity
+    return input, input
 
 
 class AddReLU(nn.Module):

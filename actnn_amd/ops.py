@@ -657,7 +657,8 @@ class batch_norm_add_relu(Function):
 
     @staticmethod
     def forward(ctx, input, residual, running_mean, running_var, weight, bias, training,
-                exponential_average_factor, eps, scheme, geo):
+                exponential_average_factor, eps, scheme, geo, skip=None):
+        ctx.skip = skip
         alloc = scheme.allocation_arguments(geo[0], geo[2], input.device)
         (output, save_mean, save_var, mn, _mx, q_bits, q_input, q_scale, mask, out_mn,
          out_mx) = ext_backward_func.hip_batch_norm_forward_quantize(
@@ -678,14 +679,69 @@ class batch_norm_add_relu(Function):
     @staticmethod
     def backward(ctx, grad_output, _grad_mn, _grad_mx):
         if grad_output is None:
-            return (None,) * 11
-        # the masked gradient is the residual's gradient, so it is written once and the batch norm reads it
+            return (None,) * 12
         fmt = ctx.saved[0].memory_format
         mask, ctx.relu_mask = ctx.relu_mask, None
+        skip, ctx.skip = ctx.skip, None
+        if skip is not None and ctx.needs_input_grad[1] and config.fused_skip_gradient:
+            # the residual is the block's own input (skip_connection): its gradient - this one, masked -
+            # is added to the gradient from the block's first convolution when that one arrives, in one
+            # pass over the two, and the batch norm masks what it reads itself
+            skip.hand_over(memory_order(grad_output.contiguous(memory_format=fmt)), mask, fmt)
+            grads = _batch_norm_backward(ctx, grad_output, relu_mask=mask)
+            return (grads[0], None) + grads[1:] + (None, None)
+        # the masked gradient is the residual's gradient, so it is written once and the batch norm reads it
         grad = logical_order(ext_quantization.relu_backward(
             memory_order(grad_output.contiguous(memory_format=fmt)), mask), fmt)
         grads = _batch_norm_backward(ctx, grad)
-        return (grads[0], grad) + grads[1:] + (None,)
+        return (grads[0], grad) + grads[1:] + (None, None)
+
+
+class SkipGradient:
+    """What the closing step of a residual block leaves for the block's input: the gradient of the
+    block's output and the closing ReLU's mask.  Their product is the gradient that reaches the input
+    over the skip connection."""
+
+    __slots__ = ("grad", "mask", "memory_format")
+
+    def __init__(self):
+        self.grad = self.mask = self.memory_format = None
+
+    def hand_over(self, grad, mask, memory_format):
+        self.grad, self.mask, self.memory_format = grad, mask, memory_format
+
+    def take(self):
+        held = (self.grad, self.mask, self.memory_format)
+        self.grad = self.mask = self.memory_format = None
+        return held
+
+
+class skip_connection(Function):
+    """The input of a residual block, once for the block's layers and once for the skip connection.
+    Autograd would add the two gradients that come back; here the closing step (batch_norm_add_relu)
+    may leave the skip connection's gradient unmasked in `skip`, and masking and addition are one pass:
+    the same values as relu_backward followed by the tensor addition."""
+
+    @staticmethod
+    def forward(ctx, input, skip):
+        ctx.skip = skip
+        ctx.set_materialize_grads(False)
+        return input.view_as(input), input.view_as(input)
+
+    @staticmethod
+    def backward(ctx, grad_main, grad_skip):
+        grad, mask, fmt = ctx.skip.take()
+        total = grad_main
+        if grad_skip is not None:
+            total = grad_skip if total is None else total + grad_skip
+        if grad is None:
+            return total, None
+        if total is None:
+            return logical_order(ext_quantization.relu_backward(grad, mask), fmt), None
+        other = memory_order(total.contiguous(memory_format=fmt))
+        if other.dtype != grad.dtype or other.data_ptr() % 16:
+            return total + logical_order(ext_quantization.relu_backward(grad, mask), fmt), None
+        return logical_order(ext_quantization.relu_backward_add(grad, mask, other), fmt), None
 
 
 class adaptive_avg_pool2d(Function):

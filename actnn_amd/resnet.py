@@ -7,7 +7,7 @@ environment; the reference benchmarks torchvision's resnet50
 import torch
 import torch.nn as nn
 
-from .layers import AddReLU, bn_add_relu, bn_relu
+from .layers import AddReLU, bn_add_relu, bn_relu, skip_connection
 
 
 class Bottleneck(nn.Module):
@@ -28,7 +28,8 @@ class Bottleneck(nn.Module):
         self.downsample = downsample
 
     def forward(self, x):
-        identity = x
+        # a block without a downsample branch adds its own input back: tie the two uses of it together
+        x, identity = skip_connection(self.relu3, x) if self.downsample is None else (x, None)
         out = bn_relu(self.bn1, self.relu1, self.conv1(x))
         out = bn_relu(self.bn2, self.relu2, self.conv2(out))
         if self.downsample is not None:

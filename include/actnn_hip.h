@@ -130,6 +130,12 @@ int actnn_relu_add_forward(const void* x, const void* residual, void* y, int32_t
                            void* mx, int64_t n, int dtype, void* stream);
 int actnn_relu_backward(const void* grad_out, const int32_t* mask, void* grad_in, int64_t n,
                         int dtype, void* stream);
+/* grad_in = other + actnn_relu_backward(grad_out, mask), in one pass: the sum rounded to `dtype` as
+ * the tensor addition of the two rounds it.  For the input of a residual block, whose gradient is
+ * the one from the block's first convolution plus the masked gradient that arrives over the skip
+ * connection (autograd's accumulation after quantization.cc:117-119 in the reference). */
+int actnn_relu_backward_add(const void* grad_out, const int32_t* mask, const void* other, void* grad_in,
+                            int64_t n, int dtype, void* stream);
 
 /* Dropout with a 1-bit keep mask (same mask layout as ReLU); y = keep ? x / (1 - p) : 0.
  * keep is drawn from the Philox stream (seed, offset) with probability 1 - p (16-bit

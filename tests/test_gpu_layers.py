@@ -1028,3 +1028,64 @@ def test_closing_step_of_a_residual_block_in_the_batch_norm_pass(dtype, channels
         assert torch.equal(u, v), i
     for i, (u, v) in enumerate(zip(two[:7], other_layout[:7])):
         assert torch.equal(u, v), i
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("channels,size", [(256, 8), (512, 4), (96, 8)])
+def test_skip_connection_gradient_in_one_pass_equals_mask_then_addition(dtype, channels, size):
+    """layers.skip_connection ties a residual block's two uses of its input together: the closing
+    step leaves the output's gradient and its ReLU mask, and the input's gradient is the gradient from
+    the block's layers plus the masked one, made in one pass.  The input's gradient, the batch norm's
+    parameter gradients, the output and the shared group min / max are those of the untied block (the
+    mask applied first, autograd adding the two), bit for bit; a shape the fold does not take, and an
+    unconverted closing layer, get the input twice."""
+    from actnn_amd import ops
+    from actnn_amd.layers import (AddReLU, QAddReLU, QBatchNorm2d, QReLU, bn_add_relu, bn_relu, known_group_minmax,
+                                  skip_connection)
+    handed = []
+    real = ops.SkipGradient.hand_over
+
+    def spy(self, *a):
+        handed.append(1)
+        return real(self, *a)
+
+    def run(tied):
+        config.reset(); QScheme.reset(); QBNScheme.reset()
+        set_optimization_level("L3")
+        config.fused_skip_gradient = tied
+        torch.manual_seed(4)
+        bn1, relu1 = QBatchNorm2d(channels).to(DEV).train(), QReLU()
+        bn3, close = QBatchNorm2d(channels).to(DEV).train(), QAddReLU()
+        with torch.no_grad():
+            for bn in (bn1, bn3):                              # either sign, none near zero: a channel that is
+                bn.weight.uniform_(0.4, 1.5)                   # almost constant turns 2-bit noise into overflowing
+                bn.weight.mul_(torch.where(torch.rand_like(bn.weight) < 0.3, -1.0, 1.0))     # float16 gradients
+                bn.bias.normal_()
+        g = torch.Generator(device=DEV).manual_seed(10)
+        leaf = (torch.randn(8, channels, size, size, device=DEV, generator=g) * 2 + 0.3).to(dtype)
+        leaf = leaf.contiguous(memory_format=torch.channels_last).requires_grad_(True)
+        go = torch.randn(8, channels, size, size, device=DEV, generator=g).to(dtype).contiguous(memory_format=torch.channels_last)
+        torch.cuda.manual_seed(22)
+        x = QReLU()(leaf)                                      # a block input that carries its group min / max
+        main, identity = skip_connection(close, x)
+        assert (known_group_minmax(main) is None) == (known_group_minmax(x) is None)
+        out = bn_add_relu(bn3, close, bn_relu(bn1, relu1, main * 0.75), identity)
+        known = known_group_minmax(out)
+        out.backward(go)
+        return [out.detach(), leaf.grad, bn1.weight.grad, bn1.bias.grad, bn3.weight.grad, bn3.bias.grad] + (
+            list(known) if known is not None else [])
+
+    ops.SkipGradient.hand_over = spy
+    try:
+        untied, tied = run(False), run(True)
+    finally:
+        ops.SkipGradient.hand_over = real
+    assert len(handed) == (1 if channels != 96 else 0)
+    assert len(untied) == len(tied)
+    for i, (u, v) in enumerate(zip(untied, tied)):
+        assert torch.isfinite(u).all(), i
+        assert torch.equal(u, v), i
+    x = torch.randn(2, 8, 4, 4, device=DEV, requires_grad=True)
+    main, identity = skip_connection(AddReLU(), x)
+    assert main is x and identity is x
+

@@ -126,6 +126,40 @@ def test_relu_of_a_sum_equals_the_addition_followed_by_relu(dtype, shape):
     assert torch.equal(ad.grad, expected) and torch.equal(bd.grad, expected)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", SHAPES + [(4, 64, 16, 16), (3, 8192 + 40)])
+def test_masked_gradient_added_to_another_equals_the_two_steps(dtype, shape):
+    """actnn_relu_backward_add: other + relu_backward(grad, mask) in one pass is torch's addition of
+    the masked gradient (which rounds the sum to the tensors' dtype), for cancelling sums, operands
+    of very different magnitude and negative zeros on either side."""
+    from actnn_amd import _lib
+    torch.manual_seed(len(shape) + 19)
+    x = torch.randn(*shape).to(dtype).to(DEV)
+    grad = torch.randn(*shape).to(dtype)
+    other = torch.randn(*shape).to(dtype)
+    fg, fo = grad.view(-1), other.view(-1)
+    fo[::5] = -fg[::5]
+    fo[1::7] = fo[1::7] * 2.0 ** -12
+    fo[3::13] = -0.0
+    fg[4::17] = -0.0
+    grad, other = grad.to(DEV), other.to(DEV)
+    _, mask = ext_q.relu_forward(x)
+    expected = other + ext_q.relu_backward(grad, mask)
+    got = ext_q.relu_backward_add(grad, mask, other)
+    assert torch.equal(got.view(torch.int16 if dtype != torch.float32 else torch.int32),
+                       expected.view(torch.int16 if dtype != torch.float32 else torch.int32))
+    assert torch.equal(expected, other + torch.where(x > 0, grad, torch.zeros_like(grad)))
+    lib = _lib.load()
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    n = grad.numel()
+    assert lib.actnn_relu_backward_add(grad.data_ptr(), mask.data_ptr(), None, got.data_ptr(), n, code, None) != 0
+    if n > 8:
+        assert lib.actnn_relu_backward_add(grad.data_ptr(), mask.data_ptr(), other.data_ptr() + other.element_size(),
+                                           got.data_ptr(), n - 8, code, None) != 0
+    assert lib.actnn_relu_backward_add(None, None, None, None, 0, code, None) == 0
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_relu_of_a_sum_with_group_min_max(dtype):
     torch.manual_seed(3)
