@@ -149,11 +149,14 @@ def hip_batch_norm_forward_stats(input, weight, bias, running_mean, running_var,
     return ws, save_mean, save_invstd, mn, mx
 
 
-def hip_batch_norm_forward_apply(input, workspace, bits=None, mn=None, mx=None):
+def hip_batch_norm_forward_apply(input, workspace, bits=None, mn=None, mx=None, relu=False, residual=None):
     """Second half -> (output, packed, scale).  With `bits` (int32 [N] on the device) and the group
     min/max, the pass also quantises the input: `packed` and `scale` are what
-    pack_mixed_precision(groups of input, mn, mx, bits, True) returns for the same generator state."""
-    from .quantization import _bits_info
+    pack_mixed_precision(groups of input, mn, mx, bits, True) returns for the same generator state.
+    With `relu` (packing only, hip_batch_norm_relu_applies) the output is relu(bn(input)) -
+    relu(bn(input) + residual) with a `residual` laid out like the input - and the tuple ends with
+    the ReLU's mask and the group min / max of the output."""
+    from .quantization import _bits_info, mask_words
     N, C, HW, channels_last = _bn_geometry(input)
     lib = _glue.lib()
     code = _glue.DTYPE_CODE[input.dtype]
@@ -166,6 +169,19 @@ def hip_batch_norm_forward_apply(input, workspace, bits=None, mn=None, mx=None):
         packed = torch.empty(total * G * 8, dtype=torch.int32, device=input.device)
         scale = torch.empty(N, G, 1, dtype=input.dtype, device=input.device)
         seed, offset = _glue.philox_args(input.device)
+    if relu:
+        if bits is None:
+            raise RuntimeError("the ReLU is folded into the packing pass only")
+        mask = torch.empty(mask_words(N * C * HW), dtype=torch.int32, device=input.device)
+        zmn = torch.empty(N * G, dtype=input.dtype, device=input.device)
+        zmx = torch.empty(N * G, dtype=input.dtype, device=input.device)
+        with _glue.on_device(input.device):
+            _glue._lib.check(lib.actnn_batch_norm_forward_apply_relu(
+                input.data_ptr(), out.data_ptr(), workspace.data_ptr(), workspace.numel() * 4, _ptr(bits),
+                _ptr(prefix), _ptr(mn), _ptr(mx), _ptr(scale), _ptr(packed), seed, offset, mask.data_ptr(),
+                zmn.data_ptr(), zmx.data_ptr(), _ptr(residual), N, C, HW, code, int(channels_last),
+                _glue.stream_ptr(input.device)), "batch_norm_forward_apply_relu")
+        return out, packed, scale, mask, zmn, zmx
     with _glue.on_device(input.device):
         _glue._lib.check(lib.actnn_batch_norm_forward_apply(
             input.data_ptr(), out.data_ptr(), workspace.data_ptr(), workspace.numel() * 4, _ptr(bits),

@@ -472,19 +472,51 @@ def batch_norm_relu_geometry(input, running_mean, running_var, weight, bias, tra
     from .qscheme import allocate_on_device
     if not config.fused_bn_relu:
         return None
+    if not scheme:
+        # one width for all (levels L1/L2): statistics, then normalise + pack with the ReLU folded in
+        if not (_fixed_width() and config.fused_bn_pack and config.stochastic and not config.swap
+                and _bn_shares_min_max(input, weight, bias, running_mean, running_var, training)):
+            return None
+        geo = ext_backward_func.hip_batch_norm_quantize_geometry(input, weight, bias, running_mean, running_var)
+        return geo if geo is not None and ext_backward_func.hip_batch_norm_relu_applies(geo, input.dtype) else None
     geo = _bn_quantize_geometry(input, running_mean, running_var, weight, bias, training, scheme)
     if geo is None or not ext_backward_func.hip_batch_norm_relu_applies(geo, input.dtype):
         return None
     return geo if allocate_on_device(geo[0], scheme.initial_bits) else None
 
 
+def _fixed_width():
+    """True when activations are compressed at one configured width (no per-sample allocation)."""
+    return (config.compress_activation and not config.simulate
+            and isinstance(config.activation_compression_bits[0], int)
+            and 1 <= config.activation_compression_bits[0] <= 8)
+
+
+def _batch_norm_relu_forward(input, residual, running_mean, running_var, weight, bias, momentum, eps, scheme, geo):
+    """-> (output, save_mean, save_invstd, saved tuple, mask, group min, group max of the output) of
+    relu(bn(input) [+ residual]) for a `geo` of batch_norm_relu_geometry."""
+    N = geo[0]
+    if scheme:
+        alloc = scheme.allocation_arguments(N, geo[2], input.device)
+        (output, save_mean, save_var, mn, _mx, q_bits, q_input, q_scale, mask, out_mn,
+         out_mx) = ext_backward_func.hip_batch_norm_forward_quantize(
+            input, geo, weight, bias, running_mean, running_var, momentum, eps, alloc, relu=True, residual=residual)
+        scheme.adopt_device_bits(q_bits, input.numel() // N, alloc)
+    else:
+        ws, save_mean, save_var, mn, mx = ext_backward_func.hip_batch_norm_forward_stats(
+            input, weight, bias, running_mean, running_var, momentum, eps)
+        q_bits = _uniform_bits(N, config.activation_compression_bits[0], input.device)
+        output, q_input, q_scale, mask, out_mn, out_mx = ext_backward_func.hip_batch_norm_forward_apply(
+            input, ws, q_bits, mn, mx, relu=True, residual=residual)
+    quantized = _mark_saved(_Quantized((q_input, q_bits, q_scale, mn.view(N, -1, 1))), input)
+    return output, save_mean, save_var, quantized, mask, out_mn, out_mx
+
+
 class batch_norm(Function):
     @staticmethod
     def forward(ctx, input, running_mean, running_var, weight, bias, training,
                 exponential_average_factor, eps, scheme):
-        fixed_width = (not scheme and config.compress_activation and not config.simulate
-                       and isinstance(config.activation_compression_bits[0], int)
-                       and 1 <= config.activation_compression_bits[0] <= 8)
+        fixed_width = not scheme and _fixed_width()
         # (the pass rounds stochastically, like pack_*; with config.stochastic off the unfused
         # sequence below is taken and pack_* refuses, as in the reference)
         fused = None
@@ -625,13 +657,8 @@ class batch_norm_relu(Function):
     @staticmethod
     def forward(ctx, input, running_mean, running_var, weight, bias, training,
                 exponential_average_factor, eps, scheme, geo):
-        alloc = scheme.allocation_arguments(geo[0], geo[2], input.device)
-        (output, save_mean, save_var, mn, _mx, q_bits, q_input, q_scale, mask, out_mn,
-         out_mx) = ext_backward_func.hip_batch_norm_forward_quantize(
-            input, geo, weight, bias, running_mean, running_var, exponential_average_factor, eps, alloc, relu=True)
-        N = geo[0]
-        scheme.adopt_device_bits(q_bits, input.numel() // N, alloc)
-        quantized = _mark_saved(_Quantized((q_input, q_bits, q_scale, mn.view(N, -1, 1))), input)
+        output, save_mean, save_var, quantized, mask, out_mn, out_mx = _batch_norm_relu_forward(
+            input, None, running_mean, running_var, weight, bias, exponential_average_factor, eps, scheme, geo)
         empty_cache(config.empty_cache_threshold)
         ctx.scheme = scheme
         ctx.other_args = input.shape
@@ -659,14 +686,8 @@ class batch_norm_add_relu(Function):
     def forward(ctx, input, residual, running_mean, running_var, weight, bias, training,
                 exponential_average_factor, eps, scheme, geo, skip=None):
         ctx.skip = skip
-        alloc = scheme.allocation_arguments(geo[0], geo[2], input.device)
-        (output, save_mean, save_var, mn, _mx, q_bits, q_input, q_scale, mask, out_mn,
-         out_mx) = ext_backward_func.hip_batch_norm_forward_quantize(
-            input, geo, weight, bias, running_mean, running_var, exponential_average_factor, eps, alloc, relu=True,
-            residual=residual)
-        N = geo[0]
-        scheme.adopt_device_bits(q_bits, input.numel() // N, alloc)
-        quantized = _mark_saved(_Quantized((q_input, q_bits, q_scale, mn.view(N, -1, 1))), input)
+        output, save_mean, save_var, quantized, mask, out_mn, out_mx = _batch_norm_relu_forward(
+            input, residual, running_mean, running_var, weight, bias, exponential_average_factor, eps, scheme, geo)
         empty_cache(config.empty_cache_threshold)
         ctx.scheme = scheme
         ctx.other_args = input.shape

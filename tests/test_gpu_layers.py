@@ -924,16 +924,18 @@ def test_fixed_width_batch_norm_takes_the_fused_passes(channels_last):
     assert (grads1[0].float() - gx).abs().max() <= 0.05 * gx.abs().max() + 0.05
 
 
+@pytest.mark.parametrize("level", ["L3", "L2"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("channels,size,folded", [(64, 8, True), (128, 4, True), (256, 8, True), (32, 8, True),
                                                   (512, 4, True), (1024, 2, True), (96, 8, False), (768, 4, False)])
-def test_relu_folded_into_the_batch_norm_pass_equals_the_two_layers(dtype, channels, size, folded):
+def test_relu_folded_into_the_batch_norm_pass_equals_the_two_layers(dtype, channels, size, folded, level):
     """layers.bn_relu hands a converted batch norm and the ReLU after it over together: where the
     shape allows (channels-last, 16-bit, C a divisor of 256 or a multiple of 512) the ReLU runs inside the normalise +
     pack pass, and the backward passes apply the ReLU's mask to the gradient as they read it.
     Output, group min / max left for the next layer, running statistics, the compressed input and
-    every gradient are those of the two layers, bit for bit - also with only the forward folded;
-    other shapes take the two layers."""
+    every gradient are those of the two layers, bit for bit - also with only the forward folded, and
+    at the level with one width for all (L2) as with per-sample widths (L3); other shapes take the
+    two layers."""
     from actnn_amd import ops
     from actnn_amd.layers import QBatchNorm2d, QReLU, bn_relu, known_group_minmax
     calls = []
@@ -941,7 +943,7 @@ def test_relu_folded_into_the_batch_norm_pass_equals_the_two_layers(dtype, chann
 
     def run(fold, fold_backward=True):
         config.reset(); QScheme.reset(); QBNScheme.reset()
-        set_optimization_level("L3")
+        set_optimization_level(level)
         config.fused_bn_relu = fold
         config.fused_bn_relu_backward = fold_backward
         torch.manual_seed(3)
@@ -976,10 +978,11 @@ def test_relu_folded_into_the_batch_norm_pass_equals_the_two_layers(dtype, chann
     assert one[0].is_contiguous(memory_format=torch.channels_last) and float(one[0].min()) == 0.0
 
 
+@pytest.mark.parametrize("level", ["L3", "L2"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("channels,size,folded", [(256, 8, True), (64, 8, True), (512, 4, True), (2048, 2, True),
                                                   (96, 8, False)])
-def test_closing_step_of_a_residual_block_in_the_batch_norm_pass(dtype, channels, size, folded):
+def test_closing_step_of_a_residual_block_in_the_batch_norm_pass(dtype, channels, size, folded, level):
     """layers.bn_add_relu: relu(bn(x) + identity) with the addition and the ReLU inside the batch norm's
     normalise + pack pass.  Output, group min / max, running statistics and the gradients of x, of the
     identity and of the batch norm's parameters are those of QBatchNorm2d, the tensor addition and
@@ -992,7 +995,7 @@ def test_closing_step_of_a_residual_block_in_the_batch_norm_pass(dtype, channels
 
     def run(fold, residual_layout=torch.channels_last):
         config.reset(); QScheme.reset(); QBNScheme.reset()
-        set_optimization_level("L3")
+        set_optimization_level(level)
         config.fused_bn_relu = fold
         torch.manual_seed(4)
         bn, close = QBatchNorm2d(channels).to(DEV).train(), QAddReLU()
@@ -1030,9 +1033,10 @@ def test_closing_step_of_a_residual_block_in_the_batch_norm_pass(dtype, channels
         assert torch.equal(u, v), i
 
 
+@pytest.mark.parametrize("level", ["L3", "L2"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("channels,size", [(256, 8), (512, 4), (96, 8)])
-def test_skip_connection_gradient_in_one_pass_equals_mask_then_addition(dtype, channels, size):
+def test_skip_connection_gradient_in_one_pass_equals_mask_then_addition(dtype, channels, size, level):
     """layers.skip_connection ties a residual block's two uses of its input together: the closing
     step leaves the output's gradient and its ReLU mask, and the input's gradient is the gradient from
     the block's layers plus the masked one, made in one pass.  The input's gradient, the batch norm's
@@ -1051,7 +1055,7 @@ def test_skip_connection_gradient_in_one_pass_equals_mask_then_addition(dtype, c
 
     def run(tied):
         config.reset(); QScheme.reset(); QBNScheme.reset()
-        set_optimization_level("L3")
+        set_optimization_level(level)
         config.fused_skip_gradient = tied
         torch.manual_seed(4)
         bn1, relu1 = QBatchNorm2d(channels).to(DEV).train(), QReLU()
