@@ -233,6 +233,13 @@ class _QBatchNormMixin:
                 if _relu_shares_min_max(memory_order(out)):
                     out._actnn_group_minmax = (mn, mx, out._version)
                 return out
+        if relu is None and config.fused_skip_gradient and input.is_cuda:
+            # (should the output become the identity of a closing step, as a downsample branch's does)
+            tie = SkipGradient()
+            out = batch_norm.apply(input, running_mean, running_var, self.weight, self.bias, bn_training, factor,
+                                   self.eps, self.scheme, tie)
+            out._actnn_skip = tie
+            return out
         out = batch_norm.apply(input, running_mean, running_var, self.weight, self.bias, bn_training, factor,
                                self.eps, self.scheme)
         return out if relu is None else relu(out) if residual is None else relu(out, residual)

@@ -515,7 +515,12 @@ def _batch_norm_relu_forward(input, residual, running_mean, running_var, weight,
 class batch_norm(Function):
     @staticmethod
     def forward(ctx, input, running_mean, running_var, weight, bias, training,
-                exponential_average_factor, eps, scheme):
+                exponential_average_factor, eps, scheme, skip=None):
+        """`skip` (a SkipGradient the caller also attaches to the output): when the output is the
+        identity of a block's closing step, that step may leave its ReLU's mask and the gradient of
+        its output there instead of returning the masked gradient."""
+        ctx.skip = skip
+        ctx.set_materialize_grads(False)
         fixed_width = not scheme and _fixed_width()
         # (the pass rounds stochastically, like pack_*; with config.stochastic off the unfused
         # sequence below is taken and pack_* refuses, as in the reference)
@@ -593,7 +598,16 @@ class batch_norm(Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        return _batch_norm_backward(ctx, grad_output)
+        skip, ctx.skip = ctx.skip, None
+        grad, mask, fmt = skip.take() if skip is not None else (None, None, None)
+        if grad is not None:
+            if grad_output is None:
+                # the output's only use was as that identity: the backward passes mask as they read
+                return _batch_norm_backward(ctx, logical_order(grad, fmt), relu_mask=mask) + (None,)
+            grad_output = grad_output + logical_order(ext_quantization.relu_backward(grad, mask), fmt)
+        if grad_output is None:
+            return (None,) * 10
+        return _batch_norm_backward(ctx, grad_output) + (None,)
 
 
 def _batch_norm_backward(ctx, grad_output, relu_mask=None):

@@ -1035,14 +1035,17 @@ def test_closing_step_of_a_residual_block_in_the_batch_norm_pass(dtype, channels
 
 @pytest.mark.parametrize("level", ["L3", "L2"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("identity_from", ["input", "batch_norm"])
 @pytest.mark.parametrize("channels,size", [(256, 8), (512, 4), (96, 8)])
-def test_skip_connection_gradient_in_one_pass_equals_mask_then_addition(dtype, channels, size, level):
+def test_skip_connection_gradient_in_one_pass_equals_mask_then_addition(dtype, channels, size, level, identity_from):
     """layers.skip_connection ties a residual block's two uses of its input together: the closing
     step leaves the output's gradient and its ReLU mask, and the input's gradient is the gradient from
     the block's layers plus the masked one, made in one pass.  The input's gradient, the batch norm's
     parameter gradients, the output and the shared group min / max are those of the untied block (the
     mask applied first, autograd adding the two), bit for bit; a shape the fold does not take, and an
-    unconverted closing layer, get the input twice."""
+    unconverted closing layer, get the input twice.  The same for an identity that is a batch norm's
+    output (a downsample branch): that batch norm's backward passes then mask the gradient as they
+    read it, and nothing is written for the identity."""
     from actnn_amd import ops
     from actnn_amd.layers import (AddReLU, QAddReLU, QBatchNorm2d, QReLU, bn_add_relu, bn_relu, known_group_minmax,
                                   skip_connection)
@@ -1060,8 +1063,9 @@ def test_skip_connection_gradient_in_one_pass_equals_mask_then_addition(dtype, c
         torch.manual_seed(4)
         bn1, relu1 = QBatchNorm2d(channels).to(DEV).train(), QReLU()
         bn3, close = QBatchNorm2d(channels).to(DEV).train(), QAddReLU()
+        bn_ds = QBatchNorm2d(channels).to(DEV).train()
         with torch.no_grad():
-            for bn in (bn1, bn3):                              # either sign, none near zero: a channel that is
+            for bn in (bn1, bn3, bn_ds):                              # either sign, none near zero: a channel that is
                 bn.weight.uniform_(0.4, 1.5)                   # almost constant turns 2-bit noise into overflowing
                 bn.weight.mul_(torch.where(torch.rand_like(bn.weight) < 0.3, -1.0, 1.0))     # float16 gradients
                 bn.bias.normal_()
@@ -1071,12 +1075,16 @@ def test_skip_connection_gradient_in_one_pass_equals_mask_then_addition(dtype, c
         go = torch.randn(8, channels, size, size, device=DEV, generator=g).to(dtype).contiguous(memory_format=torch.channels_last)
         torch.cuda.manual_seed(22)
         x = QReLU()(leaf)                                      # a block input that carries its group min / max
-        main, identity = skip_connection(close, x)
-        assert (known_group_minmax(main) is None) == (known_group_minmax(x) is None)
+        if identity_from == "input":
+            main, identity = skip_connection(close, x)
+            assert (known_group_minmax(main) is None) == (known_group_minmax(x) is None)
+        else:
+            main, identity = x, bn_ds(x * 0.5)
         out = bn_add_relu(bn3, close, bn_relu(bn1, relu1, main * 0.75), identity)
         known = known_group_minmax(out)
         out.backward(go)
         return [out.detach(), leaf.grad, bn1.weight.grad, bn1.bias.grad, bn3.weight.grad, bn3.bias.grad] + (
+            [bn_ds.weight.grad, bn_ds.bias.grad] if identity_from == "batch_norm" else []) + (
             list(known) if known is not None else [])
 
     ops.SkipGradient.hand_over = spy
