@@ -239,3 +239,28 @@ def test_no_scheme_path_keeps_group_ranges_whatever_pergroup_says():
     assert bits == 4 and torch.equal(mn.view(-1), known[0]) and torch.equal(mx.view(-1), known[1])
     _, mn_s, mx_s, _ = group_min_max(x, known)        # the schemes' rule: one range for the tensor
     assert bool((mn_s == x.min()).all()) and bool((mx_s == x.max()).all())
+
+
+def test_skip_connection_hand_over_and_ordinary_accumulation():
+    """The tie between a residual block's two uses of its input, on the host side: host tensors and
+    unconverted closing layers get the input twice; the autograd node adds the two gradients like
+    the engine would when nothing was handed over; a hand-over is taken exactly once."""
+    from actnn_amd import ops
+    from actnn_amd.layers import AddReLU, QAddReLU, skip_connection
+    x = torch.randn(2, 4, 3, 3, requires_grad=True)
+    for closing in (AddReLU(), QAddReLU()):
+        main, identity = skip_connection(closing, x)                 # a host tensor is never tied
+        assert main is x and identity is x
+    tie = ops.SkipGradient()
+    assert tie.take() == (None, None, None)
+    tie.hand_over("g", "m", torch.channels_last)
+    assert tie.take() == ("g", "m", torch.channels_last) and tie.take() == (None, None, None)
+    # nothing handed over: the node is the plain sum of what arrives on its two outputs
+    tie = ops.SkipGradient()
+    main, identity = ops.skip_connection.apply(x, tie)
+    (main * 2.0 + identity * 3.0).sum().backward()
+    assert torch.equal(x.grad, torch.full_like(x, 5.0))
+    x.grad = None
+    main, identity = ops.skip_connection.apply(x, ops.SkipGradient())
+    (identity * 3.0).sum().backward()                                # only one of the two used
+    assert torch.equal(x.grad, torch.full_like(x, 3.0))
