@@ -718,11 +718,12 @@ class batch_norm_add_relu(Function):
         fmt = ctx.saved[0].memory_format
         mask, ctx.relu_mask = ctx.relu_mask, None
         skip, ctx.skip = ctx.skip, None
-        if skip is not None and ctx.needs_input_grad[1] and config.fused_skip_gradient:
-            # the residual is the block's own input (skip_connection): its gradient - this one, masked -
-            # is added to the gradient from the block's first convolution when that one arrives, in one
-            # pass over the two, and the batch norm masks what it reads itself
-            skip.hand_over(memory_order(grad_output.contiguous(memory_format=fmt)), mask, fmt)
+        if (skip is not None and ctx.needs_input_grad[1] and config.fused_skip_gradient
+                and skip.hand_over(memory_order(grad_output.contiguous(memory_format=fmt)), mask, fmt)):
+            # the residual's producer takes it from there (skip_connection: the block's own input, whose
+            # gradient - this one, masked - is added to the one from the block's first convolution in
+            # one pass; batch_norm: the downsample branch, whose backward passes mask as they read),
+            # and this batch norm masks what it reads itself
             grads = _batch_norm_backward(ctx, grad_output, relu_mask=mask)
             return (grads[0], None) + grads[1:] + (None, None)
         # the masked gradient is the residual's gradient, so it is written once and the batch norm reads it
@@ -743,7 +744,12 @@ class SkipGradient:
         self.grad = self.mask = self.memory_format = None
 
     def hand_over(self, grad, mask, memory_format):
+        """False when something is already held (the tensor is the identity of two closing steps): the
+        caller then returns its masked gradient the ordinary way."""
+        if self.grad is not None:
+            return False
         self.grad, self.mask, self.memory_format = grad, mask, memory_format
+        return True
 
     def take(self):
         held = (self.grad, self.mask, self.memory_format)

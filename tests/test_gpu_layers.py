@@ -1101,3 +1101,39 @@ def test_skip_connection_gradient_in_one_pass_equals_mask_then_addition(dtype, c
     main, identity = skip_connection(AddReLU(), x)
     assert main is x and identity is x
 
+
+
+def test_an_identity_of_two_closing_steps_and_of_another_use_keeps_every_gradient():
+    """One tensor as the identity of two closing steps, and used once more besides: the first
+    closing step hands its gradient over, the second finds the place taken and returns its masked
+    gradient the ordinary way, the other use's gradient arrives as usual.  Output and parameter
+    gradients are those of the untied graph bit for bit; the input's gradient is a sum of five bf16
+    terms whose order of addition differs between the two graphs, so it agrees to the rounding of
+    those additions (no term lost: dropping any one of them is an error of order one)."""
+    from actnn_amd.layers import QAddReLU, QBatchNorm2d, QReLU, bn_add_relu, skip_connection
+
+    def run(tied):
+        config.reset(); QScheme.reset(); QBNScheme.reset()
+        set_optimization_level("L3")
+        config.fused_skip_gradient = tied
+        torch.manual_seed(4)
+        bns = [QBatchNorm2d(64).to(DEV).train() for _ in range(2)]
+        close = QAddReLU()
+        g = torch.Generator(device=DEV).manual_seed(10)
+        leaf = torch.randn(8, 64, 8, 8, device=DEV, generator=g).to(torch.bfloat16)
+        leaf = leaf.contiguous(memory_format=torch.channels_last).requires_grad_(True)
+        go = torch.randn(8, 64, 8, 8, device=DEV, generator=g).to(torch.bfloat16).contiguous(memory_format=torch.channels_last)
+        torch.cuda.manual_seed(22)
+        x = QReLU()(leaf)
+        main, identity = skip_connection(close, x)
+        out = bn_add_relu(bns[0], close, main * 0.75, identity) + bn_add_relu(bns[1], close, main * 1.25, identity) \
+            + identity * 0.5
+        out.backward(go)
+        return [out.detach(), leaf.grad] + [p.grad for bn in bns for p in bn.parameters()]
+
+    for i, (u, v) in enumerate(zip(run(False), run(True))):
+        assert torch.isfinite(u).all(), i
+        if i == 1:
+            assert ((u.float() - v.float()).abs() <= 2.0 ** -6 * (u.float().abs() + 1.0)).all()
+        else:
+            assert torch.equal(u, v), i

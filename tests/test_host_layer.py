@@ -253,7 +253,7 @@ def test_skip_connection_hand_over_and_ordinary_accumulation():
         assert main is x and identity is x
     tie = ops.SkipGradient()
     assert tie.take() == (None, None, None)
-    tie.hand_over("g", "m", torch.channels_last)
+    assert tie.hand_over("g", "m", torch.channels_last) and not tie.hand_over("g2", "m2", None)
     assert tie.take() == ("g", "m", torch.channels_last) and tie.take() == (None, None, None)
     # nothing handed over: the node is the plain sum of what arrives on its two outputs
     tie = ops.SkipGradient()
